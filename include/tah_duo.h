@@ -1,0 +1,110 @@
+/* tah_duo.h -- C ABI of the MI355X (gfx950) duo-causal attention library.
+ *
+ * The reference (thu-nics/TaH) has no FFI on this path: it expresses duo-causal
+ * attention as a dense additive mask + a concatenating Python KV cache + Hugging
+ * Face SDPA.  Each entry point below names the reference code whose device work
+ * it replaces.  All pointers are device pointers unless stated otherwise; all
+ * functions enqueue on `stream`, never allocate, never synchronise, keep no
+ * global state and return 0 or a negative TAH_E_* code (never throw).
+ *
+ * Layout.  Tokens are packed ("varlen"): sequence b owns rows
+ * [cu[b], cu[b+1]) of a [rows, heads, D] bf16 tensor whose innermost D elements
+ * are contiguous; row and head strides are given in elements.  Only valid tokens
+ * are packed, so within a sequence the depth-0 ("iteration 1") key at local
+ * index j has position j, and a depth-0 query at local index i has position
+ * i + (Lk1 - Lq1) (queries are the newest rows of the sequence).  Depth-1
+ * ("iteration 2") rows exist only for hard tokens and carry their position
+ * explicitly (pos_q2 / pos_k2, int32).
+ *
+ * Visibility (tah/model/tah_model.py:788): key (pos_k, depth_k) is visible to
+ * query (pos_q, depth_q) iff pos_k <= pos_q and depth_k <= depth_q.
+ * GQA: query head h reads kv head h / (Hq / Hkv)
+ * (transformers/integrations/sdpa_attention.py:15-24, repeat_kv).
+ */
+#ifndef TAH_DUO_H
+#define TAH_DUO_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TAH_DUO_ABI_VERSION 1
+
+enum {
+    TAH_OK = 0,
+    TAH_E_NULL = -1,      /* a required pointer is NULL */
+    TAH_E_SHAPE = -2,     /* unsupported head_dim / head counts / negative sizes */
+    TAH_E_ALIGN = -3,     /* pointer or stride not 16-byte aligned */
+    TAH_E_LAUNCH = -4,    /* the HIP runtime rejected the launch */
+    TAH_E_WORKSPACE = -5  /* workspace too small */
+};
+
+typedef void* tah_stream_t; /* hipStream_t */
+
+/* One query stream + its key/value segment at one depth. */
+typedef struct tah_duo_stream {
+    const void* q;          /* bf16 [total_q, Hq,  D] */
+    const void* k;          /* bf16 [total_k, Hkv, D] */
+    const void* v;          /* bf16 [total_k, Hkv, D] */
+    void* o;                /* bf16 [total_q, Hq,  D]  (forward output) */
+    float* lse;             /* f32  [Hq, total_q] natural-log normaliser (forward output) */
+    const int32_t* cu_q;    /* int32 [nseq+1] */
+    const int32_t* cu_k;    /* int32 [nseq+1] */
+    const int32_t* pos_q;   /* int32 [total_q]; NULL at depth 0 (implicit positions) */
+    const int32_t* pos_k;   /* int32 [total_k]; NULL at depth 0 */
+    int64_t q_row_stride, q_head_stride;
+    int64_t k_row_stride, k_head_stride;
+    int64_t v_row_stride, v_head_stride;
+    int64_t o_row_stride, o_head_stride;
+    int32_t total_q, total_k;
+} tah_duo_stream;
+
+typedef struct tah_duo_fwd_args {
+    tah_duo_stream s1;      /* depth 0: every token */
+    tah_duo_stream s2;      /* depth 1: hard tokens; total_q may be 0 */
+    int32_t nseq, hq, hkv, d;
+    float scale;            /* softmax scale, head_dim**-0.5 in Qwen3 */
+} tah_duo_fwd_args;
+
+int tah_duo_abi_version(void);
+const char* tah_duo_error_string(int code);
+
+/* Prefill / training forward of duo-causal attention.
+ * Replaces, per decoder layer and for both depths at once:
+ *   TaHForCausalLM._build_attention_mask        tah/model/tah_model.py:744-791
+ *   TaHCache.update / get_cache_upto_iter (cat)  tah/model/causal_cache.py:63-109
+ *   sdpa_attention_forward (repeat_kv + SDPA)    transformers/integrations/sdpa_attention.py:79-166
+ * Depth-0 queries attend to depth-0 keys; depth-1 queries attend to depth-0
+ * keys and depth-1 keys, both cut at the query's position.  `args` is a host
+ * pointer and is read before the call returns.  Rows with no visible key get
+ * o = 0, lse = -inf. */
+int tah_duo_fwd_varlen(const tah_duo_fwd_args* args, tah_stream_t stream);
+
+/* Hard-token index build: stream compaction of a (B, S) byte mask in row-major
+ * order.  Replaces the stable sort + nonzero of gather_active / scatter_back
+ * (tah/model/tah_model.py:111-119, :160-167).  For the r-th True entry, at
+ * (b, s): pos_out[r] = s, flat_out[r] = b*S + s, seq_out[r] = b (each may be
+ * NULL; capacity B*S when given); cu_out[b] = number of True entries in rows
+ * < b, cu_out[B] = total (required, B+1 entries).  Bit-exact. */
+int tah_hard_index_build(const uint8_t* mask, int32_t B, int32_t S, int32_t* pos_out, int32_t* flat_out,
+                         int32_t* seq_out, int32_t* cu_out, tah_stream_t stream);
+
+/* Destination rows of the right-padded (B, width) form used by gather_active
+ * (tah/model/tah_model.py:117-134): out[r] = seq_of[r]*width + (r - cu[seq_of[r]]). */
+int tah_pad_rows_build(const int32_t* cu, const int32_t* seq_of, int32_t n, int32_t width, int32_t* out,
+                       tah_stream_t stream);
+
+/* Row gather / scatter: dst[dst_rows ? dst_rows[r] : r] = src[src_rows ? src_rows[r] : r]
+ * for r < n, rows of row_bytes bytes at the given byte strides.  Replaces
+ * torch.gather (tah_model.py:127-133) and the boolean-mask index_put
+ * (tah_model.py:163-175).  Rows named twice in dst_rows race.  Bit-exact. */
+int tah_rows_copy(const void* src, const int32_t* src_rows, void* dst, const int32_t* dst_rows, int32_t n,
+                  int64_t row_bytes, int64_t src_stride_bytes, int64_t dst_stride_bytes, tah_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TAH_DUO_H */

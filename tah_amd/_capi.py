@@ -1,0 +1,67 @@
+"""ctypes mirror of include/tah_duo.h: structs, prototypes and error mapping.
+
+This module only describes the C ABI; :mod:`tah_amd._lib` loads the MI355X
+library and binds these prototypes to it.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+ABI_VERSION = 1
+
+c_void_p, c_int32, c_int64, c_float = C.c_void_p, C.c_int32, C.c_int64, C.c_float
+
+
+class DuoStream(C.Structure):
+    """``tah_duo_stream``"""
+
+    _fields_ = [
+        ("q", c_void_p), ("k", c_void_p), ("v", c_void_p), ("o", c_void_p), ("lse", c_void_p),
+        ("cu_q", c_void_p), ("cu_k", c_void_p), ("pos_q", c_void_p), ("pos_k", c_void_p),
+        ("q_row_stride", c_int64), ("q_head_stride", c_int64),
+        ("k_row_stride", c_int64), ("k_head_stride", c_int64),
+        ("v_row_stride", c_int64), ("v_head_stride", c_int64),
+        ("o_row_stride", c_int64), ("o_head_stride", c_int64),
+        ("total_q", c_int32), ("total_k", c_int32),
+    ]
+
+
+class DuoFwdArgs(C.Structure):
+    """``tah_duo_fwd_args``"""
+
+    _fields_ = [
+        ("s1", DuoStream), ("s2", DuoStream),
+        ("nseq", c_int32), ("hq", c_int32), ("hkv", c_int32), ("d", c_int32),
+        ("scale", c_float),
+    ]
+
+
+PROTOTYPES = {
+    "tah_duo_abi_version": (C.c_int, []),
+    "tah_duo_error_string": (C.c_char_p, [C.c_int]),
+    "tah_duo_fwd_varlen": (C.c_int, [C.POINTER(DuoFwdArgs), c_void_p]),
+    "tah_hard_index_build": (C.c_int, [c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "tah_pad_rows_build": (C.c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_void_p]),
+    "tah_rows_copy": (C.c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int64, c_void_p]),
+}
+
+
+class TahDuoError(RuntimeError):
+    pass
+
+
+def bind(lib: C.CDLL) -> C.CDLL:
+    """Attach prototypes; raises AttributeError if a declared symbol is missing."""
+    for name, (res, args) in PROTOTYPES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    got = lib.tah_duo_abi_version()
+    if got != ABI_VERSION:
+        raise TahDuoError(f"libtah_duo ABI version {got}, expected {ABI_VERSION}")
+    return lib
+
+
+def check(lib: C.CDLL, rc: int, what: str) -> None:
+    if rc != 0:
+        raise TahDuoError(f"{what}: {lib.tah_duo_error_string(rc).decode()} (code {rc})")

@@ -1,0 +1,84 @@
+// Device-side helpers shared by the duo-causal attention kernels (gfx950, wave64).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace tah {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+
+constexpr int kWave = 64;
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+constexpr float kNegInf = -__builtin_inff();
+
+// v_mfma_f32_32x32x16_bf16: D(32x32) += A(32x16) * B(16x32).
+// lane l: A[i = l%32][k = 8*(l/32) + 0..7], B[k = 8*(l/32) + 0..7][j = l%32],
+// D reg r: [i = 8*(r/4) + 4*(l/32) + r%4][j = l%32].
+__device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+// Row index inside a 32-row MFMA accumulator tile held by (lane half h, reg r).
+__device__ __forceinline__ constexpr int acc_row(int h, int r) { return 8 * (r / 4) + 4 * h + (r % 4); }
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+__device__ __forceinline__ bf16x8 ld_global_16B(const __bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
+__device__ __forceinline__ void st_global_16B(__bf16* p, bf16x8 v) { *reinterpret_cast<bf16x8*>(p) = v; }
+
+// LDS tile of R rows x 128 bf16 (256 B per row, 16 chunks of 16 B), chunk index
+// XOR-swizzled with the row so that 16 lanes reading the same logical chunk of
+// 16 consecutive rows touch 16 different bank groups.
+__device__ __forceinline__ int rowmajor128_off(int row, int chunk) { return row * 256 + ((chunk ^ (row & 15)) << 4); }
+
+// LDS tile of R rows x 64 bf16 (128 B per row, 8 chunks of 16 B), swizzled likewise.
+__device__ __forceinline__ int rowmajor64_off(int row, int chunk) { return row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4); }
+
+// Storage slot of key `key` (0..63) inside a transposed 64-key row.  The PV
+// MFMA contracts over keys; operand slot (half h, j) of 16-key step s must hold
+// the same key as S^T accumulator (half h, reg 8*(s%2)+j), i.e. key
+// 16s + 8*(j/4) + 4h + j%4.  Storing key 16s+8a+4h+b at slot 16s+8h+4a+b makes
+// each lane's 8 operand keys one contiguous 16-byte chunk.
+__device__ __forceinline__ constexpr int pv_slot(int key) {
+    return (key & ~12) | ((key & 4) << 1) | ((key & 8) >> 1);
+}
+
+__device__ __forceinline__ float wave_max_xor32(float x) { return fmaxf(x, __shfl_xor(x, 32)); }
+
+__device__ __forceinline__ int wave_reduce_max(int x) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) { int y = __shfl_xor(x, m); x = x > y ? x : y; }
+    return x;
+}
+__device__ __forceinline__ int wave_reduce_min(int x) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) { int y = __shfl_xor(x, m); x = x < y ? x : y; }
+    return x;
+}
+
+// Locate tile `slot` among sequences whose lengths are cu[b+1]-cu[b], `bm` rows
+// per tile.  On success fills seq/row0/row_end and returns true; otherwise
+// subtracts the number of tiles in this stream from `slot` and returns false.
+__device__ __forceinline__ bool find_tile(const int32_t* cu, int nseq, int bm, int& slot, int& seq, int& row0, int& row_end) {
+    for (int b = 0; b < nseq; ++b) {
+        const int lo = cu[b], hi = cu[b + 1];
+        const int n = (hi - lo + bm - 1) / bm;
+        if (slot < n) {
+            seq = b;
+            row0 = lo + slot * bm;
+            row_end = row0 + bm < hi ? row0 + bm : hi;
+            return true;
+        }
+        slot -= n;
+    }
+    return false;
+}
+
+}  // namespace tah

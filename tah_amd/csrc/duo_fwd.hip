@@ -1,0 +1,375 @@
+// Duo-causal attention forward (prefill / training), bf16 MFMA, gfx950.
+//
+// One workgroup = 8 waves = one query tile of one kv head: G = Hq/Hkv query
+// heads x (256/G) query rows, wave w -> head (w % G), row block (w / G) of 32
+// rows, so every K/V tile staged in LDS serves all query heads of the group.
+// Per key tile of 64 keys each wave computes S^T = K Q^T (keys x queries) with
+// v_mfma_f32_32x32x16_bf16, which leaves one query per lane column: the online
+// softmax needs one cross-lane exchange per tile, and the bf16 probabilities
+// are already in B-operand layout for O^T += V^T P^T.  V is transposed on its
+// way into LDS.  Key tiles come from the depth-0 segment (cut at the tile's
+// largest query position) and, for depth-1 query tiles, from the depth-1
+// segment; the two-axis mask is evaluated per element only on tiles that
+// straddle a query position, and waves skip tiles that lie entirely above
+// their rows.
+#include <hip/hip_runtime.h>
+
+#include "duo_device.h"
+#include "tah_duo.h"
+
+namespace tah {
+namespace {
+
+constexpr int kD = 128;        // head_dim
+constexpr int kBN = 64;        // keys per tile
+constexpr int kThreads = 512;  // 8 waves
+constexpr int kKBytes = kBN * kD * 2;         // 16 KiB, [key][d]
+constexpr int kVBytes = kD * kBN * 2;         // 16 KiB, [d][key slot]
+constexpr int kStageBytes = kKBytes + kVBytes + kBN * 4;  // + key positions
+constexpr int kSmemBytes = 2 * kStageBytes + 64;          // double buffered + tile bounds
+
+struct FwdStream {
+    const __bf16 *q, *k, *v;
+    __bf16* o;
+    float* lse;
+    const int32_t *cu_q, *cu_k, *pos_q, *pos_k;
+    int64_t q_rs, q_hs, k_rs, k_hs, v_rs, v_hs, o_rs, o_hs;
+    int32_t total_q, total_k;
+};
+struct FwdParams {
+    FwdStream s1, s2;
+    int32_t nseq, hq, hkv;
+    float scale_log2e;
+};
+
+struct Prefetch {
+    bf16x8 k[2], v[2];
+    int kpos;
+};
+
+template <int G>
+__global__ __launch_bounds__(kThreads) void duo_fwd_kernel(const FwdParams p) {
+    constexpr int BM = 32 * (8 / G);
+    HIP_DYNAMIC_SHARED(unsigned char, smem)
+
+    const int tid = threadIdx.x;
+    const int wave = tid / kWave;
+    const int lane = tid % kWave;
+    const int half = lane / 32;
+    const int col = lane % 32;
+    const int hk = blockIdx.x;
+
+    // ---- which tile am I ---------------------------------------------------
+    int slot = (int)(gridDim.y - 1 - blockIdx.y);  // heavy (late) tiles first
+    int seq = 0, row0 = 0, row_end = 0;
+    bool second = false;
+    if (!(p.s1.total_q > 0 && find_tile(p.s1.cu_q, p.nseq, BM, slot, seq, row0, row_end))) {
+        if (!(p.s2.total_q > 0 && find_tile(p.s2.cu_q, p.nseq, BM, slot, seq, row0, row_end))) return;
+        second = true;
+    }
+    const FwdStream& qs = second ? p.s2 : p.s1;
+
+    const int head = hk * G + wave % G;
+    const int rblk = wave / G;
+    // depth-0 key segment of this sequence (position of a key = its local index)
+    const int k1_lo = p.s1.cu_k[seq];
+    const int lk1 = p.s1.cu_k[seq + 1] - k1_lo;
+    const __bf16* k1p = p.s1.k + (int64_t)k1_lo * p.s1.k_rs + (int64_t)hk * p.s1.k_hs;
+    const __bf16* v1p = p.s1.v + (int64_t)k1_lo * p.s1.v_rs + (int64_t)hk * p.s1.v_hs;
+    const int left1 = p.s1.total_k - k1_lo;  // rows from the segment start to the end of the array
+    // depth-1 key segment (explicit positions), only seen by depth-1 queries
+    int lk2 = 0, left2 = 0;
+    const __bf16 *k2p = nullptr, *v2p = nullptr;
+    const int32_t* pos2p = nullptr;
+    if (second) {
+        const int k2_lo = p.s2.cu_k[seq];
+        lk2 = p.s2.cu_k[seq + 1] - k2_lo;
+        k2p = p.s2.k + (int64_t)k2_lo * p.s2.k_rs + (int64_t)hk * p.s2.k_hs;
+        v2p = p.s2.v + (int64_t)k2_lo * p.s2.v_rs + (int64_t)hk * p.s2.v_hs;
+        pos2p = p.s2.pos_k + k2_lo;
+        left2 = p.s2.total_k - k2_lo;
+    }
+
+    // ---- my query row, its position, the tile's position bounds ------------
+    const int row = row0 + rblk * 32 + col;
+    const bool row_ok = row < row_end;
+    const int row_ld = row_ok ? row : row_end - 1;  // tiles are never empty
+    int qpos;
+    if (second) {
+        qpos = qs.pos_q[row_ld];
+    } else {
+        const int q_lo = qs.cu_q[seq];
+        qpos = (row_ld - q_lo) + (lk1 - (qs.cu_q[seq + 1] - q_lo));
+    }
+    const int qlim1 = row_ok ? (qpos < lk1 - 1 ? qpos : lk1 - 1) : -1;  // last visible depth-0 key index
+    const int qlim2 = row_ok ? qpos : -1;                              // depth-1 keys: pos_k <= qlim2
+    const int wmax1 = wave_reduce_max(qlim1);
+    const int wmin1 = wave_reduce_min(row_ok ? qlim1 : 0x7fffffff);
+    int* bounds = reinterpret_cast<int*>(smem + 2 * kStageBytes);
+    if (lane == 0) bounds[wave] = wmax1;
+    __syncthreads();
+    int tmax1 = -1;
+#pragma unroll
+    for (int w = 0; w < 8; ++w) tmax1 = bounds[w] > tmax1 ? bounds[w] : tmax1;
+
+    const int n1 = tmax1 >= 0 ? tmax1 / kBN + 1 : 0;
+    const int n2 = second ? (lk2 + kBN - 1) / kBN : 0;
+    const int ntiles = n1 + n2;
+
+    // ---- Q fragments: B operand of S^T = K Q^T ------------------------------
+    bf16x8 qf[8];
+    {
+        const __bf16* qrow = qs.q + (int64_t)row_ld * qs.q_rs + (int64_t)head * qs.q_hs + 8 * half;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) qf[s] = ld_global_16B(qrow + 16 * s);
+    }
+
+    f32x16 oacc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
+    float m_run = kNegInf;  // running max of raw scores
+    float l_run = 0.f;      // this lane's share of the running denominator
+    const float c = p.scale_log2e;
+
+    // ---- global -> register prefetch of one K/V tile ------------------------
+    auto prefetch = [&](int it, Prefetch& pf) {
+        const bool s0 = it < n1;
+        const int base = (s0 ? it : it - n1) * kBN;
+        const __bf16* kp_ = s0 ? k1p : k2p;
+        const __bf16* vp_ = s0 ? v1p : v2p;
+        const int64_t krs = s0 ? p.s1.k_rs : p.s2.k_rs;
+        const int64_t vrs = s0 ? p.s1.v_rs : p.s2.v_rs;
+        const int left = s0 ? left1 : left2;  // clamp keeps tail loads inside the array
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int cidx = tid + kThreads * i;  // 1024 chunks of 16 B
+            int r = base + cidx / 16;
+            r = r < left ? r : left - 1;
+            pf.k[i] = ld_global_16B(kp_ + (int64_t)r * krs + (cidx % 16) * 8);
+        }
+        {
+            const int dc = tid % 16, kp = tid / 16;  // 8 d values x key pair (2kp, 2kp+1)
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                int r = base + 2 * kp + i;
+                r = r < left ? r : left - 1;
+                pf.v[i] = ld_global_16B(vp_ + (int64_t)r * vrs + dc * 8);
+            }
+        }
+        pf.kpos = 0x7fffffff;
+        if (!s0 && tid < kBN && base + tid < lk2) pf.kpos = pos2p[base + tid];
+    };
+    auto stage = [&](int buf, const Prefetch& pf) {
+        unsigned char* kt = smem + buf * kStageBytes;
+        unsigned char* vt = kt + kKBytes;
+        int* kpos = reinterpret_cast<int*>(vt + kVBytes);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int cidx = tid + kThreads * i;
+            *reinterpret_cast<bf16x8*>(kt + rowmajor128_off(cidx / 16, cidx % 16)) = pf.k[i];
+        }
+        const int dc = tid % 16, kp = tid / 16;
+        const int slot2 = pv_slot(2 * kp);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int d = dc * 8 + i;
+            bf16x2 pr;
+            pr[0] = pf.v[0][i];
+            pr[1] = pf.v[1][i];
+            *reinterpret_cast<bf16x2*>(vt + rowmajor64_off(d, slot2 / 8) + (slot2 % 8) * 2) = pr;
+        }
+        if (tid < kBN) kpos[tid] = pf.kpos;
+    };
+
+    Prefetch pf;
+    if (ntiles > 0) prefetch(0, pf);
+
+    for (int it = 0; it < ntiles; ++it) {
+        const int buf = it & 1;
+        stage(buf, pf);
+        __syncthreads();
+        if (it + 1 < ntiles) prefetch(it + 1, pf);
+
+        const bool first_seg = it < n1;
+        const int base = (first_seg ? it : it - n1) * kBN;
+        // Depth-0 tiles entirely above this wave's rows contribute nothing.
+        if (first_seg && base > wmax1) continue;
+
+        const unsigned char* kt = smem + buf * kStageBytes;
+        const unsigned char* vt = kt + kKBytes;
+        const int* kpos = reinterpret_cast<const int*>(vt + kVBytes);
+
+        // S^T (64 keys x 32 queries) = K Q^T
+        f32x16 sacc[2];
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sacc[mt][r] = 0.f;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt) {
+                const bf16x8 a = *reinterpret_cast<const bf16x8*>(kt + rowmajor128_off(32 * mt + col, 2 * s + half));
+                sacc[mt] = mfma32(a, qf[s], sacc[mt]);
+            }
+        }
+
+        // two-axis mask: only where the tile straddles a query position
+        if (first_seg) {
+            if (base + kBN - 1 > wmin1) {
+#pragma unroll
+                for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int key = base + 32 * mt + acc_row(half, r);
+                        sacc[mt][r] = key <= qlim1 ? sacc[mt][r] : kNegInf;
+                    }
+            }
+        } else {
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int kp = kpos[32 * mt + acc_row(half, r)];
+                    sacc[mt][r] = kp <= qlim2 ? sacc[mt][r] : kNegInf;
+                }
+        }
+
+        // online softmax, one query per lane column (two lanes per query)
+        float mx = kNegInf;
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[mt][r]);
+        mx = wave_max_xor32(mx);
+        const float m_new = fmaxf(m_run, mx);
+        const float m_use = m_new == kNegInf ? 0.f : m_new;
+        const float alpha = fast_exp2((m_run - m_use) * c);
+        m_run = m_new;
+        const float mc = m_use * c;
+        float psum = 0.f;
+        bf16x8 pfrag[4];
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float e = fast_exp2(sacc[mt][r] * c - mc);
+                psum += e;
+                pfrag[2 * mt + r / 8][r % 8] = (__bf16)e;
+            }
+        l_run = l_run * alpha + psum;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+
+        // O^T (128 d x 32 queries) += V^T P^T
+#pragma unroll
+        for (int st = 0; st < 4; ++st) {
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt) {
+                const bf16x8 a = *reinterpret_cast<const bf16x8*>(vt + rowmajor64_off(32 * dt + col, 2 * st + half));
+                oacc[dt] = mfma32(a, pfrag[st], oacc[dt]);
+            }
+        }
+    }
+
+    // ---- epilogue -----------------------------------------------------------
+    const float l_tot = l_run + __shfl_xor(l_run, 32);
+    const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+    if (row_ok) {
+        __bf16* orow = qs.o + (int64_t)row * qs.o_rs + (int64_t)head * qs.o_hs;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                bf16x4 v4;
+#pragma unroll
+                for (int b = 0; b < 4; ++b) v4[b] = (__bf16)(oacc[dt][4 * g4 + b] * inv);
+                *reinterpret_cast<bf16x4*>(orow + 32 * dt + 8 * g4 + 4 * half) = v4;
+            }
+        if (half == 0)
+            qs.lse[(int64_t)head * qs.total_q + row] =
+                l_tot > 0.f ? (m_run * c + fast_log2(l_tot)) * kLn2 : kNegInf;
+    }
+}
+
+FwdStream to_dev(const tah_duo_stream& s) {
+    FwdStream d;
+    d.q = static_cast<const __bf16*>(s.q);
+    d.k = static_cast<const __bf16*>(s.k);
+    d.v = static_cast<const __bf16*>(s.v);
+    d.o = static_cast<__bf16*>(s.o);
+    d.lse = s.lse;
+    d.cu_q = s.cu_q;
+    d.cu_k = s.cu_k;
+    d.pos_q = s.pos_q;
+    d.pos_k = s.pos_k;
+    d.q_rs = s.q_row_stride; d.q_hs = s.q_head_stride;
+    d.k_rs = s.k_row_stride; d.k_hs = s.k_head_stride;
+    d.v_rs = s.v_row_stride; d.v_hs = s.v_head_stride;
+    d.o_rs = s.o_row_stride; d.o_hs = s.o_head_stride;
+    d.total_q = s.total_q;
+    d.total_k = s.total_k;
+    return d;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+int check_stream(const tah_duo_stream& s, bool second) {
+    if (s.total_q < 0 || s.total_k < 0) return TAH_E_SHAPE;
+    if (s.total_q == 0) return TAH_OK;
+    if (!s.q || !s.o || !s.lse || !s.cu_q || !s.cu_k) return TAH_E_NULL;
+    if (s.total_k > 0 && (!s.k || !s.v)) return TAH_E_NULL;
+    if (second && (!s.pos_q || (s.total_k > 0 && !s.pos_k))) return TAH_E_NULL;
+    if (!aligned16(s.q) || !aligned16(s.k) || !aligned16(s.v) || !aligned16(s.o)) return TAH_E_ALIGN;
+    const int64_t st[] = {s.q_row_stride, s.q_head_stride, s.k_row_stride, s.k_head_stride,
+                          s.v_row_stride, s.v_head_stride, s.o_row_stride, s.o_head_stride};
+    for (int64_t x : st)
+        if (x % 8 != 0) return TAH_E_ALIGN;
+    return TAH_OK;
+}
+
+template <int G>
+int launch_fwd(const FwdParams& p, hipStream_t stream) {
+    constexpr int BM = 32 * (8 / G);
+    int tiles = 0;  // upper bound on sum_b ceil(len_b / BM), no device read needed
+    if (p.s1.total_q > 0) tiles += p.s1.total_q / BM + p.nseq;
+    if (p.s2.total_q > 0) tiles += p.s2.total_q / BM + p.nseq;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&duo_fwd_kernel<G>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes) != hipSuccess)
+        return TAH_E_LAUNCH;
+    hipLaunchKernelGGL(duo_fwd_kernel<G>, dim3(p.hkv, tiles), dim3(kThreads), kSmemBytes, stream, p);
+    return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
+}
+
+}  // namespace
+}  // namespace tah
+
+extern "C" int tah_duo_fwd_varlen(const tah_duo_fwd_args* a, tah_stream_t stream) {
+    using namespace tah;
+    if (!a) return TAH_E_NULL;
+    if (a->d != kD || a->nseq < 0 || a->hq <= 0 || a->hkv <= 0 || a->hq % a->hkv != 0) return TAH_E_SHAPE;
+    const int g = a->hq / a->hkv;
+    if (g != 1 && g != 2 && g != 4 && g != 8) return TAH_E_SHAPE;
+    if (int rc = check_stream(a->s1, false)) return rc;
+    if (int rc = check_stream(a->s2, true)) return rc;
+    if (a->s2.total_q > 0 && (!a->s1.cu_k || (a->s1.total_k > 0 && (!a->s1.k || !a->s1.v)))) return TAH_E_NULL;
+    if (a->nseq == 0 || (a->s1.total_q == 0 && a->s2.total_q == 0)) return TAH_OK;
+    FwdParams p;
+    p.s1 = to_dev(a->s1);
+    p.s2 = to_dev(a->s2);
+    p.nseq = a->nseq;
+    p.hq = a->hq;
+    p.hkv = a->hkv;
+    p.scale_log2e = a->scale * kLog2e;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (g) {
+        case 1: return launch_fwd<1>(p, st);
+        case 2: return launch_fwd<2>(p, st);
+        case 4: return launch_fwd<4>(p, st);
+        default: return launch_fwd<8>(p, st);
+    }
+}

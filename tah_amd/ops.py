@@ -1,0 +1,149 @@
+"""Thin torch-facing wrappers over the C ABI (include/tah_duo.h).
+
+Every function here hands raw device pointers, sizes and the current HIP stream
+to libtah_duo.so.  Nothing is computed in Python or by torch operators: torch
+only owns the memory.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional, Tuple
+
+import torch
+
+from . import _capi, _lib
+
+# Set only by the CPU-execution tests, which bind the same prototypes to a host
+# build of the kernels; the product never touches it.
+_HOST_POINTERS_OK = False
+
+
+def _stream(t: torch.Tensor) -> int:
+    if t.is_cuda:
+        return torch.cuda.current_stream(t.device).cuda_stream
+    return 0
+
+
+def _dev_check(*ts: Optional[torch.Tensor]) -> None:
+    dev = None
+    for t in ts:
+        if t is None:
+            continue
+        if not t.is_cuda and not _HOST_POINTERS_OK:
+            raise _capi.TahDuoError("tah_amd ops need CUDA/HIP tensors (no CPU path exists)")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise _capi.TahDuoError(f"tensors on different devices: {dev} vs {t.device}")
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None or t.numel() == 0 else t.data_ptr()
+
+
+def _i32(t: torch.Tensor, name: str) -> torch.Tensor:
+    if t.dtype != torch.int32 or not t.is_contiguous():
+        raise _capi.TahDuoError(f"{name} must be a contiguous int32 tensor")
+    return t
+
+
+def _thd(t: torch.Tensor, name: str) -> torch.Tensor:
+    if t.dim() != 3 or t.dtype != torch.bfloat16:
+        raise _capi.TahDuoError(f"{name} must be a bf16 [rows, heads, head_dim] tensor, got {t.dtype} {tuple(t.shape)}")
+    if t.numel() and t.stride(2) != 1:
+        raise _capi.TahDuoError(f"{name}: head_dim must be contiguous")
+    return t
+
+
+def _fill_stream(s: _capi.DuoStream, q, k, v, o, lse, cu_q, cu_k, pos_q, pos_k) -> None:
+    s.q, s.k, s.v, s.o, s.lse = _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse)
+    s.cu_q, s.cu_k = cu_q.data_ptr(), cu_k.data_ptr()
+    s.pos_q, s.pos_k = _ptr(pos_q), _ptr(pos_k)
+    s.q_row_stride, s.q_head_stride = q.stride(0), q.stride(1)
+    s.k_row_stride, s.k_head_stride = k.stride(0), k.stride(1)
+    s.v_row_stride, s.v_head_stride = v.stride(0), v.stride(1)
+    s.o_row_stride, s.o_head_stride = o.stride(0), o.stride(1)
+    s.total_q, s.total_k = q.shape[0], k.shape[0]
+
+
+def duo_fwd_varlen(q1, k1, v1, cu_q1, cu_k1, q2, k2, v2, pos_q2, pos_k2, cu_q2, cu_k2, scale: float
+                   ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Duo-causal attention forward on packed varlen bf16 tensors.
+
+    q1 [T1q,Hq,D], k1/v1 [T1k,Hkv,D], cu_q1/cu_k1 int32 [nseq+1]: depth-0 stream.
+    q2 [T2q,Hq,D], k2/v2 [T2k,Hkv,D], pos_q2/pos_k2 int32, cu_q2/cu_k2: depth-1 stream
+    (hard tokens).  Returns o1, lse1 [Hq,T1q], o2, lse2 [Hq,T2q].
+    """
+    lib = _lib.lib()
+    for n, t in (("q1", q1), ("k1", k1), ("v1", v1), ("q2", q2), ("k2", k2), ("v2", v2)):
+        _thd(t, n)
+    for n, t in (("cu_q1", cu_q1), ("cu_k1", cu_k1), ("cu_q2", cu_q2), ("cu_k2", cu_k2),
+                 ("pos_q2", pos_q2), ("pos_k2", pos_k2)):
+        _i32(t, n)
+    _dev_check(q1, k1, v1, q2, k2, v2, cu_q1, cu_k1, cu_q2, cu_k2, pos_q2, pos_k2)
+    nseq = cu_q1.numel() - 1
+    if not (cu_k1.numel() == cu_q2.numel() == cu_k2.numel() == nseq + 1):
+        raise _capi.TahDuoError("cu_seqlens tensors must all have nseq+1 entries")
+    if pos_q2.numel() != q2.shape[0] or pos_k2.numel() != k2.shape[0] or k1.shape != v1.shape or k2.shape != v2.shape:
+        raise _capi.TahDuoError("inconsistent row counts")
+    hq, d = q1.shape[1], q1.shape[2]
+    hkv = k1.shape[1]
+    o1 = torch.empty((q1.shape[0], hq, d), dtype=q1.dtype, device=q1.device)
+    o2 = torch.empty((q2.shape[0], hq, d), dtype=q1.dtype, device=q1.device)
+    lse1 = torch.empty((hq, q1.shape[0]), dtype=torch.float32, device=q1.device)
+    lse2 = torch.empty((hq, q2.shape[0]), dtype=torch.float32, device=q1.device)
+    a = _capi.DuoFwdArgs()
+    _fill_stream(a.s1, q1, k1, v1, o1, lse1, cu_q1, cu_k1, None, None)
+    _fill_stream(a.s2, q2, k2, v2, o2, lse2, cu_q2, cu_k2, pos_q2, pos_k2)
+    a.nseq, a.hq, a.hkv, a.d, a.scale = nseq, hq, hkv, d, float(scale)
+    _capi.check(lib, lib.tah_duo_fwd_varlen(ctypes.byref(a), _stream(q1)), "tah_duo_fwd_varlen")
+    return o1, lse1, o2, lse2
+
+
+def hard_index_build(mask: torch.Tensor):
+    """(B, S) bool/uint8 mask -> pos int32 [B*S cap], flat int32, seq int32, cu int32 [B+1].
+
+    Only the first cu[B] entries of pos/flat/seq are defined.  No host sync.
+    """
+    lib = _lib.lib()
+    _dev_check(mask)
+    if mask.dim() != 2 or mask.dtype not in (torch.bool, torch.uint8):
+        raise _capi.TahDuoError("mask must be a (B, S) bool or uint8 tensor")
+    m = mask.contiguous()
+    B, S = m.shape
+    cap = max(B * S, 1)
+    pos = torch.empty(cap, dtype=torch.int32, device=m.device)
+    flat = torch.empty(cap, dtype=torch.int32, device=m.device)
+    seq = torch.empty(cap, dtype=torch.int32, device=m.device)
+    cu = torch.empty(B + 1, dtype=torch.int32, device=m.device)
+    _capi.check(lib, lib.tah_hard_index_build(_ptr(m), B, S, pos.data_ptr(), flat.data_ptr(), seq.data_ptr(),
+                                              cu.data_ptr(), _stream(m)), "tah_hard_index_build")
+    return pos, flat, seq, cu
+
+
+def pad_rows_build(cu: torch.Tensor, seq_of: torch.Tensor, n: int, width: int) -> torch.Tensor:
+    lib = _lib.lib()
+    _dev_check(cu, seq_of)
+    out = torch.empty(max(n, 1), dtype=torch.int32, device=cu.device)
+    _capi.check(lib, lib.tah_pad_rows_build(cu.data_ptr(), seq_of.data_ptr(), n, width, out.data_ptr(), _stream(cu)),
+                "tah_pad_rows_build")
+    return out[:n]
+
+
+def rows_copy(src: torch.Tensor, src_rows: Optional[torch.Tensor], dst: torch.Tensor,
+              dst_rows: Optional[torch.Tensor], n: int) -> None:
+    """dst[dst_rows[r]] = src[src_rows[r]] for r < n; src/dst are [rows, ...] with contiguous rows."""
+    lib = _lib.lib()
+    _dev_check(src, dst, src_rows, dst_rows)
+    if n == 0:
+        return
+    if src.dtype != dst.dtype or src.shape[1:] != dst.shape[1:]:
+        raise _capi.TahDuoError("rows_copy: src and dst rows differ in dtype or shape")
+    for t in (src, dst):
+        if not t[0].is_contiguous():
+            raise _capi.TahDuoError("rows_copy: rows must be contiguous")
+    row_bytes = src[0].numel() * src.element_size()
+    sstride = (src.stride(0) if src.shape[0] > 1 else src[0].numel()) * src.element_size()
+    dstride = (dst.stride(0) if dst.shape[0] > 1 else dst[0].numel()) * dst.element_size()
+    _capi.check(lib, lib.tah_rows_copy(src.data_ptr(), _ptr(src_rows), dst.data_ptr(), _ptr(dst_rows), n, row_bytes,
+                                       sstride, dstride, _stream(src)), "tah_rows_copy")
