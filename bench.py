@@ -1,0 +1,115 @@
+#!/usr/bin/env python3
+"""Benchmark of the duo-causal attention hot path on one MI355X.
+
+A step is one duo-causal prefill forward (both iteration streams, one launch) over
+the BASELINE.json configs[1] workload: batch 4, seq 4096, 16 query heads, 8 kv
+heads, head_dim 128, bf16, 6 % hard tokens, inputs resident in HBM.  The single
+JSON line reports algorithmic TFLOP/s (4*D*Hq*visible_pairs per forward), the
+MFMA roofline fraction of the dominant kernel, and the reference formulation
+(dense additive mask + SDPA, fp32, torch) timed on the host CPU on a bounded
+sample as a baseline.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, vendor figure
+PEAK_HBM_GBS = 8000.0
+
+
+def visible_pairs(case):
+    from oracle.duo_oracle import visible_pairs as vp
+    return vp(case["cu_q1"], case["cu_k1"], case["pos_q2"], case["pos_k2"], case["cu_q2"], case["cu_k2"])
+
+
+def cpu_baseline(seed: int, T: int, p: float, reps: int = 3):
+    """Reference formulation on the host: dense mask + GQA expansion + softmax(QK^T s + M)V, fp32."""
+    import torch
+
+    from oracle import duo_oracle as O
+    from tests.cases import dense_to_varlen, make_dense_case
+
+    c = make_dense_case(seed, B=1, T=T, p_hard=p)
+    for k in ("q1", "k1", "v1", "q2", "k2", "v2"):
+        c[k] = c[k] * 0.5
+    pairs = visible_pairs(dense_to_varlen(c))
+    flops = 4.0 * 128 * 16 * pairs
+    ts = []
+    with torch.no_grad():
+        for _ in range(reps + 1):
+            t0 = time.perf_counter()
+            O.duo_prefill_dense(c["q1"], c["k1"], c["v1"], c["q2"], c["k2"], c["v2"], c["hard"], c["scale"])
+            ts.append(time.perf_counter() - t0)
+    t = sorted(ts[1:])[len(ts[1:]) // 2]
+    return {
+        "value": flops / t / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"1 of 4 sequences (B=1, T={T}, p={p}), fp32 dense mask + SDPA restatement, median of {reps}, "
+                  f"{t * 1e3:.1f} ms, os.cpu_count()={os.cpu_count()}",
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no sharding, no collectives); use --gpus 1", file=sys.stderr)
+        return 2
+
+    import torch
+
+    from tah_amd import ops
+    from tests.cases import make_varlen_case, varlen_args
+    from tests.gpu_util import to_device
+
+    seed, B, T, p = 1235, 4, 4096, 0.06
+    case = make_varlen_case(seed, [T] * B, p, std=0.5)
+    dev = to_device(case)
+    a = varlen_args(dev)
+    pairs = visible_pairs(case)
+    flops = 4.0 * 128 * 16 * pairs
+
+    for _ in range(args.warmup):
+        ops.duo_fwd_varlen(*a)
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()
+    for _ in range(args.steps):
+        ops.duo_fwd_varlen(*a)
+    ev1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms = ev0.elapsed_time(ev1) / args.steps  # events on the stream the kernel is launched on
+    tflops = flops / (ms * 1e-3) / 1e12
+
+    out = {
+        "metric": "duo-causal attn TFLOP/s (% bf16 MFMA peak) prefill; decode HBM GB/s",
+        "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": wall * 1e3 / args.steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "configs[1]: duo-causal prefill forward, B=4, T=4096, Hq=16, Hkv=8, D=128, p_hard=0.06",
+                   "visible_pairs_per_head": pairs, "flop_per_step": flops, "tokens_per_s": B * T / (ms * 1e-3)},
+        "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "duo_fwd_kernel<2>",
+                     "kernel_ms": ms},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(seed, T, p)
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
