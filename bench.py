@@ -56,6 +56,46 @@ def cpu_baseline(seed: int, T: int, p: float, reps: int = 3):
     }
 
 
+def bench_decode(steps: int, warmup: int):
+    """BASELINE configs[2]: one decode step, 64 sequences, context uniform in [1024, 16384], 6 % depth-1 rows."""
+    import torch
+
+    from tah_amd import kv_cache
+    from tests.cases import build_slabs, make_decode_case
+
+    g = torch.Generator().manual_seed(1236)
+    lens = torch.randint(1024, 16385, (64,), generator=g).tolist()
+    c = make_decode_case(1236, lens, 0.06)
+    s1, s2 = build_slabs(c, 16384, 2048, device="cuda")
+    nseq = len(lens)
+    hr = torch.tensor(c["hard_rows"], dtype=torch.int32, device="cuda")
+    slot = torch.cat([torch.arange(nseq, dtype=torch.int32, device="cuda"), hr])
+    qpos1 = torch.from_numpy(c["q_pos"]).cuda()
+    qpos = torch.cat([qpos1, qpos1[hr.long()]])
+    qd = torch.tensor([0] * nseq + [1] * len(hr), dtype=torch.int32, device="cuda")
+    q = torch.cat([c["q1"].cuda(), c["q2"].cuda()])
+    n2 = [int(c["cu_k2"][b + 1] - c["cu_k2"][b]) for b in range(nseq)]
+    rows = sum(lens) + sum(lens[b] + n2[b] for b in c["hard_rows"])
+    nbytes = rows * 2 * 8 * 128 * 2  # K and V, 8 kv heads, 128 bf16
+    run = lambda: kv_cache.decode(q, slot, qpos, s1, s2, scale=c["scale"], q_depth=qd)
+    for _ in range(warmup):
+        run()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        run()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    return {"workload": "configs[2]: decode step, 64 seqs, ctx U[1024,16384], 6% depth-1 rows, Hq=16, Hkv=8, D=128",
+            "ms_per_step": ms, "visible_rows": rows, "algorithmic_bytes": nbytes, "hbm_gbs": gbs,
+            "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
+                         "kernels": "duo_decode_split_kernel<2> + duo_decode_merge_kernel"},
+            "tokens_per_s": nseq / (ms * 1e-3)}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -94,6 +134,8 @@ def main() -> int:
     ms = ev0.elapsed_time(ev1) / args.steps  # events on the stream the kernel is launched on
     tflops = flops / (ms * 1e-3) / 1e12
 
+    extra = {"decode": bench_decode(args.steps, args.warmup)}
+
     out = {
         "metric": "duo-causal attn TFLOP/s (% bf16 MFMA peak) prefill; decode HBM GB/s",
         "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -105,6 +147,7 @@ def main() -> int:
                      "frac": tflops / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "duo_fwd_kernel<2>",
                      "kernel_ms": ms},
     }
+    out["extra"] = extra
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(seed, T, p)
     print(json.dumps(out))

@@ -83,6 +83,72 @@ const char* tah_duo_error_string(int code);
  * o = 0, lse = -inf. */
 int tah_duo_fwd_varlen(const tah_duo_fwd_args* args, tah_stream_t stream);
 
+/* One depth of the native KV cache of one decoder layer.  Each sequence slot s
+ * owns a slab: row j of kv head h lives at
+ *   base + (start[s] + j) * row_stride + h * head_stride      (elements, D contiguous)
+ * which covers both token-major [rows, Hkv, D] slabs and the head-major
+ * [slot, Hkv, capacity, D] layout the decode kernel streams best.  len[s] rows
+ * are in use.  Depth 0 holds every token of the sequence in position order
+ * (position of row j is j); depth 1 holds hard tokens only, with pos[] giving
+ * each row's position.
+ * Replaces the per-(layer, depth) tensors of TaHCache (tah/model/causal_cache.py:43-48). */
+typedef struct tah_kv_segment {
+    void* k;                 /* bf16 */
+    void* v;                 /* bf16 */
+    int32_t* pos;            /* int32 [nslots * capacity], row j of slot s at pos[s*capacity + j]; NULL at depth 0 */
+    const int32_t* start;    /* int32 [nslots] first row of each slab, in rows of row_stride */
+    int32_t* len;            /* int32 [nslots] rows in use */
+    int64_t k_row_stride, k_head_stride, v_row_stride, v_head_stride;
+    int32_t capacity;        /* rows per slab; also the upper bound on len[] used to size grids */
+    int32_t nslots;
+} tah_kv_segment;
+
+typedef struct tah_duo_decode_args {
+    const void* q;           /* bf16 [nq, Hq, D]: one query row per (sequence, depth) being decoded */
+    void* o;                 /* bf16 [nq, Hq, D] */
+    float* lse;              /* f32 [nq, Hq] natural-log normaliser, may be NULL */
+    int64_t q_row_stride, q_head_stride, o_row_stride, o_head_stride;
+    const int32_t* q_slot;   /* int32 [nq] cache slot of each query's sequence */
+    const int32_t* q_pos;    /* int32 [nq] position of each query */
+    const int32_t* q_depth;  /* int32 [nq] 0 or 1; NULL: every query is at `depth` */
+    int32_t depth;
+    tah_kv_segment c1;       /* depth-0 cache, already holding the new token's K/V */
+    tah_kv_segment c2;       /* depth-1 cache; only read by depth-1 queries */
+    void* workspace;         /* >= tah_duo_decode_workspace_bytes(...) bytes, 16-byte aligned */
+    size_t workspace_bytes;
+    int32_t nq, hq, hkv, d;
+    float scale;
+} tah_duo_decode_args;
+
+/* Bytes of split-K scratch tah_duo_decode needs for nq queries. */
+size_t tah_duo_decode_workspace_bytes(int32_t nq, int32_t hq, int32_t capacity1, int32_t capacity2);
+
+/* Decode step of duo-causal attention against the KV cache: every query row
+ * attends to the depth-0 rows of its sequence with index <= q_pos, and, if it
+ * is a depth-1 query, to the depth-1 rows with pos <= q_pos.  Split-K over
+ * 512-row chunks of both segments plus a merge kernel.  Replaces, for Tq == 1:
+ *   TaHForCausalLM._build_attention_mask        tah/model/tah_model.py:744-791
+ *   TaHCache.get_cache_upto_iter (cat it1|it2)   tah/model/causal_cache.py:101-109
+ *   sdpa_attention_forward                       transformers/integrations/sdpa_attention.py:79-166
+ * Queries with no visible row get o = 0, lse = -inf. */
+int tah_duo_decode(const tah_duo_decode_args* args, tah_stream_t stream);
+
+typedef struct tah_kv_append_args {
+    const void* k_new;       /* bf16 [total_new, Hkv, D] */
+    const void* v_new;
+    const int32_t* pos_new;  /* int32 [total_new] or NULL (depth 0) */
+    int64_t k_row_stride, k_head_stride, v_row_stride, v_head_stride;
+    const int32_t* cu_new;   /* int32 [nseq+1]: rows [cu_new[i], cu_new[i+1]) go to slot slot_of[i] */
+    const int32_t* slot_of;  /* int32 [nseq] or NULL (slot i) */
+    int32_t nseq, total_new, hkv, d;
+    tah_kv_segment cache;    /* destination; len[] is advanced by the number of rows appended */
+    int32_t* overflow;       /* optional device flag, set to 1 if a slab would exceed capacity (rows dropped) */
+} tah_kv_append_args;
+
+/* In-place append of new K/V rows (and positions) to the per-sequence slabs.
+ * Replaces the torch.cat growth of TaHCache.update (tah/model/causal_cache.py:84-95). */
+int tah_kv_append(const tah_kv_append_args* args, tah_stream_t stream);
+
 /* Hard-token index build: stream compaction of a (B, S) byte mask in row-major
  * order.  Replaces the stable sort + nonzero of gather_active / scatter_back
  * (tah/model/tah_model.py:111-119, :160-167).  For the r-th True entry, at

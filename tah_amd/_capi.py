@@ -36,10 +36,51 @@ class DuoFwdArgs(C.Structure):
     ]
 
 
+class KvSegment(C.Structure):
+    """``tah_kv_segment``"""
+
+    _fields_ = [
+        ("k", c_void_p), ("v", c_void_p), ("pos", c_void_p), ("start", c_void_p), ("len", c_void_p),
+        ("k_row_stride", c_int64), ("k_head_stride", c_int64), ("v_row_stride", c_int64), ("v_head_stride", c_int64),
+        ("capacity", c_int32), ("nslots", c_int32),
+    ]
+
+
+class DuoDecodeArgs(C.Structure):
+    """``tah_duo_decode_args``"""
+
+    _fields_ = [
+        ("q", c_void_p), ("o", c_void_p), ("lse", c_void_p),
+        ("q_row_stride", c_int64), ("q_head_stride", c_int64), ("o_row_stride", c_int64), ("o_head_stride", c_int64),
+        ("q_slot", c_void_p), ("q_pos", c_void_p), ("q_depth", c_void_p),
+        ("depth", c_int32),
+        ("c1", KvSegment), ("c2", KvSegment),
+        ("workspace", c_void_p), ("workspace_bytes", C.c_size_t),
+        ("nq", c_int32), ("hq", c_int32), ("hkv", c_int32), ("d", c_int32),
+        ("scale", c_float),
+    ]
+
+
+class KvAppendArgs(C.Structure):
+    """``tah_kv_append_args``"""
+
+    _fields_ = [
+        ("k_new", c_void_p), ("v_new", c_void_p), ("pos_new", c_void_p),
+        ("k_row_stride", c_int64), ("k_head_stride", c_int64), ("v_row_stride", c_int64), ("v_head_stride", c_int64),
+        ("cu_new", c_void_p), ("slot_of", c_void_p),
+        ("nseq", c_int32), ("total_new", c_int32), ("hkv", c_int32), ("d", c_int32),
+        ("cache", KvSegment),
+        ("overflow", c_void_p),
+    ]
+
+
 PROTOTYPES = {
     "tah_duo_abi_version": (C.c_int, []),
     "tah_duo_error_string": (C.c_char_p, [C.c_int]),
     "tah_duo_fwd_varlen": (C.c_int, [C.POINTER(DuoFwdArgs), c_void_p]),
+    "tah_duo_decode_workspace_bytes": (C.c_size_t, [c_int32, c_int32, c_int32, c_int32]),
+    "tah_duo_decode": (C.c_int, [C.POINTER(DuoDecodeArgs), c_void_p]),
+    "tah_kv_append": (C.c_int, [C.POINTER(KvAppendArgs), c_void_p]),
     "tah_hard_index_build": (C.c_int, [c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "tah_pad_rows_build": (C.c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_void_p]),
     "tah_rows_copy": (C.c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int64, c_void_p]),

@@ -1,0 +1,390 @@
+// Duo-causal decode step against the KV cache (bandwidth-bound), gfx950.
+//
+// Split-K: one workgroup (4 waves) streams one 512-row chunk of one kv head of
+// one query's sequence, from the depth-0 slab or (depth-1 queries only) the
+// depth-1 slab, for all G = Hq/Hkv query heads at once so K and V are read from
+// HBM exactly once.  A wave covers 128 consecutive rows; each load instruction
+// moves 1 KiB of contiguous cache (4 rows x 256 B, 16 B per lane).  Scores use
+// v_dot2_f32_bf16 on the packed bf16 pairs plus a 16-lane DPP reduction; the
+// online softmax runs per group of 4 rows so the accumulator is rescaled once
+// per 16 rows.  Partial (max, sum, acc) triples go to a workspace and a second
+// small kernel merges the chunks of each query.
+#include <hip/hip_runtime.h>
+
+#include "duo_device.h"
+#include "tah_duo.h"
+
+namespace tah {
+namespace {
+
+constexpr int kD = 128;
+constexpr int kChunk = 512;          // rows per workgroup
+constexpr int kDecThreads = 256;     // 4 waves x 128 rows
+constexpr int kRowsPerWave = kChunk / 4;
+constexpr int kUnroll = 4;           // 4 loads of 4 rows in flight per wave and tensor
+constexpr int kPart = kD + 2;        // acc[128], m, l  (floats per partial)
+
+struct Seg {
+    const __bf16 *k, *v;
+    const int32_t *pos, *start, *len;
+    int64_t k_rs, k_hs, v_rs, v_hs;
+    int32_t capacity;
+};
+struct DecParams {
+    const __bf16* q;
+    __bf16* o;
+    float* lse;
+    int64_t q_rs, q_hs, o_rs, o_hs;
+    const int32_t *q_slot, *q_pos, *q_depth;
+    int32_t depth;
+    Seg c1, c2;
+    float* ws;
+    int32_t nq, hq, hkv, nchunk1, nchunk2;
+    float scale_log2e;
+};
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float x) {
+    return x + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, true));
+}
+// Sum over the 16 lanes of a DPP row; every lane of the row gets the total.
+__device__ __forceinline__ float row16_sum(float x) {
+    x = dpp_add<0xB1>(x);   // quad_perm [1,0,3,2]
+    x = dpp_add<0x4E>(x);   // quad_perm [2,3,0,1]
+    x = dpp_add<0x141>(x);  // row_half_mirror
+    x = dpp_add<0x140>(x);  // row_mirror
+    return x;
+}
+
+// c + a.lo*b.lo + a.hi*b.hi on packed bf16 pairs (v_dot2_f32_bf16).
+__device__ __forceinline__ float dot2_acc(uint32_t a, uint32_t b, float c) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
+}
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __int_as_float((int)(w << 16)); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __int_as_float((int)(w & 0xffff0000u)); }
+
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
+
+// Visible rows of the chunk's segment for this query (0 = nothing to do).
+__device__ __forceinline__ int visible_len(const DecParams& p, bool second, int slot, int qpos, int qdepth) {
+    if (!second) {
+        const int n = p.c1.len[slot];
+        return qpos + 1 < n ? (qpos + 1 > 0 ? qpos + 1 : 0) : n;
+    }
+    return qdepth >= 1 ? p.c2.len[slot] : 0;
+}
+
+template <int G>
+__global__ __launch_bounds__(kDecThreads) void duo_decode_split_kernel(const DecParams p) {
+    __shared__ float red[16][G][kPart];  // one partial per (wave, row group)
+
+    const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+    const int kq = lane / 16, dc = lane % 16;  // row within a 4-row load, 8-element d slice
+    const int chunk = blockIdx.x, qi = blockIdx.y, hk = blockIdx.z;
+    const bool second = chunk >= p.nchunk1;
+    const int cidx = second ? chunk - p.nchunk1 : chunk;
+    const int slot = p.q_slot[qi];
+    const int qpos = p.q_pos[qi];
+    const int qdepth = p.q_depth ? p.q_depth[qi] : p.depth;
+    const int nvis = visible_len(p, second, slot, qpos, qdepth);
+    const int row0 = cidx * kChunk;
+    if (row0 >= nvis) return;  // uniform per workgroup
+    const Seg& sg = second ? p.c2 : p.c1;
+    const int row_end = row0 + kChunk < nvis ? row0 + kChunk : nvis;
+    const int64_t base_row = sg.start[slot];
+    const __bf16* kbase = sg.k + base_row * sg.k_rs + (int64_t)hk * sg.k_hs + dc * 8;
+    const __bf16* vbase = sg.v + base_row * sg.v_rs + (int64_t)hk * sg.v_hs + dc * 8;
+    const int32_t* posbase = second ? sg.pos + (int64_t)slot * sg.capacity : nullptr;
+
+    // query slices: packed bf16 pairs for the dot products
+    u32x4 qv[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+        qv[g] = *reinterpret_cast<const u32x4*>(p.q + (int64_t)qi * p.q_rs + (int64_t)(hk * G + g) * p.q_hs + dc * 8);
+
+    float m_run[G], l_run[G], acc[G][8];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        m_run[g] = kNegInf;
+        l_run[g] = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[g][i] = 0.f;
+    }
+
+    const int wrow0 = row0 + wave * kRowsPerWave;
+    for (int it = 0; it < kRowsPerWave / (4 * kUnroll); ++it) {
+        const int r_it = wrow0 + it * 4 * kUnroll;
+        if (r_it >= row_end) break;  // uniform per wave
+        u32x4 kreg[kUnroll], vreg[kUnroll];
+        int kpos[kUnroll];
+        bool ok[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const int r = r_it + u * 4 + kq;
+            ok[u] = r < row_end;
+            const int rl = ok[u] ? r : row_end - 1;  // keep tail loads inside the slab
+            kreg[u] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)rl * sg.k_rs);
+            vreg[u] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)rl * sg.v_rs);
+            kpos[u] = second ? posbase[rl] : 0;
+        }
+        float s[kUnroll][G];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const bool vis = ok[u] && (!second || kpos[u] <= qpos);
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                float d = 0.f;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    d = dot2_acc(kreg[u][i], qv[g][i], d);
+                d = row16_sum(d) * p.scale_log2e;
+                s[u][g] = vis ? d : kNegInf;
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            float mx = m_run[g];
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) mx = fmaxf(mx, s[u][g]);
+            const float m_use = mx == kNegInf ? 0.f : mx;
+            const float alpha = fast_exp2(m_run[g] - m_use);
+            m_run[g] = mx;
+            float pr[kUnroll], psum = 0.f;
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                pr[u] = fast_exp2(s[u][g] - m_use);
+                psum += pr[u];
+            }
+            l_run[g] = l_run[g] * alpha + psum;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[g][i] *= alpha;
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    acc[g][2 * i] += pr[u] * bf16_lo(vreg[u][i]);
+                    acc[g][2 * i + 1] += pr[u] * bf16_hi(vreg[u][i]);
+                }
+        }
+    }
+
+    // ---- merge the 16 (wave, row group) partials of this workgroup ----------
+    const int grp = wave * 4 + kq;
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) red[grp][g][dc * 8 + i] = acc[g][i];
+        if (dc == 0) {
+            red[grp][g][kD] = m_run[g];
+            red[grp][g][kD + 1] = l_run[g];
+        }
+    }
+    __syncthreads();
+    const int nslots = p.nchunk1 + p.nchunk2;
+    for (int e = tid; e < G * kD; e += kDecThreads) {
+        const int g = e / kD, d = e % kD;
+        float mx = kNegInf;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) mx = fmaxf(mx, red[j][g][kD]);
+        const float m_use = mx == kNegInf ? 0.f : mx;
+        float a = 0.f, l = 0.f;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const float w = fast_exp2(red[j][g][kD] - m_use);
+            a += w * red[j][g][d];
+            l += w * red[j][g][kD + 1];
+        }
+        float* out = p.ws + ((int64_t)(qi * p.hq + hk * G + g) * nslots + chunk) * kPart;
+        out[d] = a;
+        if (d == 0) {
+            out[kD] = mx;
+            out[kD + 1] = l;
+        }
+    }
+}
+
+// One workgroup of 128 threads per (query, head): merge the chunk partials.
+__global__ __launch_bounds__(kD) void duo_decode_merge_kernel(const DecParams p) {
+    const int qi = blockIdx.x, head = blockIdx.y, d = threadIdx.x;
+    const int slot = p.q_slot[qi];
+    const int qpos = p.q_pos[qi];
+    const int qdepth = p.q_depth ? p.q_depth[qi] : p.depth;
+    const int n1 = (visible_len(p, false, slot, qpos, qdepth) + kChunk - 1) / kChunk;
+    const int n2 = (visible_len(p, true, slot, qpos, qdepth) + kChunk - 1) / kChunk;
+    const int nslots = p.nchunk1 + p.nchunk2;
+    const float* part = p.ws + (int64_t)(qi * p.hq + head) * nslots * kPart;
+    float mx = kNegInf;
+    for (int c = 0; c < n1; ++c) mx = fmaxf(mx, part[(int64_t)c * kPart + kD]);
+    for (int c = 0; c < n2; ++c) mx = fmaxf(mx, part[(int64_t)(p.nchunk1 + c) * kPart + kD]);
+    const float m_use = mx == kNegInf ? 0.f : mx;
+    float a = 0.f, l = 0.f;
+    for (int c = 0; c < n1 + n2; ++c) {
+        const float* pc = part + (int64_t)(c < n1 ? c : p.nchunk1 + (c - n1)) * kPart;
+        const float w = fast_exp2(pc[kD] - m_use);
+        a += w * pc[d];
+        l += w * pc[kD + 1];
+    }
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    p.o[(int64_t)qi * p.o_rs + (int64_t)head * p.o_hs + d] = (__bf16)(a * inv);
+    if (p.lse && d == 0) p.lse[(int64_t)qi * p.hq + head] = l > 0.f ? (mx + fast_log2(l)) * kLn2 : kNegInf;
+}
+
+// ---- KV append --------------------------------------------------------------
+struct AppendParams {
+    const __bf16 *k_new, *v_new;
+    const int32_t *pos_new, *cu_new, *slot_of;
+    int64_t kn_rs, kn_hs, vn_rs, vn_hs;
+    __bf16 *ck, *cv;
+    int32_t* cpos;
+    const int32_t* start;
+    int32_t* len;
+    int64_t ck_rs, ck_hs, cv_rs, cv_hs;
+    int32_t capacity, nseq, hkv;
+    int32_t* overflow;
+};
+
+// grid (rows, kv heads), 32 threads: one 256-byte K row and V row per workgroup.
+__global__ void kv_append_rows_kernel(const AppendParams a) {
+    const int r = blockIdx.x, h = blockIdx.y, t = threadIdx.x;
+    int seq = 0;  // sequence of new row r
+    for (int b = 0; b < a.nseq; ++b)
+        if (r >= a.cu_new[b + 1]) seq = b + 1;
+    if (seq >= a.nseq) return;
+    const int slot = a.slot_of ? a.slot_of[seq] : seq;
+    const int dst = a.len[slot] + (r - a.cu_new[seq]);
+    if (dst >= a.capacity) {
+        if (a.overflow && t == 0 && h == 0) *a.overflow = 1;
+        return;
+    }
+    const int64_t drow = (int64_t)a.start[slot] + dst;
+    if (t < 16) {
+        *reinterpret_cast<bf16x8*>(a.ck + drow * a.ck_rs + (int64_t)h * a.ck_hs + t * 8) =
+            *reinterpret_cast<const bf16x8*>(a.k_new + (int64_t)r * a.kn_rs + (int64_t)h * a.kn_hs + t * 8);
+    } else {
+        const int u = t - 16;
+        *reinterpret_cast<bf16x8*>(a.cv + drow * a.cv_rs + (int64_t)h * a.cv_hs + u * 8) =
+            *reinterpret_cast<const bf16x8*>(a.v_new + (int64_t)r * a.vn_rs + (int64_t)h * a.vn_hs + u * 8);
+    }
+    if (a.cpos && a.pos_new && h == 0 && t == 0) a.cpos[(int64_t)slot * a.capacity + dst] = a.pos_new[r];
+}
+
+// Runs after the row copies on the same stream: advance the slab lengths.
+__global__ void kv_append_len_kernel(const AppendParams a) {
+    const int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= a.nseq) return;
+    const int slot = a.slot_of ? a.slot_of[b] : b;
+    const int n = a.len[slot] + (a.cu_new[b + 1] - a.cu_new[b]);
+    a.len[slot] = n < a.capacity ? n : a.capacity;
+}
+
+Seg to_seg(const tah_kv_segment& s) {
+    Seg d;
+    d.k = static_cast<const __bf16*>(s.k);
+    d.v = static_cast<const __bf16*>(s.v);
+    d.pos = s.pos;
+    d.start = s.start;
+    d.len = s.len;
+    d.k_rs = s.k_row_stride; d.k_hs = s.k_head_stride;
+    d.v_rs = s.v_row_stride; d.v_hs = s.v_head_stride;
+    d.capacity = s.capacity;
+    return d;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+int check_seg(const tah_kv_segment& s, bool need_pos) {
+    if (s.capacity < 0 || s.nslots < 0) return TAH_E_SHAPE;
+    if (s.capacity == 0) return TAH_OK;
+    if (!s.k || !s.v || !s.start || !s.len || (need_pos && !s.pos)) return TAH_E_NULL;
+    if (!aligned16(s.k) || !aligned16(s.v)) return TAH_E_ALIGN;
+    if (s.k_row_stride % 8 || s.k_head_stride % 8 || s.v_row_stride % 8 || s.v_head_stride % 8) return TAH_E_ALIGN;
+    return TAH_OK;
+}
+
+template <int G>
+int launch_decode(const DecParams& p, hipStream_t st) {
+    hipLaunchKernelGGL(duo_decode_split_kernel<G>, dim3(p.nchunk1 + p.nchunk2, p.nq, p.hkv), dim3(kDecThreads), 0, st, p);
+    hipLaunchKernelGGL(duo_decode_merge_kernel, dim3(p.nq, p.hq), dim3(kD), 0, st, p);
+    return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
+}
+
+}  // namespace
+}  // namespace tah
+
+extern "C" size_t tah_duo_decode_workspace_bytes(int32_t nq, int32_t hq, int32_t capacity1, int32_t capacity2) {
+    using namespace tah;
+    if (nq <= 0 || hq <= 0 || capacity1 < 0 || capacity2 < 0) return 0;
+    const size_t chunks = (size_t)(capacity1 + kChunk - 1) / kChunk + (size_t)(capacity2 + kChunk - 1) / kChunk;
+    return (size_t)nq * hq * chunks * kPart * sizeof(float);
+}
+
+extern "C" int tah_duo_decode(const tah_duo_decode_args* a, tah_stream_t stream) {
+    using namespace tah;
+    if (!a) return TAH_E_NULL;
+    if (a->d != kD || a->nq < 0 || a->hq <= 0 || a->hkv <= 0 || a->hq % a->hkv) return TAH_E_SHAPE;
+    const int g = a->hq / a->hkv;
+    if (g != 1 && g != 2 && g != 4) return TAH_E_SHAPE;  // merge buffer for 8 heads would not fit static LDS
+    if (a->nq == 0) return TAH_OK;
+    if (a->nq > 65535 || a->hkv > 65535) return TAH_E_SHAPE;
+    if (!a->q || !a->o || !a->q_slot || !a->q_pos || !a->workspace) return TAH_E_NULL;
+    if (!aligned16(a->q) || !aligned16(a->workspace) || a->q_row_stride % 8 || a->q_head_stride % 8) return TAH_E_ALIGN;
+    if (int rc = check_seg(a->c1, false)) return rc;
+    const bool any_depth1 = a->q_depth != nullptr || a->depth >= 1;
+    if (any_depth1)
+        if (int rc = check_seg(a->c2, true)) return rc;
+    const int cap2 = any_depth1 ? a->c2.capacity : 0;
+    if (a->workspace_bytes < tah_duo_decode_workspace_bytes(a->nq, a->hq, a->c1.capacity, cap2)) return TAH_E_WORKSPACE;
+    DecParams p;
+    p.q = static_cast<const __bf16*>(a->q);
+    p.o = static_cast<__bf16*>(a->o);
+    p.lse = a->lse;
+    p.q_rs = a->q_row_stride; p.q_hs = a->q_head_stride;
+    p.o_rs = a->o_row_stride; p.o_hs = a->o_head_stride;
+    p.q_slot = a->q_slot; p.q_pos = a->q_pos; p.q_depth = a->q_depth;
+    p.depth = a->depth;
+    p.c1 = to_seg(a->c1);
+    p.c2 = to_seg(a->c2);
+    p.ws = static_cast<float*>(a->workspace);
+    p.nq = a->nq; p.hq = a->hq; p.hkv = a->hkv;
+    p.nchunk1 = (a->c1.capacity + kChunk - 1) / kChunk;
+    p.nchunk2 = (cap2 + kChunk - 1) / kChunk;
+    p.scale_log2e = a->scale * kLog2e;
+    if (p.nchunk1 + p.nchunk2 == 0) return TAH_E_SHAPE;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (g) {
+        case 1: return launch_decode<1>(p, st);
+        case 2: return launch_decode<2>(p, st);
+        default: return launch_decode<4>(p, st);
+    }
+}
+
+extern "C" int tah_kv_append(const tah_kv_append_args* a, tah_stream_t stream) {
+    using namespace tah;
+    if (!a) return TAH_E_NULL;
+    if (a->d != kD || a->nseq < 0 || a->total_new < 0 || a->hkv <= 0 || a->hkv > 65535) return TAH_E_SHAPE;
+    if (a->nseq == 0 || a->total_new == 0) return TAH_OK;
+    if (!a->k_new || !a->v_new || !a->cu_new) return TAH_E_NULL;
+    if (int rc = check_seg(a->cache, a->pos_new != nullptr)) return rc;
+    if (a->cache.capacity == 0) return TAH_E_SHAPE;
+    if (!aligned16(a->k_new) || !aligned16(a->v_new) || a->k_row_stride % 8 || a->k_head_stride % 8 ||
+        a->v_row_stride % 8 || a->v_head_stride % 8)
+        return TAH_E_ALIGN;
+    AppendParams p;
+    p.k_new = static_cast<const __bf16*>(a->k_new);
+    p.v_new = static_cast<const __bf16*>(a->v_new);
+    p.pos_new = a->pos_new; p.cu_new = a->cu_new; p.slot_of = a->slot_of;
+    p.kn_rs = a->k_row_stride; p.kn_hs = a->k_head_stride; p.vn_rs = a->v_row_stride; p.vn_hs = a->v_head_stride;
+    p.ck = static_cast<__bf16*>(a->cache.k);
+    p.cv = static_cast<__bf16*>(a->cache.v);
+    p.cpos = a->cache.pos;
+    p.start = a->cache.start;
+    p.len = a->cache.len;
+    p.ck_rs = a->cache.k_row_stride; p.ck_hs = a->cache.k_head_stride;
+    p.cv_rs = a->cache.v_row_stride; p.cv_hs = a->cache.v_head_stride;
+    p.capacity = a->cache.capacity; p.nseq = a->nseq; p.hkv = a->hkv;
+    p.overflow = a->overflow;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(kv_append_rows_kernel, dim3(a->total_new, a->hkv), dim3(32), 0, st, p);
+    hipLaunchKernelGGL(kv_append_len_kernel, dim3((a->nseq + 63) / 64), dim3(64), 0, st, p);
+    return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
+}

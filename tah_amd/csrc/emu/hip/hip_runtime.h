@@ -225,6 +225,30 @@ inline emu_f32x4 emu_mfma_16x16x32_bf16(emu_bf16x8 a, emu_bf16x8 b, emu_f32x4 c,
 #define __builtin_amdgcn_mfma_f32_32x32x16_bf16 emu_mfma_32x32x16_bf16
 #define __builtin_amdgcn_mfma_f32_16x16x32_bf16 emu_mfma_16x16x32_bf16
 
+// v_dot2_f32_bf16 on the raw 32-bit pairs (4-byte bf16 vectors are not passed reliably by value on the host ABI).
+inline float emu_bf16_bits(uint32_t hi16) { float f; uint32_t w = hi16 << 16; memcpy(&f, &w, 4); return f; }
+inline float emu_fdot2_bits(uint32_t a, uint32_t b, float c) {
+    return c + emu_bf16_bits(a & 0xffffu) * emu_bf16_bits(b & 0xffffu) + emu_bf16_bits(a >> 16) * emu_bf16_bits(b >> 16);
+}
+#define __builtin_amdgcn_fdot2_f32_bf16(a, b, c, clamp) \
+    emu_fdot2_bits(__builtin_bit_cast(uint32_t, (a)), __builtin_bit_cast(uint32_t, (b)), (c))
+inline int __float_as_int(float x) { int i; memcpy(&i, &x, 4); return i; }
+inline float __int_as_float(int i) { float x; memcpy(&x, &i, 4); return x; }
+// DPP lane selects used by the kernels: quad_perm, row_shl/shr, row_mirror, row_half_mirror.
+inline int emu_update_dpp(int old, int src, int ctrl, int, int, bool bound_ctrl) {
+    const int l = emu::t_lane, row = l & ~15, i = l & 15;
+    int from = -1;
+    if (ctrl < 0x100) from = (l & ~3) + ((ctrl >> (2 * (l & 3))) & 3);
+    else if (ctrl >= 0x101 && ctrl <= 0x10f) { int j = i + (ctrl & 15); from = j < 16 ? row + j : -1; }
+    else if (ctrl >= 0x111 && ctrl <= 0x11f) { int j = i - (ctrl & 15); from = j >= 0 ? row + j : -1; }
+    else if (ctrl == 0x140) from = row + 15 - i;
+    else if (ctrl == 0x141) from = row + (i & 8) + 7 - (i & 7);
+    else { fprintf(stderr, "emu: unsupported dpp_ctrl 0x%x\n", ctrl); abort(); }
+    const int got = emu::exchange(src, from < 0 ? l : from);
+    return from < 0 ? (bound_ctrl ? 0 : old) : got;
+}
+#define __builtin_amdgcn_update_dpp emu_update_dpp
+
 #define __builtin_amdgcn_exp2f(x) exp2f(x)
 #define __builtin_amdgcn_logf(x) log2f(x)
 #define __builtin_amdgcn_rcpf(x) (1.0f / (x))

@@ -84,3 +84,42 @@ def dense_to_varlen(c):
         q2=tok(c["q2"])[sel2], k2=tok(c["k2"])[sel2], v2=tok(c["v2"])[sel2],
         pos_q2=p2, pos_k2=p2, cu_q2=cu2, cu_k2=cu2, scale=c["scale"],
     )
+
+
+def make_decode_case(seed, lens, p_hard, Hq=16, Hkv=8, D=128, hard_new=None, std=1.0):
+    """Decode-step inputs: packed depth-0 cache (every position, new token included), depth-1 cache
+    (a Bernoulli(p_hard) subset of the positions, new token included when hard_new[b]), one depth-0
+    query per sequence and one depth-1 query per hard sequence.  All float tensors bf16-representable."""
+    g = torch.Generator().manual_seed(seed)
+    rn = lambda *s: (torch.randn(*s, generator=g) * std).to(torch.bfloat16)
+    lens = list(lens)
+    nseq = len(lens)
+    cu1 = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    k1, v1 = rn(int(cu1[-1]), Hkv, D), rn(int(cu1[-1]), Hkv, D)
+    if hard_new is None:
+        hard_new = (torch.rand(nseq, generator=g) < p_hard).tolist()
+    pos2, cu2 = [], [0]
+    for b, L in enumerate(lens):
+        h = torch.rand(L, generator=g) < p_hard
+        h[L - 1] = bool(hard_new[b])
+        pos2 += torch.nonzero(h).flatten().tolist()
+        cu2.append(len(pos2))
+    k2, v2 = rn(len(pos2), Hkv, D), rn(len(pos2), Hkv, D)
+    q1 = rn(nseq, Hq, D)
+    hard_rows = [b for b in range(nseq) if hard_new[b]]
+    q2 = rn(len(hard_rows), Hq, D)
+    return dict(lens=lens, k1=k1, v1=v1, cu_k1=cu1, k2=k2, v2=v2, pos_k2=np.asarray(pos2, dtype=np.int32),
+                cu_k2=np.asarray(cu2, dtype=np.int32), q1=q1, q2=q2, hard_rows=hard_rows,
+                q_pos=np.asarray([L - 1 for L in lens], dtype=np.int32), scale=float(D) ** -0.5)
+
+
+def build_slabs(c, capacity1, capacity2, device="cpu"):
+    from tah_amd.kv_cache import KvSlabs
+    hkv = c["k1"].shape[1]
+    nseq = len(c["lens"])
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)
+    s1 = KvSlabs(nseq, capacity1, hkv, with_pos=False, device=device)
+    s2 = KvSlabs(nseq, capacity2, hkv, with_pos=True, device=device)
+    s1.append(c["k1"].to(device), c["v1"].to(device), t(c["cu_k1"]))
+    s2.append(c["k2"].to(device), c["v2"].to(device), t(c["cu_k2"]), pos_new=t(c["pos_k2"]))
+    return s1, s2
