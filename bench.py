@@ -96,6 +96,47 @@ def bench_decode(steps: int, warmup: int):
             "tokens_per_s": nseq / (ms * 1e-3)}
 
 
+def bench_fwd_bwd(name: str, seqlens, p_hard: float, seed: int, steps: int, warmup: int):
+    """Training forward+backward of duo-causal attention on one packed varlen batch."""
+    import torch
+
+    from tah_amd import ops
+    from tests.cases import make_varlen_case, varlen_args
+    from tests.gpu_util import to_device
+
+    case = make_varlen_case(seed, seqlens, p_hard, std=0.5)
+    dev = to_device(case)
+    a = varlen_args(dev)
+    g = torch.Generator().manual_seed(seed + 1)
+    do1 = torch.randn(dev["q1"].shape, generator=g).to(torch.bfloat16).cuda()
+    do2 = torch.randn(dev["q2"].shape, generator=g).to(torch.bfloat16).cuda()
+    pairs = visible_pairs(case)
+    fwd_flops = 4.0 * 128 * 16 * pairs
+
+    def step():
+        o1, lse1, o2, lse2 = ops.duo_fwd_varlen(*a)
+        ops.duo_bwd_varlen(dev["q1"], dev["k1"], dev["v1"], o1, lse1, do1, dev["cu_q1"], dev["cu_k1"],
+                           dev["q2"], dev["k2"], dev["v2"], o2, lse2, do2, dev["pos_q2"], dev["pos_k2"],
+                           dev["cu_q2"], dev["cu_k2"], dev["scale"])
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    tf = 3.5 * fwd_flops / (ms * 1e-3) / 1e12
+    return {"workload": name, "ms_per_step": ms, "visible_pairs_per_head": pairs, "flop_per_step": 3.5 * fwd_flops,
+            "tflops": tf, "roofline": {"bound": "mfma", "achieved": tf, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                                       "frac": tf / PEAK_BF16_TFLOPS,
+                                       "kernels": "duo_fwd_kernel + duo_bwd_delta/dq/dkdv kernels"},
+            "tokens_per_s": sum(seqlens) / (ms * 1e-3)}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -135,6 +176,12 @@ def main() -> int:
     tflops = flops / (ms * 1e-3) / 1e12
 
     extra = {"decode": bench_decode(args.steps, args.warmup)}
+    extra["fwd_bwd_seq8192_p06"] = bench_fwd_bwd(
+        "north-star headline: fwd+bwd, one sequence of 8192, p_hard=0.06, Hq=16, Hkv=8, D=128", [8192], 0.06, 1238,
+        max(args.steps // 2, 1), max(args.warmup // 2, 1))
+    extra["fwd_bwd_4docs_p10"] = bench_fwd_bwd(
+        "configs[3]: fwd+bwd, 8192 packed tokens in 4 documents, p_hard=0.10", [1397, 3210, 2561, 1024], 0.10, 1237,
+        max(args.steps // 2, 1), max(args.warmup // 2, 1))
 
     out = {
         "metric": "duo-causal attn TFLOP/s (% bf16 MFMA peak) prefill; decode HBM GB/s",

@@ -83,6 +83,32 @@ const char* tah_duo_error_string(int code);
  * o = 0, lse = -inf. */
 int tah_duo_fwd_varlen(const tah_duo_fwd_args* args, tah_stream_t stream);
 
+/* Gradient tensors of one stream (same row/head layout as the forward tensors). */
+typedef struct tah_duo_bwd_stream {
+    const void* d_o;        /* bf16 [total_q, Hq,  D] upstream gradient of o */
+    void* dq;               /* bf16 [total_q, Hq,  D] */
+    void* dk;               /* bf16 [total_k, Hkv, D] */
+    void* dv;               /* bf16 [total_k, Hkv, D] */
+    float* delta;           /* f32  [Hq, total_q] scratch (rowsum(dO*O)), written by the call */
+    int64_t do_row_stride, do_head_stride;
+    int64_t dq_row_stride, dq_head_stride;
+    int64_t dk_row_stride, dk_head_stride;
+    int64_t dv_row_stride, dv_head_stride;
+} tah_duo_bwd_stream;
+
+typedef struct tah_duo_bwd_args {
+    tah_duo_fwd_args fwd;   /* the forward call's tensors; o and lse are inputs here */
+    tah_duo_bwd_stream g1;  /* depth 0 */
+    tah_duo_bwd_stream g2;  /* depth 1 */
+} tah_duo_bwd_args;
+
+/* Backward of tah_duo_fwd_varlen: dQ, dK, dV of both depths.  Replaces torch
+ * autograd through SDPA + torch.cat + repeat_kv on this path; the reference
+ * keeps cached K/V attached to the graph (tah/model/causal_cache.py:92-93), so
+ * depth-0 dK/dV collect the contributions of depth-0 and depth-1 queries, summed
+ * over the query heads of each kv head.  Deterministic (no atomics). */
+int tah_duo_bwd_varlen(const tah_duo_bwd_args* args, tah_stream_t stream);
+
 /* One depth of the native KV cache of one decoder layer.  Each sequence slot s
  * owns a slab: row j of kv head h lives at
  *   base + (start[s] + j) * row_stride + h * head_stride      (elements, D contiguous)

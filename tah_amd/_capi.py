@@ -36,6 +36,24 @@ class DuoFwdArgs(C.Structure):
     ]
 
 
+class DuoBwdStream(C.Structure):
+    """``tah_duo_bwd_stream``"""
+
+    _fields_ = [
+        ("d_o", c_void_p), ("dq", c_void_p), ("dk", c_void_p), ("dv", c_void_p), ("delta", c_void_p),
+        ("do_row_stride", c_int64), ("do_head_stride", c_int64),
+        ("dq_row_stride", c_int64), ("dq_head_stride", c_int64),
+        ("dk_row_stride", c_int64), ("dk_head_stride", c_int64),
+        ("dv_row_stride", c_int64), ("dv_head_stride", c_int64),
+    ]
+
+
+class DuoBwdArgs(C.Structure):
+    """``tah_duo_bwd_args``"""
+
+    _fields_ = [("fwd", DuoFwdArgs), ("g1", DuoBwdStream), ("g2", DuoBwdStream)]
+
+
 class KvSegment(C.Structure):
     """``tah_kv_segment``"""
 
@@ -78,6 +96,7 @@ PROTOTYPES = {
     "tah_duo_abi_version": (C.c_int, []),
     "tah_duo_error_string": (C.c_char_p, [C.c_int]),
     "tah_duo_fwd_varlen": (C.c_int, [C.POINTER(DuoFwdArgs), c_void_p]),
+    "tah_duo_bwd_varlen": (C.c_int, [C.POINTER(DuoBwdArgs), c_void_p]),
     "tah_duo_decode_workspace_bytes": (C.c_size_t, [c_int32, c_int32, c_int32, c_int32]),
     "tah_duo_decode": (C.c_int, [C.POINTER(DuoDecodeArgs), c_void_p]),
     "tah_kv_append": (C.c_int, [C.POINTER(KvAppendArgs), c_void_p]),

@@ -1,0 +1,563 @@
+// Duo-causal attention backward (training), bf16 MFMA, gfx950.
+//
+// Three kernels, no atomics, deterministic:
+//   delta     delta[h][row] = sum_d dO*O                                (fp32)
+//   dq        one workgroup per query tile, same tiling as the forward:
+//             S^T = K Q^T, dP^T = V dO^T, dS^T = P^T o (dP^T - delta),
+//             dQ^T += K^T dS^T  (K^T operand via LDS transpose reads)
+//   dkdv      one workgroup (4 waves) per 64-key tile of one kv head; loops
+//             over every query tile that can see it, for all query heads of
+//             the group and for both query streams (depth-0 keys collect
+//             gradient from depth-0 and depth-1 queries):
+//             S = Q K^T, dP = dO V^T, dV += P^T dO, dK += dS^T Q
+// P is recomputed from the saved log-sum-exp.  In dkdv each lane owns one key
+// (accumulator column) and K/V fragments stay in registers for the whole
+// workgroup; Q and dO tiles are staged in LDS and read both row-wise (A
+// operand) and, through ds_read_b64_tr_b16, column-wise (B operand).
+#include <hip/hip_runtime.h>
+
+#include "duo_device.h"
+#include "tah_duo.h"
+
+namespace tah {
+namespace {
+
+constexpr int kD = 128;
+constexpr int kBN = 64;
+constexpr int kTileBytes = kBN * kD * 2;  // one 64 x 128 bf16 tile
+
+struct BwdStream {
+    const __bf16 *q, *k, *v, *o, *d_o;
+    __bf16 *dq, *dk, *dv;
+    const float* lse;
+    float* delta;
+    const int32_t *cu_q, *cu_k, *pos_q, *pos_k;
+    int64_t q_rs, q_hs, k_rs, k_hs, v_rs, v_hs, o_rs, o_hs;
+    int64_t do_rs, do_hs, dq_rs, dq_hs, dk_rs, dk_hs, dv_rs, dv_hs;
+    int32_t total_q, total_k;
+};
+struct BwdParams {
+    BwdStream s1, s2;
+    int32_t nseq, hq, hkv;
+    float scale, scale_log2e;
+};
+
+// ---------------------------------------------------------------------------
+// delta = rowsum(dO * O): 16 lanes per (row, head), 8 elements each
+// ---------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float x) {
+    return x + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, true));
+}
+
+__global__ __launch_bounds__(256) void duo_bwd_delta_kernel(const BwdStream s, int hq) {
+    const int64_t item = (int64_t)blockIdx.x * 16 + threadIdx.x / 16;  // (row, head) pair
+    const int dc = threadIdx.x % 16;
+    const int64_t total = (int64_t)s.total_q * hq;
+    const int64_t it = item < total ? item : total - 1;
+    const int row = (int)(it / hq), head = (int)(it % hq);
+    const bf16x8 a = ld_global_16B(s.o + (int64_t)row * s.o_rs + (int64_t)head * s.o_hs + dc * 8);
+    const bf16x8 b = ld_global_16B(s.d_o + (int64_t)row * s.do_rs + (int64_t)head * s.do_hs + dc * 8);
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc += (float)a[i] * (float)b[i];
+    acc = dpp_add<0xB1>(acc);
+    acc = dpp_add<0x4E>(acc);
+    acc = dpp_add<0x141>(acc);
+    acc = dpp_add<0x140>(acc);
+    if (dc == 0 && item < total) s.delta[(int64_t)head * s.total_q + row] = acc;
+}
+
+// ---------------------------------------------------------------------------
+// dQ kernel
+// ---------------------------------------------------------------------------
+constexpr int kDqThreads = 512;
+constexpr int kDqStage = 2 * kTileBytes + kBN * 4;   // K tile, V tile, key positions
+constexpr int kDqSmem = 2 * kDqStage + 64;
+
+struct KvPrefetch {
+    bf16x8 k[2], v[2];
+    int kpos;
+};
+
+template <int G>
+__global__ __launch_bounds__(kDqThreads) void duo_bwd_dq_kernel(const BwdParams p) {
+    constexpr int BM = 32 * (8 / G);
+    HIP_DYNAMIC_SHARED(unsigned char, smem)
+    const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+    const int half = lane / 32, col = lane % 32;
+    const int hk = blockIdx.x;
+
+    int slot = (int)(gridDim.y - 1 - blockIdx.y);
+    int seq = 0, row0 = 0, row_end = 0;
+    bool second = false;
+    if (!(p.s1.total_q > 0 && find_tile(p.s1.cu_q, p.nseq, BM, slot, seq, row0, row_end))) {
+        if (!(p.s2.total_q > 0 && find_tile(p.s2.cu_q, p.nseq, BM, slot, seq, row0, row_end))) return;
+        second = true;
+    }
+    const BwdStream& qs = second ? p.s2 : p.s1;
+    const int head = hk * G + wave % G;
+    const int rblk = wave / G;
+    const int k1_lo = p.s1.cu_k[seq];
+    const int lk1 = p.s1.cu_k[seq + 1] - k1_lo;
+    const __bf16* k1p = p.s1.k + (int64_t)k1_lo * p.s1.k_rs + (int64_t)hk * p.s1.k_hs;
+    const __bf16* v1p = p.s1.v + (int64_t)k1_lo * p.s1.v_rs + (int64_t)hk * p.s1.v_hs;
+    const int left1 = p.s1.total_k - k1_lo;
+    int lk2 = 0, left2 = 0;
+    const __bf16 *k2p = nullptr, *v2p = nullptr;
+    const int32_t* pos2p = nullptr;
+    if (second) {
+        const int k2_lo = p.s2.cu_k[seq];
+        lk2 = p.s2.cu_k[seq + 1] - k2_lo;
+        k2p = p.s2.k + (int64_t)k2_lo * p.s2.k_rs + (int64_t)hk * p.s2.k_hs;
+        v2p = p.s2.v + (int64_t)k2_lo * p.s2.v_rs + (int64_t)hk * p.s2.v_hs;
+        pos2p = p.s2.pos_k + k2_lo;
+        left2 = p.s2.total_k - k2_lo;
+    }
+
+    const int row = row0 + rblk * 32 + col;
+    const bool row_ok = row < row_end;
+    const int row_ld = row_ok ? row : row_end - 1;
+    int qpos;
+    if (second) {
+        qpos = qs.pos_q[row_ld];
+    } else {
+        const int q_lo = qs.cu_q[seq];
+        qpos = (row_ld - q_lo) + (lk1 - (qs.cu_q[seq + 1] - q_lo));
+    }
+    const int qlim1 = row_ok ? (qpos < lk1 - 1 ? qpos : lk1 - 1) : -1;
+    const int qlim2 = row_ok ? qpos : -1;
+    const int wmax1 = wave_reduce_max(qlim1);
+    const int wmin1 = wave_reduce_min(row_ok ? qlim1 : 0x7fffffff);
+    int* bounds = reinterpret_cast<int*>(smem + 2 * kDqStage);
+    if (lane == 0) bounds[wave] = wmax1;
+    __syncthreads();
+    int tmax1 = -1;
+#pragma unroll
+    for (int w = 0; w < 8; ++w) tmax1 = bounds[w] > tmax1 ? bounds[w] : tmax1;
+    const int n1 = tmax1 >= 0 ? tmax1 / kBN + 1 : 0;
+    const int n2 = second ? (lk2 + kBN - 1) / kBN : 0;
+    const int ntiles = n1 + n2;
+
+    bf16x8 qf[8], dof[8];
+    {
+        const __bf16* qrow = qs.q + (int64_t)row_ld * qs.q_rs + (int64_t)head * qs.q_hs + 8 * half;
+        const __bf16* gorow = qs.d_o + (int64_t)row_ld * qs.do_rs + (int64_t)head * qs.do_hs + 8 * half;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            qf[s] = ld_global_16B(qrow + 16 * s);
+            dof[s] = ld_global_16B(gorow + 16 * s);
+        }
+    }
+    const float c = p.scale_log2e;
+    const float lse_c = qs.lse[(int64_t)head * qs.total_q + row_ld] * kLog2e;
+    const float delta = qs.delta[(int64_t)head * qs.total_q + row_ld];
+
+    f32x16 dqacc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dqacc[i][r] = 0.f;
+
+    auto prefetch = [&](int it, KvPrefetch& pf) {
+        const bool s0 = it < n1;
+        const int base = (s0 ? it : it - n1) * kBN;
+        const __bf16* kp_ = s0 ? k1p : k2p;
+        const __bf16* vp_ = s0 ? v1p : v2p;
+        const int64_t krs = s0 ? p.s1.k_rs : p.s2.k_rs;
+        const int64_t vrs = s0 ? p.s1.v_rs : p.s2.v_rs;
+        const int left = s0 ? left1 : left2;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int cidx = tid + kDqThreads * i;
+            int r = base + cidx / 16;
+            r = r < left ? r : left - 1;
+            pf.k[i] = ld_global_16B(kp_ + (int64_t)r * krs + (cidx % 16) * 8);
+            pf.v[i] = ld_global_16B(vp_ + (int64_t)r * vrs + (cidx % 16) * 8);
+        }
+        pf.kpos = 0x7fffffff;
+        if (!s0 && tid < kBN && base + tid < lk2) pf.kpos = pos2p[base + tid];
+    };
+    auto stage = [&](int buf, const KvPrefetch& pf) {
+        unsigned char* kt = smem + buf * kDqStage;
+        unsigned char* vt = kt + kTileBytes;
+        int* kpos = reinterpret_cast<int*>(vt + kTileBytes);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int cidx = tid + kDqThreads * i;
+            *reinterpret_cast<bf16x8*>(kt + rowmajor128_off(cidx / 16, cidx % 16)) = pf.k[i];
+            *reinterpret_cast<bf16x8*>(vt + rowmajor128_off(cidx / 16, cidx % 16)) = pf.v[i];
+        }
+        if (tid < kBN) kpos[tid] = pf.kpos;
+    };
+
+    KvPrefetch pf;
+    if (ntiles > 0) prefetch(0, pf);
+    for (int it = 0; it < ntiles; ++it) {
+        const int buf = it & 1;
+        stage(buf, pf);
+        __syncthreads();
+        if (it + 1 < ntiles) prefetch(it + 1, pf);
+        const bool first_seg = it < n1;
+        const int base = (first_seg ? it : it - n1) * kBN;
+        if (first_seg && base > wmax1) continue;
+        const unsigned char* kt = smem + buf * kDqStage;
+        const unsigned char* vt = kt + kTileBytes;
+        const int* kpos = reinterpret_cast<const int*>(vt + kTileBytes);
+        const bool need_mask = !first_seg || base + kBN - 1 > wmin1;
+
+        bf16x8 dsf[4];
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt) {
+            f32x16 sacc, dpacc;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; dpacc[r] = 0.f; }
+#pragma unroll
+            for (int s = 0; s < 8; ++s) {
+                const bf16x8 ka = *reinterpret_cast<const bf16x8*>(kt + rowmajor128_off(32 * mt + col, 2 * s + half));
+                sacc = mfma32(ka, qf[s], sacc);
+                const bf16x8 va = *reinterpret_cast<const bf16x8*>(vt + rowmajor128_off(32 * mt + col, 2 * s + half));
+                dpacc = mfma32(va, dof[s], dpacc);
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                bool vis = true;
+                if (need_mask) {
+                    const int kl = 32 * mt + acc_row(half, r);
+                    vis = first_seg ? (base + kl <= qlim1) : (kpos[kl] <= qlim2);
+                }
+                const float pr = vis ? fast_exp2(sacc[r] * c - lse_c) : 0.f;
+                dsf[2 * mt + r / 8][r % 8] = (__bf16)(pr * (dpacc[r] - delta));
+            }
+        }
+        // dQ^T (128 d x 32 queries) += K^T dS^T
+#pragma unroll
+        for (int st = 0; st < 4; ++st)
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt) {
+                const bf16x8 a = lds_read_rows_as_k(kt, 16 * st, 32 * dt, lane);
+                dqacc[dt] = mfma32(a, dsf[st], dqacc[dt]);
+            }
+    }
+
+    if (row_ok) {
+        __bf16* drow = qs.dq + (int64_t)row * qs.dq_rs + (int64_t)head * qs.dq_hs;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                bf16x4 v4;
+#pragma unroll
+                for (int b = 0; b < 4; ++b) v4[b] = (__bf16)(dqacc[dt][4 * g4 + b] * p.scale);
+                *reinterpret_cast<bf16x4*>(drow + 32 * dt + 8 * g4 + 4 * half) = v4;
+            }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// dK/dV kernel
+// ---------------------------------------------------------------------------
+constexpr int kKvThreads = 256;
+constexpr int kBQ = 64;                                   // query rows per staged tile
+constexpr int kKvStage = 2 * kTileBytes + 3 * kBQ * 4;    // Q tile, dO tile, lse, delta, qpos
+constexpr int kKvSmem = 2 * kKvStage;                     // double buffered (>= 64 KiB for the final reduction)
+
+struct QPrefetch {
+    bf16x8 q[4], g[4];
+    float lse, delta;
+    int qpos;
+};
+
+template <int G>
+__global__ __launch_bounds__(kKvThreads) void duo_bwd_dkdv_kernel(const BwdParams p) {
+    HIP_DYNAMIC_SHARED(unsigned char, smem)
+    const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+    const int half = lane / 32, col = lane % 32;
+    const int kb = wave % 2, qh = wave / 2;  // 32-key block, 32-row half of the query tile
+    const int hk = blockIdx.x;
+
+    int slot = (int)blockIdx.y;
+    int seq = 0, key0 = 0, key_end = 0;
+    bool second = false;
+    if (!(p.s1.total_k > 0 && find_tile(p.s1.cu_k, p.nseq, kBN, slot, seq, key0, key_end))) {
+        if (!(p.s2.total_k > 0 && find_tile(p.s2.cu_k, p.nseq, kBN, slot, seq, key0, key_end))) return;
+        second = true;
+    }
+    const BwdStream& ks = second ? p.s2 : p.s1;
+    const int k_lo = ks.cu_k[seq];
+    const int lk1 = p.s1.cu_k[seq + 1] - p.s1.cu_k[seq];
+    const int q1_lo = p.s1.total_q > 0 ? p.s1.cu_q[seq] : 0;
+    const int lq1 = p.s1.total_q > 0 ? p.s1.cu_q[seq + 1] - q1_lo : 0;
+    const int q2_lo = p.s2.total_q > 0 ? p.s2.cu_q[seq] : 0;
+    const int lq2 = p.s2.total_q > 0 ? p.s2.cu_q[seq + 1] - q2_lo : 0;
+    const int off = lk1 - lq1;  // position of depth-0 query i is i + off
+
+    // my key (accumulator column) and its position
+    const int key = key0 + 32 * kb + col;
+    const bool key_ok = key < key_end;
+    const int key_ld = key_ok ? key : key_end - 1;
+    const int kpos = key_ok ? (second ? ks.pos_k[key_ld] : key_ld - k_lo) : 0x7fffffff;
+
+    bf16x8 kf[8], vf[8];  // B operands: K^T, V^T columns of my key
+    {
+        const __bf16* kr = ks.k + (int64_t)key_ld * ks.k_rs + (int64_t)hk * ks.k_hs + 8 * half;
+        const __bf16* vr = ks.v + (int64_t)key_ld * ks.v_rs + (int64_t)hk * ks.v_hs + 8 * half;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            kf[s] = ld_global_16B(kr + 16 * s);
+            vf[s] = ld_global_16B(vr + 16 * s);
+        }
+    }
+
+    // query tiles that can see this key tile
+    const int kl0 = key0 - k_lo;  // local index of the tile's first key (depth-0 tiles: its position)
+    int t1_begin = 0, nt1 = 0;
+    if (!second && lq1 > 0) {
+        const int first_q = kl0 - off > 0 ? kl0 - off : 0;  // first depth-0 query row with position >= kl0
+        t1_begin = first_q / kBQ;
+        nt1 = (lq1 + kBQ - 1) / kBQ - t1_begin;
+        if (nt1 < 0) nt1 = 0;
+    }
+    const int nt2 = (lq2 + kBQ - 1) / kBQ;
+    const int nitems = (nt1 + nt2) * G;
+
+    f32x16 dkacc[4], dvacc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { dkacc[i][r] = 0.f; dvacc[i][r] = 0.f; }
+    const float c = p.scale_log2e;
+
+    auto item_rows = [&](int item, bool& q2s, int& r0, int& r_end, int& head) {
+        const int t = item / G;
+        head = hk * G + item % G;
+        q2s = t >= nt1;
+        if (!q2s) {
+            r0 = q1_lo + (t1_begin + t) * kBQ;
+            r_end = q1_lo + lq1;
+        } else {
+            r0 = q2_lo + (t - nt1) * kBQ;
+            r_end = q2_lo + lq2;
+        }
+        r_end = r0 + kBQ < r_end ? r0 + kBQ : r_end;
+    };
+    auto prefetch = [&](int item, QPrefetch& pf) {
+        bool q2s;
+        int r0, r_end, head;
+        item_rows(item, q2s, r0, r_end, head);
+        const BwdStream& qs = q2s ? p.s2 : p.s1;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int cidx = tid + kKvThreads * i;  // 1024 chunks of 16 B per tile
+            int r = r0 + cidx / 16;
+            r = r < r_end ? r : r_end - 1;
+            pf.q[i] = ld_global_16B(qs.q + (int64_t)r * qs.q_rs + (int64_t)head * qs.q_hs + (cidx % 16) * 8);
+            pf.g[i] = ld_global_16B(qs.d_o + (int64_t)r * qs.do_rs + (int64_t)head * qs.do_hs + (cidx % 16) * 8);
+        }
+        pf.lse = 0.f;
+        pf.delta = 0.f;
+        pf.qpos = -1;
+        if (tid < kBQ && r0 + tid < r_end) {
+            const int r = r0 + tid;
+            pf.lse = qs.lse[(int64_t)head * qs.total_q + r] * kLog2e;
+            pf.delta = qs.delta[(int64_t)head * qs.total_q + r];
+            pf.qpos = q2s ? qs.pos_q[r] : (r - q1_lo) + off;
+        }
+    };
+    auto stage = [&](int buf, const QPrefetch& pf) {
+        unsigned char* qt = smem + buf * kKvStage;
+        unsigned char* gt = qt + kTileBytes;
+        float* meta = reinterpret_cast<float*>(gt + kTileBytes);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int cidx = tid + kKvThreads * i;
+            *reinterpret_cast<bf16x8*>(qt + rowmajor128_off(cidx / 16, cidx % 16)) = pf.q[i];
+            *reinterpret_cast<bf16x8*>(gt + rowmajor128_off(cidx / 16, cidx % 16)) = pf.g[i];
+        }
+        if (tid < kBQ) {
+            meta[tid] = pf.lse;
+            meta[kBQ + tid] = pf.delta;
+            reinterpret_cast<int*>(meta)[2 * kBQ + tid] = pf.qpos;
+        }
+    };
+
+    QPrefetch pf;
+    if (nitems > 0) prefetch(0, pf);
+    for (int item = 0; item < nitems; ++item) {
+        const int buf = item & 1;
+        stage(buf, pf);
+        __syncthreads();
+        if (item + 1 < nitems) prefetch(item + 1, pf);
+
+        const unsigned char* qt = smem + buf * kKvStage;
+        const unsigned char* gt = qt + kTileBytes;
+        const float* meta = reinterpret_cast<const float*>(gt + kTileBytes);
+        const int* qposs = reinterpret_cast<const int*>(meta) + 2 * kBQ;
+
+        // S = Q K^T and dP = dO V^T for my 32 queries x 32 keys (lane = key, reg = query)
+        f32x16 sacc, dpacc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; dpacc[r] = 0.f; }
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            const bf16x8 qa = *reinterpret_cast<const bf16x8*>(qt + rowmajor128_off(32 * qh + col, 2 * s + half));
+            sacc = mfma32(qa, kf[s], sacc);
+            const bf16x8 ga = *reinterpret_cast<const bf16x8*>(gt + rowmajor128_off(32 * qh + col, 2 * s + half));
+            dpacc = mfma32(ga, vf[s], dpacc);
+        }
+        bf16x8 pfr[2], dsfr[2];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int qr = 32 * qh + acc_row(half, r);
+            const bool vis = kpos <= qposs[qr];
+            const float pr = vis ? fast_exp2(sacc[r] * c - meta[qr]) : 0.f;
+            pfr[r / 8][r % 8] = (__bf16)pr;
+            dsfr[r / 8][r % 8] = (__bf16)(pr * (dpacc[r] - meta[kBQ + qr]));
+        }
+        // dV (32 keys x 128 d) += P^T dO ;  dK += dS^T Q   (contraction over my 32 queries)
+#pragma unroll
+        for (int st = 0; st < 2; ++st)
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt) {
+                const bf16x8 gb = lds_read_rows_as_k(gt, 32 * qh + 16 * st, 32 * dt, lane);
+                dvacc[dt] = mfma32(pfr[st], gb, dvacc[dt]);
+                const bf16x8 qb = lds_read_rows_as_k(qt, 32 * qh + 16 * st, 32 * dt, lane);
+                dkacc[dt] = mfma32(dsfr[st], qb, dkacc[dt]);
+            }
+    }
+
+    // ---- add the two query halves and store ---------------------------------
+    __syncthreads();
+    float* red = reinterpret_cast<float*>(smem);  // [2 key blocks][128 regs][64 lanes]
+    if (qh == 1) {
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                red[(kb * 128 + dt * 16 + r) * 64 + lane] = dkacc[dt][r];
+                red[(kb * 128 + 64 + dt * 16 + r) * 64 + lane] = dvacc[dt][r];
+            }
+    }
+    __syncthreads();
+    if (qh == 0) {
+        // accumulator (dt, reg r, lane): key = 32*kb + acc_row(half, r), d = 32*dt + col
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int krow = key0 + 32 * kb + acc_row(half, r);
+                const float dkv = (dkacc[dt][r] + red[(kb * 128 + dt * 16 + r) * 64 + lane]) * p.scale;
+                const float dvv = dvacc[dt][r] + red[(kb * 128 + 64 + dt * 16 + r) * 64 + lane];
+                if (krow < key_end) {
+                    ks.dk[(int64_t)krow * ks.dk_rs + (int64_t)hk * ks.dk_hs + 32 * dt + col] = (__bf16)dkv;
+                    ks.dv[(int64_t)krow * ks.dv_rs + (int64_t)hk * ks.dv_hs + 32 * dt + col] = (__bf16)dvv;
+                }
+            }
+    }
+}
+
+BwdStream to_dev(const tah_duo_stream& s, const tah_duo_bwd_stream& g) {
+    BwdStream d;
+    d.q = static_cast<const __bf16*>(s.q);
+    d.k = static_cast<const __bf16*>(s.k);
+    d.v = static_cast<const __bf16*>(s.v);
+    d.o = static_cast<const __bf16*>(s.o);
+    d.d_o = static_cast<const __bf16*>(g.d_o);
+    d.dq = static_cast<__bf16*>(g.dq);
+    d.dk = static_cast<__bf16*>(g.dk);
+    d.dv = static_cast<__bf16*>(g.dv);
+    d.lse = s.lse;
+    d.delta = g.delta;
+    d.cu_q = s.cu_q; d.cu_k = s.cu_k; d.pos_q = s.pos_q; d.pos_k = s.pos_k;
+    d.q_rs = s.q_row_stride; d.q_hs = s.q_head_stride;
+    d.k_rs = s.k_row_stride; d.k_hs = s.k_head_stride;
+    d.v_rs = s.v_row_stride; d.v_hs = s.v_head_stride;
+    d.o_rs = s.o_row_stride; d.o_hs = s.o_head_stride;
+    d.do_rs = g.do_row_stride; d.do_hs = g.do_head_stride;
+    d.dq_rs = g.dq_row_stride; d.dq_hs = g.dq_head_stride;
+    d.dk_rs = g.dk_row_stride; d.dk_hs = g.dk_head_stride;
+    d.dv_rs = g.dv_row_stride; d.dv_hs = g.dv_head_stride;
+    d.total_q = s.total_q;
+    d.total_k = s.total_k;
+    return d;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+int check_bwd_stream(const tah_duo_stream& s, const tah_duo_bwd_stream& g, bool second) {
+    if (s.total_q < 0 || s.total_k < 0) return TAH_E_SHAPE;
+    if (!s.cu_q || !s.cu_k) return TAH_E_NULL;
+    if (s.total_q > 0) {
+        if (!s.q || !s.o || !s.lse || !g.d_o || !g.dq || !g.delta) return TAH_E_NULL;
+        if (second && !s.pos_q) return TAH_E_NULL;
+        if (!aligned16(s.q) || !aligned16(s.o) || !aligned16(g.d_o) || !aligned16(g.dq)) return TAH_E_ALIGN;
+    }
+    if (s.total_k > 0) {
+        if (!s.k || !s.v || !g.dk || !g.dv) return TAH_E_NULL;
+        if (second && !s.pos_k) return TAH_E_NULL;
+        if (!aligned16(s.k) || !aligned16(s.v)) return TAH_E_ALIGN;
+    }
+    const int64_t st[] = {s.q_row_stride, s.q_head_stride, s.k_row_stride, s.k_head_stride, s.v_row_stride, s.v_head_stride,
+                          s.o_row_stride, s.o_head_stride, g.do_row_stride, g.do_head_stride, g.dq_row_stride, g.dq_head_stride};
+    for (int64_t x : st)
+        if (x % 8 != 0) return TAH_E_ALIGN;
+    return TAH_OK;
+}
+
+template <int G>
+int launch_bwd(const BwdParams& p, hipStream_t st) {
+    constexpr int BM = 32 * (8 / G);
+    for (const BwdStream* s : {&p.s1, &p.s2}) {
+        if (s->total_q == 0) continue;
+        const int64_t items = (int64_t)s->total_q * p.hq;
+        hipLaunchKernelGGL(duo_bwd_delta_kernel, dim3((unsigned)((items + 15) / 16)), dim3(256), 0, st, *s, p.hq);
+    }
+    int qtiles = 0, ktiles = 0;
+    if (p.s1.total_q > 0) qtiles += p.s1.total_q / BM + p.nseq;
+    if (p.s2.total_q > 0) qtiles += p.s2.total_q / BM + p.nseq;
+    if (p.s1.total_k > 0) ktiles += p.s1.total_k / kBN + p.nseq;
+    if (p.s2.total_k > 0) ktiles += p.s2.total_k / kBN + p.nseq;
+    if (qtiles > 0) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&duo_bwd_dq_kernel<G>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kDqSmem) != hipSuccess)
+            return TAH_E_LAUNCH;
+        hipLaunchKernelGGL(duo_bwd_dq_kernel<G>, dim3(p.hkv, qtiles), dim3(kDqThreads), kDqSmem, st, p);
+    }
+    if (ktiles > 0) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&duo_bwd_dkdv_kernel<G>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kKvSmem) != hipSuccess)
+            return TAH_E_LAUNCH;
+        hipLaunchKernelGGL(duo_bwd_dkdv_kernel<G>, dim3(p.hkv, ktiles), dim3(kKvThreads), kKvSmem, st, p);
+    }
+    return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
+}
+
+}  // namespace
+}  // namespace tah
+
+extern "C" int tah_duo_bwd_varlen(const tah_duo_bwd_args* a, tah_stream_t stream) {
+    using namespace tah;
+    if (!a) return TAH_E_NULL;
+    const tah_duo_fwd_args& f = a->fwd;
+    if (f.d != kD || f.nseq < 0 || f.hq <= 0 || f.hkv <= 0 || f.hq % f.hkv != 0) return TAH_E_SHAPE;
+    const int g = f.hq / f.hkv;
+    if (g != 1 && g != 2 && g != 4 && g != 8) return TAH_E_SHAPE;
+    if (f.nseq == 0) return TAH_OK;
+    if (int rc = check_bwd_stream(f.s1, a->g1, false)) return rc;
+    if (int rc = check_bwd_stream(f.s2, a->g2, true)) return rc;
+    BwdParams p;
+    p.s1 = to_dev(f.s1, a->g1);
+    p.s2 = to_dev(f.s2, a->g2);
+    p.nseq = f.nseq;
+    p.hq = f.hq;
+    p.hkv = f.hkv;
+    p.scale = f.scale;
+    p.scale_log2e = f.scale * kLog2e;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (g) {
+        case 1: return launch_bwd<1>(p, st);
+        case 2: return launch_bwd<2>(p, st);
+        case 4: return launch_bwd<4>(p, st);
+        default: return launch_bwd<8>(p, st);
+    }
+}

@@ -41,6 +41,30 @@ __device__ __forceinline__ int rowmajor128_off(int row, int chunk) { return row 
 // LDS tile of R rows x 64 bf16 (128 B per row, 8 chunks of 16 B), swizzled likewise.
 __device__ __forceinline__ int rowmajor64_off(int row, int chunk) { return row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4); }
 
+// ds_read_b64_tr_b16: each lane supplies the LDS address of 4 consecutive bf16 (a row fragment).
+// Within each group of 16 lanes the fragments form a flat array G[64] in lane order and lane i
+// of the group receives G[i], G[16+i], G[32+i], G[48+i].  With lane r of the group pointing at
+// element [row0 + r/4][col0 + 4*(r%4)] of a row-major tile, lane i ends up with
+// [row0 + t][col0 + i] for t = 0..3: four rows of one column, i.e. a transposed fragment.
+__device__ __forceinline__ bf16x4 lds_read_tr16(const unsigned char* p) {
+    typedef __attribute__((address_space(3))) bf16x4 lds_bf16x4;
+    return __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)p);
+}
+
+// MFMA operand whose contraction index runs over the ROWS of a row-major [rows][128] bf16 LDS
+// tile (rowmajor128_off layout): returns, for this lane, the 8 values
+// tile[row16 + 8*a + 4*half + b][col32 + lane%32], a = 0..1, b = 0..3, in slot order 4*a + b --
+// the slot order in which a 32x32 accumulator (lane half, reg) enumerates its rows, so that an
+// accumulator converted to bf16 is directly the other operand of the same MFMA.
+__device__ __forceinline__ bf16x8 lds_read_rows_as_k(const unsigned char* tile, int row16, int col32, int lane) {
+    const int half = lane >> 5, r = lane & 15, grp = (lane >> 4) & 1;
+    const int col = col32 + 16 * grp + 4 * (r & 3);
+    const int row = row16 + 4 * half + (r >> 2);
+    const bf16x4 lo = lds_read_tr16(tile + rowmajor128_off(row, col >> 3) + (col & 7) * 2);
+    const bf16x4 hi = lds_read_tr16(tile + rowmajor128_off(row + 8, col >> 3) + (col & 7) * 2);
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
 // Storage slot of key `key` (0..63) inside a transposed 64-key row.  The PV
 // MFMA contracts over keys; operand slot (half h, j) of 16-key step s must hold
 // the same key as S^T accumulator (half h, reg 8*(s%2)+j), i.e. key

@@ -249,6 +249,28 @@ inline int emu_update_dpp(int old, int src, int ctrl, int, int, bool bound_ctrl)
 }
 #define __builtin_amdgcn_update_dpp emu_update_dpp
 
+// ds_read_b64_tr_b16: within each group of 16 lanes, the 16 addressed 4-element rows form a flat array
+// G[64] (lane-major); lane i of the group receives G[i], G[16+i], G[32+i], G[48+i].
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 emu_bf16x4;
+inline uint64_t emu_ds_read_tr16_b64(const void* p) {
+    uint16_t mine[4];
+    memcpy(mine, p, 8);
+    memcpy(emu::t_wave->box[emu::t_lane], mine, 8);
+    emu::wave_sync();
+    const int l = emu::t_lane, base = l & ~15, i = l & 15;
+    uint16_t out[4];
+    for (int t = 0; t < 4; ++t) {
+        const int flat = 16 * t + i;
+        memcpy(&out[t], emu::t_wave->box[base + flat / 4] + 2 * (flat % 4), 2);
+    }
+    emu::wave_sync();
+    uint64_t r;
+    memcpy(&r, out, 8);
+    return r;
+}
+#define __builtin_amdgcn_ds_read_tr16_b64_v4bf16(p) \
+    __builtin_bit_cast(emu_bf16x4, emu_ds_read_tr16_b64((const void*)(p)))
+
 #define __builtin_amdgcn_exp2f(x) exp2f(x)
 #define __builtin_amdgcn_logf(x) log2f(x)
 #define __builtin_amdgcn_rcpf(x) (1.0f / (x))

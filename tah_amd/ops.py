@@ -100,6 +100,45 @@ def duo_fwd_varlen(q1, k1, v1, cu_q1, cu_k1, q2, k2, v2, pos_q2, pos_k2, cu_q2, 
     return o1, lse1, o2, lse2
 
 
+def _fill_bwd_stream(g: _capi.DuoBwdStream, d_o, dq, dk, dv, delta) -> None:
+    g.d_o, g.dq, g.dk, g.dv, g.delta = _ptr(d_o), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(delta)
+    g.do_row_stride, g.do_head_stride = d_o.stride(0), d_o.stride(1)
+    g.dq_row_stride, g.dq_head_stride = dq.stride(0), dq.stride(1)
+    g.dk_row_stride, g.dk_head_stride = dk.stride(0), dk.stride(1)
+    g.dv_row_stride, g.dv_head_stride = dv.stride(0), dv.stride(1)
+
+
+def duo_bwd_varlen(q1, k1, v1, o1, lse1, do1, cu_q1, cu_k1, q2, k2, v2, o2, lse2, do2, pos_q2, pos_k2, cu_q2, cu_k2,
+                   scale: float):
+    """Backward of :func:`duo_fwd_varlen`; returns dq1, dk1, dv1, dq2, dk2, dv2 (bf16)."""
+    lib = _lib.lib()
+    for n, t in (("q1", q1), ("k1", k1), ("v1", v1), ("o1", o1), ("do1", do1),
+                 ("q2", q2), ("k2", k2), ("v2", v2), ("o2", o2), ("do2", do2)):
+        _thd(t, n)
+    for n, t in (("cu_q1", cu_q1), ("cu_k1", cu_k1), ("cu_q2", cu_q2), ("cu_k2", cu_k2),
+                 ("pos_q2", pos_q2), ("pos_k2", pos_k2)):
+        _i32(t, n)
+    _dev_check(q1, k1, v1, o1, lse1, do1, q2, k2, v2, o2, lse2, do2, cu_q1, cu_k1, cu_q2, cu_k2, pos_q2, pos_k2)
+    if do1.shape != q1.shape or do2.shape != q2.shape or o1.shape != q1.shape or o2.shape != q2.shape:
+        raise _capi.TahDuoError("o / dO shapes must match q")
+    if lse1.dtype != torch.float32 or lse2.dtype != torch.float32 or not lse1.is_contiguous() or not lse2.is_contiguous():
+        raise _capi.TahDuoError("lse must be contiguous float32 [Hq, rows]")
+    nseq = cu_q1.numel() - 1
+    hq, d = q1.shape[1], q1.shape[2]
+    dq1, dk1, dv1 = torch.empty_like(q1, memory_format=torch.contiguous_format), torch.empty(k1.shape, dtype=k1.dtype, device=k1.device), torch.empty(v1.shape, dtype=v1.dtype, device=v1.device)
+    dq2, dk2, dv2 = torch.empty_like(q2, memory_format=torch.contiguous_format), torch.empty(k2.shape, dtype=k2.dtype, device=k2.device), torch.empty(v2.shape, dtype=v2.dtype, device=v2.device)
+    delta1 = torch.empty((hq, q1.shape[0]), dtype=torch.float32, device=q1.device)
+    delta2 = torch.empty((hq, q2.shape[0]), dtype=torch.float32, device=q1.device)
+    a = _capi.DuoBwdArgs()
+    _fill_stream(a.fwd.s1, q1, k1, v1, o1, lse1, cu_q1, cu_k1, None, None)
+    _fill_stream(a.fwd.s2, q2, k2, v2, o2, lse2, cu_q2, cu_k2, pos_q2, pos_k2)
+    a.fwd.nseq, a.fwd.hq, a.fwd.hkv, a.fwd.d, a.fwd.scale = nseq, hq, k1.shape[1], d, float(scale)
+    _fill_bwd_stream(a.g1, do1, dq1, dk1, dv1, delta1)
+    _fill_bwd_stream(a.g2, do2, dq2, dk2, dv2, delta2)
+    _capi.check(lib, lib.tah_duo_bwd_varlen(ctypes.byref(a), _stream(q1)), "tah_duo_bwd_varlen")
+    return dq1, dk1, dv1, dq2, dk2, dv2
+
+
 def hard_index_build(mask: torch.Tensor):
     """(B, S) bool/uint8 mask -> pos int32 [B*S cap], flat int32, seq int32, cu int32 [B+1].
 

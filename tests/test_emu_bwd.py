@@ -1,0 +1,55 @@
+"""Backward kernels (delta, dQ, dK/dV) on the CPU execution shim against the analytic C oracle.  No GPU."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import duo_ref as R
+from tests import emu_util
+from tests.cases import make_varlen_case, varlen_args
+from tests.test_emu_fwd import _to_dev
+
+pytestmark = pytest.mark.skipif(not emu_util.have_host_clang(), reason="host clang++ not available")
+
+NAMES = ("dq1", "dk1", "dv1", "dq2", "dk2", "dv2")
+
+
+def run_bwd(dev, seed):
+    """Forward + backward through tah_amd.ops; returns kernel grads and oracle grads (on the bf16-rounded inputs)."""
+    from tah_amd import ops
+    g = torch.Generator().manual_seed(seed)
+    mk = lambda t: torch.randn(t.shape, generator=g).to(torch.bfloat16).to(t.device)
+    do1, do2 = mk(dev["q1"]), mk(dev["q2"])
+    o1, lse1, o2, lse2 = ops.duo_fwd_varlen(*varlen_args(dev))
+    got = ops.duo_bwd_varlen(dev["q1"], dev["k1"], dev["v1"], o1, lse1, do1, dev["cu_q1"], dev["cu_k1"],
+                             dev["q2"], dev["k2"], dev["v2"], o2, lse2, do2, dev["pos_q2"], dev["pos_k2"],
+                             dev["cu_q2"], dev["cu_k2"], dev["scale"])
+    host = [a.float().cpu().numpy() if torch.is_tensor(a) and a.is_floating_point() else
+            (a.cpu().numpy() if torch.is_tensor(a) else a) for a in varlen_args(dev)]
+    want = R.bwd(*host, do1.float().cpu().numpy(), do2.float().cpu().numpy())
+    return got, want
+
+
+def check_grads(got, want, max_rel=2e-2, mean_rel=6e-3):
+    """max|a-b| <= max_rel * max|b| and mean|a-b| <= mean_rel * mean|b| per gradient tensor (bf16 outputs)."""
+    out = {}
+    for n, a, b in zip(NAMES, got, want):
+        if b.size == 0:
+            continue
+        d = np.abs(a.float().cpu().numpy().astype(np.float64) - b)
+        ma, mr = d.max() / max(np.abs(b).max(), 1e-30), d.mean() / max(np.abs(b).mean(), 1e-30)
+        out[n] = (float(ma), float(mr))
+        assert ma <= max_rel and mr <= mean_rel, f"{n}: max-err/max|ref| {ma:.3e} (tol {max_rel}), mean-rel-err {mr:.3e} (tol {mean_rel})"
+    return out
+
+
+@pytest.mark.parametrize("hq,hkv,seqlens,p,kw", [
+    (2, 1, [70], 0.3, {}),
+    (2, 2, [130, 3], 0.1, {}),
+    (4, 1, [65, 64], 0.2, {}),
+    (2, 1, [5, 40], 0.5, dict(seqlens_k=[90, 40], extra_k2=70)),
+])
+def test_bwd_kernels_on_cpu_shim(hq, hkv, seqlens, p, kw):
+    dev = _to_dev(make_varlen_case(200 + hq, seqlens, p, Hq=hq, Hkv=hkv, D=128, **kw))
+    with emu_util.emulated():
+        got, want = run_bwd(dev, 5)
+    print(check_grads(got, want))
