@@ -190,11 +190,14 @@ int tah_pad_rows_build(const int32_t* cu, const int32_t* seq_of, int32_t n, int3
                        tah_stream_t stream);
 
 /* Row gather / scatter: dst[dst_rows ? dst_rows[r] : r] = src[src_rows ? src_rows[r] : r]
- * for r < n, rows of row_bytes bytes at the given byte strides.  Replaces
- * torch.gather (tah_model.py:127-133) and the boolean-mask index_put
- * (tah_model.py:163-175).  Rows named twice in dst_rows race.  Bit-exact. */
-int tah_rows_copy(const void* src, const int32_t* src_rows, void* dst, const int32_t* dst_rows, int32_t n,
-                  int64_t row_bytes, int64_t src_stride_bytes, int64_t dst_stride_bytes, tah_stream_t stream);
+ * for r < n, rows of row_bytes bytes at the given byte strides; when dst_enable
+ * is given (one byte per destination row) rows whose byte is 0 are left
+ * untouched -- the assignment_mask of scatter_back.  Replaces torch.gather
+ * (tah_model.py:127-133) and the boolean-mask index_put (tah_model.py:163-175).
+ * Rows named twice in dst_rows race.  Bit-exact. */
+int tah_rows_copy(const void* src, const int32_t* src_rows, void* dst, const int32_t* dst_rows,
+                  const uint8_t* dst_enable, int32_t n, int64_t row_bytes, int64_t src_stride_bytes,
+                  int64_t dst_stride_bytes, tah_stream_t stream);
 
 #ifdef __cplusplus
 }

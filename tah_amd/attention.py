@@ -1,0 +1,288 @@
+"""Duo-causal attention behind the reference's call sites.
+
+Three layers, from the bottom up:
+
+* :func:`duo_attn_varlen` -- differentiable packed-varlen op (forward and
+  backward HIP kernels), both iteration streams in one launch;
+* :class:`DuoMask` / :func:`build_attention_mask` -- the stand-in for the dense
+  additive mask of ``TaHForCausalLM._build_attention_mask``
+  (tah/model/tah_model.py:744-791): same arguments, but it returns a small
+  carrier of (positions, valid flags, cache, depth) instead of a (B,1,Tq,Tkv)
+  tensor, because the kernels evaluate the predicate themselves;
+* :func:`duo_attention_forward` -- a Hugging Face attention-interface callable
+  (same signature and return convention as ``sdpa_attention_forward``,
+  transformers/integrations/sdpa_attention.py:79-166) that takes the carrier in
+  the ``attention_mask`` slot.
+
+Contract inherited from the kernels: within each batch row the valid tokens'
+positions are their rank among the valid tokens of that sequence (what the
+model's forward computes when ``position_ids`` is None, tah_model.py:555-559),
+and a depth-1 token's depth-0 key is already in the cache.  Query rows that are
+not valid get zeros.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import kv_cache, ops
+from ._capi import TahDuoError
+from .cache import TaHDuoCache
+from .pack import HardIndex
+
+
+class _DuoAttnVarlen(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q1, k1, v1, q2, k2, v2, cu_q1, cu_k1, pos_q2, pos_k2, cu_q2, cu_k2, scale):
+        o1, lse1, o2, lse2 = ops.duo_fwd_varlen(q1, k1, v1, cu_q1, cu_k1, q2, k2, v2, pos_q2, pos_k2, cu_q2, cu_k2, scale)
+        ctx.save_for_backward(q1, k1, v1, o1, lse1, q2, k2, v2, o2, lse2, cu_q1, cu_k1, pos_q2, pos_k2, cu_q2, cu_k2)
+        ctx.scale = scale
+        ctx.mark_non_differentiable(lse1, lse2)
+        return o1, o2, lse1, lse2
+
+    @staticmethod
+    def backward(ctx, do1, do2, _dl1, _dl2):
+        q1, k1, v1, o1, lse1, q2, k2, v2, o2, lse2, cu_q1, cu_k1, pos_q2, pos_k2, cu_q2, cu_k2 = ctx.saved_tensors
+        c = lambda g, like: (torch.zeros_like(like) if g is None else g.contiguous())
+        dq1, dk1, dv1, dq2, dk2, dv2 = ops.duo_bwd_varlen(
+            q1, k1, v1, o1, lse1, c(do1, o1), cu_q1, cu_k1, q2, k2, v2, o2, lse2, c(do2, o2),
+            pos_q2, pos_k2, cu_q2, cu_k2, ctx.scale)
+        return dq1, dk1, dv1, dq2, dk2, dv2, None, None, None, None, None, None, None
+
+
+def duo_attn_varlen(q1, k1, v1, cu_q1, cu_k1, q2, k2, v2, pos_q2, pos_k2, cu_q2, cu_k2, scale: float,
+                    return_lse: bool = False):
+    """Duo-causal attention on packed varlen bf16 tensors, differentiable.
+
+    Depth-0 stream: q1 [T1q,Hq,D], k1/v1 [T1k,Hkv,D], cu_q1/cu_k1 int32 [nseq+1].
+    Depth-1 stream (hard tokens): q2 [T2q,Hq,D], k2/v2 [T2k,Hkv,D], int32 positions
+    pos_q2/pos_k2 and cu_q2/cu_k2.  Key (pos_k, depth_k) is visible to query
+    (pos_q, depth_q) iff pos_k <= pos_q and depth_k <= depth_q.  Returns (o1, o2).
+    """
+    o1, o2, lse1, lse2 = _DuoAttnVarlen.apply(q1, k1, v1, q2, k2, v2, cu_q1, cu_k1, pos_q2, pos_k2, cu_q2, cu_k2,
+                                              float(scale))
+    return (o1, o2, lse1, lse2) if return_lse else (o1, o2)
+
+
+class DuoMask:
+    """What the dense mask of tah_model.py:744-791 is computed from, kept symbolic."""
+
+    def __init__(self, position_ids: torch.Tensor, valid_mask: torch.Tensor, cache: Optional[TaHDuoCache], iter_depth: int):
+        self.position_ids, self.valid_mask, self.cache, self.iter_depth = position_ids, valid_mask, cache, iter_depth
+        self._packed = None  # per-step packing metadata, shared by all decoder layers
+
+    def dense(self, dtype: torch.dtype = torch.float32) -> Optional[torch.Tensor]:
+        """The (B,1,Tq,Tkv) additive mask the reference would have built (for inspection only)."""
+        B, T = self.position_ids.shape
+        c, d, dev = self.cache, self.iter_depth, self.position_ids.device
+        if c is not None and c.has_layer(0):
+            it = c.get_cache_iter_index_upto_iter(0, d)
+            pos = c.get_position_id_upto_iter(0, d, B)
+            val = c.get_valid_mask_upto_iter(0, d, B)
+        else:
+            it = torch.empty((0,), dtype=torch.long, device=dev)
+            pos = torch.empty((B, 0), dtype=torch.long, device=dev)
+            val = torch.empty((B, 0), dtype=torch.long, device=dev)
+        if it.numel() + T == 0:
+            return None
+        kv_pos = torch.cat((pos, self.position_ids), -1)[:, None, :]
+        kv_val = torch.cat((val, self.valid_mask), -1)[:, None, :]
+        kv_it = torch.cat((it, torch.full((T,), d, dtype=torch.long, device=dev)))[None, None, :]
+        see = (kv_pos <= self.position_ids[:, :, None]) & (kv_it <= d) & (kv_val == 1)
+        m = torch.full(see.shape, torch.finfo(dtype).min, dtype=dtype, device=dev)
+        m[see] = 0.0
+        return m[:, None]
+
+
+def build_attention_mask(active_position_ids, active_valid_mask, cache, iter_depth, dtype=None) -> Optional[DuoMask]:
+    """Drop-in for ``TaHForCausalLM._build_attention_mask`` (tah_model.py:744-751): same arguments;
+    returns a :class:`DuoMask` (or ``None`` when there is nothing to attend to, as tah_model.py:773-775)."""
+    del dtype
+    n_cached = cache.get_kv_length_upto_iter(0, iter_depth) if cache is not None and cache.has_layer(0) else 0
+    if n_cached + active_position_ids.shape[1] == 0:
+        return None
+    return DuoMask(active_position_ids, active_valid_mask, cache, iter_depth)
+
+
+# ---------------------------------------------------------------------------
+# packing helpers
+# ---------------------------------------------------------------------------
+
+
+def _rows(x: torch.Tensor) -> torch.Tensor:
+    """(B, H, T, D) -> [B*T, H, D]; free when x is the usual transposed view of a (B,T,H,D) projection."""
+    B, H, T, D = x.shape
+    return x.transpose(1, 2).reshape(B * T, H, D)
+
+
+class _Packed:
+    """Valid-row packing of one (B, T) block: row ids, per-sequence offsets, int32 positions."""
+
+    def __init__(self, valid: Optional[torch.Tensor], pos: Optional[torch.Tensor], B: int, T: int, device):
+        self.B, self.T = B, T
+        all_valid = valid is None
+        if not all_valid:
+            idx = HardIndex(valid)
+            all_valid = idx.n == B * T
+        if all_valid:
+            self.rows, self.n = None, B * T
+            self.cu = torch.arange(0, (B + 1) * T, T, dtype=torch.int32, device=device)
+        else:
+            self.rows, self.n, self.cu = idx.flat, idx.n, idx.cu
+        self.pos = None
+        if pos is not None:
+            p32 = pos.to(torch.int32).contiguous().view(B * T, 1)
+            if self.rows is not None:
+                out = torch.empty((self.n, 1), dtype=torch.int32, device=device)
+                ops.rows_copy(p32, self.rows, out, None, self.n)
+                p32 = out
+            self.pos = p32.view(-1)
+
+    def pack(self, x: torch.Tensor) -> torch.Tensor:
+        r = _rows(x)
+        if self.rows is None:
+            return r
+        return _GatherRows.apply(r.contiguous(), self.rows, self.n)
+
+    def unpack(self, o: torch.Tensor, Hq: int, D: int) -> torch.Tensor:
+        """[n, Hq, D] -> (B, T, Hq, D) with zeros at rows that were not packed."""
+        if self.rows is None:
+            return o.view(self.B, self.T, Hq, D)
+        return _ScatterRows.apply(o, self.rows, self.n, self.B * self.T).view(self.B, self.T, Hq, D)
+
+
+class _GatherRows(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, src, rows, n):
+        out = torch.empty((n,) + tuple(src.shape[1:]), dtype=src.dtype, device=src.device)
+        ops.rows_copy(src, rows, out, None, n)
+        ctx.save_for_backward(rows)
+        ctx.n, ctx.total = n, src.shape[0]
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        (rows,) = ctx.saved_tensors
+        gs = torch.zeros((ctx.total,) + tuple(g.shape[1:]), dtype=g.dtype, device=g.device)
+        ops.rows_copy(g.contiguous(), None, gs, rows, ctx.n)
+        return gs, None, None
+
+
+class _ScatterRows(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, src, rows, n, total):
+        out = torch.zeros((total,) + tuple(src.shape[1:]), dtype=src.dtype, device=src.device)
+        ops.rows_copy(src.contiguous(), None, out, rows, n)
+        ctx.save_for_backward(rows)
+        ctx.n = n
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        (rows,) = ctx.saved_tensors
+        gs = torch.empty((ctx.n,) + tuple(g.shape[1:]), dtype=g.dtype, device=g.device)
+        ops.rows_copy(g.contiguous(), rows, gs, None, ctx.n)
+        return gs, None, None, None
+
+
+def _segment(cache: TaHDuoCache, layer_idx: int, depth: int, B: int, with_pos: bool):
+    """All rows written at (layer, depth), packed per sequence: k, v [rows,Hkv,D], cu int32, pos int32 or None.
+
+    One chunk (prefill / training, the only case on the backward path) packs without copies when every
+    token is valid; several chunks (a cache grown by earlier calls) are concatenated per sequence.
+    """
+    chunks = cache.chunks(layer_idx, depth)
+    if not chunks:
+        raise TahDuoError(f"no keys cached for layer {layer_idx} at depth {depth}")
+    dev = chunks[0][0].device
+    if len(chunks) == 1:
+        k, v, pos, valid = chunks[0]
+        pk = _Packed(valid, pos if with_pos else None, B, k.shape[2], dev)
+        return pk.pack(k), pk.pack(v), pk.cu, pk.pos
+    k = torch.cat([c[0] for c in chunks], dim=2)
+    v = torch.cat([c[1] for c in chunks], dim=2)
+    T = k.shape[2]
+    one = lambda c, fill: (torch.full((B, c[0].shape[2]), fill, dtype=torch.long, device=dev))
+    valid = torch.cat([c[3] if c[3] is not None else one(c, 1) for c in chunks], dim=1)
+    pos = torch.cat([c[2] if c[2] is not None else one(c, 0) for c in chunks], dim=1) if with_pos else None
+    pk = _Packed(valid, pos, B, T, dev)
+    return pk.pack(k), pk.pack(v), pk.cu, pk.pos
+
+
+def duo_attention_forward(module, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
+                          attention_mask, dropout: float = 0.0, scaling: Optional[float] = None,
+                          is_causal: Optional[bool] = None, **kwargs) -> Tuple[torch.Tensor, None]:
+    """Hugging Face attention-interface callable for duo-causal attention.
+
+    query (B,Hq,Tq,D); key/value are whatever ``cache.update`` returned (the new rows); ``attention_mask``
+    is the :class:`DuoMask` built for this step; ``module.layer_idx`` names the layer.  Returns
+    ``(attn_output (B,Tq,Hq,D), None)`` like sdpa_attention_forward (sdpa_attention.py:164-166).
+    A dense tensor mask is refused: there is no dense-mask code path.
+    """
+    del is_causal, kwargs
+    if not isinstance(attention_mask, DuoMask):
+        raise TahDuoError("duo_attention_forward needs the DuoMask from tah_amd.attention.build_attention_mask in the "
+                          "attention_mask slot (a dense additive mask is not accepted)")
+    if dropout:
+        raise TahDuoError("attention dropout is not supported (the reference runs with 0.0)")
+    m = attention_mask
+    cache, depth = m.cache, m.iter_depth
+    if cache is None:
+        raise TahDuoError("the DuoMask carries no cache; pass the cache that update() was called on")
+    layer = int(getattr(module, "layer_idx", 0))
+    B, Hq, Tq, D = query.shape
+    scale = float(scaling) if scaling is not None else float(D) ** -0.5
+    dev = query.device
+
+    # decode fast path: one query row per sequence, slabs hold every cached row (incl. this step's)
+    s1 = cache.slabs(layer, 0)
+    if Tq == 1 and s1 is not None and not (torch.is_grad_enabled() and query.requires_grad):
+        if m._packed is None:
+            idx = HardIndex(m.valid_mask)
+            qpos = torch.empty((max(idx.n, 1), 1), dtype=torch.int32, device=dev)
+            ops.rows_copy(m.position_ids.to(torch.int32).contiguous().view(B, 1), idx.flat, qpos, None, idx.n)
+            m._packed = (idx, qpos.view(-1)[: idx.n])
+        idx, qpos = m._packed
+        out = torch.zeros((B, 1, Hq, D), dtype=query.dtype, device=dev)
+        if idx.n:
+            q = _rows(query)
+            if idx.n != B:
+                qp = torch.empty((idx.n, Hq, D), dtype=query.dtype, device=dev)
+                ops.rows_copy(q.contiguous(), idx.flat, qp, None, idx.n)
+                q = qp
+            o = kv_cache.decode(q, idx.flat if idx.n != B else torch.arange(B, dtype=torch.int32, device=dev), qpos,
+                                s1, cache.slabs(layer, 1) if depth >= 1 else None, scale=scale, depth=depth)
+            if idx.n != B:
+                ops.rows_copy(o, None, out.view(B, Hq, D), idx.flat, idx.n)
+            else:
+                out = o.view(B, 1, Hq, D)
+        return out, None
+
+    # general path: packed varlen forward (+ backward through autograd)
+    if m._packed is None:
+        m._packed = _Packed(m.valid_mask, m.position_ids if depth >= 1 else None, B, Tq, dev)
+    pq = m._packed
+    if not isinstance(pq, _Packed):
+        raise TahDuoError("a DuoMask cannot be shared between the decode path and the varlen path")
+    q = pq.pack(query)
+    zc = torch.zeros(B + 1, dtype=torch.int32, device=dev)
+    zi = torch.zeros(0, dtype=torch.int32, device=dev)
+    k1, v1, cu_k1, _ = _segment(cache, layer, 0, B, with_pos=False)
+    if depth == 0:
+        e_q = q[:0]
+        e_k = k1[:0]
+        o, _ = duo_attn_varlen(q, k1, v1, pq.cu, cu_k1, e_q, e_k, e_k, zi, zi, zc, zc, scale)
+    else:
+        k2, v2, cu_k2, pos_k2 = _segment(cache, layer, 1, B, with_pos=True)
+        e_q = q[:0]
+        _, o = duo_attn_varlen(e_q, k1, v1, zc, cu_k1, q, k2, v2, pq.pos, pos_k2, pq.cu, cu_k2, scale)
+    return pq.unpack(o, Hq, D), None
+
+
+def register_with_transformers(name: str = "tah_duo") -> str:
+    """Register :func:`duo_attention_forward` under ``attn_implementation=name`` (needs transformers)."""
+    from transformers import AttentionInterface
+
+    AttentionInterface.register(name, duo_attention_forward)
+    return name

@@ -78,11 +78,13 @@ __global__ void pad_rows_kernel(const int32_t* cu, const int32_t* seq_of, int n,
 
 template <typename V>
 __global__ void rows_copy_kernel(const unsigned char* src, const int32_t* src_rows, unsigned char* dst,
-                                 const int32_t* dst_rows, int n, int vec_per_row, int64_t src_stride, int64_t dst_stride) {
+                                 const int32_t* dst_rows, const uint8_t* dst_enable, int n, int vec_per_row,
+                                 int64_t src_stride, int64_t dst_stride, int row_base) {
     const int r = blockIdx.y;
     if (r >= n) return;
-    const int64_t sr = src_rows ? src_rows[r] : r;
-    const int64_t dr = dst_rows ? dst_rows[r] : r;
+    const int64_t sr = src_rows ? src_rows[r] : row_base + r;
+    const int64_t dr = dst_rows ? dst_rows[r] : row_base + r;
+    if (dst_enable && !dst_enable[dr]) return;
     const V* s = reinterpret_cast<const V*>(src + sr * src_stride);
     V* d = reinterpret_cast<V*>(dst + dr * dst_stride);
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < vec_per_row; i += gridDim.x * blockDim.x) d[i] = s[i];
@@ -91,18 +93,16 @@ __global__ void rows_copy_kernel(const unsigned char* src, const int32_t* src_ro
 struct alignas(16) V16 { uint32_t x[4]; };
 
 template <typename V>
-int launch_copy(const void* src, const int32_t* src_rows, void* dst, const int32_t* dst_rows, int n, int64_t row_bytes,
-                int64_t src_stride, int64_t dst_stride, hipStream_t st) {
+int launch_copy(const void* src, const int32_t* src_rows, void* dst, const int32_t* dst_rows, const uint8_t* dst_enable, int n,
+                int64_t row_bytes, int64_t src_stride, int64_t dst_stride, hipStream_t st) {
     const int vec = (int)(row_bytes / (int64_t)sizeof(V));
     int gx = (vec + 255) / 256;
     gx = gx < 1 ? 1 : (gx > 64 ? 64 : gx);
     for (int r0 = 0; r0 < n; r0 += 65535) {  // grid.y limit
         const int nr = n - r0 < 65535 ? n - r0 : 65535;
-        hipLaunchKernelGGL(rows_copy_kernel<V>, dim3(gx, nr), dim3(256), 0, st,
-                           static_cast<const unsigned char*>(src) + (src_rows ? 0 : (int64_t)r0 * src_stride),
-                           src_rows ? src_rows + r0 : nullptr,
-                           static_cast<unsigned char*>(dst) + (dst_rows ? 0 : (int64_t)r0 * dst_stride),
-                           dst_rows ? dst_rows + r0 : nullptr, nr, vec, src_stride, dst_stride);
+        hipLaunchKernelGGL(rows_copy_kernel<V>, dim3(gx, nr), dim3(256), 0, st, static_cast<const unsigned char*>(src),
+                           src_rows ? src_rows + r0 : nullptr, static_cast<unsigned char*>(dst),
+                           dst_rows ? dst_rows + r0 : nullptr, dst_enable, nr, vec, src_stride, dst_stride, r0);
     }
     return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
 }
@@ -132,8 +132,9 @@ extern "C" int tah_pad_rows_build(const int32_t* cu, const int32_t* seq_of, int3
     return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
 }
 
-extern "C" int tah_rows_copy(const void* src, const int32_t* src_rows, void* dst, const int32_t* dst_rows, int32_t n,
-                             int64_t row_bytes, int64_t src_stride_bytes, int64_t dst_stride_bytes, tah_stream_t stream) {
+extern "C" int tah_rows_copy(const void* src, const int32_t* src_rows, void* dst, const int32_t* dst_rows,
+                             const uint8_t* dst_enable, int32_t n, int64_t row_bytes, int64_t src_stride_bytes,
+                             int64_t dst_stride_bytes, tah_stream_t stream) {
     using namespace tah;
     if (n < 0 || row_bytes < 0) return TAH_E_SHAPE;
     if (n == 0 || row_bytes == 0) return TAH_OK;
@@ -141,11 +142,11 @@ extern "C" int tah_rows_copy(const void* src, const int32_t* src_rows, void* dst
     hipStream_t st = static_cast<hipStream_t>(stream);
     const uintptr_t bits = reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst) | (uintptr_t)row_bytes |
                            (uintptr_t)src_stride_bytes | (uintptr_t)dst_stride_bytes;
-    if (bits % 16 == 0) return launch_copy<V16>(src, src_rows, dst, dst_rows, n, row_bytes, src_stride_bytes, dst_stride_bytes, st);
-    if (bits % 8 == 0) return launch_copy<uint64_t>(src, src_rows, dst, dst_rows, n, row_bytes, src_stride_bytes, dst_stride_bytes, st);
-    if (bits % 4 == 0) return launch_copy<uint32_t>(src, src_rows, dst, dst_rows, n, row_bytes, src_stride_bytes, dst_stride_bytes, st);
-    if (bits % 2 == 0) return launch_copy<uint16_t>(src, src_rows, dst, dst_rows, n, row_bytes, src_stride_bytes, dst_stride_bytes, st);
-    return launch_copy<uint8_t>(src, src_rows, dst, dst_rows, n, row_bytes, src_stride_bytes, dst_stride_bytes, st);
+    if (bits % 16 == 0) return launch_copy<V16>(src, src_rows, dst, dst_rows, dst_enable, n, row_bytes, src_stride_bytes, dst_stride_bytes, st);
+    if (bits % 8 == 0) return launch_copy<uint64_t>(src, src_rows, dst, dst_rows, dst_enable, n, row_bytes, src_stride_bytes, dst_stride_bytes, st);
+    if (bits % 4 == 0) return launch_copy<uint32_t>(src, src_rows, dst, dst_rows, dst_enable, n, row_bytes, src_stride_bytes, dst_stride_bytes, st);
+    if (bits % 2 == 0) return launch_copy<uint16_t>(src, src_rows, dst, dst_rows, dst_enable, n, row_bytes, src_stride_bytes, dst_stride_bytes, st);
+    return launch_copy<uint8_t>(src, src_rows, dst, dst_rows, dst_enable, n, row_bytes, src_stride_bytes, dst_stride_bytes, st);
 }
 
 extern "C" int tah_duo_abi_version(void) { return TAH_DUO_ABI_VERSION; }

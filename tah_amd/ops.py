@@ -170,10 +170,16 @@ def pad_rows_build(cu: torch.Tensor, seq_of: torch.Tensor, n: int, width: int) -
 
 
 def rows_copy(src: torch.Tensor, src_rows: Optional[torch.Tensor], dst: torch.Tensor,
-              dst_rows: Optional[torch.Tensor], n: int) -> None:
-    """dst[dst_rows[r]] = src[src_rows[r]] for r < n; src/dst are [rows, ...] with contiguous rows."""
+              dst_rows: Optional[torch.Tensor], n: int, dst_enable: Optional[torch.Tensor] = None) -> None:
+    """dst[dst_rows[r]] = src[src_rows[r]] for r < n; src/dst are [rows, ...] with contiguous rows.
+
+    dst_enable (bool/uint8, one entry per row of dst): rows whose entry is 0 are left untouched.
+    """
     lib = _lib.lib()
-    _dev_check(src, dst, src_rows, dst_rows)
+    _dev_check(src, dst, src_rows, dst_rows, dst_enable)
+    if dst_enable is not None and (dst_enable.dtype not in (torch.bool, torch.uint8) or not dst_enable.is_contiguous()
+                                   or dst_enable.numel() != dst.shape[0]):
+        raise _capi.TahDuoError("rows_copy: dst_enable must be a contiguous bool/uint8 tensor with one entry per dst row")
     if n == 0:
         return
     if src.dtype != dst.dtype or src.shape[1:] != dst.shape[1:]:
@@ -184,5 +190,5 @@ def rows_copy(src: torch.Tensor, src_rows: Optional[torch.Tensor], dst: torch.Te
     row_bytes = src[0].numel() * src.element_size()
     sstride = (src.stride(0) if src.shape[0] > 1 else src[0].numel()) * src.element_size()
     dstride = (dst.stride(0) if dst.shape[0] > 1 else dst[0].numel()) * dst.element_size()
-    _capi.check(lib, lib.tah_rows_copy(src.data_ptr(), _ptr(src_rows), dst.data_ptr(), _ptr(dst_rows), n, row_bytes,
-                                       sstride, dstride, _stream(src)), "tah_rows_copy")
+    _capi.check(lib, lib.tah_rows_copy(src.data_ptr(), _ptr(src_rows), dst.data_ptr(), _ptr(dst_rows), _ptr(dst_enable), n,
+                                       row_bytes, sstride, dstride, _stream(src)), "tah_rows_copy")

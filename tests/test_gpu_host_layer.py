@@ -1,0 +1,58 @@
+"""GPU: the host layer (pack API, cache, mask carrier, HF attention callable) end to end on the HIP path."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import duo_oracle as O
+from tests.cases import make_dense_case
+from tests.test_host_layer import _forward_two_depths, _oracle_two_depths
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("B,T,p,left_pad", [(2, 300, 0.1, None), (3, 200, 0.2, [0, 37, 150]), (1, 512, 0.06, None)])
+def test_forward_loop_matches_dense_reference_gpu(B, T, p, left_pad):
+    from tah_amd.cache import TaHDuoCache
+    c = make_dense_case(50 + B, B=B, T=T, p_hard=p, left_pad=left_pad)
+    _, o1, o2, pad = _forward_two_depths(c, TaHDuoCache(), device="cuda")
+    w1, w2, wpad = _oracle_two_depths(c)
+    assert torch.equal(pad.cpu(), wpad)
+    valid = c["valid"].bool()
+    np.testing.assert_allclose(o1.cpu()[valid].float().numpy(), w1[valid].numpy(), atol=2e-2, rtol=2e-2)
+    assert (o1.cpu()[~valid] == 0).all()
+    np.testing.assert_allclose(o2.cpu()[~pad.cpu()].float().numpy(), w2[~wpad].numpy(), atol=2e-2, rtol=2e-2)
+
+
+def test_forward_loop_gradients_gpu():
+    from tah_amd.cache import TaHDuoCache
+    c = make_dense_case(60, B=2, T=160, p_hard=0.2, left_pad=[0, 30])
+    t, o1, o2, pad = _forward_two_depths(c, TaHDuoCache(), requires_grad=True, device="cuda")
+    g = torch.Generator().manual_seed(1)
+    w1, w2 = torch.randn(o1.shape, generator=g), torch.randn(o2.shape, generator=g)
+    ((o1.float() * w1.cuda()).sum() + (o2.float() * w2.cuda()).sum()).backward()
+    ref = {k: c[k].to(torch.bfloat16).double().requires_grad_(True) for k in t}
+    r1, r2, rpad = O.duo_prefill_dense(ref["q1"], ref["k1"], ref["v1"], ref["q2"], ref["k2"], ref["v2"], c["hard"],
+                                       c["scale"], valid_mask=c["valid"])
+    valid = c["valid"].bool()
+    # invalid query rows are out of contract: they take no part in the loss
+    ((r1 * (w1 * valid[:, :, None, None]).to(torch.bfloat16).double()).sum()
+     + (r2 * (w2 * ~rpad[:, :, None, None]).to(torch.bfloat16).double()).sum()).backward()
+    for n in ("q1", "k1", "v1", "q2", "k2", "v2"):
+        a, b = t[n].grad.float().cpu(), ref[n].grad.float()
+        err = (a - b).abs().max() / b.abs().max()
+        assert err < 3e-2, (n, float(err))
+
+
+def test_gather_scatter_large_gpu():
+    from tah_amd.pack import gather_active, scatter_back
+    g = torch.Generator().manual_seed(7)
+    B, S, H = 4, 4096, 2048
+    mask = (torch.rand(B, S, generator=g) < 0.06).cuda()
+    x = torch.randn(B, S, H, generator=g).to(torch.bfloat16).cuda()
+    pos = torch.arange(S).expand(B, S).contiguous().cuda()
+    pad, gx, gp = gather_active(mask, x, pos)
+    assert torch.equal(gx[~pad], x[mask]) and torch.equal(gp[~pad], pos[mask])
+    assert (gx[pad] == 0).all() and pad.shape[1] == int(mask.sum(1).max())
+    dest = torch.zeros_like(x)
+    out = scatter_back(mask, gx, dest)
+    assert torch.equal(out[mask], x[mask]) and (out[~mask] == 0).all()

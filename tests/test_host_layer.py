@@ -1,0 +1,238 @@
+"""Host layer (pack API, cache protocol, mask carrier, HF attention callable) driven the way the reference's
+forward loop drives it, with the kernels running on the CPU execution shim.  No GPU."""
+import types
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import duo_oracle as O
+from tests import emu_util
+from tests.cases import make_dense_case
+
+pytestmark = pytest.mark.skipif(not emu_util.have_host_clang(), reason="host clang++ not available")
+
+
+@pytest.fixture()
+def emu():
+    with emu_util.emulated() as lib:
+        yield lib
+
+
+@pytest.mark.parametrize("seed,p", [(0, 0.3), (1, 0.0), (2, 1.0)])
+def test_gather_scatter_match_reference_semantics(emu, seed, p):
+    from tah_amd.pack import gather_active, scatter_back
+    g = torch.Generator().manual_seed(seed)
+    B, S = 3, 21
+    mask = torch.rand(B, S, generator=g) < p
+    if seed == 0:
+        mask[1] = False
+    x = torch.randn(B, S, 8, generator=g).to(torch.bfloat16)
+    ids = torch.arange(B * S).view(B, S)
+    got = gather_active(mask, x, ids, None)
+    want = O.gather_active(mask, x, ids, None)
+    assert got[3] is None and len(got) == 4
+    for a, b in zip(got[:3], want[:3]):
+        assert a.shape == b.shape and a.dtype == b.dtype and torch.equal(a, b)
+    lab = gather_active(mask, ids, pad_value=-100)[1]
+    assert torch.equal(lab, O.gather_active(mask, ids, pad_value=-100)[1])
+    dest = torch.full((B, S, 8), -7.0).to(torch.bfloat16)
+    assert torch.equal(scatter_back(mask, got[1], dest), O.scatter_back(mask, want[1], dest))
+    amask = torch.rand(B, S, generator=g) < 0.5
+    assert torch.equal(scatter_back(mask, got[1], dest, assignment_mask=amask),
+                       O.scatter_back(mask, want[1], dest, assignment_mask=amask))
+    d2 = dest.clone()
+    assert scatter_back(mask, got[1], d2, in_place=True) is d2 and torch.equal(d2, O.scatter_back(mask, want[1], dest))
+    fin = torch.zeros(B, S, dtype=torch.bool)
+    fm = torch.ones_like(got[0])
+    scatter_back(mask, fm, fin, in_place=True)
+    assert torch.equal(fin, mask)
+
+
+def test_gather_scatter_autograd(emu):
+    from tah_amd.pack import gather_active, scatter_back
+    g = torch.Generator().manual_seed(5)
+    B, S = 2, 9
+    mask = torch.rand(B, S, generator=g) < 0.5
+    x = torch.randn(B, S, 4, generator=g, requires_grad=True)
+    xr = x.detach().clone().requires_grad_(True)
+    w = torch.randn(B, int(mask.sum(1).max()), 4, generator=g)
+    (gather_active(mask, x)[1] * w).sum().backward()
+    pad, gx = O.gather_active(mask, xr)
+    idx = torch.nonzero(mask)
+    ref = torch.zeros_like(xr)
+    for b in range(B):
+        cols = torch.nonzero(mask[b]).flatten()
+        ref[b, cols] = w[b, : len(cols)]
+    assert torch.equal(x.grad, ref)
+    src = torch.randn(B, w.shape[1], 4, generator=g, requires_grad=True)
+    dest = torch.randn(B, S, 4, generator=g, requires_grad=True)
+    amask = torch.rand(B, S, generator=g) < 0.6
+    wo = torch.randn(B, S, 4, generator=g)
+    out = scatter_back(mask, src, dest, assignment_mask=amask)
+    assert torch.equal(out.detach(), O.scatter_back(mask, src.detach(), dest.detach(), assignment_mask=amask))
+    (out * wo).sum().backward()
+    fm = mask & amask
+    assert torch.equal(dest.grad, torch.where(fm[..., None], torch.zeros_like(wo), wo))
+    gs = torch.zeros_like(src)
+    for b in range(B):
+        for k, c in enumerate(torch.nonzero(mask[b]).flatten().tolist()):
+            if fm[b, c]:
+                gs[b, k] = wo[b, c]
+    assert torch.equal(src.grad, gs)
+
+
+def _layer(layer_idx=0):
+    return types.SimpleNamespace(layer_idx=layer_idx, num_key_value_groups=2)
+
+
+def _forward_two_depths(c, cache, requires_grad=False, device="cpu"):
+    """The reference's forward loop around one attention layer (tah_model.py:580-623), two depths."""
+    from tah_amd.attention import build_attention_mask, duo_attention_forward
+    from tah_amd.pack import gather_active
+    bf = lambda x: x.to(torch.bfloat16).to(device)
+    c = dict(c, hard=c["hard"].to(device), valid=c["valid"].to(device))
+    B, T = c["hard"].shape
+    valid = c["valid"]
+    pos = (torch.cumsum(valid, -1) - 1).clamp(min=0)
+    t = {k: bf(c[k]).clone().requires_grad_(requires_grad) for k in ("q1", "k1", "v1", "q2", "k2", "v2")}
+    m0 = build_attention_mask(pos, valid, cache, 0, dtype=torch.bfloat16)
+    cache.current_iter_depth, cache.position_ids_to_cache, cache.valid_mask_to_cache = 0, pos, valid
+    k, v = cache.update(t["k1"], t["v1"], 0)
+    o1, none = duo_attention_forward(_layer(), t["q1"], k, v, m0, dropout=0.0, scaling=c["scale"])
+    assert none is None and o1.shape == (B, T, t["q1"].shape[1], 128)
+    tok = lambda x: x.transpose(1, 2)
+    pad, q2, k2, v2, pos2, val2 = gather_active(c["hard"], tok(t["q2"]), tok(t["k2"]), tok(t["v2"]), pos, valid)
+    if pad.shape[1] == 0:
+        return t, o1, None, pad
+    m1 = build_attention_mask(pos2, val2, cache, 1, dtype=torch.bfloat16)
+    cache.current_iter_depth, cache.position_ids_to_cache, cache.valid_mask_to_cache = 1, pos2, val2
+    k, v = cache.update(tok(k2), tok(v2), 0)
+    o2, _ = duo_attention_forward(_layer(), tok(q2), k, v, m1, scaling=c["scale"])
+    return t, o1, o2, pad
+
+
+def _oracle_two_depths(c):
+    r = lambda x: x.to(torch.bfloat16).float()
+    return O.duo_prefill_dense(r(c["q1"]), r(c["k1"]), r(c["v1"]), r(c["q2"]), r(c["k2"]), r(c["v2"]), c["hard"],
+                               c["scale"], valid_mask=c["valid"])
+
+
+@pytest.mark.parametrize("left_pad", [None, [0, 9]])
+def test_forward_loop_matches_dense_reference(emu, left_pad):
+    from tah_amd.cache import TaHDuoCache
+    c = make_dense_case(31, B=2, T=40, p_hard=0.25, Hq=4, Hkv=2, D=128, left_pad=left_pad)
+    cache = TaHDuoCache()
+    _, o1, o2, pad = _forward_two_depths(c, cache)
+    w1, w2, wpad = _oracle_two_depths(c)
+    assert torch.equal(pad, wpad)
+    valid = c["valid"].bool()
+    np.testing.assert_allclose(o1[valid].float().numpy(), w1[valid].numpy(), atol=2e-2, rtol=2e-2)
+    assert (o1[~valid] == 0).all()
+    np.testing.assert_allclose(o2[~pad].float().numpy(), w2[~pad].numpy(), atol=2e-2, rtol=2e-2)
+    assert (o2[pad] == 0).all()
+    # cache protocol: same lengths / metadata as the reference's cache after the same writes
+    n2 = pad.shape[1]
+    assert cache.get_seq_length(0) == 40 and cache.get_cache_length(0) == 40 + n2
+    assert cache.get_kv_length_upto_iter(0, 1) == 40 + n2 and cache.get_cache_length(0, 1) == n2
+    assert cache.get_cache_iter_index_upto_iter(0, 1).tolist() == [0] * 40 + [1] * n2
+    assert cache.get_position_id_upto_iter(0, 1).shape == (2, 40 + n2)
+    assert cache.get_valid_mask_upto_iter(0, 0).tolist() == c["valid"].tolist()
+    assert cache.has_layer(0) and not cache.has_layer(1) and cache.batch_size == 2
+    K, V = cache.get_cache_upto_iter(0, 1)
+    assert K.shape == (2, 2, 40 + n2, 128)
+    with pytest.raises(AssertionError):
+        cache.update(K[:1], V[:1], 0)
+
+
+def test_dense_mask_of_carrier_equals_reference_mask(emu):
+    from tah_amd.attention import build_attention_mask
+    from tah_amd.cache import TaHDuoCache
+    c = make_dense_case(32, B=2, T=12, p_hard=0.4, Hq=2, Hkv=1, D=128, left_pad=[3, 0])
+    cache, ocache = TaHDuoCache(), O.OracleCache()
+    pos = (torch.cumsum(c["valid"], -1) - 1).clamp(min=0)
+    m = build_attention_mask(pos, c["valid"], cache, 0, torch.float32)
+    assert torch.equal(m.dense(), O.build_attention_mask(pos, c["valid"], ocache, 0, torch.float32))
+    for ch in (cache, ocache):
+        ch.current_iter_depth, ch.position_ids_to_cache, ch.valid_mask_to_cache = 0, pos, c["valid"]
+        ch.update(c["k1"].to(torch.bfloat16), c["v1"].to(torch.bfloat16), 0)
+    pad, pos2, val2 = O.gather_active(c["hard"], pos, c["valid"])
+    m1 = build_attention_mask(pos2, val2, cache, 1, torch.float32)
+    assert torch.equal(m1.dense(), O.build_attention_mask(pos2, val2, ocache, 1, torch.float32))
+    assert build_attention_mask(pos[:, :0], c["valid"][:, :0], None, 0) is None
+
+
+def test_forward_loop_gradients(emu):
+    from tah_amd.cache import TaHDuoCache
+    c = make_dense_case(33, B=1, T=36, p_hard=0.3, Hq=2, Hkv=1, D=128)
+    t, o1, o2, pad = _forward_two_depths(c, TaHDuoCache(), requires_grad=True)
+    g = torch.Generator().manual_seed(1)
+    w1, w2 = torch.randn(o1.shape, generator=g), torch.randn(o2.shape, generator=g)
+    ((o1.float() * w1).sum() + (o2.float() * w2).sum()).backward()
+    ref = {k: c[k].to(torch.bfloat16).double().requires_grad_(True) for k in t}
+    r1, r2, rpad = O.duo_prefill_dense(ref["q1"], ref["k1"], ref["v1"], ref["q2"], ref["k2"], ref["v2"], c["hard"], c["scale"])
+    ((r1 * w1.to(torch.bfloat16).double()).sum() + (r2 * w2.to(torch.bfloat16).double()).sum()).backward()
+    hard = c["hard"][0]
+    for n in ("q1", "k1", "v1", "q2", "k2", "v2"):
+        a, b = t[n].grad.float(), ref[n].grad.float()
+        if n.endswith("2"):  # only hard rows of the depth-1 projections take part
+            assert (a[0, :, ~hard] == 0).all()
+        err = (a - b).abs().max() / b.abs().max()
+        assert err < 3e-2, (n, float(err))
+
+
+def test_decode_steps_through_cache_and_callable(emu):
+    """Prefill then two decode steps with slabs; compare with the dense reference over the grown cache."""
+    from tah_amd.attention import build_attention_mask, duo_attention_forward
+    from tah_amd.cache import TaHDuoCache
+    from tah_amd.pack import gather_active
+    T0, steps = 20, 2
+    c = make_dense_case(34, B=2, T=T0 + steps, p_hard=0.3, Hq=2, Hkv=1, D=128, left_pad=[0, 5])
+    bf = lambda x: x.to(torch.bfloat16)
+    cache = TaHDuoCache().enable_slabs(64, 32)
+    ocache = O.OracleCache()
+    valid_all = c["valid"]
+    pos_all = (torch.cumsum(valid_all, -1) - 1).clamp(min=0)
+    tok = lambda x: x.transpose(1, 2)
+
+    def step(lo, hi):
+        """Feed tokens [lo, hi) at depth 0, then their hard subset at depth 1, to both implementations."""
+        sl = slice(lo, hi)
+        pos, valid, hard = pos_all[:, sl], valid_all[:, sl], c["hard"][:, sl]
+        q1, k1, v1 = (bf(c[n][:, :, sl]) for n in ("q1", "k1", "v1"))
+        outs = []
+        for ch, fwd in ((cache, None), (ocache, "ref")):
+            mk = build_attention_mask if fwd is None else O.build_attention_mask
+            m0 = mk(pos, valid, ch, 0, torch.float32)
+            ch.current_iter_depth, ch.position_ids_to_cache, ch.valid_mask_to_cache = 0, pos, valid
+            if fwd is None:
+                k, v = ch.update(k1, v1, 0)
+                o1, _ = duo_attention_forward(_layer(), q1, k, v, m0, scaling=c["scale"])
+                pad, q2, k2, v2, pos2, val2 = gather_active(hard, *(tok(bf(c[n][:, :, sl])) for n in ("q2", "k2", "v2")), pos, valid)
+            else:
+                K, V = ch.update(k1.float(), v1.float(), 0)
+                o1 = O.sdpa_dense(q1.float(), K, V, m0, c["scale"])
+                pad, q2, k2, v2, pos2, val2 = O.gather_active(hard, *(tok(bf(c[n][:, :, sl]).float()) for n in ("q2", "k2", "v2")), pos, valid)
+            o2 = None
+            if pad.shape[1]:
+                m1 = mk(pos2, val2, ch, 1, torch.float32)
+                ch.current_iter_depth, ch.position_ids_to_cache, ch.valid_mask_to_cache = 1, pos2, val2
+                if fwd is None:
+                    k, v = ch.update(tok(k2), tok(v2), 0)
+                    o2, _ = duo_attention_forward(_layer(), tok(q2), k, v, m1, scaling=c["scale"])
+                else:
+                    K, V = ch.update(tok(k2), tok(v2), 0)
+                    o2 = O.sdpa_dense(tok(q2), K, V, m1, c["scale"])
+            outs.append((o1, o2, pad, valid.bool()))
+        (a1, a2, pad, vb), (b1, b2, _, _) = outs
+        np.testing.assert_allclose(a1[vb].float().numpy(), b1[vb].numpy(), atol=2e-2, rtol=2e-2)
+        if a2 is not None:
+            np.testing.assert_allclose(a2[~pad].float().numpy(), b2[~pad].numpy(), atol=2e-2, rtol=2e-2)
+
+    with torch.no_grad():
+        step(0, T0)
+        for s in range(steps):
+            step(T0 + s, T0 + s + 1)
+    s1 = cache.slabs(0, 0)
+    assert s1.len.tolist() == valid_all.sum(1).tolist() and int(s1.overflow) == 0
+    assert cache.slabs(0, 1).len.tolist() == (c["hard"] & valid_all.bool()).sum(1).tolist()
