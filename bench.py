@@ -143,6 +143,10 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only", choices=["all", "fwd", "decode", "fwd_bwd"], default="all",
+                    help="profiling aid: run only one leg (the JSON line then lacks the other legs)")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="profiling aid: also run one plain 256 MiB device copy (known traffic for counter scaling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no sharding, no collectives); use --gpus 1", file=sys.stderr)
@@ -161,32 +165,40 @@ def main() -> int:
     pairs = visible_pairs(case)
     flops = 4.0 * 128 * 16 * pairs
 
-    for _ in range(args.warmup):
+    fwd_steps = args.steps if args.only in ("all", "fwd") else 1
+    for _ in range(args.warmup if args.only in ("all", "fwd") else 1):
         ops.duo_fwd_varlen(*a)
     torch.cuda.synchronize()
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     ev0.record()
-    for _ in range(args.steps):
+    for _ in range(fwd_steps):
         ops.duo_fwd_varlen(*a)
     ev1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    ms = ev0.elapsed_time(ev1) / args.steps  # events on the stream the kernel is launched on
+    ms = ev0.elapsed_time(ev1) / fwd_steps  # events on the stream the kernel is launched on
     tflops = flops / (ms * 1e-3) / 1e12
 
-    extra = {"decode": bench_decode(args.steps, args.warmup)}
-    extra["fwd_bwd_seq8192_p06"] = bench_fwd_bwd(
+    if args.calib_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
+        src.clone()
+        torch.cuda.synchronize()
+    extra = {}
+    if args.only in ("all", "decode"):
+        extra["decode"] = bench_decode(args.steps, args.warmup)
+    if args.only in ("all", "fwd_bwd"):
+      extra["fwd_bwd_seq8192_p06"] = bench_fwd_bwd(
         "north-star headline: fwd+bwd, one sequence of 8192, p_hard=0.06, Hq=16, Hkv=8, D=128", [8192], 0.06, 1238,
         max(args.steps // 2, 1), max(args.warmup // 2, 1))
-    extra["fwd_bwd_4docs_p10"] = bench_fwd_bwd(
+      extra["fwd_bwd_4docs_p10"] = bench_fwd_bwd(
         "configs[3]: fwd+bwd, 8192 packed tokens in 4 documents, p_hard=0.10", [1397, 3210, 2561, 1024], 0.10, 1237,
         max(args.steps // 2, 1), max(args.warmup // 2, 1))
 
     out = {
         "metric": "duo-causal attn TFLOP/s (% bf16 MFMA peak) prefill; decode HBM GB/s",
         "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": wall * 1e3 / args.steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": wall * 1e3 / fwd_steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "configs[1]: duo-causal prefill forward, B=4, T=4096, Hq=16, Hkv=8, D=128, p_hard=0.06",
                    "visible_pairs_per_head": pairs, "flop_per_step": flops, "tokens_per_s": B * T / (ms * 1e-3)},

@@ -26,6 +26,12 @@ __device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
 // Row index inside a 32-row MFMA accumulator tile held by (lane half h, reg r).
 __device__ __forceinline__ constexpr int acc_row(int h, int r) { return 8 * (r / 4) + 4 * h + (r % 4); }
 
+// x *= a with the product forced into x's own register, so that an accumulator rescaled inside a
+// rarely taken branch is not copied to a second register set on the common path.
+#ifndef TAH_MUL_INPLACE
+#define TAH_MUL_INPLACE(x, a) asm volatile("v_mul_f32 %0, %1, %0" : "+v"(x) : "v"(a))
+#endif
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
@@ -33,10 +39,28 @@ __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcp
 __device__ __forceinline__ bf16x8 ld_global_16B(const __bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
 __device__ __forceinline__ void st_global_16B(__bf16* p, bf16x8 v) { *reinterpret_cast<bf16x8*>(p) = v; }
 
-// LDS tile of R rows x 128 bf16 (256 B per row, 16 chunks of 16 B), chunk index
-// XOR-swizzled with the row so that 16 lanes reading the same logical chunk of
-// 16 consecutive rows touch 16 different bank groups.
-__device__ __forceinline__ int rowmajor128_off(int row, int chunk) { return row * 256 + ((chunk ^ (row & 15)) << 4); }
+// Asynchronous global -> LDS copy of 16 bytes per lane (global_load_lds_dwordx4): lane l's bytes
+// land at lds_wave_base + 16*l; lds_wave_base must be wave-uniform.  Completion is tracked by
+// vmcnt: call wait_vmem() before the barrier that publishes the tile.
+__device__ __forceinline__ void async_copy_16B(const void* gsrc, unsigned char* lds_wave_base) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
+                                     (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+}
+// Occupancy the kernel is written for; lets the scheduler spend registers on latency hiding.
+#ifndef TAH_WAVES_PER_EU
+#define TAH_WAVES_PER_EU(lo, hi) __attribute__((amdgpu_waves_per_eu(lo, hi)))
+#endif
+#ifndef TAH_WAIT_VMEM
+#define TAH_WAIT_VMEM() asm volatile("s_waitcnt vmcnt(0)" ::: "memory")
+#endif
+
+// LDS tile of R rows x 128 bf16 (256 B per row, 16 chunks of 16 B).  The chunk index is XORed
+// with a 4-bit function of the row that (a) takes 16 different values over 16 consecutive rows,
+// so 16 lanes reading the same logical chunk of consecutive rows (MFMA A operand, b128) touch 16
+// different bank groups, and (b) moves 4 consecutive rows into 4 different aligned groups of 4
+// chunks, so a transpose read (4 rows x 64 contiguous bytes per half-wave) is conflict-free too.
+__device__ __forceinline__ constexpr int row_swizzle(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
+__device__ __forceinline__ int rowmajor128_off(int row, int chunk) { return row * 256 + ((chunk ^ row_swizzle(row)) << 4); }
 
 // LDS tile of R rows x 64 bf16 (128 B per row, 8 chunks of 16 B), swizzled likewise.
 __device__ __forceinline__ int rowmajor64_off(int row, int chunk) { return row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4); }
@@ -74,7 +98,15 @@ __device__ __forceinline__ constexpr int pv_slot(int key) {
     return (key & ~12) | ((key & 4) << 1) | ((key & 8) >> 1);
 }
 
-__device__ __forceinline__ float wave_max_xor32(float x) { return fmaxf(x, __shfl_xor(x, 32)); }
+// max over the two lanes l and l^32 (v_permlane32_swap: no LDS traffic)
+__device__ __forceinline__ float wave_max_xor32(float x) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float wave_sum_xor32(float x) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
 
 __device__ __forceinline__ int wave_reduce_max(int x) {
 #pragma unroll

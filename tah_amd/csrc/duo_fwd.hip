@@ -6,13 +6,17 @@
 // Per key tile of 64 keys each wave computes S^T = K Q^T (keys x queries) with
 // v_mfma_f32_32x32x16_bf16, which leaves one query per lane column: the online
 // softmax needs one cross-lane exchange per tile, and the bf16 probabilities
-// are already in B-operand layout for O^T += V^T P^T.  V is transposed on its
-// way into LDS.  Key tiles come from the depth-0 segment (cut at the tile's
-// largest query position) and, for depth-1 query tiles, from the depth-1
+// are already in B-operand layout for O^T += V^T P^T.  K and V tiles are
+// copied global -> LDS asynchronously (global_load_lds, no registers), sit
+// row-major and swizzled there, and the V^T operand is read column-wise with
+// ds_read_b64_tr_b16.  Key tiles come from the depth-0 segment (cut at the
+// tile's largest query position) and, for depth-1 query tiles, from the depth-1
 // segment; the two-axis mask is evaluated per element only on tiles that
-// straddle a query position, and waves skip tiles that lie entirely above
-// their rows.
+// straddle a query position (a separate, mask-free instance of the tile body
+// handles the rest), and waves skip tiles that lie entirely above their rows.
 #include <hip/hip_runtime.h>
+
+#include <type_traits>
 
 #include "duo_device.h"
 #include "tah_duo.h"
@@ -24,7 +28,7 @@ constexpr int kD = 128;        // head_dim
 constexpr int kBN = 64;        // keys per tile
 constexpr int kThreads = 512;  // 8 waves
 constexpr int kKBytes = kBN * kD * 2;         // 16 KiB, [key][d]
-constexpr int kVBytes = kD * kBN * 2;         // 16 KiB, [d][key slot]
+constexpr int kVBytes = kBN * kD * 2;         // 16 KiB, [key][d]
 constexpr int kStageBytes = kKBytes + kVBytes + kBN * 4;  // + key positions
 constexpr int kSmemBytes = 2 * kStageBytes + 64;          // double buffered + tile bounds
 
@@ -42,13 +46,10 @@ struct FwdParams {
     float scale_log2e;
 };
 
-struct Prefetch {
-    bf16x8 k[2], v[2];
-    int kpos;
-};
+enum class Mask { kNone, kIndex, kPos };
 
 template <int G>
-__global__ __launch_bounds__(kThreads) void duo_fwd_kernel(const FwdParams p) {
+__global__ __launch_bounds__(kThreads) TAH_WAVES_PER_EU(2, 2) void duo_fwd_kernel(const FwdParams p) {
     constexpr int BM = 32 * (8 / G);
     HIP_DYNAMIC_SHARED(unsigned char, smem)
 
@@ -112,9 +113,18 @@ __global__ __launch_bounds__(kThreads) void duo_fwd_kernel(const FwdParams p) {
 #pragma unroll
     for (int w = 0; w < 8; ++w) tmax1 = bounds[w] > tmax1 ? bounds[w] : tmax1;
 
+    // Tile schedule.  All waves walk the same n1 + n2 tiles (one barrier each); what a wave does
+    // with a depth-0 tile depends on where the tile lies relative to the wave's own rows:
+    //   [0, n_plain)         every key visible to every row of the wave: no mask code at all
+    //   [n_plain, n_active)  tile straddles a row's position: per-element index mask
+    //   [n_active, n1)       tile wholly above the wave's rows: no compute
+    // followed by the n2 depth-1 tiles (per-element position mask).
     const int n1 = tmax1 >= 0 ? tmax1 / kBN + 1 : 0;
     const int n2 = second ? (lk2 + kBN - 1) / kBN : 0;
     const int ntiles = n1 + n2;
+    const int n_active = wmax1 >= 0 ? wmax1 / kBN + 1 : 0;
+    int n_plain = wmin1 >= kBN - 1 ? (wmin1 - (kBN - 1)) / kBN + 1 : 0;
+    n_plain = n_plain < n_active ? n_plain : n_active;
 
     // ---- Q fragments: B operand of S^T = K Q^T ------------------------------
     bf16x8 qf[8];
@@ -133,8 +143,10 @@ __global__ __launch_bounds__(kThreads) void duo_fwd_kernel(const FwdParams p) {
     float l_run = 0.f;      // this lane's share of the running denominator
     const float c = p.scale_log2e;
 
-    // ---- global -> register prefetch of one K/V tile ------------------------
-    auto prefetch = [&](int it, Prefetch& pf) {
+    // ---- asynchronous global -> LDS copy of one K/V tile (no registers, no ds_write) ----------
+    // 16 blocks of 4 rows per tile, two per wave; lane l fills row 4*blk + l/16, physical chunk
+    // l%16, i.e. fetches logical chunk (l%16) ^ row_swizzle(row) of that row.
+    auto issue_tile = [&](int it, int buf) {
         const bool s0 = it < n1;
         const int base = (s0 ? it : it - n1) * kBN;
         const __bf16* kp_ = s0 ? k1p : k2p;
@@ -142,99 +154,76 @@ __global__ __launch_bounds__(kThreads) void duo_fwd_kernel(const FwdParams p) {
         const int64_t krs = s0 ? p.s1.k_rs : p.s2.k_rs;
         const int64_t vrs = s0 ? p.s1.v_rs : p.s2.v_rs;
         const int left = s0 ? left1 : left2;  // clamp keeps tail loads inside the array
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int cidx = tid + kThreads * i;  // 1024 chunks of 16 B
-            int r = base + cidx / 16;
-            r = r < left ? r : left - 1;
-            pf.k[i] = ld_global_16B(kp_ + (int64_t)r * krs + (cidx % 16) * 8);
-        }
-        {
-            const int dc = tid % 16, kp = tid / 16;  // 8 d values x key pair (2kp, 2kp+1)
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                int r = base + 2 * kp + i;
-                r = r < left ? r : left - 1;
-                pf.v[i] = ld_global_16B(vp_ + (int64_t)r * vrs + dc * 8);
-            }
-        }
-        pf.kpos = 0x7fffffff;
-        if (!s0 && tid < kBN && base + tid < lk2) pf.kpos = pos2p[base + tid];
-    };
-    auto stage = [&](int buf, const Prefetch& pf) {
         unsigned char* kt = smem + buf * kStageBytes;
         unsigned char* vt = kt + kKBytes;
-        int* kpos = reinterpret_cast<int*>(vt + kVBytes);
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            const int cidx = tid + kThreads * i;
-            *reinterpret_cast<bf16x8*>(kt + rowmajor128_off(cidx / 16, cidx % 16)) = pf.k[i];
+            const int blk = 2 * wave + i;
+            const int lrow = 4 * blk + (lane >> 4);
+            int r = base + lrow;
+            r = r < left ? r : left - 1;
+            const int chunk = (lane & 15) ^ row_swizzle(lrow);
+            async_copy_16B(kp_ + (int64_t)r * krs + chunk * 8, kt + blk * 1024);
+            async_copy_16B(vp_ + (int64_t)r * vrs + chunk * 8, vt + blk * 1024);
         }
-        const int dc = tid % 16, kp = tid / 16;
-        const int slot2 = pv_slot(2 * kp);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int d = dc * 8 + i;
-            bf16x2 pr;
-            pr[0] = pf.v[0][i];
-            pr[1] = pf.v[1][i];
-            *reinterpret_cast<bf16x2*>(vt + rowmajor64_off(d, slot2 / 8) + (slot2 % 8) * 2) = pr;
-        }
-        if (tid < kBN) kpos[tid] = pf.kpos;
+        if (!s0 && tid < kBN)
+            reinterpret_cast<int*>(vt + kVBytes)[tid] = base + tid < lk2 ? pos2p[base + tid] : 0x7fffffff;
+    };
+    // publish tile `it` (stage it & 1) and start fetching the next one into the other stage
+    auto advance = [&](int it) {
+        TAH_WAIT_VMEM();   // my share of tile `it` has landed
+        __syncthreads();   // everybody's has; everybody is done reading the other stage
+        if (it + 1 < ntiles) issue_tile(it + 1, (it & 1) ^ 1);
     };
 
-    Prefetch pf;
-    if (ntiles > 0) prefetch(0, pf);
-
-    for (int it = 0; it < ntiles; ++it) {
-        const int buf = it & 1;
-        stage(buf, pf);
-        __syncthreads();
-        if (it + 1 < ntiles) prefetch(it + 1, pf);
-
-        const bool first_seg = it < n1;
-        const int base = (first_seg ? it : it - n1) * kBN;
-        // Depth-0 tiles entirely above this wave's rows contribute nothing.
-        if (first_seg && base > wmax1) continue;
-
-        const unsigned char* kt = smem + buf * kStageBytes;
-        const unsigned char* vt = kt + kKBytes;
-        const int* kpos = reinterpret_cast<const int*>(vt + kVBytes);
-
-        // S^T (64 keys x 32 queries) = K Q^T
-        f32x16 sacc[2];
+    // per-lane LDS read offsets (tile-relative), computed once
+    int koff[8];       // K row `col` (+32 per mt), chunk 2s + half
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt)
+    for (int s8 = 0; s8 < 8; ++s8) koff[s8] = rowmajor128_off(col, 2 * s8 + half);
+    int voff_lo[4], voff_hi[4];  // V rows 4*half + r/4 (+8), columns 32*dt + 16*grp + 4*(r%4), +16 rows per step
+    {
+        const int r16 = lane & 15, grp = (lane >> 4) & 1;
+        const int vrow = 4 * half + (r16 >> 2);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) sacc[mt][r] = 0.f;
-#pragma unroll
-        for (int s = 0; s < 8; ++s) {
-#pragma unroll
-            for (int mt = 0; mt < 2; ++mt) {
-                const bf16x8 a = *reinterpret_cast<const bf16x8*>(kt + rowmajor128_off(32 * mt + col, 2 * s + half));
-                sacc[mt] = mfma32(a, qf[s], sacc[mt]);
-            }
+        for (int dt = 0; dt < 4; ++dt) {
+            const int vcol = 32 * dt + 16 * grp + 4 * (r16 & 3);
+            voff_lo[dt] = rowmajor128_off(vrow, vcol >> 3) + (vcol & 7) * 2;
+            voff_hi[dt] = rowmajor128_off(vrow + 8, vcol >> 3) + (vcol & 7) * 2;
         }
+    }
 
-        // two-axis mask: only where the tile straddles a query position
-        if (first_seg) {
-            if (base + kBN - 1 > wmin1) {
+    // ---- one key tile: S^T = K Q^T, mask, online softmax, O^T += V^T P^T -----------------------
+    auto tile = [&](int it, auto mask_tag) __attribute__((always_inline)) {
+        constexpr Mask kMask = decltype(mask_tag)::value;
+        const unsigned char* kt = smem + (it & 1) * kStageBytes;
+        const unsigned char* vt = kt + kKBytes;
+
+        f32x16 sacc[2];
+        {
+            const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt)
+                sacc[mt] = mfma32(*reinterpret_cast<const bf16x8*>(kt + koff[0] + mt * 8192), qf[0], zero);
+#pragma unroll
+            for (int s = 1; s < 8; ++s)
 #pragma unroll
                 for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int key = base + 32 * mt + acc_row(half, r);
-                        sacc[mt][r] = key <= qlim1 ? sacc[mt][r] : kNegInf;
-                    }
-            }
-        } else {
+                    sacc[mt] = mfma32(*reinterpret_cast<const bf16x8*>(kt + koff[s] + mt * 8192), qf[s], sacc[mt]);
+        }
+        if constexpr (kMask == Mask::kIndex) {
+            const int base = it * kBN;
 #pragma unroll
             for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int kp = kpos[32 * mt + acc_row(half, r)];
-                    sacc[mt][r] = kp <= qlim2 ? sacc[mt][r] : kNegInf;
-                }
+                for (int r = 0; r < 16; ++r)
+                    sacc[mt][r] = base + 32 * mt + acc_row(half, r) <= qlim1 ? sacc[mt][r] : kNegInf;
+        } else if constexpr (kMask == Mask::kPos) {
+            const int* kpos = reinterpret_cast<const int*>(vt + kVBytes);
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    sacc[mt][r] = kpos[32 * mt + acc_row(half, r)] <= qlim2 ? sacc[mt][r] : kNegInf;
         }
 
         // online softmax, one query per lane column (two lanes per query)
@@ -261,23 +250,32 @@ __global__ __launch_bounds__(kThreads) void duo_fwd_kernel(const FwdParams p) {
             }
         l_run = l_run * alpha + psum;
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+        for (int dt = 0; dt < 4; ++dt) oacc[dt] = oacc[dt] * alpha;
 
-        // O^T (128 d x 32 queries) += V^T P^T
+        // O^T (128 d x 32 queries) += V^T P^T, V^T read column-wise from the row-major tile
 #pragma unroll
         for (int st = 0; st < 4; ++st) {
 #pragma unroll
             for (int dt = 0; dt < 4; ++dt) {
-                const bf16x8 a = *reinterpret_cast<const bf16x8*>(vt + rowmajor64_off(32 * dt + col, 2 * st + half));
-                oacc[dt] = mfma32(a, pfrag[st], oacc[dt]);
+                const bf16x4 lo = lds_read_tr16(vt + voff_lo[dt] + st * 4096);
+                const bf16x4 hi = lds_read_tr16(vt + voff_hi[dt] + st * 4096);
+                oacc[dt] = mfma32(__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7), pfrag[st], oacc[dt]);
             }
         }
-    }
+    };
+    using PlainTag = std::integral_constant<Mask, Mask::kNone>;
+    using IndexTag = std::integral_constant<Mask, Mask::kIndex>;
+    using PosTag = std::integral_constant<Mask, Mask::kPos>;
+
+    if (ntiles > 0) issue_tile(0, 0);
+    int it = 0;
+    for (; it < n_plain; ++it) { advance(it); tile(it, PlainTag{}); }
+    for (; it < n_active; ++it) { advance(it); tile(it, IndexTag{}); }
+    for (; it < n1; ++it) advance(it);
+    for (; it < ntiles; ++it) { advance(it); tile(it, PosTag{}); }
 
     // ---- epilogue -----------------------------------------------------------
-    const float l_tot = l_run + __shfl_xor(l_run, 32);
+    const float l_tot = wave_sum_xor32(l_run);
     const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
     if (row_ok) {
         __bf16* orow = qs.o + (int64_t)row * qs.o_rs + (int64_t)head * qs.o_hs;

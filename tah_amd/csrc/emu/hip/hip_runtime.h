@@ -29,6 +29,9 @@
 #include <vector>
 
 #define TAH_CPU_EMU 1
+#define TAH_MUL_INPLACE(x, a) ((x) *= (a))
+#define TAH_WAIT_VMEM() ((void)0)
+#define TAH_WAVES_PER_EU(lo, hi)
 #define __global__
 #define __device__
 #define __host__
@@ -232,6 +235,22 @@ inline float emu_fdot2_bits(uint32_t a, uint32_t b, float c) {
 }
 #define __builtin_amdgcn_fdot2_f32_bf16(a, b, c, clamp) \
     emu_fdot2_bits(__builtin_bit_cast(uint32_t, (a)), __builtin_bit_cast(uint32_t, (b)), (c))
+inline unsigned __float_as_uint(float x) { unsigned i; memcpy(&i, &x, 4); return i; }
+inline float __uint_as_float(unsigned i) { float x; memcpy(&x, &i, 4); return x; }
+// v_permlane32_swap(a, b): lanes < 32 get (a[l], a[l+32]); lanes >= 32 get (b[l-32], b[l]).
+struct emu_u32pair { unsigned v[2]; unsigned operator[](int i) const { return v[i]; } };
+inline emu_u32pair emu_permlane32_swap(unsigned a, unsigned b, bool, bool) {
+    unsigned mine[2] = {a, b};
+    memcpy(emu::t_wave->box[emu::t_lane], mine, 8);
+    emu::wave_sync();
+    const int l = emu::t_lane;
+    unsigned lo[2], hi[2];
+    memcpy(lo, emu::t_wave->box[l & 31], 8);
+    memcpy(hi, emu::t_wave->box[(l & 31) + 32], 8);
+    emu::wave_sync();
+    return l < 32 ? emu_u32pair{{lo[0], hi[0]}} : emu_u32pair{{lo[1], hi[1]}};
+}
+#define __builtin_amdgcn_permlane32_swap emu_permlane32_swap
 inline int __float_as_int(float x) { int i; memcpy(&i, &x, 4); return i; }
 inline float __int_as_float(int i) { float x; memcpy(&x, &i, 4); return x; }
 // DPP lane selects used by the kernels: quad_perm, row_shl/shr, row_mirror, row_half_mirror.
@@ -270,6 +289,10 @@ inline uint64_t emu_ds_read_tr16_b64(const void* p) {
 }
 #define __builtin_amdgcn_ds_read_tr16_b64_v4bf16(p) \
     __builtin_bit_cast(emu_bf16x4, emu_ds_read_tr16_b64((const void*)(p)))
+
+// global_load_lds: lane l copies `size` bytes from its global address to lds_base + size*l (synchronously here).
+#define __builtin_amdgcn_global_load_lds(g, l, size, off, aux) \
+    memcpy((unsigned char*)(void*)(l) + (off) + (size) * emu::t_lane, (const void*)(g), (size))
 
 #define __builtin_amdgcn_exp2f(x) exp2f(x)
 #define __builtin_amdgcn_logf(x) log2f(x)
