@@ -12,7 +12,8 @@ import os
 from . import _capi
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libtah_duo.so")
+# TAH_DUO_LIB: developer override naming another build of the same library (kernel tuning).
+LIB_PATH = os.environ.get("TAH_DUO_LIB") or os.path.join(_HERE, "libtah_duo.so")
 _lib = None
 
 

@@ -40,18 +40,33 @@ __device__ __forceinline__ bf16x8 ld_global_16B(const __bf16* p) { return *reint
 __device__ __forceinline__ void st_global_16B(__bf16* p, bf16x8 v) { *reinterpret_cast<bf16x8*>(p) = v; }
 
 // Asynchronous global -> LDS copy of 16 bytes per lane (global_load_lds_dwordx4): lane l's bytes
-// land at lds_wave_base + 16*l; lds_wave_base must be wave-uniform.  Completion is tracked by
-// vmcnt: call wait_vmem() before the barrier that publishes the tile.
+// land at lds_wave_base + 16*l; lds_wave_base must be wave-uniform.  Issued through inline
+// assembly on purpose: the compiler then does not order later LDS reads of *other* tiles behind
+// this copy (it cannot prove they do not alias and would wait for vmcnt(0) in the middle of the
+// compute phase).  Completion is tracked by vmcnt: TAH_WAIT_VMEM() before the barrier that
+// publishes the tile.
+#ifndef TAH_ASYNC_COPY_16B
+#define TAH_ASYNC_COPY_16B(gsrc, lds_wave_base)                                                                    \
+    do {                                                                                                           \
+        const unsigned tah_m0_ = __builtin_amdgcn_readfirstlane(                                                   \
+            (unsigned)(uintptr_t)(__attribute__((address_space(3))) void*)(lds_wave_base));                        \
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"                             \
+                     :                                                                                             \
+                     : "s"(tah_m0_), "v"(gsrc)                                                                     \
+                     : "memory");  /* m0 is reserved: the compiler reloads it before each own use */                                                                            \
+    } while (0)
+#endif
 __device__ __forceinline__ void async_copy_16B(const void* gsrc, unsigned char* lds_wave_base) {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
-                                     (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+    TAH_ASYNC_COPY_16B(gsrc, lds_wave_base);
 }
 // Occupancy the kernel is written for; lets the scheduler spend registers on latency hiding.
 #ifndef TAH_WAVES_PER_EU
 #define TAH_WAVES_PER_EU(lo, hi) __attribute__((amdgpu_waves_per_eu(lo, hi)))
 #endif
 #ifndef TAH_WAIT_VMEM
-#define TAH_WAIT_VMEM() asm volatile("s_waitcnt vmcnt(0)" ::: "memory")
+// s_waitcnt vmcnt(0) (expcnt/lgkmcnt untouched) as a builtin, so the compiler's own wait-count
+// bookkeeping also learns that no ordinary load is pending past this point.
+#define TAH_WAIT_VMEM() __builtin_amdgcn_s_waitcnt(0x0F70)
 #endif
 
 // LDS tile of R rows x 128 bf16 (256 B per row, 16 chunks of 16 B).  The chunk index is XORed

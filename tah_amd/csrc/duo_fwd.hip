@@ -21,6 +21,10 @@
 #include "duo_device.h"
 #include "tah_duo.h"
 
+#ifndef TAH_FWD_SCHED
+#define TAH_FWD_SCHED 1
+#endif
+
 namespace tah {
 namespace {
 
@@ -156,6 +160,9 @@ __global__ __launch_bounds__(kThreads) TAH_WAVES_PER_EU(2, 2) void duo_fwd_kerne
         const int left = s0 ? left1 : left2;  // clamp keeps tail loads inside the array
         unsigned char* kt = smem + buf * kStageBytes;
         unsigned char* vt = kt + kKBytes;
+        // key positions first: the wait for this ordinary load must not sit behind the async copies
+        if (!s0 && tid < kBN)
+            reinterpret_cast<int*>(vt + kVBytes)[tid] = base + tid < lk2 ? pos2p[base + tid] : 0x7fffffff;
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             const int blk = 2 * wave + i;
@@ -166,8 +173,6 @@ __global__ __launch_bounds__(kThreads) TAH_WAVES_PER_EU(2, 2) void duo_fwd_kerne
             async_copy_16B(kp_ + (int64_t)r * krs + chunk * 8, kt + blk * 1024);
             async_copy_16B(vp_ + (int64_t)r * vrs + chunk * 8, vt + blk * 1024);
         }
-        if (!s0 && tid < kBN)
-            reinterpret_cast<int*>(vt + kVBytes)[tid] = base + tid < lk2 ? pos2p[base + tid] : 0x7fffffff;
     };
     // publish tile `it` (stage it & 1) and start fetching the next one into the other stage
     auto advance = [&](int it) {
@@ -210,6 +215,16 @@ __global__ __launch_bounds__(kThreads) TAH_WAVES_PER_EU(2, 2) void duo_fwd_kerne
                 for (int mt = 0; mt < 2; ++mt)
                     sacc[mt] = mfma32(*reinterpret_cast<const bf16x8*>(kt + koff[s] + mt * 8192), qf[s], sacc[mt]);
         }
+#if TAH_FWD_SCHED >= 1
+        // keep six K fragments in flight ahead of the MFMAs that consume them
+        __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+#pragma unroll
+        for (int i = 0; i < 5; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 6, 0);
+#endif
         if constexpr (kMask == Mask::kIndex) {
             const int base = it * kBN;
 #pragma unroll
@@ -262,11 +277,27 @@ __global__ __launch_bounds__(kThreads) TAH_WAVES_PER_EU(2, 2) void duo_fwd_kerne
                 oacc[dt] = mfma32(__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7), pfrag[st], oacc[dt]);
             }
         }
+#if TAH_FWD_SCHED >= 2
+        // V^T fragments four MFMAs ahead; the exp/convert work of later key groups fills the MFMA shadows
+        __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+        for (int i = 0; i < 12; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+        }
+#endif
     };
     using PlainTag = std::integral_constant<Mask, Mask::kNone>;
     using IndexTag = std::integral_constant<Mask, Mask::kIndex>;
     using PosTag = std::integral_constant<Mask, Mask::kPos>;
 
+    TAH_WAIT_VMEM();  // Q fragments are in: no ordinary load stays pending across the tile loop
     if (ntiles > 0) issue_tile(0, 0);
     int it = 0;
     for (; it < n_plain; ++it) { advance(it); tile(it, PlainTag{}); }
