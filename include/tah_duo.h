@@ -152,7 +152,8 @@ size_t tah_duo_decode_workspace_bytes(int32_t nq, int32_t hq, int32_t capacity1,
 /* Decode step of duo-causal attention against the KV cache: every query row
  * attends to the depth-0 rows of its sequence with index <= q_pos, and, if it
  * is a depth-1 query, to the depth-1 rows with pos <= q_pos.  Split-K over
- * 512-row chunks of both segments plus a merge kernel.  Replaces, for Tq == 1:
+ * 1024-row chunks of both segments, then a merge kernel.
+ * Calls that share a workspace must be ordered on one stream.  Replaces, for Tq == 1:
  *   TaHForCausalLM._build_attention_mask        tah/model/tah_model.py:744-791
  *   TaHCache.get_cache_upto_iter (cat it1|it2)   tah/model/causal_cache.py:101-109
  *   sdpa_attention_forward                       transformers/integrations/sdpa_attention.py:79-166

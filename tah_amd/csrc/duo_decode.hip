@@ -1,14 +1,17 @@
 // Duo-causal decode step against the KV cache (bandwidth-bound), gfx950.
 //
-// Split-K: one workgroup (4 waves) streams one 512-row chunk of one kv head of
+// Split-K: one workgroup (4 waves) streams one 1024-row chunk of one kv head of
 // one query's sequence, from the depth-0 slab or (depth-1 queries only) the
 // depth-1 slab, for all G = Hq/Hkv query heads at once so K and V are read from
-// HBM exactly once.  A wave covers 128 consecutive rows; each load instruction
+// HBM exactly once.  A wave covers 256 consecutive rows; each load instruction
 // moves 1 KiB of contiguous cache (4 rows x 256 B, 16 B per lane).  Scores use
 // v_dot2_f32_bf16 on the packed bf16 pairs plus a 16-lane DPP reduction; the
 // online softmax runs per group of 4 rows so the accumulator is rescaled once
 // per 16 rows.  Partial (max, sum, acc) triples go to a workspace and a second
-// small kernel merges the chunks of each query.
+// small kernel merges the chunks of each (query, head), eight chunks at a time.
+// (Merging in the workgroup that finishes last would need device-scope fences,
+// which cost an L2 write-back per item across the eight XCDs; a persistent grid
+// striding over the items balanced worse than the hardware dispatcher.)
 #include <hip/hip_runtime.h>
 
 #include "duo_device.h"
@@ -18,11 +21,21 @@ namespace tah {
 namespace {
 
 constexpr int kD = 128;
-constexpr int kChunk = 512;          // rows per workgroup
-constexpr int kDecThreads = 256;     // 4 waves x 128 rows
+#ifndef TAH_DEC_NT
+#define TAH_DEC_NT 1   // streaming (nontemporal) K/V loads: every cache row is read exactly once
+#endif
+#ifndef TAH_DEC_CHUNK
+#define TAH_DEC_CHUNK 1024
+#endif
+#ifndef TAH_DEC_UNROLL
+#define TAH_DEC_UNROLL 4
+#endif
+constexpr int kChunk = TAH_DEC_CHUNK;  // rows per workgroup
+constexpr int kDecThreads = 256;     // 4 waves x (kChunk / 4) rows
 constexpr int kRowsPerWave = kChunk / 4;
-constexpr int kUnroll = 4;           // 4 loads of 4 rows in flight per wave and tensor
+constexpr int kUnroll = TAH_DEC_UNROLL;  // loads of 4 rows in flight per wave and tensor
 constexpr int kPart = kD + 2;        // acc[128], m, l  (floats per partial)
+
 
 struct Seg {
     const __bf16 *k, *v;
@@ -80,153 +93,179 @@ __global__ __launch_bounds__(kDecThreads) void duo_decode_split_kernel(const Dec
 
     const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
     const int kq = lane / 16, dc = lane % 16;  // row within a 4-row load, 8-element d slice
-    const int chunk = blockIdx.x, qi = blockIdx.y, hk = blockIdx.z;
-    const bool second = chunk >= p.nchunk1;
-    const int cidx = second ? chunk - p.nchunk1 : chunk;
-    const int slot = p.q_slot[qi];
-    const int qpos = p.q_pos[qi];
-    const int qdepth = p.q_depth ? p.q_depth[qi] : p.depth;
-    const int nvis = visible_len(p, second, slot, qpos, qdepth);
-    const int row0 = cidx * kChunk;
-    if (row0 >= nvis) return;  // uniform per workgroup
-    const Seg& sg = second ? p.c2 : p.c1;
-    const int row_end = row0 + kChunk < nvis ? row0 + kChunk : nvis;
-    const int64_t base_row = sg.start[slot];
-    const __bf16* kbase = sg.k + base_row * sg.k_rs + (int64_t)hk * sg.k_hs + dc * 8;
-    const __bf16* vbase = sg.v + base_row * sg.v_rs + (int64_t)hk * sg.v_hs + dc * 8;
-    const int32_t* posbase = second ? sg.pos + (int64_t)slot * sg.capacity : nullptr;
+    const int nslots = p.nchunk1 + p.nchunk2;
+    {
+        const int chunk = blockIdx.x, qi = blockIdx.y, hk = blockIdx.z;
+        const bool second = chunk >= p.nchunk1;
+        const int cidx = second ? chunk - p.nchunk1 : chunk;
+        const int slot = p.q_slot[qi];
+        const int qpos = p.q_pos[qi];
+        const int qdepth = p.q_depth ? p.q_depth[qi] : p.depth;
+        const int nvis = visible_len(p, second, slot, qpos, qdepth);
+        const int row0 = cidx * kChunk;
+        if (row0 >= nvis) return;  // uniform per workgroup
+        const Seg& sg = second ? p.c2 : p.c1;
+        const int row_end = row0 + kChunk < nvis ? row0 + kChunk : nvis;
+        const int64_t base_row = sg.start[slot];
+        const __bf16* kbase = sg.k + base_row * sg.k_rs + (int64_t)hk * sg.k_hs + dc * 8;
+        const __bf16* vbase = sg.v + base_row * sg.v_rs + (int64_t)hk * sg.v_hs + dc * 8;
+        const int32_t* posbase = second ? sg.pos + (int64_t)slot * sg.capacity : nullptr;
 
-    // query slices: packed bf16 pairs for the dot products
-    u32x4 qv[G];
+        // query slices: packed bf16 pairs for the dot products
+        u32x4 qv[G];
 #pragma unroll
-    for (int g = 0; g < G; ++g)
-        qv[g] = *reinterpret_cast<const u32x4*>(p.q + (int64_t)qi * p.q_rs + (int64_t)(hk * G + g) * p.q_hs + dc * 8);
+        for (int g = 0; g < G; ++g)
+            qv[g] = *reinterpret_cast<const u32x4*>(p.q + (int64_t)qi * p.q_rs + (int64_t)(hk * G + g) * p.q_hs + dc * 8);
 
-    float m_run[G], l_run[G], acc[G][8];
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-        m_run[g] = kNegInf;
-        l_run[g] = 0.f;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) acc[g][i] = 0.f;
-    }
-
-    const int wrow0 = row0 + wave * kRowsPerWave;
-    for (int it = 0; it < kRowsPerWave / (4 * kUnroll); ++it) {
-        const int r_it = wrow0 + it * 4 * kUnroll;
-        if (r_it >= row_end) break;  // uniform per wave
-        u32x4 kreg[kUnroll], vreg[kUnroll];
-        int kpos[kUnroll];
-        bool ok[kUnroll];
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            const int r = r_it + u * 4 + kq;
-            ok[u] = r < row_end;
-            const int rl = ok[u] ? r : row_end - 1;  // keep tail loads inside the slab
-            kreg[u] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)rl * sg.k_rs);
-            vreg[u] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)rl * sg.v_rs);
-            kpos[u] = second ? posbase[rl] : 0;
-        }
-        float s[kUnroll][G];
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            const bool vis = ok[u] && (!second || kpos[u] <= qpos);
-#pragma unroll
-            for (int g = 0; g < G; ++g) {
-                float d = 0.f;
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    d = dot2_acc(kreg[u][i], qv[g][i], d);
-                d = row16_sum(d) * p.scale_log2e;
-                s[u][g] = vis ? d : kNegInf;
-            }
-        }
+        float m_run[G], l_run[G], acc[G][8];
 #pragma unroll
         for (int g = 0; g < G; ++g) {
-            float mx = m_run[g];
+            m_run[g] = kNegInf;
+            l_run[g] = 0.f;
 #pragma unroll
-            for (int u = 0; u < kUnroll; ++u) mx = fmaxf(mx, s[u][g]);
-            const float m_use = mx == kNegInf ? 0.f : mx;
-            const float alpha = fast_exp2(m_run[g] - m_use);
-            m_run[g] = mx;
-            float pr[kUnroll], psum = 0.f;
+            for (int i = 0; i < 8; ++i) acc[g][i] = 0.f;
+        }
+
+        const int wrow0 = row0 + wave * kRowsPerWave;
+        for (int it = 0; it < kRowsPerWave / (4 * kUnroll); ++it) {
+            const int r_it = wrow0 + it * 4 * kUnroll;
+            if (r_it >= row_end) break;  // uniform per wave
+            u32x4 kreg[kUnroll], vreg[kUnroll];
+            int kpos[kUnroll];
+            bool ok[kUnroll];
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u) {
-                pr[u] = fast_exp2(s[u][g] - m_use);
-                psum += pr[u];
+                const int r = r_it + u * 4 + kq;
+                ok[u] = r < row_end;
+                const int rl = ok[u] ? r : row_end - 1;  // keep tail loads inside the slab
+#if TAH_DEC_NT
+                kreg[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kbase + (int64_t)rl * sg.k_rs));
+                vreg[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vbase + (int64_t)rl * sg.v_rs));
+#else
+                kreg[u] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)rl * sg.k_rs);
+                vreg[u] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)rl * sg.v_rs);
+#endif
+                kpos[u] = second ? posbase[rl] : 0;
             }
-            l_run[g] = l_run[g] * alpha + psum;
+            float s[kUnroll][G];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) acc[g][i] *= alpha;
+            for (int u = 0; u < kUnroll; ++u) {
+                const bool vis = ok[u] && (!second || kpos[u] <= qpos);
 #pragma unroll
-            for (int u = 0; u < kUnroll; ++u)
+                for (int g = 0; g < G; ++g) {
+                    float d = 0.f;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    acc[g][2 * i] += pr[u] * bf16_lo(vreg[u][i]);
-                    acc[g][2 * i + 1] += pr[u] * bf16_hi(vreg[u][i]);
+                    for (int i = 0; i < 4; ++i) d = dot2_acc(kreg[u][i], qv[g][i], d);
+                    d = row16_sum(d) * p.scale_log2e;
+                    s[u][g] = vis ? d : kNegInf;
                 }
+            }
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                float mx = m_run[g];
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u) mx = fmaxf(mx, s[u][g]);
+                const float m_use = mx == kNegInf ? 0.f : mx;
+                const float alpha = fast_exp2(m_run[g] - m_use);
+                m_run[g] = mx;
+                float pr[kUnroll], psum = 0.f;
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u) {
+                    pr[u] = fast_exp2(s[u][g] - m_use);
+                    psum += pr[u];
+                }
+                l_run[g] = l_run[g] * alpha + psum;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc[g][i] *= alpha;
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        acc[g][2 * i] += pr[u] * bf16_lo(vreg[u][i]);
+                        acc[g][2 * i + 1] += pr[u] * bf16_hi(vreg[u][i]);
+                    }
+            }
         }
-    }
 
-    // ---- merge the 16 (wave, row group) partials of this workgroup ----------
-    const int grp = wave * 4 + kq;
+        // ---- merge the 16 (wave, row group) partials of this workgroup ----------
+        const int grp = wave * 4 + kq;
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
+        for (int g = 0; g < G; ++g) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) red[grp][g][dc * 8 + i] = acc[g][i];
-        if (dc == 0) {
-            red[grp][g][kD] = m_run[g];
-            red[grp][g][kD + 1] = l_run[g];
+            for (int i = 0; i < 8; ++i) red[grp][g][dc * 8 + i] = acc[g][i];
+            if (dc == 0) {
+                red[grp][g][kD] = m_run[g];
+                red[grp][g][kD + 1] = l_run[g];
+            }
         }
-    }
-    __syncthreads();
-    const int nslots = p.nchunk1 + p.nchunk2;
-    for (int e = tid; e < G * kD; e += kDecThreads) {
-        const int g = e / kD, d = e % kD;
-        float mx = kNegInf;
+        __syncthreads();
+        for (int e = tid; e < G * kD; e += kDecThreads) {
+            const int g = e / kD, d = e % kD;
+            float mx = kNegInf;
 #pragma unroll
-        for (int j = 0; j < 16; ++j) mx = fmaxf(mx, red[j][g][kD]);
-        const float m_use = mx == kNegInf ? 0.f : mx;
-        float a = 0.f, l = 0.f;
+            for (int j = 0; j < 16; ++j) mx = fmaxf(mx, red[j][g][kD]);
+            const float m_use = mx == kNegInf ? 0.f : mx;
+            float a = 0.f, l = 0.f;
 #pragma unroll
-        for (int j = 0; j < 16; ++j) {
-            const float w = fast_exp2(red[j][g][kD] - m_use);
-            a += w * red[j][g][d];
-            l += w * red[j][g][kD + 1];
+            for (int j = 0; j < 16; ++j) {
+                const float w = fast_exp2(red[j][g][kD] - m_use);
+                a += w * red[j][g][d];
+                l += w * red[j][g][kD + 1];
+            }
+            float* out = p.ws + ((int64_t)(qi * p.hq + hk * G + g) * nslots + chunk) * kPart;
+            out[d] = a;
+            if (d == 0) {
+                out[kD] = mx;
+                out[kD + 1] = l;
+            }
         }
-        float* out = p.ws + ((int64_t)(qi * p.hq + hk * G + g) * nslots + chunk) * kPart;
-        out[d] = a;
-        if (d == 0) {
-            out[kD] = mx;
-            out[kD + 1] = l;
-        }
+
     }
 }
 
-// One workgroup of 128 threads per (query, head): merge the chunk partials.
-__global__ __launch_bounds__(kD) void duo_decode_merge_kernel(const DecParams p) {
-    const int qi = blockIdx.x, head = blockIdx.y, d = threadIdx.x;
+// Merge the chunk partials of one (query, head): 256 threads = 8 chunk lanes x 32 threads of four
+// d values, so the chunks are read eight at a time with float4 loads instead of one after another.
+__global__ __launch_bounds__(256) void duo_decode_merge_kernel(const DecParams p) {
+    __shared__ float mbuf[64];
+    __shared__ float red4[8][kD + 4];
+    const int qi = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
     const int slot = p.q_slot[qi];
     const int qpos = p.q_pos[qi];
     const int qdepth = p.q_depth ? p.q_depth[qi] : p.depth;
     const int n1 = (visible_len(p, false, slot, qpos, qdepth) + kChunk - 1) / kChunk;
     const int n2 = (visible_len(p, true, slot, qpos, qdepth) + kChunk - 1) / kChunk;
-    const int nslots = p.nchunk1 + p.nchunk2;
+    const int n = n1 + n2, nslots = p.nchunk1 + p.nchunk2;
     const float* part = p.ws + (int64_t)(qi * p.hq + head) * nslots * kPart;
+    auto slot_of = [&](int c) { return c < n1 ? c : p.nchunk1 + (c - n1); };
+    // global max over the chunk maxima (n <= a few dozen; 64 per pass)
     float mx = kNegInf;
-    for (int c = 0; c < n1; ++c) mx = fmaxf(mx, part[(int64_t)c * kPart + kD]);
-    for (int c = 0; c < n2; ++c) mx = fmaxf(mx, part[(int64_t)(p.nchunk1 + c) * kPart + kD]);
+    for (int c0 = 0; c0 < n; c0 += 64) {
+        if (tid < 64) mbuf[tid] = c0 + tid < n ? part[(int64_t)slot_of(c0 + tid) * kPart + kD] : kNegInf;
+        __syncthreads();
+        for (int j = 0; j < 64; ++j) mx = fmaxf(mx, mbuf[j]);
+        __syncthreads();
+    }
     const float m_use = mx == kNegInf ? 0.f : mx;
-    float a = 0.f, l = 0.f;
-    for (int c = 0; c < n1 + n2; ++c) {
-        const float* pc = part + (int64_t)(c < n1 ? c : p.nchunk1 + (c - n1)) * kPart;
+    const int cl = tid / 32, d4 = (tid % 32) * 4;
+    f32x4 a = {0.f, 0.f, 0.f, 0.f};
+    float l = 0.f;
+    for (int c = cl; c < n; c += 8) {
+        const float* pc = part + (int64_t)slot_of(c) * kPart;
         const float w = fast_exp2(pc[kD] - m_use);
-        a += w * pc[d];
+        a[0] += w * pc[d4]; a[1] += w * pc[d4 + 1]; a[2] += w * pc[d4 + 2]; a[3] += w * pc[d4 + 3];
         l += w * pc[kD + 1];
     }
-    const float inv = l > 0.f ? 1.0f / l : 0.f;
-    p.o[(int64_t)qi * p.o_rs + (int64_t)head * p.o_hs + d] = (__bf16)(a * inv);
-    if (p.lse && d == 0) p.lse[(int64_t)qi * p.hq + head] = l > 0.f ? (mx + fast_log2(l)) * kLn2 : kNegInf;
+    red4[cl][d4] = a[0]; red4[cl][d4 + 1] = a[1]; red4[cl][d4 + 2] = a[2]; red4[cl][d4 + 3] = a[3];
+    if (d4 == 0) red4[cl][kD] = l;
+    __syncthreads();
+    if (tid < kD) {
+        float o = 0.f, lt = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { o += red4[j][tid]; lt += red4[j][kD]; }
+        const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+        p.o[(int64_t)qi * p.o_rs + (int64_t)head * p.o_hs + tid] = (__bf16)(o * inv);
+        if (p.lse && tid == 0) p.lse[(int64_t)qi * p.hq + head] = lt > 0.f ? (mx + fast_log2(lt)) * kLn2 : kNegInf;
+    }
 }
 
 // ---- KV append --------------------------------------------------------------
@@ -304,7 +343,7 @@ int check_seg(const tah_kv_segment& s, bool need_pos) {
 template <int G>
 int launch_decode(const DecParams& p, hipStream_t st) {
     hipLaunchKernelGGL(duo_decode_split_kernel<G>, dim3(p.nchunk1 + p.nchunk2, p.nq, p.hkv), dim3(kDecThreads), 0, st, p);
-    hipLaunchKernelGGL(duo_decode_merge_kernel, dim3(p.nq, p.hq), dim3(kD), 0, st, p);
+    hipLaunchKernelGGL(duo_decode_merge_kernel, dim3(p.nq, p.hq), dim3(256), 0, st, p);
     return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
 }
 
@@ -325,7 +364,7 @@ extern "C" int tah_duo_decode(const tah_duo_decode_args* a, tah_stream_t stream)
     const int g = a->hq / a->hkv;
     if (g != 1 && g != 2 && g != 4) return TAH_E_SHAPE;  // merge buffer for 8 heads would not fit static LDS
     if (a->nq == 0) return TAH_OK;
-    if (a->nq > 65535 || a->hkv > 65535) return TAH_E_SHAPE;
+    if (a->nq > 65535 || a->hq > 65535) return TAH_E_SHAPE;
     if (!a->q || !a->o || !a->q_slot || !a->q_pos || !a->workspace) return TAH_E_NULL;
     if (!aligned16(a->q) || !aligned16(a->workspace) || a->q_row_stride % 8 || a->q_head_stride % 8) return TAH_E_ALIGN;
     if (int rc = check_seg(a->c1, false)) return rc;

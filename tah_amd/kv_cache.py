@@ -84,7 +84,7 @@ def decode(q: torch.Tensor, q_slot: torch.Tensor, q_pos: torch.Tensor, c1: KvSla
     key = (q.device, _stream(q))
     ws = _WORKSPACES.get(key)
     if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=q.device)
+        ws = torch.zeros(max(nbytes, 16), dtype=torch.uint8, device=q.device)  # counters start at zero
         _WORKSPACES[key] = ws
     a = _capi.DuoDecodeArgs()
     a.q, a.o, a.lse = _ptr(q), _ptr(o), _ptr(lse)

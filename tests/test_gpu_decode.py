@@ -106,4 +106,4 @@ def test_decode_rejects_small_workspace_and_bad_shapes():
     assert lib.tah_duo_decode(ctypes.byref(a), None) == -2
     a.d = 128
     assert lib.tah_duo_decode(ctypes.byref(a), None) == -1
-    assert lib.tah_duo_decode_workspace_bytes(64, 16, 16384, 2048) == 64 * 16 * (32 + 4) * 130 * 4
+    assert lib.tah_duo_decode_workspace_bytes(64, 16, 16384, 2048) == 64 * 16 * (16 + 2) * 130 * 4
