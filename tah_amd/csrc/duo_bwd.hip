@@ -5,7 +5,7 @@
 //   dq        one workgroup per query tile, same tiling as the forward:
 //             S^T = K Q^T, dP^T = V dO^T, dS^T = P^T o (dP^T - delta),
 //             dQ^T += K^T dS^T  (K^T operand via LDS transpose reads)
-//   dkdv      one workgroup (4 waves) per 64-key tile of one kv head; loops
+//   dkdv      one workgroup (8 waves) per 128-key tile of one kv head; loops
 //             over every query tile that can see it, for all query heads of
 //             the group and for both query streams (depth-0 keys collect
 //             gradient from depth-0 and depth-1 queries):
@@ -15,6 +15,8 @@
 // workgroup; Q and dO tiles are staged in LDS and read both row-wise (A
 // operand) and, through ds_read_b64_tr_b16, column-wise (B operand).
 #include <hip/hip_runtime.h>
+
+#include <type_traits>
 
 #include "duo_device.h"
 #include "tah_duo.h"
@@ -75,13 +77,10 @@ constexpr int kDqThreads = 512;
 constexpr int kDqStage = 2 * kTileBytes + kBN * 4;   // K tile, V tile, key positions
 constexpr int kDqSmem = 2 * kDqStage + 64;
 
-struct KvPrefetch {
-    bf16x8 k[2], v[2];
-    int kpos;
-};
+enum class Mask { kNone, kIndex, kPos };
 
 template <int G>
-__global__ __launch_bounds__(kDqThreads) void duo_bwd_dq_kernel(const BwdParams p) {
+__global__ __launch_bounds__(kDqThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dq_kernel(const BwdParams p) {
     constexpr int BM = 32 * (8 / G);
     HIP_DYNAMIC_SHARED(unsigned char, smem)
     const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
@@ -135,9 +134,13 @@ __global__ __launch_bounds__(kDqThreads) void duo_bwd_dq_kernel(const BwdParams 
     int tmax1 = -1;
 #pragma unroll
     for (int w = 0; w < 8; ++w) tmax1 = bounds[w] > tmax1 ? bounds[w] : tmax1;
+    // same tile schedule as the forward kernel: plain / index-masked / idle depth-0 tiles, then depth-1 tiles
     const int n1 = tmax1 >= 0 ? tmax1 / kBN + 1 : 0;
     const int n2 = second ? (lk2 + kBN - 1) / kBN : 0;
     const int ntiles = n1 + n2;
+    const int n_active = wmax1 >= 0 ? wmax1 / kBN + 1 : 0;
+    int n_plain = wmin1 >= kBN - 1 ? (wmin1 - (kBN - 1)) / kBN + 1 : 0;
+    n_plain = n_plain < n_active ? n_plain : n_active;
 
     bf16x8 qf[8], dof[8];
     {
@@ -159,7 +162,8 @@ __global__ __launch_bounds__(kDqThreads) void duo_bwd_dq_kernel(const BwdParams 
 #pragma unroll
         for (int r = 0; r < 16; ++r) dqacc[i][r] = 0.f;
 
-    auto prefetch = [&](int it, KvPrefetch& pf) {
+    // asynchronous global -> LDS copy of one K/V tile (both row-major, swizzled), as in the forward kernel
+    auto issue_tile = [&](int it, int buf) {
         const bool s0 = it < n1;
         const int base = (s0 ? it : it - n1) * kBN;
         const __bf16* kp_ = s0 ? k1p : k2p;
@@ -167,78 +171,77 @@ __global__ __launch_bounds__(kDqThreads) void duo_bwd_dq_kernel(const BwdParams 
         const int64_t krs = s0 ? p.s1.k_rs : p.s2.k_rs;
         const int64_t vrs = s0 ? p.s1.v_rs : p.s2.v_rs;
         const int left = s0 ? left1 : left2;
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int cidx = tid + kDqThreads * i;
-            int r = base + cidx / 16;
-            r = r < left ? r : left - 1;
-            pf.k[i] = ld_global_16B(kp_ + (int64_t)r * krs + (cidx % 16) * 8);
-            pf.v[i] = ld_global_16B(vp_ + (int64_t)r * vrs + (cidx % 16) * 8);
-        }
-        pf.kpos = 0x7fffffff;
-        if (!s0 && tid < kBN && base + tid < lk2) pf.kpos = pos2p[base + tid];
-    };
-    auto stage = [&](int buf, const KvPrefetch& pf) {
         unsigned char* kt = smem + buf * kDqStage;
         unsigned char* vt = kt + kTileBytes;
-        int* kpos = reinterpret_cast<int*>(vt + kTileBytes);
+        if (!s0 && tid < kBN)
+            reinterpret_cast<int*>(vt + kTileBytes)[tid] = base + tid < lk2 ? pos2p[base + tid] : 0x7fffffff;
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            const int cidx = tid + kDqThreads * i;
-            *reinterpret_cast<bf16x8*>(kt + rowmajor128_off(cidx / 16, cidx % 16)) = pf.k[i];
-            *reinterpret_cast<bf16x8*>(vt + rowmajor128_off(cidx / 16, cidx % 16)) = pf.v[i];
+            const int blk = 2 * wave + i;
+            const int lrow = 4 * blk + (lane >> 4);
+            int r = base + lrow;
+            r = r < left ? r : left - 1;
+            const int chunk = (lane & 15) ^ row_swizzle(lrow);
+            async_copy_16B(kp_ + (int64_t)r * krs + chunk * 8, kt + blk * 1024);
+            async_copy_16B(vp_ + (int64_t)r * vrs + chunk * 8, vt + blk * 1024);
         }
-        if (tid < kBN) kpos[tid] = pf.kpos;
+    };
+    auto advance = [&](int it) {
+        TAH_WAIT_VMEM();
+        __syncthreads();
+        if (it + 1 < ntiles) issue_tile(it + 1, (it & 1) ^ 1);
     };
 
-    KvPrefetch pf;
-    if (ntiles > 0) prefetch(0, pf);
-    for (int it = 0; it < ntiles; ++it) {
-        const int buf = it & 1;
-        stage(buf, pf);
-        __syncthreads();
-        if (it + 1 < ntiles) prefetch(it + 1, pf);
-        const bool first_seg = it < n1;
-        const int base = (first_seg ? it : it - n1) * kBN;
-        if (first_seg && base > wmax1) continue;
-        const unsigned char* kt = smem + buf * kDqStage;
+    int koff[8];
+#pragma unroll
+    for (int s8 = 0; s8 < 8; ++s8) koff[s8] = rowmajor128_off(col, 2 * s8 + half);
+
+    auto tile = [&](int it, auto mask_tag) __attribute__((always_inline)) {
+        constexpr Mask kMask = decltype(mask_tag)::value;
+        const unsigned char* kt = smem + (it & 1) * kDqStage;
         const unsigned char* vt = kt + kTileBytes;
         const int* kpos = reinterpret_cast<const int*>(vt + kTileBytes);
-        const bool need_mask = !first_seg || base + kBN - 1 > wmin1;
-
+        const int base = (it < n1 ? it : it - n1) * kBN;
+        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         bf16x8 dsf[4];
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt) {
-            f32x16 sacc, dpacc;
+            // S^T = K Q^T and dP^T = V dO^T for 32 keys x 32 queries
+            f32x16 sacc = mfma32(*reinterpret_cast<const bf16x8*>(kt + koff[0] + mt * 8192), qf[0], zero);
+            f32x16 dpacc = mfma32(*reinterpret_cast<const bf16x8*>(vt + koff[0] + mt * 8192), dof[0], zero);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; dpacc[r] = 0.f; }
-#pragma unroll
-            for (int s = 0; s < 8; ++s) {
-                const bf16x8 ka = *reinterpret_cast<const bf16x8*>(kt + rowmajor128_off(32 * mt + col, 2 * s + half));
-                sacc = mfma32(ka, qf[s], sacc);
-                const bf16x8 va = *reinterpret_cast<const bf16x8*>(vt + rowmajor128_off(32 * mt + col, 2 * s + half));
-                dpacc = mfma32(va, dof[s], dpacc);
+            for (int s = 1; s < 8; ++s) {
+                sacc = mfma32(*reinterpret_cast<const bf16x8*>(kt + koff[s] + mt * 8192), qf[s], sacc);
+                dpacc = mfma32(*reinterpret_cast<const bf16x8*>(vt + koff[s] + mt * 8192), dof[s], dpacc);
             }
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 bool vis = true;
-                if (need_mask) {
-                    const int kl = 32 * mt + acc_row(half, r);
-                    vis = first_seg ? (base + kl <= qlim1) : (kpos[kl] <= qlim2);
-                }
+                const int kl = 32 * mt + acc_row(half, r);
+                if constexpr (kMask == Mask::kIndex) vis = base + kl <= qlim1;
+                if constexpr (kMask == Mask::kPos) vis = kpos[kl] <= qlim2;
                 const float pr = vis ? fast_exp2(sacc[r] * c - lse_c) : 0.f;
                 dsf[2 * mt + r / 8][r % 8] = (__bf16)(pr * (dpacc[r] - delta));
             }
         }
-        // dQ^T (128 d x 32 queries) += K^T dS^T
+        // dQ^T (128 d x 32 queries) += K^T dS^T, K^T read column-wise from the row-major tile
 #pragma unroll
         for (int st = 0; st < 4; ++st)
 #pragma unroll
-            for (int dt = 0; dt < 4; ++dt) {
-                const bf16x8 a = lds_read_rows_as_k(kt, 16 * st, 32 * dt, lane);
-                dqacc[dt] = mfma32(a, dsf[st], dqacc[dt]);
-            }
-    }
+            for (int dt = 0; dt < 4; ++dt)
+                dqacc[dt] = mfma32(lds_read_rows_as_k(kt, 16 * st, 32 * dt, lane), dsf[st], dqacc[dt]);
+    };
+    using PlainTag = std::integral_constant<Mask, Mask::kNone>;
+    using IndexTag = std::integral_constant<Mask, Mask::kIndex>;
+    using PosTag = std::integral_constant<Mask, Mask::kPos>;
+
+    TAH_WAIT_VMEM();  // Q / dO fragments, lse and delta are in
+    if (ntiles > 0) issue_tile(0, 0);
+    int it = 0;
+    for (; it < n_plain; ++it) { advance(it); tile(it, PlainTag{}); }
+    for (; it < n_active; ++it) { advance(it); tile(it, IndexTag{}); }
+    for (; it < n1; ++it) advance(it);
+    for (; it < ntiles; ++it) { advance(it); tile(it, PosTag{}); }
 
     if (row_ok) {
         __bf16* drow = qs.dq + (int64_t)row * qs.dq_rs + (int64_t)head * qs.dq_hs;
@@ -257,30 +260,27 @@ __global__ __launch_bounds__(kDqThreads) void duo_bwd_dq_kernel(const BwdParams 
 // ---------------------------------------------------------------------------
 // dK/dV kernel
 // ---------------------------------------------------------------------------
-constexpr int kKvThreads = 256;
+constexpr int kKvThreads = 512;                           // 8 waves = 4 key blocks x 2 query halves
+constexpr int kKB = 4;                                    // 32-key blocks per workgroup
+constexpr int kBK = 32 * kKB;                             // keys per workgroup
 constexpr int kBQ = 64;                                   // query rows per staged tile
-constexpr int kKvStage = 2 * kTileBytes + 3 * kBQ * 4;    // Q tile, dO tile, lse, delta, qpos
-constexpr int kKvSmem = 2 * kKvStage;                     // double buffered (>= 64 KiB for the final reduction)
-
-struct QPrefetch {
-    bf16x8 q[4], g[4];
-    float lse, delta;
-    int qpos;
-};
+constexpr int kKvStage = 2 * kTileBytes + 3 * kBQ * 4;    // Q tile, dO tile, lse, delta, query positions
+constexpr int kKvRed = kKB * 128 * 64 * 4;                // final reduction: [key block][128 regs][64 lanes] f32
+constexpr int kKvSmem = 2 * kKvStage > kKvRed ? 2 * kKvStage : kKvRed;
 
 template <int G>
-__global__ __launch_bounds__(kKvThreads) void duo_bwd_dkdv_kernel(const BwdParams p) {
+__global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkdv_kernel(const BwdParams p) {
     HIP_DYNAMIC_SHARED(unsigned char, smem)
     const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
     const int half = lane / 32, col = lane % 32;
-    const int kb = wave % 2, qh = wave / 2;  // 32-key block, 32-row half of the query tile
+    const int kb = wave % kKB, qh = wave / kKB;  // 32-key block, 32-row half of the query tile
     const int hk = blockIdx.x;
 
     int slot = (int)blockIdx.y;
     int seq = 0, key0 = 0, key_end = 0;
     bool second = false;
-    if (!(p.s1.total_k > 0 && find_tile(p.s1.cu_k, p.nseq, kBN, slot, seq, key0, key_end))) {
-        if (!(p.s2.total_k > 0 && find_tile(p.s2.cu_k, p.nseq, kBN, slot, seq, key0, key_end))) return;
+    if (!(p.s1.total_k > 0 && find_tile(p.s1.cu_k, p.nseq, kBK, slot, seq, key0, key_end))) {
+        if (!(p.s2.total_k > 0 && find_tile(p.s2.cu_k, p.nseq, kBK, slot, seq, key0, key_end))) return;
         second = true;
     }
     const BwdStream& ks = second ? p.s2 : p.s1;
@@ -328,6 +328,7 @@ __global__ __launch_bounds__(kKvThreads) void duo_bwd_dkdv_kernel(const BwdParam
         for (int r = 0; r < 16; ++r) { dkacc[i][r] = 0.f; dvacc[i][r] = 0.f; }
     const float c = p.scale_log2e;
 
+    // item = (query tile, query head): rows [r0, r_end) of stream q2s, head `head`
     auto item_rows = [&](int item, bool& q2s, int& r0, int& r_end, int& head) {
         const int t = item / G;
         head = hk * G + item % G;
@@ -341,76 +342,72 @@ __global__ __launch_bounds__(kKvThreads) void duo_bwd_dkdv_kernel(const BwdParam
         }
         r_end = r0 + kBQ < r_end ? r0 + kBQ : r_end;
     };
-    auto prefetch = [&](int item, QPrefetch& pf) {
+    // asynchronous global -> LDS copy of one item: Q and dO tiles (16 blocks of 4 rows each, two per
+    // wave), then lse / delta / positions as one dword per lane (waves 0, 1, 2)
+    auto issue_item = [&](int item, int buf) {
         bool q2s;
         int r0, r_end, head;
         item_rows(item, q2s, r0, r_end, head);
         const BwdStream& qs = q2s ? p.s2 : p.s1;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int cidx = tid + kKvThreads * i;  // 1024 chunks of 16 B per tile
-            int r = r0 + cidx / 16;
-            r = r < r_end ? r : r_end - 1;
-            pf.q[i] = ld_global_16B(qs.q + (int64_t)r * qs.q_rs + (int64_t)head * qs.q_hs + (cidx % 16) * 8);
-            pf.g[i] = ld_global_16B(qs.d_o + (int64_t)r * qs.do_rs + (int64_t)head * qs.do_hs + (cidx % 16) * 8);
-        }
-        pf.lse = 0.f;
-        pf.delta = 0.f;
-        pf.qpos = -1;
-        if (tid < kBQ && r0 + tid < r_end) {
-            const int r = r0 + tid;
-            pf.lse = qs.lse[(int64_t)head * qs.total_q + r] * kLog2e;
-            pf.delta = qs.delta[(int64_t)head * qs.total_q + r];
-            pf.qpos = q2s ? qs.pos_q[r] : (r - q1_lo) + off;
-        }
-    };
-    auto stage = [&](int buf, const QPrefetch& pf) {
         unsigned char* qt = smem + buf * kKvStage;
         unsigned char* gt = qt + kTileBytes;
         float* meta = reinterpret_cast<float*>(gt + kTileBytes);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int cidx = tid + kKvThreads * i;
-            *reinterpret_cast<bf16x8*>(qt + rowmajor128_off(cidx / 16, cidx % 16)) = pf.q[i];
-            *reinterpret_cast<bf16x8*>(gt + rowmajor128_off(cidx / 16, cidx % 16)) = pf.g[i];
+        for (int i = 0; i < 2; ++i) {
+            const int blk = 2 * wave + i;
+            const int lrow = 4 * blk + (lane >> 4);
+            int r = r0 + lrow;
+            r = r < r_end ? r : r_end - 1;
+            const int chunk = (lane & 15) ^ row_swizzle(lrow);
+            async_copy_16B(qs.q + (int64_t)r * qs.q_rs + (int64_t)head * qs.q_hs + chunk * 8, qt + blk * 1024);
+            async_copy_16B(qs.d_o + (int64_t)r * qs.do_rs + (int64_t)head * qs.do_hs + chunk * 8, gt + blk * 1024);
         }
-        if (tid < kBQ) {
-            meta[tid] = pf.lse;
-            meta[kBQ + tid] = pf.delta;
-            reinterpret_cast<int*>(meta)[2 * kBQ + tid] = pf.qpos;
-        }
+        int rm = r0 + lane;
+        rm = rm < r_end ? rm : r_end - 1;
+        if (wave == 0) async_copy_4B(qs.lse + (int64_t)head * qs.total_q + rm, meta);
+        if (wave == 1) async_copy_4B(qs.delta + (int64_t)head * qs.total_q + rm, meta + kBQ);
+        if (wave == 2 && q2s) async_copy_4B(qs.pos_q + rm, meta + 2 * kBQ);
+    };
+    auto advance = [&](int item) {
+        TAH_WAIT_VMEM();
+        __syncthreads();
+        if (item + 1 < nitems) issue_item(item + 1, (item & 1) ^ 1);
     };
 
-    QPrefetch pf;
-    if (nitems > 0) prefetch(0, pf);
-    for (int item = 0; item < nitems; ++item) {
-        const int buf = item & 1;
-        stage(buf, pf);
-        __syncthreads();
-        if (item + 1 < nitems) prefetch(item + 1, pf);
+    int aoff[8];  // A-operand rows 32*qh + col of the Q / dO tiles, chunk 2s + half
+#pragma unroll
+    for (int s8 = 0; s8 < 8; ++s8) aoff[s8] = rowmajor128_off(32 * qh + col, 2 * s8 + half);
 
-        const unsigned char* qt = smem + buf * kKvStage;
+    TAH_WAIT_VMEM();  // K / V fragments are in
+    if (nitems > 0) issue_item(0, 0);
+    for (int item = 0; item < nitems; ++item) {
+        advance(item);
+        bool q2s;
+        int r0, r_end, head;
+        item_rows(item, q2s, r0, r_end, head);
+        const unsigned char* qt = smem + (item & 1) * kKvStage;
         const unsigned char* gt = qt + kTileBytes;
         const float* meta = reinterpret_cast<const float*>(gt + kTileBytes);
         const int* qposs = reinterpret_cast<const int*>(meta) + 2 * kBQ;
+        const int nvalid = r_end - r0;             // rows of the tile that exist
+        const int pos0 = (r0 - q1_lo) + off;       // depth-0 stream: position of tile row 0
 
         // S = Q K^T and dP = dO V^T for my 32 queries x 32 keys (lane = key, reg = query)
-        f32x16 sacc, dpacc;
+        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        f32x16 sacc = mfma32(*reinterpret_cast<const bf16x8*>(qt + aoff[0]), kf[0], zero);
+        f32x16 dpacc = mfma32(*reinterpret_cast<const bf16x8*>(gt + aoff[0]), vf[0], zero);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; dpacc[r] = 0.f; }
-#pragma unroll
-        for (int s = 0; s < 8; ++s) {
-            const bf16x8 qa = *reinterpret_cast<const bf16x8*>(qt + rowmajor128_off(32 * qh + col, 2 * s + half));
-            sacc = mfma32(qa, kf[s], sacc);
-            const bf16x8 ga = *reinterpret_cast<const bf16x8*>(gt + rowmajor128_off(32 * qh + col, 2 * s + half));
-            dpacc = mfma32(ga, vf[s], dpacc);
+        for (int s = 1; s < 8; ++s) {
+            sacc = mfma32(*reinterpret_cast<const bf16x8*>(qt + aoff[s]), kf[s], sacc);
+            dpacc = mfma32(*reinterpret_cast<const bf16x8*>(gt + aoff[s]), vf[s], dpacc);
         }
         bf16x8 pfr[2], dsfr[2];
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const int qr = 32 * qh + acc_row(half, r);
-            const bool vis = kpos <= qposs[qr];
-            const float pr = vis ? fast_exp2(sacc[r] * c - meta[qr]) : 0.f;
+            const int qp = q2s ? qposs[qr] : pos0 + qr;
+            const bool vis = qr < nvalid && kpos <= qp;
+            const float pr = vis ? fast_exp2(sacc[r] * c - meta[qr] * kLog2e) : 0.f;
             pfr[r / 8][r % 8] = (__bf16)pr;
             dsfr[r / 8][r % 8] = (__bf16)(pr * (dpacc[r] - meta[kBQ + qr]));
         }
@@ -428,7 +425,7 @@ __global__ __launch_bounds__(kKvThreads) void duo_bwd_dkdv_kernel(const BwdParam
 
     // ---- add the two query halves and store ---------------------------------
     __syncthreads();
-    float* red = reinterpret_cast<float*>(smem);  // [2 key blocks][128 regs][64 lanes]
+    float* red = reinterpret_cast<float*>(smem);  // [key block][128 regs][64 lanes]
     if (qh == 1) {
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt)
@@ -515,8 +512,8 @@ int launch_bwd(const BwdParams& p, hipStream_t st) {
     int qtiles = 0, ktiles = 0;
     if (p.s1.total_q > 0) qtiles += p.s1.total_q / BM + p.nseq;
     if (p.s2.total_q > 0) qtiles += p.s2.total_q / BM + p.nseq;
-    if (p.s1.total_k > 0) ktiles += p.s1.total_k / kBN + p.nseq;
-    if (p.s2.total_k > 0) ktiles += p.s2.total_k / kBN + p.nseq;
+    if (p.s1.total_k > 0) ktiles += p.s1.total_k / kBK + p.nseq;
+    if (p.s2.total_k > 0) ktiles += p.s2.total_k / kBK + p.nseq;
     if (qtiles > 0) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(&duo_bwd_dq_kernel<G>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kDqSmem) != hipSuccess)

@@ -59,6 +59,21 @@ __device__ __forceinline__ void st_global_16B(__bf16* p, bf16x8 v) { *reinterpre
 __device__ __forceinline__ void async_copy_16B(const void* gsrc, unsigned char* lds_wave_base) {
     TAH_ASYNC_COPY_16B(gsrc, lds_wave_base);
 }
+// Same with 4 bytes per lane (global_load_lds_dword): lane l's dword lands at lds_wave_base + 4*l.
+#ifndef TAH_ASYNC_COPY_4B
+#define TAH_ASYNC_COPY_4B(gsrc, lds_wave_base)                                                                     \
+    do {                                                                                                           \
+        const unsigned tah_m0_ = __builtin_amdgcn_readfirstlane(                                                   \
+            (unsigned)(uintptr_t)(__attribute__((address_space(3))) void*)(lds_wave_base));                        \
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"                               \
+                     :                                                                                             \
+                     : "s"(tah_m0_), "v"(gsrc)                                                                     \
+                     : "memory");                                                                                  \
+    } while (0)
+#endif
+__device__ __forceinline__ void async_copy_4B(const void* gsrc, void* lds_wave_base) {
+    TAH_ASYNC_COPY_4B(gsrc, lds_wave_base);
+}
 // Occupancy the kernel is written for; lets the scheduler spend registers on latency hiding.
 #ifndef TAH_WAVES_PER_EU
 #define TAH_WAVES_PER_EU(lo, hi) __attribute__((amdgpu_waves_per_eu(lo, hi)))

@@ -33,6 +33,8 @@
 #define TAH_WAIT_VMEM() ((void)0)
 #define TAH_ASYNC_COPY_16B(gsrc, lds_wave_base) \
     memcpy((unsigned char*)(lds_wave_base) + 16 * emu::t_lane, (const void*)(gsrc), 16)
+#define TAH_ASYNC_COPY_4B(gsrc, lds_wave_base) \
+    memcpy((unsigned char*)(lds_wave_base) + 4 * emu::t_lane, (const void*)(gsrc), 4)
 #define TAH_WAVES_PER_EU(lo, hi)
 #define __global__
 #define __device__
