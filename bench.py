@@ -23,6 +23,10 @@ if ROOT not in sys.path:
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, vendor figure
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a plain copy of
+# known size (profiles/*_counters.md); valid for the default workloads only.
+TRAFFIC_FWD_BYTES = 201.4e6 + 72.2e6
+TRAFFIC_DECODE_BYTES = 2.329e9 + 5.1e6 + 5.2e6 + 0.3e6
 
 
 def visible_pairs(case):
@@ -92,7 +96,7 @@ def bench_decode(steps: int, warmup: int):
     return {"workload": "configs[2]: decode step, 64 seqs, ctx U[1024,16384], 6% depth-1 rows, Hq=16, Hkv=8, D=128",
             "ms_per_step": ms, "visible_rows": rows, "algorithmic_bytes": nbytes, "hbm_gbs": gbs,
             "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
-                         "kernels": "duo_decode_split_kernel<2> + duo_decode_merge_kernel"},
+                         "traffic": TRAFFIC_DECODE_BYTES, "kernels": "duo_decode_split_kernel<2> + duo_decode_merge_kernel"},
             "tokens_per_s": nseq / (ms * 1e-3)}
 
 
@@ -203,7 +207,7 @@ def main() -> int:
         "config": {"workload": "configs[1]: duo-causal prefill forward, B=4, T=4096, Hq=16, Hkv=8, D=128, p_hard=0.06",
                    "visible_pairs_per_head": pairs, "flop_per_step": flops, "tokens_per_s": B * T / (ms * 1e-3)},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "duo_fwd_kernel<2>",
+                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_FWD_BYTES, "kernel": "duo_fwd_kernel<2>",
                      "kernel_ms": ms},
     }
     out["extra"] = extra
