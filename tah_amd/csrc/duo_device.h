@@ -59,6 +59,26 @@ __device__ __forceinline__ void st_global_16B(__bf16* p, bf16x8 v) { *reinterpre
 __device__ __forceinline__ void async_copy_16B(const void* gsrc, unsigned char* lds_wave_base) {
     TAH_ASYNC_COPY_16B(gsrc, lds_wave_base);
 }
+// Same copy addressed as wave-uniform base + per-lane 32-bit byte offset: the base lives in scalar
+// registers and advances with scalar arithmetic, the lane offsets can be loop invariant.
+#ifndef TAH_ASYNC_COPY_16B_SO
+#define TAH_ASYNC_COPY_16B_SO(sbase, voff, lds_wave_base)                                                          \
+    do {                                                                                                           \
+        const unsigned tah_m0_ = __builtin_amdgcn_readfirstlane(                                                   \
+            (unsigned)(uintptr_t)(__attribute__((address_space(3))) void*)(lds_wave_base));                        \
+        const uint64_t tah_b_ = (uint64_t)(uintptr_t)(sbase);                                                      \
+        /* the builtin returns int: narrow to 32 bits unsigned before widening, or bit 31 smears upward */      \
+        const uint64_t tah_sb_ = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((unsigned)tah_b_) |            \
+                                 ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((unsigned)(tah_b_ >> 32)) << 32); \
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"                              \
+                     :                                                                                             \
+                     : "s"(tah_m0_), "v"(voff), "s"(tah_sb_)                                                       \
+                     : "memory");                                                                                  \
+    } while (0)
+#endif
+__device__ __forceinline__ void async_copy_16B(const void* sbase, uint32_t voff, unsigned char* lds_wave_base) {
+    TAH_ASYNC_COPY_16B_SO(sbase, voff, lds_wave_base);
+}
 // Same with 4 bytes per lane (global_load_lds_dword): lane l's dword lands at lds_wave_base + 4*l.
 #ifndef TAH_ASYNC_COPY_4B
 #define TAH_ASYNC_COPY_4B(gsrc, lds_wave_base)                                                                     \
@@ -74,6 +94,34 @@ __device__ __forceinline__ void async_copy_16B(const void* gsrc, unsigned char* 
 __device__ __forceinline__ void async_copy_4B(const void* gsrc, void* lds_wave_base) {
     TAH_ASYNC_COPY_4B(gsrc, lds_wave_base);
 }
+// acc (16 floats of an MFMA accumulator) *= a, executed only if the wave-uniform `cond` is non-zero.
+// The branch lives inside the assembly so that the compiler sees one unconditional in-place update:
+// a C++ `if` around accumulator updates makes it keep two copies of the accumulators.
+#ifndef TAH_SCALE16_IF
+#define TAH_SCALE16_IF(acc, a, cond)                                                                               \
+    asm volatile(                                                                                                  \
+        "s_cmp_eq_u32 %[cd], 0\n\t"                                                                                \
+        "s_cbranch_scc1 .Ltah_skip_%=\n\t"                                                                         \
+        "v_mul_f32 %[o0], %[al], %[o0]\n\tv_mul_f32 %[o1], %[al], %[o1]\n\t"                                       \
+        "v_mul_f32 %[o2], %[al], %[o2]\n\tv_mul_f32 %[o3], %[al], %[o3]\n\t"                                       \
+        "v_mul_f32 %[o4], %[al], %[o4]\n\tv_mul_f32 %[o5], %[al], %[o5]\n\t"                                       \
+        "v_mul_f32 %[o6], %[al], %[o6]\n\tv_mul_f32 %[o7], %[al], %[o7]\n\t"                                       \
+        "v_mul_f32 %[o8], %[al], %[o8]\n\tv_mul_f32 %[o9], %[al], %[o9]\n\t"                                       \
+        "v_mul_f32 %[o10], %[al], %[o10]\n\tv_mul_f32 %[o11], %[al], %[o11]\n\t"                                   \
+        "v_mul_f32 %[o12], %[al], %[o12]\n\tv_mul_f32 %[o13], %[al], %[o13]\n\t"                                   \
+        "v_mul_f32 %[o14], %[al], %[o14]\n\tv_mul_f32 %[o15], %[al], %[o15]\n"                                     \
+        ".Ltah_skip_%=:"                                                                                           \
+        : [o0] "+v"((acc)[0]), [o1] "+v"((acc)[1]), [o2] "+v"((acc)[2]), [o3] "+v"((acc)[3]),                      \
+          [o4] "+v"((acc)[4]), [o5] "+v"((acc)[5]), [o6] "+v"((acc)[6]), [o7] "+v"((acc)[7]),                      \
+          [o8] "+v"((acc)[8]), [o9] "+v"((acc)[9]), [o10] "+v"((acc)[10]), [o11] "+v"((acc)[11]),                  \
+          [o12] "+v"((acc)[12]), [o13] "+v"((acc)[13]), [o14] "+v"((acc)[14]), [o15] "+v"((acc)[15])               \
+        : [al] "v"(a), [cd] "s"(cond)                                                                              \
+        : "scc")
+#endif
+// Empty statement that counts as a use of four register values at this point of the program.
+#ifndef TAH_KEEP_HERE4
+#define TAH_KEEP_HERE4(a, b, c, d) asm volatile("" ::"v"(a), "v"(b), "v"(c), "v"(d))
+#endif
 // Occupancy the kernel is written for; lets the scheduler spend registers on latency hiding.
 #ifndef TAH_WAVES_PER_EU
 #define TAH_WAVES_PER_EU(lo, hi) __attribute__((amdgpu_waves_per_eu(lo, hi)))

@@ -9,11 +9,21 @@
 // are already in B-operand layout for O^T += V^T P^T.  K and V tiles are
 // copied global -> LDS asynchronously (global_load_lds, no registers), sit
 // row-major and swizzled there, and the V^T operand is read column-wise with
-// ds_read_b64_tr_b16.  Key tiles come from the depth-0 segment (cut at the
-// tile's largest query position) and, for depth-1 query tiles, from the depth-1
-// segment; the two-axis mask is evaluated per element only on tiles that
-// straddle a query position (a separate, mask-free instance of the tile body
-// handles the rest), and waves skip tiles that lie entirely above their rows.
+// ds_read_b64_tr_b16.
+//
+// Schedule.  A wave's work per key tile t is a vector phase X(t) (mask, online
+// softmax, bf16 conversion, accumulator rescale: VALU only) and a matrix phase
+// M(t) (O^T += V(t)^T P(t)^T, then S(t+1)^T = K(t+1) Q^T: MFMA + LDS reads
+// only).  The two waves that share a SIMD are kept half a tile apart by the
+// workgroup barriers -- while waves 0-3 run X(t), waves 4-7 run M(t-1), then
+// they swap -- so the matrix pipe and the vector pipe of every SIMD are busy at
+// the same time instead of taking turns.
+//
+// Key tiles come from the depth-0 segment (cut at the tile's largest query
+// position) and, for depth-1 query tiles, from the depth-1 segment; the two-axis
+// mask is evaluated per element only on tiles that straddle a query position
+// (separate, mask-free instances of the vector phase handle the rest), and
+// waves skip the arithmetic of tiles that lie entirely above their rows.
 #include <hip/hip_runtime.h>
 
 #include <type_traits>
@@ -21,8 +31,13 @@
 #include "duo_device.h"
 #include "tah_duo.h"
 
-#ifndef TAH_FWD_SCHED
-#define TAH_FWD_SCHED 1
+// Which of the two wave sets (early / late by half a tile) a wave belongs to.  Waves w and w+4 of a
+// workgroup share a SIMD.
+#ifndef TAH_FWD_PRIO
+#define TAH_FWD_PRIO 2
+#endif
+#ifndef TAH_FWD_LATE_SET
+#define TAH_FWD_LATE_SET(wave) ((wave) >> 2)
 #endif
 
 namespace tah {
@@ -33,8 +48,14 @@ constexpr int kBN = 64;        // keys per tile
 constexpr int kThreads = 512;  // 8 waves
 constexpr int kKBytes = kBN * kD * 2;         // 16 KiB, [key][d]
 constexpr int kVBytes = kBN * kD * 2;         // 16 KiB, [key][d]
-constexpr int kStageBytes = kKBytes + kVBytes + kBN * 4;  // + key positions
-constexpr int kSmemBytes = 2 * kStageBytes + 64;          // double buffered + tile bounds
+constexpr float kLazy = 8.f;                  // log2 units the row maximum may outgrow the exponent reference
+constexpr int kStages = 2;                    // K ring and V ring depth
+constexpr int kPosSlots = 4;                  // ring of depth-1 key positions (outlives its K tile by a phase)
+constexpr int kKRing = 0;
+constexpr int kVRing = kStages * kKBytes;
+constexpr int kPosRing = kVRing + kStages * kVBytes;
+constexpr int kBoundsOff = kPosRing + kPosSlots * kBN * 4;
+constexpr int kSmemBytes = kBoundsOff + 64;
 
 struct FwdStream {
     const __bf16 *q, *k, *v;
@@ -58,7 +79,7 @@ __global__ __launch_bounds__(kThreads) TAH_WAVES_PER_EU(2, 2) void duo_fwd_kerne
     HIP_DYNAMIC_SHARED(unsigned char, smem)
 
     const int tid = threadIdx.x;
-    const int wave = tid / kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);  // wave-uniform: lives in a scalar register
     const int lane = tid % kWave;
     const int half = lane / 32;
     const int col = lane % 32;
@@ -110,7 +131,7 @@ __global__ __launch_bounds__(kThreads) TAH_WAVES_PER_EU(2, 2) void duo_fwd_kerne
     const int qlim2 = row_ok ? qpos : -1;                              // depth-1 keys: pos_k <= qlim2
     const int wmax1 = wave_reduce_max(qlim1);
     const int wmin1 = wave_reduce_min(row_ok ? qlim1 : 0x7fffffff);
-    int* bounds = reinterpret_cast<int*>(smem + 2 * kStageBytes);
+    int* bounds = reinterpret_cast<int*>(smem + kBoundsOff);
     if (lane == 0) bounds[wave] = wmax1;
     __syncthreads();
     int tmax1 = -1;
@@ -123,11 +144,12 @@ __global__ __launch_bounds__(kThreads) TAH_WAVES_PER_EU(2, 2) void duo_fwd_kerne
     //   [n_plain, n_active)  tile straddles a row's position: per-element index mask
     //   [n_active, n1)       tile wholly above the wave's rows: no compute
     // followed by the n2 depth-1 tiles (per-element position mask).
-    const int n1 = tmax1 >= 0 ? tmax1 / kBN + 1 : 0;
+    // (all wave-uniform: moved to scalar registers so that the tile loops are scalar loops)
+    const int n1 = __builtin_amdgcn_readfirstlane(tmax1 >= 0 ? tmax1 / kBN + 1 : 0);
     const int n2 = second ? (lk2 + kBN - 1) / kBN : 0;
     const int ntiles = n1 + n2;
-    const int n_active = wmax1 >= 0 ? wmax1 / kBN + 1 : 0;
-    int n_plain = wmin1 >= kBN - 1 ? (wmin1 - (kBN - 1)) / kBN + 1 : 0;
+    const int n_active = __builtin_amdgcn_readfirstlane(wmax1 >= 0 ? wmax1 / kBN + 1 : 0);
+    int n_plain = __builtin_amdgcn_readfirstlane(wmin1 >= kBN - 1 ? (wmin1 - (kBN - 1)) / kBN + 1 : 0);
     n_plain = n_plain < n_active ? n_plain : n_active;
 
     // ---- Q fragments: B operand of S^T = K Q^T ------------------------------
@@ -147,38 +169,47 @@ __global__ __launch_bounds__(kThreads) TAH_WAVES_PER_EU(2, 2) void duo_fwd_kerne
     float l_run = 0.f;      // this lane's share of the running denominator
     const float c = p.scale_log2e;
 
-    // ---- asynchronous global -> LDS copy of one K/V tile (no registers, no ds_write) ----------
-    // 16 blocks of 4 rows per tile, two per wave; lane l fills row 4*blk + l/16, physical chunk
-    // l%16, i.e. fetches logical chunk (l%16) ^ row_swizzle(row) of that row.
-    auto issue_tile = [&](int it, int buf) {
-        const bool s0 = it < n1;
-        const int base = (s0 ? it : it - n1) * kBN;
-        const __bf16* kp_ = s0 ? k1p : k2p;
-        const __bf16* vp_ = s0 ? v1p : v2p;
-        const int64_t krs = s0 ? p.s1.k_rs : p.s2.k_rs;
-        const int64_t vrs = s0 ? p.s1.v_rs : p.s2.v_rs;
-        const int left = s0 ? left1 : left2;  // clamp keeps tail loads inside the array
-        unsigned char* kt = smem + buf * kStageBytes;
-        unsigned char* vt = kt + kKBytes;
-        // key positions first: the wait for this ordinary load must not sit behind the async copies
-        if (!s0 && tid < kBN)
-            reinterpret_cast<int*>(vt + kVBytes)[tid] = base + tid < lk2 ? pos2p[base + tid] : 0x7fffffff;
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int blk = 2 * wave + i;
-            const int lrow = 4 * blk + (lane >> 4);
-            int r = base + lrow;
-            r = r < left ? r : left - 1;
-            const int chunk = (lane & 15) ^ row_swizzle(lrow);
-            async_copy_16B(kp_ + (int64_t)r * krs + chunk * 8, kt + blk * 1024);
-            async_copy_16B(vp_ + (int64_t)r * vrs + chunk * 8, vt + blk * 1024);
+    // ---- asynchronous global -> LDS copies (no registers, no ds_write) ------------------------
+    // A tile is 16 blocks of 4 rows, two per wave; lane l fills row 4*blk + l/16, physical chunk
+    // l%16, i.e. fetches logical chunk (l%16) ^ row_swizzle(row) of that row.  Rows past the end
+    // of the segment are clamped to the last row of the array (finite data, masked by index).
+    // The source is addressed as (wave-uniform pointer to the tile's first row) + (per-lane byte
+    // offset < 2^30: row strides are limited to 2^23 elements by the host-side checks).
+    const int my_lrow = 8 * wave + (lane >> 4);  // second piece: 4 rows further down
+    const uint32_t my_chunk0 = (uint32_t)(((lane & 15) ^ row_swizzle(my_lrow)) * 16);
+    const uint32_t my_chunk1 = (uint32_t)(((lane & 15) ^ row_swizzle(my_lrow + 4)) * 16);
+    auto issue_rows = [&](const __bf16* src, int64_t rs, int base, int left, unsigned char* dst) {
+        const __bf16* tile0 = src + (int64_t)base * rs;
+        const int last = left - 1 - base;  // >= 0: a tile starts inside its segment
+        const uint32_t rs2 = (uint32_t)(rs * 2) & 0xffffffu;
+        const uint32_t r0 = (uint32_t)(my_lrow < last ? my_lrow : last) & 63u;
+        const uint32_t r1 = (uint32_t)(my_lrow + 4 < last ? my_lrow + 4 : last) & 63u;
+        async_copy_16B(tile0, r0 * rs2 + my_chunk0, dst + (2 * wave) * 1024);
+        async_copy_16B(tile0, r1 * rs2 + my_chunk1, dst + (2 * wave + 1) * 1024);
+    };
+    auto issue_k = [&](int it) {  // K tile `it` -> K ring, plus the positions of depth-1 keys
+        unsigned char* kt = smem + kKRing + (it % kStages) * kKBytes;
+        if (it < n1) {
+            issue_rows(k1p, p.s1.k_rs, it * kBN, left1, kt);
+        } else {
+            const int base = (it - n1) * kBN;
+            issue_rows(k2p, p.s2.k_rs, base, left2, kt);
+            if (wave == 0) {
+                int r = base + lane;
+                r = r < lk2 ? r : lk2 - 1;
+                async_copy_4B(pos2p + r, smem + kPosRing + (it % kPosSlots) * (kBN * 4));
+            }
         }
     };
-    // publish tile `it` (stage it & 1) and start fetching the next one into the other stage
-    auto advance = [&](int it) {
-        TAH_WAIT_VMEM();   // my share of tile `it` has landed
-        __syncthreads();   // everybody's has; everybody is done reading the other stage
-        if (it + 1 < ntiles) issue_tile(it + 1, (it & 1) ^ 1);
+    auto issue_v = [&](int it) {
+        unsigned char* vt = smem + kVRing + (it % kStages) * kVBytes;
+        if (it < n1) issue_rows(v1p, p.s1.v_rs, it * kBN, left1, vt);
+        else issue_rows(v2p, p.s2.v_rs, (it - n1) * kBN, left2, vt);
+    };
+    // start of even half-phase 2u: K(u+1) replaces K(u-1), V(u) replaces V(u-2)
+    auto issue = [&](int u) {
+        if (u + 1 < ntiles) issue_k(u + 1);
+        if (u < ntiles) issue_v(u);
     };
 
     // per-lane LDS read offsets (tile-relative), computed once
@@ -197,77 +228,24 @@ __global__ __launch_bounds__(kThreads) TAH_WAVES_PER_EU(2, 2) void duo_fwd_kerne
         }
     }
 
-    // ---- one key tile: S^T = K Q^T, mask, online softmax, O^T += V^T P^T -----------------------
-    auto tile = [&](int it, auto mask_tag) __attribute__((always_inline)) {
-        constexpr Mask kMask = decltype(mask_tag)::value;
-        const unsigned char* kt = smem + (it & 1) * kStageBytes;
-        const unsigned char* vt = kt + kKBytes;
+    f32x16 sacc[2];    // S^T of the tile in flight: written by M(t-1), consumed by X(t)
+    bf16x8 pfrag[4];   // its probabilities: written by X(t), consumed by M(t)
 
-        f32x16 sacc[2];
-        {
-            const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int mt = 0; mt < 2; ++mt)
-                sacc[mt] = mfma32(*reinterpret_cast<const bf16x8*>(kt + koff[0] + mt * 8192), qf[0], zero);
-#pragma unroll
-            for (int s = 1; s < 8; ++s)
-#pragma unroll
-                for (int mt = 0; mt < 2; ++mt)
-                    sacc[mt] = mfma32(*reinterpret_cast<const bf16x8*>(kt + koff[s] + mt * 8192), qf[s], sacc[mt]);
-        }
-#if TAH_FWD_SCHED >= 1
-        // keep six K fragments in flight ahead of the MFMAs that consume them
-        __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
-#pragma unroll
-        for (int i = 0; i < 5; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, 6, 0);
-#endif
-        if constexpr (kMask == Mask::kIndex) {
-            const int base = it * kBN;
-#pragma unroll
-            for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-                for (int r = 0; r < 16; ++r)
-                    sacc[mt][r] = base + 32 * mt + acc_row(half, r) <= qlim1 ? sacc[mt][r] : kNegInf;
-        } else if constexpr (kMask == Mask::kPos) {
-            const int* kpos = reinterpret_cast<const int*>(vt + kVBytes);
-#pragma unroll
-            for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-                for (int r = 0; r < 16; ++r)
-                    sacc[mt][r] = kpos[32 * mt + acc_row(half, r)] <= qlim2 ? sacc[mt][r] : kNegInf;
-        }
-
-        // online softmax, one query per lane column (two lanes per query)
-        float mx = kNegInf;
+    // ---- matrix phase pieces -------------------------------------------------------------------
+    auto qk = [&](int it) __attribute__((always_inline)) {  // S^T = K(it) Q^T
+        const unsigned char* kt = smem + kKRing + (it % kStages) * kKBytes;
+        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
+            sacc[mt] = mfma32(*reinterpret_cast<const bf16x8*>(kt + koff[0] + mt * 8192), qf[0], zero);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[mt][r]);
-        mx = wave_max_xor32(mx);
-        const float m_new = fmaxf(m_run, mx);
-        const float m_use = m_new == kNegInf ? 0.f : m_new;
-        const float alpha = fast_exp2((m_run - m_use) * c);
-        m_run = m_new;
-        const float mc = m_use * c;
-        float psum = 0.f;
-        bf16x8 pfrag[4];
+        for (int s = 1; s < 8; ++s)
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float e = fast_exp2(sacc[mt][r] * c - mc);
-                psum += e;
-                pfrag[2 * mt + r / 8][r % 8] = (__bf16)e;
-            }
-        l_run = l_run * alpha + psum;
-#pragma unroll
-        for (int dt = 0; dt < 4; ++dt) oacc[dt] = oacc[dt] * alpha;
-
-        // O^T (128 d x 32 queries) += V^T P^T, V^T read column-wise from the row-major tile
+            for (int mt = 0; mt < 2; ++mt)
+                sacc[mt] = mfma32(*reinterpret_cast<const bf16x8*>(kt + koff[s] + mt * 8192), qf[s], sacc[mt]);
+    };
+    auto pv = [&](int it) __attribute__((always_inline)) {  // O^T (128 d x 32 queries) += V(it)^T P^T
+        const unsigned char* vt = smem + kVRing + (it % kStages) * kVBytes;
 #pragma unroll
         for (int st = 0; st < 4; ++st) {
 #pragma unroll
@@ -277,33 +255,178 @@ __global__ __launch_bounds__(kThreads) TAH_WAVES_PER_EU(2, 2) void duo_fwd_kerne
                 oacc[dt] = mfma32(__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7), pfrag[st], oacc[dt]);
             }
         }
-#if TAH_FWD_SCHED >= 2
-        // V^T fragments four MFMAs ahead; the exp/convert work of later key groups fills the MFMA shadows
+    };
+    // M(t): O^T += V(t)^T P(t)^T, then (kQk) S(t+1)^T = K(t+1) Q^T, as one straight-line block whose
+    // LDS reads run four MFMAs ahead of their consumers.
+    auto matrix = [&](int t, auto qk_tag) __attribute__((always_inline)) {
+        constexpr bool kQk = decltype(qk_tag)::value;
+#if TAH_FWD_PRIO
+        __builtin_amdgcn_s_setprio(TAH_FWD_PRIO);  // the matrix pipe is the scarce one: its wave issues first
+#endif
+        pv(t);
+        if constexpr (kQk) qk(t + 1);
         __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
 #pragma unroll
         for (int i = 0; i < 12; ++i) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
+        }
+        if constexpr (kQk) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            }
         }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
-        }
+        for (int i = 0; i < 4; ++i) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+#if TAH_FWD_PRIO
+        __builtin_amdgcn_s_setprio(0);
 #endif
+    };
+    // is tile t+1 one this wave computes?
+    auto next_active = [&](int t) { return t + 1 < n_active || (t + 1 >= n1 && t + 1 < ntiles); };
+
+    // ---- vector phase: mask, online softmax (one query per lane column, two lanes per query) ----
+    auto softmax = [&](int it, auto mask_tag) __attribute__((always_inline)) {
+        constexpr Mask kMask = decltype(mask_tag)::value;
+        if constexpr (kMask == Mask::kIndex) {
+            const int base = it * kBN;
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    sacc[mt][r] = base + 32 * mt + acc_row(half, r) <= qlim1 ? sacc[mt][r] : kNegInf;
+        } else if constexpr (kMask == Mask::kPos) {
+            const int* kpos = reinterpret_cast<const int*>(smem + kPosRing + (it % kPosSlots) * (kBN * 4));
+            const int nleft = lk2 - (it - n1) * kBN;  // keys of this tile that exist
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int kk = 32 * mt + acc_row(half, r);
+                    sacc[mt][r] = (kk < nleft && kpos[kk] <= qlim2) ? sacc[mt][r] : kNegInf;
+                }
+        }
+        float mx = kNegInf;
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[mt][r]);
+        mx = wave_max_xor32(mx);
+        // Lazy reference: the exponent reference m_run follows the true row maximum only when that
+        // has grown by more than kLazy (log2 units) for some row of the wave; until then
+        // probabilities may reach 2^kLazy, which fp32 sums and bf16 operands absorb, and the 64
+        // accumulator multiplies are skipped.  O/l and the LSE do not depend on the reference.
+        const float m_new = fmaxf(m_run, mx);
+        const bool grow = (m_new - m_run) * c > kLazy;  // true for the first finite maximum (m_run = -inf)
+        const int any_grow = __builtin_amdgcn_readfirstlane((int)(__builtin_amdgcn_ballot_w64(grow) != 0));  // wave-uniform, scalar
+        const float m_next = any_grow ? m_new : m_run;
+        const float m_use = m_next == kNegInf ? 0.f : m_next;
+        const float alpha = fast_exp2((m_run - m_use) * c);  // 1 when nothing changes, 0 from -inf
+        m_run = m_next;
+        const float mc = m_use * c;
+        float psum = 0.f;
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float e = fast_exp2(sacc[mt][r] * c - mc);
+                psum += e;
+                pfrag[2 * mt + r / 8][r % 8] = (__bf16)e;
+            }
+        l_run = l_run * alpha + psum;
+        f32x16* const op = oacc;  // (asm operands alone do not make a lambda capture the array)
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) TAH_SCALE16_IF(op[dt], alpha, any_grow);
+        // Pin the results here: without a use inside this phase the optimiser sinks the whole
+        // computation to its first consumer, i.e. past the barrier into the matrix phase.
+        TAH_KEEP_HERE4(pfrag[0], pfrag[1], pfrag[2], pfrag[3]);
+        TAH_KEEP_HERE4(op[0], op[1], op[2], op[3]);
     };
     using PlainTag = std::integral_constant<Mask, Mask::kNone>;
     using IndexTag = std::integral_constant<Mask, Mask::kIndex>;
     using PosTag = std::integral_constant<Mask, Mask::kPos>;
 
+    // Workgroup timeline: half-phases h = 0 .. 2*ntiles+1, a barrier before each.  Waves of the
+    // early set run S(0) at h=0, X(t) at h=2t+1 and M(t) at h=2t+2; waves of the late set run
+    // everything one half-phase later.  Copies are issued at the start of every even half-phase
+    // and awaited at the end of the following odd one, so a tile has two half-phases to arrive.
+    // Each barrier is a scheduling fence: nothing of a vector phase may drift into a matrix phase.
+#define TAH_PHASE_BARRIER()                      \
+    do {                                         \
+        __builtin_amdgcn_sched_barrier(0);       \
+        __syncthreads();                         \
+        __builtin_amdgcn_sched_barrier(0);       \
+    } while (0)
+    auto step_early = [&](int t, auto tag, auto qk_tag) __attribute__((always_inline)) {
+        TAH_PHASE_BARRIER();
+        softmax(t, tag);
+        TAH_WAIT_VMEM();
+        TAH_PHASE_BARRIER();
+        issue(t + 1);
+        matrix(t, qk_tag);
+    };
+    auto step_late = [&](int t, auto tag, auto qk_tag) __attribute__((always_inline)) {
+        TAH_WAIT_VMEM();
+        TAH_PHASE_BARRIER();
+        issue(t + 1);
+        softmax(t, tag);
+        TAH_PHASE_BARRIER();
+        matrix(t, qk_tag);
+    };
+    auto idle_early = [&](int t) __attribute__((always_inline)) {
+        TAH_PHASE_BARRIER();
+        TAH_WAIT_VMEM();
+        TAH_PHASE_BARRIER();
+        issue(t + 1);
+        if (next_active(t)) qk(t + 1);
+    };
+    auto idle_late = [&](int t) __attribute__((always_inline)) {
+        TAH_WAIT_VMEM();
+        TAH_PHASE_BARRIER();
+        issue(t + 1);
+        TAH_PHASE_BARRIER();
+        if (next_active(t)) qk(t + 1);
+    };
+    using WithQk = std::true_type;
+    using NoQk = std::false_type;
+    // Tiles of a run whose successor is computed too take the fused PV + QK^T block; the last tile
+    // of a run (at most one iteration of each second loop) takes the PV-only block.
+    const int act_q = next_active(n_active - 1) ? n_active : n_active - 1;  // [0, act_q): successor active
+    const int plain_q = n_plain < act_q ? n_plain : act_q;
+    auto run = [&](auto late_tag) __attribute__((always_inline)) {
+        constexpr bool kLate = decltype(late_tag)::value;
+        auto step = [&](int t, auto tag, auto qk_tag) __attribute__((always_inline)) {
+            if constexpr (kLate) step_late(t, tag, qk_tag);
+            else step_early(t, tag, qk_tag);
+        };
+        int t = 0;
+        if constexpr (kLate) TAH_PHASE_BARRIER();  // before h = 1
+        if (next_active(-1)) qk(0);
+        for (; t < plain_q; ++t) step(t, PlainTag{}, WithQk{});
+        for (; t < n_plain; ++t) step(t, PlainTag{}, NoQk{});
+        for (; t < act_q; ++t) step(t, IndexTag{}, WithQk{});
+        for (; t < n_active; ++t) step(t, IndexTag{}, NoQk{});
+        for (; t < n1; ++t) {
+            if constexpr (kLate) idle_late(t);
+            else idle_early(t);
+        }
+        for (; t < ntiles - 1; ++t) step(t, PosTag{}, WithQk{});
+        for (; t < ntiles; ++t) step(t, PosTag{}, NoQk{});
+        if constexpr (!kLate) TAH_PHASE_BARRIER();  // before h = 2*ntiles + 1
+    };
+
     TAH_WAIT_VMEM();  // Q fragments are in: no ordinary load stays pending across the tile loop
-    if (ntiles > 0) issue_tile(0, 0);
-    int it = 0;
-    for (; it < n_plain; ++it) { advance(it); tile(it, PlainTag{}); }
-    for (; it < n_active; ++it) { advance(it); tile(it, IndexTag{}); }
-    for (; it < n1; ++it) advance(it);
-    for (; it < ntiles; ++it) { advance(it); tile(it, PosTag{}); }
+    if (ntiles > 0) {
+        issue_k(0);
+        TAH_WAIT_VMEM();
+        TAH_PHASE_BARRIER();  // before h = 0
+        issue(0);
+        if (TAH_FWD_LATE_SET(wave) == 0) run(std::false_type{});
+        else run(std::true_type{});
+    }
+#undef TAH_PHASE_BARRIER
 
     // ---- epilogue -----------------------------------------------------------
     const float l_tot = wave_sum_xor32(l_run);
@@ -358,6 +481,9 @@ int check_stream(const tah_duo_stream& s, bool second) {
                           s.v_row_stride, s.v_head_stride, s.o_row_stride, s.o_head_stride};
     for (int64_t x : st)
         if (x % 8 != 0) return TAH_E_ALIGN;
+    // the tile copies address rows as base + row * stride with a 24-bit multiply
+    if (s.k_row_stride < 0 || s.v_row_stride < 0 || s.k_row_stride >= (1 << 23) || s.v_row_stride >= (1 << 23))
+        return TAH_E_SHAPE;
     return TAH_OK;
 }
 

@@ -31,8 +31,13 @@
 #define TAH_CPU_EMU 1
 #define TAH_MUL_INPLACE(x, a) ((x) *= (a))
 #define TAH_WAIT_VMEM() ((void)0)
+#define TAH_KEEP_HERE4(a, b, c, d) ((void)0)
+#define TAH_SCALE16_IF(acc, a, cond) \
+    do { if (cond) for (int tah_i_ = 0; tah_i_ < 16; ++tah_i_) (acc)[tah_i_] *= (a); } while (0)
 #define TAH_ASYNC_COPY_16B(gsrc, lds_wave_base) \
     memcpy((unsigned char*)(lds_wave_base) + 16 * emu::t_lane, (const void*)(gsrc), 16)
+#define TAH_ASYNC_COPY_16B_SO(sbase, voff, lds_wave_base) \
+    memcpy((unsigned char*)(lds_wave_base) + 16 * emu::t_lane, (const unsigned char*)(sbase) + (voff), 16)
 #define TAH_ASYNC_COPY_4B(gsrc, lds_wave_base) \
     memcpy((unsigned char*)(lds_wave_base) + 4 * emu::t_lane, (const void*)(gsrc), 4)
 #define TAH_WAVES_PER_EU(lo, hi)
@@ -182,6 +187,7 @@ inline unsigned long long __ballot(int pred) {
 }
 inline int emu_readfirstlane(int v) { return emu::exchange(v, 0); }
 #define __builtin_amdgcn_readfirstlane emu_readfirstlane
+#define __builtin_amdgcn_ballot_w64(p) __ballot(p)
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 emu_bf16x8;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float emu_f32x16;
