@@ -264,14 +264,20 @@ constexpr int kKvThreads = 512;                           // 8 waves = 4 key blo
 constexpr int kKB = 4;                                    // 32-key blocks per workgroup
 constexpr int kBK = 32 * kKB;                             // keys per workgroup
 constexpr int kBQ = 64;                                   // query rows per staged tile
-constexpr int kKvStage = 2 * kTileBytes + 3 * kBQ * 4;    // Q tile, dO tile, lse, delta, query positions
-constexpr int kKvRed = kKB * 128 * 64 * 4;                // final reduction: [key block][128 regs][64 lanes] f32
-constexpr int kKvSmem = 2 * kKvStage > kKvRed ? 2 * kKvStage : kKvRed;
+constexpr int kKvSlot = 2 * kTileBytes;                   // one stage: Q tile, dO tile (32 KiB)
+constexpr int kKvK = 2 * kKvSlot;                         // after the two stages: this workgroup's K tile (128 x 128 bf16) ...
+constexpr int kKvV = kKvK + kBK * kD * 2;                 // ... and V tile
+constexpr int kKvMeta = kKvV + kBK * kD * 2;              // then per stage: lse, delta, query positions (64 dwords each)
+constexpr int kKvMetaBytes = 3 * kBQ * 4;
+constexpr int kKvSmem = kKvMeta + 2 * kKvMetaBytes;
+constexpr int kKvRed = kKB * 128 * 64 * 4;                // final reduction: [key block][128 regs][64 lanes] f32, reuses the front
+static_assert(kKvRed <= kKvSmem, "reduction buffer must fit");
 
 template <int G>
 __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkdv_kernel(const BwdParams p) {
     HIP_DYNAMIC_SHARED(unsigned char, smem)
-    const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+    const int tid = threadIdx.x, lane = tid % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);  // wave-uniform: lives in a scalar register
     const int half = lane / 32, col = lane % 32;
     const int kb = wave % kKB, qh = wave / kKB;  // 32-key block, 32-row half of the query tile
     const int hk = blockIdx.x;
@@ -298,16 +304,27 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
     const int key_ld = key_ok ? key : key_end - 1;
     const int kpos = key_ok ? (second ? ks.pos_k[key_ld] : key_ld - k_lo) : 0x7fffffff;
 
-    bf16x8 kf[8], vf[8];  // B operands: K^T, V^T columns of my key
+    // This workgroup's K and V rows go to LDS once (row-major, swizzled like every tile): they are the
+    // B operands of S = Q K^T and dP = dO V^T, read again for every item -- keeping them in registers
+    // instead would cost 64 registers per lane for the whole kernel.
     {
-        const __bf16* kr = ks.k + (int64_t)key_ld * ks.k_rs + (int64_t)hk * ks.k_hs + 8 * half;
-        const __bf16* vr = ks.v + (int64_t)key_ld * ks.v_rs + (int64_t)hk * ks.v_hs + 8 * half;
+        const __bf16* kbase = ks.k + (int64_t)key0 * ks.k_rs + (int64_t)hk * ks.k_hs;
+        const __bf16* vbase = ks.v + (int64_t)key0 * ks.v_rs + (int64_t)hk * ks.v_hs;
+        const uint32_t krs2 = (uint32_t)(ks.k_rs * 2) & 0xffffffu, vrs2 = (uint32_t)(ks.v_rs * 2) & 0xffffffu;
+        const int last = key_end - 1 - key0;
 #pragma unroll
-        for (int s = 0; s < 8; ++s) {
-            kf[s] = ld_global_16B(kr + 16 * s);
-            vf[s] = ld_global_16B(vr + 16 * s);
+        for (int i = 0; i < 4; ++i) {  // 32 blocks of 4 rows per tile, four per wave
+            const int blk = 4 * wave + i;
+            const int lrow = 4 * blk + (lane >> 4);
+            const uint32_t lr = (uint32_t)(lrow < last ? lrow : last) & 127u;
+            const uint32_t chunk = (uint32_t)(((lane & 15) ^ row_swizzle(lrow)) * 16);
+            async_copy_16B(kbase, lr * krs2 + chunk, smem + kKvK + blk * 1024);
+            async_copy_16B(vbase, lr * vrs2 + chunk, smem + kKvV + blk * 1024);
         }
     }
+    int boff[8];  // B-operand row 32*kb + col (my key) of the K tile, chunk 2s + half; V tile: + kKvV - kKvK
+#pragma unroll
+    for (int s8 = 0; s8 < 8; ++s8) boff[s8] = kKvK + rowmajor128_off(32 * kb + col, 2 * s8 + half);
 
     // query tiles that can see this key tile
     const int kl0 = key0 - k_lo;  // local index of the tile's first key (depth-0 tiles: its position)
@@ -320,6 +337,17 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
     }
     const int nt2 = (lq2 + kBQ - 1) / kBQ;
     const int nitems = (nt1 + nt2) * G;
+    // Depth-0 query tiles [t_vis, t_whole) (relative to t1_begin) need no mask for this wave: all 64 rows
+    // exist and the first row of my half already sees the last key of my block.
+    int t_whole = lq1 / kBQ - t1_begin;
+    t_whole = t_whole < 0 ? 0 : (t_whole < nt1 ? t_whole : nt1);
+    int t_vis = 0;
+    if (!second) {
+        const int need = kl0 + 32 * kb + 31 - off - 32 * qh;  // first query row that sees my last key
+        t_vis = need > 0 ? (need + kBQ - 1) / kBQ - t1_begin : 0;
+        t_vis = t_vis < 0 ? 0 : t_vis;
+    }
+    t_vis = t_vis < t_whole ? t_vis : t_whole;
 
     f32x16 dkacc[4], dvacc[4];
 #pragma unroll
@@ -342,31 +370,34 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
         }
         r_end = r0 + kBQ < r_end ? r0 + kBQ : r_end;
     };
-    // asynchronous global -> LDS copy of one item: Q and dO tiles (16 blocks of 4 rows each, two per
-    // wave), then lse / delta / positions as one dword per lane (waves 0, 1, 2)
+    // Asynchronous global -> LDS copy of one item: Q and dO tiles (16 blocks of 4 rows each, two per
+    // wave), then lse / delta / positions as one dword per lane (waves 0, 1, 2).  Sources are
+    // (wave-uniform base of the tile) + (per-lane byte offset); rows past the end repeat the last one.
+    const int my_lrow = 8 * wave + (lane >> 4);  // second piece: 4 rows further down
+    const uint32_t my_chunk0 = (uint32_t)(((lane & 15) ^ row_swizzle(my_lrow)) * 16);
+    const uint32_t my_chunk1 = (uint32_t)(((lane & 15) ^ row_swizzle(my_lrow + 4)) * 16);
     auto issue_item = [&](int item, int buf) {
         bool q2s;
         int r0, r_end, head;
         item_rows(item, q2s, r0, r_end, head);
         const BwdStream& qs = q2s ? p.s2 : p.s1;
-        unsigned char* qt = smem + buf * kKvStage;
+        unsigned char* qt = smem + buf * kKvSlot;
         unsigned char* gt = qt + kTileBytes;
-        float* meta = reinterpret_cast<float*>(gt + kTileBytes);
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int blk = 2 * wave + i;
-            const int lrow = 4 * blk + (lane >> 4);
-            int r = r0 + lrow;
-            r = r < r_end ? r : r_end - 1;
-            const int chunk = (lane & 15) ^ row_swizzle(lrow);
-            async_copy_16B(qs.q + (int64_t)r * qs.q_rs + (int64_t)head * qs.q_hs + chunk * 8, qt + blk * 1024);
-            async_copy_16B(qs.d_o + (int64_t)r * qs.do_rs + (int64_t)head * qs.do_hs + chunk * 8, gt + blk * 1024);
-        }
-        int rm = r0 + lane;
-        rm = rm < r_end ? rm : r_end - 1;
-        if (wave == 0) async_copy_4B(qs.lse + (int64_t)head * qs.total_q + rm, meta);
-        if (wave == 1) async_copy_4B(qs.delta + (int64_t)head * qs.total_q + rm, meta + kBQ);
-        if (wave == 2 && q2s) async_copy_4B(qs.pos_q + rm, meta + 2 * kBQ);
+        float* meta = reinterpret_cast<float*>(smem + kKvMeta + buf * kKvMetaBytes);
+        const int last = r_end - 1 - r0;
+        const uint32_t l0 = (uint32_t)(my_lrow < last ? my_lrow : last) & 63u;
+        const uint32_t l1 = (uint32_t)(my_lrow + 4 < last ? my_lrow + 4 : last) & 63u;
+        const uint32_t qrs2 = (uint32_t)(qs.q_rs * 2) & 0xffffffu, grs2 = (uint32_t)(qs.do_rs * 2) & 0xffffffu;
+        const __bf16* qbase = qs.q + (int64_t)r0 * qs.q_rs + (int64_t)head * qs.q_hs;
+        const __bf16* gbase = qs.d_o + (int64_t)r0 * qs.do_rs + (int64_t)head * qs.do_hs;
+        async_copy_16B(qbase, l0 * qrs2 + my_chunk0, qt + (2 * wave) * 1024);
+        async_copy_16B(gbase, l0 * grs2 + my_chunk0, gt + (2 * wave) * 1024);
+        async_copy_16B(qbase, l1 * qrs2 + my_chunk1, qt + (2 * wave + 1) * 1024);
+        async_copy_16B(gbase, l1 * grs2 + my_chunk1, gt + (2 * wave + 1) * 1024);
+        const uint32_t lm = (uint32_t)(lane < last ? lane : last) * 4u;
+        if (wave == 0) async_copy_4B(qs.lse + (int64_t)head * qs.total_q + r0, lm, meta);
+        if (wave == 1) async_copy_4B(qs.delta + (int64_t)head * qs.total_q + r0, lm, meta + kBQ);
+        if (wave == 2 && q2s) async_copy_4B(qs.pos_q + r0, lm, meta + 2 * kBQ);
     };
     auto advance = [&](int item) {
         TAH_WAIT_VMEM();
@@ -374,56 +405,107 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
         if (item + 1 < nitems) issue_item(item + 1, (item & 1) ^ 1);
     };
 
+    // per-lane LDS read offsets inside a tile, computed once
     int aoff[8];  // A-operand rows 32*qh + col of the Q / dO tiles, chunk 2s + half
 #pragma unroll
     for (int s8 = 0; s8 < 8; ++s8) aoff[s8] = rowmajor128_off(32 * qh + col, 2 * s8 + half);
-
-    TAH_WAIT_VMEM();  // K / V fragments are in
-    if (nitems > 0) issue_item(0, 0);
-    for (int item = 0; item < nitems; ++item) {
-        advance(item);
-        bool q2s;
-        int r0, r_end, head;
-        item_rows(item, q2s, r0, r_end, head);
-        const unsigned char* qt = smem + (item & 1) * kKvStage;
-        const unsigned char* gt = qt + kTileBytes;
-        const float* meta = reinterpret_cast<const float*>(gt + kTileBytes);
-        const int* qposs = reinterpret_cast<const int*>(meta) + 2 * kBQ;
-        const int nvalid = r_end - r0;             // rows of the tile that exist
-        const int pos0 = (r0 - q1_lo) + off;       // depth-0 stream: position of tile row 0
-
-        // S = Q K^T and dP = dO V^T for my 32 queries x 32 keys (lane = key, reg = query)
-        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        f32x16 sacc = mfma32(*reinterpret_cast<const bf16x8*>(qt + aoff[0]), kf[0], zero);
-        f32x16 dpacc = mfma32(*reinterpret_cast<const bf16x8*>(gt + aoff[0]), vf[0], zero);
+    int toff_lo[4], toff_hi[4];  // transpose reads: rows 32*qh + 4*half + r/4 (+8), columns 32*dt + 16*grp + 4*(r%4)
+    {
+        const int r16 = lane & 15, grp = (lane >> 4) & 1;
+        const int trow = 32 * qh + 4 * half + (r16 >> 2);
 #pragma unroll
-        for (int s = 1; s < 8; ++s) {
-            sacc = mfma32(*reinterpret_cast<const bf16x8*>(qt + aoff[s]), kf[s], sacc);
-            dpacc = mfma32(*reinterpret_cast<const bf16x8*>(gt + aoff[s]), vf[s], dpacc);
+        for (int dt = 0; dt < 4; ++dt) {
+            const int tcol = 32 * dt + 16 * grp + 4 * (r16 & 3);
+            toff_lo[dt] = rowmajor128_off(trow, tcol >> 3) + (tcol & 7) * 2;
+            toff_hi[dt] = rowmajor128_off(trow + 8, tcol >> 3) + (tcol & 7) * 2;
         }
+    }
+    const int mrow = 32 * qh + 4 * half;  // my accumulator rows: mrow + 8*(r/4) + r%4
+
+    auto body = [&](int item, auto mask_tag) __attribute__((always_inline)) {
+        constexpr bool kMasked = decltype(mask_tag)::value;
+        const unsigned char* qt = smem + (item & 1) * kKvSlot;
+        const unsigned char* gt = qt + kTileBytes;
+        const float* meta = reinterpret_cast<const float*>(smem + kKvMeta + (item & 1) * kKvMetaBytes);
+
+        // S = Q K^T for my 32 queries x 32 keys (lane = key, reg = query), P from the saved log-sum-exp;
+        // then dP = dO V^T and dS = P o (dP - delta).  One 16-register product is live at a time, and
+        // dS is formed from the bf16 P that the dV product uses.
+        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         bf16x8 pfr[2], dsfr[2];
+        {
+            f32x16 sacc = mfma32(*reinterpret_cast<const bf16x8*>(qt + aoff[0]),
+                                 *reinterpret_cast<const bf16x8*>(smem + boff[0]), zero);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int qr = 32 * qh + acc_row(half, r);
-            const int qp = q2s ? qposs[qr] : pos0 + qr;
-            const bool vis = qr < nvalid && kpos <= qp;
-            const float pr = vis ? fast_exp2(sacc[r] * c - meta[qr] * kLog2e) : 0.f;
-            pfr[r / 8][r % 8] = (__bf16)pr;
-            dsfr[r / 8][r % 8] = (__bf16)(pr * (dpacc[r] - meta[kBQ + qr]));
+            for (int s = 1; s < 8; ++s)
+                sacc = mfma32(*reinterpret_cast<const bf16x8*>(qt + aoff[s]),
+                              *reinterpret_cast<const bf16x8*>(smem + boff[s]), sacc);
+            [[maybe_unused]] bool q2s = false;
+            [[maybe_unused]] int nvalid = kBQ, pos0 = 0;
+            [[maybe_unused]] const int* qposs = reinterpret_cast<const int*>(meta) + 2 * kBQ;
+            if constexpr (kMasked) {
+                int r0, r_end, head;
+                item_rows(item, q2s, r0, r_end, head);
+                nvalid = r_end - r0;        // rows of the tile that exist
+                pos0 = (r0 - q1_lo) + off;  // depth-0 stream: position of tile row 0
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const f32x4 lse4 = *reinterpret_cast<const f32x4*>(meta + mrow + 8 * j);  // four consecutive rows
+#pragma unroll
+                for (int b4 = 0; b4 < 4; ++b4) {
+                    const int r = 4 * j + b4;
+                    float pr = fast_exp2(sacc[r] * c - lse4[b4] * kLog2e);
+                    if constexpr (kMasked) {
+                        const int qr = mrow + 8 * j + b4;
+                        const int qp = q2s ? qposs[qr] : pos0 + qr;
+                        pr = (qr < nvalid && kpos <= qp) ? pr : 0.f;
+                    }
+                    pfr[r / 8][r % 8] = (__bf16)pr;
+                }
+            }
+        }
+        {
+            f32x16 dpacc = mfma32(*reinterpret_cast<const bf16x8*>(gt + aoff[0]),
+                                  *reinterpret_cast<const bf16x8*>(smem + (kKvV - kKvK) + boff[0]), zero);
+#pragma unroll
+            for (int s = 1; s < 8; ++s)
+                dpacc = mfma32(*reinterpret_cast<const bf16x8*>(gt + aoff[s]),
+                               *reinterpret_cast<const bf16x8*>(smem + (kKvV - kKvK) + boff[s]), dpacc);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const f32x4 del4 = *reinterpret_cast<const f32x4*>(meta + kBQ + mrow + 8 * j);
+#pragma unroll
+                for (int b4 = 0; b4 < 4; ++b4) {
+                    const int r = 4 * j + b4;
+                    dsfr[r / 8][r % 8] = (__bf16)((float)pfr[r / 8][r % 8] * (dpacc[r] - del4[b4]));
+                }
+            }
         }
         // dV (32 keys x 128 d) += P^T dO ;  dK += dS^T Q   (contraction over my 32 queries)
 #pragma unroll
         for (int st = 0; st < 2; ++st)
 #pragma unroll
             for (int dt = 0; dt < 4; ++dt) {
-                const bf16x8 gb = lds_read_rows_as_k(gt, 32 * qh + 16 * st, 32 * dt, lane);
-                dvacc[dt] = mfma32(pfr[st], gb, dvacc[dt]);
-                const bf16x8 qb = lds_read_rows_as_k(qt, 32 * qh + 16 * st, 32 * dt, lane);
-                dkacc[dt] = mfma32(dsfr[st], qb, dkacc[dt]);
+                const bf16x4 glo = lds_read_tr16(gt + toff_lo[dt] + st * 4096);
+                const bf16x4 ghi = lds_read_tr16(gt + toff_hi[dt] + st * 4096);
+                dvacc[dt] = mfma32(pfr[st], __builtin_shufflevector(glo, ghi, 0, 1, 2, 3, 4, 5, 6, 7), dvacc[dt]);
+                const bf16x4 qlo = lds_read_tr16(qt + toff_lo[dt] + st * 4096);
+                const bf16x4 qhi = lds_read_tr16(qt + toff_hi[dt] + st * 4096);
+                dkacc[dt] = mfma32(dsfr[st], __builtin_shufflevector(qlo, qhi, 0, 1, 2, 3, 4, 5, 6, 7), dkacc[dt]);
             }
-    }
+    };
+    using Masked = std::true_type;
+    using Plain = std::false_type;
+
+    if (nitems > 0) issue_item(0, 0);  // (the first barrier below also publishes the K and V tiles)
+    int item = 0;
+    for (; item < t_vis * G; ++item) { advance(item); body(item, Masked{}); }
+    for (; item < t_whole * G; ++item) { advance(item); body(item, Plain{}); }
+    for (; item < nitems; ++item) { advance(item); body(item, Masked{}); }
 
     // ---- add the two query halves and store ---------------------------------
+    TAH_WAIT_VMEM();  // no copy may still be on its way into the memory the reduction reuses
     __syncthreads();
     float* red = reinterpret_cast<float*>(smem);  // [key block][128 regs][64 lanes]
     if (qh == 1) {
@@ -498,6 +580,9 @@ int check_bwd_stream(const tah_duo_stream& s, const tah_duo_bwd_stream& g, bool 
                           s.o_row_stride, s.o_head_stride, g.do_row_stride, g.do_head_stride, g.dq_row_stride, g.dq_head_stride};
     for (int64_t x : st)
         if (x % 8 != 0) return TAH_E_ALIGN;
+    // the tile copies address rows as base + row * stride with a 24-bit multiply
+    for (int64_t x : {s.q_row_stride, s.k_row_stride, s.v_row_stride, g.do_row_stride})
+        if (x < 0 || x >= (1 << 23)) return TAH_E_SHAPE;
     return TAH_OK;
 }
 

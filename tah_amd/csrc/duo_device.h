@@ -94,6 +94,24 @@ __device__ __forceinline__ void async_copy_16B(const void* sbase, uint32_t voff,
 __device__ __forceinline__ void async_copy_4B(const void* gsrc, void* lds_wave_base) {
     TAH_ASYNC_COPY_4B(gsrc, lds_wave_base);
 }
+// 4 bytes per lane from wave-uniform base + per-lane 32-bit byte offset.
+#ifndef TAH_ASYNC_COPY_4B_SO
+#define TAH_ASYNC_COPY_4B_SO(sbase, voff, lds_wave_base)                                                           \
+    do {                                                                                                           \
+        const unsigned tah_m0_ = __builtin_amdgcn_readfirstlane(                                                   \
+            (unsigned)(uintptr_t)(__attribute__((address_space(3))) void*)(lds_wave_base));                        \
+        const uint64_t tah_b_ = (uint64_t)(uintptr_t)(sbase);                                                      \
+        const uint64_t tah_sb_ = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((unsigned)tah_b_) |            \
+                                 ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((unsigned)(tah_b_ >> 32)) << 32); \
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"                                \
+                     :                                                                                             \
+                     : "s"(tah_m0_), "v"(voff), "s"(tah_sb_)                                                       \
+                     : "memory");                                                                                  \
+    } while (0)
+#endif
+__device__ __forceinline__ void async_copy_4B(const void* sbase, uint32_t voff, void* lds_wave_base) {
+    TAH_ASYNC_COPY_4B_SO(sbase, voff, lds_wave_base);
+}
 // acc (16 floats of an MFMA accumulator) *= a, executed only if the wave-uniform `cond` is non-zero.
 // The branch lives inside the assembly so that the compiler sees one unconditional in-place update:
 // a C++ `if` around accumulator updates makes it keep two copies of the accumulators.

@@ -38,6 +38,8 @@
     memcpy((unsigned char*)(lds_wave_base) + 16 * emu::t_lane, (const void*)(gsrc), 16)
 #define TAH_ASYNC_COPY_16B_SO(sbase, voff, lds_wave_base) \
     memcpy((unsigned char*)(lds_wave_base) + 16 * emu::t_lane, (const unsigned char*)(sbase) + (voff), 16)
+#define TAH_ASYNC_COPY_4B_SO(sbase, voff, lds_wave_base) \
+    memcpy((unsigned char*)(lds_wave_base) + 4 * emu::t_lane, (const unsigned char*)(sbase) + (voff), 4)
 #define TAH_ASYNC_COPY_4B(gsrc, lds_wave_base) \
     memcpy((unsigned char*)(lds_wave_base) + 4 * emu::t_lane, (const void*)(gsrc), 4)
 #define TAH_WAVES_PER_EU(lo, hi)
