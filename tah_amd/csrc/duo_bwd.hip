@@ -21,6 +21,10 @@
 #include "duo_device.h"
 #include "tah_duo.h"
 
+#ifndef TAH_DKDV_SCHED
+#define TAH_DKDV_SCHED 1  // 1: LDS reads four MFMAs ahead; n > 1: also n vector instructions behind each dP / dV MFMA; 0: compiler order
+#endif
+
 namespace tah {
 namespace {
 
@@ -482,7 +486,8 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
                 }
             }
         }
-        // dV (32 keys x 128 d) += P^T dO ;  dK += dS^T Q   (contraction over my 32 queries)
+        // dV (32 keys x 128 d) += P^T dO, then dK += dS^T Q (contraction over my 32 queries).  All of dV
+        // first: it needs P only, so the dS arithmetic can run in the shadow of its MFMAs.
 #pragma unroll
         for (int st = 0; st < 2; ++st)
 #pragma unroll
@@ -490,10 +495,40 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
                 const bf16x4 glo = lds_read_tr16(gt + toff_lo[dt] + st * 4096);
                 const bf16x4 ghi = lds_read_tr16(gt + toff_hi[dt] + st * 4096);
                 dvacc[dt] = mfma32(pfr[st], __builtin_shufflevector(glo, ghi, 0, 1, 2, 3, 4, 5, 6, 7), dvacc[dt]);
+            }
+#pragma unroll
+        for (int st = 0; st < 2; ++st)
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt) {
                 const bf16x4 qlo = lds_read_tr16(qt + toff_lo[dt] + st * 4096);
                 const bf16x4 qhi = lds_read_tr16(qt + toff_hi[dt] + st * 4096);
                 dkacc[dt] = mfma32(dsfr[st], __builtin_shufflevector(qlo, qhi, 0, 1, 2, 3, 4, 5, 6, 7), dkacc[dt]);
             }
+#if TAH_DKDV_SCHED
+        if constexpr (!kMasked) {
+            // One straight-line block of 32 MFMAs: LDS reads run about four MFMAs ahead of their
+            // consumers; the P arithmetic sits between the dP MFMAs, the dS arithmetic between the dV ones.
+            __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+#if TAH_DKDV_SCHED > 1
+                __builtin_amdgcn_sched_group_barrier(0x002, TAH_DKDV_SCHED, 0);
+#endif
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            }
+        }
+#endif
     };
     using Masked = std::true_type;
     using Plain = std::false_type;
