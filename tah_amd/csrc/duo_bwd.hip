@@ -87,7 +87,8 @@ template <int G>
 __global__ __launch_bounds__(kDqThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dq_kernel(const BwdParams p) {
     constexpr int BM = 32 * (8 / G);
     HIP_DYNAMIC_SHARED(unsigned char, smem)
-    const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+    const int tid = threadIdx.x, lane = tid % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);  // wave-uniform: lives in a scalar register
     const int half = lane / 32, col = lane % 32;
     const int hk = blockIdx.x;
 
@@ -139,11 +140,12 @@ __global__ __launch_bounds__(kDqThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dq_
 #pragma unroll
     for (int w = 0; w < 8; ++w) tmax1 = bounds[w] > tmax1 ? bounds[w] : tmax1;
     // same tile schedule as the forward kernel: plain / index-masked / idle depth-0 tiles, then depth-1 tiles
-    const int n1 = tmax1 >= 0 ? tmax1 / kBN + 1 : 0;
+    // (all wave-uniform: moved to scalar registers so that the tile loops are scalar loops)
+    const int n1 = __builtin_amdgcn_readfirstlane(tmax1 >= 0 ? tmax1 / kBN + 1 : 0);
     const int n2 = second ? (lk2 + kBN - 1) / kBN : 0;
     const int ntiles = n1 + n2;
-    const int n_active = wmax1 >= 0 ? wmax1 / kBN + 1 : 0;
-    int n_plain = wmin1 >= kBN - 1 ? (wmin1 - (kBN - 1)) / kBN + 1 : 0;
+    const int n_active = __builtin_amdgcn_readfirstlane(wmax1 >= 0 ? wmax1 / kBN + 1 : 0);
+    int n_plain = __builtin_amdgcn_readfirstlane(wmin1 >= kBN - 1 ? (wmin1 - (kBN - 1)) / kBN + 1 : 0);
     n_plain = n_plain < n_active ? n_plain : n_active;
 
     bf16x8 qf[8], dof[8];
@@ -166,29 +168,33 @@ __global__ __launch_bounds__(kDqThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dq_
 #pragma unroll
         for (int r = 0; r < 16; ++r) dqacc[i][r] = 0.f;
 
-    // asynchronous global -> LDS copy of one K/V tile (both row-major, swizzled), as in the forward kernel
+    // asynchronous global -> LDS copy of one K/V tile (both row-major, swizzled), as in the forward
+    // kernel: (wave-uniform pointer to the tile's first row) + (per-lane byte offset), rows past the
+    // end of the array repeat its last row (finite data, masked by index)
+    const int my_lrow = 8 * wave + (lane >> 4);  // second piece: 4 rows further down
+    const uint32_t my_chunk0 = (uint32_t)(((lane & 15) ^ row_swizzle(my_lrow)) * 16);
+    const uint32_t my_chunk1 = (uint32_t)(((lane & 15) ^ row_swizzle(my_lrow + 4)) * 16);
     auto issue_tile = [&](int it, int buf) {
         const bool s0 = it < n1;
         const int base = (s0 ? it : it - n1) * kBN;
-        const __bf16* kp_ = s0 ? k1p : k2p;
-        const __bf16* vp_ = s0 ? v1p : v2p;
         const int64_t krs = s0 ? p.s1.k_rs : p.s2.k_rs;
         const int64_t vrs = s0 ? p.s1.v_rs : p.s2.v_rs;
-        const int left = s0 ? left1 : left2;
+        const __bf16* kt0 = (s0 ? k1p : k2p) + (int64_t)base * krs;
+        const __bf16* vt0 = (s0 ? v1p : v2p) + (int64_t)base * vrs;
+        const int last = (s0 ? left1 : left2) - 1 - base;  // >= 0: a tile starts inside its segment
         unsigned char* kt = smem + buf * kDqStage;
         unsigned char* vt = kt + kTileBytes;
-        if (!s0 && tid < kBN)
-            reinterpret_cast<int*>(vt + kTileBytes)[tid] = base + tid < lk2 ? pos2p[base + tid] : 0x7fffffff;
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int blk = 2 * wave + i;
-            const int lrow = 4 * blk + (lane >> 4);
-            int r = base + lrow;
-            r = r < left ? r : left - 1;
-            const int chunk = (lane & 15) ^ row_swizzle(lrow);
-            async_copy_16B(kp_ + (int64_t)r * krs + chunk * 8, kt + blk * 1024);
-            async_copy_16B(vp_ + (int64_t)r * vrs + chunk * 8, vt + blk * 1024);
+        const uint32_t r0 = (uint32_t)(my_lrow < last ? my_lrow : last) & 63u;
+        const uint32_t r1 = (uint32_t)(my_lrow + 4 < last ? my_lrow + 4 : last) & 63u;
+        const uint32_t krs2 = (uint32_t)(krs * 2) & 0xffffffu, vrs2 = (uint32_t)(vrs * 2) & 0xffffffu;
+        if (!s0 && wave == 0) {  // positions of the depth-1 keys (indices past the segment repeat the last one)
+            const int nleft = lk2 - base;
+            async_copy_4B(pos2p + base, (uint32_t)(lane < nleft ? lane : nleft - 1) * 4u, vt + kTileBytes);
         }
+        async_copy_16B(kt0, r0 * krs2 + my_chunk0, kt + (2 * wave) * 1024);
+        async_copy_16B(vt0, r0 * vrs2 + my_chunk0, vt + (2 * wave) * 1024);
+        async_copy_16B(kt0, r1 * krs2 + my_chunk1, kt + (2 * wave + 1) * 1024);
+        async_copy_16B(vt0, r1 * vrs2 + my_chunk1, vt + (2 * wave + 1) * 1024);
     };
     auto advance = [&](int it) {
         TAH_WAIT_VMEM();
@@ -199,6 +205,17 @@ __global__ __launch_bounds__(kDqThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dq_
     int koff[8];
 #pragma unroll
     for (int s8 = 0; s8 < 8; ++s8) koff[s8] = rowmajor128_off(col, 2 * s8 + half);
+    int toff_lo[4], toff_hi[4];  // transpose reads of K: rows 4*half + r/4 (+8), columns 32*dt + 16*grp + 4*(r%4)
+    {
+        const int r16 = lane & 15, grp = (lane >> 4) & 1;
+        const int trow = 4 * half + (r16 >> 2);
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) {
+            const int tcol = 32 * dt + 16 * grp + 4 * (r16 & 3);
+            toff_lo[dt] = rowmajor128_off(trow, tcol >> 3) + (tcol & 7) * 2;
+            toff_hi[dt] = rowmajor128_off(trow + 8, tcol >> 3) + (tcol & 7) * 2;
+        }
+    }
 
     auto tile = [&](int it, auto mask_tag) __attribute__((always_inline)) {
         constexpr Mask kMask = decltype(mask_tag)::value;
@@ -206,6 +223,7 @@ __global__ __launch_bounds__(kDqThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dq_
         const unsigned char* vt = kt + kTileBytes;
         const int* kpos = reinterpret_cast<const int*>(vt + kTileBytes);
         const int base = (it < n1 ? it : it - n1) * kBN;
+        [[maybe_unused]] const int nleft = lk2 - base;  // depth-1 tiles: keys of this tile that exist
         const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         bf16x8 dsf[4];
 #pragma unroll
@@ -223,7 +241,7 @@ __global__ __launch_bounds__(kDqThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dq_
                 bool vis = true;
                 const int kl = 32 * mt + acc_row(half, r);
                 if constexpr (kMask == Mask::kIndex) vis = base + kl <= qlim1;
-                if constexpr (kMask == Mask::kPos) vis = kpos[kl] <= qlim2;
+                if constexpr (kMask == Mask::kPos) vis = kl < nleft && kpos[kl] <= qlim2;
                 const float pr = vis ? fast_exp2(sacc[r] * c - lse_c) : 0.f;
                 dsf[2 * mt + r / 8][r % 8] = (__bf16)(pr * (dpacc[r] - delta));
             }
@@ -232,8 +250,11 @@ __global__ __launch_bounds__(kDqThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dq_
 #pragma unroll
         for (int st = 0; st < 4; ++st)
 #pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
-                dqacc[dt] = mfma32(lds_read_rows_as_k(kt, 16 * st, 32 * dt, lane), dsf[st], dqacc[dt]);
+            for (int dt = 0; dt < 4; ++dt) {
+                const bf16x4 lo = lds_read_tr16(kt + toff_lo[dt] + st * 4096);
+                const bf16x4 hi = lds_read_tr16(kt + toff_hi[dt] + st * 4096);
+                dqacc[dt] = mfma32(__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7), dsf[st], dqacc[dt]);
+            }
     };
     using PlainTag = std::integral_constant<Mask, Mask::kNone>;
     using IndexTag = std::integral_constant<Mask, Mask::kIndex>;
