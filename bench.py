@@ -25,7 +25,7 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, vendor figure
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a plain copy of
 # known size (profiles/*_counters.md); valid for the default workloads only.
-TRAFFIC_FWD_BYTES = 201.4e6 + 72.2e6
+TRAFFIC_FWD_BYTES = 202.2e6 + 72.2e6
 TRAFFIC_DECODE_BYTES = 2.329e9 + 5.1e6 + 5.2e6 + 0.3e6
 
 

@@ -12,6 +12,10 @@ ABI_VERSION = 1
 c_void_p, c_int32, c_int64, c_float = C.c_void_p, C.c_int32, C.c_int64, C.c_float
 
 
+# error codes of include/tah_duo.h
+TAH_OK, TAH_E_NULL, TAH_E_SHAPE, TAH_E_ALIGN, TAH_E_LAUNCH, TAH_E_WORKSPACE = 0, -1, -2, -3, -4, -5
+
+
 class DuoStream(C.Structure):
     """``tah_duo_stream``"""
 

@@ -47,6 +47,28 @@ def make_varlen_case(seed, seqlens, p_hard, Hq=16, Hkv=8, D=128, dtype=torch.flo
     )
 
 
+def add_score_drift(case, nats_per_key):
+    """Makes every depth-0 score grow with the key index by about `nats_per_key` (on top of the random
+    part): all queries get a common direction u added, key j gets j * t * u.  A running-maximum softmax
+    then has to move its reference again and again (fast drift), or only every few tiles (slow drift)."""
+    D = case["q1"].shape[-1]
+    g = torch.Generator().manual_seed(1234)
+    u = torch.randn(D, generator=g)
+    u = u / u.norm()
+    a = 4.0
+    t = nats_per_key / (a * case["scale"])
+    out = dict(case)
+    out["q1"] = case["q1"] + a * u
+    out["q2"] = case["q2"] + a * u
+    k1 = case["k1"].clone()
+    for b in range(len(case["cu_k1"]) - 1):
+        lo, hi = int(case["cu_k1"][b]), int(case["cu_k1"][b + 1])
+        j = torch.arange(hi - lo, dtype=k1.dtype)
+        k1[lo:hi] += (j * t)[:, None, None] * u
+    out["k1"] = k1
+    return out
+
+
 VARLEN_KEYS = ("q1", "k1", "v1", "cu_q1", "cu_k1", "q2", "k2", "v2", "pos_q2", "pos_k2", "cu_q2", "cu_k2", "scale")
 
 

@@ -41,3 +41,48 @@ def test_product_ops_refuse_cpu_tensors():
     from tah_amd import TahDuoError, ops
     with pytest.raises(TahDuoError):
         ops.hard_index_build(torch.zeros(2, 3, dtype=torch.bool))
+
+
+def test_argument_checks_run_before_any_device_work():
+    """Validation failures are reported from the host side alone: fake (never dereferenced) pointers
+    and no GPU are enough to see the error codes for a bad head dimension, a misaligned pointer and a
+    row stride beyond what the tile copies can address."""
+    from tah_amd import _capi, _lib
+    lib = _lib.lib()
+
+    def args():
+        a = _capi.DuoFwdArgs()
+        for s in (a.s1,):
+            s.q = s.k = s.v = s.o = 0x10000
+            s.lse = 0x20000
+            s.cu_q = s.cu_k = 0x30000
+            s.q_row_stride = s.k_row_stride = s.v_row_stride = s.o_row_stride = 1024
+            s.q_head_stride = s.k_head_stride = s.v_head_stride = s.o_head_stride = 128
+            s.total_q = s.total_k = 64
+        a.nseq, a.hq, a.hkv, a.d, a.scale = 1, 8, 8, 128, 0.1
+        return a
+
+    a = args()
+    a.d = 64
+    assert lib.tah_duo_fwd_varlen(ctypes.byref(a), None) == _capi.TAH_E_SHAPE
+    a = args()
+    a.hq, a.hkv = 24, 8  # group of 3 query heads per kv head
+    assert lib.tah_duo_fwd_varlen(ctypes.byref(a), None) == _capi.TAH_E_SHAPE
+    a = args()
+    a.s1.k = 0x10008
+    assert lib.tah_duo_fwd_varlen(ctypes.byref(a), None) == _capi.TAH_E_ALIGN
+    a = args()
+    a.s1.q = None
+    assert lib.tah_duo_fwd_varlen(ctypes.byref(a), None) == _capi.TAH_E_NULL
+    a = args()
+    a.s1.k_row_stride = 1 << 23  # rows further apart than the 24-bit multiply of the tile copies covers
+    assert lib.tah_duo_fwd_varlen(ctypes.byref(a), None) == _capi.TAH_E_SHAPE
+    b = _capi.DuoBwdArgs()
+    b.fwd = args()
+    b.fwd.s1.v_row_stride = 1 << 23
+    for g in (b.g1,):
+        g.d_o = g.dq = g.dk = g.dv = 0x40000
+        g.delta = 0x50000
+        g.do_row_stride = g.dq_row_stride = g.dk_row_stride = g.dv_row_stride = 1024
+        g.do_head_stride = g.dq_head_stride = g.dk_head_stride = g.dv_head_stride = 128
+    assert lib.tah_duo_bwd_varlen(ctypes.byref(b), None) == _capi.TAH_E_SHAPE

@@ -5,7 +5,7 @@ import torch
 
 from oracle import duo_ref as R
 from tests import emu_util
-from tests.cases import make_varlen_case, varlen_args
+from tests.cases import add_score_drift, make_varlen_case, varlen_args
 
 pytestmark = pytest.mark.skipif(not emu_util.have_host_clang(), reason="host clang++ not available")
 
@@ -46,6 +46,17 @@ def _check(dev, got):
 def test_fwd_kernel_on_cpu_shim(hq, hkv, seqlens, p):
     from tah_amd import ops
     dev = _to_dev(make_varlen_case(100 + hq, seqlens, p, Hq=hq, Hkv=hkv, D=128))
+    with emu_util.emulated():
+        got = ops.duo_fwd_varlen(*varlen_args(dev))
+    _check(dev, got)
+
+
+@pytest.mark.parametrize("nats_per_key", [0.25, 0.02])
+def test_fwd_kernel_moving_softmax_reference(nats_per_key):
+    """Scores that keep growing along the keys: per 64-key tile the row maximum rises by 16 nats (the
+    exponent reference has to follow in every tile) or by 1.3 nats (it follows only every few tiles)."""
+    from tah_amd import ops
+    dev = _to_dev(add_score_drift(make_varlen_case(21, [200], 0.2, Hq=2, Hkv=1, D=128), nats_per_key))
     with emu_util.emulated():
         got = ops.duo_fwd_varlen(*varlen_args(dev))
     _check(dev, got)

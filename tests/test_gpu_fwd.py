@@ -4,7 +4,7 @@ import pytest
 import torch
 import torch.nn.functional as F
 
-from tests.cases import dense_to_varlen, make_dense_case, make_varlen_case, varlen_args
+from tests.cases import add_score_drift, dense_to_varlen, make_dense_case, make_varlen_case, varlen_args
 from tests.gpu_util import assert_close, oracle_fwd, to_device
 
 pytestmark = pytest.mark.gpu
@@ -38,6 +38,15 @@ def test_fwd_matches_oracle(hq, hkv, seqlens, p, seed):
     print(f"case hq={hq} hkv={hkv} seqlens={seqlens} p={p} seed={seed}", flush=True)
     dev = to_device(make_varlen_case(seed, seqlens, p, Hq=hq, Hkv=hkv, D=128))
     _check(dev, _run(dev), "fwd")
+
+
+@pytest.mark.parametrize("nats_per_key", [0.25, 0.02, 0.002])
+def test_fwd_moving_softmax_reference(nats_per_key):
+    """Scores that keep growing along the keys, so that the running exponent reference must follow the
+    row maximum in every tile (fast drift), every few tiles, or almost never (slow drift)."""
+    print(f"case drift nats_per_key={nats_per_key}", flush=True)
+    dev = to_device(add_score_drift(make_varlen_case(31, [1500, 333], 0.1), nats_per_key))
+    _check(dev, _run(dev), "drift")
 
 
 def test_fwd_cache_prefix_extra_depth1_keys():
