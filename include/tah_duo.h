@@ -83,6 +83,27 @@ const char* tah_duo_error_string(int code);
  * o = 0, lse = -inf. */
 int tah_duo_fwd_varlen(const tah_duo_fwd_args* args, tah_stream_t stream);
 
+/* A dense additive attention mask as Hugging Face passes it: element
+ * [seq b][head h][query i][key j], i and j counted inside sequence b (row
+ * cu_q[b] + i, key row cu_k[b] + j), strides in elements (head_stride 0 for the
+ * usual (B,1,Tq,Tkv) mask). */
+typedef struct tah_additive_mask {
+    const void* mask;
+    int64_t seq_stride, head_stride, q_stride, k_stride;
+    int32_t dtype; /* 0: bf16, 1: float */
+} tah_additive_mask;
+
+/* Compatibility mode: softmax(q k^T * scale + mask) v with an explicit additive
+ * mask, exactly the arithmetic the reference runs today
+ *   TaHForCausalLM._build_attention_mask (the mask)  tah/model/tah_model.py:744-791
+ *   sdpa_attention_forward (repeat_kv + SDPA)         transformers/integrations/sdpa_attention.py:79-166
+ * for callers that still build the (B,1,Tq,Tkv) mask.  Only stream s1 of `args`
+ * is used (s2 must be empty); every query sees every key of its sequence and the
+ * mask alone decides.  Entries of finfo.min or -inf hide a key; a row whose keys
+ * are all hidden gets o = 0, lse = -inf.  The mask is read once per (head, tile):
+ * O(Tq*Tkv) traffic that the duo-causal entry point avoids. */
+int tah_duo_fwd_masked(const tah_duo_fwd_args* args, const tah_additive_mask* mask, tah_stream_t stream);
+
 /* Gradient tensors of one stream (same row/head layout as the forward tensors). */
 typedef struct tah_duo_bwd_stream {
     const void* d_o;        /* bf16 [total_q, Hq,  D] upstream gradient of o */
@@ -108,6 +129,12 @@ typedef struct tah_duo_bwd_args {
  * depth-0 dK/dV collect the contributions of depth-0 and depth-1 queries, summed
  * over the query heads of each kv head.  Deterministic (no atomics). */
 int tah_duo_bwd_varlen(const tah_duo_bwd_args* args, tah_stream_t stream);
+
+/* Backward of tah_duo_fwd_masked (same additive mask; no gradient is formed for
+ * the mask itself, which the reference builds from integers).  Replaces torch
+ * autograd through sdpa_attention_forward with attn_mask
+ * (transformers/integrations/sdpa_attention.py:79-166). */
+int tah_duo_bwd_masked(const tah_duo_bwd_args* args, const tah_additive_mask* mask, tah_stream_t stream);
 
 /* One depth of the native KV cache of one decoder layer.  Each sequence slot s
  * owns a slab: row j of kv head h lives at

@@ -58,6 +58,16 @@ class DuoBwdArgs(C.Structure):
     _fields_ = [("fwd", DuoFwdArgs), ("g1", DuoBwdStream), ("g2", DuoBwdStream)]
 
 
+class AdditiveMask(C.Structure):
+    """``tah_additive_mask``"""
+
+    _fields_ = [
+        ("mask", c_void_p),
+        ("seq_stride", c_int64), ("head_stride", c_int64), ("q_stride", c_int64), ("k_stride", c_int64),
+        ("dtype", c_int32),
+    ]
+
+
 class KvSegment(C.Structure):
     """``tah_kv_segment``"""
 
@@ -101,6 +111,8 @@ PROTOTYPES = {
     "tah_duo_error_string": (C.c_char_p, [C.c_int]),
     "tah_duo_fwd_varlen": (C.c_int, [C.POINTER(DuoFwdArgs), c_void_p]),
     "tah_duo_bwd_varlen": (C.c_int, [C.POINTER(DuoBwdArgs), c_void_p]),
+    "tah_duo_fwd_masked": (C.c_int, [C.POINTER(DuoFwdArgs), C.POINTER(AdditiveMask), c_void_p]),
+    "tah_duo_bwd_masked": (C.c_int, [C.POINTER(DuoBwdArgs), C.POINTER(AdditiveMask), c_void_p]),
     "tah_duo_decode_workspace_bytes": (C.c_size_t, [c_int32, c_int32, c_int32, c_int32]),
     "tah_duo_decode": (C.c_int, [C.POINTER(DuoDecodeArgs), c_void_p]),
     "tah_kv_append": (C.c_int, [C.POINTER(KvAppendArgs), c_void_p]),

@@ -65,6 +65,37 @@ def duo_attn_varlen(q1, k1, v1, cu_q1, cu_k1, q2, k2, v2, pos_q2, pos_k2, cu_q2,
     return (o1, o2, lse1, lse2) if return_lse else (o1, o2)
 
 
+class _AttnMasked(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, mask, nseq, scale):
+        o, lse = ops.duo_fwd_masked(q, k, v, mask, nseq, scale)
+        ctx.save_for_backward(q, k, v, o, lse, mask)
+        ctx.nseq, ctx.scale = nseq, scale
+        ctx.mark_non_differentiable(lse)
+        return o, lse
+
+    @staticmethod
+    def backward(ctx, d_o, _dl):
+        q, k, v, o, lse, mask = ctx.saved_tensors
+        d_o = torch.zeros_like(o) if d_o is None else d_o.contiguous()
+        dq, dk, dv = ops.duo_bwd_masked(q, k, v, o, lse, d_o, mask, ctx.nseq, ctx.scale)
+        return dq, dk, dv, None, None, None
+
+
+def attn_additive_mask(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, mask: torch.Tensor,
+                       scale: float, return_lse: bool = False):
+    """Compatibility mode: what sdpa_attention_forward computes today (sdpa_attention.py:79-166) --
+    ``softmax(q k^T * scale + mask) v`` with GQA by head grouping -- for callers that still pass the dense
+    additive mask of tah_model.py:744-791.  query (B,Hq,Tq,D), key/value (B,Hkv,Tkv,D), mask
+    (B|1, Hq|1, Tq, Tkv) bf16 or float32.  Returns (B,Tq,Hq,D); differentiable in q, k, v.
+    Rows whose keys are all hidden come out as zeros.
+    """
+    B, Hq, Tq, D = query.shape
+    o, lse = _AttnMasked.apply(_rows(query), _rows(key), _rows(value), mask, B, float(scale))
+    o = o.view(B, Tq, Hq, D)
+    return (o, lse) if return_lse else o
+
+
 class DuoMask:
     """What the dense mask of tah_model.py:744-791 is computed from, kept symbolic."""
 
@@ -218,12 +249,25 @@ def duo_attention_forward(module, query: torch.Tensor, key: torch.Tensor, value:
     query (B,Hq,Tq,D); key/value are whatever ``cache.update`` returned (the new rows); ``attention_mask``
     is the :class:`DuoMask` built for this step; ``module.layer_idx`` names the layer.  Returns
     ``(attn_output (B,Tq,Hq,D), None)`` like sdpa_attention_forward (sdpa_attention.py:164-166).
-    A dense tensor mask is refused: there is no dense-mask code path.
+    A dense additive tensor in the mask slot (what tah_model.py:744-791 builds) selects the compatibility
+    mode instead: key/value must then be the full (B,Hkv,Tkv,D) tensors the mask's last axis runs over,
+    as the reference's ``cache.update`` returns them, and the result is that of SDPA with this mask.
     """
     del is_causal, kwargs
+    if torch.is_tensor(attention_mask):
+        if dropout:
+            raise TahDuoError("attention dropout is not supported (the reference runs with 0.0)")
+        if attention_mask.dim() != 4 or key.shape[2] != attention_mask.shape[-1]:
+            raise TahDuoError("a dense attention mask must be 4-D with its last axis over the rows of key/value "
+                              f"(mask {tuple(attention_mask.shape)}, key {tuple(key.shape)})")
+        D = query.shape[-1]
+        m = attention_mask
+        if m.dtype not in (torch.bfloat16, torch.float32):
+            m = m.to(torch.float32)
+        return attn_additive_mask(query, key, value, m, float(scaling) if scaling is not None else float(D) ** -0.5), None
     if not isinstance(attention_mask, DuoMask):
-        raise TahDuoError("duo_attention_forward needs the DuoMask from tah_amd.attention.build_attention_mask in the "
-                          "attention_mask slot (a dense additive mask is not accepted)")
+        raise TahDuoError("duo_attention_forward needs the DuoMask from tah_amd.attention.build_attention_mask (or the "
+                          "reference's dense additive mask) in the attention_mask slot")
     if dropout:
         raise TahDuoError("attention dropout is not supported (the reference runs with 0.0)")
     m = attention_mask

@@ -46,7 +46,17 @@ struct BwdParams {
     BwdStream s1, s2;
     int32_t nseq, hq, hkv;
     float scale, scale_log2e;
+    // additive-mask mode only: mask[seq][head][query index][key index], strides in elements
+    const void* mask;
+    int64_t mask_sb, mask_sh, mask_sq, mask_sk;
+    int32_t mask_f32;  // element type: 1 = float, 0 = bf16
+    float inv_scale;   // 1 / scale: the mask is added to raw scores as mask / scale
 };
+
+__device__ __forceinline__ float mask_value(const BwdParams& p, const unsigned char* row, int64_t k) {
+    return p.mask_f32 ? reinterpret_cast<const float*>(row)[k * p.mask_sk]
+                      : (float)reinterpret_cast<const __bf16*>(row)[k * p.mask_sk];
+}
 
 // ---------------------------------------------------------------------------
 // delta = rowsum(dO * O): 16 lanes per (row, head), 8 elements each
@@ -83,7 +93,8 @@ constexpr int kDqSmem = 2 * kDqStage + 64;
 
 enum class Mask { kNone, kIndex, kPos };
 
-template <int G>
+// kDense: additive-mask mode (see the forward kernel): every key of the sequence, visibility from the mask.
+template <int G, bool kDense>
 __global__ __launch_bounds__(kDqThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dq_kernel(const BwdParams p) {
     constexpr int BM = 32 * (8 / G);
     HIP_DYNAMIC_SHARED(unsigned char, smem)
@@ -129,7 +140,7 @@ __global__ __launch_bounds__(kDqThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dq_
         const int q_lo = qs.cu_q[seq];
         qpos = (row_ld - q_lo) + (lk1 - (qs.cu_q[seq + 1] - q_lo));
     }
-    const int qlim1 = row_ok ? (qpos < lk1 - 1 ? qpos : lk1 - 1) : -1;
+    const int qlim1 = row_ok ? ((qpos < lk1 - 1 && !kDense) ? qpos : lk1 - 1) : -1;
     const int qlim2 = row_ok ? qpos : -1;
     const int wmax1 = wave_reduce_max(qlim1);
     const int wmin1 = wave_reduce_min(row_ok ? qlim1 : 0x7fffffff);
@@ -147,6 +158,13 @@ __global__ __launch_bounds__(kDqThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dq_
     const int n_active = __builtin_amdgcn_readfirstlane(wmax1 >= 0 ? wmax1 / kBN + 1 : 0);
     int n_plain = __builtin_amdgcn_readfirstlane(wmin1 >= kBN - 1 ? (wmin1 - (kBN - 1)) / kBN + 1 : 0);
     n_plain = n_plain < n_active ? n_plain : n_active;
+    if constexpr (kDense) n_plain = 0;  // the mask is read for every tile
+    const unsigned char* mask_row = nullptr;  // additive-mask mode: this lane's mask row
+    if constexpr (kDense) {
+        const int64_t e = (int64_t)seq * p.mask_sb + (int64_t)head * p.mask_sh +
+                          (int64_t)(row_ld - qs.cu_q[seq]) * p.mask_sq;
+        mask_row = static_cast<const unsigned char*>(p.mask) + e * (p.mask_f32 ? 4 : 2);
+    }
 
     bf16x8 qf[8], dof[8];
     {
@@ -159,7 +177,8 @@ __global__ __launch_bounds__(kDqThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dq_
         }
     }
     const float c = p.scale_log2e;
-    const float lse_c = qs.lse[(int64_t)head * qs.total_q + row_ld] * kLog2e;
+    float lse_c = qs.lse[(int64_t)head * qs.total_q + row_ld] * kLog2e;
+    if constexpr (kDense) lse_c = lse_c == kNegInf ? -kNegInf : lse_c;  // a row that hides every key: P = 0, not exp(-inf + inf)
     const float delta = qs.delta[(int64_t)head * qs.total_q + row_ld];
 
     f32x16 dqacc[4];
@@ -242,7 +261,9 @@ __global__ __launch_bounds__(kDqThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dq_
                 const int kl = 32 * mt + acc_row(half, r);
                 if constexpr (kMask == Mask::kIndex) vis = base + kl <= qlim1;
                 if constexpr (kMask == Mask::kPos) vis = kl < nleft && kpos[kl] <= qlim2;
-                const float pr = vis ? fast_exp2(sacc[r] * c - lse_c) : 0.f;
+                float sc = sacc[r];
+                if constexpr (kDense) sc += mask_value(p, mask_row, vis ? base + kl : 0) * p.inv_scale;
+                const float pr = vis ? fast_exp2(sc * c - lse_c) : 0.f;
                 dsf[2 * mt + r / 8][r % 8] = (__bf16)(pr * (dpacc[r] - delta));
             }
         }
@@ -298,7 +319,7 @@ constexpr int kKvSmem = kKvMeta + 2 * kKvMetaBytes;
 constexpr int kKvRed = kKB * 128 * 64 * 4;                // final reduction: [key block][128 regs][64 lanes] f32, reuses the front
 static_assert(kKvRed <= kKvSmem, "reduction buffer must fit");
 
-template <int G>
+template <int G, bool kDense>
 __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkdv_kernel(const BwdParams p) {
     HIP_DYNAMIC_SHARED(unsigned char, smem)
     const int tid = threadIdx.x, lane = tid % kWave;
@@ -355,7 +376,8 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
     const int kl0 = key0 - k_lo;  // local index of the tile's first key (depth-0 tiles: its position)
     int t1_begin = 0, nt1 = 0;
     if (!second && lq1 > 0) {
-        const int first_q = kl0 - off > 0 ? kl0 - off : 0;  // first depth-0 query row with position >= kl0
+        // first depth-0 query row with position >= kl0 (additive-mask mode: every row, the mask decides)
+        const int first_q = (kl0 - off > 0 && !kDense) ? kl0 - off : 0;
         t1_begin = first_q / kBQ;
         nt1 = (lq1 + kBQ - 1) / kBQ - t1_begin;
         if (nt1 < 0) nt1 = 0;
@@ -373,6 +395,7 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
         t_vis = t_vis < 0 ? 0 : t_vis;
     }
     t_vis = t_vis < t_whole ? t_vis : t_whole;
+    if constexpr (kDense) t_whole = t_vis = 0;  // the mask is read for every item
 
     f32x16 dkacc[4], dvacc[4];
 #pragma unroll
@@ -468,11 +491,14 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
             [[maybe_unused]] bool q2s = false;
             [[maybe_unused]] int nvalid = kBQ, pos0 = 0;
             [[maybe_unused]] const int* qposs = reinterpret_cast<const int*>(meta) + 2 * kBQ;
+            [[maybe_unused]] int dense_head = 0, dense_q0 = 0;
             if constexpr (kMasked) {
                 int r0, r_end, head;
                 item_rows(item, q2s, r0, r_end, head);
                 nvalid = r_end - r0;        // rows of the tile that exist
                 pos0 = (r0 - q1_lo) + off;  // depth-0 stream: position of tile row 0
+                dense_head = head;
+                dense_q0 = r0 - q1_lo;      // additive-mask mode: query index of tile row 0
             }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -481,10 +507,20 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
                 for (int b4 = 0; b4 < 4; ++b4) {
                     const int r = 4 * j + b4;
                     float pr = fast_exp2(sacc[r] * c - lse4[b4] * kLog2e);
-                    if constexpr (kMasked) {
+                    if constexpr (kMasked && !kDense) {
                         const int qr = mrow + 8 * j + b4;
                         const int qp = q2s ? qposs[qr] : pos0 + qr;
                         pr = (qr < nvalid && kpos <= qp) ? pr : 0.f;
+                    }
+                    if constexpr (kDense) {  // mask[seq][head][query][my key]
+                        const int qr = mrow + 8 * j + b4;
+                        const bool ok = qr < nvalid && key_ok;
+                        const int64_t e = (int64_t)seq * p.mask_sb + (int64_t)dense_head * p.mask_sh +
+                                          (int64_t)(ok ? dense_q0 + qr : 0) * p.mask_sq;
+                        const float mv = mask_value(p, static_cast<const unsigned char*>(p.mask) + e * (p.mask_f32 ? 4 : 2),
+                                                    ok ? kl0 + 32 * kb + col : 0);
+                        const float lse_row = lse4[b4] == kNegInf ? -kNegInf : lse4[b4];  // all keys hidden: P = 0
+                        pr = ok ? fast_exp2((sacc[r] + mv * p.inv_scale) * c - lse_row * kLog2e) : 0.f;
                     }
                     pfr[r / 8][r % 8] = (__bf16)pr;
                 }
@@ -642,7 +678,7 @@ int check_bwd_stream(const tah_duo_stream& s, const tah_duo_bwd_stream& g, bool 
     return TAH_OK;
 }
 
-template <int G>
+template <int G, bool kDense>
 int launch_bwd(const BwdParams& p, hipStream_t st) {
     constexpr int BM = 32 * (8 / G);
     for (const BwdStream* s : {&p.s1, &p.s2}) {
@@ -656,16 +692,16 @@ int launch_bwd(const BwdParams& p, hipStream_t st) {
     if (p.s1.total_k > 0) ktiles += p.s1.total_k / kBK + p.nseq;
     if (p.s2.total_k > 0) ktiles += p.s2.total_k / kBK + p.nseq;
     if (qtiles > 0) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&duo_bwd_dq_kernel<G>),
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&duo_bwd_dq_kernel<G, kDense>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kDqSmem) != hipSuccess)
             return TAH_E_LAUNCH;
-        hipLaunchKernelGGL(duo_bwd_dq_kernel<G>, dim3(p.hkv, qtiles), dim3(kDqThreads), kDqSmem, st, p);
+        hipLaunchKernelGGL((duo_bwd_dq_kernel<G, kDense>), dim3(p.hkv, qtiles), dim3(kDqThreads), kDqSmem, st, p);
     }
     if (ktiles > 0) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&duo_bwd_dkdv_kernel<G>),
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&duo_bwd_dkdv_kernel<G, kDense>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kKvSmem) != hipSuccess)
             return TAH_E_LAUNCH;
-        hipLaunchKernelGGL(duo_bwd_dkdv_kernel<G>, dim3(p.hkv, ktiles), dim3(kKvThreads), kKvSmem, st, p);
+        hipLaunchKernelGGL((duo_bwd_dkdv_kernel<G, kDense>), dim3(p.hkv, ktiles), dim3(kKvThreads), kKvSmem, st, p);
     }
     return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
 }
@@ -673,13 +709,19 @@ int launch_bwd(const BwdParams& p, hipStream_t st) {
 }  // namespace
 }  // namespace tah
 
-extern "C" int tah_duo_bwd_varlen(const tah_duo_bwd_args* a, tah_stream_t stream) {
-    using namespace tah;
+namespace tah {
+namespace {
+template <bool kDense>
+int dispatch_bwd(const tah_duo_bwd_args* a, const tah_additive_mask* m, tah_stream_t stream) {
     if (!a) return TAH_E_NULL;
     const tah_duo_fwd_args& f = a->fwd;
     if (f.d != kD || f.nseq < 0 || f.hq <= 0 || f.hkv <= 0 || f.hq % f.hkv != 0) return TAH_E_SHAPE;
     const int g = f.hq / f.hkv;
     if (g != 1 && g != 2 && g != 4 && g != 8) return TAH_E_SHAPE;
+    if (kDense) {
+        if (!m || !m->mask) return TAH_E_NULL;
+        if (f.s2.total_q != 0 || f.s2.total_k != 0 || (m->dtype != 0 && m->dtype != 1) || f.scale == 0.f) return TAH_E_SHAPE;
+    }
     if (f.nseq == 0) return TAH_OK;
     if (int rc = check_bwd_stream(f.s1, a->g1, false)) return rc;
     if (int rc = check_bwd_stream(f.s2, a->g2, true)) return rc;
@@ -691,11 +733,31 @@ extern "C" int tah_duo_bwd_varlen(const tah_duo_bwd_args* a, tah_stream_t stream
     p.hkv = f.hkv;
     p.scale = f.scale;
     p.scale_log2e = f.scale * kLog2e;
+    p.mask = nullptr;
+    p.mask_sb = p.mask_sh = p.mask_sq = p.mask_sk = 0;
+    p.mask_f32 = 0;
+    p.inv_scale = 0.f;
+    if (kDense) {
+        p.mask = m->mask;
+        p.mask_sb = m->seq_stride; p.mask_sh = m->head_stride; p.mask_sq = m->q_stride; p.mask_sk = m->k_stride;
+        p.mask_f32 = m->dtype;
+        p.inv_scale = 1.0f / f.scale;
+    }
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (g) {
-        case 1: return launch_bwd<1>(p, st);
-        case 2: return launch_bwd<2>(p, st);
-        case 4: return launch_bwd<4>(p, st);
-        default: return launch_bwd<8>(p, st);
+        case 1: return launch_bwd<1, kDense>(p, st);
+        case 2: return launch_bwd<2, kDense>(p, st);
+        case 4: return launch_bwd<4, kDense>(p, st);
+        default: return launch_bwd<8, kDense>(p, st);
     }
+}
+}  // namespace
+}  // namespace tah
+
+extern "C" int tah_duo_bwd_varlen(const tah_duo_bwd_args* a, tah_stream_t stream) {
+    return tah::dispatch_bwd<false>(a, nullptr, stream);
+}
+
+extern "C" int tah_duo_bwd_masked(const tah_duo_bwd_args* a, const tah_additive_mask* m, tah_stream_t stream) {
+    return tah::dispatch_bwd<true>(a, m, stream);
 }

@@ -69,11 +69,19 @@ struct FwdParams {
     FwdStream s1, s2;
     int32_t nseq, hq, hkv;
     float scale_log2e;
+    // additive-mask mode only: mask[seq][head][query index][key index], strides in elements
+    const void* mask;
+    int64_t mask_sb, mask_sh, mask_sq, mask_sk;
+    int32_t mask_f32;  // element type: 1 = float, 0 = bf16
+    float inv_scale;   // 1 / scale: the mask is added to raw scores as mask / scale
 };
 
-enum class Mask { kNone, kIndex, kPos };
+enum class Mask { kNone, kIndex, kPos, kDense };
 
-template <int G>
+// kDense: additive-mask mode.  Every query attends to every key of its sequence and visibility comes
+// from a dense additive mask (softmax(q k^T * scale + mask) v); only stream 1 is used.  A separate
+// instantiation, so the duo-causal kernel carries none of it.
+template <int G, bool kDense>
 __global__ __launch_bounds__(kThreads) TAH_WAVES_PER_EU(2, 2) void duo_fwd_kernel(const FwdParams p) {
     constexpr int BM = 32 * (8 / G);
     HIP_DYNAMIC_SHARED(unsigned char, smem)
@@ -127,7 +135,8 @@ __global__ __launch_bounds__(kThreads) TAH_WAVES_PER_EU(2, 2) void duo_fwd_kerne
         const int q_lo = qs.cu_q[seq];
         qpos = (row_ld - q_lo) + (lk1 - (qs.cu_q[seq + 1] - q_lo));
     }
-    const int qlim1 = row_ok ? (qpos < lk1 - 1 ? qpos : lk1 - 1) : -1;  // last visible depth-0 key index
+    // last visible depth-0 key index (additive-mask mode: every key of the sequence, the mask decides)
+    const int qlim1 = row_ok ? ((qpos < lk1 - 1 && !kDense) ? qpos : lk1 - 1) : -1;
     const int qlim2 = row_ok ? qpos : -1;                              // depth-1 keys: pos_k <= qlim2
     const int wmax1 = wave_reduce_max(qlim1);
     const int wmin1 = wave_reduce_min(row_ok ? qlim1 : 0x7fffffff);
@@ -151,6 +160,14 @@ __global__ __launch_bounds__(kThreads) TAH_WAVES_PER_EU(2, 2) void duo_fwd_kerne
     const int n_active = __builtin_amdgcn_readfirstlane(wmax1 >= 0 ? wmax1 / kBN + 1 : 0);
     int n_plain = __builtin_amdgcn_readfirstlane(wmin1 >= kBN - 1 ? (wmin1 - (kBN - 1)) / kBN + 1 : 0);
     n_plain = n_plain < n_active ? n_plain : n_active;
+    if constexpr (kDense) n_plain = 0;  // the mask is read for every tile
+    // additive-mask mode: this lane's mask row
+    const unsigned char* mask_row = nullptr;
+    if constexpr (kDense) {
+        const int64_t e = (int64_t)seq * p.mask_sb + (int64_t)head * p.mask_sh +
+                          (int64_t)(row_ld - qs.cu_q[seq]) * p.mask_sq;
+        mask_row = static_cast<const unsigned char*>(p.mask) + e * (p.mask_f32 ? 4 : 2);
+    }
 
     // ---- Q fragments: B operand of S^T = K Q^T ------------------------------
     bf16x8 qf[8];
@@ -297,6 +314,19 @@ __global__ __launch_bounds__(kThreads) TAH_WAVES_PER_EU(2, 2) void duo_fwd_kerne
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
                     sacc[mt][r] = base + 32 * mt + acc_row(half, r) <= qlim1 ? sacc[mt][r] : kNegInf;
+        } else if constexpr (kMask == Mask::kDense) {
+            const int base = it * kBN;
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int kk = base + 32 * mt + acc_row(half, r);
+                    const int kc = kk <= qlim1 ? kk : 0;  // (never read past the row)
+                    const float mv = p.mask_f32
+                                         ? reinterpret_cast<const float*>(mask_row)[(int64_t)kc * p.mask_sk]
+                                         : (float)reinterpret_cast<const __bf16*>(mask_row)[(int64_t)kc * p.mask_sk];
+                    sacc[mt][r] = kk <= qlim1 ? sacc[mt][r] + mv * p.inv_scale : kNegInf;
+                }
         } else if constexpr (kMask == Mask::kPos) {
             const int* kpos = reinterpret_cast<const int*>(smem + kPosRing + (it % kPosSlots) * (kBN * 4));
             const int nleft = lk2 - (it - n1) * kBN;  // keys of this tile that exist
@@ -345,7 +375,7 @@ __global__ __launch_bounds__(kThreads) TAH_WAVES_PER_EU(2, 2) void duo_fwd_kerne
         TAH_KEEP_HERE4(op[0], op[1], op[2], op[3]);
     };
     using PlainTag = std::integral_constant<Mask, Mask::kNone>;
-    using IndexTag = std::integral_constant<Mask, Mask::kIndex>;
+    using IndexTag = std::integral_constant<Mask, kDense ? Mask::kDense : Mask::kIndex>;
     using PosTag = std::integral_constant<Mask, Mask::kPos>;
 
     // Workgroup timeline: half-phases h = 0 .. 2*ntiles+1, a barrier before each.  Waves of the
@@ -487,24 +517,21 @@ int check_stream(const tah_duo_stream& s, bool second) {
     return TAH_OK;
 }
 
-template <int G>
+template <int G, bool kDense>
 int launch_fwd(const FwdParams& p, hipStream_t stream) {
     constexpr int BM = 32 * (8 / G);
     int tiles = 0;  // upper bound on sum_b ceil(len_b / BM), no device read needed
     if (p.s1.total_q > 0) tiles += p.s1.total_q / BM + p.nseq;
     if (p.s2.total_q > 0) tiles += p.s2.total_q / BM + p.nseq;
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&duo_fwd_kernel<G>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&duo_fwd_kernel<G, kDense>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes) != hipSuccess)
         return TAH_E_LAUNCH;
-    hipLaunchKernelGGL(duo_fwd_kernel<G>, dim3(p.hkv, tiles), dim3(kThreads), kSmemBytes, stream, p);
+    hipLaunchKernelGGL((duo_fwd_kernel<G, kDense>), dim3(p.hkv, tiles), dim3(kThreads), kSmemBytes, stream, p);
     return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
 }
 
-}  // namespace
-}  // namespace tah
-
-extern "C" int tah_duo_fwd_varlen(const tah_duo_fwd_args* a, tah_stream_t stream) {
-    using namespace tah;
+template <bool kDense>
+int dispatch_fwd(const tah_duo_fwd_args* a, const tah_additive_mask* m, tah_stream_t stream) {
     if (!a) return TAH_E_NULL;
     if (a->d != kD || a->nseq < 0 || a->hq <= 0 || a->hkv <= 0 || a->hq % a->hkv != 0) return TAH_E_SHAPE;
     const int g = a->hq / a->hkv;
@@ -512,6 +539,10 @@ extern "C" int tah_duo_fwd_varlen(const tah_duo_fwd_args* a, tah_stream_t stream
     if (int rc = check_stream(a->s1, false)) return rc;
     if (int rc = check_stream(a->s2, true)) return rc;
     if (a->s2.total_q > 0 && (!a->s1.cu_k || (a->s1.total_k > 0 && (!a->s1.k || !a->s1.v)))) return TAH_E_NULL;
+    if (kDense) {
+        if (!m || !m->mask) return TAH_E_NULL;
+        if (a->s2.total_q != 0 || a->s2.total_k != 0 || (m->dtype != 0 && m->dtype != 1) || a->scale == 0.f) return TAH_E_SHAPE;
+    }
     if (a->nseq == 0 || (a->s1.total_q == 0 && a->s2.total_q == 0)) return TAH_OK;
     FwdParams p;
     p.s1 = to_dev(a->s1);
@@ -520,11 +551,32 @@ extern "C" int tah_duo_fwd_varlen(const tah_duo_fwd_args* a, tah_stream_t stream
     p.hq = a->hq;
     p.hkv = a->hkv;
     p.scale_log2e = a->scale * kLog2e;
+    p.mask = nullptr;
+    p.mask_sb = p.mask_sh = p.mask_sq = p.mask_sk = 0;
+    p.mask_f32 = 0;
+    p.inv_scale = 0.f;
+    if (kDense) {
+        p.mask = m->mask;
+        p.mask_sb = m->seq_stride; p.mask_sh = m->head_stride; p.mask_sq = m->q_stride; p.mask_sk = m->k_stride;
+        p.mask_f32 = m->dtype;
+        p.inv_scale = 1.0f / a->scale;
+    }
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (g) {
-        case 1: return launch_fwd<1>(p, st);
-        case 2: return launch_fwd<2>(p, st);
-        case 4: return launch_fwd<4>(p, st);
-        default: return launch_fwd<8>(p, st);
+        case 1: return launch_fwd<1, kDense>(p, st);
+        case 2: return launch_fwd<2, kDense>(p, st);
+        case 4: return launch_fwd<4, kDense>(p, st);
+        default: return launch_fwd<8, kDense>(p, st);
     }
+}
+
+}  // namespace
+}  // namespace tah
+
+extern "C" int tah_duo_fwd_varlen(const tah_duo_fwd_args* a, tah_stream_t stream) {
+    return tah::dispatch_fwd<false>(a, nullptr, stream);
+}
+
+extern "C" int tah_duo_fwd_masked(const tah_duo_fwd_args* a, const tah_additive_mask* m, tah_stream_t stream) {
+    return tah::dispatch_fwd<true>(a, m, stream);
 }

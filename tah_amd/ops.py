@@ -139,6 +139,83 @@ def duo_bwd_varlen(q1, k1, v1, o1, lse1, do1, cu_q1, cu_k1, q2, k2, v2, o2, lse2
     return dq1, dk1, dv1, dq2, dk2, dv2
 
 
+def _fill_mask(m: _capi.AdditiveMask, mask: torch.Tensor, nseq: int, hq: int, tq: int, tk: int) -> None:
+    """mask (B or 1, Hq or 1, Tq, Tkv) additive, bf16 or float32; broadcast dims get stride 0."""
+    if mask.dim() != 4 or mask.dtype not in (torch.bfloat16, torch.float32):
+        raise _capi.TahDuoError("additive mask must be a 4-D bf16 or float32 tensor (B|1, Hq|1, Tq, Tkv)")
+    if mask.shape[0] not in (1, nseq) or mask.shape[1] not in (1, hq) or mask.shape[2] != tq or mask.shape[3] != tk:
+        raise _capi.TahDuoError(f"additive mask shape {tuple(mask.shape)} does not match (B={nseq}, Hq={hq}, Tq={tq}, Tkv={tk})")
+    m.mask = mask.data_ptr()
+    m.seq_stride = mask.stride(0) if mask.shape[0] != 1 else 0
+    m.head_stride = mask.stride(1) if mask.shape[1] != 1 else 0
+    m.q_stride, m.k_stride = mask.stride(2), mask.stride(3)
+    m.dtype = 1 if mask.dtype == torch.float32 else 0
+
+
+def _dense_cu(q: torch.Tensor, nseq: int, t: int) -> torch.Tensor:
+    return torch.arange(0, (nseq + 1) * t, t, dtype=torch.int32, device=q.device)
+
+
+def duo_fwd_masked(q, k, v, mask, nseq: int, scale: float):
+    """Compatibility mode: ``softmax(q k^T * scale + mask) v`` with a dense additive mask.
+
+    q [B*Tq,Hq,D], k/v [B*Tkv,Hkv,D] (batch rows one after another), mask (B|1, Hq|1, Tq, Tkv).
+    Returns o [B*Tq,Hq,D] and lse [Hq, B*Tq].
+    """
+    lib = _lib.lib()
+    for n, t in (("q", q), ("k", k), ("v", v)):
+        _thd(t, n)
+    _dev_check(q, k, v, mask)
+    if nseq <= 0 or q.shape[0] % nseq or k.shape[0] % nseq or k.shape != v.shape:
+        raise _capi.TahDuoError("row counts must be multiples of the batch size")
+    tq, tk = q.shape[0] // nseq, k.shape[0] // nseq
+    hq, d = q.shape[1], q.shape[2]
+    o = torch.empty((q.shape[0], hq, d), dtype=q.dtype, device=q.device)
+    lse = torch.empty((hq, q.shape[0]), dtype=torch.float32, device=q.device)
+    cu_q, cu_k = _dense_cu(q, nseq, tq), _dense_cu(q, nseq, tk)
+    zc = torch.zeros(nseq + 1, dtype=torch.int32, device=q.device)
+    e = q[:0]
+    a = _capi.DuoFwdArgs()
+    _fill_stream(a.s1, q, k, v, o, lse, cu_q, cu_k, None, None)
+    _fill_stream(a.s2, e, k[:0], v[:0], e, lse[:, :0], zc, zc, None, None)
+    a.nseq, a.hq, a.hkv, a.d, a.scale = nseq, hq, k.shape[1], d, float(scale)
+    m = _capi.AdditiveMask()
+    _fill_mask(m, mask, nseq, hq, tq, tk)
+    _capi.check(lib, lib.tah_duo_fwd_masked(ctypes.byref(a), ctypes.byref(m), _stream(q)), "tah_duo_fwd_masked")
+    return o, lse
+
+
+def duo_bwd_masked(q, k, v, o, lse, d_o, mask, nseq: int, scale: float):
+    """Backward of :func:`duo_fwd_masked`; returns dq, dk, dv (bf16)."""
+    lib = _lib.lib()
+    for n, t in (("q", q), ("k", k), ("v", v), ("o", o), ("d_o", d_o)):
+        _thd(t, n)
+    _dev_check(q, k, v, o, lse, d_o, mask)
+    if d_o.shape != q.shape or o.shape != q.shape:
+        raise _capi.TahDuoError("o / dO shapes must match q")
+    if lse.dtype != torch.float32 or not lse.is_contiguous():
+        raise _capi.TahDuoError("lse must be contiguous float32 [Hq, rows]")
+    tq, tk = q.shape[0] // nseq, k.shape[0] // nseq
+    hq, d = q.shape[1], q.shape[2]
+    dq = torch.empty_like(q, memory_format=torch.contiguous_format)
+    dk = torch.empty(k.shape, dtype=k.dtype, device=k.device)
+    dv = torch.empty(v.shape, dtype=v.dtype, device=v.device)
+    delta = torch.empty((hq, q.shape[0]), dtype=torch.float32, device=q.device)
+    cu_q, cu_k = _dense_cu(q, nseq, tq), _dense_cu(q, nseq, tk)
+    zc = torch.zeros(nseq + 1, dtype=torch.int32, device=q.device)
+    e = q[:0]
+    a = _capi.DuoBwdArgs()
+    _fill_stream(a.fwd.s1, q, k, v, o, lse, cu_q, cu_k, None, None)
+    _fill_stream(a.fwd.s2, e, k[:0], v[:0], e, lse[:, :0], zc, zc, None, None)
+    a.fwd.nseq, a.fwd.hq, a.fwd.hkv, a.fwd.d, a.fwd.scale = nseq, hq, k.shape[1], d, float(scale)
+    _fill_bwd_stream(a.g1, d_o, dq, dk, dv, delta)
+    _fill_bwd_stream(a.g2, e, e, k[:0], v[:0], delta[:, :0])
+    m = _capi.AdditiveMask()
+    _fill_mask(m, mask, nseq, hq, tq, tk)
+    _capi.check(lib, lib.tah_duo_bwd_masked(ctypes.byref(a), ctypes.byref(m), _stream(q)), "tah_duo_bwd_masked")
+    return dq, dk, dv
+
+
 def hard_index_build(mask: torch.Tensor):
     """(B, S) bool/uint8 mask -> pos int32 [B*S cap], flat int32, seq int32, cu int32 [B+1].
 

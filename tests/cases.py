@@ -69,6 +69,24 @@ def add_score_drift(case, nats_per_key):
     return out
 
 
+def make_masked_case(seed, B, Hq, Hkv, Tq, Tk, D=128, mask_dtype=torch.float32, per_head=False, p_hide=0.4):
+    """Dense (B,H,T,D) bf16 q/k/v and an additive mask (B, 1|Hq, Tq, Tk): random small biases, a fraction
+    p_hide of entries hidden with finfo.min (as tah_model.py:790) or -inf, every row keeping at least one
+    visible key except row 0 of the last batch entry, which hides them all."""
+    g = torch.Generator().manual_seed(seed)
+    rn = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16)
+    q, k, v = rn(B, Hq, Tq, D), rn(B, Hkv, Tk, D), rn(B, Hkv, Tk, D)
+    H = Hq if per_head else 1
+    bias = (torch.randn(B, H, Tq, Tk, generator=g) * 0.5).to(mask_dtype).float()
+    hide = torch.rand(B, H, Tq, Tk, generator=g) < p_hide
+    hide[..., 0] = False
+    hide[B - 1, :, 0, :] = True
+    fm = torch.finfo(mask_dtype).min
+    use_inf = torch.rand(B, H, Tq, Tk, generator=g) < 0.5
+    mask = torch.where(hide, torch.where(use_inf, torch.tensor(float("-inf")), torch.tensor(fm)), bias).to(mask_dtype)
+    return dict(q=q, k=k, v=v, mask=mask, scale=float(D) ** -0.5)
+
+
 VARLEN_KEYS = ("q1", "k1", "v1", "cu_q1", "cu_k1", "q2", "k2", "v2", "pos_q2", "pos_k2", "cu_q2", "cu_k2", "scale")
 
 

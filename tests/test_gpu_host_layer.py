@@ -5,7 +5,7 @@ import torch
 
 from oracle import duo_oracle as O
 from tests.cases import make_dense_case
-from tests.test_host_layer import _forward_two_depths, _oracle_two_depths
+from tests.test_host_layer import _forward_two_depths, _forward_two_depths_reference_style, _oracle_two_depths
 
 pytestmark = pytest.mark.gpu
 
@@ -21,6 +21,21 @@ def test_forward_loop_matches_dense_reference_gpu(B, T, p, left_pad):
     np.testing.assert_allclose(o1.cpu()[valid].float().numpy(), w1[valid].numpy(), atol=2e-2, rtol=2e-2)
     assert (o1.cpu()[~valid] == 0).all()
     np.testing.assert_allclose(o2.cpu()[~pad.cpu()].float().numpy(), w2[~wpad].numpy(), atol=2e-2, rtol=2e-2)
+
+
+def test_reference_style_loop_with_dense_masks_gpu():
+    """Additive-mask compatibility mode end to end: dense masks + concatenated cache give what the symbolic
+    mask carrier gives (and what the dense oracle gives) on every valid row."""
+    from tah_amd.cache import TaHDuoCache
+    c = make_dense_case(51, B=3, T=200, p_hard=0.2, left_pad=[0, 37, 150])
+    o1, o2, pad = _forward_two_depths_reference_style(c, TaHDuoCache(), device="cuda")
+    _, d1, d2, _ = _forward_two_depths(c, TaHDuoCache(), device="cuda")
+    w1, w2, wpad = _oracle_two_depths(c)
+    valid = c["valid"].bool()
+    np.testing.assert_allclose(o1.cpu()[valid].float().numpy(), w1[valid].numpy(), atol=2e-2, rtol=2e-2)
+    np.testing.assert_allclose(o2.cpu()[~pad.cpu()].float().numpy(), w2[~wpad].numpy(), atol=2e-2, rtol=2e-2)
+    np.testing.assert_allclose(o1.cpu()[valid].float().numpy(), d1.cpu()[valid].float().numpy(), atol=8e-3, rtol=8e-3)
+    np.testing.assert_allclose(o2.cpu()[~pad.cpu()].float().numpy(), d2.cpu()[~pad.cpu()].float().numpy(), atol=8e-3, rtol=8e-3)
 
 
 def test_forward_loop_gradients_gpu():

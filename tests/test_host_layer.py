@@ -112,6 +112,34 @@ def _forward_two_depths(c, cache, requires_grad=False, device="cpu"):
     return t, o1, o2, pad
 
 
+def _forward_two_depths_reference_style(c, cache, device="cpu"):
+    """The same loop as the reference runs it today: a dense additive mask in the mask slot and the
+    concatenated cache as key/value (tah_model.py:604-623, causal_cache.py:97).  Exercises the
+    additive-mask compatibility mode of the attention callable."""
+    from tah_amd.attention import build_attention_mask, duo_attention_forward
+    from tah_amd.pack import gather_active
+    bf = lambda x: x.to(torch.bfloat16).to(device)
+    c = dict(c, hard=c["hard"].to(device), valid=c["valid"].to(device))
+    valid = c["valid"]
+    pos = (torch.cumsum(valid, -1) - 1).clamp(min=0)
+    t = {k: bf(c[k]) for k in ("q1", "k1", "v1", "q2", "k2", "v2")}
+    cache.current_iter_depth, cache.position_ids_to_cache, cache.valid_mask_to_cache = 0, pos, valid
+    dense0 = build_attention_mask(pos, valid, cache, 0, dtype=torch.bfloat16).dense(torch.bfloat16)
+    cache.update(t["k1"], t["v1"], 0)
+    K, V = cache.get_cache_upto_iter(0, 0)
+    o1, _ = duo_attention_forward(_layer(), t["q1"], K, V, dense0, dropout=0.0, scaling=c["scale"])
+    tok = lambda x: x.transpose(1, 2)
+    pad, q2, k2, v2, pos2, val2 = gather_active(c["hard"], tok(t["q2"]), tok(t["k2"]), tok(t["v2"]), pos, valid)
+    if pad.shape[1] == 0:
+        return o1, None, pad
+    cache.current_iter_depth, cache.position_ids_to_cache, cache.valid_mask_to_cache = 1, pos2, val2
+    dense1 = build_attention_mask(pos2, val2, cache, 1, dtype=torch.bfloat16).dense(torch.bfloat16)
+    cache.update(tok(k2), tok(v2), 0)
+    K, V = cache.get_cache_upto_iter(0, 1)
+    o2, _ = duo_attention_forward(_layer(), tok(q2), K, V, dense1, scaling=c["scale"])
+    return o1, o2, pad
+
+
 def _oracle_two_depths(c):
     r = lambda x: x.to(torch.bfloat16).float()
     return O.duo_prefill_dense(r(c["q1"]), r(c["k1"]), r(c["v1"]), r(c["q2"]), r(c["k2"]), r(c["v2"]), c["hard"],
@@ -143,6 +171,17 @@ def test_forward_loop_matches_dense_reference(emu, left_pad):
     assert K.shape == (2, 2, 40 + n2, 128)
     with pytest.raises(AssertionError):
         cache.update(K[:1], V[:1], 0)
+
+
+def test_reference_style_loop_with_dense_masks_matches_dense_reference(emu):
+    """Compatibility mode end to end: dense masks + concatenated cache, as the reference calls SDPA today."""
+    from tah_amd.cache import TaHDuoCache
+    c = make_dense_case(33, B=2, T=40, p_hard=0.25, Hq=4, Hkv=2, D=128, left_pad=[0, 9])
+    o1, o2, pad = _forward_two_depths_reference_style(c, TaHDuoCache())
+    w1, w2, wpad = _oracle_two_depths(c)
+    valid = c["valid"].bool()
+    np.testing.assert_allclose(o1[valid].float().numpy(), w1[valid].numpy(), atol=2e-2, rtol=2e-2)
+    np.testing.assert_allclose(o2[~pad].float().numpy(), w2[~pad].numpy(), atol=2e-2, rtol=2e-2)
 
 
 def test_dense_mask_of_carrier_equals_reference_mask(emu):
