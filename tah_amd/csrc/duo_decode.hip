@@ -89,7 +89,8 @@ __device__ __forceinline__ int visible_len(const DecParams& p, bool second, int 
 
 template <int G>
 __global__ __launch_bounds__(kDecThreads) void duo_decode_split_kernel(const DecParams p) {
-    __shared__ float red[16][G][kPart];  // one partial per (wave, row group)
+    HIP_DYNAMIC_SHARED(unsigned char, smem_raw)
+    float (*red)[G][kPart] = reinterpret_cast<float (*)[G][kPart]>(smem_raw);  // [16][G][kPart]: one partial per (wave, row group)
 
     const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
     const int kq = lane / 16, dc = lane % 16;  // row within a 4-row load, 8-element d slice
@@ -342,7 +343,12 @@ int check_seg(const tah_kv_segment& s, bool need_pos) {
 
 template <int G>
 int launch_decode(const DecParams& p, hipStream_t st) {
-    hipLaunchKernelGGL(duo_decode_split_kernel<G>, dim3(p.nchunk1 + p.nchunk2, p.nq, p.hkv), dim3(kDecThreads), 0, st, p);
+    constexpr int kRedBytes = 16 * G * kPart * (int)sizeof(float);  // 8.3 KB per query head of the group
+    if (kRedBytes > 64 * 1024 &&
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&duo_decode_split_kernel<G>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kRedBytes) != hipSuccess)
+        return TAH_E_LAUNCH;
+    hipLaunchKernelGGL(duo_decode_split_kernel<G>, dim3(p.nchunk1 + p.nchunk2, p.nq, p.hkv), dim3(kDecThreads), kRedBytes, st, p);
     hipLaunchKernelGGL(duo_decode_merge_kernel, dim3(p.nq, p.hq), dim3(256), 0, st, p);
     return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
 }
@@ -362,7 +368,7 @@ extern "C" int tah_duo_decode(const tah_duo_decode_args* a, tah_stream_t stream)
     if (!a) return TAH_E_NULL;
     if (a->d != kD || a->nq < 0 || a->hq <= 0 || a->hkv <= 0 || a->hq % a->hkv) return TAH_E_SHAPE;
     const int g = a->hq / a->hkv;
-    if (g != 1 && g != 2 && g != 4) return TAH_E_SHAPE;  // merge buffer for 8 heads would not fit static LDS
+    if (g != 1 && g != 2 && g != 4 && g != 8) return TAH_E_SHAPE;
     if (a->nq == 0) return TAH_OK;
     if (a->nq > 65535 || a->hq > 65535) return TAH_E_SHAPE;
     if (!a->q || !a->o || !a->q_slot || !a->q_pos || !a->workspace) return TAH_E_NULL;
@@ -393,7 +399,8 @@ extern "C" int tah_duo_decode(const tah_duo_decode_args* a, tah_stream_t stream)
     switch (g) {
         case 1: return launch_decode<1>(p, st);
         case 2: return launch_decode<2>(p, st);
-        default: return launch_decode<4>(p, st);
+        case 4: return launch_decode<4>(p, st);
+        default: return launch_decode<8>(p, st);
     }
 }
 

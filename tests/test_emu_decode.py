@@ -23,7 +23,7 @@ def oracle_decode(c):
     return o0, l0, o1[hr], l1[hr]
 
 
-@pytest.mark.parametrize("hq,hkv,lens", [(2, 1, [700, 3, 513]), (4, 1, [40]), (2, 2, [1030])])
+@pytest.mark.parametrize("hq,hkv,lens", [(2, 1, [700, 3, 513]), (4, 1, [40]), (2, 2, [1030]), (8, 1, [70, 5])])
 def test_decode_and_append_on_cpu_shim(hq, hkv, lens):
     from tah_amd import kv_cache
     c = make_decode_case(20 + hq, lens, 0.2, Hq=hq, Hkv=hkv, hard_new=[True] + [False] * (len(lens) - 1))

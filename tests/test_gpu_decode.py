@@ -55,6 +55,7 @@ def run_decode(c, cap1, cap2, fused):
     (16, 8, [1030, 2049], True),
     (8, 8, [300], False),
     (16, 4, [777, 64], True),
+    (16, 2, [1500, 33], True),   # group of 8 query heads per kv head
 ])
 def test_decode_matches_oracle(hq, hkv, lens, fused):
     print(f"decode case hq={hq} hkv={hkv} lens={lens} fused={fused}", flush=True)
