@@ -49,6 +49,19 @@ def test_fwd_moving_softmax_reference(nats_per_key):
     _check(dev, _run(dev), "drift")
 
 
+@pytest.mark.parametrize("hq,hkv,seqlens,p,seed", [
+    (32, 4, [160] * 12 + [128] * 8 + [33, 1, 97], 0.3, 41),  # 32-row tiles, many short sequences
+    (16, 8, [1100, 640, 2048, 129], 0.1, 42),                # 128-row tiles
+    (8, 8, [2304, 257, 4000, 4096, 4096], 0.05, 43),          # 256-row tiles
+    (16, 2, [3000, 1500], 0.1, 44),                          # two kv heads
+])
+def test_fwd_more_tiles_than_compute_units(hq, hkv, seqlens, p, seed):
+    """Batches with more query tiles than the device has compute units (several rounds of workgroups)."""
+    print(f"case many-tiles hq={hq} hkv={hkv} seqlens={seqlens} p={p} seed={seed}", flush=True)
+    dev = to_device(make_varlen_case(seed, seqlens, p, Hq=hq, Hkv=hkv, D=128))
+    _check(dev, _run(dev), "many-tiles")
+
+
 def test_fwd_cache_prefix_extra_depth1_keys():
     dev = to_device(make_varlen_case(11, [40, 1, 300], 0.3, seqlens_k=[500, 900, 300], extra_k2=100))
     _check(dev, _run(dev), "prefix")
