@@ -141,6 +141,16 @@ __device__ __forceinline__ void async_copy_4B(const void* sbase, uint32_t voff, 
 #define TAH_KEEP_HERE4(a, b, c, d) asm volatile("" ::"v"(a), "v"(b), "v"(c), "v"(d))
 #endif
 // Occupancy the kernel is written for; lets the scheduler spend registers on latency hiding.
+// Between LDS writes of a wave and reads, by the same wave, of what its other lanes wrote: the lanes run
+// in lockstep and the LDS serves a wave's requests in order, so all that is needed is that the compiler
+// keeps the accesses in program order.
+#ifndef TAH_WAVE_LDS_SYNC
+#define TAH_WAVE_LDS_SYNC()                                      \
+    do {                                                         \
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   \
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");   \
+    } while (0)
+#endif
 #ifndef TAH_WAVES_PER_EU
 #define TAH_WAVES_PER_EU(lo, hi) __attribute__((amdgpu_waves_per_eu(lo, hi)))
 #endif
@@ -215,12 +225,21 @@ __device__ __forceinline__ int wave_reduce_min(int x) {
     return x;
 }
 
+// Element i of an int32 array that no kernel of this library writes (sequence boundaries), read with
+// a wave-uniform index: through the constant address space, i.e. with a scalar load when the address is
+// uniform — a fraction of the latency of a vector load, which matters in the serial walk over the
+// boundaries at the start of a workgroup.
+#ifndef TAH_CONST_AS
+#define TAH_CONST_AS __attribute__((address_space(4)))
+#endif
+__device__ __forceinline__ int32_t const_i32(const int32_t* a, int i) { return ((const TAH_CONST_AS int32_t*)a)[i]; }
+
 // Locate tile `slot` among sequences whose lengths are cu[b+1]-cu[b], `bm` rows
 // per tile.  On success fills seq/row0/row_end and returns true; otherwise
 // subtracts the number of tiles in this stream from `slot` and returns false.
 __device__ __forceinline__ bool find_tile(const int32_t* cu, int nseq, int bm, int& slot, int& seq, int& row0, int& row_end) {
     for (int b = 0; b < nseq; ++b) {
-        const int lo = cu[b], hi = cu[b + 1];
+        const int lo = const_i32(cu, b), hi = const_i32(cu, b + 1);
         const int n = (hi - lo + bm - 1) / bm;
         if (slot < n) {
             seq = b;

@@ -55,7 +55,8 @@ constexpr int kKRing = 0;
 constexpr int kVRing = kStages * kKBytes;
 constexpr int kPosRing = kVRing + kStages * kVBytes;
 constexpr int kBoundsOff = kPosRing + kPosSlots * kBN * 4;
-constexpr int kSmemBytes = kBoundsOff + 64;
+constexpr int kStageOff = (kBoundsOff + 64 + 255) / 256 * 256;  // output staging: 8 KB per wave (32 rows x 256 B)
+constexpr int kSmemBytes = kStageOff + 8 * 8192;
 
 struct FwdStream {
     const __bf16 *q, *k, *v;
@@ -106,8 +107,8 @@ __global__ __launch_bounds__(kThreads) TAH_WAVES_PER_EU(2, 2) void duo_fwd_kerne
     const int head = hk * G + wave % G;
     const int rblk = wave / G;
     // depth-0 key segment of this sequence (position of a key = its local index)
-    const int k1_lo = p.s1.cu_k[seq];
-    const int lk1 = p.s1.cu_k[seq + 1] - k1_lo;
+    const int k1_lo = const_i32(p.s1.cu_k, seq);
+    const int lk1 = const_i32(p.s1.cu_k, seq + 1) - k1_lo;
     const __bf16* k1p = p.s1.k + (int64_t)k1_lo * p.s1.k_rs + (int64_t)hk * p.s1.k_hs;
     const __bf16* v1p = p.s1.v + (int64_t)k1_lo * p.s1.v_rs + (int64_t)hk * p.s1.v_hs;
     const int left1 = p.s1.total_k - k1_lo;  // rows from the segment start to the end of the array
@@ -116,8 +117,8 @@ __global__ __launch_bounds__(kThreads) TAH_WAVES_PER_EU(2, 2) void duo_fwd_kerne
     const __bf16 *k2p = nullptr, *v2p = nullptr;
     const int32_t* pos2p = nullptr;
     if (second) {
-        const int k2_lo = p.s2.cu_k[seq];
-        lk2 = p.s2.cu_k[seq + 1] - k2_lo;
+        const int k2_lo = const_i32(p.s2.cu_k, seq);
+        lk2 = const_i32(p.s2.cu_k, seq + 1) - k2_lo;
         k2p = p.s2.k + (int64_t)k2_lo * p.s2.k_rs + (int64_t)hk * p.s2.k_hs;
         v2p = p.s2.v + (int64_t)k2_lo * p.s2.v_rs + (int64_t)hk * p.s2.v_hs;
         pos2p = p.s2.pos_k + k2_lo;
@@ -132,8 +133,8 @@ __global__ __launch_bounds__(kThreads) TAH_WAVES_PER_EU(2, 2) void duo_fwd_kerne
     if (second) {
         qpos = qs.pos_q[row_ld];
     } else {
-        const int q_lo = qs.cu_q[seq];
-        qpos = (row_ld - q_lo) + (lk1 - (qs.cu_q[seq + 1] - q_lo));
+        const int q_lo = const_i32(qs.cu_q, seq);
+        qpos = (row_ld - q_lo) + (lk1 - (const_i32(qs.cu_q, seq + 1) - q_lo));
     }
     // last visible depth-0 key index (additive-mask mode: every key of the sequence, the mask decides)
     const int qlim1 = row_ok ? ((qpos < lk1 - 1 && !kDense) ? qpos : lk1 - 1) : -1;
@@ -447,10 +448,9 @@ __global__ __launch_bounds__(kThreads) TAH_WAVES_PER_EU(2, 2) void duo_fwd_kerne
         if constexpr (!kLate) TAH_PHASE_BARRIER();  // before h = 2*ntiles + 1
     };
 
-    TAH_WAIT_VMEM();  // Q fragments are in: no ordinary load stays pending across the tile loop
+    if (ntiles > 0) issue_k(0);
+    TAH_WAIT_VMEM();  // K(0) and the Q fragments are in: no ordinary load stays pending across the tile loop
     if (ntiles > 0) {
-        issue_k(0);
-        TAH_WAIT_VMEM();
         TAH_PHASE_BARRIER();  // before h = 0
         issue(0);
         if (TAH_FWD_LATE_SET(wave) == 0) run(std::false_type{});
@@ -461,21 +461,35 @@ __global__ __launch_bounds__(kThreads) TAH_WAVES_PER_EU(2, 2) void duo_fwd_kerne
     // ---- epilogue -----------------------------------------------------------
     const float l_tot = wave_sum_xor32(l_run);
     const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-    if (row_ok) {
-        __bf16* orow = qs.o + (int64_t)row * qs.o_rs + (int64_t)head * qs.o_hs;
+    // The accumulators hold O^T (a lane owns one query row, four values of d at a time): written out
+    // directly every store instruction would touch 32 rows with 8 bytes each.  The wave turns its
+    // 32 x 128 tile through a private piece of LDS instead (16-byte chunks of a row XOR-swizzled by the
+    // row number, so that neither side runs into bank conflicts) and stores whole rows: 4 rows x 256
+    // contiguous bytes per instruction.  Nobody else reads or writes this piece: no barrier.
+    unsigned char* stage = smem + kStageOff + wave * 8192;
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
+    for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-            for (int g4 = 0; g4 < 4; ++g4) {
-                bf16x4 v4;
+        for (int g4 = 0; g4 < 4; ++g4) {
+            bf16x4 v4;
 #pragma unroll
-                for (int b = 0; b < 4; ++b) v4[b] = (__bf16)(oacc[dt][4 * g4 + b] * inv);
-                *reinterpret_cast<bf16x4*>(orow + 32 * dt + 8 * g4 + 4 * half) = v4;
-            }
-        if (half == 0)
-            qs.lse[(int64_t)head * qs.total_q + row] =
-                l_tot > 0.f ? (m_run * c + fast_log2(l_tot)) * kLn2 : kNegInf;
+            for (int b = 0; b < 4; ++b) v4[b] = (__bf16)(oacc[dt][4 * g4 + b] * inv);
+            *reinterpret_cast<bf16x4*>(stage + col * 256 + (((4 * dt + g4) ^ (col & 15)) * 16) + half * 8) = v4;
+        }
+    TAH_WAVE_LDS_SYNC();  // the reads below are of other lanes' writes
+    {
+        const int ch = lane & 15;
+        __bf16* obase = qs.o + (int64_t)head * qs.o_hs + ch * 8;
+        const int tile_row0 = row0 + rblk * 32;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int r = 4 * i + (lane >> 4);
+            const bf16x8 v = *reinterpret_cast<const bf16x8*>(stage + r * 256 + ((ch ^ (r & 15)) * 16));
+            if (tile_row0 + r < row_end) st_global_16B(obase + (int64_t)(tile_row0 + r) * qs.o_rs, v);
+        }
     }
+    if (row_ok && half == 0)
+        qs.lse[(int64_t)head * qs.total_q + row] = l_tot > 0.f ? (m_run * c + fast_log2(l_tot)) * kLn2 : kNegInf;
 }
 
 FwdStream to_dev(const tah_duo_stream& s) {

@@ -153,6 +153,8 @@ void launch(K kernel, dim3 grid, dim3 block, size_t shmem, Args... args) {
 #define gridDim (emu::g_gridDim)
 #define hipLaunchKernelGGL(kernel, grid, block, shmem, stream, ...) \
     emu::launch(kernel, dim3(grid), dim3(block), (size_t)(shmem), ##__VA_ARGS__)
+#define TAH_WAVE_LDS_SYNC() emu::wave_sync()
+#define TAH_CONST_AS
 #define HIP_DYNAMIC_SHARED(type, var) type* var = reinterpret_cast<type*>(emu::g_block->dyn_smem);
 
 inline void __syncthreads() { pthread_barrier_wait(&emu::g_block->bar); }
