@@ -141,13 +141,53 @@ def bench_fwd_bwd(name: str, seqlens, p_hard: float, seed: int, steps: int, warm
             "tokens_per_s": sum(seqlens) / (ms * 1e-3)}
 
 
+def bench_qk_prep(steps: int, warmup: int):
+    """q/k RMSNorm + rotary embedding + KV append for the prefill rows of configs[1] (B=4, T=4096): the
+    step before the attention call.  HBM-bound: every q, k, v row is read and written once."""
+    import torch
+
+    from tah_amd.kv_cache import KvSlabs, qk_norm_rope
+    from tests.qk_prep_cases import make_case, to_torch
+
+    B, T, hq, hkv = 4, 4096, 16, 8
+    rows = B * T
+    c = make_case(1240, rows, hq, hkv, scale=0.5, max_pos=T)
+    t = to_torch(c, "cuda")
+    cu = torch.arange(0, rows + 1, T, dtype=torch.int32, device="cuda")
+    slabs = KvSlabs(B, T, hkv, with_pos=False, device="cuda")
+
+    def step():
+        slabs.len.zero_()
+        qk_norm_rope(t["q"], t["k"], t["qw"], t["kw"], t["cos"], t["sin"], c["eps"], v=t["v"], cache=slabs, cu_new=cu)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    # per token row: q, k, v read and q, K, V written (256 B per head), cos and sin rows read
+    nbytes = rows * (2 * (hq + 2 * hkv) * 256 + 2 * 256)
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    return {"workload": "step before attention for configs[1]: q/k RMSNorm + rotary + KV append, 16384 token rows, "
+                        "Hq=16, Hkv=8, D=128 (includes a 4-element length reset per step)",
+            "ms_per_step": ms, "algorithmic_bytes": nbytes, "hbm_gbs": gbs,
+            "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
+                         "traffic": None, "kernels": "qk_prep_kernel + kv_append_len_kernel"},
+            "tokens_per_s": rows / (ms * 1e-3)}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["all", "fwd", "decode", "fwd_bwd"], default="all",
+    ap.add_argument("--only", choices=["all", "fwd", "decode", "fwd_bwd", "qk_prep"], default="all",
                     help="profiling aid: run only one leg (the JSON line then lacks the other legs)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="profiling aid: also run one plain 256 MiB device copy (known traffic for counter scaling)")
@@ -198,6 +238,9 @@ def main() -> int:
       extra["fwd_bwd_4docs_p10"] = bench_fwd_bwd(
         "configs[3]: fwd+bwd, 8192 packed tokens in 4 documents, p_hard=0.10", [1397, 3210, 2561, 1024], 0.10, 1237,
         max(args.steps // 2, 1), max(args.warmup // 2, 1))
+
+    if args.only in ("all", "qk_prep"):
+        extra["qk_prep_prefill"] = bench_qk_prep(args.steps, args.warmup)
 
     out = {
         "metric": "duo-causal attn TFLOP/s (% bf16 MFMA peak) prefill; decode HBM GB/s",

@@ -203,6 +203,42 @@ typedef struct tah_kv_append_args {
  * Replaces the torch.cat growth of TaHCache.update (tah/model/causal_cache.py:84-95). */
 int tah_kv_append(const tah_kv_append_args* args, tah_stream_t stream);
 
+typedef struct tah_qk_prep_args {
+    const void* q;           /* bf16 [rows, Hq, D]  projected queries, one row per token */
+    const void* k;           /* bf16 [rows, Hkv, D] */
+    const void* v;           /* bf16 [rows, Hkv, D]; may be NULL when V is neither copied nor appended */
+    void* q_out;             /* bf16 [rows, Hq, D]; may alias q */
+    void* k_out;             /* bf16 [rows, Hkv, D]; may alias k; unused with append */
+    void* v_out;             /* optional copy of v; unused with append */
+    int64_t q_row_stride, q_head_stride, k_row_stride, k_head_stride, v_row_stride, v_head_stride;
+    int64_t q_out_row_stride, q_out_head_stride, k_out_row_stride, k_out_head_stride, v_out_row_stride, v_out_head_stride;
+    const void* q_weight;    /* bf16 [D] RMSNorm weight of the query heads */
+    const void* k_weight;    /* bf16 [D] */
+    const void* cos;         /* bf16 [rows, D] rotary cosines of each token's position */
+    const void* sin;         /* bf16 [rows, D] */
+    int64_t cos_sin_row_stride;
+    float eps;               /* RMSNorm epsilon */
+    int32_t rows, hq, hkv, d;
+    /* append != 0: K (after norm and rotation) and V go to the slabs of `cache`, rows
+     * [cu_new[i], cu_new[i+1]) to slot slot_of[i], and len[] advances, as in tah_kv_append */
+    int32_t append;
+    const int32_t* cu_new;   /* int32 [nseq+1] */
+    const int32_t* slot_of;  /* int32 [nseq] or NULL (slot i) */
+    const int32_t* pos_new;  /* int32 [rows] or NULL (depth 0) */
+    int32_t nseq;
+    tah_kv_segment cache;
+    int32_t* overflow;       /* optional device flag, as in tah_kv_append */
+} tah_qk_prep_args;
+
+/* Per-head RMSNorm of q and k, rotary embedding of both, and optionally the KV-cache append,
+ * in one pass over the token rows; each arithmetic step rounds to bf16 where the reference's
+ * eager bf16 modules do.  Replaces, between the projections and the attention call of
+ *   Qwen3Attention.forward        transformers/models/qwen3/modeling_qwen3.py (q_norm, k_norm,
+ *                                 apply_rotary_pos_emb; third party, pinned 4.52.4 by the reference)
+ *   TaHCache.update               tah/model/causal_cache.py:63-97 (with append)
+ * head_dim 128 only.  In-place use (q_out == q, k_out == k) is allowed. */
+int tah_qk_prep(const tah_qk_prep_args* args, tah_stream_t stream);
+
 /* Hard-token index build: stream compaction of a (B, S) byte mask in row-major
  * order.  Replaces the stable sort + nonzero of gather_active / scatter_back
  * (tah/model/tah_model.py:111-119, :160-167).  For the r-th True entry, at

@@ -106,6 +106,27 @@ class KvAppendArgs(C.Structure):
     ]
 
 
+class QkPrepArgs(C.Structure):
+    """``tah_qk_prep_args``"""
+
+    _fields_ = [
+        ("q", c_void_p), ("k", c_void_p), ("v", c_void_p), ("q_out", c_void_p), ("k_out", c_void_p), ("v_out", c_void_p),
+        ("q_row_stride", c_int64), ("q_head_stride", c_int64), ("k_row_stride", c_int64), ("k_head_stride", c_int64),
+        ("v_row_stride", c_int64), ("v_head_stride", c_int64),
+        ("q_out_row_stride", c_int64), ("q_out_head_stride", c_int64), ("k_out_row_stride", c_int64),
+        ("k_out_head_stride", c_int64), ("v_out_row_stride", c_int64), ("v_out_head_stride", c_int64),
+        ("q_weight", c_void_p), ("k_weight", c_void_p), ("cos", c_void_p), ("sin", c_void_p),
+        ("cos_sin_row_stride", c_int64),
+        ("eps", C.c_float),
+        ("rows", c_int32), ("hq", c_int32), ("hkv", c_int32), ("d", c_int32),
+        ("append", c_int32),
+        ("cu_new", c_void_p), ("slot_of", c_void_p), ("pos_new", c_void_p),
+        ("nseq", c_int32),
+        ("cache", KvSegment),
+        ("overflow", c_void_p),
+    ]
+
+
 PROTOTYPES = {
     "tah_duo_abi_version": (C.c_int, []),
     "tah_duo_error_string": (C.c_char_p, [C.c_int]),
@@ -116,6 +137,7 @@ PROTOTYPES = {
     "tah_duo_decode_workspace_bytes": (C.c_size_t, [c_int32, c_int32, c_int32, c_int32]),
     "tah_duo_decode": (C.c_int, [C.POINTER(DuoDecodeArgs), c_void_p]),
     "tah_kv_append": (C.c_int, [C.POINTER(KvAppendArgs), c_void_p]),
+    "tah_qk_prep": (C.c_int, [C.POINTER(QkPrepArgs), c_void_p]),
     "tah_hard_index_build": (C.c_int, [c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "tah_pad_rows_build": (C.c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_void_p]),
     "tah_rows_copy": (C.c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int64,

@@ -317,6 +317,117 @@ __global__ void kv_append_len_kernel(const AppendParams a) {
     a.len[slot] = n < a.capacity ? n : a.capacity;
 }
 
+// ---- q/k RMSNorm + rotary embedding (+ append) --------------------------------
+// What Qwen3Attention.forward does between the projections and the attention call
+// (transformers/models/qwen3/modeling_qwen3.py: Qwen3RMSNorm.forward on the q and k heads,
+// apply_rotary_pos_emb, then TaHCache.update), with the roundings of its bf16 eager arithmetic:
+//   n = bf16(x * rsqrt(mean(x^2) + eps));  y = bf16(w * n)                       (per head, D = 128)
+//   out[i] = bf16(bf16(y[i] * cos[i]) + bf16(rot[i] * sin[i])),  rot = (-y[64:], y[:64])
+// V is only moved.  With `append`, K and V go to the token's place in
+// the per-sequence slabs (as kv_append_rows_kernel does) instead of k_out / v_out.
+struct PrepParams {
+    const __bf16 *q, *k, *v;
+    __bf16 *q_out, *k_out, *v_out;
+    int64_t q_rs, q_hs, k_rs, k_hs, v_rs, v_hs, qo_rs, qo_hs, ko_rs, ko_hs, vo_rs, vo_hs;
+    const __bf16 *qw, *kw, *cos, *sin;
+    int64_t cs_rs;
+    float eps;
+    int32_t rows, hq, hkv, append;
+    AppendParams a;  // destination slabs (append != 0); its k_new / v_new fields are not used
+};
+
+// Two floats rounded to bfloat16 (nearest, ties to even) and packed, lo in the low half: one
+// v_cvt_pk_bf16_f32.  Going through the packed bits on purpose: a scalar cast to __bf16 and back may be
+// evaluated in excess precision by the compiler, i.e. not round at all.
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2e __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    const f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2e));
+}
+// a.lo*b.lo and a.hi*b.hi, each rounded to bf16, packed (a, b: packed bf16 pairs)
+__device__ __forceinline__ uint32_t mul_bf16x2(uint32_t a, uint32_t b) {
+    return pack_bf16(bf16_lo(a) * bf16_lo(b), bf16_hi(a) * bf16_hi(b));
+}
+
+// One workgroup (4 waves) per token row.  A head is handled by 16 lanes, 8 elements (16 bytes) each, so
+// a wave takes 4 heads at a time and the workgroup 16: the mean of squares is a DPP reduction inside
+// the row of 16 lanes, and the rotary partner of lane j's elements (+-64) sits in lane j^8 of the
+// same row.
+__global__ __launch_bounds__(256) void qk_prep_kernel(const PrepParams p) {
+    const int r = blockIdx.x;
+    const int lane = threadIdx.x % kWave;
+    const int sub = threadIdx.x / 16, j = lane % 16;  // head slot 0..15 of a pass, 16-byte piece of the head
+    __bf16 *kdst = nullptr, *vdst = nullptr;
+    int64_t kd_hs = 0, vd_hs = 0;
+    if (p.append) {
+        int seq = 0;  // sequence of new row r
+        for (int b = 0; b < p.a.nseq; ++b)
+            if (r >= p.a.cu_new[b + 1]) seq = b + 1;
+        if (seq < p.a.nseq) {
+            const int slot = p.a.slot_of ? p.a.slot_of[seq] : seq;
+            const int dst = p.a.len[slot] + (r - p.a.cu_new[seq]);
+            if (dst >= p.a.capacity) {
+                if (p.a.overflow && threadIdx.x == 0) *p.a.overflow = 1;
+            } else {
+                const int64_t drow = (int64_t)p.a.start[slot] + dst;
+                kdst = p.a.ck + drow * p.a.ck_rs;
+                vdst = p.a.cv + drow * p.a.cv_rs;
+                kd_hs = p.a.ck_hs;
+                vd_hs = p.a.cv_hs;
+                if (p.a.cpos && p.a.pos_new && threadIdx.x == 0) p.a.cpos[(int64_t)slot * p.a.capacity + dst] = p.a.pos_new[r];
+            }
+        }
+    } else {
+        kdst = p.k_out + (int64_t)r * p.ko_rs;
+        kd_hs = p.ko_hs;
+        if (p.v_out) {
+            vdst = p.v_out + (int64_t)r * p.vo_rs;
+            vd_hs = p.vo_hs;
+        }
+    }
+    const u32x4 cs = *reinterpret_cast<const u32x4*>(p.cos + (int64_t)r * p.cs_rs + 8 * j);
+    const u32x4 sn = *reinterpret_cast<const u32x4*>(p.sin + (int64_t)r * p.cs_rs + 8 * j);
+    const u32x4 qw = *reinterpret_cast<const u32x4*>(p.qw + 8 * j), kw = *reinterpret_cast<const u32x4*>(p.kw + 8 * j);
+    const uint32_t sign = j < 8 ? 0x80008000u : 0u;  // lower half of the head: -partner * sin
+    const int items = p.hq + 2 * p.hkv;
+    // (every lane of a wave walks the same number of passes and takes part in every lane exchange;
+    // what a 16-lane row has no head for is predicated off)
+    for (int base = 0; base < items; base += 16) {
+        const int it = base + sub;
+        const bool is_q = it < p.hq, is_k = !is_q && it < p.hq + p.hkv, is_v = !is_q && !is_k && it < items;
+        if (is_v && vdst) {  // a V head: moved as it is
+            const int h = it - p.hq - p.hkv;
+            *reinterpret_cast<u32x4*>(vdst + (int64_t)h * vd_hs + 8 * j) =
+                *reinterpret_cast<const u32x4*>(p.v + (int64_t)r * p.v_rs + (int64_t)h * p.v_hs + 8 * j);
+        }
+        const int h = is_q ? it : it - p.hq;
+        const __bf16* x = is_q ? p.q + (int64_t)r * p.q_rs + (int64_t)h * p.q_hs : p.k + (int64_t)r * p.k_rs + (int64_t)h * p.k_hs;
+        __bf16* y = is_q ? p.q_out + (int64_t)r * p.qo_rs + (int64_t)h * p.qo_hs
+                         : (is_k && kdst ? kdst + (int64_t)h * kd_hs : nullptr);  // null: no head, or the row overflows its slab
+        u32x4 xin = {0u, 0u, 0u, 0u};
+        if (is_q || is_k) xin = *reinterpret_cast<const u32x4*>(x + 8 * j);
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ss += bf16_lo(xin[i]) * bf16_lo(xin[i]) + bf16_hi(xin[i]) * bf16_hi(xin[i]);
+        ss = row16_sum(ss);
+        const float rs = 1.0f / sqrtf(ss * (1.0f / 128.0f) + p.eps);
+        const u32x4 w = is_q ? qw : kw;
+        u32x4 yn, out;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            yn[i] = mul_bf16x2(w[i], pack_bf16(bf16_lo(xin[i]) * rs, bf16_hi(xin[i]) * rs));
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            // the partner's normalised values: lane j^8 of this row (row rotation by 8)
+            const uint32_t pn = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)yn[i], 0x128, 0xf, 0xf, false) ^ sign;
+            const uint32_t a = mul_bf16x2(yn[i], cs[i]), b = mul_bf16x2(pn, sn[i]);
+            out[i] = pack_bf16(bf16_lo(a) + bf16_lo(b), bf16_hi(a) + bf16_hi(b));
+        }
+        if (y) *reinterpret_cast<u32x4*>(y + 8 * j) = out;
+    }
+}
+
 Seg to_seg(const tah_kv_segment& s) {
     Seg d;
     d.k = static_cast<const __bf16*>(s.k);
@@ -402,6 +513,61 @@ extern "C" int tah_duo_decode(const tah_duo_decode_args* a, tah_stream_t stream)
         case 4: return launch_decode<4>(p, st);
         default: return launch_decode<8>(p, st);
     }
+}
+
+extern "C" int tah_qk_prep(const tah_qk_prep_args* a, tah_stream_t stream) {
+    using namespace tah;
+    if (!a) return TAH_E_NULL;
+    if (a->d != kD || a->rows < 0 || a->hq <= 0 || a->hkv <= 0) return TAH_E_SHAPE;
+    if (a->rows == 0) return TAH_OK;
+    if (!a->q || !a->k || !a->q_out || !a->q_weight || !a->k_weight || !a->cos || !a->sin) return TAH_E_NULL;
+    if (a->append) {
+        if (!a->v || !a->cu_new) return TAH_E_NULL;
+        if (a->nseq <= 0 || a->cache.capacity <= 0) return TAH_E_SHAPE;
+        if (int rc = check_seg(a->cache, a->pos_new != nullptr)) return rc;
+    } else {
+        if (!a->k_out) return TAH_E_NULL;
+        if (a->v_out && !a->v) return TAH_E_NULL;
+    }
+    const int64_t strides[] = {a->q_row_stride, a->q_head_stride, a->k_row_stride, a->k_head_stride, a->v_row_stride,
+                               a->v_head_stride, a->q_out_row_stride, a->q_out_head_stride, a->k_out_row_stride,
+                               a->k_out_head_stride, a->v_out_row_stride, a->v_out_head_stride};
+    for (int64_t x : strides)
+        if (x % 8 != 0) return TAH_E_ALIGN;  // every access is 16 bytes wide (eight elements)
+    if (a->cos_sin_row_stride % 8 != 0) return TAH_E_ALIGN;
+    const void* ptrs[] = {a->q, a->k, a->v, a->q_out, a->k_out, a->v_out, a->q_weight, a->k_weight, a->cos, a->sin,
+                          a->append ? a->cache.k : nullptr, a->append ? a->cache.v : nullptr};
+    for (const void* q : ptrs)
+        if (q && !aligned16(q)) return TAH_E_ALIGN;
+    PrepParams p;
+    p.q = static_cast<const __bf16*>(a->q); p.k = static_cast<const __bf16*>(a->k); p.v = static_cast<const __bf16*>(a->v);
+    p.q_out = static_cast<__bf16*>(a->q_out); p.k_out = static_cast<__bf16*>(a->k_out); p.v_out = static_cast<__bf16*>(a->v_out);
+    p.q_rs = a->q_row_stride; p.q_hs = a->q_head_stride; p.k_rs = a->k_row_stride; p.k_hs = a->k_head_stride;
+    p.v_rs = a->v_row_stride; p.v_hs = a->v_head_stride;
+    p.qo_rs = a->q_out_row_stride; p.qo_hs = a->q_out_head_stride; p.ko_rs = a->k_out_row_stride; p.ko_hs = a->k_out_head_stride;
+    p.vo_rs = a->v_out_row_stride; p.vo_hs = a->v_out_head_stride;
+    p.qw = static_cast<const __bf16*>(a->q_weight); p.kw = static_cast<const __bf16*>(a->k_weight);
+    p.cos = static_cast<const __bf16*>(a->cos); p.sin = static_cast<const __bf16*>(a->sin);
+    p.cs_rs = a->cos_sin_row_stride;
+    p.eps = a->eps;
+    p.rows = a->rows; p.hq = a->hq; p.hkv = a->hkv; p.append = a->append ? 1 : 0;
+    p.a = AppendParams{};
+    if (a->append) {
+        p.a.pos_new = a->pos_new; p.a.cu_new = a->cu_new; p.a.slot_of = a->slot_of;
+        p.a.ck = static_cast<__bf16*>(a->cache.k);
+        p.a.cv = static_cast<__bf16*>(a->cache.v);
+        p.a.cpos = a->cache.pos;
+        p.a.start = a->cache.start;
+        p.a.len = a->cache.len;
+        p.a.ck_rs = a->cache.k_row_stride; p.a.ck_hs = a->cache.k_head_stride;
+        p.a.cv_rs = a->cache.v_row_stride; p.a.cv_hs = a->cache.v_head_stride;
+        p.a.capacity = a->cache.capacity; p.a.nseq = a->nseq; p.a.hkv = a->hkv;
+        p.a.overflow = a->overflow;
+    }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(qk_prep_kernel, dim3(a->rows), dim3(256), 0, st, p);
+    if (a->append) hipLaunchKernelGGL(kv_append_len_kernel, dim3((a->nseq + 63) / 64), dim3(64), 0, st, p.a);
+    return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
 }
 
 extern "C" int tah_kv_append(const tah_kv_append_args* a, tah_stream_t stream) {

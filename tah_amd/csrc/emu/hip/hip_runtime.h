@@ -267,13 +267,14 @@ inline emu_u32pair emu_permlane32_swap(unsigned a, unsigned b, bool, bool) {
 #define __builtin_amdgcn_permlane32_swap emu_permlane32_swap
 inline int __float_as_int(float x) { int i; memcpy(&i, &x, 4); return i; }
 inline float __int_as_float(int i) { float x; memcpy(&x, &i, 4); return x; }
-// DPP lane selects used by the kernels: quad_perm, row_shl/shr, row_mirror, row_half_mirror.
+// DPP lane selects used by the kernels: quad_perm, row_shl/shr/ror, row_mirror, row_half_mirror.
 inline int emu_update_dpp(int old, int src, int ctrl, int, int, bool bound_ctrl) {
     const int l = emu::t_lane, row = l & ~15, i = l & 15;
     int from = -1;
     if (ctrl < 0x100) from = (l & ~3) + ((ctrl >> (2 * (l & 3))) & 3);
     else if (ctrl >= 0x101 && ctrl <= 0x10f) { int j = i + (ctrl & 15); from = j < 16 ? row + j : -1; }
     else if (ctrl >= 0x111 && ctrl <= 0x11f) { int j = i - (ctrl & 15); from = j >= 0 ? row + j : -1; }
+    else if (ctrl >= 0x121 && ctrl <= 0x12f) from = row + ((i - (ctrl & 15)) & 15);  // row_ror
     else if (ctrl == 0x140) from = row + 15 - i;
     else if (ctrl == 0x141) from = row + (i & 8) + 7 - (i & 7);
     else { fprintf(stderr, "emu: unsupported dpp_ctrl 0x%x\n", ctrl); abort(); }

@@ -60,6 +60,66 @@ class KvSlabs:
         _capi.check(lib, lib.tah_kv_append(ctypes.byref(a), _stream(self.k)), "tah_kv_append")
 
 
+def qk_norm_rope(q: torch.Tensor, k: torch.Tensor, q_weight: torch.Tensor, k_weight: torch.Tensor,
+                 cos: torch.Tensor, sin: torch.Tensor, eps: float, *, v: Optional[torch.Tensor] = None,
+                 cache: Optional[KvSlabs] = None, cu_new: Optional[torch.Tensor] = None,
+                 pos_new: Optional[torch.Tensor] = None, slot_of: Optional[torch.Tensor] = None,
+                 in_place: bool = False):
+    """Per-head RMSNorm of q and k, rotary embedding of both and, with ``cache``, the KV append, in one
+    kernel: the steps of ``Qwen3Attention.forward`` between the projections and the attention call
+    (``q_norm``, ``k_norm``, ``apply_rotary_pos_emb``, ``past_key_values.update``), with bf16 roundings
+    where the eager modules round.
+
+    q ``[rows, Hq, 128]``, k / v ``[rows, Hkv, 128]`` (token-major, as the projections produce them),
+    weights ``[128]``, cos / sin ``[rows, 128]``, all bf16.  Returns ``(q_out, k_out)``; with ``cache``
+    K and V go to the slabs (rows ``[cu_new[i], cu_new[i+1])`` to slot ``slot_of[i]``) and ``k_out`` is
+    ``None``."""
+    lib = _lib.lib()
+    _thd(q, "q"), _thd(k, "k")
+    _dev_check(q, k, v, q_weight, k_weight, cos, sin, cu_new, pos_new, slot_of, cache.k if cache is not None else None)
+    for t, name in ((q_weight, "q_weight"), (k_weight, "k_weight")):
+        if t.dtype != torch.bfloat16 or t.shape != (q.shape[2],) or not t.is_contiguous():
+            raise _capi.TahDuoError(f"{name} must be a contiguous bf16 [{q.shape[2]}] tensor")
+    for t, name in ((cos, "cos"), (sin, "sin")):
+        if t.dtype != torch.bfloat16 or t.shape != (q.shape[0], q.shape[2]) or t.stride(1) != 1:
+            raise _capi.TahDuoError(f"{name} must be a bf16 [rows, {q.shape[2]}] tensor with unit inner stride")
+    if cos.stride(0) != sin.stride(0):
+        raise _capi.TahDuoError("cos and sin must share their row stride")
+    if k.shape[0] != q.shape[0]:
+        raise _capi.TahDuoError("q and k must have one row per token")
+    a = _capi.QkPrepArgs()
+    q_out = q if in_place else torch.empty_like(q)
+    a.q, a.k, a.v, a.q_out = _ptr(q), _ptr(k), _ptr(v), _ptr(q_out)
+    a.q_row_stride, a.q_head_stride = q.stride(0), q.stride(1)
+    a.k_row_stride, a.k_head_stride = k.stride(0), k.stride(1)
+    a.q_out_row_stride, a.q_out_head_stride = q_out.stride(0), q_out.stride(1)
+    if v is not None:
+        _thd(v, "v")
+        a.v_row_stride, a.v_head_stride = v.stride(0), v.stride(1)
+    a.q_weight, a.k_weight, a.cos, a.sin = _ptr(q_weight), _ptr(k_weight), _ptr(cos), _ptr(sin)
+    a.cos_sin_row_stride = cos.stride(0)
+    a.eps = float(eps)
+    a.rows, a.hq, a.hkv, a.d = q.shape[0], q.shape[1], k.shape[1], q.shape[2]
+    k_out = None
+    if cache is not None:
+        if v is None or cu_new is None:
+            raise _capi.TahDuoError("appending needs v and cu_new")
+        if (pos_new is None) != (cache.pos is None):
+            raise _capi.TahDuoError("pos_new must be given exactly for slabs created with_pos=True")
+        _i32(cu_new, "cu_new")
+        a.append = 1
+        a.cu_new, a.slot_of, a.pos_new = cu_new.data_ptr(), _ptr(slot_of), _ptr(pos_new)
+        a.nseq = cu_new.numel() - 1
+        a.cache = cache.segment()
+        a.overflow = cache.overflow.data_ptr()
+    else:
+        k_out = k if in_place else torch.empty_like(k)
+        a.k_out = _ptr(k_out)
+        a.k_out_row_stride, a.k_out_head_stride = k_out.stride(0), k_out.stride(1)
+    _capi.check(lib, lib.tah_qk_prep(ctypes.byref(a), _stream(q)), "tah_qk_prep")
+    return q_out, k_out
+
+
 _WORKSPACES = {}
 
 

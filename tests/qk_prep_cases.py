@@ -1,0 +1,38 @@
+"""Shared input builder and checks for the q/k RMSNorm + rotary (+ append) tests."""
+import numpy as np
+import torch
+
+from oracle import qk_prep_ref as R
+
+
+def make_case(seed, rows, hq, hkv, d=128, scale=1.0, max_pos=40000):
+    g = np.random.default_rng(seed)
+    rb = lambda *s: R.bf16_round((g.standard_normal(s) * scale).astype(np.float32))
+    pos = g.integers(0, max_pos, rows)
+    cos, sin = R.rotary_tables(pos)
+    return dict(q=rb(rows, hq, d), k=rb(rows, hkv, d), v=rb(rows, hkv, d),
+                qw=R.bf16_round((1.0 + 0.2 * g.standard_normal(d)).astype(np.float32)),
+                kw=R.bf16_round((1.0 + 0.2 * g.standard_normal(d)).astype(np.float32)),
+                cos=cos, sin=sin, pos=pos.astype(np.int32), eps=1e-6)
+
+
+def to_torch(case, device):
+    return {k: (torch.from_numpy(v).to(torch.bfloat16).to(device) if isinstance(v, np.ndarray) and v.dtype == np.float32
+                else (torch.from_numpy(v).to(device) if isinstance(v, np.ndarray) else v)) for k, v in case.items()}
+
+
+def assert_bf16_close(got: torch.Tensor, want: np.ndarray, what: str):
+    """The kernel and the oracle round at the same places; what is left is the summation order of the
+    mean and the reciprocal square root, i.e. one bf16 unit in the last place of a normalised value
+    now and then.  The rotation adds two products that may cancel, so the bound is stated against the
+    size of the rotary pair (which the rotation keeps), not of the element: error <= 2^-6 of it, and
+    all but a few elements equal bit for bit."""
+    g = got.float().cpu().numpy()
+    half = want.shape[-1] // 2
+    mag = np.sqrt(want[..., :half].astype(np.float64) ** 2 + want[..., half:].astype(np.float64) ** 2)
+    mag = np.concatenate([mag, mag], axis=-1)
+    err = np.abs(g.astype(np.float64) - want)
+    exact = float(np.mean(g == want))
+    worst = float(np.max(err / np.maximum(mag, 1e-30)))
+    assert worst <= 2.0 ** -6 and exact >= 0.995, f"{what}: worst error / pair size {worst:.3e}, exact fraction {exact:.5f}"
+    return exact

@@ -1,0 +1,73 @@
+"""q/k RMSNorm + rotary embedding (+ KV append) kernel on the CPU execution shim against the oracle.  No GPU."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import qk_prep_ref as R
+from tests import emu_util
+from tests.qk_prep_cases import assert_bf16_close, make_case, to_torch
+
+pytestmark = pytest.mark.skipif(not emu_util.have_host_clang(), reason="host clang++ not available")
+
+
+@pytest.mark.parametrize("rows,hq,hkv,scale", [(5, 4, 2, 1.0), (3, 2, 2, 20.0), (4, 8, 1, 0.03)])
+def test_norm_rope_matches_oracle(rows, hq, hkv, scale):
+    from tah_amd.kv_cache import qk_norm_rope
+    c = make_case(10 + rows, rows, hq, hkv, scale=scale)
+    t = to_torch(c, "cpu")
+    with emu_util.emulated():
+        q_out, k_out = qk_norm_rope(t["q"], t["k"], t["qw"], t["kw"], t["cos"], t["sin"], c["eps"])
+    wq, wk = R.qk_prep(c["q"], c["k"], c["qw"], c["kw"], c["cos"], c["sin"], c["eps"])
+    assert_bf16_close(q_out, wq, "q")
+    assert_bf16_close(k_out, wk, "k")
+
+
+def test_in_place_on_strided_views_of_a_fused_projection():
+    from tah_amd.kv_cache import qk_norm_rope
+    c = make_case(21, 6, 4, 2)
+    t = to_torch(c, "cpu")
+    fused = torch.zeros(6, 4 + 2 + 2, 128, dtype=torch.bfloat16)
+    fused[:, :4], fused[:, 4:6], fused[:, 6:] = t["q"], t["k"], t["v"]
+    with emu_util.emulated():
+        q_out, k_out = qk_norm_rope(fused[:, :4], fused[:, 4:6], t["qw"], t["kw"], t["cos"], t["sin"], c["eps"], in_place=True)
+    wq, wk = R.qk_prep(c["q"], c["k"], c["qw"], c["kw"], c["cos"], c["sin"], c["eps"])
+    assert q_out.data_ptr() == fused.data_ptr()
+    assert_bf16_close(fused[:, :4], wq, "q")
+    assert_bf16_close(fused[:, 4:6], wk, "k")
+    assert torch.equal(fused[:, 6:], t["v"])
+
+
+def test_fused_append_equals_norm_rope_then_append():
+    from tah_amd.kv_cache import KvSlabs, qk_norm_rope
+    c = make_case(22, 7, 4, 2)
+    t = to_torch(c, "cpu")
+    cu = torch.tensor([0, 3, 7], dtype=torch.int32)
+    slot_of = torch.tensor([2, 0], dtype=torch.int32)
+    with emu_util.emulated():
+        a, b = KvSlabs(3, 5, 2, with_pos=True, device="cpu"), KvSlabs(3, 5, 2, with_pos=True, device="cpu")
+        q1, none = qk_norm_rope(t["q"], t["k"], t["qw"], t["kw"], t["cos"], t["sin"], c["eps"], v=t["v"], cache=a,
+                                cu_new=cu, pos_new=t["pos"], slot_of=slot_of)
+        q2, k2 = qk_norm_rope(t["q"], t["k"], t["qw"], t["kw"], t["cos"], t["sin"], c["eps"])
+        b.append(k2, t["v"], cu, pos_new=t["pos"], slot_of=slot_of)
+        assert none is None and torch.equal(q1, q2)
+        for x, y in ((a.k, b.k), (a.v, b.v), (a.pos, b.pos), (a.len, b.len), (a.overflow, b.overflow)):
+            assert torch.equal(x, y)
+        assert a.len.tolist() == [4, 0, 3]
+        # a second append that does not fit: rows dropped, flag raised, as tah_kv_append does
+        qk_norm_rope(t["q"][:3], t["k"][:3], t["qw"], t["kw"], t["cos"][:3], t["sin"][:3], c["eps"], v=t["v"][:3], cache=a,
+                     cu_new=torch.tensor([0, 3], dtype=torch.int32), pos_new=t["pos"][:3], slot_of=torch.tensor([0], dtype=torch.int32))
+        assert a.overflow.item() == 1 and a.len.tolist() == [5, 0, 3]
+
+
+def test_argument_checks():
+    from tah_amd import TahDuoError
+    from tah_amd.kv_cache import qk_norm_rope
+    c = make_case(23, 2, 2, 1)
+    t = to_torch(c, "cpu")
+    with emu_util.emulated():
+        with pytest.raises(TahDuoError):
+            qk_norm_rope(t["q"], t["k"], t["qw"].float(), t["kw"], t["cos"], t["sin"], 1e-6)
+        with pytest.raises(TahDuoError):
+            qk_norm_rope(t["q"], t["k"][:1], t["qw"], t["kw"], t["cos"], t["sin"], 1e-6)
+        with pytest.raises(TahDuoError):
+            qk_norm_rope(t["q"], t["k"], t["qw"], t["kw"], t["cos"][:, :64], t["sin"][:, :64], 1e-6)
