@@ -358,19 +358,39 @@ __global__ __launch_bounds__(256) void qk_prep_kernel(const PrepParams p) {
     const int r = blockIdx.x;
     const int lane = threadIdx.x % kWave;
     const int sub = threadIdx.x / 16, j = lane % 16;  // head slot 0..15 of a pass, 16-byte piece of the head
+    const int items = p.hq + 2 * p.hkv;
+    // the row's data first: nothing below that decides where the results go depends on it, and the
+    // loads then fly while the destination is looked up
+    auto load_item = [&](int it) {
+        u32x4 x = {0u, 0u, 0u, 0u};
+        if (it < p.hq) x = *reinterpret_cast<const u32x4*>(p.q + (int64_t)r * p.q_rs + (int64_t)it * p.q_hs + 8 * j);
+        else if (it < p.hq + p.hkv)
+            x = *reinterpret_cast<const u32x4*>(p.k + (int64_t)r * p.k_rs + (int64_t)(it - p.hq) * p.k_hs + 8 * j);
+        else if (it < items && p.v && (p.append || p.v_out))
+            x = *reinterpret_cast<const u32x4*>(p.v + (int64_t)r * p.v_rs + (int64_t)(it - p.hq - p.hkv) * p.v_hs + 8 * j);
+        return x;
+    };
+    constexpr int kAhead = 2;  // passes loaded up front (32 heads: the whole row at Hq = 16, Hkv = 8)
+    u32x4 ahead[kAhead];
+#pragma unroll
+    for (int i = 0; i < kAhead; ++i) ahead[i] = load_item(16 * i + sub);
+    const u32x4 cs = *reinterpret_cast<const u32x4*>(p.cos + (int64_t)r * p.cs_rs + 8 * j);
+    const u32x4 sn = *reinterpret_cast<const u32x4*>(p.sin + (int64_t)r * p.cs_rs + 8 * j);
+    const u32x4 qw = *reinterpret_cast<const u32x4*>(p.qw + 8 * j), kw = *reinterpret_cast<const u32x4*>(p.kw + 8 * j);
+
     __bf16 *kdst = nullptr, *vdst = nullptr;
     int64_t kd_hs = 0, vd_hs = 0;
     if (p.append) {
         int seq = 0;  // sequence of new row r
         for (int b = 0; b < p.a.nseq; ++b)
-            if (r >= p.a.cu_new[b + 1]) seq = b + 1;
+            if (r >= const_i32(p.a.cu_new, b + 1)) seq = b + 1;
         if (seq < p.a.nseq) {
-            const int slot = p.a.slot_of ? p.a.slot_of[seq] : seq;
-            const int dst = p.a.len[slot] + (r - p.a.cu_new[seq]);
+            const int slot = p.a.slot_of ? const_i32(p.a.slot_of, seq) : seq;
+            const int dst = p.a.len[slot] + (r - const_i32(p.a.cu_new, seq));
             if (dst >= p.a.capacity) {
                 if (p.a.overflow && threadIdx.x == 0) *p.a.overflow = 1;
             } else {
-                const int64_t drow = (int64_t)p.a.start[slot] + dst;
+                const int64_t drow = (int64_t)const_i32(p.a.start, slot) + dst;
                 kdst = p.a.ck + drow * p.a.ck_rs;
                 vdst = p.a.cv + drow * p.a.cv_rs;
                 kd_hs = p.a.ck_hs;
@@ -386,32 +406,25 @@ __global__ __launch_bounds__(256) void qk_prep_kernel(const PrepParams p) {
             vd_hs = p.vo_hs;
         }
     }
-    const u32x4 cs = *reinterpret_cast<const u32x4*>(p.cos + (int64_t)r * p.cs_rs + 8 * j);
-    const u32x4 sn = *reinterpret_cast<const u32x4*>(p.sin + (int64_t)r * p.cs_rs + 8 * j);
-    const u32x4 qw = *reinterpret_cast<const u32x4*>(p.qw + 8 * j), kw = *reinterpret_cast<const u32x4*>(p.kw + 8 * j);
     const uint32_t sign = j < 8 ? 0x80008000u : 0u;  // lower half of the head: -partner * sin
-    const int items = p.hq + 2 * p.hkv;
     // (every lane of a wave walks the same number of passes and takes part in every lane exchange;
     // what a 16-lane row has no head for is predicated off)
-    for (int base = 0; base < items; base += 16) {
-        const int it = base + sub;
+    for (int pass = 0; pass * 16 < items; ++pass) {
+        const int it = pass * 16 + sub;
         const bool is_q = it < p.hq, is_k = !is_q && it < p.hq + p.hkv, is_v = !is_q && !is_k && it < items;
-        if (is_v && vdst) {  // a V head: moved as it is
-            const int h = it - p.hq - p.hkv;
-            *reinterpret_cast<u32x4*>(vdst + (int64_t)h * vd_hs + 8 * j) =
-                *reinterpret_cast<const u32x4*>(p.v + (int64_t)r * p.v_rs + (int64_t)h * p.v_hs + 8 * j);
-        }
+        const u32x4 xin = pass == 0 ? ahead[0] : pass == 1 ? ahead[1] : load_item(it);
+        if (is_v && vdst)  // a V head: moved as it is
+            *reinterpret_cast<u32x4*>(vdst + (int64_t)(it - p.hq - p.hkv) * vd_hs + 8 * j) = xin;
         const int h = is_q ? it : it - p.hq;
-        const __bf16* x = is_q ? p.q + (int64_t)r * p.q_rs + (int64_t)h * p.q_hs : p.k + (int64_t)r * p.k_rs + (int64_t)h * p.k_hs;
         __bf16* y = is_q ? p.q_out + (int64_t)r * p.qo_rs + (int64_t)h * p.qo_hs
                          : (is_k && kdst ? kdst + (int64_t)h * kd_hs : nullptr);  // null: no head, or the row overflows its slab
-        u32x4 xin = {0u, 0u, 0u, 0u};
-        if (is_q || is_k) xin = *reinterpret_cast<const u32x4*>(x + 8 * j);
         float ss = 0.f;
 #pragma unroll
         for (int i = 0; i < 4; ++i) ss += bf16_lo(xin[i]) * bf16_lo(xin[i]) + bf16_hi(xin[i]) * bf16_hi(xin[i]);
         ss = row16_sum(ss);
-        const float rs = 1.0f / sqrtf(ss * (1.0f / 128.0f) + p.eps);
+        // hardware reciprocal square root (1 ulp): whether it or the order of the sum above decides
+        // the last bit of a normalised value before the bf16 rounding is the same kind of difference
+        const float rs = __builtin_amdgcn_rsqf(ss * (1.0f / 128.0f) + p.eps);
         const u32x4 w = is_q ? qw : kw;
         u32x4 yn, out;
 #pragma unroll
