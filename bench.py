@@ -25,8 +25,9 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, vendor figure
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a plain copy of
 # known size (profiles/*_counters.md); valid for the default workloads only.
-TRAFFIC_FWD_BYTES = 202.2e6 + 72.2e6
+TRAFFIC_FWD_BYTES = 203.3e6 + 72.2e6
 TRAFFIC_DECODE_BYTES = 2.329e9 + 5.1e6 + 5.2e6 + 0.3e6
+TRAFFIC_QK_PREP_BYTES = 142.7e6 + 134.2e6
 
 
 def visible_pairs(case):
@@ -177,7 +178,7 @@ def bench_qk_prep(steps: int, warmup: int):
                         "Hq=16, Hkv=8, D=128 (includes a 4-element length reset per step)",
             "ms_per_step": ms, "algorithmic_bytes": nbytes, "hbm_gbs": gbs,
             "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
-                         "traffic": None, "kernels": "qk_prep_kernel + kv_append_len_kernel"},
+                         "traffic": TRAFFIC_QK_PREP_BYTES, "kernels": "qk_prep_kernel + kv_append_len_kernel"},
             "tokens_per_s": rows / (ms * 1e-3)}
 
 
