@@ -6,7 +6,9 @@ third-party code, so these vectors come from this repository's own restatements:
 value below is produced by oracle/duo_ref.c (float64 accumulation, analytic backward) and is only
 written after the independent float64 row-loop / torch-autograd restatement in
 oracle/duo_oracle.py agrees with it.  Inputs are stored as bf16 bit patterns (uint16), expected
-values as float32.  Run from the repo root:  python tests/golden/make_golden.py
+values as float32.  qk_prep_small.npz is the exception: its expected values are the outputs of the
+third-party modules the reference calls (transformers' Qwen3RMSNorm / apply_rotary_pos_emb, installed
+version recorded in the file), bf16 bit patterns.  Run from the repo root:  python tests/golden/make_golden.py
 """
 import os
 import sys
@@ -103,10 +105,39 @@ def pack():
         scattered_assigned=O.scatter_back(mask, gx, dest, assignment_mask=amask).numpy())
 
 
+def qk_prep():
+    """Expected values from the third-party modules themselves (the installed transformers'
+    Qwen3RMSNorm and apply_rotary_pos_emb, bf16 on the CPU), written only if the oracle's restatement
+    agrees with them to one bf16 unit in the last place on at most 0.1 % of the elements."""
+    from transformers.models.qwen3 import modeling_qwen3 as m
+
+    from oracle import qk_prep_ref as Q
+    from tests.qk_prep_cases import make_case
+
+    c = make_case(4246, 19, 4, 2, scale=1.5)
+    bf = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(torch.bfloat16)
+    qn, kn = m.Qwen3RMSNorm(128, eps=c["eps"]).to(torch.bfloat16), m.Qwen3RMSNorm(128, eps=c["eps"]).to(torch.bfloat16)
+    with torch.no_grad():
+        qn.weight.copy_(bf(c["qw"])), kn.weight.copy_(bf(c["kw"]))
+        tq, tk = qn(bf(c["q"])).transpose(0, 1)[None], kn(bf(c["k"])).transpose(0, 1)[None]
+        wq, wk = m.apply_rotary_pos_emb(tq, tk, bf(c["cos"])[None], bf(c["sin"])[None])
+    wq, wk = wq[0].transpose(0, 1).contiguous(), wk[0].transpose(0, 1).contiguous()
+    gq, gk = Q.qk_prep(c["q"], c["k"], c["qw"], c["kw"], c["cos"], c["sin"], c["eps"])
+    for got, want in ((gq, wq.float().numpy()), (gk, wk.float().numpy())):
+        ulp = np.abs(got.view(np.int32).astype(np.int64) - want.view(np.int32).astype(np.int64)) >> 16
+        assert np.mean(got == want) > 0.999 and ulp.max() <= 1
+    np.savez_compressed(
+        os.path.join(HERE, "qk_prep_small.npz"),
+        **{n: bits(bf(c[n])) for n in ("q", "k", "v", "qw", "kw", "cos", "sin")},
+        pos=c["pos"], eps=np.float32(c["eps"]), q_out=bits(wq), k_out=bits(wk),
+        transformers_version=np.array(__import__("transformers").__version__))
+
+
 if __name__ == "__main__":
     prefill()
     decode()
     pack()
+    qk_prep()
     for f in sorted(os.listdir(HERE)):
         if f.endswith(".npz"):
             print(f, os.path.getsize(os.path.join(HERE, f)), "bytes")

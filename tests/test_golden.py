@@ -95,12 +95,40 @@ def _check_pack(device):
     assert np.array_equal(scatter_back(mask, gx, dest, assignment_mask=am).cpu().numpy(), z["scattered_assigned"])
 
 
+def _load_qk_prep():
+    z = np.load(os.path.join(G, "qk_prep_small.npz"))
+    return z, {k: _bf16(z[k]) for k in ("q", "k", "v", "qw", "kw", "cos", "sin", "q_out", "k_out")}
+
+
+def test_oracle_reproduces_qk_prep_fixture():
+    """The fixture's expected values come from the third-party modules themselves."""
+    from oracle import qk_prep_ref as Q
+    from tests.qk_prep_cases import assert_bf16_close
+    z, c = _load_qk_prep()
+    f = lambda k: c[k].float().numpy()
+    gq, gk = Q.qk_prep(f("q"), f("k"), f("qw"), f("kw"), f("cos"), f("sin"), float(z["eps"]))
+    assert np.mean(gq == f("q_out")) > 0.999 and np.mean(gk == f("k_out")) > 0.999
+    assert_bf16_close(torch.from_numpy(gq), f("q_out"), "q")
+    assert_bf16_close(torch.from_numpy(gk), f("k_out"), "k")
+
+
+def _check_qk_prep(device):
+    from tah_amd.kv_cache import qk_norm_rope
+    from tests.qk_prep_cases import assert_bf16_close
+    z, c = _load_qk_prep()
+    d = {k: v.to(device) for k, v in c.items()}
+    q_out, k_out = qk_norm_rope(d["q"], d["k"], d["qw"], d["kw"], d["cos"], d["sin"], float(z["eps"]))
+    assert_bf16_close(q_out, c["q_out"].float().numpy(), "q vs fixture")
+    assert_bf16_close(k_out, c["k_out"].float().numpy(), "k vs fixture")
+
+
 @pytest.mark.skipif(not emu_util.have_host_clang(), reason="host clang++ not available")
 def test_kernels_on_cpu_shim_match_fixtures():
     with emu_util.emulated():
         _check_prefill(lambda t: t)
         _check_decode("cpu")
         _check_pack("cpu")
+        _check_qk_prep("cpu")
 
 
 @pytest.mark.gpu
@@ -108,3 +136,4 @@ def test_hip_path_matches_fixtures():
     _check_prefill(lambda t: t.cuda())
     _check_decode("cuda")
     _check_pack("cuda")
+    _check_qk_prep("cuda")
