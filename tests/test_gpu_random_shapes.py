@@ -42,3 +42,28 @@ def test_random_shape_forward_and_backward(seed):
     got, want = run_bwd(dev, seed + 1)
     torch.cuda.synchronize()
     check_grads(got, want)
+
+
+def _draw_decode(seed):
+    g = np.random.default_rng(seed)
+    hkv = int(g.choice([1, 2, 4, 8]))
+    hq = min(32, hkv * int(g.choice([1, 2, 4, 8])))
+    nseq = int(g.integers(1, 9))
+    lens = [int(x) for x in 1 + (g.pareto(1.2, nseq) * 300).astype(int) % 5000]
+    return hq, hkv, lens, float(g.choice([0.0, 0.06, 0.3, 1.0])), bool(g.random() < 0.5)
+
+
+@pytest.mark.parametrize("seed", list(range(600, 616)))
+def test_random_shape_decode(seed):
+    from tests.cases import make_decode_case
+    from tests.test_gpu_decode import oracle_decode_c, run_decode
+    hq, hkv, lens, p, fused = _draw_decode(seed)
+    print(f"case random decode seed={seed} hq={hq} hkv={hkv} lens={lens} p={p} fused={fused}", flush=True)
+    c = make_decode_case(seed, lens, p, Hq=hq, Hkv=hkv)
+    got = run_decode(c, 5120, 5120, fused)
+    w0, wl0, w1, wl1 = oracle_decode_c(c)
+    assert_close(got[0], w0, "decode o depth0")
+    np.testing.assert_allclose(got[1].cpu().numpy(), wl0, atol=5e-3, rtol=1e-3)
+    if len(c["hard_rows"]):
+        assert_close(got[2], w1, "decode o depth1")
+        np.testing.assert_allclose(got[3].cpu().numpy(), wl1, atol=5e-3, rtol=1e-3)
