@@ -22,6 +22,20 @@ def test_norm_rope_matches_oracle(rows, hq, hkv, scale):
     assert_bf16_close(k_out, wk, "k")
 
 
+def test_more_heads_than_one_pass_pair_and_empty_input():
+    """48 head slots per row (three passes of 16; the first two are loaded up front), and a call with no rows."""
+    from tah_amd.kv_cache import qk_norm_rope
+    c = make_case(31, 3, 32, 8)
+    t = to_torch(c, "cpu")
+    with emu_util.emulated():
+        q_out, k_out = qk_norm_rope(t["q"], t["k"], t["qw"], t["kw"], t["cos"], t["sin"], c["eps"])
+        e_q, e_k = qk_norm_rope(t["q"][:0], t["k"][:0], t["qw"], t["kw"], t["cos"][:0], t["sin"][:0], c["eps"])
+    wq, wk = R.qk_prep(c["q"], c["k"], c["qw"], c["kw"], c["cos"], c["sin"], c["eps"])
+    assert_bf16_close(q_out, wq, "q")
+    assert_bf16_close(k_out, wk, "k")
+    assert e_q.shape == (0, 32, 128) and e_k.shape == (0, 8, 128)
+
+
 def test_in_place_on_strided_views_of_a_fused_projection():
     from tah_amd.kv_cache import qk_norm_rope
     c = make_case(21, 6, 4, 2)

@@ -14,6 +14,7 @@ pytestmark = pytest.mark.gpu
     (1000, 16, 8, 25.0, 2),    # large activations
     (77, 8, 1, 0.02, 3),       # small activations (eps matters), group of 8
     (1, 4, 4, 1.0, 4),         # one decode row
+    (65, 32, 8, 1.0, 8),       # 48 head slots per row: three passes
 ])
 def test_norm_rope_matches_oracle(rows, hq, hkv, scale, seed):
     from tah_amd.kv_cache import qk_norm_rope
