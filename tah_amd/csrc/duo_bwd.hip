@@ -11,9 +11,11 @@
 //             gradient from depth-0 and depth-1 queries):
 //             S = Q K^T, dP = dO V^T, dV += P^T dO, dK += dS^T Q
 // P is recomputed from the saved log-sum-exp.  In dkdv each lane owns one key
-// (accumulator column) and K/V fragments stay in registers for the whole
-// workgroup; Q and dO tiles are staged in LDS and read both row-wise (A
-// operand) and, through ds_read_b64_tr_b16, column-wise (B operand).
+// (accumulator column); the workgroup's K and V tiles and the staged Q and dO
+// tiles sit in LDS, the latter read both row-wise (A operand) and, through
+// ds_read_b64_tr_b16, column-wise (B operand).  The 32 MFMAs of an item are
+// laid out as explicit slots with their LDS reads issued two to three slots
+// ahead and the exp / convert arithmetic sliced in behind the dP and dV MFMAs.
 #include <hip/hip_runtime.h>
 
 #include <type_traits>
@@ -21,12 +23,11 @@
 #include "duo_device.h"
 #include "tah_duo.h"
 
-#ifndef TAH_DKDV_SCHED
-#define TAH_DKDV_SCHED 1  // 1: LDS reads four MFMAs ahead; n > 1: also n vector instructions behind each dP / dV MFMA; 0: compiler order
-#endif
 
 namespace tah {
 namespace {
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kD = 128;
 constexpr int kBN = 64;
@@ -368,9 +369,9 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
             async_copy_16B(vbase, lr * vrs2 + chunk, smem + kKvV + blk * 1024);
         }
     }
-    int boff[8];  // B-operand row 32*kb + col (my key) of the K tile, chunk 2s + half; V tile: + kKvV - kKvK
-#pragma unroll
-    for (int s8 = 0; s8 < 8; ++s8) boff[s8] = kKvK + rowmajor128_off(32 * kb + col, 2 * s8 + half);
+    // B-operand row 32*kb + col (my key) of the K tile, chunk 2s + half; V tile: + kKvV - kKvK.  The
+    // swizzle XORs the chunk index, so chunk 2s + half sits at (offset of chunk `half`) ^ 32s.
+    const int boff0 = kKvK + rowmajor128_off(32 * kb + col, half);
 
     // query tiles that can see this key tile
     const int kl0 = key0 - k_lo;  // local index of the tile's first key (depth-0 tiles: its position)
@@ -424,177 +425,227 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
     const int my_lrow = 8 * wave + (lane >> 4);  // second piece: 4 rows further down
     const uint32_t my_chunk0 = (uint32_t)(((lane & 15) ^ row_swizzle(my_lrow)) * 16);
     const uint32_t my_chunk1 = (uint32_t)(((lane & 15) ^ row_swizzle(my_lrow + 4)) * 16);
-    auto issue_item = [&](int item, int buf) {
-        bool q2s;
-        int r0, r_end, head;
-        item_rows(item, q2s, r0, r_end, head);
+    // The query stream that staged items come from, held in scalar registers: its fields are read from
+    // the kernel arguments once per stream, not once per item (each read is a scalar-memory round trip
+    // that every wave would sit through right after the barrier).
+    struct ItemSrc {
+        const __bf16 *q, *g;
+        const float *lse, *delta;
+        const int32_t* pos;
+        uint32_t qrs2, grs2;
+        int64_t q_hs, g_hs;
+        int32_t total_q, row_lo, row_end, tile0;
+    };
+    auto stream_src = [&](bool q2s) {
         const BwdStream& qs = q2s ? p.s2 : p.s1;
+        ItemSrc r;
+        r.q = qs.q; r.g = qs.d_o; r.lse = qs.lse; r.delta = qs.delta; r.pos = qs.pos_q;
+        r.qrs2 = (uint32_t)(qs.q_rs * 2) & 0xffffffu;
+        r.grs2 = (uint32_t)(qs.do_rs * 2) & 0xffffffu;
+        r.q_hs = qs.q_hs; r.g_hs = qs.do_hs;
+        r.total_q = qs.total_q;
+        r.row_lo = q2s ? q2_lo : q1_lo + t1_begin * kBQ;
+        r.row_end = q2s ? q2_lo + lq2 : q1_lo + lq1;
+        r.tile0 = q2s ? nt1 : 0;
+        return r;
+    };
+    ItemSrc src = stream_src(nt1 == 0);
+    auto issue_item = [&](int item, int buf) {
+        const int t = item / G, head = hk * G + item % G;
+        const bool q2s = src.tile0 != 0 || nt1 == 0;
+        const int r0 = src.row_lo + (t - src.tile0) * kBQ;
+        const int r_end = r0 + kBQ < src.row_end ? r0 + kBQ : src.row_end;
         unsigned char* qt = smem + buf * kKvSlot;
         unsigned char* gt = qt + kTileBytes;
         float* meta = reinterpret_cast<float*>(smem + kKvMeta + buf * kKvMetaBytes);
         const int last = r_end - 1 - r0;
         const uint32_t l0 = (uint32_t)(my_lrow < last ? my_lrow : last) & 63u;
         const uint32_t l1 = (uint32_t)(my_lrow + 4 < last ? my_lrow + 4 : last) & 63u;
-        const uint32_t qrs2 = (uint32_t)(qs.q_rs * 2) & 0xffffffu, grs2 = (uint32_t)(qs.do_rs * 2) & 0xffffffu;
-        const __bf16* qbase = qs.q + (int64_t)r0 * qs.q_rs + (int64_t)head * qs.q_hs;
-        const __bf16* gbase = qs.d_o + (int64_t)r0 * qs.do_rs + (int64_t)head * qs.do_hs;
-        async_copy_16B(qbase, l0 * qrs2 + my_chunk0, qt + (2 * wave) * 1024);
-        async_copy_16B(gbase, l0 * grs2 + my_chunk0, gt + (2 * wave) * 1024);
-        async_copy_16B(qbase, l1 * qrs2 + my_chunk1, qt + (2 * wave + 1) * 1024);
-        async_copy_16B(gbase, l1 * grs2 + my_chunk1, gt + (2 * wave + 1) * 1024);
+        const __bf16* qbase = src.q + ((int64_t)r0 * (src.qrs2 >> 1) + (int64_t)head * src.q_hs);
+        const __bf16* gbase = src.g + ((int64_t)r0 * (src.grs2 >> 1) + (int64_t)head * src.g_hs);
+        async_copy_16B(qbase, l0 * src.qrs2 + my_chunk0, qt + (2 * wave) * 1024);
+        async_copy_16B(gbase, l0 * src.grs2 + my_chunk0, gt + (2 * wave) * 1024);
+        async_copy_16B(qbase, l1 * src.qrs2 + my_chunk1, qt + (2 * wave + 1) * 1024);
+        async_copy_16B(gbase, l1 * src.grs2 + my_chunk1, gt + (2 * wave + 1) * 1024);
         const uint32_t lm = (uint32_t)(lane < last ? lane : last) * 4u;
-        if (wave == 0) async_copy_4B(qs.lse + (int64_t)head * qs.total_q + r0, lm, meta);
-        if (wave == 1) async_copy_4B(qs.delta + (int64_t)head * qs.total_q + r0, lm, meta + kBQ);
-        if (wave == 2 && q2s) async_copy_4B(qs.pos_q + r0, lm, meta + 2 * kBQ);
+        const int64_t hrow = (int64_t)head * src.total_q + r0;
+        if (wave == 0) async_copy_4B(src.lse + hrow, lm, meta);
+        if (wave == 1) async_copy_4B(src.delta + hrow, lm, meta + kBQ);
+        if (wave == 2 && q2s) async_copy_4B(src.pos + r0, lm, meta + 2 * kBQ);
     };
     auto advance = [&](int item) {
         TAH_WAIT_VMEM();
         __syncthreads();
+        if (item + 1 == nt1 * G) src = stream_src(true);  // the next item is the first of the depth-1 stream
         if (item + 1 < nitems) issue_item(item + 1, (item & 1) ^ 1);
     };
 
     // per-lane LDS read offsets inside a tile, computed once
-    int aoff[8];  // A-operand rows 32*qh + col of the Q / dO tiles, chunk 2s + half
-#pragma unroll
-    for (int s8 = 0; s8 < 8; ++s8) aoff[s8] = rowmajor128_off(32 * qh + col, 2 * s8 + half);
-    int toff_lo[4], toff_hi[4];  // transpose reads: rows 32*qh + 4*half + r/4 (+8), columns 32*dt + 16*grp + 4*(r%4)
+    const int aoff0 = rowmajor128_off(32 * qh + col, half);  // A-operand rows 32*qh + col of the Q / dO tiles, chunk 2s + half: ^ 32s
+    // transpose reads: rows 32*qh + 4*half + r/4 (+8), columns 32*dt + 16*grp + 4*(r%4); column block dt
+    // sits at (offset of block 0) ^ 64dt
+    int toff_lo0, toff_hi0;
     {
         const int r16 = lane & 15, grp = (lane >> 4) & 1;
         const int trow = 32 * qh + 4 * half + (r16 >> 2);
-#pragma unroll
-        for (int dt = 0; dt < 4; ++dt) {
-            const int tcol = 32 * dt + 16 * grp + 4 * (r16 & 3);
-            toff_lo[dt] = rowmajor128_off(trow, tcol >> 3) + (tcol & 7) * 2;
-            toff_hi[dt] = rowmajor128_off(trow + 8, tcol >> 3) + (tcol & 7) * 2;
-        }
+        const int tcol = 16 * grp + 4 * (r16 & 3);
+        toff_lo0 = rowmajor128_off(trow, tcol >> 3) + (tcol & 7) * 2;
+        toff_hi0 = rowmajor128_off(trow + 8, tcol >> 3) + (tcol & 7) * 2;
     }
     const int mrow = 32 * qh + 4 * half;  // my accumulator rows: mrow + 8*(r/4) + r%4
 
-    auto body = [&](int item, auto mask_tag) __attribute__((always_inline)) {
+    // One item = 32 MFMAs per wave (S 8, dP 8, dV 8, dK 8), written as 32 slots in program order with
+    // scheduling fences between them so that the order below is the order in the binary: every slot
+    // first issues the LDS reads of a later slot (two slots ahead for the S / dP operand pairs, three
+    // for the transpose reads of dV / dK), then its MFMA, then a slice of the vector work -- P for two
+    // query rows behind each dP MFMA, dS for two rows behind each dV MFMA -- so LDS latency and the
+    // exp / convert arithmetic run in the shadow of the matrix pipe.
+    auto body = [&](int item, auto mask_tag, auto stage_tag) __attribute__((always_inline)) {
         constexpr bool kMasked = decltype(mask_tag)::value;
-        const unsigned char* qt = smem + (item & 1) * kKvSlot;
+        constexpr int kStage = decltype(stage_tag)::value;  // 0 / 1: stage known at compile time; -1: item & 1
+        const int stage = kStage >= 0 ? kStage : (item & 1);
+        const unsigned char* qt = smem + stage * kKvSlot;
         const unsigned char* gt = qt + kTileBytes;
-        const float* meta = reinterpret_cast<const float*>(smem + kKvMeta + (item & 1) * kKvMetaBytes);
+        const float* meta = reinterpret_cast<const float*>(smem + kKvMeta + stage * kKvMetaBytes);
 
-        // S = Q K^T for my 32 queries x 32 keys (lane = key, reg = query), P from the saved log-sum-exp;
-        // then dP = dO V^T and dS = P o (dP - delta).  One 16-register product is live at a time, and
-        // dS is formed from the bf16 P that the dV product uses.
-        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        [[maybe_unused]] bool q2s = false;
+        [[maybe_unused]] int nvalid = kBQ, pos0 = 0;
+        [[maybe_unused]] const int* qposs = reinterpret_cast<const int*>(meta) + 2 * kBQ;
+        [[maybe_unused]] int dense_head = 0, dense_q0 = 0;
+        if constexpr (kMasked) {
+            int r0, r_end, head;
+            item_rows(item, q2s, r0, r_end, head);
+            nvalid = r_end - r0;        // rows of the tile that exist
+            pos0 = (r0 - q1_lo) + off;  // depth-0 stream: position of tile row 0
+            dense_head = head;
+            dense_q0 = r0 - q1_lo;      // additive-mask mode: query index of tile row 0
+        }
+
+        bf16x8 ra[3], rb[3], rt[4];  // operand rings
+        f32x4 lse4[2], del4[2];      // log-sum-exp / delta of four consecutive rows, two sets in flight
+        f32x16 sacc, dpacc;
         bf16x8 pfr[2], dsfr[2];
-        {
-            f32x16 sacc = mfma32(*reinterpret_cast<const bf16x8*>(qt + aoff[0]),
-                                 *reinterpret_cast<const bf16x8*>(smem + boff[0]), zero);
+        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+        // operands of slot n < 16: rows of the Q (S) or dO (dP) tile, my key's row of the K or V tile
+        // (their addresses are one XOR away from two base registers: cheaper than sixteen registers
+        // that stay live through the loop)
+        int abase = aoff0, bbase = boff0, tlo = toff_lo0, thi = toff_hi0;
+        TAH_OPAQUE2(abase, bbase);
+        TAH_OPAQUE2(tlo, thi);
+        // (likewise the sixteen row numbers and position addresses of the masked variants)
+        [[maybe_unused]] int mrow_m = mrow, kpos_m = kpos;
+        if constexpr (kMasked) TAH_OPAQUE2(mrow_m, kpos_m);
+        auto load_ab = [&](int n) __attribute__((always_inline)) {
+            ra[n % 3] = *reinterpret_cast<const bf16x8*>((n < 8 ? qt : gt) + (abase ^ (32 * (n % 8))));
+            rb[n % 3] = *reinterpret_cast<const bf16x8*>(smem + (n < 8 ? 0 : kKvV - kKvK) + (bbase ^ (32 * (n % 8))));
+        };
+        // B operand of tail slot m: dO columns (dV, m < 8) or Q columns (dK) of my 32 query rows
+        auto load_t = [&](int m) __attribute__((always_inline)) {
+            const unsigned char* t = m < 8 ? gt : qt;
+            const int st = (m % 8) / 4, dt = m % 4;
+            const bf16x4 lo = lds_read_tr16(t + (tlo ^ (64 * dt)) + st * 4096);
+            const bf16x4 hi = lds_read_tr16(t + (thi ^ (64 * dt)) + st * 4096);
+            rt[m % 4] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        };
+        // P for accumulator rows r, r + 1 (r even) from S and the saved log-sum-exp
+        auto p_rows = [&](int r) __attribute__((always_inline)) {
+            float pr[2];
 #pragma unroll
-            for (int s = 1; s < 8; ++s)
-                sacc = mfma32(*reinterpret_cast<const bf16x8*>(qt + aoff[s]),
-                              *reinterpret_cast<const bf16x8*>(smem + boff[s]), sacc);
-            [[maybe_unused]] bool q2s = false;
-            [[maybe_unused]] int nvalid = kBQ, pos0 = 0;
-            [[maybe_unused]] const int* qposs = reinterpret_cast<const int*>(meta) + 2 * kBQ;
-            [[maybe_unused]] int dense_head = 0, dense_q0 = 0;
-            if constexpr (kMasked) {
-                int r0, r_end, head;
-                item_rows(item, q2s, r0, r_end, head);
-                nvalid = r_end - r0;        // rows of the tile that exist
-                pos0 = (r0 - q1_lo) + off;  // depth-0 stream: position of tile row 0
-                dense_head = head;
-                dense_q0 = r0 - q1_lo;      // additive-mask mode: query index of tile row 0
-            }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const f32x4 lse4 = *reinterpret_cast<const f32x4*>(meta + mrow + 8 * j);  // four consecutive rows
-#pragma unroll
-                for (int b4 = 0; b4 < 4; ++b4) {
-                    const int r = 4 * j + b4;
-                    float pr = fast_exp2(sacc[r] * c - lse4[b4] * kLog2e);
-                    if constexpr (kMasked && !kDense) {
-                        const int qr = mrow + 8 * j + b4;
-                        const int qp = q2s ? qposs[qr] : pos0 + qr;
-                        pr = (qr < nvalid && kpos <= qp) ? pr : 0.f;
-                    }
-                    if constexpr (kDense) {  // mask[seq][head][query][my key]
-                        const int qr = mrow + 8 * j + b4;
-                        const bool ok = qr < nvalid && key_ok;
-                        const int64_t e = (int64_t)seq * p.mask_sb + (int64_t)dense_head * p.mask_sh +
-                                          (int64_t)(ok ? dense_q0 + qr : 0) * p.mask_sq;
-                        const float mv = mask_value(p, static_cast<const unsigned char*>(p.mask) + e * (p.mask_f32 ? 4 : 2),
-                                                    ok ? kl0 + 32 * kb + col : 0);
-                        const float lse_row = lse4[b4] == kNegInf ? -kNegInf : lse4[b4];  // all keys hidden: P = 0
-                        pr = ok ? fast_exp2((sacc[r] + mv * p.inv_scale) * c - lse_row * kLog2e) : 0.f;
-                    }
-                    pfr[r / 8][r % 8] = (__bf16)pr;
+            for (int u = 0; u < 2; ++u) {
+                const int rr = r + u, j = rr / 4, b4 = rr % 4;
+                const float lse = lse4[j % 2][b4];
+                pr[u] = fast_exp2(sacc[rr] * c - lse * kLog2e);
+                if constexpr (kMasked && !kDense) {
+                    const int qr = mrow_m + 8 * j + b4;
+                    const int qp = q2s ? qposs[qr] : pos0 + qr;
+                    pr[u] = (qr < nvalid && kpos_m <= qp) ? pr[u] : 0.f;
+                }
+                if constexpr (kDense) {  // mask[seq][head][query][my key]
+                    const int qr = mrow_m + 8 * j + b4;
+                    const bool ok = qr < nvalid && key_ok;
+                    const int64_t e = (int64_t)seq * p.mask_sb + (int64_t)dense_head * p.mask_sh +
+                                      (int64_t)(ok ? dense_q0 + qr : 0) * p.mask_sq;
+                    const float mv = mask_value(p, static_cast<const unsigned char*>(p.mask) + e * (p.mask_f32 ? 4 : 2),
+                                                ok ? kl0 + 32 * kb + col : 0);
+                    const float lse_row = lse == kNegInf ? -kNegInf : lse;  // all keys hidden: P = 0
+                    pr[u] = ok ? fast_exp2((sacc[rr] + mv * p.inv_scale) * c - lse_row * kLog2e) : 0.f;
                 }
             }
+            const f32x2 pr2 = {pr[0], pr[1]};
+            const bf16x2 pk = __builtin_convertvector(pr2, bf16x2);
+            pfr[r / 8][r % 8] = pk[0];
+            pfr[r / 8][r % 8 + 1] = pk[1];
+        };
+        // dS = P o (dP - delta) for rows r, r + 1, from the bf16 P that the dV product uses
+        auto ds_rows = [&](int r) __attribute__((always_inline)) {
+            const int j = r / 4, b4 = r % 4;
+            const f32x2 ds2 = {(float)pfr[r / 8][r % 8] * (dpacc[r] - del4[j % 2][b4]),
+                               (float)pfr[r / 8][r % 8 + 1] * (dpacc[r + 1] - del4[j % 2][b4 + 1])};
+            const bf16x2 pk = __builtin_convertvector(ds2, bf16x2);
+            dsfr[r / 8][r % 8] = pk[0];
+            dsfr[r / 8][r % 8 + 1] = pk[1];
+        };
+        auto load_lse = [&](int j) __attribute__((always_inline)) {
+            lse4[j % 2] = *reinterpret_cast<const f32x4*>(meta + mrow + 8 * j);
+        };
+        auto load_del = [&](int j) __attribute__((always_inline)) {
+            del4[j % 2] = *reinterpret_cast<const f32x4*>(meta + kBQ + mrow + 8 * j);
+        };
+
+        load_ab(0);
+        load_ab(1);
+#pragma unroll
+        for (int n = 0; n < 32; ++n) {
+            // reads for later slots
+            if (n + 2 < 16) load_ab(n + 2);
+            if (n + 3 >= 16 && n + 3 < 32) load_t(n + 3 - 16);
+            if (n >= 7 && n < 15 && (n - 7) % 2 == 0) load_lse((n - 7) / 2);   // rows 4j.. are used from slot 8 + 2j on
+            if (n >= 15 && n < 23 && (n - 15) % 2 == 0) load_del((n - 15) / 2);
+            __builtin_amdgcn_sched_barrier(0);
+            if (n < 8) {
+                sacc = mfma32(ra[n % 3], rb[n % 3], n == 0 ? zero : sacc);
+            } else if (n < 16) {
+                dpacc = mfma32(ra[n % 3], rb[n % 3], n == 8 ? zero : dpacc);
+                p_rows(2 * (n - 8));
+            } else if (n < 24) {
+                // dV (32 keys x 128 d) += P^T dO: needs P only, so the dS slices ride behind it
+                dvacc[n % 4] = mfma32(pfr[(n - 16) / 4], rt[n % 4], dvacc[n % 4]);
+                ds_rows(2 * (n - 16));
+            } else {
+                // dK += dS^T Q (contraction over my 32 queries)
+                dkacc[n % 4] = mfma32(dsfr[(n - 24) / 4], rt[n % 4], dkacc[n % 4]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
-        {
-            f32x16 dpacc = mfma32(*reinterpret_cast<const bf16x8*>(gt + aoff[0]),
-                                  *reinterpret_cast<const bf16x8*>(smem + (kKvV - kKvK) + boff[0]), zero);
-#pragma unroll
-            for (int s = 1; s < 8; ++s)
-                dpacc = mfma32(*reinterpret_cast<const bf16x8*>(gt + aoff[s]),
-                               *reinterpret_cast<const bf16x8*>(smem + (kKvV - kKvK) + boff[s]), dpacc);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const f32x4 del4 = *reinterpret_cast<const f32x4*>(meta + kBQ + mrow + 8 * j);
-#pragma unroll
-                for (int b4 = 0; b4 < 4; ++b4) {
-                    const int r = 4 * j + b4;
-                    dsfr[r / 8][r % 8] = (__bf16)((float)pfr[r / 8][r % 8] * (dpacc[r] - del4[b4]));
-                }
-            }
-        }
-        // dV (32 keys x 128 d) += P^T dO, then dK += dS^T Q (contraction over my 32 queries).  All of dV
-        // first: it needs P only, so the dS arithmetic can run in the shadow of its MFMAs.
-#pragma unroll
-        for (int st = 0; st < 2; ++st)
-#pragma unroll
-            for (int dt = 0; dt < 4; ++dt) {
-                const bf16x4 glo = lds_read_tr16(gt + toff_lo[dt] + st * 4096);
-                const bf16x4 ghi = lds_read_tr16(gt + toff_hi[dt] + st * 4096);
-                dvacc[dt] = mfma32(pfr[st], __builtin_shufflevector(glo, ghi, 0, 1, 2, 3, 4, 5, 6, 7), dvacc[dt]);
-            }
-#pragma unroll
-        for (int st = 0; st < 2; ++st)
-#pragma unroll
-            for (int dt = 0; dt < 4; ++dt) {
-                const bf16x4 qlo = lds_read_tr16(qt + toff_lo[dt] + st * 4096);
-                const bf16x4 qhi = lds_read_tr16(qt + toff_hi[dt] + st * 4096);
-                dkacc[dt] = mfma32(dsfr[st], __builtin_shufflevector(qlo, qhi, 0, 1, 2, 3, 4, 5, 6, 7), dkacc[dt]);
-            }
-#if TAH_DKDV_SCHED
-        if constexpr (!kMasked) {
-            // One straight-line block of 32 MFMAs: LDS reads run about four MFMAs ahead of their
-            // consumers; the P arithmetic sits between the dP MFMAs, the dS arithmetic between the dV ones.
-            __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-            }
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-#if TAH_DKDV_SCHED > 1
-                __builtin_amdgcn_sched_group_barrier(0x002, TAH_DKDV_SCHED, 0);
-#endif
-            }
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-            }
-        }
-#endif
     };
     using Masked = std::true_type;
     using Plain = std::false_type;
+    using Stage0 = std::integral_constant<int, 0>;
+    using Stage1 = std::integral_constant<int, 1>;
+    using StageAny = std::integral_constant<int, -1>;
 
     if (nitems > 0) issue_item(0, 0);  // (the first barrier below also publishes the K and V tiles)
-    int item = 0;
-    for (; item < t_vis * G; ++item) { advance(item); body(item, Masked{}); }
-    for (; item < t_whole * G; ++item) { advance(item); body(item, Plain{}); }
-    for (; item < nitems; ++item) { advance(item); body(item, Masked{}); }
+    // The three ranges start and end at multiples of G, so with an even G the stage of an item is
+    // its parity inside the pair and the LDS offsets of both stages are compile-time constants.
+    auto run = [&](int from, int to, auto mask_tag) __attribute__((always_inline)) {
+        if constexpr (G % 2 == 0) {
+            for (int item = from; item < to; item += 2) {
+                advance(item);
+                body(item, mask_tag, Stage0{});
+                advance(item + 1);
+                body(item + 1, mask_tag, Stage1{});
+            }
+        } else {
+            for (int item = from; item < to; ++item) {
+                advance(item);
+                body(item, mask_tag, StageAny{});
+            }
+        }
+    };
+    run(0, t_vis * G, Masked{});
+    run(t_vis * G, t_whole * G, Plain{});
+    run(t_whole * G, nitems, Masked{});
 
     // ---- add the two query halves and store ---------------------------------
     TAH_WAIT_VMEM();  // no copy may still be on its way into the memory the reduction reuses

@@ -140,6 +140,11 @@ __device__ __forceinline__ void async_copy_4B(const void* sbase, uint32_t voff, 
 #ifndef TAH_KEEP_HERE4
 #define TAH_KEEP_HERE4(a, b, c, d) asm volatile("" ::"v"(a), "v"(b), "v"(c), "v"(d))
 #endif
+// Makes two register values opaque to the optimiser at this point, so that what is derived from them
+// afterwards is computed here (and not hoisted out of a loop into registers of its own).
+#ifndef TAH_OPAQUE2
+#define TAH_OPAQUE2(a, b) asm volatile("" : "+v"(a), "+v"(b))
+#endif
 // Occupancy the kernel is written for; lets the scheduler spend registers on latency hiding.
 // Between LDS writes of a wave and reads, by the same wave, of what its other lanes wrote: the lanes run
 // in lockstep and the LDS serves a wave's requests in order, so all that is needed is that the compiler
