@@ -696,7 +696,7 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
 // ---------------------------------------------------------------------------
 constexpr int kKv4Threads = 256;
 constexpr int kKv4Meta = 2 * kKvSlot;                     // after the two stages: per stage lse, delta, query positions
-constexpr int kKv4Smem = kKv4Meta + 2 * kKvMetaBytes;
+[[maybe_unused]] constexpr int kKv4Smem = kKv4Meta + 2 * kKvMetaBytes;
 
 template <int G, bool kDense>
 __global__ __launch_bounds__(kKv4Threads) TAH_WAVES_PER_EU(1, 1) void duo_bwd_dkdv4_kernel(const BwdParams p) {
