@@ -37,3 +37,27 @@ def test_fused_layer_prefill_then_decode_on_cpu_shim():
 def test_fused_layer_prefill_then_decode_gpu():
     for ref, got in run_prefill_then_decode("cuda", B=3, T=200, steps=3):
         _check(got, ref)
+
+
+def _check_model(outs):
+    (ref0, ref1), (got0, got1) = outs
+    for got, want in ((got0, ref0), (got1, ref1)):
+        err = (got - want).abs().max().item()
+        ref = want.abs().max().item()
+        assert err <= 3e-2 * max(ref, 1.0), (err, ref)
+
+
+@pytest.mark.skipif(not emu_util.have_host_clang(), reason="host clang++ not available")
+def test_patched_model_two_depths_on_cpu_shim():
+    from tests.hf_model_case import run as run_model
+
+    with emu_util.emulated():
+        outs = run_model("cpu", B=2, T=12, layers=2)
+    _check_model(outs)
+
+
+@pytest.mark.gpu
+def test_patched_model_two_depths_gpu():
+    from tests.hf_model_case import run as run_model
+
+    _check_model(run_model("cuda", B=3, T=150, layers=2))
