@@ -183,11 +183,13 @@ class TaHDuoCache:
         return cache_position.shape[0] + self.get_cache_length(layer_idx), 0
 
     def reorder_cache(self, beam_idx: torch.LongTensor) -> None:
-        if self._slabs:
-            raise TahDuoError("reorder_cache is not supported once slabs are enabled")
+        """Batch row i continues from row beam_idx[i] (causal_cache.py:201-205: K and V only, the staged positions
+        and valid flags of the chunks stay as they are).  Slabs move their rows, positions and lengths together."""
         for store in (self._k, self._v):
             for slot, ts in store.items():
                 store[slot] = [t.index_select(0, beam_idx.to(t.device)) for t in ts]
+        for sl in self._slabs.values():
+            sl.reorder(beam_idx)
 
     # ── device / dtype (causal_cache.py:209-239) ──────────────────────────
     @property

@@ -41,6 +41,16 @@ class KvSlabs:
         s.capacity, s.nslots = self.capacity, self.nslots
         return s
 
+    def reorder(self, index: torch.Tensor) -> None:
+        """Slot i takes the rows, positions and length of slot index[i] (beam search: several beams may continue
+        the same sequence).  In place, through one temporary copy per tensor, so the slab addresses stay valid."""
+        idx = index.to(device=self.k.device, dtype=torch.int64)
+        if idx.numel() != self.nslots:
+            raise _capi.TahDuoError(f"KvSlabs.reorder: {idx.numel()} indices for {self.nslots} slots")
+        for t in (self.k, self.v, self.pos, self.len):
+            if t is not None:
+                t.copy_(t.index_select(0, idx))
+
     def append(self, k_new: torch.Tensor, v_new: torch.Tensor, cu_new: torch.Tensor,
                pos_new: Optional[torch.Tensor] = None, slot_of: Optional[torch.Tensor] = None) -> None:
         """Append rows [cu_new[i], cu_new[i+1]) of k_new/v_new ([rows, Hkv, D]) to slot slot_of[i] (default i)."""

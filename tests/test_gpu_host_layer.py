@@ -71,3 +71,10 @@ def test_gather_scatter_large_gpu():
     dest = torch.zeros_like(x)
     out = scatter_back(mask, gx, dest)
     assert torch.equal(out[mask], x[mask]) and (out[~mask] == 0).all()
+
+
+def test_reorder_cache_with_slabs_gpu():
+    from tests.reorder_case import run
+    plain, moved, beam = run("cuda", beam=(3, 0, 0, 2), T0=70)
+    for a, b in zip(plain, moved):
+        assert torch.equal(a[beam], b)

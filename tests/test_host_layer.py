@@ -275,3 +275,26 @@ def test_decode_steps_through_cache_and_callable(emu):
     s1 = cache.slabs(0, 0)
     assert s1.len.tolist() == valid_all.sum(1).tolist() and int(s1.overflow) == 0
     assert cache.slabs(0, 1).len.tolist() == (c["hard"] & valid_all.bool()).sum(1).tolist()
+
+
+def test_reorder_cache_with_slabs(emu):
+    """Beam-search reorder moves slab rows, positions and lengths together (causal_cache.py:201-205 for K/V)."""
+    from tests.reorder_case import run
+    plain, moved, beam = run("cpu")
+    for a, b in zip(plain, moved):
+        assert torch.equal(a[beam], b)
+
+
+def test_reorder_cache_chunks_only():
+    """Without slabs: K and V chunks are index-selected along the batch axis, nothing else changes."""
+    from tah_amd.cache import TaHDuoCache
+    c = TaHDuoCache()
+    pos = torch.arange(5)[None].expand(3, 5)
+    c.current_iter_depth, c.position_ids_to_cache, c.valid_mask_to_cache = 0, pos, torch.ones(3, 5, dtype=torch.long)
+    k, v = torch.randn(3, 2, 5, 8), torch.randn(3, 2, 5, 8)
+    c.update(k, v, 0)
+    beam = torch.tensor([1, 1, 0])
+    c.reorder_cache(beam)
+    K, V = c.get_cache_upto_iter(0, 0)
+    assert torch.equal(K, k[beam]) and torch.equal(V, v[beam])
+    assert torch.equal(c.get_position_id_upto_iter(0, 0), pos)
