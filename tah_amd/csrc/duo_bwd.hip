@@ -485,7 +485,6 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
         TAH_WAIT_VMEM();
         __syncthreads();
         if (item + 1 == nt1 * G) src = stream_src(true);  // the next item is the first of the depth-1 stream
-        if (item + 1 < nitems) issue_item(item + 1, (item & 1) ^ 1);
     };
 
     // per-lane LDS read offsets inside a tile, computed once
@@ -611,6 +610,13 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
             if (n >= 7 && n < 15 && (n - 7) % 2 == 0) load_lse((n - 7) / 2);   // rows 4j.. are used from slot 8 + 2j on
             if (n >= 15 && n < 23 && (n - 15) % 2 == 0) load_del((n - 15) / 2);
             __builtin_amdgcn_sched_barrier(0);
+            // The copies of the next item (its stage is free since the barrier): a copy instruction holds
+            // a wave's issue for about 80 clocks, so the two waves of a SIMD send theirs half an item apart
+            // and each does it while the other has MFMAs to issue.
+            if ((n == 2 && qh == 0) || (n == 18 && qh == 1)) {
+                if (item + 1 < nitems) issue_item(item + 1, stage ^ 1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
             if (n < 8) {
                 sacc = mfma32(ra[n % 3], rb[n % 3], n == 0 ? zero : sacc);
             } else if (n < 16) {
