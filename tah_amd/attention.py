@@ -130,10 +130,46 @@ def build_attention_mask(active_position_ids, active_valid_mask, cache, iter_dep
     """Drop-in for ``TaHForCausalLM._build_attention_mask`` (tah_model.py:744-751): same arguments;
     returns a :class:`DuoMask` (or ``None`` when there is nothing to attend to, as tah_model.py:773-775)."""
     del dtype
+    _check_depth(iter_depth)
     n_cached = cache.get_kv_length_upto_iter(0, iter_depth) if cache is not None and cache.has_layer(0) else 0
     if n_cached + active_position_ids.shape[1] == 0:
         return None
     return DuoMask(active_position_ids, active_valid_mask, cache, iter_depth)
+
+
+def _check_depth(iter_depth: int) -> None:
+    """The kernels know two latent iterations; the reference's mask handles any depth (tah_model.py:788) and
+    its deciders accept ``max_iter`` 3, so a deeper call must fail here and not be computed as depth 1."""
+    if not 0 <= int(iter_depth) <= 1:
+        raise TahDuoError(f"iter_depth = {iter_depth}: duo-causal attention is implemented for depths 0 and 1 "
+                          "(max_iter = 2, as in every shipped recipe)")
+
+
+# Debug switch: verify on the device (one host sync per model step) that the positions handed in are the
+# valid tokens' ranks inside their sequence -- what the kernels assume for depth 0 (index-causal order) and
+# for the depth-0 keys that depth-1 queries see.  The model's forward computes exactly these when
+# ``position_ids`` is None (tah_model.py:555-561); a caller that passes its own position_ids can turn this on.
+CHECK_POSITIONS = False
+
+
+def _assert_rank_positions(m: "DuoMask") -> None:
+    c, B = m.cache, m.position_ids.shape[0]
+    prev = 0
+    if c is not None and c.has_layer(0):
+        # valid depth-0 tokens already cached (the step's own rows are written by update() before attention runs)
+        cached = c.get_valid_mask_upto_iter(0, 0, B)
+        own = m.valid_mask.shape[1] if m.iter_depth == 0 and cached.shape[1] >= m.valid_mask.shape[1] else 0
+        prev = cached[:, : cached.shape[1] - own].sum(-1, keepdim=True) if cached.shape[1] - own > 0 else 0
+    v = m.valid_mask != 0
+    if m.iter_depth == 0:
+        want = torch.cumsum(v.long(), -1) - 1 + prev
+        bad = ((m.position_ids != want) & v).any()
+    else:  # depth-1 rows name tokens that exist at depth 0: positions below the number of valid depth-0 tokens
+        total0 = c.get_valid_mask_upto_iter(0, 0, B).sum(-1, keepdim=True)
+        bad = (((m.position_ids < 0) | (m.position_ids >= total0)) & v).any()
+    if bool(bad):
+        raise TahDuoError("position_ids are not the valid tokens' ranks inside their sequence; the kernels take the "
+                          "depth-0 position of a token from its index among the valid tokens")
 
 
 # ---------------------------------------------------------------------------
@@ -229,7 +265,15 @@ def _segment(cache: TaHDuoCache, layer_idx: int, depth: int, B: int, with_pos: b
     dev = chunks[0][0].device
     if len(chunks) == 1:
         k, v, pos, valid = chunks[0]
-        pk = _Packed(valid, pos if with_pos else None, B, k.shape[2], dev)
+        # every decoder layer caches the same (valid, pos) tensors of the step: build the index once
+        key = (id(valid), id(pos) if with_pos else None, k.shape[2])
+        memo = cache._key_memo.get(key)
+        if memo is None or memo[0] is not valid or (with_pos and memo[1] is not pos):
+            memo = (valid, pos, _Packed(valid, pos if with_pos else None, B, k.shape[2], dev))
+            if len(cache._key_memo) > 8:
+                cache._key_memo.clear()
+            cache._key_memo[key] = memo
+        pk = memo[2]
         return pk.pack(k), pk.pack(v), pk.cu, pk.pos
     k = torch.cat([c[0] for c in chunks], dim=2)
     v = torch.cat([c[1] for c in chunks], dim=2)
@@ -272,6 +316,9 @@ def duo_attention_forward(module, query: torch.Tensor, key: torch.Tensor, value:
         raise TahDuoError("attention dropout is not supported (the reference runs with 0.0)")
     m = attention_mask
     cache, depth = m.cache, m.iter_depth
+    _check_depth(depth)
+    if CHECK_POSITIONS and m._packed is None:
+        _assert_rank_positions(m)
     if cache is None:
         raise TahDuoError("the DuoMask carries no cache; pass the cache that update() was called on")
     layer = int(getattr(module, "layer_idx", 0))

@@ -12,7 +12,9 @@ unchanged.  What differs is storage and what ``update`` hands back:
   layer per decode step, causal_cache.py:84-90);
 * with ``enable_slabs`` the valid rows of every write are also appended, in
   place, to preallocated per-sequence slabs (tah_amd.kv_cache.KvSlabs) that the
-  decode kernel streams;
+  decode kernel streams; from the first single-token write on, the slabs are the
+  only copy of K and V (the chunk lists keep positions, valid flags and lengths),
+  so a long generation holds one copy of its cache and no list of tiny tensors;
 * ``update`` returns the new (key, value) tensors themselves: the duo attention
   callable (tah_amd.attention.duo_attention_forward) reads the visible segments
   from the cache, so the depth-0 | depth-1 concatenation of
@@ -42,12 +44,16 @@ class TaHDuoCache:
         self.valid_mask_to_cache: Optional[torch.Tensor] = None
         self.batch_size: Optional[int] = None
         self.return_concat = return_concat
+        self._rows: Dict[_Slot, int] = {}       # rows written per slot (pad rows included), the reference's length
+        self._kv_dropped: Dict[_Slot, bool] = {}  # K/V of the slot live in the slabs only
         self._device: Optional[torch.device] = None
         self._dtype: Optional[torch.dtype] = None
         # native decode storage
         self._slab_cfg: Optional[Tuple[int, int]] = None
         self._slabs: Dict[_Slot, KvSlabs] = {}
+        self._slab_rows: Dict[_Slot, int] = {}  # host-side upper bound on the rows any slab of the slot holds
         self._pack_memo: Dict[int, Any] = {}
+        self._key_memo: Dict[Any, Any] = {}     # packed key segments of single-chunk slots, per (layer-independent) valid mask
 
     # ── native storage ────────────────────────────────────────────────────
     def enable_slabs(self, capacity_depth0: int, capacity_depth1: int) -> "TaHDuoCache":
@@ -67,6 +73,15 @@ class TaHDuoCache:
         if sl is None:
             sl = KvSlabs(B, self._slab_cfg[slot[1]], hkv, d, with_pos=slot[1] > 0, device=k.device, dtype=k.dtype)
             self._slabs[slot] = sl
+        # A slab that is full drops rows on the device (and raises a flag nobody waits for): refuse on the
+        # host instead.  Every write adds at most T rows to a sequence (T counts pad rows too, so the bound
+        # is conservative); it needs no device read.
+        written = self._slab_rows.get(slot, 0) + T
+        if written > sl.capacity:
+            raise TahDuoError(
+                f"KV slabs of layer {slot[0]}, depth {slot[1]} hold {sl.capacity} rows per sequence; this write "
+                f"brings a sequence to as many as {written}: enable_slabs() with a larger capacity")
+        self._slab_rows[slot] = written
         # one compaction of the valid mask per forward step, shared by all layers
         key = id(valid) if valid is not None else -T
         memo = self._pack_memo.get(key)
@@ -101,7 +116,7 @@ class TaHDuoCache:
 
     # ── write path (causal_cache.py:63-97) ────────────────────────────────
     def has_layer(self, layer_idx: int = 0) -> bool:
-        return any(l == layer_idx for (l, _) in self._k)
+        return any(l == layer_idx for (l, _) in self._rows)
 
     def update(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int,
                cache_kwargs: Optional[Dict[str, Any]] = None):
@@ -112,25 +127,50 @@ class TaHDuoCache:
             assert key_states.shape[0] == self.batch_size, (
                 f"batch size mismatch: cached {self.batch_size}, got {key_states.shape[0]}")
         self._device, self._dtype = key_states.device, key_states.dtype
+        if not 0 <= int(self.current_iter_depth) <= 1:
+            raise TahDuoError(f"current_iter_depth = {self.current_iter_depth}: the kernels implement two latent "
+                              "iterations (depth 0 and depth 1), as every shipped recipe uses (max_iter = 2)")
         slot = (layer_idx, self.current_iter_depth)
-        self._k.setdefault(slot, []).append(key_states)
-        self._v.setdefault(slot, []).append(value_states)
+        to_slabs = self._slab_cfg is not None and not (torch.is_grad_enabled() and key_states.requires_grad)
+        if to_slabs:
+            self._append_slabs(slot, key_states, value_states, self.position_ids_to_cache, self.valid_mask_to_cache)
+        self._rows[slot] = self._rows.get(slot, 0) + key_states.shape[-2]
+        # Single-token writes that went to the slabs are not kept a second time, and what the slot kept
+        # before (the prompt's chunk) is released: the decode kernel reads the slabs.
+        if to_slabs and key_states.shape[-2] == 1 and not self.return_concat and self._slabs_cover(slot):
+            self._kv_dropped[slot] = True
+            self._k.pop(slot, None)
+            self._v.pop(slot, None)
+        else:
+            if self._kv_dropped.get(slot):
+                raise TahDuoError("this cache slot keeps K/V in its slabs only (single-token decode steps were written); "
+                                  "a multi-token or differentiable write can no longer be mixed in")
+            self._k.setdefault(slot, []).append(key_states)
+            self._v.setdefault(slot, []).append(value_states)
         self._pos.setdefault(slot, []).append(self.position_ids_to_cache)
         self._valid.setdefault(slot, []).append(self.valid_mask_to_cache)
-        if self._slab_cfg is not None and not (torch.is_grad_enabled() and key_states.requires_grad):
-            self._append_slabs(slot, key_states, value_states, self.position_ids_to_cache, self.valid_mask_to_cache)
         if self.return_concat:
             return self.get_cache_upto_iter(layer_idx, self.current_iter_depth)
         return key_states, value_states
+
+    def _slabs_cover(self, slot: _Slot) -> bool:
+        """True when every row ever written to the slot also went to its slabs."""
+        return slot in self._slabs and self._slab_rows.get(slot, 0) == self._rows.get(slot, 0)
 
     # ── chunk access for the attention callable ───────────────────────────
     def chunks(self, layer_idx: int, depth: int):
         """[(k, v, pos, valid), ...] written at (layer, depth), in write order."""
         s = (layer_idx, depth)
+        if self._kv_dropped.get(s):
+            raise TahDuoError(f"K/V of layer {layer_idx}, depth {depth} live in the slabs only; the packed-varlen path "
+                              "(multi-token queries, backward) needs a cache that kept its chunks")
         return list(zip(self._k.get(s, []), self._v.get(s, []), self._pos.get(s, []), self._valid.get(s, [])))
 
     # ── read views (causal_cache.py:101-158) ──────────────────────────────
     def get_cache_upto_iter(self, layer_idx: int, upto_iter_idx: int):
+        if any(self._kv_dropped.get((layer_idx, d)) for d in range(upto_iter_idx + 1)):
+            raise TahDuoError("get_cache_upto_iter: K/V of this layer live in the slabs only (decode steps were "
+                              "written with enable_slabs); construct the cache with return_concat=True to keep them")
         ks = [t for d in range(upto_iter_idx + 1) for t in self._k.get((layer_idx, d), [])]
         if not ks:
             return None, None
@@ -138,7 +178,12 @@ class TaHDuoCache:
         return (ks[0], vs[0]) if len(ks) == 1 else (torch.cat(ks, dim=-2), torch.cat(vs, dim=-2))
 
     def _meta_upto_iter(self, store, layer_idx: int, upto_iter_idx: int, init_batch_size: int) -> torch.Tensor:
-        parts = [t for d in range(upto_iter_idx + 1) for t in store.get((layer_idx, d), [])]
+        parts = []
+        for d in range(upto_iter_idx + 1):
+            ts = store.get((layer_idx, d), [])
+            if len(ts) > 1 and all(t is not None for t in ts):
+                ts[:] = [torch.cat(ts, dim=-1)]  # fold the per-step pieces once, so a long generation stays cheap
+            parts += ts
         if not parts:
             return torch.empty((init_batch_size, 0), device=self.device, dtype=torch.long)
         return parts[0] if len(parts) == 1 else torch.cat(parts, dim=-1)
@@ -157,11 +202,7 @@ class TaHDuoCache:
 
     # ── lengths & misc protocol (causal_cache.py:162-205) ─────────────────
     def get_cache_length(self, layer_idx: Optional[int] = 0, iter_idx: Optional[int] = None) -> int:
-        tot = 0
-        for (l, d), ts in self._k.items():
-            if l == layer_idx and (iter_idx is None or d == iter_idx):
-                tot += sum(t.shape[-2] for t in ts)
-        return tot
+        return sum(n for (l, d), n in self._rows.items() if l == layer_idx and (iter_idx is None or d == iter_idx))
 
     def get_kv_length_upto_iter(self, layer_idx: int = 0, upto_iter_idx: int = 0) -> int:
         return sum(self.get_cache_length(layer_idx, d) for d in range(upto_iter_idx + 1))
@@ -225,4 +266,4 @@ class TaHDuoCache:
         return self
 
     def __len__(self) -> int:
-        return len({l for (l, _) in self._k})
+        return len({l for (l, _) in self._rows})

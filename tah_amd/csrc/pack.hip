@@ -22,6 +22,9 @@ __global__ __launch_bounds__(kScanThreads) void hard_index_kernel(const uint8_t*
     const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
     const int64_t total = (int64_t)B * S;
     if (tid == 0) carry_s = 0;
+    // a mask without columns has no element (b, 0) to carry a row's boundary: every boundary is 0
+    if (S == 0)
+        for (int b = tid; b < B; b += kScanThreads) cu_out[b] = 0;
     __syncthreads();
     for (int64_t chunk = 0; chunk < total; chunk += (int64_t)kScanThreads * kPerThread) {
         const int64_t f0 = chunk + (int64_t)tid * kPerThread;

@@ -67,3 +67,32 @@ def test_bwd_full_size_training_config_vs_torch_fp32():
     ((r1 * do1.float()).sum() + (r2 * do2.float()).sum()).backward()
     want = [leaf[n].grad.cpu().numpy() for n in ("q1", "k1", "v1", "q2", "k2", "v2")]
     print("full-size fwd+bwd:", check_grads(got, want), flush=True)
+
+
+def test_fwd_bwd_headline_seq8192_vs_torch_fp32():
+    """The headline shape (one sequence of 8192 tokens, 6 % hard, Hq=16, Hkv=8, D=128): outputs of both depths and
+    all six gradients against torch fp32 autograd through the dense-mask formulation on the device."""
+    from tah_amd import ops
+    from tests.gpu_util import assert_close
+    dev = to_device(make_varlen_case(1238, [8192], 0.06, std=0.5))
+    gen = torch.Generator().manual_seed(6)
+    do1 = torch.randn(dev["q1"].shape, generator=gen).to(torch.bfloat16).cuda()
+    do2 = torch.randn(dev["q2"].shape, generator=gen).to(torch.bfloat16).cuda()
+    o1, lse1, o2, lse2 = ops.duo_fwd_varlen(*varlen_args(dev))
+    got = ops.duo_bwd_varlen(dev["q1"], dev["k1"], dev["v1"], o1, lse1, do1, dev["cu_q1"], dev["cu_k1"],
+                             dev["q2"], dev["k2"], dev["v2"], o2, lse2, do2, dev["pos_q2"], dev["pos_k2"],
+                             dev["cu_q2"], dev["cu_k2"], dev["scale"])
+    torch.cuda.synchronize()
+    leaf = {k: (v.float().requires_grad_(True) if torch.is_tensor(v) and v.is_floating_point() else
+                (v.cpu().numpy() if torch.is_tensor(v) else v)) for k, v in dev.items()}
+    torch_default = torch.get_default_device()
+    torch.set_default_device("cuda")
+    try:
+        r1, r2 = O.duo_varlen_torch(*varlen_args(leaf))
+    finally:
+        torch.set_default_device(torch_default)
+    print("headline fwd: o1", assert_close(o1, r1.detach().cpu().numpy(), "headline o1"),
+          "o2", assert_close(o2, r2.detach().cpu().numpy(), "headline o2"), flush=True)
+    ((r1 * do1.float()).sum() + (r2 * do2.float()).sum()).backward()
+    want = [leaf[n].grad.cpu().numpy() for n in ("q1", "k1", "v1", "q2", "k2", "v2")]
+    print("headline fwd+bwd:", check_grads(got, want), flush=True)

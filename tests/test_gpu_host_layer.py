@@ -78,3 +78,28 @@ def test_reorder_cache_with_slabs_gpu():
     plain, moved, beam = run("cuda", beam=(3, 0, 0, 2), T0=70)
     for a, b in zip(plain, moved):
         assert torch.equal(a[beam], b)
+
+
+def test_decode_steps_both_depths_through_cache_and_callable_gpu():
+    """Prefill + decode steps at depth 0 and depth 1 (hard subset, pad rows, left padding, slabs on) through
+    TaHDuoCache + duo_attention_forward on the device, against the concatenating oracle cache + dense SDPA
+    (tah_model.py:116-118 pad rows, causal_cache.py:84-97 depth-1 appends for all B rows)."""
+    from tests.decode_steps_case import run
+    cache, n1 = run("cuda", T0=150, steps=5, B=3, left_pad=(0, 37, 9), seed=61, Hq=16, Hkv=8,
+                    force_hard=[[0], [], [0, 1, 2], [2], [1]])
+    assert n1 == 4
+    from tah_amd import TahDuoError
+    with pytest.raises(TahDuoError):
+        cache.get_cache_upto_iter(0, 0)
+
+
+def test_slab_overflow_raises_gpu():
+    from tah_amd import TahDuoError
+    from tah_amd.cache import TaHDuoCache
+    cache = TaHDuoCache().enable_slabs(4, 4)
+    k = torch.zeros(2, 8, 3, 128, dtype=torch.bfloat16, device="cuda")
+    pos, one = torch.arange(3, device="cuda")[None].expand(2, 3), torch.ones(2, 3, dtype=torch.long, device="cuda")
+    cache.current_iter_depth, cache.position_ids_to_cache, cache.valid_mask_to_cache = 0, pos, one
+    cache.update(k, k, 0)
+    with pytest.raises(TahDuoError, match="capacity"):
+        cache.update(k, k, 0)

@@ -221,60 +221,92 @@ def test_forward_loop_gradients(emu):
 
 
 def test_decode_steps_through_cache_and_callable(emu):
-    """Prefill then two decode steps with slabs; compare with the dense reference over the grown cache."""
+    """Prefill then decode steps at both depths with slabs; compare with the dense reference over the grown cache."""
+    from tests.decode_steps_case import run
+    cache, n1 = run("cpu", steps=4, force_hard=[[0], [], [0, 1], [1]])
+    assert n1 == 3  # three of the four decode steps had a depth-1 pass (one with a pad row, one with both rows hard)
+    # decode steps leave K/V in the slabs only: the concatenating getter says so instead of returning a partial cache
+    from tah_amd import TahDuoError
+    with pytest.raises(TahDuoError):
+        cache.get_cache_upto_iter(0, 0)
+
+
+def test_slab_overflow_raises_through_cache_update(emu):
+    """A generation that outgrows the slab capacity fails on the host at the write, not silently on the device."""
+    from tah_amd import TahDuoError
     from tah_amd.attention import build_attention_mask, duo_attention_forward
     from tah_amd.cache import TaHDuoCache
-    from tah_amd.pack import gather_active
-    T0, steps = 20, 2
-    c = make_dense_case(34, B=2, T=T0 + steps, p_hard=0.3, Hq=2, Hkv=1, D=128, left_pad=[0, 5])
+    c = make_dense_case(35, B=1, T=9, p_hard=0.0, Hq=2, Hkv=1, D=128)
     bf = lambda x: x.to(torch.bfloat16)
-    cache = TaHDuoCache().enable_slabs(64, 32)
-    ocache = O.OracleCache()
-    valid_all = c["valid"]
-    pos_all = (torch.cumsum(valid_all, -1) - 1).clamp(min=0)
-    tok = lambda x: x.transpose(1, 2)
+    cache = TaHDuoCache().enable_slabs(6, 4)
+    pos_all = torch.arange(9)[None]
+    one = torch.ones(1, 9, dtype=torch.long)
 
-    def step(lo, hi):
-        """Feed tokens [lo, hi) at depth 0, then their hard subset at depth 1, to both implementations."""
+    def feed(lo, hi):
         sl = slice(lo, hi)
-        pos, valid, hard = pos_all[:, sl], valid_all[:, sl], c["hard"][:, sl]
-        q1, k1, v1 = (bf(c[n][:, :, sl]) for n in ("q1", "k1", "v1"))
-        outs = []
-        for ch, fwd in ((cache, None), (ocache, "ref")):
-            mk = build_attention_mask if fwd is None else O.build_attention_mask
-            m0 = mk(pos, valid, ch, 0, torch.float32)
-            ch.current_iter_depth, ch.position_ids_to_cache, ch.valid_mask_to_cache = 0, pos, valid
-            if fwd is None:
-                k, v = ch.update(k1, v1, 0)
-                o1, _ = duo_attention_forward(_layer(), q1, k, v, m0, scaling=c["scale"])
-                pad, q2, k2, v2, pos2, val2 = gather_active(hard, *(tok(bf(c[n][:, :, sl])) for n in ("q2", "k2", "v2")), pos, valid)
-            else:
-                K, V = ch.update(k1.float(), v1.float(), 0)
-                o1 = O.sdpa_dense(q1.float(), K, V, m0, c["scale"])
-                pad, q2, k2, v2, pos2, val2 = O.gather_active(hard, *(tok(bf(c[n][:, :, sl]).float()) for n in ("q2", "k2", "v2")), pos, valid)
-            o2 = None
-            if pad.shape[1]:
-                m1 = mk(pos2, val2, ch, 1, torch.float32)
-                ch.current_iter_depth, ch.position_ids_to_cache, ch.valid_mask_to_cache = 1, pos2, val2
-                if fwd is None:
-                    k, v = ch.update(tok(k2), tok(v2), 0)
-                    o2, _ = duo_attention_forward(_layer(), tok(q2), k, v, m1, scaling=c["scale"])
-                else:
-                    K, V = ch.update(tok(k2), tok(v2), 0)
-                    o2 = O.sdpa_dense(tok(q2), K, V, m1, c["scale"])
-            outs.append((o1, o2, pad, valid.bool()))
-        (a1, a2, pad, vb), (b1, b2, _, _) = outs
-        np.testing.assert_allclose(a1[vb].float().numpy(), b1[vb].numpy(), atol=2e-2, rtol=2e-2)
-        if a2 is not None:
-            np.testing.assert_allclose(a2[~pad].float().numpy(), b2[~pad].numpy(), atol=2e-2, rtol=2e-2)
+        m = build_attention_mask(pos_all[:, sl], one[:, sl], cache, 0)
+        cache.current_iter_depth, cache.position_ids_to_cache, cache.valid_mask_to_cache = 0, pos_all[:, sl], one[:, sl]
+        k, v = cache.update(bf(c["k1"][:, :, sl]), bf(c["v1"][:, :, sl]), 0)
+        return duo_attention_forward(_layer(), bf(c["q1"][:, :, sl]), k, v, m, scaling=c["scale"])[0]
 
     with torch.no_grad():
-        step(0, T0)
-        for s in range(steps):
-            step(T0 + s, T0 + s + 1)
-    s1 = cache.slabs(0, 0)
-    assert s1.len.tolist() == valid_all.sum(1).tolist() and int(s1.overflow) == 0
-    assert cache.slabs(0, 1).len.tolist() == (c["hard"] & valid_all.bool()).sum(1).tolist()
+        feed(0, 5)
+        feed(5, 6)
+        with pytest.raises(TahDuoError, match="capacity"):
+            feed(6, 7)
+    assert int(cache.slabs(0, 0).overflow) == 0 and cache.slabs(0, 0).len.tolist() == [6]
+
+
+def test_depth_two_is_refused(emu):
+    """The reference's mask and cache take any depth (tah_model.py:788); this build has two and says so."""
+    from tah_amd import TahDuoError
+    from tah_amd.attention import DuoMask, build_attention_mask, duo_attention_forward
+    from tah_amd.cache import TaHDuoCache
+    cache = TaHDuoCache()
+    pos, one = torch.arange(4)[None], torch.ones(1, 4, dtype=torch.long)
+    with pytest.raises(TahDuoError, match="depth"):
+        build_attention_mask(pos, one, cache, 2)
+    k = torch.zeros(1, 1, 4, 128, dtype=torch.bfloat16)
+    cache.current_iter_depth, cache.position_ids_to_cache, cache.valid_mask_to_cache = 2, pos, one
+    with pytest.raises(TahDuoError, match="depth"):
+        cache.update(k, k, 0)
+    cache.current_iter_depth = 0
+    cache.update(k, k, 0)
+    with pytest.raises(TahDuoError, match="depth"):
+        duo_attention_forward(_layer(), torch.zeros(1, 2, 4, 128, dtype=torch.bfloat16), k, k, DuoMask(pos, one, cache, 2))
+
+
+def test_position_check_switch(emu):
+    """CHECK_POSITIONS: positions that are not the valid tokens' ranks are refused (the kernels would use the ranks)."""
+    from tah_amd import TahDuoError, attention
+    from tah_amd.cache import TaHDuoCache
+    c = make_dense_case(36, B=2, T=8, p_hard=0.0, Hq=2, Hkv=1, D=128, left_pad=[0, 3])
+    bf = lambda x: x.to(torch.bfloat16)
+    pos = (torch.cumsum(c["valid"], -1) - 1).clamp(min=0)
+    attention.CHECK_POSITIONS = True
+    try:
+        for shift, ok in ((0, True), (10, False)):
+            cache = TaHDuoCache()
+            p = pos + shift
+            m = attention.build_attention_mask(p, c["valid"], cache, 0)
+            cache.current_iter_depth, cache.position_ids_to_cache, cache.valid_mask_to_cache = 0, p, c["valid"]
+            k, v = cache.update(bf(c["k1"]), bf(c["v1"]), 0)
+            if ok:
+                attention.duo_attention_forward(_layer(), bf(c["q1"]), k, v, m, scaling=c["scale"])
+            else:
+                with pytest.raises(TahDuoError, match="position"):
+                    attention.duo_attention_forward(_layer(), bf(c["q1"]), k, v, m, scaling=c["scale"])
+    finally:
+        attention.CHECK_POSITIONS = False
+
+
+def test_hard_index_of_mask_without_columns(emu):
+    """S == 0: every boundary is zero (nothing read from uninitialised memory)."""
+    from tah_amd.pack import HardIndex, gather_active
+    idx = HardIndex(torch.zeros(3, 0, dtype=torch.bool))
+    assert idx.cu.tolist() == [0, 0, 0, 0] and idx.n == 0 and idx.width == 0
+    pad, x = gather_active(torch.zeros(3, 0, dtype=torch.bool), torch.zeros(3, 0, 4))
+    assert pad.shape == (3, 0) and x.shape == (3, 0, 4)
 
 
 def test_reorder_cache_with_slabs(emu):
