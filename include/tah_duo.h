@@ -39,7 +39,8 @@ enum {
     TAH_E_SHAPE = -2,     /* unsupported head_dim / head counts / negative sizes */
     TAH_E_ALIGN = -3,     /* pointer or stride not 16-byte aligned */
     TAH_E_LAUNCH = -4,    /* the HIP runtime rejected the launch */
-    TAH_E_WORKSPACE = -5  /* workspace too small */
+    TAH_E_WORKSPACE = -5, /* workspace too small */
+    TAH_E_SCRATCH = -6    /* tah_duo_decode_static: the call needs more than TAH_DUO_STATIC_SCRATCH_BYTES */
 };
 
 typedef void* tah_stream_t; /* hipStream_t */
@@ -186,6 +187,20 @@ size_t tah_duo_decode_workspace_bytes(int32_t nq, int32_t hq, int32_t capacity1,
  *   sdpa_attention_forward                       transformers/integrations/sdpa_attention.py:79-166
  * Queries with no visible row get o = 0, lse = -inf. */
 int tah_duo_decode(const tah_duo_decode_args* args, tah_stream_t stream);
+
+/* Split-K scratch held inside the library for tah_duo_decode_static, per GPU. */
+#define TAH_DUO_STATIC_SCRATCH_BYTES (16u << 20)
+
+/* tah_duo_decode for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc): same arguments, same kernels and same results, but the
+ * split-K partials go to a buffer of TAH_DUO_STATIC_SCRATCH_BYTES that the library itself holds on each GPU
+ * (`workspace` / `workspace_bytes` are ignored).  It has no counterpart in the reference.  Calls needing
+ * more than that -- tah_duo_decode_workspace_bytes(nq, hq, capacity1, capacity2) bytes, e.g. nq * hq *
+ * (chunks of 1024 rows over both capacities) * 520 -- return TAH_E_SCRATCH and launch nothing.  It calls no
+ * hipMalloc / hipFree; the first call on a device looks the buffer's address up once.  All calls on one
+ * GPU share the buffer (nothing in it needs clearing between calls): two calls that overlap in time on
+ * one GPU -- different streams, or graphs replayed concurrently -- race. */
+int tah_duo_decode_static(const tah_duo_decode_args* args, tah_stream_t stream);
 
 typedef struct tah_kv_append_args {
     const void* k_new;       /* bf16 [total_new, Hkv, D] */

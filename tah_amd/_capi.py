@@ -13,7 +13,8 @@ c_void_p, c_int32, c_int64, c_float = C.c_void_p, C.c_int32, C.c_int64, C.c_floa
 
 
 # error codes of include/tah_duo.h
-TAH_OK, TAH_E_NULL, TAH_E_SHAPE, TAH_E_ALIGN, TAH_E_LAUNCH, TAH_E_WORKSPACE = 0, -1, -2, -3, -4, -5
+TAH_OK, TAH_E_NULL, TAH_E_SHAPE, TAH_E_ALIGN, TAH_E_LAUNCH, TAH_E_WORKSPACE, TAH_E_SCRATCH = 0, -1, -2, -3, -4, -5, -6
+STATIC_SCRATCH_BYTES = 16 << 20
 
 
 class DuoStream(C.Structure):
@@ -136,6 +137,7 @@ PROTOTYPES = {
     "tah_duo_bwd_masked": (C.c_int, [C.POINTER(DuoBwdArgs), C.POINTER(AdditiveMask), c_void_p]),
     "tah_duo_decode_workspace_bytes": (C.c_size_t, [c_int32, c_int32, c_int32, c_int32]),
     "tah_duo_decode": (C.c_int, [C.POINTER(DuoDecodeArgs), c_void_p]),
+    "tah_duo_decode_static": (C.c_int, [C.POINTER(DuoDecodeArgs), c_void_p]),
     "tah_kv_append": (C.c_int, [C.POINTER(KvAppendArgs), c_void_p]),
     "tah_qk_prep": (C.c_int, [C.POINTER(QkPrepArgs), c_void_p]),
     "tah_hard_index_build": (C.c_int, [c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),

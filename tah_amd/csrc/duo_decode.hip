@@ -14,8 +14,15 @@
 // striding over the items balanced worse than the hardware dispatcher.)
 #include <hip/hip_runtime.h>
 
+#include <mutex>
+
 #include "duo_device.h"
 #include "tah_duo.h"
+
+// Split-K partials of tah_duo_decode_static: device memory owned by the library (every GPU the library
+// runs on holds its own copy until the process ends), for callers that cannot allocate.  In host code this
+// name is only a handle for hipGetSymbolAddress; the kernels get the address that call returned.
+static __device__ __align__(256) unsigned char scratch[TAH_DUO_STATIC_SCRATCH_BYTES];
 
 namespace tah {
 namespace {
@@ -487,22 +494,25 @@ extern "C" size_t tah_duo_decode_workspace_bytes(int32_t nq, int32_t hq, int32_t
     return (size_t)nq * hq * chunks * kPart * sizeof(float);
 }
 
-extern "C" int tah_duo_decode(const tah_duo_decode_args* a, tah_stream_t stream) {
-    using namespace tah;
+namespace tah {
+namespace {
+
+// Shared by the two decode entry points: `ws` is the caller's workspace or the library's static scratch.
+int decode_impl(const tah_duo_decode_args* a, void* ws, size_t ws_bytes, int too_small, tah_stream_t stream) {
     if (!a) return TAH_E_NULL;
     if (a->d != kD || a->nq < 0 || a->hq <= 0 || a->hkv <= 0 || a->hq % a->hkv) return TAH_E_SHAPE;
     const int g = a->hq / a->hkv;
     if (g != 1 && g != 2 && g != 4 && g != 8) return TAH_E_SHAPE;
     if (a->nq == 0) return TAH_OK;
     if (a->nq > 65535 || a->hq > 65535) return TAH_E_SHAPE;
-    if (!a->q || !a->o || !a->q_slot || !a->q_pos || !a->workspace) return TAH_E_NULL;
-    if (!aligned16(a->q) || !aligned16(a->workspace) || a->q_row_stride % 8 || a->q_head_stride % 8) return TAH_E_ALIGN;
+    if (!a->q || !a->o || !a->q_slot || !a->q_pos || !ws) return TAH_E_NULL;
+    if (!aligned16(a->q) || !aligned16(ws) || a->q_row_stride % 8 || a->q_head_stride % 8) return TAH_E_ALIGN;
     if (int rc = check_seg(a->c1, false)) return rc;
     const bool any_depth1 = a->q_depth != nullptr || a->depth >= 1;
     if (any_depth1)
         if (int rc = check_seg(a->c2, true)) return rc;
     const int cap2 = any_depth1 ? a->c2.capacity : 0;
-    if (a->workspace_bytes < tah_duo_decode_workspace_bytes(a->nq, a->hq, a->c1.capacity, cap2)) return TAH_E_WORKSPACE;
+    if (ws_bytes < tah_duo_decode_workspace_bytes(a->nq, a->hq, a->c1.capacity, cap2)) return too_small;
     DecParams p;
     p.q = static_cast<const __bf16*>(a->q);
     p.o = static_cast<__bf16*>(a->o);
@@ -513,7 +523,7 @@ extern "C" int tah_duo_decode(const tah_duo_decode_args* a, tah_stream_t stream)
     p.depth = a->depth;
     p.c1 = to_seg(a->c1);
     p.c2 = to_seg(a->c2);
-    p.ws = static_cast<float*>(a->workspace);
+    p.ws = static_cast<float*>(ws);
     p.nq = a->nq; p.hq = a->hq; p.hkv = a->hkv;
     p.nchunk1 = (a->c1.capacity + kChunk - 1) / kChunk;
     p.nchunk2 = (cap2 + kChunk - 1) / kChunk;
@@ -526,6 +536,40 @@ extern "C" int tah_duo_decode(const tah_duo_decode_args* a, tah_stream_t stream)
         case 4: return launch_decode<4>(p, st);
         default: return launch_decode<8>(p, st);
     }
+}
+
+// Device address of `scratch` on the current device, looked up once per device (each GPU holds its own
+// copy of the array at its own address).  Returns nullptr if the runtime refuses.
+void* static_scratch_of_current_device() {
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static void* addr[kMaxDevices] = {};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!addr[dev]) {
+        void* ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess) return nullptr;
+        addr[dev] = ptr;
+    }
+    return addr[dev];
+}
+
+}  // namespace
+}  // namespace tah
+
+extern "C" int tah_duo_decode(const tah_duo_decode_args* a, tah_stream_t stream) {
+    if (!a) return TAH_E_NULL;
+    return tah::decode_impl(a, a->workspace, a->workspace_bytes, TAH_E_WORKSPACE, stream);
+}
+
+extern "C" int tah_duo_decode_static(const tah_duo_decode_args* a, tah_stream_t stream) {
+    if (!a) return TAH_E_NULL;
+    void* ws = tah::static_scratch_of_current_device();
+    if (!ws) return TAH_E_LAUNCH;
+    // No partial has to start at zero: the merge kernel reads exactly the chunks the split kernel of the
+    // same call wrote, so what an earlier (larger) call left behind is never read.
+    return tah::decode_impl(a, ws, TAH_DUO_STATIC_SCRATCH_BYTES, TAH_E_SCRATCH, stream);
 }
 
 extern "C" int tah_qk_prep(const tah_qk_prep_args* a, tah_stream_t stream) {

@@ -162,6 +162,7 @@ extern "C" const char* tah_duo_error_string(int code) {
         case TAH_E_ALIGN: return "pointers must be 16-byte aligned and strides multiples of 8 elements";
         case TAH_E_LAUNCH: return "HIP launch failed";
         case TAH_E_WORKSPACE: return "workspace too small";
+        case TAH_E_SCRATCH: return "the call needs more split-K scratch than tah_duo_decode_static holds (TAH_DUO_STATIC_SCRATCH_BYTES)";
         default: return "unknown error";
     }
 }

@@ -134,12 +134,17 @@ _WORKSPACES = {}
 
 
 def decode(q: torch.Tensor, q_slot: torch.Tensor, q_pos: torch.Tensor, c1: KvSlabs, c2: Optional[KvSlabs], *,
-           scale: float, depth: int = 0, q_depth: Optional[torch.Tensor] = None, return_lse: bool = False):
+           scale: float, depth: int = 0, q_depth: Optional[torch.Tensor] = None, return_lse: bool = False,
+           out: Optional[torch.Tensor] = None, lse_out: Optional[torch.Tensor] = None, static_scratch: bool = False):
     """One decode step: q [nq, Hq, D] bf16, one row per (sequence, depth) being decoded.
 
     Row i belongs to cache slot q_slot[i], sits at position q_pos[i], and sees the
     depth-0 rows with index <= q_pos[i] plus, at depth 1, the depth-1 rows with
     pos <= q_pos[i].  ``q_depth`` (int32 [nq]) overrides ``depth`` per row.
+    ``out`` / ``lse_out`` take the results when given.  ``static_scratch=True`` calls
+    ``tah_duo_decode_static``: the split-K partials go to the buffer the library holds on the GPU, so with
+    ``out`` given the call allocates nothing (callers under graph capture); requests beyond
+    ``_capi.STATIC_SCRATCH_BYTES`` raise.
     """
     lib = _lib.lib()
     _thd(q, "q"), _i32(q_slot, "q_slot"), _i32(q_pos, "q_pos")
@@ -148,14 +153,18 @@ def decode(q: torch.Tensor, q_slot: torch.Tensor, q_pos: torch.Tensor, c1: KvSla
     need2 = q_depth is not None or depth >= 1
     if need2 and c2 is None:
         raise _capi.TahDuoError("depth-1 queries need the depth-1 cache")
-    o = torch.empty((nq, hq, d), dtype=q.dtype, device=q.device)
-    lse = torch.empty((nq, hq), dtype=torch.float32, device=q.device) if return_lse else None
-    nbytes = lib.tah_duo_decode_workspace_bytes(nq, hq, c1.capacity, c2.capacity if need2 else 0)
-    key = (q.device, _stream(q))
-    ws = _WORKSPACES.get(key)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.zeros(max(nbytes, 16), dtype=torch.uint8, device=q.device)  # counters start at zero
-        _WORKSPACES[key] = ws
+    o = out if out is not None else torch.empty((nq, hq, d), dtype=q.dtype, device=q.device)
+    if o.shape != (nq, hq, d) or o.dtype != q.dtype or o.stride(2) != 1:
+        raise _capi.TahDuoError("decode: out must be a [nq, Hq, D] tensor of q's dtype")
+    lse = lse_out if lse_out is not None else (torch.empty((nq, hq), dtype=torch.float32, device=q.device) if return_lse else None)
+    ws = None
+    if not static_scratch:
+        nbytes = lib.tah_duo_decode_workspace_bytes(nq, hq, c1.capacity, c2.capacity if need2 else 0)
+        key = (q.device, _stream(q))
+        ws = _WORKSPACES.get(key)
+        if ws is None or ws.numel() < nbytes:
+            ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=q.device)
+            _WORKSPACES[key] = ws
     a = _capi.DuoDecodeArgs()
     a.q, a.o, a.lse = _ptr(q), _ptr(o), _ptr(lse)
     a.q_row_stride, a.q_head_stride, a.o_row_stride, a.o_head_stride = q.stride(0), q.stride(1), o.stride(0), o.stride(1)
@@ -164,7 +173,10 @@ def decode(q: torch.Tensor, q_slot: torch.Tensor, q_pos: torch.Tensor, c1: KvSla
     a.c1 = c1.segment()
     if need2:
         a.c2 = c2.segment()
-    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
     a.nq, a.hq, a.hkv, a.d, a.scale = nq, hq, c1.hkv, d, float(scale)
-    _capi.check(lib, lib.tah_duo_decode(ctypes.byref(a), _stream(q)), "tah_duo_decode")
+    if static_scratch:
+        _capi.check(lib, lib.tah_duo_decode_static(ctypes.byref(a), _stream(q)), "tah_duo_decode_static")
+    else:
+        a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+        _capi.check(lib, lib.tah_duo_decode(ctypes.byref(a), _stream(q)), "tah_duo_decode")
     return (o, lse) if return_lse else o
