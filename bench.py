@@ -54,10 +54,22 @@ def cpu_baseline(seed: int, T: int, p: float, reps: int = 3):
             O.duo_prefill_dense(c["q1"], c["k1"], c["v1"], c["q2"], c["k2"], c["v2"], c["hard"], c["scale"])
             ts.append(time.perf_counter() - t0)
     t = sorted(ts[1:])[len(ts[1:]) // 2]
+    # BASELINE configs[0] exactly as stated: B=1, T=512, fp32, N(0,1) inputs, Bernoulli(0.06) hard tokens
+    c0 = make_dense_case(1234, B=1, T=512, p_hard=0.06)
+    f0 = 4.0 * 128 * 16 * visible_pairs(dense_to_varlen(c0))
+    t0s = []
+    with torch.no_grad():
+        for _ in range(11):
+            t0 = time.perf_counter()
+            O.duo_prefill_dense(c0["q1"], c0["k1"], c0["v1"], c0["q2"], c0["k2"], c0["v2"], c0["hard"], c0["scale"])
+            t0s.append(time.perf_counter() - t0)
+    tc0 = sorted(t0s[1:])[5]
     return {
         "value": flops / t / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
         "sample": f"1 of 4 sequences (B=1, T={T}, p={p}), fp32 dense mask + SDPA restatement, median of {reps}, "
                   f"{t * 1e3:.1f} ms, os.cpu_count()={os.cpu_count()}",
+        "configs0": {"workload": "configs[0]: B=1, T=512, Hq=16, Hkv=8, D=128, fp32, p_hard=0.06, as stated",
+                     "ms": tc0 * 1e3, "tflops": f0 / tc0 / 1e12, "flop": f0, "median_of": 10},
     }
 
 
@@ -71,7 +83,10 @@ def bench_decode(steps: int, warmup: int):
     g = torch.Generator().manual_seed(1236)
     lens = torch.randint(1024, 16385, (64,), generator=g).tolist()
     c = make_decode_case(1236, lens, 0.06)
-    s1, s2 = build_slabs(c, 16384, 2048, device="cuda")
+    # Three copies of the cache, used in turn: a step never reads bytes the two steps before it touched,
+    # so nothing is served from what the 256 MB last-level cache kept of an earlier step (2.3 GB per step).
+    sets = [build_slabs(c, 16384, 2048, device="cuda") for _ in range(3)]
+    s1, s2 = sets[0]
     nseq = len(lens)
     hr = torch.tensor(c["hard_rows"], dtype=torch.int32, device="cuda")
     slot = torch.cat([torch.arange(nseq, dtype=torch.int32, device="cuda"), hr])
@@ -82,26 +97,27 @@ def bench_decode(steps: int, warmup: int):
     n2 = [int(c["cu_k2"][b + 1] - c["cu_k2"][b]) for b in range(nseq)]
     rows = sum(lens) + sum(lens[b] + n2[b] for b in c["hard_rows"])
     nbytes = rows * 2 * 8 * 128 * 2  # K and V, 8 kv heads, 128 bf16
-    run = lambda: kv_cache.decode(q, slot, qpos, s1, s2, scale=c["scale"], q_depth=qd)
-    for _ in range(warmup):
-        run()
+    run = lambda i: kv_cache.decode(q, slot, qpos, sets[i % 3][0], sets[i % 3][1], scale=c["scale"], q_depth=qd)
+    for i in range(warmup):
+        run(i)
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
-    for _ in range(steps):
-        run()
+    for i in range(steps):
+        run(i)
     e1.record()
     torch.cuda.synchronize()
     ms = e0.elapsed_time(e1) / steps
     gbs = nbytes / (ms * 1e-3) / 1e9
-    return {"workload": "configs[2]: decode step, 64 seqs, ctx U[1024,16384], 6% depth-1 rows, Hq=16, Hkv=8, D=128",
+    return {"workload": "configs[2]: decode step, 64 seqs, ctx U[1024,16384], 6% depth-1 rows, Hq=16, Hkv=8, D=128 "
+                        "(three copies of the cache read in rotation)",
             "ms_per_step": ms, "visible_rows": rows, "algorithmic_bytes": nbytes, "hbm_gbs": gbs,
             "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
                          "traffic": TRAFFIC_DECODE_BYTES, "kernels": "duo_decode_split_kernel<2> + duo_decode_merge_kernel"},
             "tokens_per_s": nseq / (ms * 1e-3)}
 
 
-def bench_fwd_bwd(name: str, seqlens, p_hard: float, seed: int, steps: int, warmup: int):
+def bench_fwd_bwd(name: str, seqlens, p_hard: float, seed: int, steps: int, warmup: int, traffic=None):
     """Training forward+backward of duo-causal attention on one packed varlen batch."""
     import torch
 
@@ -134,11 +150,30 @@ def bench_fwd_bwd(name: str, seqlens, p_hard: float, seed: int, steps: int, warm
     e1.record()
     torch.cuda.synchronize()
     ms = e0.elapsed_time(e1) / steps
+    # the two halves on their own (events on the launch stream around each call)
+    o1, lse1, o2, lse2 = ops.duo_fwd_varlen(*a)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+    half = {"fwd": 0.0, "bwd": 0.0}
+    for _ in range(steps):
+        ev[0].record()
+        ops.duo_fwd_varlen(*a)
+        ev[1].record()
+        ops.duo_bwd_varlen(dev["q1"], dev["k1"], dev["v1"], o1, lse1, do1, dev["cu_q1"], dev["cu_k1"],
+                           dev["q2"], dev["k2"], dev["v2"], o2, lse2, do2, dev["pos_q2"], dev["pos_k2"],
+                           dev["cu_q2"], dev["cu_k2"], dev["scale"])
+        ev[2].record()
+        torch.cuda.synchronize()
+        half["fwd"] += ev[0].elapsed_time(ev[1]) / steps
+        half["bwd"] += ev[1].elapsed_time(ev[2]) / steps
     tf = 3.5 * fwd_flops / (ms * 1e-3) / 1e12
     return {"workload": name, "ms_per_step": ms, "visible_pairs_per_head": pairs, "flop_per_step": 3.5 * fwd_flops,
             "tflops": tf, "roofline": {"bound": "mfma", "achieved": tf, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                                       "frac": tf / PEAK_BF16_TFLOPS,
-                                       "kernels": "duo_fwd_kernel + duo_bwd_delta/dq/dkdv kernels"},
+                                       "frac": tf / PEAK_BF16_TFLOPS, "traffic": traffic,
+                                       "kernels": "duo_fwd_kernel + duo_bwd_delta/dq/dkdv kernels",
+                                       "kernel_ms": {"forward (duo_fwd_kernel)": half["fwd"],
+                                                     "backward (delta x2, dq, dkdv)": half["bwd"]},
+                                       "frac_forward": fwd_flops / (half["fwd"] * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+                                       "frac_backward": 2.5 * fwd_flops / (half["bwd"] * 1e-3) / 1e12 / PEAK_BF16_TFLOPS},
             "tokens_per_s": sum(seqlens) / (ms * 1e-3)}
 
 
@@ -155,19 +190,24 @@ def bench_qk_prep(steps: int, warmup: int):
     c = make_case(1240, rows, hq, hkv, scale=0.5, max_pos=T)
     t = to_torch(c, "cuda")
     cu = torch.arange(0, rows + 1, T, dtype=torch.int32, device="cuda")
-    slabs = KvSlabs(B, T, hkv, with_pos=False, device="cuda")
+    # every step appends to slabs of its own (67 MB a set), so no step has to reset lengths first; beyond 64
+    # steps the sets are used again and their lengths cleared on the way (one extra 4-element fill per 64 steps)
+    nsets = min(steps + warmup, 64)
+    sets = [KvSlabs(B, T, hkv, with_pos=False, device="cuda") for _ in range(nsets)]
 
-    def step():
-        slabs.len.zero_()
+    def step(i):
+        slabs = sets[i % nsets]
+        if i >= nsets:
+            slabs.len.zero_()
         qk_norm_rope(t["q"], t["k"], t["qw"], t["kw"], t["cos"], t["sin"], c["eps"], v=t["v"], cache=slabs, cu_new=cu)
 
-    for _ in range(warmup):
-        step()
+    for i in range(warmup):
+        step(i)
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
-    for _ in range(steps):
-        step()
+    for i in range(steps):
+        step(warmup + i)
     e1.record()
     torch.cuda.synchronize()
     ms = e0.elapsed_time(e1) / steps
@@ -175,7 +215,7 @@ def bench_qk_prep(steps: int, warmup: int):
     nbytes = rows * (2 * (hq + 2 * hkv) * 256 + 2 * 256)
     gbs = nbytes / (ms * 1e-3) / 1e9
     return {"workload": "step before attention for configs[1]: q/k RMSNorm + rotary + KV append, 16384 token rows, "
-                        "Hq=16, Hkv=8, D=128 (includes a 4-element length reset per step)",
+                        "Hq=16, Hkv=8, D=128 (fresh slabs every step)",
             "ms_per_step": ms, "algorithmic_bytes": nbytes, "hbm_gbs": gbs,
             "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
                          "traffic": TRAFFIC_QK_PREP_BYTES, "kernels": "qk_prep_kernel + kv_append_len_kernel"},

@@ -24,14 +24,6 @@
 #include "tah_duo.h"
 
 
-// dK/dV kernel: 8 waves (two per SIMD, 256 registers each; the default) or 4 (one per SIMD, 512
-// registers, K / V rows in registers).  Both give the same results; on the seq-8192 backward the 4-wave
-// kernel reads 29 % fewer LDS bytes and is 10 % slower (its vector work is not yet spread over the MFMA-only
-// slots), so it is built only with -DTAH_DKDV_WAVES=4.
-#ifndef TAH_DKDV_WAVES
-#define TAH_DKDV_WAVES 8
-#endif
-
 namespace tah {
 namespace {
 
@@ -692,359 +684,6 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
     }
 }
 
-// ---------------------------------------------------------------------------
-// dK/dV kernel, one wave per SIMD: 4 waves, each owning 32 keys of the 128-key tile and ALL 64 query
-// rows of an item.  With 512 registers per lane the wave keeps its K and V rows in registers (the B
-// operands of S = Q K^T and dP = dO V^T), so only the staged Q / dO tiles live in LDS and every LDS
-// byte read feeds one MFMA (1 KiB per MFMA instead of 2 KiB in the S / dP chains of the 8-wave
-// kernel); there is no second wave on the SIMD, so all latency hiding is in the slot order of the
-// body.  No reduction at the end: a wave's accumulators are complete.
-// ---------------------------------------------------------------------------
-constexpr int kKv4Threads = 256;
-constexpr int kKv4Meta = 2 * kKvSlot;                     // after the two stages: per stage lse, delta, query positions
-[[maybe_unused]] constexpr int kKv4Smem = kKv4Meta + 2 * kKvMetaBytes;
-
-template <int G, bool kDense>
-__global__ __launch_bounds__(kKv4Threads) TAH_WAVES_PER_EU(1, 1) void duo_bwd_dkdv4_kernel(const BwdParams p) {
-    HIP_DYNAMIC_SHARED(unsigned char, smem)
-    const int tid = threadIdx.x, lane = tid % kWave;
-    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);  // wave-uniform: lives in a scalar register
-    const int half = lane / 32, col = lane % 32;
-    const int kb = wave;  // 32-key block
-    const int hk = blockIdx.x;
-
-    int slot = (int)blockIdx.y;
-    int seq = 0, key0 = 0, key_end = 0;
-    bool second = false;
-    if (!(p.s1.total_k > 0 && find_tile(p.s1.cu_k, p.nseq, kBK, slot, seq, key0, key_end))) {
-        if (!(p.s2.total_k > 0 && find_tile(p.s2.cu_k, p.nseq, kBK, slot, seq, key0, key_end))) return;
-        second = true;
-    }
-    const BwdStream& ks = second ? p.s2 : p.s1;
-    const int k_lo = ks.cu_k[seq];
-    const int lk1 = p.s1.cu_k[seq + 1] - p.s1.cu_k[seq];
-    const int q1_lo = p.s1.total_q > 0 ? p.s1.cu_q[seq] : 0;
-    const int lq1 = p.s1.total_q > 0 ? p.s1.cu_q[seq + 1] - q1_lo : 0;
-    const int q2_lo = p.s2.total_q > 0 ? p.s2.cu_q[seq] : 0;
-    const int lq2 = p.s2.total_q > 0 ? p.s2.cu_q[seq + 1] - q2_lo : 0;
-    const int off = lk1 - lq1;  // position of depth-0 query i is i + off
-
-    // my key (accumulator column) and its position
-    const int key = key0 + 32 * kb + col;
-    const bool key_ok = key < key_end;
-    const int key_ld = key_ok ? key : key_end - 1;
-    const int kpos = key_ok ? (second ? ks.pos_k[key_ld] : key_ld - k_lo) : 0x7fffffff;
-
-    // my key's K and V rows, as B operands: step s holds elements 16s + 8*half .. + 7
-    bf16x8 kfr[8], vfr[8];
-    {
-        const __bf16* krow = ks.k + (int64_t)key_ld * ks.k_rs + (int64_t)hk * ks.k_hs + 8 * half;
-        const __bf16* vrow = ks.v + (int64_t)key_ld * ks.v_rs + (int64_t)hk * ks.v_hs + 8 * half;
-#pragma unroll
-        for (int s8 = 0; s8 < 8; ++s8) {
-            kfr[s8] = ld_global_16B(krow + 16 * s8);
-            vfr[s8] = ld_global_16B(vrow + 16 * s8);
-        }
-    }
-
-    // query tiles that can see this key tile
-    const int kl0 = key0 - k_lo;  // local index of the tile's first key (depth-0 tiles: its position)
-    int t1_begin = 0, nt1 = 0;
-    if (!second && lq1 > 0) {
-        const int first_q = (kl0 - off > 0 && !kDense) ? kl0 - off : 0;
-        t1_begin = first_q / kBQ;
-        nt1 = (lq1 + kBQ - 1) / kBQ - t1_begin;
-        if (nt1 < 0) nt1 = 0;
-    }
-    const int nt2 = (lq2 + kBQ - 1) / kBQ;
-    const int nitems = (nt1 + nt2) * G;
-    // Depth-0 query tiles [t_vis, t_whole) (relative to t1_begin) need no mask for this wave: all 64 rows
-    // exist and the first row already sees the last key of my block.
-    int t_whole = lq1 / kBQ - t1_begin;
-    t_whole = t_whole < 0 ? 0 : (t_whole < nt1 ? t_whole : nt1);
-    int t_vis = 0;
-    if (!second) {
-        const int need = kl0 + 32 * kb + 31 - off;  // first query row that sees my last key
-        t_vis = need > 0 ? (need + kBQ - 1) / kBQ - t1_begin : 0;
-        t_vis = t_vis < 0 ? 0 : t_vis;
-    }
-    t_vis = t_vis < t_whole ? t_vis : t_whole;
-    if constexpr (kDense) t_whole = t_vis = 0;  // the mask is read for every item
-    // the ranges below must be the same for all waves (they share the barriers): the masked prefix is
-    // as long as the longest one (the last key block's)
-    {
-        int tv = 0;
-        if (!second) {
-            const int need = kl0 + kBK - 1 - off;
-            tv = need > 0 ? (need + kBQ - 1) / kBQ - t1_begin : 0;
-            tv = tv < 0 ? 0 : tv;
-        }
-        tv = tv < t_whole ? tv : t_whole;
-        t_vis = tv;
-    }
-
-    f32x16 dkacc[4], dvacc[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) { dkacc[i][r] = 0.f; dvacc[i][r] = 0.f; }
-    const float c = p.scale_log2e;
-
-    auto item_rows = [&](int item, bool& q2s, int& r0, int& r_end, int& head) {
-        const int t = item / G;
-        head = hk * G + item % G;
-        q2s = t >= nt1;
-        if (!q2s) {
-            r0 = q1_lo + (t1_begin + t) * kBQ;
-            r_end = q1_lo + lq1;
-        } else {
-            r0 = q2_lo + (t - nt1) * kBQ;
-            r_end = q2_lo + lq2;
-        }
-        r_end = r0 + kBQ < r_end ? r0 + kBQ : r_end;
-    };
-    // Asynchronous global -> LDS copy of one item: Q and dO tiles (16 blocks of 4 rows each, four per
-    // wave), then lse / delta / positions as one dword per lane (waves 0, 1, 2).
-    const int my_lrow = 16 * wave + (lane >> 4);  // pieces: 4, 8, 12 rows further down
-    uint32_t my_chunk[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) my_chunk[i] = (uint32_t)(((lane & 15) ^ row_swizzle(my_lrow + 4 * i)) * 16);
-    struct ItemSrc {
-        const __bf16 *q, *g;
-        const float *lse, *delta;
-        const int32_t* pos;
-        uint32_t qrs2, grs2;
-        int64_t q_hs, g_hs;
-        int32_t total_q, row_lo, row_end, tile0;
-    };
-    auto stream_src = [&](bool q2s) {
-        const BwdStream& qs = q2s ? p.s2 : p.s1;
-        ItemSrc r;
-        r.q = qs.q; r.g = qs.d_o; r.lse = qs.lse; r.delta = qs.delta; r.pos = qs.pos_q;
-        r.qrs2 = (uint32_t)(qs.q_rs * 2) & 0xffffffu;
-        r.grs2 = (uint32_t)(qs.do_rs * 2) & 0xffffffu;
-        r.q_hs = qs.q_hs; r.g_hs = qs.do_hs;
-        r.total_q = qs.total_q;
-        r.row_lo = q2s ? q2_lo : q1_lo + t1_begin * kBQ;
-        r.row_end = q2s ? q2_lo + lq2 : q1_lo + lq1;
-        r.tile0 = q2s ? nt1 : 0;
-        return r;
-    };
-    ItemSrc src = stream_src(nt1 == 0);
-    auto issue_item = [&](int item, int buf) {
-        const int t = item / G, head = hk * G + item % G;
-        const bool q2s = src.tile0 != 0 || nt1 == 0;
-        const int r0 = src.row_lo + (t - src.tile0) * kBQ;
-        const int r_end = r0 + kBQ < src.row_end ? r0 + kBQ : src.row_end;
-        unsigned char* qt = smem + buf * kKvSlot;
-        unsigned char* gt = qt + kTileBytes;
-        float* meta = reinterpret_cast<float*>(smem + kKv4Meta + buf * kKvMetaBytes);
-        const int last = r_end - 1 - r0;
-        const __bf16* qbase = src.q + ((int64_t)r0 * (src.qrs2 >> 1) + (int64_t)head * src.q_hs);
-        const __bf16* gbase = src.g + ((int64_t)r0 * (src.grs2 >> 1) + (int64_t)head * src.g_hs);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const uint32_t l = (uint32_t)(my_lrow + 4 * i < last ? my_lrow + 4 * i : last) & 63u;
-            async_copy_16B(qbase, l * src.qrs2 + my_chunk[i], qt + (4 * wave + i) * 1024);
-            async_copy_16B(gbase, l * src.grs2 + my_chunk[i], gt + (4 * wave + i) * 1024);
-        }
-        const uint32_t lm = (uint32_t)(lane < last ? lane : last) * 4u;
-        const int64_t hrow = (int64_t)head * src.total_q + r0;
-        if (wave == 0) async_copy_4B(src.lse + hrow, lm, meta);
-        if (wave == 1) async_copy_4B(src.delta + hrow, lm, meta + kBQ);
-        if (wave == 2 && q2s) async_copy_4B(src.pos + r0, lm, meta + 2 * kBQ);
-    };
-    auto advance = [&](int item) {
-        TAH_WAIT_VMEM();
-        __syncthreads();
-        if (item + 1 == nt1 * G) src = stream_src(true);  // the next item is the first of the depth-1 stream
-        if (item + 1 < nitems) issue_item(item + 1, (item & 1) ^ 1);
-    };
-
-    // per-lane LDS offsets (chunk 2s + half of a row sits at (offset of chunk `half`) ^ 32s, column block
-    // dt of a transpose read at (block 0) ^ 64dt; 32 rows further down is + 8192 with the same swizzle)
-    const int aoff0 = rowmajor128_off(col, half);  // A-operand rows col (+ 32) of the Q / dO tiles
-    int toff_lo0, toff_hi0;  // transpose reads: rows 16*ks + 4*half + r/4 (+8), columns 32*dt + 16*grp + 4*(r%4)
-    {
-        const int r16 = lane & 15, grp = (lane >> 4) & 1;
-        const int trow = 4 * half + (r16 >> 2);
-        const int tcol = 16 * grp + 4 * (r16 & 3);
-        toff_lo0 = rowmajor128_off(trow, tcol >> 3) + (tcol & 7) * 2;
-        toff_hi0 = rowmajor128_off(trow + 8, tcol >> 3) + (tcol & 7) * 2;
-    }
-    const int mrow = 4 * half;  // my accumulator rows of query block qb: 32*qb + mrow + 8*(r/4) + r%4
-
-    // One item = 64 MFMAs, as 64 slots in program order with scheduling fences between them:
-    // 0-15 S (step s = n/2, query block n%2), 16-31 dP likewise with P for two rows behind each,
-    // 32-47 dV (16-query step ks = (n-32)/4, column block dt = n%4) with dS for two rows behind each,
-    // 48-63 dK.  Every slot first issues the LDS reads of a later slot.
-    auto body = [&](int item, auto mask_tag, auto stage_tag) __attribute__((always_inline)) {
-        constexpr bool kMasked = decltype(mask_tag)::value;
-        constexpr int kStage = decltype(stage_tag)::value;  // 0 / 1: stage known at compile time; -1: item & 1
-        const int stage = kStage >= 0 ? kStage : (item & 1);
-        const unsigned char* qt = smem + stage * kKvSlot;
-        const unsigned char* gt = qt + kTileBytes;
-        const float* meta = reinterpret_cast<const float*>(smem + kKv4Meta + stage * kKvMetaBytes);
-
-        [[maybe_unused]] bool q2s = false;
-        [[maybe_unused]] int nvalid = kBQ, pos0 = 0;
-        [[maybe_unused]] const int* qposs = reinterpret_cast<const int*>(meta) + 2 * kBQ;
-        [[maybe_unused]] int dense_head = 0, dense_q0 = 0;
-        if constexpr (kMasked) {
-            int r0, r_end, head;
-            item_rows(item, q2s, r0, r_end, head);
-            nvalid = r_end - r0;        // rows of the tile that exist
-            pos0 = (r0 - q1_lo) + off;  // depth-0 stream: position of tile row 0
-            dense_head = head;
-            dense_q0 = r0 - q1_lo;      // additive-mask mode: query index of tile row 0
-        }
-
-        bf16x8 ra[4], rt[4];     // operand rings
-        f32x4 lse4[2], del4[2];  // log-sum-exp / delta of four consecutive rows, two sets in flight
-        f32x16 sacc[2], dpacc[2];
-        bf16x8 pfr[4], dsfr[4];
-        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        int abase = aoff0, tlo = toff_lo0, thi = toff_hi0;
-        TAH_OPAQUE2(abase, tlo);
-        TAH_OPAQUE2(thi, abase);
-        [[maybe_unused]] int mrow_m = mrow, kpos_m = kpos;
-        if constexpr (kMasked) TAH_OPAQUE2(mrow_m, kpos_m);
-
-        // A operand of slot n < 32: rows of query block n % 2 of the Q (S) or dO (dP) tile, step (n % 16) / 2
-        auto load_a = [&](int n) __attribute__((always_inline)) {
-            ra[n % 4] = *reinterpret_cast<const bf16x8*>((n < 16 ? qt : gt) + (abase ^ (32 * ((n % 16) / 2))) + (n % 2) * 8192);
-        };
-        // B operand of tail slot m: dO columns (dV, m < 16) or Q columns (dK) of the 16 query rows of step (m % 16) / 4
-        auto load_t = [&](int m) __attribute__((always_inline)) {
-            const unsigned char* t = m < 16 ? gt : qt;
-            const int ksp = (m % 16) / 4, dt = m % 4;
-            const bf16x4 lo = lds_read_tr16(t + (tlo ^ (64 * dt)) + ksp * 4096);
-            const bf16x4 hi = lds_read_tr16(t + (thi ^ (64 * dt)) + ksp * 4096);
-            rt[m % 4] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        };
-        // P for accumulator rows r, r + 1 (r even) of query block qb
-        auto p_rows = [&](int qb, int r) __attribute__((always_inline)) {
-            float pr[2];
-#pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                const int rr = r + u, j = rr / 4, b4 = rr % 4;
-                const float lse = lse4[j % 2][b4];
-                pr[u] = fast_exp2(sacc[qb][rr] * c - lse * kLog2e);
-                if constexpr (kMasked && !kDense) {
-                    const int qr = 32 * qb + mrow_m + 8 * j + b4;
-                    const int qp = q2s ? qposs[qr] : pos0 + qr;
-                    pr[u] = (qr < nvalid && kpos_m <= qp) ? pr[u] : 0.f;
-                }
-                if constexpr (kDense) {  // mask[seq][head][query][my key]
-                    const int qr = 32 * qb + mrow_m + 8 * j + b4;
-                    const bool ok = qr < nvalid && key_ok;
-                    const int64_t e = (int64_t)seq * p.mask_sb + (int64_t)dense_head * p.mask_sh +
-                                      (int64_t)(ok ? dense_q0 + qr : 0) * p.mask_sq;
-                    const float mv = mask_value(p, static_cast<const unsigned char*>(p.mask) + e * (p.mask_f32 ? 4 : 2),
-                                                ok ? kl0 + 32 * kb + col : 0);
-                    const float lse_row = lse == kNegInf ? -kNegInf : lse;  // all keys hidden: P = 0
-                    pr[u] = ok ? fast_exp2((sacc[qb][rr] + mv * p.inv_scale) * c - lse_row * kLog2e) : 0.f;
-                }
-            }
-            const f32x2 pr2 = {pr[0], pr[1]};
-            const bf16x2 pk = __builtin_convertvector(pr2, bf16x2);
-            pfr[2 * qb + r / 8][r % 8] = pk[0];
-            pfr[2 * qb + r / 8][r % 8 + 1] = pk[1];
-        };
-        // dS = P o (dP - delta) for rows r, r + 1 of query block qb, from the bf16 P that the dV product uses
-        auto ds_rows = [&](int qb, int r) __attribute__((always_inline)) {
-            const int j = r / 4, b4 = r % 4, f = 2 * qb + r / 8;
-            const f32x2 ds2 = {(float)pfr[f][r % 8] * (dpacc[qb][r] - del4[j % 2][b4]),
-                               (float)pfr[f][r % 8 + 1] * (dpacc[qb][r + 1] - del4[j % 2][b4 + 1])};
-            const bf16x2 pk = __builtin_convertvector(ds2, bf16x2);
-            dsfr[f][r % 8] = pk[0];
-            dsfr[f][r % 8 + 1] = pk[1];
-        };
-        // row group g8 = 0..7: query block g8 / 4, rows 8*(g8 % 4) + mrow .. + 3
-        auto load_lse = [&](int g8) __attribute__((always_inline)) {
-            lse4[g8 % 2] = *reinterpret_cast<const f32x4*>(meta + 32 * (g8 / 4) + mrow + 8 * (g8 % 4));
-        };
-        auto load_del = [&](int g8) __attribute__((always_inline)) {
-            del4[g8 % 2] = *reinterpret_cast<const f32x4*>(meta + kBQ + 32 * (g8 / 4) + mrow + 8 * (g8 % 4));
-        };
-
-        load_a(0);
-        load_a(1);
-        load_a(2);
-        auto slot = [&](int n) __attribute__((always_inline)) {
-            // reads for later slots
-            if (n + 3 < 32) load_a(n + 3);
-            if (n + 3 >= 32 && n + 3 < 64) load_t(n + 3 - 32);
-            if (n >= 15 && n < 31 && (n - 15) % 2 == 0) load_lse((n - 15) / 2);  // group g8 is used by slots 16 + 2*g8, + 1
-            if (n >= 31 && n < 47 && (n - 31) % 2 == 0) load_del((n - 31) / 2);
-            __builtin_amdgcn_sched_barrier(0);
-            if (n < 16) {
-                sacc[n % 2] = mfma32(ra[n % 4], kfr[n / 2], n < 2 ? zero : sacc[n % 2]);
-            } else if (n < 32) {
-                dpacc[n % 2] = mfma32(ra[n % 4], vfr[(n - 16) / 2], n < 18 ? zero : dpacc[n % 2]);
-                // slot 16 + k: rows 2*(k % 8), + 1 of query block k / 8
-                p_rows((n - 16) / 8, 2 * ((n - 16) % 8));
-            } else if (n < 48) {
-                // dV (32 keys x 128 d) += P^T dO over 64 queries: needs P only, so the dS slices ride behind it
-                dvacc[n % 4] = mfma32(pfr[(n - 32) / 4], rt[n % 4], dvacc[n % 4]);
-                ds_rows((n - 32) / 8, 2 * ((n - 32) % 8));
-            } else {
-                // dK += dS^T Q
-                dkacc[n % 4] = mfma32(dsfr[(n - 48) / 4], rt[n % 4], dkacc[n % 4]);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        };
-        // (four loops: one fully unrolled loop of 64 slots is past the unroller's size limit, and what it
-        // leaves behind indexes the register arrays at run time)
-#pragma unroll
-        for (int n = 0; n < 16; ++n) slot(n);
-#pragma unroll
-        for (int n = 16; n < 32; ++n) slot(n);
-#pragma unroll
-        for (int n = 32; n < 48; ++n) slot(n);
-#pragma unroll
-        for (int n = 48; n < 64; ++n) slot(n);
-    };
-    using Masked = std::true_type;
-    using Plain = std::false_type;
-    using Stage0 = std::integral_constant<int, 0>;
-    using Stage1 = std::integral_constant<int, 1>;
-    using StageAny = std::integral_constant<int, -1>;
-
-    TAH_WAIT_VMEM();  // my K and V rows are in
-    if (nitems > 0) issue_item(0, 0);
-    auto run = [&](int from, int to, auto mask_tag) __attribute__((always_inline)) {
-        if constexpr (G % 2 == 0) {
-            for (int item = from; item < to; item += 2) {
-                advance(item);
-                body(item, mask_tag, Stage0{});
-                advance(item + 1);
-                body(item + 1, mask_tag, Stage1{});
-            }
-        } else {
-            for (int item = from; item < to; ++item) {
-                advance(item);
-                body(item, mask_tag, StageAny{});
-            }
-        }
-    };
-    run(0, t_vis * G, Masked{});
-    run(t_vis * G, t_whole * G, Plain{});
-    run(t_whole * G, nitems, Masked{});
-
-    // accumulator (dt, reg r, lane): key = 32*kb + acc_row(half, r), d = 32*dt + col
-#pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int krow = key0 + 32 * kb + acc_row(half, r);
-            if (krow < key_end) {
-                ks.dk[(int64_t)krow * ks.dk_rs + (int64_t)hk * ks.dk_hs + 32 * dt + col] = (__bf16)(dkacc[dt][r] * p.scale);
-                ks.dv[(int64_t)krow * ks.dv_rs + (int64_t)hk * ks.dv_hs + 32 * dt + col] = (__bf16)dvacc[dt][r];
-            }
-        }
-}
-
 BwdStream to_dev(const tah_duo_stream& s, const tah_duo_bwd_stream& g) {
     BwdStream d;
     d.q = static_cast<const __bf16*>(s.q);
@@ -1116,17 +755,10 @@ int launch_bwd(const BwdParams& p, hipStream_t st) {
         hipLaunchKernelGGL((duo_bwd_dq_kernel<G, kDense>), dim3(p.hkv, qtiles), dim3(kDqThreads), kDqSmem, st, p);
     }
     if (ktiles > 0) {
-#if TAH_DKDV_WAVES == 4
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&duo_bwd_dkdv4_kernel<G, kDense>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, kKv4Smem) != hipSuccess)
-            return TAH_E_LAUNCH;
-        hipLaunchKernelGGL((duo_bwd_dkdv4_kernel<G, kDense>), dim3(p.hkv, ktiles), dim3(kKv4Threads), kKv4Smem, st, p);
-#else
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(&duo_bwd_dkdv_kernel<G, kDense>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kKvSmem) != hipSuccess)
             return TAH_E_LAUNCH;
         hipLaunchKernelGGL((duo_bwd_dkdv_kernel<G, kDense>), dim3(p.hkv, ktiles), dim3(kKvThreads), kKvSmem, st, p);
-#endif
     }
     return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
 }

@@ -290,29 +290,42 @@ struct AppendParams {
     int32_t* overflow;
 };
 
-// grid (rows, kv heads), 32 threads: one 256-byte K row and V row per workgroup.
-__global__ void kv_append_rows_kernel(const AppendParams a) {
-    const int r = blockIdx.x, h = blockIdx.y, t = threadIdx.x;
-    int seq = 0;  // sequence of new row r
-    for (int b = 0; b < a.nseq; ++b)
-        if (r >= a.cu_new[b + 1]) seq = b + 1;
+// Sequence of new row r: the b with cu_new[b] <= r < cu_new[b+1] (binary search; nseq if r is past the end).
+__device__ __forceinline__ int seq_of_row(const int32_t* cu_new, int nseq, int r) {
+    int lo = 0, hi = nseq;  // invariant: cu_new[lo] <= r (or lo == 0), answer in [lo, hi]
+    while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (r >= cu_new[mid + 1]) lo = mid + 1;
+        else hi = mid;
+    }
+    return lo;
+}
+
+// 256 threads = 8 rows per workgroup: 32 lanes move one token row, K and V of one kv head per pass
+// (16 lanes x 16 bytes each).
+__global__ __launch_bounds__(256) void kv_append_rows_kernel(const AppendParams a, int total_new) {
+    const int r = blockIdx.x * 8 + threadIdx.x / 32, t = threadIdx.x % 32;
+    if (r >= total_new) return;
+    const int seq = seq_of_row(a.cu_new, a.nseq, r);
     if (seq >= a.nseq) return;
     const int slot = a.slot_of ? a.slot_of[seq] : seq;
     const int dst = a.len[slot] + (r - a.cu_new[seq]);
     if (dst >= a.capacity) {
-        if (a.overflow && t == 0 && h == 0) *a.overflow = 1;
+        if (a.overflow && t == 0) *a.overflow = 1;
         return;
     }
     const int64_t drow = (int64_t)a.start[slot] + dst;
-    if (t < 16) {
-        *reinterpret_cast<bf16x8*>(a.ck + drow * a.ck_rs + (int64_t)h * a.ck_hs + t * 8) =
-            *reinterpret_cast<const bf16x8*>(a.k_new + (int64_t)r * a.kn_rs + (int64_t)h * a.kn_hs + t * 8);
-    } else {
-        const int u = t - 16;
-        *reinterpret_cast<bf16x8*>(a.cv + drow * a.cv_rs + (int64_t)h * a.cv_hs + u * 8) =
-            *reinterpret_cast<const bf16x8*>(a.v_new + (int64_t)r * a.vn_rs + (int64_t)h * a.vn_hs + u * 8);
+    const int u = t % 16;
+    for (int h = 0; h < a.hkv; ++h) {
+        if (t < 16) {
+            *reinterpret_cast<bf16x8*>(a.ck + drow * a.ck_rs + (int64_t)h * a.ck_hs + u * 8) =
+                *reinterpret_cast<const bf16x8*>(a.k_new + (int64_t)r * a.kn_rs + (int64_t)h * a.kn_hs + u * 8);
+        } else {
+            *reinterpret_cast<bf16x8*>(a.cv + drow * a.cv_rs + (int64_t)h * a.cv_hs + u * 8) =
+                *reinterpret_cast<const bf16x8*>(a.v_new + (int64_t)r * a.vn_rs + (int64_t)h * a.vn_hs + u * 8);
+        }
     }
-    if (a.cpos && a.pos_new && h == 0 && t == 0) a.cpos[(int64_t)slot * a.capacity + dst] = a.pos_new[r];
+    if (a.cpos && a.pos_new && t == 0) a.cpos[(int64_t)slot * a.capacity + dst] = a.pos_new[r];
 }
 
 // Runs after the row copies on the same stream: advance the slab lengths.
@@ -388,9 +401,7 @@ __global__ __launch_bounds__(256) void qk_prep_kernel(const PrepParams p) {
     __bf16 *kdst = nullptr, *vdst = nullptr;
     int64_t kd_hs = 0, vd_hs = 0;
     if (p.append) {
-        int seq = 0;  // sequence of new row r
-        for (int b = 0; b < p.a.nseq; ++b)
-            if (r >= const_i32(p.a.cu_new, b + 1)) seq = b + 1;
+        const int seq = seq_of_row(p.a.cu_new, p.a.nseq, r);
         if (seq < p.a.nseq) {
             const int slot = p.a.slot_of ? const_i32(p.a.slot_of, seq) : seq;
             const int dst = p.a.len[slot] + (r - const_i32(p.a.cu_new, seq));
@@ -653,7 +664,7 @@ extern "C" int tah_kv_append(const tah_kv_append_args* a, tah_stream_t stream) {
     p.capacity = a->cache.capacity; p.nseq = a->nseq; p.hkv = a->hkv;
     p.overflow = a->overflow;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    hipLaunchKernelGGL(kv_append_rows_kernel, dim3(a->total_new, a->hkv), dim3(32), 0, st, p);
+    hipLaunchKernelGGL(kv_append_rows_kernel, dim3((a->total_new + 7) / 8), dim3(256), 0, st, p, a->total_new);
     hipLaunchKernelGGL(kv_append_len_kernel, dim3((a->nseq + 63) / 64), dim3(64), 0, st, p);
     return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
 }
