@@ -222,13 +222,103 @@ def bench_qk_prep(steps: int, warmup: int):
             "tokens_per_s": rows / (ms * 1e-3)}
 
 
+def bench_e2e_decode(new_tokens: int, B: int = 32, prompt_len: int = 512):
+    """BASELINE configs[4]: end-to-end TaH decode, Qwen3-1.7B architecture with random weights, a two-layer MLP
+    decider whose threshold is set so that about 6 % of the prompt tokens iterate, batch 32, 512-token prompts.
+    One HIP graph replay per generated token (both latent iterations, sampling included)."""
+    import torch
+
+    from tah_amd.engine import EngineConfig, TaHDecodeEngine, Weights
+    from tah_amd.kv_cache import decode as kv_decode, qk_norm_rope
+
+    cfg = EngineConfig()
+    w = Weights.random_init(cfg, "cuda", seed=1239)
+    eng = TaHDecodeEngine(w, B, prompt_len + new_tokens + 8, max_hard=prompt_len // 4 + new_tokens + 8, device="cuda")
+    g = torch.Generator().manual_seed(1239)
+    ids = torch.randint(0, cfg.vocab, (B * prompt_len,), generator=g).cuda()
+    cu = torch.arange(0, B * prompt_len + 1, prompt_len, dtype=torch.int32, device="cuda")
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    first, hard = eng.prefill(ids, cu, calibrate=0.06)
+    torch.cuda.synchronize()
+    prefill_s = time.perf_counter() - t0
+    # eager steps (every kernel launched from Python): what the host layer costs without the graph
+    n_eager = 8
+    eng.generate(first, 1, use_graph=False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(n_eager):
+        eng._step_inplace(0.0, -1)
+    host_eager = (time.perf_counter() - t0) / n_eager
+    torch.cuda.synchronize()
+    eager_s = (time.perf_counter() - t0) / n_eager
+    eng.host_positions += n_eager
+    eng.host_hard_rows += n_eager
+    # graph replays
+    gr = eng.capture(0.0, -1)
+    hard0, steps0 = int(eng.n_hard), int(eng.n_steps)
+    n = new_tokens - 1 - n_eager
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(n):
+        gr.replay()
+    e1.record()
+    host_s = time.perf_counter() - t0
+    torch.cuda.synchronize()
+    step_ms = e0.elapsed_time(e1) / n
+    frac_hard = (int(eng.n_hard) - hard0) / max(int(eng.n_steps) - steps0, 1)
+    # the duo-causal attention part of a step on the final cache: q/k preparation + decode kernels of all
+    # layers for both latent iterations (no append, so the cache stays as it is), replayed as a graph
+    pos = eng.pos - 1
+    cos, sin = eng.cos[pos.long()], eng.sin[pos.long()]
+    qkv = torch.randn(B, cfg.hq + 2 * cfg.hkv, cfg.head_dim, device="cuda").to(torch.bfloat16)
+    hard_rows = torch.rand(B, device="cuda") < frac_hard
+    qpos1 = torch.where(hard_rows, pos, eng.minus1)
+
+    def attn_only():
+        for l, L in enumerate(w.layers):
+            for depth in (0, 1):
+                qo, _ = qk_norm_rope(qkv[:, :cfg.hq], qkv[:, cfg.hq:cfg.hq + cfg.hkv], L["qn"], L["kn"], cos, sin, cfg.rms_eps)
+                kv_decode(qo, eng.rows, pos if depth == 0 else qpos1, eng.slabs0[l], eng.slabs1[l], scale=eng.scale,
+                          q_depth=eng.zeros_i if depth == 0 else hard_rows.to(torch.int32), static_scratch=True)
+
+    attn_only()
+    ga = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(ga):
+        attn_only()
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(50):
+        ga.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    attn_ms = e0.elapsed_time(e1) / 50
+    ctx = float(eng.pos.float().mean())
+    attn_bytes = cfg.layers * B * ctx * 2 * cfg.hkv * cfg.head_dim * 2
+    params = sum(t.numel() for L in w.layers for t in L.values()) + w.embed.numel() + w.norm.numel()
+    return {"workload": f"configs[4]: end-to-end TaH decode, Qwen3-1.7B architecture (28 layers, hidden 2048, 16/8 heads, "
+                        f"vocab 151936), random weights, B={B}, {prompt_len}-token prompts, {new_tokens} generated tokens, "
+                        "greedy sampling, MLP decider 2048->512->1 thresholded at the 94th percentile of the prompt tokens",
+            "tokens_per_s": B / (step_ms * 1e-3), "ms_per_step": step_ms, "steps_timed": n,
+            "hard_fraction_decode": frac_hard, "hard_fraction_prompt": float(hard.float().mean()),
+            "attention_ms_per_step": attn_ms, "attention_share_of_step": attn_ms / step_ms,
+            "attention_kernels": "qk_prep_kernel + duo_decode_split_kernel<2> + duo_decode_merge_kernel, 28 layers x 2 iterations",
+            "attention_cache_bytes_per_step": attn_bytes, "attention_cache_gbs": attn_bytes / (attn_ms * 1e-3) / 1e9,
+            "host_ms_per_step_graph": host_s / n * 1e3, "eager_ms_per_step": eager_s * 1e3,
+            "host_ms_per_step_eager": host_eager * 1e3, "prefill_s": prefill_s,
+            "weight_bytes": params * 2, "mean_context_at_end": ctx}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["all", "fwd", "decode", "fwd_bwd", "qk_prep"], default="all",
+    ap.add_argument("--e2e-tokens", type=int, default=1024, help="generated tokens of the end-to-end decode leg")
+    ap.add_argument("--only", choices=["all", "fwd", "decode", "fwd_bwd", "qk_prep", "e2e"], default="all",
                     help="profiling aid: run only one leg (the JSON line then lacks the other legs)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="profiling aid: also run one plain 256 MiB device copy (known traffic for counter scaling)")
@@ -282,6 +372,9 @@ def main() -> int:
 
     if args.only in ("all", "qk_prep"):
         extra["qk_prep_prefill"] = bench_qk_prep(args.steps, args.warmup)
+
+    if args.only in ("all", "e2e"):
+        extra["e2e_decode"] = bench_e2e_decode(args.e2e_tokens)
 
     out = {
         "metric": "duo-causal attn TFLOP/s (% bf16 MFMA peak) prefill; decode HBM GB/s",

@@ -208,7 +208,7 @@ typedef struct tah_kv_append_args {
     const int32_t* pos_new;  /* int32 [total_new] or NULL (depth 0) */
     int64_t k_row_stride, k_head_stride, v_row_stride, v_head_stride;
     const int32_t* cu_new;   /* int32 [nseq+1]: rows [cu_new[i], cu_new[i+1]) go to slot slot_of[i] */
-    const int32_t* slot_of;  /* int32 [nseq] or NULL (slot i) */
+    const int32_t* slot_of;  /* int32 [nseq] or NULL (slot i); a negative entry: that sequence's rows are skipped */
     int32_t nseq, total_new, hkv, d;
     tah_kv_segment cache;    /* destination; len[] is advanced by the number of rows appended */
     int32_t* overflow;       /* optional device flag, set to 1 if a slab would exceed capacity (rows dropped) */
@@ -238,7 +238,7 @@ typedef struct tah_qk_prep_args {
      * [cu_new[i], cu_new[i+1]) to slot slot_of[i], and len[] advances, as in tah_kv_append */
     int32_t append;
     const int32_t* cu_new;   /* int32 [nseq+1] */
-    const int32_t* slot_of;  /* int32 [nseq] or NULL (slot i) */
+    const int32_t* slot_of;  /* int32 [nseq] or NULL (slot i); a negative entry: q is prepared, K/V of those rows are not cached */
     const int32_t* pos_new;  /* int32 [rows] or NULL (depth 0) */
     int32_t nseq;
     tah_kv_segment cache;

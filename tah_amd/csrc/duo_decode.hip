@@ -309,6 +309,7 @@ __global__ __launch_bounds__(256) void kv_append_rows_kernel(const AppendParams 
     const int seq = seq_of_row(a.cu_new, a.nseq, r);
     if (seq >= a.nseq) return;
     const int slot = a.slot_of ? a.slot_of[seq] : seq;
+    if (slot < 0) return;  // this sequence's rows are not cached
     const int dst = a.len[slot] + (r - a.cu_new[seq]);
     if (dst >= a.capacity) {
         if (a.overflow && t == 0) *a.overflow = 1;
@@ -333,6 +334,7 @@ __global__ void kv_append_len_kernel(const AppendParams a) {
     const int b = blockIdx.x * blockDim.x + threadIdx.x;
     if (b >= a.nseq) return;
     const int slot = a.slot_of ? a.slot_of[b] : b;
+    if (slot < 0) return;
     const int n = a.len[slot] + (a.cu_new[b + 1] - a.cu_new[b]);
     a.len[slot] = n < a.capacity ? n : a.capacity;
 }
@@ -403,9 +405,11 @@ __global__ __launch_bounds__(256) void qk_prep_kernel(const PrepParams p) {
     if (p.append) {
         const int seq = seq_of_row(p.a.cu_new, p.a.nseq, r);
         if (seq < p.a.nseq) {
-            const int slot = p.a.slot_of ? const_i32(p.a.slot_of, seq) : seq;
-            const int dst = p.a.len[slot] + (r - const_i32(p.a.cu_new, seq));
-            if (dst >= p.a.capacity) {
+            const int slot = p.a.slot_of ? p.a.slot_of[seq] : seq;  // (may be written by an earlier kernel of the step)
+            const int dst = slot < 0 ? 0 : p.a.len[slot] + (r - const_i32(p.a.cu_new, seq));
+            if (slot < 0) {
+                // not cached: q is still prepared, K and V of the row go nowhere
+            } else if (dst >= p.a.capacity) {
                 if (p.a.overflow && threadIdx.x == 0) *p.a.overflow = 1;
             } else {
                 const int64_t drow = (int64_t)const_i32(p.a.start, slot) + dst;

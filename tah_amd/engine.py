@@ -1,0 +1,378 @@
+"""Decode loop for a Think-at-Hard model on the native kernels.
+
+The reference generates with ``TaHForCasualLM_generate`` (tah/model/utils.py:196-264): one
+``TaHForCausalLM.forward`` per new token, each of which re-concatenates the KV cache per layer
+(causal_cache.py:84-90), rebuilds a dense mask (tah_model.py:744-791), synchronises with the host several
+times (tah_model.py:116, 580, 686, 705) and reads every sampled token back row by row (utils.py:243-245).
+:class:`TaHDecodeEngine` runs the same computation -- the iteration loop of tah_model.py:580-706 for one
+new token per sequence -- with
+
+* per-(layer, depth) KV slabs preallocated for the whole generation (tah_amd.kv_cache.KvSlabs), appended
+  in place by the fused q/k preparation kernel (``tah_qk_prep``) and read by the split-K decode kernel
+  (``tah_duo_decode_static``: no allocation, so the step can be captured);
+* a step of fixed shape: the second latent iteration runs for all B rows with the rows the decider did
+  not select masked out (no K/V appended, no cache rows read, results dropped), so nothing in the step
+  depends on a value the host would have to read -- no ``.item()``, no ``.any()``;
+* batched sampling and end-of-sequence handling on the device;
+* the whole step captured once in a HIP graph and replayed per token.
+
+The linear layers are torch GEMMs (rocBLAS / hipBLASLt); everything between them that touches the cache is
+this library's kernels.  What is kept from the reference's forward loop, with the place it comes from:
+depth-0 logits are the running sum (``additive_logits_update``, tah_model.py:78-83); the decider sees the
+last hidden state (a two-layer MLP, hidden -> 512 -> 1, sigmoid, threshold -- the form the end-to-end
+workload names; the reference's ``MLPIterDecider`` is a larger network over several layers,
+iter_decider.py:193-301); hard rows get the top-k softmax mix of embedding rows as their next input
+(``topk_softmax_input_update``, tah_model.py:57-75) at the same position (tah_model.py:618), see the depth-0
+and depth-1 caches, and their final logits are the sum of both iterations' logits.  LoRA adapters on the
+second iteration (tah_model.py:581) are not modelled: both iterations use the same weights.
+"""
+from __future__ import annotations
+
+import dataclasses
+import math
+from typing import List, Optional, Tuple
+
+import torch
+import torch.nn.functional as F
+
+from . import ops
+from ._capi import TahDuoError
+from .kv_cache import KvSlabs, decode as _decode, qk_norm_rope
+
+
+@dataclasses.dataclass
+class EngineConfig:
+    """Qwen3-1.7B by default (the architecture of the end-to-end workload)."""
+    hidden: int = 2048
+    layers: int = 28
+    hq: int = 16
+    hkv: int = 8
+    head_dim: int = 128
+    intermediate: int = 6144
+    vocab: int = 151936
+    rms_eps: float = 1e-6
+    rope_theta: float = 1e6
+    decider_hidden: int = 512
+    topk: int = 100
+
+
+class Weights:
+    """Plain tensors of a Qwen3-shaped decoder, the output head and the decider MLP (all bf16)."""
+
+    def __init__(self, cfg: EngineConfig):
+        self.cfg = cfg
+        self.embed: torch.Tensor = None          # [V, H]
+        self.lm_head: torch.Tensor = None        # [V, H] (the embedding itself when tied)
+        self.norm: torch.Tensor = None           # [H]
+        self.layers: List[dict] = []             # ln1, wqkv, qn, kn, wo, ln2, wgu, wdown
+        self.dec_w1: torch.Tensor = None         # [Hd, H]
+        self.dec_b1: torch.Tensor = None
+        self.dec_w2: torch.Tensor = None         # [1, Hd]
+        self.dec_b2: torch.Tensor = None
+        self.threshold: float = 0.5
+
+    @staticmethod
+    def random_init(cfg: EngineConfig, device, seed: int = 0, dtype=torch.bfloat16) -> "Weights":
+        gdev = torch.device(device)
+        g = torch.Generator(device=gdev).manual_seed(seed)  # drawn where the weights live (1.7 G values at full size)
+        w = Weights(cfg)
+
+        def lin(o, i, std=None):
+            std = std if std is not None else 1.0 / math.sqrt(i)
+            out = torch.empty(o, i, dtype=dtype, device=gdev)
+            rows = max(1, (1 << 26) // i)  # in pieces: the float32 draws stay small
+            for r in range(0, o, rows):
+                n = min(rows, o - r)
+                out[r:r + n] = (torch.randn(n, i, generator=g, device=gdev) * std).to(dtype)
+            return out
+
+        H, D, I = cfg.hidden, cfg.head_dim, cfg.intermediate
+        w.embed = lin(cfg.vocab, H, std=0.02)
+        w.lm_head = w.embed
+        ones = lambda n: (1.0 + 0.05 * torch.randn(n, generator=g, device=gdev)).to(dtype)
+        w.norm = ones(H)
+        for _ in range(cfg.layers):
+            w.layers.append(dict(ln1=ones(H), wqkv=lin((cfg.hq + 2 * cfg.hkv) * D, H), qn=ones(D), kn=ones(D),
+                                 wo=lin(H, cfg.hq * D), ln2=ones(H), wgu=lin(2 * I, H), wdown=lin(H, I)))
+        w.dec_w1, w.dec_b1 = lin(cfg.decider_hidden, H), torch.zeros(cfg.decider_hidden, dtype=dtype, device=gdev)
+        w.dec_w2, w.dec_b2 = lin(1, cfg.decider_hidden), torch.zeros(1, dtype=dtype, device=gdev)
+        return w
+
+    @staticmethod
+    def from_hf(model, cfg: EngineConfig, device, dtype=torch.bfloat16) -> "Weights":
+        """Copies the tensors of a Hugging Face ``Qwen3ForCausalLM`` (q/k/v and gate/up fused row-wise)."""
+        w = Weights(cfg)
+        t = lambda x: x.detach().to(device=device, dtype=dtype).contiguous()
+        base = model.model
+        w.embed, w.norm = t(base.embed_tokens.weight), t(base.norm.weight)
+        w.lm_head = w.embed if model.lm_head.weight is base.embed_tokens.weight else t(model.lm_head.weight)
+        for lyr in base.layers:
+            a, m = lyr.self_attn, lyr.mlp
+            w.layers.append(dict(
+                ln1=t(lyr.input_layernorm.weight),
+                wqkv=t(torch.cat([a.q_proj.weight, a.k_proj.weight, a.v_proj.weight], 0)),
+                qn=t(a.q_norm.weight), kn=t(a.k_norm.weight), wo=t(a.o_proj.weight),
+                ln2=t(lyr.post_attention_layernorm.weight),
+                wgu=t(torch.cat([m.gate_proj.weight, m.up_proj.weight], 0)), wdown=t(m.down_proj.weight)))
+        return w
+
+
+def rope_tables(max_len: int, head_dim: int, theta: float, device, dtype=torch.bfloat16) -> Tuple[torch.Tensor, torch.Tensor]:
+    """cos / sin rows as ``Qwen3RotaryEmbedding`` produces them (float32 angles, cast to the model dtype)."""
+    inv = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))
+    ang = torch.arange(max_len, dtype=torch.float32)[:, None] * inv[None]
+    emb = torch.cat([ang, ang], -1)
+    return emb.cos().to(dtype).to(device), emb.sin().to(dtype).to(device)
+
+
+def topk_softmax_mix(logits: torch.Tensor, embedding: torch.Tensor, topk: int) -> torch.Tensor:
+    """Next-iteration input of a hard token (tah_model.py:57-75): softmax over the top-k logits, weighted sum of
+    the corresponding embedding rows, in the embedding's dtype."""
+    k = min(topk, logits.shape[-1])
+    val, idx = torch.topk(logits, k=k, dim=-1)
+    prob = torch.softmax(val, dim=-1)
+    return torch.sum(prob.unsqueeze(-1) * embedding[idx], dim=-2).to(embedding.dtype)
+
+
+class TaHDecodeEngine:
+    def __init__(self, weights: Weights, batch: int, max_len: int, *, max_hard: Optional[int] = None, device="cuda"):
+        cfg = weights.cfg
+        if cfg.head_dim != 128:
+            raise TahDuoError("the kernels are built for head_dim 128")
+        self.w, self.cfg, self.B, self.max_len = weights, cfg, batch, max_len
+        self.device = torch.device(device)
+        self.max_hard = max_hard if max_hard is not None else max_len
+        self.cos, self.sin = rope_tables(max_len, cfg.head_dim, cfg.rope_theta, self.device)
+        self.slabs0 = [KvSlabs(batch, max_len, cfg.hkv, cfg.head_dim, with_pos=False, device=self.device) for _ in range(cfg.layers)]
+        self.slabs1 = [KvSlabs(batch, self.max_hard, cfg.hkv, cfg.head_dim, with_pos=True, device=self.device) for _ in range(cfg.layers)]
+        dev = self.device
+        self.rows = torch.arange(batch, dtype=torch.int32, device=dev)
+        self.cu_rows = torch.arange(batch + 1, dtype=torch.int32, device=dev)
+        self.minus1 = torch.full((batch,), -1, dtype=torch.int32, device=dev)
+        self.zeros_i = torch.zeros(batch, dtype=torch.int32, device=dev)
+        # generation state (all on the device)
+        self.tok = torch.zeros(batch, dtype=torch.long, device=dev)       # token fed to the next step
+        self.pos = torch.zeros(batch, dtype=torch.int32, device=dev)      # its position
+        self.finished = torch.zeros(batch, dtype=torch.bool, device=dev)
+        self.n_hard = torch.zeros((), dtype=torch.long, device=dev)       # tokens that took a second iteration
+        self.n_steps = torch.zeros((), dtype=torch.long, device=dev)      # tokens decoded (active rows x steps)
+        self.step_idx = torch.zeros(1, dtype=torch.long, device=dev)
+        self.out_tokens = torch.zeros(batch, max_len, dtype=torch.long, device=dev)  # generated tokens, column = step
+        self.scale = float(cfg.head_dim) ** -0.5
+        self.host_positions = 0  # upper bound on any sequence's length, kept on the host for capacity checks
+        self.host_hard_rows = 0
+        self._graph = None
+        self.static_scratch = self.device.type == "cuda"
+
+    # ── model pieces ─────────────────────────────────────────────────────
+    def _rms(self, x, w):
+        return F.rms_norm(x, (x.shape[-1],), w, self.cfg.rms_eps)
+
+    def _mlp(self, x, L):
+        gu = self._rms(x, L["ln2"]) @ L["wgu"].t()
+        I = self.cfg.intermediate
+        return x + (F.silu(gu[:, :I]) * gu[:, I:]) @ L["wdown"].t()
+
+    def _split_qkv(self, qkv):
+        c = self.cfg
+        n = qkv.shape[0]
+        qkv = qkv.view(n, c.hq + 2 * c.hkv, c.head_dim)
+        return qkv[:, :c.hq], qkv[:, c.hq:c.hq + c.hkv], qkv[:, c.hq + c.hkv:]
+
+    def decide(self, hidden: torch.Tensor) -> torch.Tensor:
+        """Continue probability of the two-layer decider MLP on the last hidden state, float32 [rows]."""
+        w = self.w
+        h = F.relu(hidden @ w.dec_w1.t() + w.dec_b1)
+        return torch.sigmoid((h @ w.dec_w2.t() + w.dec_b2).float()).view(-1)
+
+    # ── one token per sequence through all layers at one depth ───────────
+    def _pass_single(self, x, pos, depth: int, slot_of, q_pos, q_depth):
+        """x [B, H]; appends this token's K/V to the depth's slabs (rows with slot_of < 0 are not cached) and
+        attends with q_pos / q_depth per row (q_pos < 0: the row sees nothing and is dropped by the caller)."""
+        c = self.cfg
+        cos, sin = self.cos[pos.long()], self.sin[pos.long()]
+        for l, L in enumerate(self.w.layers):
+            qkv = self._rms(x, L["ln1"]) @ L["wqkv"].t()
+            q, k, v = self._split_qkv(qkv)
+            cache = self.slabs0[l] if depth == 0 else self.slabs1[l]
+            qo, _ = qk_norm_rope(q, k, L["qn"], L["kn"], cos, sin, c.rms_eps, v=v, cache=cache, cu_new=self.cu_rows,
+                                 slot_of=slot_of, pos_new=pos if depth == 1 else None)
+            o = _decode(qo, self.rows, q_pos, self.slabs0[l], self.slabs1[l], scale=self.scale, q_depth=q_depth,
+                        static_scratch=self.static_scratch)
+            x = x + o.view(x.shape[0], c.hq * c.head_dim) @ L["wo"].t()
+            x = self._mlp(x, L)
+        return self._rms(x, self.w.norm)
+
+    def step_logits(self, tok: torch.Tensor, force_hard: Optional[torch.Tensor] = None, active: Optional[torch.Tensor] = None):
+        """The iteration loop of tah_model.py:580-706 for one new token per sequence, on ``self.pos``.
+
+        Returns (final logits float32 [B, V], hard bool [B]).  ``force_hard`` replaces the decider's decision
+        (tests drive both implementations with the same decisions).  Rows that are not ``active`` are neither
+        cached nor attended; their logits are meaningless."""
+        B = self.B
+        pos = self.pos
+        act = active if active is not None else torch.ones(B, dtype=torch.bool, device=self.device)
+        slot0 = torch.where(act, self.rows, self.minus1)
+        qpos0 = torch.where(act, pos, self.minus1)
+        h0 = self._pass_single(self.w.embed[tok], pos, 0, slot0, qpos0, self.zeros_i)
+        l0 = (h0 @ self.w.lm_head.t()).float()
+        hard = (self.decide(h0) > self.w.threshold) if force_hard is None else force_hard
+        hard = hard & act
+        x1 = topk_softmax_mix(l0.to(self.w.embed.dtype), self.w.embed, self.cfg.topk)
+        slot1 = torch.where(hard, self.rows, self.minus1)
+        qpos1 = torch.where(hard, pos, self.minus1)
+        h1 = self._pass_single(x1, pos, 1, slot1, qpos1, hard.to(torch.int32))
+        l1 = (h1 @ self.w.lm_head.t()).float()
+        # running sum of the iterations' logits, rounded to the model dtype as the reference's buffers are
+        # (tah_model.py:543, 628)
+        dt = self.w.embed.dtype
+        both = (l0.to(dt) + l1.to(dt)).float()
+        return torch.where(hard[:, None], both, l0.to(dt).float()), hard
+
+    # ── prefill: packed prompts, both depths, through the varlen kernels ──
+    @torch.no_grad()
+    def prefill(self, ids: torch.Tensor, cu: torch.Tensor, *, force_hard: Optional[torch.Tensor] = None,
+                calibrate: Optional[float] = None):
+        """ids int64 [N] (the prompts one after another), cu int32 [B+1].  Fills both caches and returns
+        (logits float32 [B, V] of each prompt's last token, hard bool [N]).  ``calibrate=p`` first sets the
+        decider threshold to the (1-p) quantile of its outputs on these prompts."""
+        c, w, dev = self.cfg, self.w, self.device
+        B = self.B
+        if cu.numel() != B + 1:
+            raise TahDuoError("cu must have batch + 1 entries")
+        cu_h = cu.cpu()
+        lens = (cu_h[1:] - cu_h[:-1]).tolist()
+        N = int(cu_h[-1])
+        if max(lens) > self.max_len:
+            raise TahDuoError("prompt longer than the cache capacity")
+        seq = torch.repeat_interleave(torch.arange(B, device=dev), torch.tensor(lens, device=dev))
+        pos = (torch.arange(N, device=dev) - cu.long()[seq]).to(torch.int32)
+        cos, sin = self.cos[pos.long()], self.sin[pos.long()]
+        zc = torch.zeros(B + 1, dtype=torch.int32, device=dev)
+        zi = torch.zeros(0, dtype=torch.int32, device=dev)
+        x = w.embed[ids]
+        kv_tok = []
+        for l, L in enumerate(w.layers):
+            q, k, v = self._split_qkv(self._rms(x, L["ln1"]) @ L["wqkv"].t())
+            qo, ko = qk_norm_rope(q, k, L["qn"], L["kn"], cos, sin, c.rms_eps)
+            o1, _, _, _ = ops.duo_fwd_varlen(qo, ko, v, cu, cu, qo[:0], ko[:0], v[:0], zi, zi, zc, zc, self.scale)
+            self.slabs0[l].append(ko, v, cu)
+            kv_tok.append((ko, v))
+            x = x + o1.view(N, -1) @ L["wo"].t()
+            x = self._mlp(x, L)
+        h0 = self._rms(x, w.norm)
+        prob = self.decide(h0)
+        if calibrate is not None:
+            w.threshold = float(torch.quantile(prob, 1.0 - calibrate))
+        hard = (prob > w.threshold) if force_hard is None else force_hard
+        last = (cu[1:] - 1).long()
+        logits_last = (h0[last] @ w.lm_head.t())  # model dtype, like the reference's logits buffers
+        rows2 = torch.nonzero(hard).flatten()
+        n2 = rows2.numel()
+        if n2:
+            counts = torch.zeros(B, dtype=torch.long, device=dev).index_add_(0, seq[rows2], torch.ones_like(rows2))
+            if int(counts.max()) > self.max_hard:
+                raise TahDuoError("more hard tokens in a prompt than the depth-1 cache holds")
+            cu2 = torch.cat([torch.zeros(1, dtype=torch.long, device=dev), counts.cumsum(0)]).to(torch.int32)
+            l0h = h0[rows2] @ w.lm_head.t()
+            x2 = topk_softmax_mix(l0h, w.embed, c.topk)
+            pos2 = pos[rows2].contiguous()
+            cos2, sin2 = self.cos[pos2.long()], self.sin[pos2.long()]
+            for l, L in enumerate(w.layers):
+                q, k, v = self._split_qkv(self._rms(x2, L["ln1"]) @ L["wqkv"].t())
+                qo, ko = qk_norm_rope(q, k, L["qn"], L["kn"], cos2, sin2, c.rms_eps)
+                k1, v1 = kv_tok[l]
+                _, _, o2, _ = ops.duo_fwd_varlen(qo[:0], k1, v1, zc, cu, qo, ko, v, pos2, pos2, cu2, cu2, self.scale)
+                self.slabs1[l].append(ko, v, cu2, pos_new=pos2)
+                x2 = x2 + o2.view(n2, -1) @ L["wo"].t()
+                x2 = self._mlp(x2, L)
+            l1h = self._rms(x2, w.norm) @ w.lm_head.t()
+            both = l0h + l1h
+            # a prompt whose last token is hard: its final logits are the sum of both iterations'
+            is_last = torch.isin(rows2, last)
+            if bool(is_last.any()):
+                which = seq[rows2[is_last]]
+                logits_last[which] = both[is_last]
+            self.host_hard_rows = int(counts.max())
+        self.pos.copy_(torch.tensor(lens, dtype=torch.int32))
+        self.host_positions = max(lens)
+        self.finished.zero_()
+        return logits_last.float(), hard
+
+    # ── sampling / generation ────────────────────────────────────────────
+    @staticmethod
+    def sample(logits: torch.Tensor, temperature: float) -> torch.Tensor:
+        """Batched: greedy at temperature 0, else the Gumbel-max form of sampling from softmax(logits / T)."""
+        if temperature <= 0.0:
+            return torch.argmax(logits, dim=-1)
+        u = torch.empty_like(logits).exponential_()
+        return torch.argmax(logits / temperature - torch.log(u), dim=-1)
+
+    def _step_inplace(self, temperature: float, eos: int):
+        """One generated token for every unfinished row; every state change is an in-place device update."""
+        act = ~self.finished
+        logits, hard = self.step_logits(self.tok, active=act)
+        nxt = self.sample(logits, temperature)
+        nxt = torch.where(act, nxt, torch.zeros_like(nxt))
+        self.out_tokens.scatter_(1, self.step_idx.expand(self.B, 1), nxt[:, None])
+        self.n_hard += hard.sum()
+        self.n_steps += act.sum()
+        self.pos += act.to(torch.int32)
+        self.step_idx += 1
+        if eos >= 0:
+            self.finished |= nxt == eos
+        self.tok.copy_(nxt)
+
+    @torch.no_grad()
+    def generate(self, first_logits: torch.Tensor, max_new_tokens: int, *, temperature: float = 0.0, eos: int = -1,
+                 use_graph: bool = True):
+        """Continues after :meth:`prefill`.  Returns tokens int64 [B, max_new_tokens] (0 after a row's end)."""
+        if self.host_positions + max_new_tokens > self.max_len or self.host_hard_rows + max_new_tokens > self.max_hard:
+            raise TahDuoError("generation would outgrow the KV slabs: construct the engine with a larger max_len / max_hard")
+        dev = self.device
+        self.out_tokens.zero_()
+        self.step_idx.zero_()
+        first = self.sample(first_logits, temperature)
+        self.out_tokens[:, 0] = first
+        self.tok.copy_(first)
+        if eos >= 0:
+            self.finished |= first == eos
+        self.step_idx += 1
+        n = max_new_tokens - 1
+        if n <= 0:
+            return self.out_tokens[:, :max_new_tokens]
+        if use_graph and dev.type == "cuda":
+            self.capture(temperature, eos)
+            for _ in range(n):
+                self._graph.replay()
+        else:
+            for _ in range(n):
+                self._step_inplace(temperature, eos)
+        self.host_positions += n
+        self.host_hard_rows += n
+        return self.out_tokens[:, :max_new_tokens]
+
+    def capture(self, temperature: float = 0.0, eos: int = -1):
+        """Captures one generation step in a HIP graph (after a warm-up step run on a side stream whose state
+        changes are undone, so that library workspaces exist before the capture)."""
+        if self._graph is not None and self._graph_key == (temperature, eos):
+            return self._graph
+        state = [t.clone() for t in (self.tok, self.pos, self.finished, self.n_hard, self.n_steps, self.step_idx, self.out_tokens)]
+        lens = [(s.len.clone(), ) for s in self.slabs0 + self.slabs1]
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            self._step_inplace(temperature, eos)
+        torch.cuda.current_stream().wait_stream(s)
+        torch.cuda.synchronize()
+        # undo the warm-up step: state tensors and slab lengths (the rows it wrote lie beyond the lengths)
+        for t, old in zip((self.tok, self.pos, self.finished, self.n_hard, self.n_steps, self.step_idx, self.out_tokens), state):
+            t.copy_(old)
+        for sl, (ln,) in zip(self.slabs0 + self.slabs1, lens):
+            sl.len.copy_(ln)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            self._step_inplace(temperature, eos)
+        # the capture itself does not run the step
+        self._graph, self._graph_key = g, (temperature, eos)
+        return g

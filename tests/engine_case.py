@@ -1,0 +1,108 @@
+"""The decode engine (tah_amd.engine) against the reference's forward loop restated around a Hugging Face
+``Qwen3Model``: dense additive masks (oracle.duo_oracle.build_attention_mask = tah_model.py:744-791), a cache
+that returns the concatenated K/V (oracle.duo_oracle.OracleCache = causal_cache.py:63-109), ``gather_active`` /
+``scatter_back`` packing, the top-k softmax mix and the running sum of logits (tah_model.py:57-83, 580-706), in
+float32 on the host.  Both sides are fed the same tokens and the same hard decisions (teacher forcing), so the
+comparison is of logits, step by step, not of trajectories."""
+import pytest
+import torch
+
+from oracle import duo_oracle as O
+
+
+class _Cache(O.OracleCache):
+    """What transformers' model code asks of a cache object besides update()."""
+
+    def get_seq_length(self, layer_idx=0):
+        return sum(t.shape[-2] for t in self.k.get((layer_idx, 0), []))
+
+    def get_mask_sizes(self, cache_position, layer_idx):
+        return cache_position.shape[0] + self.get_seq_length(layer_idx), 0
+
+
+def _ref_forward(model, embed, cache, ids, valid, hard, topk):
+    """tah_model.py:495-706 for max_iter = 2 with the decider's decisions given: returns final logits (B, T, V)."""
+    B, T = ids.shape
+    x = embed[ids]
+    cached_valid = cache.get_valid_mask_upto_iter(0, 0, B)
+    pos = (torch.cumsum(torch.cat((cached_valid, valid), -1), -1)[:, -T:] - 1).clamp(min=0)  # tah_model.py:555-561
+    m0 = O.build_attention_mask(pos, valid, cache, 0, torch.float32)
+    cache.current_iter_depth, cache.position_ids_to_cache, cache.valid_mask_to_cache = 0, pos, valid
+    h = model(inputs_embeds=x, attention_mask={"full_attention": m0}, position_ids=pos, past_key_values=cache,
+              use_cache=True).last_hidden_state
+    cum = h @ embed.t()
+    final = cum.clone()
+    cur = hard & (valid == 1)
+    if cur.any():
+        pad, a_cum, a_pos, a_valid = O.gather_active(cur, cum, pos, valid)
+        k = min(topk, a_cum.shape[-1])
+        tv, ti = torch.topk(a_cum, k=k, dim=-1)
+        a_x = torch.sum(torch.softmax(tv, -1).unsqueeze(-1) * embed[ti], dim=-2)  # tah_model.py:57-75
+        m1 = O.build_attention_mask(a_pos, a_valid, cache, 1, torch.float32)
+        cache.current_iter_depth, cache.position_ids_to_cache, cache.valid_mask_to_cache = 1, a_pos, a_valid
+        h1 = model(inputs_embeds=a_x, attention_mask={"full_attention": m1}, position_ids=a_pos, past_key_values=cache,
+                   use_cache=True).last_hidden_state
+        final = O.scatter_back(cur, a_cum + h1 @ embed.t(), final)  # additive_logits_update, tah_model.py:78-83
+    return final
+
+
+def run(device, *, prompt=(9, 6, 12), steps=5, layers=2, seed=0, vocab=96, topk=100):
+    pytest.importorskip("transformers.models.qwen3.modeling_qwen3")
+    from transformers import Qwen3Config, Qwen3Model
+
+    from tah_amd.engine import EngineConfig, TaHDecodeEngine, Weights
+
+    torch.manual_seed(seed)
+    hf = Qwen3Config(hidden_size=256, num_attention_heads=4, num_key_value_heads=2, head_dim=128,
+                     num_hidden_layers=layers, intermediate_size=512, vocab_size=vocab, rope_theta=1e6,
+                     attention_dropout=0.0, rms_norm_eps=1e-6)
+    hf._attn_implementation = "sdpa"
+    ref = Qwen3Model(hf).to(torch.bfloat16).float().eval()  # bf16-representable weights, float32 arithmetic
+    cfg = EngineConfig(hidden=256, layers=layers, hq=4, hkv=2, head_dim=128, intermediate=512, vocab=vocab,
+                       decider_hidden=32, topk=topk)
+
+    class _LM:  # the pieces Weights.from_hf reads: tied output head
+        model = ref
+        lm_head = type("H", (), {"weight": ref.embed_tokens.weight})
+    w = Weights.from_hf(_LM, cfg, device)
+    g = torch.Generator().manual_seed(seed + 1)
+    w.dec_w1 = torch.randn(32, 256, generator=g).to(torch.bfloat16).to(device)
+    w.dec_b1 = torch.zeros(32, dtype=torch.bfloat16, device=device)
+    w.dec_w2 = torch.randn(1, 32, generator=g).to(torch.bfloat16).to(device)
+    w.dec_b2 = torch.zeros(1, dtype=torch.bfloat16, device=device)
+
+    B, Tm = len(prompt), max(prompt)
+    eng = TaHDecodeEngine(w, B, Tm + steps + 4, device=device)
+    ids = torch.randint(0, vocab, (B, Tm + steps), generator=g)
+    valid = torch.zeros(B, Tm, dtype=torch.long)
+    for b, n in enumerate(prompt):
+        valid[b, Tm - n:] = 1  # left padding, as the reference batches prompts
+    hard = torch.rand(B, Tm + steps, generator=g) < 0.35
+    hard[:, Tm] = torch.tensor([True] + [False] * (B - 1))   # first decode step: one hard row, the rest pad rows
+    hard[:, Tm + 1] = False                                  # second: nobody iterates
+    hard[:, Tm + 2] = True                                   # third: every row does
+    hard[0, Tm - 1] = True                                   # a prompt whose last token is hard
+    embed = ref.embed_tokens.weight.detach()
+
+    out = []
+    with torch.no_grad():
+        cache = _Cache()
+        want = _ref_forward(ref, embed, cache, ids[:, :Tm], valid, hard[:, :Tm], topk)[:, -1]
+        packed = torch.cat([ids[b, Tm - n:Tm] for b, n in enumerate(prompt)]).to(device)
+        hard_packed = torch.cat([hard[b, Tm - n:Tm] for b, n in enumerate(prompt)]).to(device)
+        cu = torch.tensor([0] + list(torch.tensor(prompt).cumsum(0)), dtype=torch.int32, device=device)
+        got, _ = eng.prefill(packed, cu, force_hard=hard_packed)
+        out.append((got.cpu(), want))
+        one = torch.ones(B, 1, dtype=torch.long)
+        for s in range(steps):
+            t = Tm + s
+            want = _ref_forward(ref, embed, cache, ids[:, t:t + 1], one, hard[:, t:t + 1], topk)[:, 0]
+            got, h = eng.step_logits(ids[:, t].to(device), force_hard=hard[:, t].to(device))
+            eng.pos += 1
+            assert torch.equal(h.cpu(), hard[:, t])
+            out.append((got.cpu(), want))
+    lens0 = [n + steps for n in prompt]
+    assert all(sl.len.tolist() == lens0 for sl in eng.slabs0)
+    n1 = [int(hard[b, Tm - n:].sum()) for b, n in enumerate(prompt)]
+    assert all(sl.len.tolist() == n1 for sl in eng.slabs1)
+    return out
