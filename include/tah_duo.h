@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define TAH_DUO_ABI_VERSION 1
+#define TAH_DUO_ABI_VERSION 2
 
 enum {
     TAH_OK = 0,
@@ -243,6 +243,9 @@ typedef struct tah_qk_prep_args {
     int32_t nseq;
     tah_kv_segment cache;
     int32_t* overflow;       /* optional device flag, as in tah_kv_append */
+    /* != 0: the caller promises that every sequence brings at most one row and that the slots named are all
+     * different (a decode step): the lengths are then advanced by the same launch instead of a second one */
+    int32_t append_one_row_per_seq;
 } tah_qk_prep_args;
 
 /* Per-head RMSNorm of q and k, rotary embedding of both, and optionally the KV-cache append,
@@ -253,6 +256,30 @@ typedef struct tah_qk_prep_args {
  *   TaHCache.update               tah/model/causal_cache.py:63-97 (with append)
  * head_dim 128 only.  In-place use (q_out == q, k_out == k) is allowed. */
 int tah_qk_prep(const tah_qk_prep_args* args, tah_stream_t stream);
+
+typedef struct tah_topk_mix_args {
+    const void* logits;        /* bf16 [rows, vocab], vocab contiguous */
+    const void* embedding;     /* bf16 [vocab, hidden], 16-byte aligned rows */
+    void* out;                 /* bf16 [rows, hidden] */
+    const uint8_t* row_enable; /* optional, one byte per row: rows whose byte is 0 are skipped (out untouched) */
+    int64_t logits_row_stride, embedding_row_stride, out_row_stride; /* elements */
+    int32_t rows, vocab, hidden, topk; /* topk <= 256, vocab <= 155648, hidden a multiple of 8 */
+} tah_topk_mix_args;
+
+/* Next-iteration input of hard tokens: softmax over each row's top-k logits, then the probability-weighted
+ * sum of the corresponding embedding rows.  Replaces topk_softmax_input_update (tah/model/tah_model.py:57-75:
+ * torch.topk + softmax + gather of (rows, k, hidden) embedding rows + sum) with one pass per row and no
+ * (rows, k, hidden) intermediate.  Among equal logits at the k-th place the lower vocabulary indices are
+ * taken (torch.topk leaves that choice open).  Probabilities and products round to bf16 where the bf16
+ * eager arithmetic rounds; sums are float32 in index order, so results do not vary from run to run. */
+int tah_topk_mix(const tah_topk_mix_args* args, tah_stream_t stream);
+
+/* Gate of the Qwen3 MLP for a decode step: out[r][i] = silu(gate_up[r][i]) * gate_up[r][inter + i], both
+ * steps rounded to bf16 as the eager modules round them -- `act_fn(gate_proj(x)) * up_proj(x)` of Qwen3MLP.forward
+ * (transformers/models/qwen3/modeling_qwen3.py, third party; the layer the reference's base model runs,
+ * tah/model/tah_model.py:616-623) on the output of one fused gate|up projection.  One launch instead of two. */
+int tah_silu_mul(const void* gate_up, void* out, int32_t rows, int32_t inter, int64_t gate_up_row_stride,
+                 int64_t out_row_stride, tah_stream_t stream);
 
 /* Hard-token index build: stream compaction of a (B, S) byte mask in row-major
  * order.  Replaces the stable sort + nonzero of gather_active / scatter_back

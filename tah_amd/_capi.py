@@ -7,7 +7,7 @@ from __future__ import annotations
 
 import ctypes as C
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 c_void_p, c_int32, c_int64, c_float = C.c_void_p, C.c_int32, C.c_int64, C.c_float
 
@@ -125,6 +125,17 @@ class QkPrepArgs(C.Structure):
         ("nseq", c_int32),
         ("cache", KvSegment),
         ("overflow", c_void_p),
+        ("append_one_row_per_seq", c_int32),
+    ]
+
+
+class TopkMixArgs(C.Structure):
+    """``tah_topk_mix_args``"""
+
+    _fields_ = [
+        ("logits", c_void_p), ("embedding", c_void_p), ("out", c_void_p), ("row_enable", c_void_p),
+        ("logits_row_stride", c_int64), ("embedding_row_stride", c_int64), ("out_row_stride", c_int64),
+        ("rows", c_int32), ("vocab", c_int32), ("hidden", c_int32), ("topk", c_int32),
     ]
 
 
@@ -140,6 +151,8 @@ PROTOTYPES = {
     "tah_duo_decode_static": (C.c_int, [C.POINTER(DuoDecodeArgs), c_void_p]),
     "tah_kv_append": (C.c_int, [C.POINTER(KvAppendArgs), c_void_p]),
     "tah_qk_prep": (C.c_int, [C.POINTER(QkPrepArgs), c_void_p]),
+    "tah_topk_mix": (C.c_int, [C.POINTER(TopkMixArgs), c_void_p]),
+    "tah_silu_mul": (C.c_int, [c_void_p, c_void_p, c_int32, c_int32, c_int64, c_int64, c_void_p]),
     "tah_hard_index_build": (C.c_int, [c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "tah_pad_rows_build": (C.c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_void_p]),
     "tah_rows_copy": (C.c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int64,

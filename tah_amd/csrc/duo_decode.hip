@@ -355,6 +355,7 @@ struct PrepParams {
     int64_t cs_rs;
     float eps;
     int32_t rows, hq, hkv, append;
+    int32_t own_len;  // every sequence appends at most one row: the row's workgroup advances the length itself
     AppendParams a;  // destination slabs (append != 0); its k_new / v_new fields are not used
 };
 
@@ -407,6 +408,8 @@ __global__ __launch_bounds__(256) void qk_prep_kernel(const PrepParams p) {
         if (seq < p.a.nseq) {
             const int slot = p.a.slot_of ? p.a.slot_of[seq] : seq;  // (may be written by an earlier kernel of the step)
             const int dst = slot < 0 ? 0 : p.a.len[slot] + (r - const_i32(p.a.cu_new, seq));
+            if (p.own_len) __syncthreads();  // every wave has read the old length before thread 0 replaces it (the
+                                             // branch is uniform: one row, one sequence, one slot per workgroup)
             if (slot < 0) {
                 // not cached: q is still prepared, K and V of the row go nowhere
             } else if (dst >= p.a.capacity) {
@@ -418,6 +421,7 @@ __global__ __launch_bounds__(256) void qk_prep_kernel(const PrepParams p) {
                 kd_hs = p.a.ck_hs;
                 vd_hs = p.a.cv_hs;
                 if (p.a.cpos && p.a.pos_new && threadIdx.x == 0) p.a.cpos[(int64_t)slot * p.a.capacity + dst] = p.a.pos_new[r];
+                if (p.own_len && threadIdx.x == 0) p.a.len[slot] = dst + 1;  // nobody else reads or writes this slot's length
             }
         }
     } else {
@@ -623,6 +627,7 @@ extern "C" int tah_qk_prep(const tah_qk_prep_args* a, tah_stream_t stream) {
     p.cs_rs = a->cos_sin_row_stride;
     p.eps = a->eps;
     p.rows = a->rows; p.hq = a->hq; p.hkv = a->hkv; p.append = a->append ? 1 : 0;
+    p.own_len = (a->append && a->append_one_row_per_seq) ? 1 : 0;
     p.a = AppendParams{};
     if (a->append) {
         p.a.pos_new = a->pos_new; p.a.cu_new = a->cu_new; p.a.slot_of = a->slot_of;
@@ -638,7 +643,7 @@ extern "C" int tah_qk_prep(const tah_qk_prep_args* a, tah_stream_t stream) {
     }
     hipStream_t st = static_cast<hipStream_t>(stream);
     hipLaunchKernelGGL(qk_prep_kernel, dim3(a->rows), dim3(256), 0, st, p);
-    if (a->append) hipLaunchKernelGGL(kv_append_len_kernel, dim3((a->nseq + 63) / 64), dim3(64), 0, st, p.a);
+    if (a->append && !p.own_len) hipLaunchKernelGGL(kv_append_len_kernel, dim3((a->nseq + 63) / 64), dim3(64), 0, st, p.a);
     return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
 }
 

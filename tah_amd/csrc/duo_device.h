@@ -145,6 +145,9 @@ __device__ __forceinline__ void async_copy_4B(const void* sbase, uint32_t voff, 
 #ifndef TAH_OPAQUE2
 #define TAH_OPAQUE2(a, b) asm volatile("" : "+v"(a), "+v"(b))
 #endif
+#ifndef TAH_OPAQUE1
+#define TAH_OPAQUE1(a) asm volatile("" : "+v"(a))
+#endif
 // Occupancy the kernel is written for; lets the scheduler spend registers on latency hiding.
 // Between LDS writes of a wave and reads, by the same wave, of what its other lanes wrote: the lanes run
 // in lockstep and the LDS serves a wave's requests in order, so all that is needed is that the compiler

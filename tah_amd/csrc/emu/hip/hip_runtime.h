@@ -33,6 +33,7 @@
 #define TAH_WAIT_VMEM() ((void)0)
 #define TAH_KEEP_HERE4(a, b, c, d) ((void)0)
 #define TAH_OPAQUE2(a, b) ((void)0)
+#define TAH_OPAQUE1(a) ((void)0)
 #define TAH_SCALE16_IF(acc, a, cond) \
     do { if (cond) for (int tah_i_ = 0; tah_i_ < 16; ++tah_i_) (acc)[tah_i_] *= (a); } while (0)
 #define TAH_ASYNC_COPY_16B(gsrc, lds_wave_base) \

@@ -1,0 +1,266 @@
+// Top-k softmax mix of embedding rows: the next-iteration input of a hard token, gfx950.
+//
+//   out[row] = sum_j softmax(top-k logits of the row)_j * embedding[index_j]
+//
+// One workgroup (1024 threads) per row.  The row's logits (bf16) are loaded once into registers as
+// order-preserving 16-bit keys; the k-th largest key is found by bisection on the 16-bit key space with a
+// block-wide count per step (no histogram atomics, no sort), ties at the threshold are broken towards the
+// lower vocabulary index by a second bisection on the index, the <= k selected (index, value) pairs are
+// gathered into LDS and ordered by index (so that the float sums below have one fixed order), and the mix is
+// accumulated in float over bf16-rounded products, as the bf16 eager arithmetic it replaces rounds them.
+#include <hip/hip_runtime.h>
+
+#include "duo_device.h"
+#include "tah_duo.h"
+
+namespace tah {
+namespace {
+
+constexpr int kMixThreads = 1024;
+constexpr int kMixWaves = kMixThreads / kWave;
+constexpr int kMaxTopk = 256;
+constexpr int kMaxVec = 19;  // 16-byte pieces of the row per thread: vocabularies up to 19 * 8 * 1024 = 155648
+
+struct MixParams {
+    const __bf16* logits;
+    const __bf16* emb;
+    __bf16* out;
+    const uint8_t* row_enable;
+    int64_t l_rs, e_rs, o_rs;
+    int32_t rows, vocab, hidden, topk;
+};
+
+// bf16 bits -> unsigned key with the same order as the values (negative values reversed below the positive ones)
+__device__ __forceinline__ uint32_t order_key(uint32_t bits) { return (bits & 0x8000u) ? (~bits & 0xffffu) : (bits | 0x8000u); }
+__device__ __forceinline__ float key_value(uint32_t key) {
+    const uint32_t bits = (key & 0x8000u) ? (key & 0x7fffu) : (~key & 0xffffu);
+    return __uint_as_float(bits << 16);
+}
+
+// Sum of `x` over the workgroup, returned to every thread.  `red` holds kMixWaves ints; two barriers.
+__device__ __forceinline__ int block_sum(int x, int* red, int wave, int lane) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) x += __shfl_xor(x, m);
+    __syncthreads();  // earlier readers of red are done
+    if (lane == 0) red[wave] = x;
+    __syncthreads();
+    int t = 0;
+#pragma unroll
+    for (int w = 0; w < kMixWaves; ++w) t += red[w];
+    return t;
+}
+
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2e __attribute__((ext_vector_type(2)));
+// x rounded to bfloat16 (nearest even), as a float.  Through the packed conversion on purpose: a scalar
+// cast to __bf16 and back may be evaluated in excess precision, i.e. not round at all.
+__device__ __forceinline__ float round_bf16(float x) {
+    const f32x2 v = {x, 0.f};
+    return __uint_as_float(__builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2e)) << 16);
+}
+
+// NVEC: 16-byte pieces of the row per thread, a compile-time bound (the keys must stay in registers).
+template <int NVEC>
+__global__ __launch_bounds__(kMixThreads) void topk_mix_kernel(const MixParams p) {
+    __shared__ int red[kMixWaves];
+    __shared__ int sel_idx[kMaxTopk];
+    __shared__ float sel_val[kMaxTopk];
+    __shared__ int ord_idx[kMaxTopk];
+    __shared__ float ord_w[kMaxTopk];
+    __shared__ int n_sel;
+    HIP_DYNAMIC_SHARED(unsigned char, dyn)  // float partial sums of the mix: [parts][hidden]
+
+    const int row = blockIdx.x;
+    if (p.row_enable && !p.row_enable[row]) return;  // uniform per workgroup
+    const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    const int V = p.vocab;
+    const int k = p.topk < V ? p.topk : V;
+    const __bf16* lrow = p.logits + (int64_t)row * p.l_rs;
+
+    // ---- the row as keys: piece j of thread t covers indices (j * 1024 + t) * 8 .. + 7 (coalesced loads) ----
+    uint32_t keys[NVEC][4];  // two keys per dword, low half = even index
+    // loaded four pieces at a time and turned into keys in place, with a scheduling fence per group: left
+    // alone, the scheduler issues every load first and the row sits in registers twice (raw and as keys)
+    constexpr int kGroup = 4;
+#pragma unroll
+    for (int j0 = 0; j0 < NVEC; j0 += kGroup) {
+#pragma unroll
+        for (int j = j0; j < j0 + kGroup && j < NVEC; ++j) {
+            const int i0 = (j * kMixThreads + tid) * 8;
+            u32x4 w = {0u, 0u, 0u, 0u};
+            if (i0 + 8 <= V && ((reinterpret_cast<uintptr_t>(lrow + i0) & 15) == 0)) {
+                w = *reinterpret_cast<const u32x4*>(lrow + i0);
+            } else if (i0 < V) {
+                const uint16_t* h = reinterpret_cast<const uint16_t*>(lrow);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const uint32_t b = i0 + e < V ? h[i0 + e] : 0u;
+                    w[e / 2] |= b << (16 * (e % 2));
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                uint32_t lo = order_key(w[q] & 0xffffu), hi = order_key(w[q] >> 16);
+                // indices past the end get key 0 (below every real key) so that they are never selected
+                if (i0 + 2 * q >= V) lo = 0u;
+                if (i0 + 2 * q + 1 >= V) hi = 0u;
+                keys[j][q] = lo | (hi << 16);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    auto count_ge = [&](uint32_t t) {  // elements of this thread with key >= t
+        int c = 0;
+#pragma unroll
+        for (int j = 0; j < NVEC; ++j) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                uint32_t w = keys[j][q];
+                TAH_OPAQUE1(w);  // the two halves are split here, every time: hoisted out of the bisection
+                                 // loop they would double the registers the row occupies
+                c += ((w & 0xffffu) >= t) + ((w >> 16) >= t);
+            }
+        }
+        return c;
+    };
+
+    // ---- largest key T with count(key >= T) >= k: bisection, invariant count(>= lo) >= k > count(>= hi) ----
+    uint32_t lo = 1u, hi = 0x10000u;  // key 0 only marks indices past the end
+    while (hi - lo > 1) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (block_sum(count_ge(mid), red, wave, lane) >= k) lo = mid;
+        else hi = mid;
+    }
+    const uint32_t T = lo;
+    const int n_gt = block_sum(count_ge(T + 1), red, wave, lane);
+    const int need_eq = k - n_gt;  // >= 1: that many elements with key == T are taken, lowest indices first
+    // ---- smallest index bound M with count(key == T and index < M) >= need_eq ----
+    auto count_eq_below = [&](int m) {
+        int c = 0;
+#pragma unroll
+        for (int j = 0; j < NVEC; ++j) {
+            int d = m - (j * kMixThreads + tid) * 8;  // index e of this piece is below the bound iff e < d
+            TAH_OPAQUE1(d);                           // (compared with constants: no per-element index registers)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                uint32_t w = keys[j][q];
+                TAH_OPAQUE1(w);
+                c += ((w & 0xffffu) == T) && (2 * q < d);
+                c += ((w >> 16) == T) && (2 * q + 1 < d);
+            }
+        }
+        return c;
+    };
+    int mlo = 0, mhi = V;  // invariant: count(< mlo) < need_eq <= count(< mhi)
+    while (mhi - mlo > 1) {
+        const int mid = (mlo + mhi) >> 1;
+        if (block_sum(count_eq_below(mid), red, wave, lane) >= need_eq) mhi = mid;
+        else mlo = mid;
+    }
+    const int M = mhi;
+
+    // ---- gather the k selected (index, value) pairs ----
+    if (tid == 0) n_sel = 0;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < NVEC; ++j) {
+        int i0 = (j * kMixThreads + tid) * 8;
+        TAH_OPAQUE1(i0);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            uint32_t w = keys[j][e / 2];
+            TAH_OPAQUE1(w);
+            const uint32_t key = (w >> (16 * (e % 2))) & 0xffffu;
+            if (key > T || (key == T && e < M - i0)) {
+                const int s = atomicAdd(&n_sel, 1);
+                if (s < kMaxTopk) {
+                    sel_idx[s] = i0 + e;
+                    sel_val[s] = key_value(key);
+                }
+            }
+        }
+    }
+    __syncthreads();
+    const int n = n_sel < kMaxTopk ? n_sel : kMaxTopk;  // == k
+    // order by index (all distinct): rank = number of selected entries with a smaller index
+    float vmax = kNegInf;
+    for (int i = 0; i < n; ++i) vmax = fmaxf(vmax, sel_val[i]);
+    if (tid < n) {
+        int rank = 0;
+        for (int i = 0; i < n; ++i) rank += sel_idx[i] < sel_idx[tid];
+        ord_idx[rank] = sel_idx[tid];
+        ord_w[rank] = fast_exp2((sel_val[tid] - vmax) * kLog2e);
+    }
+    __syncthreads();
+    float denom = 0.f;
+    for (int i = 0; i < n; ++i) denom += ord_w[i];  // same order in every thread and every run
+    const float inv = 1.0f / denom;
+
+    // ---- mix: thread = (part, column group of 8); a part takes every parts-th selected row ----
+    const int H = p.hidden, cgs = H / 8;
+    float* partial = reinterpret_cast<float*>(dyn);
+    const int parts = cgs >= kMixThreads ? 1 : kMixThreads / cgs;
+    for (int cg0 = 0; cg0 < cgs; cg0 += kMixThreads) {
+        const int part = cgs >= kMixThreads ? 0 : tid / cgs;
+        const int cg = cg0 + (cgs >= kMixThreads ? tid : tid % cgs);
+        float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if (cg < cgs && part < parts) {
+            for (int i = part; i < n; i += parts) {
+                // probability rounded to bf16 (softmax output of the bf16 arithmetic), product rounded to bf16
+                const float pr = round_bf16(ord_w[i] * inv);
+                const bf16x8 e = *reinterpret_cast<const bf16x8*>(p.emb + (int64_t)ord_idx[i] * p.e_rs + cg * 8);
+#pragma unroll
+                for (int c = 0; c < 8; ++c) acc[c] += round_bf16(pr * (float)e[c]);
+            }
+#pragma unroll
+            for (int c = 0; c < 8; ++c) partial[(int64_t)part * H + cg * 8 + c] = acc[c];
+        }
+        __syncthreads();
+        if (cg < cgs && part == 0) {
+            bf16x8 o;
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                float s = 0.f;
+                for (int q = 0; q < parts; ++q) s += partial[(int64_t)q * H + cg * 8 + c];
+                o[c] = (__bf16)s;
+            }
+            *reinterpret_cast<bf16x8*>(p.out + (int64_t)row * p.o_rs + cg * 8) = o;
+        }
+        __syncthreads();
+    }
+}
+
+}  // namespace
+}  // namespace tah
+
+extern "C" int tah_topk_mix(const tah_topk_mix_args* a, tah_stream_t stream) {
+    using namespace tah;
+    if (!a) return TAH_E_NULL;
+    if (a->rows < 0 || a->vocab <= 0 || a->hidden <= 0 || a->topk <= 0) return TAH_E_SHAPE;
+    if (a->topk > kMaxTopk || a->vocab > kMaxVec * 8 * kMixThreads || a->hidden % 8 != 0) return TAH_E_SHAPE;
+    if (a->rows == 0) return TAH_OK;
+    if (!a->logits || !a->embedding || !a->out) return TAH_E_NULL;
+    if ((reinterpret_cast<uintptr_t>(a->embedding) & 15) || (reinterpret_cast<uintptr_t>(a->out) & 15) ||
+        (reinterpret_cast<uintptr_t>(a->logits) & 1) || a->embedding_row_stride % 8 || a->out_row_stride % 8)
+        return TAH_E_ALIGN;
+    MixParams p;
+    p.logits = static_cast<const __bf16*>(a->logits);
+    p.emb = static_cast<const __bf16*>(a->embedding);
+    p.out = static_cast<__bf16*>(a->out);
+    p.row_enable = a->row_enable;
+    p.l_rs = a->logits_row_stride; p.e_rs = a->embedding_row_stride; p.o_rs = a->out_row_stride;
+    p.rows = a->rows; p.vocab = a->vocab; p.hidden = a->hidden; p.topk = a->topk;
+    const int cgs = a->hidden / 8;
+    const int parts = cgs >= kMixThreads ? 1 : kMixThreads / cgs;
+    const size_t smem = (size_t)parts * a->hidden * sizeof(float);
+    if (smem > 48 * 1024) return TAH_E_SHAPE;  // (32 KiB whenever hidden < 8192)
+    const int nvec = (a->vocab + 8 * kMixThreads - 1) / (8 * kMixThreads);
+    const dim3 grid(a->rows), block(kMixThreads);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (nvec <= 2) hipLaunchKernelGGL(topk_mix_kernel<2>, grid, block, smem, st, p);
+    else if (nvec <= 8) hipLaunchKernelGGL(topk_mix_kernel<8>, grid, block, smem, st, p);
+    else if (nvec <= 14) hipLaunchKernelGGL(topk_mix_kernel<14>, grid, block, smem, st, p);
+    else hipLaunchKernelGGL(topk_mix_kernel<kMaxVec>, grid, block, smem, st, p);
+    return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
+}

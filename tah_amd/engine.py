@@ -22,7 +22,7 @@ depth-0 logits are the running sum (``additive_logits_update``, tah_model.py:78-
 last hidden state (a two-layer MLP, hidden -> 512 -> 1, sigmoid, threshold -- the form the end-to-end
 workload names; the reference's ``MLPIterDecider`` is a larger network over several layers,
 iter_decider.py:193-301); hard rows get the top-k softmax mix of embedding rows as their next input
-(``topk_softmax_input_update``, tah_model.py:57-75) at the same position (tah_model.py:618), see the depth-0
+(``topk_softmax_input_update``, tah_model.py:57-75; here one ``tah_topk_mix`` launch) at the same position (tah_model.py:618), see the depth-0
 and depth-1 caches, and their final logits are the sum of both iterations' logits.  LoRA adapters on the
 second iteration (tah_model.py:581) are not modelled: both iterations use the same weights.
 """
@@ -125,15 +125,6 @@ def rope_tables(max_len: int, head_dim: int, theta: float, device, dtype=torch.b
     return emb.cos().to(dtype).to(device), emb.sin().to(dtype).to(device)
 
 
-def topk_softmax_mix(logits: torch.Tensor, embedding: torch.Tensor, topk: int) -> torch.Tensor:
-    """Next-iteration input of a hard token (tah_model.py:57-75): softmax over the top-k logits, weighted sum of
-    the corresponding embedding rows, in the embedding's dtype."""
-    k = min(topk, logits.shape[-1])
-    val, idx = torch.topk(logits, k=k, dim=-1)
-    prob = torch.softmax(val, dim=-1)
-    return torch.sum(prob.unsqueeze(-1) * embedding[idx], dim=-2).to(embedding.dtype)
-
-
 class TaHDecodeEngine:
     def __init__(self, weights: Weights, batch: int, max_len: int, *, max_hard: Optional[int] = None, device="cuda"):
         cfg = weights.cfg
@@ -170,8 +161,7 @@ class TaHDecodeEngine:
 
     def _mlp(self, x, L):
         gu = self._rms(x, L["ln2"]) @ L["wgu"].t()
-        I = self.cfg.intermediate
-        return x + (F.silu(gu[:, :I]) * gu[:, I:]) @ L["wdown"].t()
+        return torch.addmm(x, ops.silu_mul(gu), L["wdown"].t())
 
     def _split_qkv(self, qkv):
         c = self.cfg
@@ -196,10 +186,10 @@ class TaHDecodeEngine:
             q, k, v = self._split_qkv(qkv)
             cache = self.slabs0[l] if depth == 0 else self.slabs1[l]
             qo, _ = qk_norm_rope(q, k, L["qn"], L["kn"], cos, sin, c.rms_eps, v=v, cache=cache, cu_new=self.cu_rows,
-                                 slot_of=slot_of, pos_new=pos if depth == 1 else None)
+                                 slot_of=slot_of, pos_new=pos if depth == 1 else None, one_row_per_seq=True)
             o = _decode(qo, self.rows, q_pos, self.slabs0[l], self.slabs1[l], scale=self.scale, q_depth=q_depth,
                         static_scratch=self.static_scratch)
-            x = x + o.view(x.shape[0], c.hq * c.head_dim) @ L["wo"].t()
+            x = torch.addmm(x, o.view(x.shape[0], c.hq * c.head_dim), L["wo"].t())  # residual add in the GEMM
             x = self._mlp(x, L)
         return self._rms(x, self.w.norm)
 
@@ -218,7 +208,8 @@ class TaHDecodeEngine:
         l0 = (h0 @ self.w.lm_head.t()).float()
         hard = (self.decide(h0) > self.w.threshold) if force_hard is None else force_hard
         hard = hard & act
-        x1 = topk_softmax_mix(l0.to(self.w.embed.dtype), self.w.embed, self.cfg.topk)
+        # next-iteration input of the hard rows (tah_model.py:693-697); the other rows keep zeros
+        x1 = ops.topk_mix(l0.to(self.w.embed.dtype), self.w.embed, self.cfg.topk, row_enable=hard)
         slot1 = torch.where(hard, self.rows, self.minus1)
         qpos1 = torch.where(hard, pos, self.minus1)
         h1 = self._pass_single(x1, pos, 1, slot1, qpos1, hard.to(torch.int32))
@@ -275,7 +266,7 @@ class TaHDecodeEngine:
                 raise TahDuoError("more hard tokens in a prompt than the depth-1 cache holds")
             cu2 = torch.cat([torch.zeros(1, dtype=torch.long, device=dev), counts.cumsum(0)]).to(torch.int32)
             l0h = h0[rows2] @ w.lm_head.t()
-            x2 = topk_softmax_mix(l0h, w.embed, c.topk)
+            x2 = ops.topk_mix(l0h, w.embed, c.topk)
             pos2 = pos[rows2].contiguous()
             cos2, sin2 = self.cos[pos2.long()], self.sin[pos2.long()]
             for l, L in enumerate(w.layers):

@@ -74,7 +74,7 @@ def qk_norm_rope(q: torch.Tensor, k: torch.Tensor, q_weight: torch.Tensor, k_wei
                  cos: torch.Tensor, sin: torch.Tensor, eps: float, *, v: Optional[torch.Tensor] = None,
                  cache: Optional[KvSlabs] = None, cu_new: Optional[torch.Tensor] = None,
                  pos_new: Optional[torch.Tensor] = None, slot_of: Optional[torch.Tensor] = None,
-                 in_place: bool = False):
+                 in_place: bool = False, one_row_per_seq: bool = False):
     """Per-head RMSNorm of q and k, rotary embedding of both and, with ``cache``, the KV append, in one
     kernel: the steps of ``Qwen3Attention.forward`` between the projections and the attention call
     (``q_norm``, ``k_norm``, ``apply_rotary_pos_emb``, ``past_key_values.update``), with bf16 roundings
@@ -83,7 +83,8 @@ def qk_norm_rope(q: torch.Tensor, k: torch.Tensor, q_weight: torch.Tensor, k_wei
     q ``[rows, Hq, 128]``, k / v ``[rows, Hkv, 128]`` (token-major, as the projections produce them),
     weights ``[128]``, cos / sin ``[rows, 128]``, all bf16.  Returns ``(q_out, k_out)``; with ``cache``
     K and V go to the slabs (rows ``[cu_new[i], cu_new[i+1])`` to slot ``slot_of[i]``) and ``k_out`` is
-    ``None``."""
+    ``None``.  ``one_row_per_seq=True`` (a decode step: every sequence brings at most one row, all slots
+    different) lets the same launch advance the slab lengths."""
     lib = _lib.lib()
     _thd(q, "q"), _thd(k, "k")
     _dev_check(q, k, v, q_weight, k_weight, cos, sin, cu_new, pos_new, slot_of, cache.k if cache is not None else None)
@@ -118,6 +119,7 @@ def qk_norm_rope(q: torch.Tensor, k: torch.Tensor, q_weight: torch.Tensor, k_wei
             raise _capi.TahDuoError("pos_new must be given exactly for slabs created with_pos=True")
         _i32(cu_new, "cu_new")
         a.append = 1
+        a.append_one_row_per_seq = 1 if one_row_per_seq else 0
         a.cu_new, a.slot_of, a.pos_new = cu_new.data_ptr(), _ptr(slot_of), _ptr(pos_new)
         a.nseq = cu_new.numel() - 1
         a.cache = cache.segment()

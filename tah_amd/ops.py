@@ -269,3 +269,45 @@ def rows_copy(src: torch.Tensor, src_rows: Optional[torch.Tensor], dst: torch.Te
     dstride = (dst.stride(0) if dst.shape[0] > 1 else dst[0].numel()) * dst.element_size()
     _capi.check(lib, lib.tah_rows_copy(src.data_ptr(), _ptr(src_rows), dst.data_ptr(), _ptr(dst_rows), _ptr(dst_enable), n,
                                        row_bytes, sstride, dstride, _stream(src)), "tah_rows_copy")
+
+
+def topk_mix(logits: torch.Tensor, embedding: torch.Tensor, topk: int, row_enable: Optional[torch.Tensor] = None,
+             out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Soft input embedding of hard tokens (tah_model.py:57-75): logits bf16 [rows, V] -> bf16 [rows, H], the
+    softmax over each row's top-k logits times the matching rows of ``embedding`` [V, H].  ``row_enable``
+    (bool/uint8 [rows]): rows with 0 are skipped and keep what ``out`` held."""
+    lib = _lib.lib()
+    _dev_check(logits, embedding, row_enable, out)
+    if logits.dim() != 2 or embedding.dim() != 2 or logits.dtype != torch.bfloat16 or embedding.dtype != torch.bfloat16:
+        raise _capi.TahDuoError("topk_mix: logits [rows, V] and embedding [V, H] must be bf16")
+    if logits.shape[1] != embedding.shape[0] or logits.stride(1) != 1 or embedding.stride(1) != 1:
+        raise _capi.TahDuoError("topk_mix: vocabulary sizes differ or the inner dimension is not contiguous")
+    rows, H = logits.shape[0], embedding.shape[1]
+    if out is None:
+        out = torch.zeros((rows, H), dtype=embedding.dtype, device=logits.device) if row_enable is not None else \
+            torch.empty((rows, H), dtype=embedding.dtype, device=logits.device)
+    if out.shape != (rows, H) or out.dtype != embedding.dtype or out.stride(1) != 1:
+        raise _capi.TahDuoError("topk_mix: out must be bf16 [rows, H]")
+    if row_enable is not None and (row_enable.dtype not in (torch.bool, torch.uint8) or row_enable.numel() != rows
+                                   or not row_enable.is_contiguous()):
+        raise _capi.TahDuoError("topk_mix: row_enable must be a contiguous bool/uint8 [rows] tensor")
+    a = _capi.TopkMixArgs()
+    a.logits, a.embedding, a.out, a.row_enable = _ptr(logits), _ptr(embedding), _ptr(out), _ptr(row_enable)
+    a.logits_row_stride = logits.stride(0) if rows > 1 else logits.shape[1]
+    a.embedding_row_stride, a.out_row_stride = embedding.stride(0), (out.stride(0) if rows > 1 else H)
+    a.rows, a.vocab, a.hidden, a.topk = rows, logits.shape[1], H, int(topk)
+    _capi.check(lib, lib.tah_topk_mix(ctypes.byref(a), _stream(logits)), "tah_topk_mix")
+    return out
+
+
+def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
+    """``silu(gate) * up`` of a fused gate|up projection, bf16 [rows, 2*I] -> [rows, I], in one launch."""
+    lib = _lib.lib()
+    _dev_check(gate_up)
+    if gate_up.dim() != 2 or gate_up.dtype != torch.bfloat16 or gate_up.shape[1] % 16 or gate_up.stride(1) != 1:
+        raise _capi.TahDuoError("silu_mul: gate_up must be bf16 [rows, 2*I] with I a multiple of 8 and a contiguous inner dimension")
+    rows, inter = gate_up.shape[0], gate_up.shape[1] // 2
+    out = torch.empty((rows, inter), dtype=gate_up.dtype, device=gate_up.device)
+    _capi.check(lib, lib.tah_silu_mul(_ptr(gate_up), _ptr(out), rows, inter, gate_up.stride(0) if rows > 1 else 2 * inter,
+                                      inter, _stream(gate_up)), "tah_silu_mul")
+    return out

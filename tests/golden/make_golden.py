@@ -133,11 +133,29 @@ def qk_prep():
         transformers_version=np.array(__import__("transformers").__version__))
 
 
+def topk_mix():
+    """Top-k softmax mix (tah_model.py:57-75): distinct logits, so that torch's own topk / softmax / sum in bf16
+    (the reference's call sequence, library routines) and the oracle name the same rows; the fixture keeps the
+    oracle's output after the two agree to one bf16 step."""
+    from oracle.topk_mix_ref import topk_mix as ref
+    from tests.topk_mix_cases import make_case
+
+    logits, emb = make_case(4247, 3, 1200, 48, distinct=True)
+    k = 100
+    out = ref(logits, emb, k)
+    lg, em = torch.from_numpy(logits).to(torch.bfloat16), torch.from_numpy(emb).to(torch.bfloat16)
+    tv, ti = torch.topk(lg, k=k, dim=-1)
+    lib = torch.sum(torch.softmax(tv, -1).unsqueeze(-1) * em[ti], dim=-2).to(em.dtype).float().numpy()
+    assert (np.abs(out - lib) <= np.maximum(np.abs(lib), 1e-3) * 2.0 ** -7).all() and (out == lib).mean() > 0.9
+    np.savez_compressed(os.path.join(HERE, "topk_mix_small.npz"), logits=logits, emb=emb, k=np.int32(k), out=out)
+
+
 if __name__ == "__main__":
     prefill()
     decode()
     pack()
     qk_prep()
+    topk_mix()
     for f in sorted(os.listdir(HERE)):
         if f.endswith(".npz"):
             print(f, os.path.getsize(os.path.join(HERE, f)), "bytes")

@@ -1,0 +1,107 @@
+"""tah_topk_mix (top-k softmax mix of embedding rows, tah_model.py:57-75) against its oracle: on the CPU
+execution build of the kernel, and on the GPU through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from oracle.topk_mix_ref import topk_mix as ref_mix
+from tests import emu_util
+from tests.topk_mix_cases import make_case, to_torch
+
+GOLDEN = __import__("os").path.join(__import__("os").path.dirname(__file__), "golden", "topk_mix_small.npz")
+
+
+def _check(got, want):
+    got = got.float().cpu().numpy()
+    tol = np.maximum(np.abs(want), 1e-3) * 2.0 ** -7  # one bf16 step: exp2-based softmax vs exp
+    assert (np.abs(got - want) <= tol).all(), float(np.abs(got - want).max())
+    assert (got == want).mean() > 0.97
+
+
+def _run(device, seed, rows, V, H, k, **kw):
+    from tah_amd import ops
+    logits, emb = make_case(seed, rows, V, H, **kw)
+    out = ops.topk_mix(to_torch(logits, device), to_torch(emb, device), k)
+    _check(out, ref_mix(logits, emb, k))
+
+
+@pytest.mark.skipif(not emu_util.have_host_clang(), reason="host clang++ not available")
+@pytest.mark.parametrize("seed,rows,V,H,k,kw", [
+    (0, 2, 700, 64, 100, {}), (1, 1, 9000, 32, 17, dict(ties=0.05)), (2, 2, 90, 16, 100, {}), (3, 1, 17000, 256, 100, {}),
+    (4, 1, 1003, 8, 256, dict(ties=0.3)),
+])
+def test_topk_mix_on_cpu_shim(seed, rows, V, H, k, kw):
+    with emu_util.emulated():
+        _run("cpu", seed, rows, V, H, k, **kw)
+
+
+@pytest.mark.skipif(not emu_util.have_host_clang(), reason="host clang++ not available")
+def test_topk_mix_golden_and_row_enable_on_cpu_shim():
+    from tah_amd import ops
+    z = np.load(GOLDEN)
+    with emu_util.emulated():
+        out = ops.topk_mix(to_torch(z["logits"], "cpu"), to_torch(z["emb"], "cpu"), int(z["k"]))
+        assert np.array_equal(out.float().numpy(), z["out"])
+        en = torch.tensor([1, 0, 1], dtype=torch.uint8)
+        keep = torch.full((3, z["emb"].shape[1]), 7.0, dtype=torch.bfloat16)
+        ops.topk_mix(to_torch(z["logits"], "cpu"), to_torch(z["emb"], "cpu"), int(z["k"]), row_enable=en, out=keep)
+    assert np.array_equal(keep[0].float().numpy(), z["out"][0]) and (keep[1] == 7).all()
+
+
+def test_oracle_reproduces_golden():
+    z = np.load(GOLDEN)
+    assert np.array_equal(ref_mix(z["logits"], z["emb"], int(z["k"])), z["out"])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed,rows,V,H,k,kw", [
+    (10, 32, 151936, 2048, 100, {}),                 # the end-to-end workload's shape
+    (11, 5, 151936, 2048, 100, dict(ties=0.02)),     # thousands of equal logits around the 100th place
+    (12, 3, 50000, 256, 1, {}), (13, 4, 777, 64, 100, dict(ties=0.2)), (14, 2, 64, 128, 100, {}), (15, 7, 20001, 1024, 256, {}),
+])
+def test_topk_mix_gpu(seed, rows, V, H, k, kw):
+    print(f"topk_mix case seed={seed} rows={rows} V={V} H={H} k={k} {kw}", flush=True)
+    _run("cuda", seed, rows, V, H, k, **kw)
+
+
+@pytest.mark.gpu
+def test_topk_mix_gpu_vs_torch_ops_on_device_and_strided_logits():
+    """Against the reference's call sequence in torch on the device (distinct values: no tie to break), with the
+    logits a strided slice of a larger buffer."""
+    from tah_amd import ops
+    logits, emb = make_case(20, 6, 4001, 512, distinct=True)
+    buf = torch.zeros(6, 4100, dtype=torch.bfloat16, device="cuda")
+    buf[:, 3:4004] = to_torch(logits, "cuda")
+    lg, em = buf[:, 3:4004], to_torch(emb, "cuda")
+    out = ops.topk_mix(lg, em, 100)
+    tv, ti = torch.topk(lg, k=100, dim=-1)
+    want = torch.sum(torch.softmax(tv, -1).unsqueeze(-1) * em[ti], dim=-2).to(em.dtype)
+    _check(out, want.float().cpu().numpy())
+    z = np.load(GOLDEN)
+    out = ops.topk_mix(to_torch(z["logits"], "cuda"), to_torch(z["emb"], "cuda"), int(z["k"]))
+    assert np.array_equal(out.float().cpu().numpy(), z["out"])
+
+
+def _silu_mul_check(device):
+    """tah_silu_mul against torch's own silu and product in bf16 (the eager modules' arithmetic; a library routine)."""
+    import torch.nn.functional as F
+
+    from tah_amd import ops
+    g = torch.Generator().manual_seed(3)
+    gu = (torch.randn(5, 2 * 1536, generator=g) * 2).to(torch.bfloat16).to(device)
+    got = ops.silu_mul(gu)
+    want = F.silu(gu[:, :1536]) * gu[:, 1536:]
+    d = (got.float() - want.float()).abs()
+    assert (d <= want.float().abs() * 2.0 ** -7 + 1e-30).all()  # exp2-based sigmoid: at most one bf16 step
+    assert (got == want).float().mean() > 0.98
+
+
+@pytest.mark.skipif(not emu_util.have_host_clang(), reason="host clang++ not available")
+def test_silu_mul_on_cpu_shim():
+    with emu_util.emulated():
+        _silu_mul_check("cpu")
+
+
+@pytest.mark.gpu
+def test_silu_mul_gpu():
+    _silu_mul_check("cuda")
