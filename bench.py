@@ -229,11 +229,10 @@ def bench_e2e_decode(new_tokens: int, B: int = 32, prompt_len: int = 512):
     import torch
 
     from tah_amd.engine import EngineConfig, TaHDecodeEngine, Weights
-    from tah_amd.kv_cache import decode as kv_decode, qk_norm_rope
 
     cfg = EngineConfig()
     w = Weights.random_init(cfg, "cuda", seed=1239)
-    eng = TaHDecodeEngine(w, B, prompt_len + new_tokens + 8, max_hard=prompt_len // 4 + new_tokens + 8, device="cuda")
+    eng = TaHDecodeEngine(w, B, prompt_len + new_tokens + 8, device="cuda")
     g = torch.Generator().manual_seed(1239)
     ids = torch.randint(0, cfg.vocab, (B * prompt_len,), generator=g).cuda()
     cu = torch.arange(0, B * prompt_len + 1, prompt_len, dtype=torch.int32, device="cuda")
@@ -269,32 +268,22 @@ def bench_e2e_decode(new_tokens: int, B: int = 32, prompt_len: int = 512):
     torch.cuda.synchronize()
     step_ms = e0.elapsed_time(e1) / n
     frac_hard = (int(eng.n_hard) - hard0) / max(int(eng.n_steps) - steps0, 1)
-    # the duo-causal attention part of a step on the final cache: q/k preparation + decode kernels of all
-    # layers for both latent iterations (no append, so the cache stays as it is), replayed as a graph
-    pos = eng.pos - 1
-    cos, sin = eng.cos[pos.long()], eng.sin[pos.long()]
-    qkv = torch.randn(B, cfg.hq + 2 * cfg.hkv, cfg.head_dim, device="cuda").to(torch.bfloat16)
-    hard_rows = torch.rand(B, device="cuda") < frac_hard
-    qpos1 = torch.where(hard_rows, pos, eng.minus1)
-
-    def attn_only():
-        for l, L in enumerate(w.layers):
-            for depth in (0, 1):
-                qo, _ = qk_norm_rope(qkv[:, :cfg.hq], qkv[:, cfg.hq:cfg.hq + cfg.hkv], L["qn"], L["kn"], cos, sin, cfg.rms_eps)
-                kv_decode(qo, eng.rows, pos if depth == 0 else qpos1, eng.slabs0[l], eng.slabs1[l], scale=eng.scale,
-                          q_depth=eng.zeros_i if depth == 0 else hard_rows.to(torch.int32), static_scratch=True)
-
-    attn_only()
-    ga = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(ga):
-        attn_only()
+    # the duo-causal attention part of a step: the same captured step with the q/k preparation and decode
+    # kernels of all layers and both latent iterations left out, replayed on the final cache; the difference
+    # is what those kernels cost inside the step
+    eng.measure_without_attention = True
+    eng._graph = None
+    g0 = eng.capture(0.0, -1)
     torch.cuda.synchronize()
     e0.record()
-    for _ in range(50):
-        ga.replay()
+    for _ in range(30):
+        g0.replay()
     e1.record()
     torch.cuda.synchronize()
-    attn_ms = e0.elapsed_time(e1) / 50
+    without_ms = e0.elapsed_time(e1) / 30
+    eng.measure_without_attention = False
+    eng._graph = None
+    attn_ms = max(step_ms - without_ms, 0.0)
     ctx = float(eng.pos.float().mean())
     attn_bytes = cfg.layers * B * ctx * 2 * cfg.hkv * cfg.head_dim * 2
     params = sum(t.numel() for L in w.layers for t in L.values()) + w.embed.numel() + w.norm.numel()
@@ -304,6 +293,7 @@ def bench_e2e_decode(new_tokens: int, B: int = 32, prompt_len: int = 512):
             "tokens_per_s": B / (step_ms * 1e-3), "ms_per_step": step_ms, "steps_timed": n,
             "hard_fraction_decode": frac_hard, "hard_fraction_prompt": float(hard.float().mean()),
             "attention_ms_per_step": attn_ms, "attention_share_of_step": attn_ms / step_ms,
+            "step_ms_without_attention_kernels": without_ms,
             "attention_kernels": "qk_prep_kernel + duo_decode_split_kernel<2> + duo_decode_merge_kernel, 28 layers x 2 iterations",
             "attention_cache_bytes_per_step": attn_bytes, "attention_cache_gbs": attn_bytes / (attn_ms * 1e-3) / 1e9,
             "host_ms_per_step_graph": host_s / n * 1e3, "eager_ms_per_step": eager_s * 1e3,

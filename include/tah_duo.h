@@ -291,19 +291,22 @@ int tah_hard_index_build(const uint8_t* mask, int32_t B, int32_t S, int32_t* pos
                          int32_t* seq_out, int32_t* cu_out, tah_stream_t stream);
 
 /* Destination rows of the right-padded (B, width) form used by gather_active
- * (tah/model/tah_model.py:117-134): out[r] = seq_of[r]*width + (r - cu[seq_of[r]]). */
-int tah_pad_rows_build(const int32_t* cu, const int32_t* seq_of, int32_t n, int32_t width, int32_t* out,
-                       tah_stream_t stream);
+ * (tah/model/tah_model.py:117-134): out[r] = seq_of[r]*width + (r - cu[seq_of[r]]) for r < n.  When n_dev is
+ * given (a device int32, e.g. &cu[B] as tah_hard_index_build wrote it) only the first min(n, *n_dev) entries
+ * are produced, so that a caller that never reads the count back can pass an upper bound as n.  An entry
+ * whose rank inside its row is >= width gets -1 (tah_rows_copy skips it) and sets *overflow (optional). */
+int tah_pad_rows_build(const int32_t* cu, const int32_t* seq_of, int32_t n, const int32_t* n_dev, int32_t width,
+                       int32_t* out, int32_t* overflow, tah_stream_t stream);
 
 /* Row gather / scatter: dst[dst_rows ? dst_rows[r] : r] = src[src_rows ? src_rows[r] : r]
- * for r < n, rows of row_bytes bytes at the given byte strides; when dst_enable
- * is given (one byte per destination row) rows whose byte is 0 are left
- * untouched -- the assignment_mask of scatter_back.  Replaces torch.gather
- * (tah_model.py:127-133) and the boolean-mask index_put (tah_model.py:163-175).
- * Rows named twice in dst_rows race.  Bit-exact. */
+ * for r < n (and r < *n_dev when n_dev is given: the count stays on the device), rows of row_bytes bytes at
+ * the given byte strides; when dst_enable is given (one byte per destination row) rows whose byte is 0 are
+ * left untouched -- the assignment_mask of scatter_back; a negative row index skips the entry.  Replaces
+ * torch.gather (tah_model.py:127-133) and the boolean-mask index_put (tah_model.py:163-175), and with n_dev
+ * the host synchronisation of tah_model.py:116.  Rows named twice in dst_rows race.  Bit-exact. */
 int tah_rows_copy(const void* src, const int32_t* src_rows, void* dst, const int32_t* dst_rows,
-                  const uint8_t* dst_enable, int32_t n, int64_t row_bytes, int64_t src_stride_bytes,
-                  int64_t dst_stride_bytes, tah_stream_t stream);
+                  const uint8_t* dst_enable, int32_t n, const int32_t* n_dev, int64_t row_bytes,
+                  int64_t src_stride_bytes, int64_t dst_stride_bytes, tah_stream_t stream);
 
 #ifdef __cplusplus
 }

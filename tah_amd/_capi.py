@@ -154,9 +154,9 @@ PROTOTYPES = {
     "tah_topk_mix": (C.c_int, [C.POINTER(TopkMixArgs), c_void_p]),
     "tah_silu_mul": (C.c_int, [c_void_p, c_void_p, c_int32, c_int32, c_int64, c_int64, c_void_p]),
     "tah_hard_index_build": (C.c_int, [c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
-    "tah_pad_rows_build": (C.c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_void_p]),
-    "tah_rows_copy": (C.c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int64,
-                                c_void_p]),
+    "tah_pad_rows_build": (C.c_int, [c_void_p, c_void_p, c_int32, c_void_p, c_int32, c_void_p, c_void_p, c_void_p]),
+    "tah_rows_copy": (C.c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_int64, c_int64,
+                                c_int64, c_void_p]),
 }
 
 

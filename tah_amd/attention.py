@@ -184,25 +184,30 @@ def _rows(x: torch.Tensor) -> torch.Tensor:
 
 
 class _Packed:
-    """Valid-row packing of one (B, T) block: row ids, per-sequence offsets, int32 positions."""
+    """Valid-row packing of one (B, T) block: row ids, per-sequence offsets, int32 positions.
+
+    With ``tah_amd.pack.HOST_SYNC`` off nothing is read back from the device: packed tensors keep the full
+    B*T rows (zero beyond the valid count, so that a key tile never mixes in uninitialised rows), the kernels
+    find the real extent in ``cu``, and the row copies stop at the count held on the device."""
 
     def __init__(self, valid: Optional[torch.Tensor], pos: Optional[torch.Tensor], B: int, T: int, device):
         self.B, self.T = B, T
+        self.n_dev = None
         all_valid = valid is None
         if not all_valid:
             idx = HardIndex(valid)
-            all_valid = idx.n == B * T
+            all_valid = idx.synced and idx.n == B * T
         if all_valid:
             self.rows, self.n = None, B * T
             self.cu = torch.arange(0, (B + 1) * T, T, dtype=torch.int32, device=device)
         else:
-            self.rows, self.n, self.cu = idx.flat, idx.n, idx.cu
+            self.rows, self.n, self.cu, self.n_dev = idx.flat, idx.bound, idx.cu, idx.n_dev
         self.pos = None
         if pos is not None:
             p32 = pos.to(torch.int32).contiguous().view(B * T, 1)
             if self.rows is not None:
-                out = torch.empty((self.n, 1), dtype=torch.int32, device=device)
-                ops.rows_copy(p32, self.rows, out, None, self.n)
+                out = torch.zeros((self.n, 1), dtype=torch.int32, device=device)
+                ops.rows_copy(p32, self.rows, out, None, self.n, None, self.n_dev)
                 p32 = out
             self.pos = p32.view(-1)
 
@@ -210,47 +215,49 @@ class _Packed:
         r = _rows(x)
         if self.rows is None:
             return r
-        return _GatherRows.apply(r.contiguous(), self.rows, self.n)
+        return _GatherRows.apply(r.contiguous(), self.rows, self.n, self.n_dev)
 
     def unpack(self, o: torch.Tensor, Hq: int, D: int) -> torch.Tensor:
         """[n, Hq, D] -> (B, T, Hq, D) with zeros at rows that were not packed."""
         if self.rows is None:
             return o.view(self.B, self.T, Hq, D)
-        return _ScatterRows.apply(o, self.rows, self.n, self.B * self.T).view(self.B, self.T, Hq, D)
+        return _ScatterRows.apply(o, self.rows, self.n, self.B * self.T, self.n_dev).view(self.B, self.T, Hq, D)
 
 
 class _GatherRows(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, src, rows, n):
-        out = torch.empty((n,) + tuple(src.shape[1:]), dtype=src.dtype, device=src.device)
-        ops.rows_copy(src, rows, out, None, n)
-        ctx.save_for_backward(rows)
+    def forward(ctx, src, rows, n, n_dev=None):
+        alloc = torch.empty if n_dev is None else torch.zeros  # rows past a device-side count stay zero
+        out = alloc((n,) + tuple(src.shape[1:]), dtype=src.dtype, device=src.device)
+        ops.rows_copy(src, rows, out, None, n, None, n_dev)
+        ctx.save_for_backward(rows, n_dev)
         ctx.n, ctx.total = n, src.shape[0]
         return out
 
     @staticmethod
     def backward(ctx, g):
-        (rows,) = ctx.saved_tensors
+        rows, n_dev = ctx.saved_tensors
         gs = torch.zeros((ctx.total,) + tuple(g.shape[1:]), dtype=g.dtype, device=g.device)
-        ops.rows_copy(g.contiguous(), None, gs, rows, ctx.n)
-        return gs, None, None
+        ops.rows_copy(g.contiguous(), None, gs, rows, ctx.n, None, n_dev)
+        return gs, None, None, None
 
 
 class _ScatterRows(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, src, rows, n, total):
+    def forward(ctx, src, rows, n, total, n_dev=None):
         out = torch.zeros((total,) + tuple(src.shape[1:]), dtype=src.dtype, device=src.device)
-        ops.rows_copy(src.contiguous(), None, out, rows, n)
-        ctx.save_for_backward(rows)
+        ops.rows_copy(src.contiguous(), None, out, rows, n, None, n_dev)
+        ctx.save_for_backward(rows, n_dev)
         ctx.n = n
         return out
 
     @staticmethod
     def backward(ctx, g):
-        (rows,) = ctx.saved_tensors
-        gs = torch.empty((ctx.n,) + tuple(g.shape[1:]), dtype=g.dtype, device=g.device)
-        ops.rows_copy(g.contiguous(), rows, gs, None, ctx.n)
-        return gs, None, None, None
+        rows, n_dev = ctx.saved_tensors
+        alloc = torch.empty if n_dev is None else torch.zeros
+        gs = alloc((ctx.n,) + tuple(g.shape[1:]), dtype=g.dtype, device=g.device)
+        ops.rows_copy(g.contiguous(), rows, gs, None, ctx.n, None, n_dev)
+        return gs, None, None, None, None
 
 
 def _segment(cache: TaHDuoCache, layer_idx: int, depth: int, B: int, with_pos: bool):
@@ -329,26 +336,16 @@ def duo_attention_forward(module, query: torch.Tensor, key: torch.Tensor, value:
     # decode fast path: one query row per sequence, slabs hold every cached row (incl. this step's)
     s1 = cache.slabs(layer, 0)
     if Tq == 1 and s1 is not None and not (torch.is_grad_enabled() and query.requires_grad):
+        # every batch row is a query row; a row that is not valid (a pad row of the depth-1 pack, tah_model.py:116-118)
+        # gets position -1, sees nothing and comes back as zeros -- no index to build, nothing read back
         if m._packed is None:
-            idx = HardIndex(m.valid_mask)
-            qpos = torch.empty((max(idx.n, 1), 1), dtype=torch.int32, device=dev)
-            ops.rows_copy(m.position_ids.to(torch.int32).contiguous().view(B, 1), idx.flat, qpos, None, idx.n)
-            m._packed = (idx, qpos.view(-1)[: idx.n])
-        idx, qpos = m._packed
-        out = torch.zeros((B, 1, Hq, D), dtype=query.dtype, device=dev)
-        if idx.n:
-            q = _rows(query)
-            if idx.n != B:
-                qp = torch.empty((idx.n, Hq, D), dtype=query.dtype, device=dev)
-                ops.rows_copy(q.contiguous(), idx.flat, qp, None, idx.n)
-                q = qp
-            o = kv_cache.decode(q, idx.flat if idx.n != B else torch.arange(B, dtype=torch.int32, device=dev), qpos,
-                                s1, cache.slabs(layer, 1) if depth >= 1 else None, scale=scale, depth=depth)
-            if idx.n != B:
-                ops.rows_copy(o, None, out.view(B, Hq, D), idx.flat, idx.n)
-            else:
-                out = o.view(B, 1, Hq, D)
-        return out, None
+            pos32 = m.position_ids.to(torch.int32).reshape(B)
+            qpos = torch.where(m.valid_mask.reshape(B) != 0, pos32, torch.full_like(pos32, -1))
+            m._packed = (torch.arange(B, dtype=torch.int32, device=dev), qpos)
+        slots, qpos = m._packed
+        o = kv_cache.decode(_rows(query), slots, qpos, s1, cache.slabs(layer, 1) if depth >= 1 else None, scale=scale,
+                            depth=depth)
+        return o.view(B, 1, Hq, D), None
 
     # general path: packed varlen forward (+ backward through autograd)
     if m._packed is None:

@@ -82,37 +82,56 @@ class TaHDuoCache:
                 f"KV slabs of layer {slot[0]}, depth {slot[1]} hold {sl.capacity} rows per sequence; this write "
                 f"brings a sequence to as many as {written}: enable_slabs() with a larger capacity")
         self._slab_rows[slot] = written
+        if T == 1:
+            # a decode step: one row per sequence, appended in place from where it lies -- rows that are not
+            # valid (pad rows of the depth-1 pack) name slot -1 and are skipped; nothing is packed or read back
+            key = ("step", id(valid))
+            memo = self._pack_memo.get(key)
+            if memo is None or memo[0] is not valid:
+                rows = torch.arange(B, dtype=torch.int32, device=k.device)
+                slot_of = rows if valid is None else torch.where(valid.reshape(B) != 0, rows, torch.full_like(rows, -1))
+                cu1 = torch.arange(B + 1, dtype=torch.int32, device=k.device)
+                memo = (valid, slot_of, cu1)
+                self._pack_memo = {key: memo}
+            _, slot_of, cu1 = memo
+            pos_rows = pos.to(torch.int32).reshape(B).contiguous() if slot[1] > 0 else None
+            sl.append(k.transpose(1, 2).reshape(B, hkv, d), v.transpose(1, 2).reshape(B, hkv, d), cu1, pos_new=pos_rows,
+                      slot_of=slot_of)
+            return
         # one compaction of the valid mask per forward step, shared by all layers
         key = id(valid) if valid is not None else -T
         memo = self._pack_memo.get(key)
         if memo is None or memo[0] is not valid:
             if valid is None:
                 cu = torch.arange(0, (B + 1) * T, T, dtype=torch.int32, device=k.device)
-                memo = (valid, None, cu, B * T)
+                memo = (valid, None, cu, B * T, None)
             else:
                 idx = HardIndex(valid)
-                memo = (valid, idx.flat, idx.cu, idx.n)
+                if idx.synced and idx.n == B * T:
+                    memo = (valid, None, torch.arange(0, (B + 1) * T, T, dtype=torch.int32, device=k.device), B * T, None)
+                else:
+                    memo = (valid, idx.flat, idx.cu, idx.bound, idx.n_dev)
             self._pack_memo = {key: memo}
-        _, rows, cu, n = memo
+        _, rows, cu, n, n_dev = memo
         kt = k.transpose(1, 2).reshape(B * T, hkv, d)  # a view when k came from a (B,T,H,D) projection
         vt = v.transpose(1, 2).reshape(B * T, hkv, d)
         pos_rows = None
         if rows is not None:
             kp = torch.empty((n, hkv, d), dtype=k.dtype, device=k.device)
             vp = torch.empty((n, hkv, d), dtype=k.dtype, device=k.device)
-            ops.rows_copy(kt.contiguous(), rows, kp, None, n)
-            ops.rows_copy(vt.contiguous(), rows, vp, None, n)
+            ops.rows_copy(kt.contiguous(), rows, kp, None, n, None, n_dev)
+            ops.rows_copy(vt.contiguous(), rows, vp, None, n, None, n_dev)
             kt, vt = kp, vp
         if slot[1] > 0:
             p32 = pos.to(torch.int32).contiguous().view(B * T, 1)
             if rows is not None:
                 pos_rows = torch.empty((n, 1), dtype=torch.int32, device=k.device)
-                ops.rows_copy(p32, rows, pos_rows, None, n)
+                ops.rows_copy(p32, rows, pos_rows, None, n, None, n_dev)
             else:
                 pos_rows = p32
             pos_rows = pos_rows.view(-1)
         if n:
-            sl.append(kt, vt, cu, pos_new=pos_rows)
+            sl.append(kt, vt, cu, pos_new=pos_rows)  # (the append stops at cu[B]: n may be an upper bound)
 
     # ── write path (causal_cache.py:63-97) ────────────────────────────────
     def has_layer(self, layer_idx: int = 0) -> bool:

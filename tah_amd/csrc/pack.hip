@@ -71,22 +71,27 @@ __global__ __launch_bounds__(kScanThreads) void hard_index_kernel(const uint8_t*
     if (tid == 0) cu_out[B] = carry_s;
 }
 
-__global__ void pad_rows_kernel(const int32_t* cu, const int32_t* seq_of, int n, int width, int32_t* out) {
+__global__ void pad_rows_kernel(const int32_t* cu, const int32_t* seq_of, int n, const int32_t* n_dev, int width,
+                                int32_t* out, int32_t* overflow) {
     const int r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (n_dev && *n_dev < n) n = *n_dev;
     if (r < n) {
         const int b = seq_of[r];
-        out[r] = b * width + (r - cu[b]);
+        const int rank = r - cu[b];
+        out[r] = rank < width ? b * width + rank : -1;  // an entry that does not fit its row is dropped by the copy
+        if (rank >= width && overflow) *overflow = 1;
     }
 }
 
 template <typename V>
 __global__ void rows_copy_kernel(const unsigned char* src, const int32_t* src_rows, unsigned char* dst,
-                                 const int32_t* dst_rows, const uint8_t* dst_enable, int n, int vec_per_row,
-                                 int64_t src_stride, int64_t dst_stride, int row_base) {
+                                 const int32_t* dst_rows, const uint8_t* dst_enable, int n, const int32_t* n_dev,
+                                 int vec_per_row, int64_t src_stride, int64_t dst_stride, int row_base) {
     const int r = blockIdx.y;
-    if (r >= n) return;
+    if (r >= n || (n_dev && row_base + r >= *n_dev)) return;
     const int64_t sr = src_rows ? src_rows[r] : row_base + r;
     const int64_t dr = dst_rows ? dst_rows[r] : row_base + r;
+    if (sr < 0 || dr < 0) return;  // dropped entry (see pad_rows_kernel)
     if (dst_enable && !dst_enable[dr]) return;
     const V* s = reinterpret_cast<const V*>(src + sr * src_stride);
     V* d = reinterpret_cast<V*>(dst + dr * dst_stride);
@@ -97,7 +102,7 @@ struct alignas(16) V16 { uint32_t x[4]; };
 
 template <typename V>
 int launch_copy(const void* src, const int32_t* src_rows, void* dst, const int32_t* dst_rows, const uint8_t* dst_enable, int n,
-                int64_t row_bytes, int64_t src_stride, int64_t dst_stride, hipStream_t st) {
+                const int32_t* n_dev, int64_t row_bytes, int64_t src_stride, int64_t dst_stride, hipStream_t st) {
     const int vec = (int)(row_bytes / (int64_t)sizeof(V));
     int gx = (vec + 255) / 256;
     gx = gx < 1 ? 1 : (gx > 64 ? 64 : gx);
@@ -105,7 +110,7 @@ int launch_copy(const void* src, const int32_t* src_rows, void* dst, const int32
         const int nr = n - r0 < 65535 ? n - r0 : 65535;
         hipLaunchKernelGGL(rows_copy_kernel<V>, dim3(gx, nr), dim3(256), 0, st, static_cast<const unsigned char*>(src),
                            src_rows ? src_rows + r0 : nullptr, static_cast<unsigned char*>(dst),
-                           dst_rows ? dst_rows + r0 : nullptr, dst_enable, nr, vec, src_stride, dst_stride, r0);
+                           dst_rows ? dst_rows + r0 : nullptr, dst_enable, nr, n_dev, vec, src_stride, dst_stride, r0);
     }
     return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
 }
@@ -124,20 +129,20 @@ extern "C" int tah_hard_index_build(const uint8_t* mask, int32_t B, int32_t S, i
     return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
 }
 
-extern "C" int tah_pad_rows_build(const int32_t* cu, const int32_t* seq_of, int32_t n, int32_t width, int32_t* out,
-                                  tah_stream_t stream) {
+extern "C" int tah_pad_rows_build(const int32_t* cu, const int32_t* seq_of, int32_t n, const int32_t* n_dev, int32_t width,
+                                  int32_t* out, int32_t* overflow, tah_stream_t stream) {
     using namespace tah;
     if (n < 0 || width < 0) return TAH_E_SHAPE;
     if (n == 0) return TAH_OK;
     if (!cu || !seq_of || !out) return TAH_E_NULL;
     hipLaunchKernelGGL(pad_rows_kernel, dim3((n + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream), cu, seq_of, n,
-                       width, out);
+                       n_dev, width, out, overflow);
     return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
 }
 
 extern "C" int tah_rows_copy(const void* src, const int32_t* src_rows, void* dst, const int32_t* dst_rows,
-                             const uint8_t* dst_enable, int32_t n, int64_t row_bytes, int64_t src_stride_bytes,
-                             int64_t dst_stride_bytes, tah_stream_t stream) {
+                             const uint8_t* dst_enable, int32_t n, const int32_t* n_dev, int64_t row_bytes,
+                             int64_t src_stride_bytes, int64_t dst_stride_bytes, tah_stream_t stream) {
     using namespace tah;
     if (n < 0 || row_bytes < 0) return TAH_E_SHAPE;
     if (n == 0 || row_bytes == 0) return TAH_OK;
@@ -145,11 +150,11 @@ extern "C" int tah_rows_copy(const void* src, const int32_t* src_rows, void* dst
     hipStream_t st = static_cast<hipStream_t>(stream);
     const uintptr_t bits = reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst) | (uintptr_t)row_bytes |
                            (uintptr_t)src_stride_bytes | (uintptr_t)dst_stride_bytes;
-    if (bits % 16 == 0) return launch_copy<V16>(src, src_rows, dst, dst_rows, dst_enable, n, row_bytes, src_stride_bytes, dst_stride_bytes, st);
-    if (bits % 8 == 0) return launch_copy<uint64_t>(src, src_rows, dst, dst_rows, dst_enable, n, row_bytes, src_stride_bytes, dst_stride_bytes, st);
-    if (bits % 4 == 0) return launch_copy<uint32_t>(src, src_rows, dst, dst_rows, dst_enable, n, row_bytes, src_stride_bytes, dst_stride_bytes, st);
-    if (bits % 2 == 0) return launch_copy<uint16_t>(src, src_rows, dst, dst_rows, dst_enable, n, row_bytes, src_stride_bytes, dst_stride_bytes, st);
-    return launch_copy<uint8_t>(src, src_rows, dst, dst_rows, dst_enable, n, row_bytes, src_stride_bytes, dst_stride_bytes, st);
+    if (bits % 16 == 0) return launch_copy<V16>(src, src_rows, dst, dst_rows, dst_enable, n, n_dev, row_bytes, src_stride_bytes, dst_stride_bytes, st);
+    if (bits % 8 == 0) return launch_copy<uint64_t>(src, src_rows, dst, dst_rows, dst_enable, n, n_dev, row_bytes, src_stride_bytes, dst_stride_bytes, st);
+    if (bits % 4 == 0) return launch_copy<uint32_t>(src, src_rows, dst, dst_rows, dst_enable, n, n_dev, row_bytes, src_stride_bytes, dst_stride_bytes, st);
+    if (bits % 2 == 0) return launch_copy<uint16_t>(src, src_rows, dst, dst_rows, dst_enable, n, n_dev, row_bytes, src_stride_bytes, dst_stride_bytes, st);
+    return launch_copy<uint8_t>(src, src_rows, dst, dst_rows, dst_enable, n, n_dev, row_bytes, src_stride_bytes, dst_stride_bytes, st);
 }
 
 extern "C" int tah_duo_abi_version(void) { return TAH_DUO_ABI_VERSION; }

@@ -154,6 +154,7 @@ class TaHDecodeEngine:
         self.host_hard_rows = 0
         self._graph = None
         self.static_scratch = self.device.type == "cuda"
+        self.measure_without_attention = False
 
     # ── model pieces ─────────────────────────────────────────────────────
     def _rms(self, x, w):
@@ -161,7 +162,7 @@ class TaHDecodeEngine:
 
     def _mlp(self, x, L):
         gu = self._rms(x, L["ln2"]) @ L["wgu"].t()
-        return torch.addmm(x, ops.silu_mul(gu), L["wdown"].t())
+        return x.addmm_(ops.silu_mul(gu), L["wdown"].t())
 
     def _split_qkv(self, qkv):
         c = self.cfg
@@ -185,11 +186,14 @@ class TaHDecodeEngine:
             qkv = self._rms(x, L["ln1"]) @ L["wqkv"].t()
             q, k, v = self._split_qkv(qkv)
             cache = self.slabs0[l] if depth == 0 else self.slabs1[l]
-            qo, _ = qk_norm_rope(q, k, L["qn"], L["kn"], cos, sin, c.rms_eps, v=v, cache=cache, cu_new=self.cu_rows,
-                                 slot_of=slot_of, pos_new=pos if depth == 1 else None, one_row_per_seq=True)
-            o = _decode(qo, self.rows, q_pos, self.slabs0[l], self.slabs1[l], scale=self.scale, q_depth=q_depth,
-                        static_scratch=self.static_scratch)
-            x = torch.addmm(x, o.view(x.shape[0], c.hq * c.head_dim), L["wo"].t())  # residual add in the GEMM
+            if self.measure_without_attention:  # timing aid: the step minus its q/k preparation and decode kernels
+                o = q.contiguous()
+            else:
+                qo, _ = qk_norm_rope(q, k, L["qn"], L["kn"], cos, sin, c.rms_eps, v=v, cache=cache, cu_new=self.cu_rows,
+                                     slot_of=slot_of, pos_new=pos if depth == 1 else None, one_row_per_seq=True)
+                o = _decode(qo, self.rows, q_pos, self.slabs0[l], self.slabs1[l], scale=self.scale, q_depth=q_depth,
+                            static_scratch=self.static_scratch)
+            x = x.addmm_(o.view(x.shape[0], c.hq * c.head_dim), L["wo"].t())  # residual add inside the GEMM, in place
             x = self._mlp(x, L)
         return self._rms(x, self.w.norm)
 

@@ -237,23 +237,29 @@ def hard_index_build(mask: torch.Tensor):
     return pos, flat, seq, cu
 
 
-def pad_rows_build(cu: torch.Tensor, seq_of: torch.Tensor, n: int, width: int) -> torch.Tensor:
+def pad_rows_build(cu: torch.Tensor, seq_of: torch.Tensor, n: int, width: int, n_dev: Optional[torch.Tensor] = None,
+                   overflow: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Rows of the packed entries inside the right-padded (B, width) layout.  ``n_dev`` (device int32, one
+    element): only the first ``min(n, n_dev)`` entries are defined -- ``n`` may then be an upper bound."""
     lib = _lib.lib()
-    _dev_check(cu, seq_of)
+    _dev_check(cu, seq_of, n_dev, overflow)
     out = torch.empty(max(n, 1), dtype=torch.int32, device=cu.device)
-    _capi.check(lib, lib.tah_pad_rows_build(cu.data_ptr(), seq_of.data_ptr(), n, width, out.data_ptr(), _stream(cu)),
-                "tah_pad_rows_build")
+    _capi.check(lib, lib.tah_pad_rows_build(cu.data_ptr(), seq_of.data_ptr(), n, _ptr(n_dev), width, out.data_ptr(),
+                                            _ptr(overflow), _stream(cu)), "tah_pad_rows_build")
     return out[:n]
 
 
 def rows_copy(src: torch.Tensor, src_rows: Optional[torch.Tensor], dst: torch.Tensor,
-              dst_rows: Optional[torch.Tensor], n: int, dst_enable: Optional[torch.Tensor] = None) -> None:
+              dst_rows: Optional[torch.Tensor], n: int, dst_enable: Optional[torch.Tensor] = None,
+              n_dev: Optional[torch.Tensor] = None) -> None:
     """dst[dst_rows[r]] = src[src_rows[r]] for r < n; src/dst are [rows, ...] with contiguous rows.
 
     dst_enable (bool/uint8, one entry per row of dst): rows whose entry is 0 are left untouched.
+    n_dev (device int32, one element): entries r >= n_dev are skipped too, so ``n`` may be an upper bound
+    and the true count never has to reach the host.
     """
     lib = _lib.lib()
-    _dev_check(src, dst, src_rows, dst_rows, dst_enable)
+    _dev_check(src, dst, src_rows, dst_rows, dst_enable, n_dev)
     if dst_enable is not None and (dst_enable.dtype not in (torch.bool, torch.uint8) or not dst_enable.is_contiguous()
                                    or dst_enable.numel() != dst.shape[0]):
         raise _capi.TahDuoError("rows_copy: dst_enable must be a contiguous bool/uint8 tensor with one entry per dst row")
@@ -268,7 +274,7 @@ def rows_copy(src: torch.Tensor, src_rows: Optional[torch.Tensor], dst: torch.Te
     sstride = (src.stride(0) if src.shape[0] > 1 else src[0].numel()) * src.element_size()
     dstride = (dst.stride(0) if dst.shape[0] > 1 else dst[0].numel()) * dst.element_size()
     _capi.check(lib, lib.tah_rows_copy(src.data_ptr(), _ptr(src_rows), dst.data_ptr(), _ptr(dst_rows), _ptr(dst_enable), n,
-                                       row_bytes, sstride, dstride, _stream(src)), "tah_rows_copy")
+                                       _ptr(n_dev), row_bytes, sstride, dstride, _stream(src)), "tah_rows_copy")
 
 
 def topk_mix(logits: torch.Tensor, embedding: torch.Tensor, topk: int, row_enable: Optional[torch.Tensor] = None,

@@ -103,3 +103,11 @@ def test_slab_overflow_raises_gpu():
     cache.update(k, k, 0)
     with pytest.raises(TahDuoError, match="capacity"):
         cache.update(k, k, 0)
+
+
+def test_forward_loop_without_host_sync_gpu():
+    """Prefill + a decode step at both depths through the host layer with no host synchronisation at all
+    (torch.cuda.set_sync_debug_mode("error") is on while the loop runs; tah_model.py:116, 580 are the syncs the
+    reference's loop has there)."""
+    from tests.sync_free_case import run
+    assert run("cuda", B=3, T=300, p=0.1, left_pad=(0, 37, 150), Hq=16, Hkv=8)

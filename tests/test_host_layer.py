@@ -300,6 +300,42 @@ def test_position_check_switch(emu):
         attention.CHECK_POSITIONS = False
 
 
+def test_forward_loop_without_host_sync(emu):
+    """HOST_SYNC = False: prefill (left-padded batch) and a decode step at both depths, packed by upper bounds."""
+    from tests.sync_free_case import run
+    assert run("cpu", B=2, T=24, left_pad=(0, 7), Hq=2, Hkv=1)
+
+
+def test_gather_with_max_active_and_overflow_flag(emu):
+    from tah_amd.pack import gather_active, scatter_back
+    g = torch.Generator().manual_seed(8)
+    B, S = 3, 17
+    mask = torch.rand(B, S, generator=g) < 0.4
+    mask[1] = False
+    x = torch.randn(B, S, 4, generator=g).to(torch.bfloat16)
+    ids = torch.arange(B * S).view(B, S)
+    wpad, wx, wi = O.gather_active(mask, x, ids)
+    n = wpad.shape[1]
+    pad, gx, gi = gather_active(mask, x, ids, max_active=n + 2)
+    assert int(pad.overflow) == 0 and pad.shape == (B, n + 2)
+    assert torch.equal(pad[:, :n], wpad) and pad[:, n:].all()
+    assert torch.equal(gx[:, :n], wx) and torch.equal(gi[:, :n], wi) and (gx[:, n:] == 0).all()
+    dest = torch.full((B, S, 4), -7.0).to(torch.bfloat16)
+    assert torch.equal(scatter_back(mask, gx, dest, host_sync=False), O.scatter_back(mask, wx, dest))
+    # a width below the busiest row: the surplus is dropped and the flag raised
+    pad, gx = gather_active(mask, x, max_active=n - 1)
+    assert int(pad.overflow) == 1 and torch.equal(gx, wx[:, : n - 1])
+    part = scatter_back(mask, gx, dest, host_sync=False)
+    want = O.scatter_back(mask, wx, dest)
+    counts = mask.sum(1)
+    for b in range(B):
+        cols = torch.nonzero(mask[b]).flatten()
+        kept = cols[: n - 1]
+        assert torch.equal(part[b, kept], want[b, kept])
+        if counts[b] == n:
+            assert (part[b, cols[-1]] == -7).all()  # the dropped entry's place keeps what dest held
+
+
 def test_hard_index_of_mask_without_columns(emu):
     """S == 0: every boundary is zero (nothing read from uninitialised memory)."""
     from tah_amd.pack import HardIndex, gather_active
