@@ -181,7 +181,8 @@ class TaHDecodeEngine:
         """x [B, H]; appends this token's K/V to the depth's slabs (rows with slot_of < 0 are not cached) and
         attends with q_pos / q_depth per row (q_pos < 0: the row sees nothing and is dropped by the caller)."""
         c = self.cfg
-        cos, sin = self.cos[pos.long()], self.sin[pos.long()]
+        at = pos.long().clamp(0, self.max_len - 1)  # a position past the tables (a caller replaying beyond the
+        cos, sin = self.cos[at], self.sin[at]       # capacity) must not read outside them
         for l, L in enumerate(self.w.layers):
             qkv = self._rms(x, L["ln1"]) @ L["wqkv"].t()
             q, k, v = self._split_qkv(qkv)

@@ -25,7 +25,7 @@ class KvSlabs:
         self.v = torch.zeros((nslots, hkv, capacity, d), dtype=dtype, device=device)
         self.pos = torch.zeros((nslots, capacity), dtype=torch.int32, device=device) if with_pos else None
         # first row of each slab in units of row_stride (= d elements)
-        self.start = (torch.arange(nslots, dtype=torch.int64) * hkv * capacity).to(torch.int32).to(device)
+        self.start = (torch.arange(nslots, dtype=torch.int64, device=device) * (hkv * capacity)).to(torch.int32)
         self.len = torch.zeros(nslots, dtype=torch.int32, device=device)
         self.overflow = torch.zeros(1, dtype=torch.int32, device=device)
         if nslots * hkv * capacity >= 2 ** 31:
