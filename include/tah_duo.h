@@ -180,7 +180,8 @@ size_t tah_duo_decode_workspace_bytes(int32_t nq, int32_t hq, int32_t capacity1,
 /* Decode step of duo-causal attention against the KV cache: every query row
  * attends to the depth-0 rows of its sequence with index <= q_pos, and, if it
  * is a depth-1 query, to the depth-1 rows with pos <= q_pos.  Split-K over
- * 1024-row chunks of both segments, then a merge kernel.
+ * chunks of both segments (1024 rows; 256 rows when nq * hq * chunks is too small to fill the chip), then a
+ * merge kernel.
  * Calls that share a workspace must be ordered on one stream.  Replaces, for Tq == 1:
  *   TaHForCausalLM._build_attention_mask        tah/model/tah_model.py:744-791
  *   TaHCache.get_cache_upto_iter (cat it1|it2)   tah/model/causal_cache.py:101-109
@@ -196,7 +197,7 @@ int tah_duo_decode(const tah_duo_decode_args* args, tah_stream_t stream);
  * split-K partials go to a buffer of TAH_DUO_STATIC_SCRATCH_BYTES that the library itself holds on each GPU
  * (`workspace` / `workspace_bytes` are ignored).  It has no counterpart in the reference.  Calls needing
  * more than that -- tah_duo_decode_workspace_bytes(nq, hq, capacity1, capacity2) bytes, e.g. nq * hq *
- * (chunks of 1024 rows over both capacities) * 520 -- return TAH_E_SCRATCH and launch nothing.  It calls no
+ * (chunks of 1024 or 256 rows over both capacities) * 520 -- return TAH_E_SCRATCH and launch nothing.  It calls no
  * hipMalloc / hipFree; the first call on a device looks the buffer's address up once.  All calls on one
  * GPU share the buffer (nothing in it needs clearing between calls): two calls that overlap in time on
  * one GPU -- different streams, or graphs replayed concurrently -- race. */

@@ -1,6 +1,6 @@
 // Duo-causal decode step against the KV cache (bandwidth-bound), gfx950.
 //
-// Split-K: one workgroup (4 waves) streams one 1024-row chunk of one kv head of
+// Split-K: one workgroup (4 waves) streams one chunk (1024 rows, or 256 when few rows are in play) of one kv head of
 // one query's sequence, from the depth-0 slab or (depth-1 queries only) the
 // depth-1 slab, for all G = Hq/Hkv query heads at once so K and V are read from
 // HBM exactly once.  A wave covers 256 consecutive rows; each load instruction
@@ -37,9 +37,10 @@ constexpr int kD = 128;
 #ifndef TAH_DEC_UNROLL
 #define TAH_DEC_UNROLL 4
 #endif
-constexpr int kChunk = TAH_DEC_CHUNK;  // rows per workgroup
-constexpr int kDecThreads = 256;     // 4 waves x (kChunk / 4) rows
-constexpr int kRowsPerWave = kChunk / 4;
+constexpr int kChunk = TAH_DEC_CHUNK;  // rows per workgroup when there are rows enough to fill the chip
+constexpr int kChunkSmall = 256;       // ... and when there are not (few sequences, short contexts): four
+                                       // times the workgroups, so that enough loads are in flight
+constexpr int kDecThreads = 256;     // 4 waves x (chunk / 4) rows
 constexpr int kUnroll = TAH_DEC_UNROLL;  // loads of 4 rows in flight per wave and tensor
 constexpr int kPart = kD + 2;        // acc[128], m, l  (floats per partial)
 
@@ -60,8 +61,15 @@ struct DecParams {
     Seg c1, c2;
     float* ws;
     int32_t nq, hq, hkv, nchunk1, nchunk2;
+    int32_t chunk;  // rows per workgroup (kChunk or kChunkSmall)
     float scale_log2e;
 };
+
+// Which chunk size a call uses: decided from sizes the host knows, the same way when the workspace is sized.
+__host__ __device__ inline int chunk_rows(int nq, int hq, int capacity1) {
+    const long big = (long)nq * hq * ((capacity1 + kChunk - 1) / kChunk);  // (query, head, chunk) triples at the large size
+    return big < 4096 ? kChunkSmall : kChunk;
+}
 
 template <int CTRL>
 __device__ __forceinline__ float dpp_add(float x) {
@@ -94,8 +102,9 @@ __device__ __forceinline__ int visible_len(const DecParams& p, bool second, int 
     return qdepth >= 1 ? p.c2.len[slot] : 0;
 }
 
-template <int G>
+template <int G, int CH>
 __global__ __launch_bounds__(kDecThreads) void duo_decode_split_kernel(const DecParams p) {
+    constexpr int kRowsPerWave = CH / 4;
     HIP_DYNAMIC_SHARED(unsigned char, smem_raw)
     float (*red)[G][kPart] = reinterpret_cast<float (*)[G][kPart]>(smem_raw);  // [16][G][kPart]: one partial per (wave, row group)
 
@@ -110,10 +119,10 @@ __global__ __launch_bounds__(kDecThreads) void duo_decode_split_kernel(const Dec
         const int qpos = p.q_pos[qi];
         const int qdepth = p.q_depth ? p.q_depth[qi] : p.depth;
         const int nvis = visible_len(p, second, slot, qpos, qdepth);
-        const int row0 = cidx * kChunk;
+        const int row0 = cidx * CH;
         if (row0 >= nvis) return;  // uniform per workgroup
         const Seg& sg = second ? p.c2 : p.c1;
-        const int row_end = row0 + kChunk < nvis ? row0 + kChunk : nvis;
+        const int row_end = row0 + CH < nvis ? row0 + CH : nvis;
         const int64_t base_row = sg.start[slot];
         const __bf16* kbase = sg.k + base_row * sg.k_rs + (int64_t)hk * sg.k_hs + dc * 8;
         const __bf16* vbase = sg.v + base_row * sg.v_rs + (int64_t)hk * sg.v_hs + dc * 8;
@@ -240,8 +249,8 @@ __global__ __launch_bounds__(256) void duo_decode_merge_kernel(const DecParams p
     const int slot = p.q_slot[qi];
     const int qpos = p.q_pos[qi];
     const int qdepth = p.q_depth ? p.q_depth[qi] : p.depth;
-    const int n1 = (visible_len(p, false, slot, qpos, qdepth) + kChunk - 1) / kChunk;
-    const int n2 = (visible_len(p, true, slot, qpos, qdepth) + kChunk - 1) / kChunk;
+    const int n1 = (visible_len(p, false, slot, qpos, qdepth) + p.chunk - 1) / p.chunk;
+    const int n2 = (visible_len(p, true, slot, qpos, qdepth) + p.chunk - 1) / p.chunk;
     const int n = n1 + n2, nslots = p.nchunk1 + p.nchunk2;
     const float* part = p.ws + (int64_t)(qi * p.hq + head) * nslots * kPart;
     auto slot_of = [&](int c) { return c < n1 ? c : p.nchunk1 + (c - n1); };
@@ -494,11 +503,20 @@ int check_seg(const tah_kv_segment& s, bool need_pos) {
 template <int G>
 int launch_decode(const DecParams& p, hipStream_t st) {
     constexpr int kRedBytes = 16 * G * kPart * (int)sizeof(float);  // 8.3 KB per query head of the group
-    if (kRedBytes > 64 * 1024 &&
-        hipFuncSetAttribute(reinterpret_cast<const void*>(&duo_decode_split_kernel<G>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kRedBytes) != hipSuccess)
-        return TAH_E_LAUNCH;
-    hipLaunchKernelGGL(duo_decode_split_kernel<G>, dim3(p.nchunk1 + p.nchunk2, p.nq, p.hkv), dim3(kDecThreads), kRedBytes, st, p);
+    const dim3 grid(p.nchunk1 + p.nchunk2, p.nq, p.hkv);
+    if (p.chunk == kChunk) {
+        if (kRedBytes > 64 * 1024 &&
+            hipFuncSetAttribute(reinterpret_cast<const void*>(&duo_decode_split_kernel<G, kChunk>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kRedBytes) != hipSuccess)
+            return TAH_E_LAUNCH;
+        hipLaunchKernelGGL((duo_decode_split_kernel<G, kChunk>), grid, dim3(kDecThreads), kRedBytes, st, p);
+    } else {
+        if (kRedBytes > 64 * 1024 &&
+            hipFuncSetAttribute(reinterpret_cast<const void*>(&duo_decode_split_kernel<G, kChunkSmall>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kRedBytes) != hipSuccess)
+            return TAH_E_LAUNCH;
+        hipLaunchKernelGGL((duo_decode_split_kernel<G, kChunkSmall>), grid, dim3(kDecThreads), kRedBytes, st, p);
+    }
     hipLaunchKernelGGL(duo_decode_merge_kernel, dim3(p.nq, p.hq), dim3(256), 0, st, p);
     return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
 }
@@ -509,7 +527,8 @@ int launch_decode(const DecParams& p, hipStream_t st) {
 extern "C" size_t tah_duo_decode_workspace_bytes(int32_t nq, int32_t hq, int32_t capacity1, int32_t capacity2) {
     using namespace tah;
     if (nq <= 0 || hq <= 0 || capacity1 < 0 || capacity2 < 0) return 0;
-    const size_t chunks = (size_t)(capacity1 + kChunk - 1) / kChunk + (size_t)(capacity2 + kChunk - 1) / kChunk;
+    const int ch = chunk_rows(nq, hq, capacity1);
+    const size_t chunks = (size_t)(capacity1 + ch - 1) / ch + (size_t)(capacity2 + ch - 1) / ch;
     return (size_t)nq * hq * chunks * kPart * sizeof(float);
 }
 
@@ -544,8 +563,9 @@ int decode_impl(const tah_duo_decode_args* a, void* ws, size_t ws_bytes, int too
     p.c2 = to_seg(a->c2);
     p.ws = static_cast<float*>(ws);
     p.nq = a->nq; p.hq = a->hq; p.hkv = a->hkv;
-    p.nchunk1 = (a->c1.capacity + kChunk - 1) / kChunk;
-    p.nchunk2 = (cap2 + kChunk - 1) / kChunk;
+    p.chunk = chunk_rows(a->nq, a->hq, a->c1.capacity);
+    p.nchunk1 = (a->c1.capacity + p.chunk - 1) / p.chunk;
+    p.nchunk2 = (cap2 + p.chunk - 1) / p.chunk;
     p.scale_log2e = a->scale * kLog2e;
     if (p.nchunk1 + p.nchunk2 == 0) return TAH_E_SHAPE;
     hipStream_t st = static_cast<hipStream_t>(stream);
