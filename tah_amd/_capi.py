@@ -1,7 +1,8 @@
-"""ctypes mirror of include/tah_duo.h: structs, prototypes and error mapping.
+"""ctypes mirror of include/tah_duo.h: structs, prototypes, error codes.
 
-This module only describes the C ABI; :mod:`tah_amd._lib` loads the MI355X
-library and binds these prototypes to it.
+The package itself reaches the library through its PyTorch extension (``tah_amd._C``, csrc/torch_ext.cpp).
+This module describes the same C ABI for callers that want to bind it without torch (``bind`` attaches the
+prototypes to a ``ctypes.CDLL``) and for the tests that call entry points with hand-made arguments.
 """
 from __future__ import annotations
 

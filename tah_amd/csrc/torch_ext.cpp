@@ -1,0 +1,482 @@
+// PyTorch-ROCm extension over the C ABI of include/tah_duo.h.
+//
+// Python hands tensors to the functions below; each one checks shapes, dtypes and devices, allocates the
+// outputs through torch, fills the plain C argument struct (raw device pointers, strides, sizes) and calls
+// the entry point on torch's current HIP stream.  Nothing is computed here.  The library itself is opened at
+// run time (load_library), so the same extension serves libtah_duo.so and, in the CPU tests, the host build
+// of the kernels.  There is no fallback: without a loaded library every call throws.
+#include <c10/hip/HIPStream.h>
+#include <dlfcn.h>
+#include <torch/extension.h>
+
+#include <string>
+#include <tuple>
+
+#include "tah_duo.h"
+
+namespace {
+
+using at::Tensor;
+using c10::optional;
+
+struct Api {
+    void* handle = nullptr;
+    bool allow_host = false;
+    decltype(&tah_duo_abi_version) abi_version = nullptr;
+    decltype(&tah_duo_error_string) error_string = nullptr;
+    decltype(&tah_duo_fwd_varlen) fwd_varlen = nullptr;
+    decltype(&tah_duo_bwd_varlen) bwd_varlen = nullptr;
+    decltype(&tah_duo_fwd_masked) fwd_masked = nullptr;
+    decltype(&tah_duo_bwd_masked) bwd_masked = nullptr;
+    decltype(&tah_duo_decode_workspace_bytes) decode_workspace_bytes = nullptr;
+    decltype(&tah_duo_decode) decode = nullptr;
+    decltype(&tah_duo_decode_static) decode_static = nullptr;
+    decltype(&tah_kv_append) kv_append = nullptr;
+    decltype(&tah_qk_prep) qk_prep = nullptr;
+    decltype(&tah_topk_mix) topk_mix = nullptr;
+    decltype(&tah_silu_mul) silu_mul = nullptr;
+    decltype(&tah_hard_index_build) hard_index_build = nullptr;
+    decltype(&tah_pad_rows_build) pad_rows_build = nullptr;
+    decltype(&tah_rows_copy) rows_copy = nullptr;
+} g;
+
+template <class F>
+void bind(F& f, const char* name) {
+    f = reinterpret_cast<F>(dlsym(g.handle, name));
+    TORCH_CHECK(f != nullptr, "tah_amd: ", name, " is not exported by the loaded library");
+}
+
+void load_library(const std::string& path, bool allow_host) {
+    void* h = dlopen(path.c_str(), RTLD_NOW | RTLD_LOCAL);
+    TORCH_CHECK(h != nullptr, "tah_amd: cannot load ", path, ": ", dlerror(),
+                " (the HIP library is not built? there is no CPU or PyTorch fallback)");
+    g = Api{};
+    g.handle = h;
+    g.allow_host = allow_host;
+    bind(g.abi_version, "tah_duo_abi_version");
+    bind(g.error_string, "tah_duo_error_string");
+    bind(g.fwd_varlen, "tah_duo_fwd_varlen");
+    bind(g.bwd_varlen, "tah_duo_bwd_varlen");
+    bind(g.fwd_masked, "tah_duo_fwd_masked");
+    bind(g.bwd_masked, "tah_duo_bwd_masked");
+    bind(g.decode_workspace_bytes, "tah_duo_decode_workspace_bytes");
+    bind(g.decode, "tah_duo_decode");
+    bind(g.decode_static, "tah_duo_decode_static");
+    bind(g.kv_append, "tah_kv_append");
+    bind(g.qk_prep, "tah_qk_prep");
+    bind(g.topk_mix, "tah_topk_mix");
+    bind(g.silu_mul, "tah_silu_mul");
+    bind(g.hard_index_build, "tah_hard_index_build");
+    bind(g.pad_rows_build, "tah_pad_rows_build");
+    bind(g.rows_copy, "tah_rows_copy");
+    const int got = g.abi_version();
+    TORCH_CHECK(got == TAH_DUO_ABI_VERSION, "tah_amd: library ABI version ", got, ", extension built for ", TAH_DUO_ABI_VERSION);
+}
+
+void need_lib() { TORCH_CHECK(g.handle != nullptr, "tah_amd: no library loaded (tah_amd._lib.lib() loads libtah_duo.so)"); }
+
+void check_rc(int rc, const char* what) {
+    TORCH_CHECK(rc == 0, what, ": ", g.error_string(rc), " (code ", rc, ")");
+}
+
+// One device for all tensors; host tensors only when the loaded library is the host build of the kernels.
+struct Dev {
+    bool set = false;
+    c10::Device dev{c10::kCPU};
+    void see(const Tensor& t) {
+        if (!t.defined()) return;
+        TORCH_CHECK(t.is_cuda() || g.allow_host, "tah_amd ops need CUDA/HIP tensors (no CPU path exists)");
+        if (!set) { dev = t.device(); set = true; }
+        else TORCH_CHECK(t.device() == dev, "tensors on different devices: ", dev, " vs ", t.device());
+    }
+    void see(const optional<Tensor>& t) { if (t.has_value()) see(*t); }
+    tah_stream_t stream() const {
+        if (set && dev.is_cuda()) return static_cast<tah_stream_t>(c10::hip::getCurrentHIPStream(dev.index()).stream());
+        return nullptr;
+    }
+};
+
+const void* ptr(const Tensor& t) { return (!t.defined() || t.numel() == 0) ? nullptr : t.data_ptr(); }
+void* mptr(const Tensor& t) { return (!t.defined() || t.numel() == 0) ? nullptr : t.data_ptr(); }
+const void* ptr(const optional<Tensor>& t) { return t.has_value() ? ptr(*t) : nullptr; }
+
+void thd(const Tensor& t, const char* name) {
+    TORCH_CHECK(t.dim() == 3 && t.scalar_type() == at::kBFloat16, name, " must be a bf16 [rows, heads, head_dim] tensor");
+    TORCH_CHECK(t.numel() == 0 || t.stride(2) == 1, name, ": head_dim must be contiguous");
+}
+void i32(const Tensor& t, const char* name) {
+    TORCH_CHECK(t.scalar_type() == at::kInt && t.is_contiguous(), name, " must be a contiguous int32 tensor");
+}
+
+void fill_stream(tah_duo_stream& s, const Tensor& q, const Tensor& k, const Tensor& v, const Tensor& o, const Tensor& lse,
+                 const Tensor& cu_q, const Tensor& cu_k, const Tensor* pos_q, const Tensor* pos_k) {
+    s.q = ptr(q); s.k = ptr(k); s.v = ptr(v); s.o = mptr(o); s.lse = static_cast<float*>(mptr(lse));
+    s.cu_q = static_cast<const int32_t*>(cu_q.data_ptr());
+    s.cu_k = static_cast<const int32_t*>(cu_k.data_ptr());
+    s.pos_q = pos_q ? static_cast<const int32_t*>(ptr(*pos_q)) : nullptr;
+    s.pos_k = pos_k ? static_cast<const int32_t*>(ptr(*pos_k)) : nullptr;
+    s.q_row_stride = q.stride(0); s.q_head_stride = q.stride(1);
+    s.k_row_stride = k.stride(0); s.k_head_stride = k.stride(1);
+    s.v_row_stride = v.stride(0); s.v_head_stride = v.stride(1);
+    s.o_row_stride = o.stride(0); s.o_head_stride = o.stride(1);
+    s.total_q = (int32_t)q.size(0); s.total_k = (int32_t)k.size(0);
+}
+
+std::tuple<Tensor, Tensor, Tensor, Tensor> duo_fwd_varlen(const Tensor& q1, const Tensor& k1, const Tensor& v1, const Tensor& cu_q1,
+                                                          const Tensor& cu_k1, const Tensor& q2, const Tensor& k2, const Tensor& v2,
+                                                          const Tensor& pos_q2, const Tensor& pos_k2, const Tensor& cu_q2,
+                                                          const Tensor& cu_k2, double scale) {
+    need_lib();
+    thd(q1, "q1"); thd(k1, "k1"); thd(v1, "v1"); thd(q2, "q2"); thd(k2, "k2"); thd(v2, "v2");
+    i32(cu_q1, "cu_q1"); i32(cu_k1, "cu_k1"); i32(cu_q2, "cu_q2"); i32(cu_k2, "cu_k2"); i32(pos_q2, "pos_q2"); i32(pos_k2, "pos_k2");
+    Dev d;
+    for (const Tensor* t : {&q1, &k1, &v1, &q2, &k2, &v2, &cu_q1, &cu_k1, &cu_q2, &cu_k2, &pos_q2, &pos_k2}) d.see(*t);
+    const int64_t nseq = cu_q1.numel() - 1;
+    TORCH_CHECK(cu_k1.numel() == nseq + 1 && cu_q2.numel() == nseq + 1 && cu_k2.numel() == nseq + 1,
+                "cu_seqlens tensors must all have nseq+1 entries");
+    TORCH_CHECK(pos_q2.numel() == q2.size(0) && pos_k2.numel() == k2.size(0) && k1.sizes() == v1.sizes() && k2.sizes() == v2.sizes(),
+                "inconsistent row counts");
+    const int64_t hq = q1.size(1), dd = q1.size(2);
+    auto o1 = at::empty({q1.size(0), hq, dd}, q1.options());
+    auto o2 = at::empty({q2.size(0), hq, dd}, q1.options());
+    auto lse1 = at::empty({hq, q1.size(0)}, q1.options().dtype(at::kFloat));
+    auto lse2 = at::empty({hq, q2.size(0)}, q1.options().dtype(at::kFloat));
+    tah_duo_fwd_args a{};
+    fill_stream(a.s1, q1, k1, v1, o1, lse1, cu_q1, cu_k1, nullptr, nullptr);
+    fill_stream(a.s2, q2, k2, v2, o2, lse2, cu_q2, cu_k2, &pos_q2, &pos_k2);
+    a.nseq = (int32_t)nseq; a.hq = (int32_t)hq; a.hkv = (int32_t)k1.size(1); a.d = (int32_t)dd; a.scale = (float)scale;
+    check_rc(g.fwd_varlen(&a, d.stream()), "tah_duo_fwd_varlen");
+    return {o1, lse1, o2, lse2};
+}
+
+void fill_bwd_stream(tah_duo_bwd_stream& s, const Tensor& d_o, const Tensor& dq, const Tensor& dk, const Tensor& dv, const Tensor& delta) {
+    s.d_o = ptr(d_o); s.dq = mptr(dq); s.dk = mptr(dk); s.dv = mptr(dv); s.delta = static_cast<float*>(mptr(delta));
+    s.do_row_stride = d_o.stride(0); s.do_head_stride = d_o.stride(1);
+    s.dq_row_stride = dq.stride(0); s.dq_head_stride = dq.stride(1);
+    s.dk_row_stride = dk.stride(0); s.dk_head_stride = dk.stride(1);
+    s.dv_row_stride = dv.stride(0); s.dv_head_stride = dv.stride(1);
+}
+
+std::vector<Tensor> duo_bwd_varlen(const Tensor& q1, const Tensor& k1, const Tensor& v1, const Tensor& o1, const Tensor& lse1,
+                                   const Tensor& do1, const Tensor& cu_q1, const Tensor& cu_k1, const Tensor& q2, const Tensor& k2,
+                                   const Tensor& v2, const Tensor& o2, const Tensor& lse2, const Tensor& do2, const Tensor& pos_q2,
+                                   const Tensor& pos_k2, const Tensor& cu_q2, const Tensor& cu_k2, double scale) {
+    need_lib();
+    for (auto p : {std::make_pair(&q1, "q1"), {&k1, "k1"}, {&v1, "v1"}, {&o1, "o1"}, {&do1, "do1"}, {&q2, "q2"}, {&k2, "k2"},
+                   {&v2, "v2"}, {&o2, "o2"}, {&do2, "do2"}})
+        thd(*p.first, p.second);
+    i32(cu_q1, "cu_q1"); i32(cu_k1, "cu_k1"); i32(cu_q2, "cu_q2"); i32(cu_k2, "cu_k2"); i32(pos_q2, "pos_q2"); i32(pos_k2, "pos_k2");
+    Dev d;
+    for (const Tensor* t : {&q1, &k1, &v1, &o1, &lse1, &do1, &q2, &k2, &v2, &o2, &lse2, &do2, &cu_q1, &cu_k1, &cu_q2, &cu_k2, &pos_q2, &pos_k2})
+        d.see(*t);
+    TORCH_CHECK(do1.sizes() == q1.sizes() && do2.sizes() == q2.sizes() && o1.sizes() == q1.sizes() && o2.sizes() == q2.sizes(),
+                "o / dO shapes must match q");
+    TORCH_CHECK(lse1.scalar_type() == at::kFloat && lse2.scalar_type() == at::kFloat && lse1.is_contiguous() && lse2.is_contiguous(),
+                "lse must be contiguous float32 [Hq, rows]");
+    const int64_t hq = q1.size(1);
+    auto dq1 = at::empty(q1.sizes(), q1.options()), dk1 = at::empty(k1.sizes(), k1.options()), dv1 = at::empty(v1.sizes(), v1.options());
+    auto dq2 = at::empty(q2.sizes(), q2.options()), dk2 = at::empty(k2.sizes(), k2.options()), dv2 = at::empty(v2.sizes(), v2.options());
+    auto delta1 = at::empty({hq, q1.size(0)}, q1.options().dtype(at::kFloat));
+    auto delta2 = at::empty({hq, q2.size(0)}, q1.options().dtype(at::kFloat));
+    tah_duo_bwd_args a{};
+    fill_stream(a.fwd.s1, q1, k1, v1, o1, lse1, cu_q1, cu_k1, nullptr, nullptr);
+    fill_stream(a.fwd.s2, q2, k2, v2, o2, lse2, cu_q2, cu_k2, &pos_q2, &pos_k2);
+    a.fwd.nseq = (int32_t)(cu_q1.numel() - 1); a.fwd.hq = (int32_t)hq; a.fwd.hkv = (int32_t)k1.size(1); a.fwd.d = (int32_t)q1.size(2);
+    a.fwd.scale = (float)scale;
+    fill_bwd_stream(a.g1, do1, dq1, dk1, dv1, delta1);
+    fill_bwd_stream(a.g2, do2, dq2, dk2, dv2, delta2);
+    check_rc(g.bwd_varlen(&a, d.stream()), "tah_duo_bwd_varlen");
+    return {dq1, dk1, dv1, dq2, dk2, dv2};
+}
+
+void fill_mask(tah_additive_mask& m, const Tensor& mask, int64_t nseq, int64_t hq, int64_t tq, int64_t tk) {
+    TORCH_CHECK(mask.dim() == 4 && (mask.scalar_type() == at::kBFloat16 || mask.scalar_type() == at::kFloat),
+                "additive mask must be a 4-D bf16 or float32 tensor (B|1, Hq|1, Tq, Tkv)");
+    TORCH_CHECK((mask.size(0) == 1 || mask.size(0) == nseq) && (mask.size(1) == 1 || mask.size(1) == hq) && mask.size(2) == tq &&
+                    mask.size(3) == tk,
+                "additive mask shape ", mask.sizes(), " does not match (B=", nseq, ", Hq=", hq, ", Tq=", tq, ", Tkv=", tk, ")");
+    m.mask = mask.data_ptr();
+    m.seq_stride = mask.size(0) != 1 ? mask.stride(0) : 0;
+    m.head_stride = mask.size(1) != 1 ? mask.stride(1) : 0;
+    m.q_stride = mask.stride(2); m.k_stride = mask.stride(3);
+    m.dtype = mask.scalar_type() == at::kFloat ? 1 : 0;
+}
+
+Tensor dense_cu(const Tensor& like, int64_t nseq, int64_t t) {
+    return at::arange(0, (nseq + 1) * t, t, like.options().dtype(at::kInt));
+}
+
+std::tuple<Tensor, Tensor> duo_fwd_masked(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor& mask, int64_t nseq, double scale) {
+    need_lib();
+    thd(q, "q"); thd(k, "k"); thd(v, "v");
+    Dev d; d.see(q); d.see(k); d.see(v); d.see(mask);
+    TORCH_CHECK(nseq > 0 && q.size(0) % nseq == 0 && k.size(0) % nseq == 0 && k.sizes() == v.sizes(),
+                "row counts must be multiples of the batch size");
+    const int64_t tq = q.size(0) / nseq, tk = k.size(0) / nseq, hq = q.size(1), dd = q.size(2);
+    auto o = at::empty({q.size(0), hq, dd}, q.options());
+    auto lse = at::empty({hq, q.size(0)}, q.options().dtype(at::kFloat));
+    auto cu_q = dense_cu(q, nseq, tq), cu_k = dense_cu(q, nseq, tk);
+    auto zc = at::zeros({nseq + 1}, q.options().dtype(at::kInt));
+    auto e = q.narrow(0, 0, 0), ek = k.narrow(0, 0, 0), el = lse.narrow(1, 0, 0);
+    tah_duo_fwd_args a{};
+    fill_stream(a.s1, q, k, v, o, lse, cu_q, cu_k, nullptr, nullptr);
+    fill_stream(a.s2, e, ek, ek, e, el, zc, zc, nullptr, nullptr);
+    a.nseq = (int32_t)nseq; a.hq = (int32_t)hq; a.hkv = (int32_t)k.size(1); a.d = (int32_t)dd; a.scale = (float)scale;
+    tah_additive_mask m{};
+    fill_mask(m, mask, nseq, hq, tq, tk);
+    check_rc(g.fwd_masked(&a, &m, d.stream()), "tah_duo_fwd_masked");
+    return {o, lse};
+}
+
+std::vector<Tensor> duo_bwd_masked(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor& o, const Tensor& lse,
+                                   const Tensor& d_o, const Tensor& mask, int64_t nseq, double scale) {
+    need_lib();
+    thd(q, "q"); thd(k, "k"); thd(v, "v"); thd(o, "o"); thd(d_o, "d_o");
+    Dev d;
+    for (const Tensor* t : {&q, &k, &v, &o, &lse, &d_o, &mask}) d.see(*t);
+    TORCH_CHECK(d_o.sizes() == q.sizes() && o.sizes() == q.sizes(), "o / dO shapes must match q");
+    TORCH_CHECK(lse.scalar_type() == at::kFloat && lse.is_contiguous(), "lse must be contiguous float32 [Hq, rows]");
+    const int64_t tq = q.size(0) / nseq, tk = k.size(0) / nseq, hq = q.size(1);
+    auto dq = at::empty(q.sizes(), q.options()), dk = at::empty(k.sizes(), k.options()), dv = at::empty(v.sizes(), v.options());
+    auto delta = at::empty({hq, q.size(0)}, q.options().dtype(at::kFloat));
+    auto cu_q = dense_cu(q, nseq, tq), cu_k = dense_cu(q, nseq, tk);
+    auto zc = at::zeros({nseq + 1}, q.options().dtype(at::kInt));
+    auto e = q.narrow(0, 0, 0), ek = k.narrow(0, 0, 0), el = lse.narrow(1, 0, 0), ed = delta.narrow(1, 0, 0);
+    tah_duo_bwd_args a{};
+    fill_stream(a.fwd.s1, q, k, v, o, lse, cu_q, cu_k, nullptr, nullptr);
+    fill_stream(a.fwd.s2, e, ek, ek, e, el, zc, zc, nullptr, nullptr);
+    a.fwd.nseq = (int32_t)nseq; a.fwd.hq = (int32_t)hq; a.fwd.hkv = (int32_t)k.size(1); a.fwd.d = (int32_t)q.size(2); a.fwd.scale = (float)scale;
+    fill_bwd_stream(a.g1, d_o, dq, dk, dv, delta);
+    fill_bwd_stream(a.g2, e, e, ek, ek, ed);
+    tah_additive_mask m{};
+    fill_mask(m, mask, nseq, hq, tq, tk);
+    check_rc(g.bwd_masked(&a, &m, d.stream()), "tah_duo_bwd_masked");
+    return {dq, dk, dv};
+}
+
+// One depth of the slab cache as tensors: k, v [slot, Hkv, capacity, D]; pos [slot, capacity] or none; start, len [slot].
+tah_kv_segment segment(const Tensor& k, const Tensor& v, const optional<Tensor>& pos, const Tensor& start, const Tensor& len) {
+    TORCH_CHECK(k.dim() == 4 && v.sizes() == k.sizes() && k.is_contiguous() && v.is_contiguous(), "slabs must be contiguous [slot, Hkv, capacity, D]");
+    tah_kv_segment s{};
+    s.k = k.data_ptr(); s.v = v.data_ptr();
+    s.pos = pos.has_value() ? static_cast<int32_t*>(pos->data_ptr()) : nullptr;
+    s.start = static_cast<const int32_t*>(start.data_ptr());
+    s.len = static_cast<int32_t*>(len.data_ptr());
+    s.k_row_stride = s.v_row_stride = k.size(3);
+    s.k_head_stride = s.v_head_stride = k.size(2) * k.size(3);
+    s.capacity = (int32_t)k.size(2);
+    s.nslots = (int32_t)k.size(0);
+    return s;
+}
+
+int64_t decode_workspace_bytes(int64_t nq, int64_t hq, int64_t cap1, int64_t cap2) {
+    need_lib();
+    return (int64_t)g.decode_workspace_bytes((int32_t)nq, (int32_t)hq, (int32_t)cap1, (int32_t)cap2);
+}
+
+void duo_decode(const Tensor& q, const Tensor& o, const optional<Tensor>& lse, const Tensor& q_slot, const Tensor& q_pos,
+                const optional<Tensor>& q_depth, int64_t depth, const Tensor& k1, const Tensor& v1, const Tensor& start1,
+                const Tensor& len1, const optional<Tensor>& k2, const optional<Tensor>& v2, const optional<Tensor>& pos2,
+                const optional<Tensor>& start2, const optional<Tensor>& len2, const optional<Tensor>& workspace, double scale) {
+    need_lib();
+    thd(q, "q"); i32(q_slot, "q_slot"); i32(q_pos, "q_pos");
+    Dev d; d.see(q); d.see(o); d.see(lse); d.see(q_slot); d.see(q_pos); d.see(q_depth); d.see(k1); d.see(workspace);
+    const bool need2 = q_depth.has_value() || depth >= 1;
+    TORCH_CHECK(!need2 || (k2.has_value() && v2.has_value() && pos2.has_value() && start2.has_value() && len2.has_value()),
+                "depth-1 queries need the depth-1 cache");
+    tah_duo_decode_args a{};
+    a.q = ptr(q); a.o = mptr(o); a.lse = lse.has_value() ? static_cast<float*>(lse->data_ptr()) : nullptr;
+    a.q_row_stride = q.stride(0); a.q_head_stride = q.stride(1); a.o_row_stride = o.stride(0); a.o_head_stride = o.stride(1);
+    a.q_slot = static_cast<const int32_t*>(q_slot.data_ptr());
+    a.q_pos = static_cast<const int32_t*>(q_pos.data_ptr());
+    a.q_depth = q_depth.has_value() ? static_cast<const int32_t*>(q_depth->data_ptr()) : nullptr;
+    a.depth = (int32_t)depth;
+    a.c1 = segment(k1, v1, c10::nullopt, start1, len1);
+    if (need2) a.c2 = segment(*k2, *v2, pos2, *start2, *len2);
+    a.nq = (int32_t)q.size(0); a.hq = (int32_t)q.size(1); a.hkv = (int32_t)k1.size(1); a.d = (int32_t)q.size(2); a.scale = (float)scale;
+    if (workspace.has_value()) {
+        a.workspace = workspace->data_ptr();
+        a.workspace_bytes = (size_t)workspace->numel() * workspace->element_size();
+        check_rc(g.decode(&a, d.stream()), "tah_duo_decode");
+    } else {
+        check_rc(g.decode_static(&a, d.stream()), "tah_duo_decode_static");
+    }
+}
+
+void kv_append(const Tensor& k_new, const Tensor& v_new, const Tensor& cu_new, const optional<Tensor>& pos_new,
+               const optional<Tensor>& slot_of, const Tensor& ck, const Tensor& cv, const optional<Tensor>& cpos, const Tensor& start,
+               const Tensor& len, const Tensor& overflow) {
+    need_lib();
+    thd(k_new, "k_new"); thd(v_new, "v_new"); i32(cu_new, "cu_new");
+    Dev d; d.see(k_new); d.see(v_new); d.see(cu_new); d.see(pos_new); d.see(slot_of); d.see(ck);
+    TORCH_CHECK(pos_new.has_value() == cpos.has_value(), "pos_new must be given exactly for slabs created with_pos=True");
+    tah_kv_append_args a{};
+    a.k_new = ptr(k_new); a.v_new = ptr(v_new); a.pos_new = static_cast<const int32_t*>(ptr(pos_new));
+    a.k_row_stride = k_new.stride(0); a.k_head_stride = k_new.stride(1);
+    a.v_row_stride = v_new.stride(0); a.v_head_stride = v_new.stride(1);
+    a.cu_new = static_cast<const int32_t*>(cu_new.data_ptr());
+    a.slot_of = static_cast<const int32_t*>(ptr(slot_of));
+    a.nseq = (int32_t)(cu_new.numel() - 1); a.total_new = (int32_t)k_new.size(0); a.hkv = (int32_t)ck.size(1); a.d = (int32_t)ck.size(3);
+    a.cache = segment(ck, cv, cpos, start, len);
+    a.overflow = static_cast<int32_t*>(overflow.data_ptr());
+    check_rc(g.kv_append(&a, d.stream()), "tah_kv_append");
+}
+
+// q/k RMSNorm + rotary (+ append): returns nothing, the caller allocated q_out / k_out.
+void qk_prep(const Tensor& q, const Tensor& k, const optional<Tensor>& v, const Tensor& q_out, const optional<Tensor>& k_out,
+             const Tensor& q_weight, const Tensor& k_weight, const Tensor& cos, const Tensor& sin, double eps,
+             const optional<Tensor>& ck, const optional<Tensor>& cv, const optional<Tensor>& cpos, const optional<Tensor>& start,
+             const optional<Tensor>& len, const optional<Tensor>& overflow, const optional<Tensor>& cu_new,
+             const optional<Tensor>& pos_new, const optional<Tensor>& slot_of, bool one_row_per_seq) {
+    need_lib();
+    thd(q, "q"); thd(k, "k");
+    Dev d; d.see(q); d.see(k); d.see(v); d.see(q_weight); d.see(k_weight); d.see(cos); d.see(sin); d.see(cu_new); d.see(pos_new);
+    d.see(slot_of); d.see(ck);
+    const int64_t D = q.size(2);
+    for (auto p : {std::make_pair(&q_weight, "q_weight"), {&k_weight, "k_weight"}})
+        TORCH_CHECK(p.first->scalar_type() == at::kBFloat16 && p.first->dim() == 1 && p.first->size(0) == D && p.first->is_contiguous(),
+                    p.second, " must be a contiguous bf16 [", D, "] tensor");
+    for (auto p : {std::make_pair(&cos, "cos"), {&sin, "sin"}})
+        TORCH_CHECK(p.first->scalar_type() == at::kBFloat16 && p.first->dim() == 2 && p.first->size(0) == q.size(0) &&
+                        p.first->size(1) == D && p.first->stride(1) == 1,
+                    p.second, " must be a bf16 [rows, ", D, "] tensor with unit inner stride");
+    TORCH_CHECK(cos.stride(0) == sin.stride(0), "cos and sin must share their row stride");
+    TORCH_CHECK(k.size(0) == q.size(0), "q and k must have one row per token");
+    tah_qk_prep_args a{};
+    a.q = ptr(q); a.k = ptr(k); a.v = ptr(v); a.q_out = mptr(q_out);
+    a.q_row_stride = q.stride(0); a.q_head_stride = q.stride(1);
+    a.k_row_stride = k.stride(0); a.k_head_stride = k.stride(1);
+    a.q_out_row_stride = q_out.stride(0); a.q_out_head_stride = q_out.stride(1);
+    if (v.has_value()) { thd(*v, "v"); a.v_row_stride = v->stride(0); a.v_head_stride = v->stride(1); }
+    a.q_weight = ptr(q_weight); a.k_weight = ptr(k_weight); a.cos = ptr(cos); a.sin = ptr(sin);
+    a.cos_sin_row_stride = cos.stride(0);
+    a.eps = (float)eps;
+    a.rows = (int32_t)q.size(0); a.hq = (int32_t)q.size(1); a.hkv = (int32_t)k.size(1); a.d = (int32_t)D;
+    if (ck.has_value()) {
+        TORCH_CHECK(v.has_value() && cu_new.has_value(), "appending needs v and cu_new");
+        TORCH_CHECK(pos_new.has_value() == cpos.has_value(), "pos_new must be given exactly for slabs created with_pos=True");
+        i32(*cu_new, "cu_new");
+        a.append = 1;
+        a.append_one_row_per_seq = one_row_per_seq ? 1 : 0;
+        a.cu_new = static_cast<const int32_t*>(cu_new->data_ptr());
+        a.slot_of = static_cast<const int32_t*>(ptr(slot_of));
+        a.pos_new = static_cast<const int32_t*>(ptr(pos_new));
+        a.nseq = (int32_t)(cu_new->numel() - 1);
+        a.cache = segment(*ck, *cv, cpos, *start, *len);
+        a.overflow = overflow.has_value() ? static_cast<int32_t*>(overflow->data_ptr()) : nullptr;
+    } else {
+        TORCH_CHECK(k_out.has_value(), "k_out is needed when nothing is appended");
+        a.k_out = mptr(*k_out);
+        a.k_out_row_stride = k_out->stride(0); a.k_out_head_stride = k_out->stride(1);
+    }
+    check_rc(g.qk_prep(&a, d.stream()), "tah_qk_prep");
+}
+
+std::tuple<Tensor, Tensor, Tensor, Tensor> hard_index_build(const Tensor& mask) {
+    need_lib();
+    Dev d; d.see(mask);
+    TORCH_CHECK(mask.dim() == 2 && (mask.scalar_type() == at::kBool || mask.scalar_type() == at::kByte),
+                "mask must be a (B, S) bool or uint8 tensor");
+    auto m = mask.contiguous();
+    const int64_t B = m.size(0), S = m.size(1), cap = std::max<int64_t>(B * S, 1);
+    auto io = m.options().dtype(at::kInt);
+    auto pos = at::empty({cap}, io), flat = at::empty({cap}, io), seq = at::empty({cap}, io), cu = at::empty({B + 1}, io);
+    check_rc(g.hard_index_build(static_cast<const uint8_t*>(ptr(m)), (int32_t)B, (int32_t)S, static_cast<int32_t*>(pos.data_ptr()),
+                                static_cast<int32_t*>(flat.data_ptr()), static_cast<int32_t*>(seq.data_ptr()),
+                                static_cast<int32_t*>(cu.data_ptr()), d.stream()),
+             "tah_hard_index_build");
+    return {pos, flat, seq, cu};
+}
+
+Tensor pad_rows_build(const Tensor& cu, const Tensor& seq_of, int64_t n, int64_t width, const optional<Tensor>& n_dev,
+                      const optional<Tensor>& overflow) {
+    need_lib();
+    Dev d; d.see(cu); d.see(seq_of); d.see(n_dev); d.see(overflow);
+    auto out = at::empty({std::max<int64_t>(n, 1)}, cu.options().dtype(at::kInt));
+    check_rc(g.pad_rows_build(static_cast<const int32_t*>(cu.data_ptr()), static_cast<const int32_t*>(seq_of.data_ptr()), (int32_t)n,
+                              static_cast<const int32_t*>(ptr(n_dev)), (int32_t)width, static_cast<int32_t*>(out.data_ptr()),
+                              overflow.has_value() ? static_cast<int32_t*>(overflow->data_ptr()) : nullptr, d.stream()),
+             "tah_pad_rows_build");
+    return out.narrow(0, 0, n);
+}
+
+void rows_copy(const Tensor& src, const optional<Tensor>& src_rows, const Tensor& dst, const optional<Tensor>& dst_rows, int64_t n,
+               const optional<Tensor>& dst_enable, const optional<Tensor>& n_dev) {
+    need_lib();
+    Dev d; d.see(src); d.see(dst); d.see(src_rows); d.see(dst_rows); d.see(dst_enable); d.see(n_dev);
+    if (dst_enable.has_value())
+        TORCH_CHECK((dst_enable->scalar_type() == at::kBool || dst_enable->scalar_type() == at::kByte) && dst_enable->is_contiguous() &&
+                        dst_enable->numel() == dst.size(0),
+                    "rows_copy: dst_enable must be a contiguous bool/uint8 tensor with one entry per dst row");
+    if (n == 0) return;
+    TORCH_CHECK(src.scalar_type() == dst.scalar_type() && src.sizes().slice(1) == dst.sizes().slice(1),
+                "rows_copy: src and dst rows differ in dtype or shape");
+    TORCH_CHECK(src.select(0, 0).is_contiguous() && dst.select(0, 0).is_contiguous(), "rows_copy: rows must be contiguous");
+    const int64_t row_elems = src.select(0, 0).numel(), es = src.element_size();
+    const int64_t sstride = (src.size(0) > 1 ? src.stride(0) : row_elems) * es;
+    const int64_t dstride = (dst.size(0) > 1 ? dst.stride(0) : row_elems) * es;
+    check_rc(g.rows_copy(src.data_ptr(), static_cast<const int32_t*>(ptr(src_rows)), dst.data_ptr(),
+                         static_cast<const int32_t*>(ptr(dst_rows)), static_cast<const uint8_t*>(ptr(dst_enable)), (int32_t)n,
+                         static_cast<const int32_t*>(ptr(n_dev)), row_elems * es, sstride, dstride, d.stream()),
+             "tah_rows_copy");
+}
+
+Tensor topk_mix(const Tensor& logits, const Tensor& embedding, int64_t topk, const optional<Tensor>& row_enable, const optional<Tensor>& out_) {
+    need_lib();
+    Dev d; d.see(logits); d.see(embedding); d.see(row_enable); d.see(out_);
+    TORCH_CHECK(logits.dim() == 2 && embedding.dim() == 2 && logits.scalar_type() == at::kBFloat16 && embedding.scalar_type() == at::kBFloat16,
+                "topk_mix: logits [rows, V] and embedding [V, H] must be bf16");
+    TORCH_CHECK(logits.size(1) == embedding.size(0) && logits.stride(1) == 1 && embedding.stride(1) == 1,
+                "topk_mix: vocabulary sizes differ or the inner dimension is not contiguous");
+    const int64_t rows = logits.size(0), H = embedding.size(1);
+    Tensor out = out_.has_value() ? *out_ : (row_enable.has_value() ? at::zeros({rows, H}, embedding.options()) : at::empty({rows, H}, embedding.options()));
+    TORCH_CHECK(out.dim() == 2 && out.size(0) == rows && out.size(1) == H && out.scalar_type() == embedding.scalar_type() && out.stride(1) == 1,
+                "topk_mix: out must be bf16 [rows, H]");
+    if (row_enable.has_value())
+        TORCH_CHECK((row_enable->scalar_type() == at::kBool || row_enable->scalar_type() == at::kByte) && row_enable->numel() == rows &&
+                        row_enable->is_contiguous(),
+                    "topk_mix: row_enable must be a contiguous bool/uint8 [rows] tensor");
+    tah_topk_mix_args a{};
+    a.logits = ptr(logits); a.embedding = ptr(embedding); a.out = mptr(out);
+    a.row_enable = static_cast<const uint8_t*>(ptr(row_enable));
+    a.logits_row_stride = rows > 1 ? logits.stride(0) : logits.size(1);
+    a.embedding_row_stride = embedding.stride(0);
+    a.out_row_stride = rows > 1 ? out.stride(0) : H;
+    a.rows = (int32_t)rows; a.vocab = (int32_t)logits.size(1); a.hidden = (int32_t)H; a.topk = (int32_t)topk;
+    check_rc(g.topk_mix(&a, d.stream()), "tah_topk_mix");
+    return out;
+}
+
+Tensor silu_mul(const Tensor& gate_up) {
+    need_lib();
+    Dev d; d.see(gate_up);
+    TORCH_CHECK(gate_up.dim() == 2 && gate_up.scalar_type() == at::kBFloat16 && gate_up.size(1) % 16 == 0 && gate_up.stride(1) == 1,
+                "silu_mul: gate_up must be bf16 [rows, 2*I] with I a multiple of 8 and a contiguous inner dimension");
+    const int64_t rows = gate_up.size(0), inter = gate_up.size(1) / 2;
+    auto out = at::empty({rows, inter}, gate_up.options());
+    check_rc(g.silu_mul(ptr(gate_up), mptr(out), (int32_t)rows, (int32_t)inter, rows > 1 ? gate_up.stride(0) : 2 * inter, inter, d.stream()),
+             "tah_silu_mul");
+    return out;
+}
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+    m.doc() = "PyTorch-ROCm binding of the duo-causal attention C ABI (include/tah_duo.h)";
+    m.def("load_library", &load_library, py::arg("path"), py::arg("allow_host") = false);
+    m.def("loaded", [] { return g.handle != nullptr; });
+    m.def("abi_version", [] { need_lib(); return g.abi_version(); });
+    m.def("duo_fwd_varlen", &duo_fwd_varlen);
+    m.def("duo_bwd_varlen", &duo_bwd_varlen);
+    m.def("duo_fwd_masked", &duo_fwd_masked);
+    m.def("duo_bwd_masked", &duo_bwd_masked);
+    m.def("decode_workspace_bytes", &decode_workspace_bytes);
+    m.def("duo_decode", &duo_decode);
+    m.def("kv_append", &kv_append);
+    m.def("qk_prep", &qk_prep);
+    m.def("hard_index_build", &hard_index_build);
+    m.def("pad_rows_build", &pad_rows_build);
+    m.def("rows_copy", &rows_copy);
+    m.def("topk_mix", &topk_mix);
+    m.def("silu_mul", &silu_mul);
+}

@@ -37,13 +37,15 @@ def build(san: str = "") -> str:
 
 @contextlib.contextmanager
 def emulated():
-    """Route tah_amd.ops to the CPU execution build for the duration of the block."""
-    from tah_amd import _capi, _lib, ops
+    """Have the package's extension open the CPU execution build (and accept host tensors) for the duration of
+    the block; afterwards it opens the MI355X library again.  Yields the same library bound with ctypes, for
+    tests that call the C ABI directly."""
+    from tah_amd import _capi, _lib
 
-    lib = _capi.bind(ctypes.CDLL(build()))
-    old = (_lib._lib, ops._HOST_POINTERS_OK)
-    _lib._lib, ops._HOST_POINTERS_OK = lib, True
+    path = build()
+    ext = _lib.ext()
+    ext.load_library(path, True)
     try:
-        yield lib
+        yield _capi.bind(ctypes.CDLL(path))
     finally:
-        _lib._lib, ops._HOST_POINTERS_OK = old
+        ext.load_library(_lib.LIB_PATH, False)

@@ -20,9 +20,20 @@ def test_header_symbols_are_exported_and_bound():
     for n in names:
         assert hasattr(lib, n), f"{n} declared in include/tah_duo.h but not exported by libtah_duo.so"
     assert sorted(_capi.PROTOTYPES) == names
-    bound = _lib.lib()
+    bound = _capi.bind(lib)
     assert bound.tah_duo_abi_version() == _capi.ABI_VERSION
     assert bound.tah_duo_error_string(-2).decode().startswith("unsupported shape")
+
+
+def test_torch_extension_loads_the_library_and_exposes_every_op():
+    """The PyTorch extension (the binding the package uses) opens libtah_duo.so without a GPU, agrees on the ABI
+    version and has one function per compute entry point of the header."""
+    from tah_amd import _capi, _lib
+    ext = _lib.lib()
+    assert ext.loaded() and ext.abi_version() == _capi.ABI_VERSION
+    for n in ("duo_fwd_varlen", "duo_bwd_varlen", "duo_fwd_masked", "duo_bwd_masked", "duo_decode", "decode_workspace_bytes",
+              "kv_append", "qk_prep", "hard_index_build", "pad_rows_build", "rows_copy", "topk_mix", "silu_mul"):
+        assert callable(getattr(ext, n))
 
 
 def test_struct_sizes_match_c_layout():
@@ -48,7 +59,7 @@ def test_argument_checks_run_before_any_device_work():
     and no GPU are enough to see the error codes for a bad head dimension, a misaligned pointer and a
     row stride beyond what the tile copies can address."""
     from tah_amd import _capi, _lib
-    lib = _lib.lib()
+    lib = _capi.bind(ctypes.CDLL(_lib.LIB_PATH))
 
     def args():
         a = _capi.DuoFwdArgs()

@@ -101,7 +101,7 @@ def test_decode_query_before_end_of_cache_sees_prefix_only():
 def test_decode_rejects_small_workspace_and_bad_shapes():
     import ctypes
     from tah_amd import _capi, _lib
-    lib = _lib.lib()
+    lib = _capi.bind(ctypes.CDLL(_lib.LIB_PATH))
     a = _capi.DuoDecodeArgs()
     a.d, a.nq, a.hq, a.hkv = 64, 1, 2, 1
     assert lib.tah_duo_decode(ctypes.byref(a), None) == -2
