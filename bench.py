@@ -28,6 +28,10 @@ PEAK_HBM_GBS = 8000.0
 TRAFFIC_FWD_BYTES = 203.3e6 + 72.2e6
 TRAFFIC_DECODE_BYTES = 2.329e9 + 5.1e6 + 5.2e6 + 0.3e6
 TRAFFIC_QK_PREP_BYTES = 142.7e6 + 134.2e6
+# forward + backward legs, all kernels of one step (forward, two delta kernels, dQ, dK/dV): bytes fetched + written
+# (profiles/duo_fwd_bwd_seq8192_and_4docs_counters.md)
+TRAFFIC_FWD_BWD_SEQ8192_BYTES = 610.5e6 + 113.2e6
+TRAFFIC_FWD_BWD_4DOCS_BYTES = 439.6e6 + 116.9e6
 
 
 def visible_pairs(case):
@@ -356,10 +360,10 @@ def main() -> int:
     if args.only in ("all", "fwd_bwd"):
       extra["fwd_bwd_seq8192_p06"] = bench_fwd_bwd(
         "north-star headline: fwd+bwd, one sequence of 8192, p_hard=0.06, Hq=16, Hkv=8, D=128", [8192], 0.06, 1238,
-        max(args.steps // 2, 1), max(args.warmup // 2, 1))
+        max(args.steps // 2, 1), max(args.warmup // 2, 1), TRAFFIC_FWD_BWD_SEQ8192_BYTES)
       extra["fwd_bwd_4docs_p10"] = bench_fwd_bwd(
         "configs[3]: fwd+bwd, 8192 packed tokens in 4 documents, p_hard=0.10", [1397, 3210, 2561, 1024], 0.10, 1237,
-        max(args.steps // 2, 1), max(args.warmup // 2, 1))
+        max(args.steps // 2, 1), max(args.warmup // 2, 1), TRAFFIC_FWD_BWD_4DOCS_BYTES)
 
     if args.only in ("all", "qk_prep"):
         extra["qk_prep_prefill"] = bench_qk_prep(args.steps, args.warmup)

@@ -149,6 +149,7 @@ class TaHDecodeEngine:
         self.n_steps = torch.zeros((), dtype=torch.long, device=dev)      # tokens decoded (active rows x steps)
         self.step_idx = torch.zeros(1, dtype=torch.long, device=dev)
         self.out_tokens = torch.zeros(batch, max_len, dtype=torch.long, device=dev)  # generated tokens, column = step
+        self.out_len = torch.zeros(batch, dtype=torch.int32, device=dev)             # tokens of each row before its end
         self.scale = float(cfg.head_dim) ** -0.5
         self.host_positions = 0  # upper bound on any sequence's length, kept on the host for capacity checks
         self.host_hard_rows = 0
@@ -297,78 +298,137 @@ class TaHDecodeEngine:
 
     # ── sampling / generation ────────────────────────────────────────────
     @staticmethod
-    def sample(logits: torch.Tensor, temperature: float) -> torch.Tensor:
-        """Batched: greedy at temperature 0, else the Gumbel-max form of sampling from softmax(logits / T)."""
+    def sample(logits: torch.Tensor, temperature: float = 0.0, *, top_p: float = 1.0, top_k: int = 0, min_p: float = 0.0) -> torch.Tensor:
+        """One token per row, batched on the device: ``sample_next_token`` of the reference
+        (tah/model/utils.py:84-125) -- temperature, softmax, then min_p / top_k / top_p filters with
+        renormalisation, then one draw per row -- with ``temperature <= 0`` meaning ``do_sample=False`` (arg-max).
+        The draw is the exponential-race form of a multinomial draw (arg-max of p / e, e ~ Exp(1)), which can be
+        captured in a graph."""
         if temperature <= 0.0:
             return torch.argmax(logits, dim=-1)
-        u = torch.empty_like(logits).exponential_()
-        return torch.argmax(logits / temperature - torch.log(u), dim=-1)
+        probs = F.softmax(logits / temperature if temperature != 1.0 else logits, dim=-1)
+        if min_p > 0.0:
+            probs = torch.where(probs >= min_p * probs.max(dim=-1, keepdim=True).values, probs, torch.zeros_like(probs))
+            probs = probs / probs.sum(dim=-1, keepdim=True)
+        if top_k > 0:
+            kth = torch.topk(probs, min(top_k, probs.size(-1)), dim=-1).values[..., -1:]
+            probs = torch.where(probs < kth, torch.zeros_like(probs), probs)
+            probs = probs / probs.sum(dim=-1, keepdim=True)
+        if top_p < 1.0:
+            sp, si = torch.sort(probs, descending=True, dim=-1)
+            remove = torch.cumsum(sp, dim=-1) > top_p
+            remove = torch.cat([torch.zeros_like(remove[..., :1]), remove[..., :-1]], dim=-1)  # keep the one that crosses
+            probs = torch.where(torch.zeros_like(remove).scatter_(-1, si, remove), torch.zeros_like(probs), probs)
+            probs = probs / probs.sum(dim=-1, keepdim=True)
+        return torch.argmax(probs / torch.empty_like(probs).exponential_(), dim=-1)
 
-    def _step_inplace(self, temperature: float, eos: int):
+    def _step_inplace(self, temperature: float, eos: int, **filters):
         """One generated token for every unfinished row; every state change is an in-place device update."""
         act = ~self.finished
         logits, hard = self.step_logits(self.tok, active=act)
-        nxt = self.sample(logits, temperature)
+        nxt = self.sample(logits, temperature, **filters)
         nxt = torch.where(act, nxt, torch.zeros_like(nxt))
-        self.out_tokens.scatter_(1, self.step_idx.expand(self.B, 1), nxt[:, None])
+        if eos >= 0:
+            self.finished |= nxt == eos
+        # a row's output ends before its end-of-sequence token (utils.py:241-245); finished rows write zeros
+        keep = ~self.finished
+        self.out_tokens.scatter_(1, self.step_idx.expand(self.B, 1), torch.where(keep, nxt, torch.zeros_like(nxt))[:, None])
+        self.out_len += keep.to(torch.int32)
         self.n_hard += hard.sum()
         self.n_steps += act.sum()
         self.pos += act.to(torch.int32)
         self.step_idx += 1
-        if eos >= 0:
-            self.finished |= nxt == eos
         self.tok.copy_(nxt)
+
+    def _state(self):
+        return (self.tok, self.pos, self.finished, self.n_hard, self.n_steps, self.step_idx, self.out_tokens, self.out_len)
 
     @torch.no_grad()
     def generate(self, first_logits: torch.Tensor, max_new_tokens: int, *, temperature: float = 0.0, eos: int = -1,
-                 use_graph: bool = True):
-        """Continues after :meth:`prefill`.  Returns tokens int64 [B, max_new_tokens] (0 after a row's end)."""
+                 use_graph: bool = True, check_every: int = 64, **filters):
+        """Continues after :meth:`prefill`.  Returns tokens int64 [B, max_new_tokens]; a row's tokens end before its
+        end-of-sequence token and are 0 from there on (``self.out_len`` holds each row's count).  With ``eos`` the
+        loop looks every ``check_every`` steps whether all rows are done (the only host synchronisation)."""
         if self.host_positions + max_new_tokens > self.max_len or self.host_hard_rows + max_new_tokens > self.max_hard:
             raise TahDuoError("generation would outgrow the KV slabs: construct the engine with a larger max_len / max_hard")
         dev = self.device
         self.out_tokens.zero_()
+        self.out_len.zero_()
         self.step_idx.zero_()
-        first = self.sample(first_logits, temperature)
-        self.out_tokens[:, 0] = first
-        self.tok.copy_(first)
+        first = self.sample(first_logits, temperature, **filters)
         if eos >= 0:
             self.finished |= first == eos
+        keep = ~self.finished
+        self.out_tokens[:, 0] = torch.where(keep, first, torch.zeros_like(first))
+        self.out_len += keep.to(torch.int32)
+        self.tok.copy_(first)
         self.step_idx += 1
         n = max_new_tokens - 1
-        if n <= 0:
-            return self.out_tokens[:, :max_new_tokens]
-        if use_graph and dev.type == "cuda":
-            self.capture(temperature, eos)
-            for _ in range(n):
-                self._graph.replay()
-        else:
-            for _ in range(n):
-                self._step_inplace(temperature, eos)
-        self.host_positions += n
-        self.host_hard_rows += n
+        graph = self.capture(temperature, eos, **filters) if (use_graph and dev.type == "cuda" and n > 0) else None
+        done = 0
+        for i in range(n):
+            if graph is not None:
+                graph.replay()
+            else:
+                self._step_inplace(temperature, eos, **filters)
+            done += 1
+            if eos >= 0 and (i + 1) % check_every == 0 and bool(self.finished.all()):
+                break
+        self.host_positions += done
+        self.host_hard_rows += done
         return self.out_tokens[:, :max_new_tokens]
 
-    def capture(self, temperature: float = 0.0, eos: int = -1):
+    def capture(self, temperature: float = 0.0, eos: int = -1, **filters):
         """Captures one generation step in a HIP graph (after a warm-up step run on a side stream whose state
         changes are undone, so that library workspaces exist before the capture)."""
-        if self._graph is not None and self._graph_key == (temperature, eos):
+        key = (temperature, eos, tuple(sorted(filters.items())), self.measure_without_attention)
+        if self._graph is not None and self._graph_key == key:
             return self._graph
-        state = [t.clone() for t in (self.tok, self.pos, self.finished, self.n_hard, self.n_steps, self.step_idx, self.out_tokens)]
-        lens = [(s.len.clone(), ) for s in self.slabs0 + self.slabs1]
+        state = [t.clone() for t in self._state()]
+        lens = [sl.len.clone() for sl in self.slabs0 + self.slabs1]
         s = torch.cuda.Stream()
         s.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(s):
-            self._step_inplace(temperature, eos)
+            self._step_inplace(temperature, eos, **filters)
         torch.cuda.current_stream().wait_stream(s)
         torch.cuda.synchronize()
         # undo the warm-up step: state tensors and slab lengths (the rows it wrote lie beyond the lengths)
-        for t, old in zip((self.tok, self.pos, self.finished, self.n_hard, self.n_steps, self.step_idx, self.out_tokens), state):
+        for t, old in zip(self._state(), state):
             t.copy_(old)
-        for sl, (ln,) in zip(self.slabs0 + self.slabs1, lens):
+        for sl, ln in zip(self.slabs0 + self.slabs1, lens):
             sl.len.copy_(ln)
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
-            self._step_inplace(temperature, eos)
-        # the capture itself does not run the step
-        self._graph, self._graph_key = g, (temperature, eos)
+            self._step_inplace(temperature, eos, **filters)
+        self._graph, self._graph_key = g, key
         return g
+
+
+def generate(engine: TaHDecodeEngine, tokenizer, model_inputs: dict, *, max_new_tokens: int = 1024, do_sample: bool = True,
+             temperature: float = 1.0, top_p: float = 1.0, top_k: int = 0, min_p: float = 0.0, verbose: bool = False,
+             use_graph: bool = True, **kwargs):
+    """``TaHForCasualLM_generate`` (tah/model/utils.py:196-264) on the engine: same arguments (the engine in the
+    model's place) and the same return value ``(output_tokens, generated_texts)`` -- per batch row the list of
+    generated token ids up to, not including, the end-of-sequence token, and their decoded strings.
+
+    ``model_inputs["input_ids"]`` (B, T) with an optional left-padding ``attention_mask``; the prompts are packed
+    (pad tokens dropped) before the prefill.  Tokens are read back once, after the loop, not row by row per step
+    (utils.py:243-245).  ``verbose`` (the reference prints every token coloured by its iteration count) is
+    accepted and ignored."""
+    del verbose, kwargs
+    ids = model_inputs["input_ids"].to(engine.device)
+    B, T = ids.shape
+    if B != engine.B:
+        raise TahDuoError(f"the engine was built for batch {engine.B}, got {B}")
+    mask = model_inputs.get("attention_mask")
+    valid = torch.ones_like(ids, dtype=torch.bool) if mask is None else mask.to(engine.device) != 0
+    lens = valid.sum(1)
+    cu = torch.cat([torch.zeros(1, dtype=lens.dtype, device=lens.device), lens.cumsum(0)]).to(torch.int32)
+    first, _ = engine.prefill(ids[valid], cu)
+    eos = tokenizer.eos_token_id if getattr(tokenizer, "eos_token_id", None) is not None else -1
+    t = float(temperature) if do_sample else 0.0
+    toks = engine.generate(first, max_new_tokens, temperature=t, eos=int(eos), use_graph=use_graph,
+                           top_p=float(top_p), top_k=int(top_k), min_p=float(min_p))
+    toks_h, len_h = toks.cpu(), engine.out_len.cpu()  # the one read-back
+    out = [toks_h[b, : int(len_h[b])].tolist() for b in range(B)]
+    return out, [tokenizer.decode(t_) if t_ else "" for t_ in out]

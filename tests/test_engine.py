@@ -68,3 +68,66 @@ def test_engine_graph_replay_equals_eager_gpu():
         runs.append((toks, int(eng.n_hard), [sl.len.tolist() for sl in eng.slabs0 + eng.slabs1], eng.pos.tolist()))
     assert torch.equal(runs[0][0], runs[1][0]) and runs[0][1:] == runs[1][1:]
     assert runs[0][1] > 0  # some token took the second iteration
+
+
+def test_sampling_filters_follow_the_reference_semantics():
+    """``TaHDecodeEngine.sample`` against the rules of ``sample_next_token`` (tah/model/utils.py:84-125): arg-max
+    when not sampling; min_p / top_k / top_p each confine the draw to the set the rule names."""
+    from tah_amd.engine import TaHDecodeEngine as E
+    g = torch.Generator().manual_seed(0)
+    logits = torch.randn(6, 50, generator=g) * 2
+    am = logits.argmax(-1)
+    assert torch.equal(E.sample(logits, 0.0), am)
+    torch.manual_seed(1)
+    for kw in (dict(top_k=1), dict(min_p=1.0), dict(top_p=1e-6)):
+        assert torch.equal(E.sample(logits, 0.7, **kw), am), kw
+    probs = torch.softmax(logits / 0.7, -1)
+    top3 = probs.topk(3, -1).indices
+    sp, si = probs.sort(descending=True, dim=-1)
+    # top_p = 0.5: the smallest prefix of the sorted distribution whose mass reaches 0.5
+    npfx = ((sp.cumsum(-1) - sp) < 0.5).sum(-1)
+    seen_k, seen_p = set(), set()
+    for _ in range(300):
+        a = E.sample(logits, 0.7, top_k=3)
+        assert all(a[r] in top3[r] for r in range(6))
+        seen_k.add(int(a[0]))
+        b = E.sample(logits, 0.7, top_p=0.5)
+        assert all(b[r] in si[r, : int(npfx[r])] for r in range(6))
+        c = E.sample(logits, 0.7, min_p=0.3)
+        assert all(probs[r, c[r]] >= 0.3 * probs[r].max() for r in range(6))
+    assert len(seen_k) > 1  # it does sample
+    # the draw follows the distribution: frequencies of a 3-way choice within 4 sigma
+    lg = torch.log(torch.tensor([[0.6, 0.3, 0.1]])).expand(4000, 3)
+    freq = torch.bincount(E.sample(lg, 1.0), minlength=3).float() / 4000
+    assert (freq - torch.tensor([0.6, 0.3, 0.1])).abs().max() < 4 * (0.25 / 4000) ** 0.5
+
+
+@pytest.mark.gpu
+def test_generate_wrapper_returns_tokens_up_to_eos_gpu():
+    """``tah_amd.engine.generate`` (the call signature and return value of TaHForCasualLM_generate): greedy tokens
+    equal the engine's own stepping; with an end-of-sequence id a row's list stops before it, other rows go on."""
+    import types
+
+    from tah_amd.engine import EngineConfig, TaHDecodeEngine, Weights, generate
+    cfg = EngineConfig(hidden=256, layers=2, hq=4, hkv=2, head_dim=128, intermediate=512, vocab=300, decider_hidden=32)
+    w = Weights.random_init(cfg, "cuda", seed=5)
+    B, T, new = 3, 20, 24
+    g = torch.Generator().manual_seed(2)
+    ids = torch.randint(0, cfg.vocab, (B, T), generator=g).cuda()
+    mask = torch.ones(B, T, dtype=torch.long, device="cuda")
+    mask[1, :6] = 0  # a left-padded prompt
+    tok = types.SimpleNamespace(eos_token_id=None, decode=lambda t: " ".join(map(str, t)))
+    w.threshold = 0.45
+    free, texts = generate(TaHDecodeEngine(w, B, T + new + 2), tok, dict(input_ids=ids, attention_mask=mask),
+                           max_new_tokens=new, do_sample=False)
+    assert [len(t) for t in free] == [new] * B and texts[0] == " ".join(map(str, free[0]))
+    eager, _ = generate(TaHDecodeEngine(w, B, T + new + 2), tok, dict(input_ids=ids, attention_mask=mask),
+                        max_new_tokens=new, do_sample=False, use_graph=False)
+    assert eager == free
+    tok.eos_token_id = free[0][5]
+    cut, _ = generate(TaHDecodeEngine(w, B, T + new + 2), tok, dict(input_ids=ids, attention_mask=mask),
+                      max_new_tokens=new, do_sample=False)
+    for b in range(B):
+        stop = free[b].index(tok.eos_token_id) if tok.eos_token_id in free[b] else new
+        assert cut[b] == free[b][:stop], b
+    assert len(cut[0]) <= 5
