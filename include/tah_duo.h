@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define TAH_DUO_ABI_VERSION 2
+#define TAH_DUO_ABI_VERSION 3
 
 enum {
     TAH_OK = 0,
@@ -68,6 +68,7 @@ typedef struct tah_duo_fwd_args {
     tah_duo_stream s2;      /* depth 1: hard tokens; total_q may be 0 */
     int32_t nseq, hq, hkv, d;
     float scale;            /* softmax scale, head_dim**-0.5 in Qwen3 */
+    const void* schedule;   /* launch-order table from tah_duo_schedule_build for these boundaries, or NULL */
 } tah_duo_fwd_args;
 
 int tah_duo_abi_version(void);
@@ -83,6 +84,32 @@ const char* tah_duo_error_string(int code);
  * pointer and is read before the call returns.  Rows with no visible key get
  * o = 0, lse = -inf. */
 int tah_duo_fwd_varlen(const tah_duo_fwd_args* args, tah_stream_t stream);
+
+/* Launch order of a varlen call's tiles, heaviest first (optional).  The kernels start one workgroup per
+ * (kv head, 128-row tile); with several documents of unequal length in a batch, handing the tiles out in
+ * sequence order leaves the long tiles of later documents for the end of the launch.  This call sorts the
+ * tiles of both depths by the work they will do, on the device, from the same boundary arrays the
+ * attention calls take; pass the table as `schedule` to tah_duo_fwd_varlen / tah_duo_bwd_varlen as long as
+ * nseq, the totals, hq / hkv and the contents of cu_* and pos_q2 stay what they were when it was built
+ * (one table serves every layer and the backward pass of a batch).  A table that does not fit a call's
+ * sizes is ignored.  It changes the order in which tiles are started, never a result.
+ * No counterpart in the reference, whose SDPA call launches a dense rectangular problem
+ * (transformers/integrations/sdpa_attention.py:79-166). */
+typedef struct tah_duo_schedule_args {
+    const int32_t* cu_q1;   /* int32 [nseq+1] depth-0 query boundaries */
+    const int32_t* cu_k1;   /* int32 [nseq+1] depth-0 key boundaries */
+    const int32_t* cu_q2;   /* depth 1; may be NULL when total_q2 == 0 */
+    const int32_t* cu_k2;   /* may be NULL when total_k2 == 0 */
+    const int32_t* pos_q2;  /* int32 [total_q2] positions of the depth-1 query rows */
+    int32_t nseq, hq, hkv;  /* nseq <= 4095 */
+    int32_t total_q1, total_k1, total_q2, total_k2;
+    void* schedule;         /* >= tah_duo_schedule_bytes(...) bytes, 4-byte aligned */
+    size_t schedule_bytes;
+} tah_duo_schedule_args;
+
+size_t tah_duo_schedule_bytes(int32_t nseq, int32_t hq, int32_t hkv, int32_t total_q1, int32_t total_k1,
+                              int32_t total_q2, int32_t total_k2);
+int tah_duo_schedule_build(const tah_duo_schedule_args* args, tah_stream_t stream);
 
 /* A dense additive attention mask as Hugging Face passes it: element
  * [seq b][head h][query i][key j], i and j counted inside sequence b (row

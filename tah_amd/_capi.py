@@ -8,7 +8,7 @@ from __future__ import annotations
 
 import ctypes as C
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 c_void_p, c_int32, c_int64, c_float = C.c_void_p, C.c_int32, C.c_int64, C.c_float
 
@@ -39,6 +39,18 @@ class DuoFwdArgs(C.Structure):
         ("s1", DuoStream), ("s2", DuoStream),
         ("nseq", c_int32), ("hq", c_int32), ("hkv", c_int32), ("d", c_int32),
         ("scale", c_float),
+        ("schedule", c_void_p),
+    ]
+
+
+class DuoScheduleArgs(C.Structure):
+    """``tah_duo_schedule_args``"""
+
+    _fields_ = [
+        ("cu_q1", c_void_p), ("cu_k1", c_void_p), ("cu_q2", c_void_p), ("cu_k2", c_void_p), ("pos_q2", c_void_p),
+        ("nseq", c_int32), ("hq", c_int32), ("hkv", c_int32),
+        ("total_q1", c_int32), ("total_k1", c_int32), ("total_q2", c_int32), ("total_k2", c_int32),
+        ("schedule", c_void_p), ("schedule_bytes", C.c_size_t),
     ]
 
 
@@ -145,6 +157,8 @@ PROTOTYPES = {
     "tah_duo_error_string": (C.c_char_p, [C.c_int]),
     "tah_duo_fwd_varlen": (C.c_int, [C.POINTER(DuoFwdArgs), c_void_p]),
     "tah_duo_bwd_varlen": (C.c_int, [C.POINTER(DuoBwdArgs), c_void_p]),
+    "tah_duo_schedule_bytes": (C.c_size_t, [c_int32] * 7),
+    "tah_duo_schedule_build": (C.c_int, [C.POINTER(DuoScheduleArgs), c_void_p]),
     "tah_duo_fwd_masked": (C.c_int, [C.POINTER(DuoFwdArgs), C.POINTER(AdditiveMask), c_void_p]),
     "tah_duo_bwd_masked": (C.c_int, [C.POINTER(DuoBwdArgs), C.POINTER(AdditiveMask), c_void_p]),
     "tah_duo_decode_workspace_bytes": (C.c_size_t, [c_int32, c_int32, c_int32, c_int32]),

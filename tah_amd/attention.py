@@ -34,10 +34,12 @@ from .pack import HardIndex
 
 class _DuoAttnVarlen(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, q1, k1, v1, q2, k2, v2, cu_q1, cu_k1, pos_q2, pos_k2, cu_q2, cu_k2, scale):
-        o1, lse1, o2, lse2 = ops.duo_fwd_varlen(q1, k1, v1, cu_q1, cu_k1, q2, k2, v2, pos_q2, pos_k2, cu_q2, cu_k2, scale)
+    def forward(ctx, q1, k1, v1, q2, k2, v2, cu_q1, cu_k1, pos_q2, pos_k2, cu_q2, cu_k2, scale, schedule=None):
+        o1, lse1, o2, lse2 = ops.duo_fwd_varlen(q1, k1, v1, cu_q1, cu_k1, q2, k2, v2, pos_q2, pos_k2, cu_q2, cu_k2, scale,
+                                                schedule)
         ctx.save_for_backward(q1, k1, v1, o1, lse1, q2, k2, v2, o2, lse2, cu_q1, cu_k1, pos_q2, pos_k2, cu_q2, cu_k2)
         ctx.scale = scale
+        ctx.schedule = schedule
         ctx.mark_non_differentiable(lse1, lse2)
         return o1, o2, lse1, lse2
 
@@ -47,21 +49,23 @@ class _DuoAttnVarlen(torch.autograd.Function):
         c = lambda g, like: (torch.zeros_like(like) if g is None else g.contiguous())
         dq1, dk1, dv1, dq2, dk2, dv2 = ops.duo_bwd_varlen(
             q1, k1, v1, o1, lse1, c(do1, o1), cu_q1, cu_k1, q2, k2, v2, o2, lse2, c(do2, o2),
-            pos_q2, pos_k2, cu_q2, cu_k2, ctx.scale)
-        return dq1, dk1, dv1, dq2, dk2, dv2, None, None, None, None, None, None, None
+            pos_q2, pos_k2, cu_q2, cu_k2, ctx.scale, ctx.schedule)
+        return dq1, dk1, dv1, dq2, dk2, dv2, None, None, None, None, None, None, None, None
 
 
 def duo_attn_varlen(q1, k1, v1, cu_q1, cu_k1, q2, k2, v2, pos_q2, pos_k2, cu_q2, cu_k2, scale: float,
-                    return_lse: bool = False):
+                    return_lse: bool = False, schedule=None):
     """Duo-causal attention on packed varlen bf16 tensors, differentiable.
 
     Depth-0 stream: q1 [T1q,Hq,D], k1/v1 [T1k,Hkv,D], cu_q1/cu_k1 int32 [nseq+1].
     Depth-1 stream (hard tokens): q2 [T2q,Hq,D], k2/v2 [T2k,Hkv,D], int32 positions
     pos_q2/pos_k2 and cu_q2/cu_k2.  Key (pos_k, depth_k) is visible to query
-    (pos_q, depth_q) iff pos_k <= pos_q and depth_k <= depth_q.  Returns (o1, o2).
+    (pos_q, depth_q) iff pos_k <= pos_q and depth_k <= depth_q.  ``schedule``: the launch-order table
+    :func:`tah_amd.ops.duo_schedule` built for these boundaries (forward and backward use it), or None.
+    Returns (o1, o2).
     """
     o1, o2, lse1, lse2 = _DuoAttnVarlen.apply(q1, k1, v1, q2, k2, v2, cu_q1, cu_k1, pos_q2, pos_k2, cu_q2, cu_k2,
-                                              float(scale))
+                                              float(scale), schedule)
     return (o1, o2, lse1, lse2) if return_lse else (o1, o2)
 
 
@@ -102,6 +106,7 @@ class DuoMask:
     def __init__(self, position_ids: torch.Tensor, valid_mask: torch.Tensor, cache: Optional[TaHDuoCache], iter_depth: int):
         self.position_ids, self.valid_mask, self.cache, self.iter_depth = position_ids, valid_mask, cache, iter_depth
         self._packed = None  # per-step packing metadata, shared by all decoder layers
+        self._sched = None   # launch-order table of the step's varlen calls, likewise
 
     def dense(self, dtype: torch.dtype = torch.float32) -> Optional[torch.Tensor]:
         """The (B,1,Tq,Tkv) additive mask the reference would have built (for inspection only)."""
@@ -357,15 +362,37 @@ def duo_attention_forward(module, query: torch.Tensor, key: torch.Tensor, value:
     zc = torch.zeros(B + 1, dtype=torch.int32, device=dev)
     zi = torch.zeros(0, dtype=torch.int32, device=dev)
     k1, v1, cu_k1, _ = _segment(cache, layer, 0, B, with_pos=False)
+    Hkv = k1.shape[1]
     if depth == 0:
         e_q = q[:0]
         e_k = k1[:0]
-        o, _ = duo_attn_varlen(q, k1, v1, pq.cu, cu_k1, e_q, e_k, e_k, zi, zi, zc, zc, scale)
+        sched = _schedule_of(m, (pq.cu, cu_k1, zc, zc, zi, Hq, Hkv, q.shape[0], k1.shape[0], 0))
+        o, _ = duo_attn_varlen(q, k1, v1, pq.cu, cu_k1, e_q, e_k, e_k, zi, zi, zc, zc, scale, schedule=sched)
     else:
         k2, v2, cu_k2, pos_k2 = _segment(cache, layer, 1, B, with_pos=True)
         e_q = q[:0]
-        _, o = duo_attn_varlen(e_q, k1, v1, zc, cu_k1, q, k2, v2, pq.pos, pos_k2, pq.cu, cu_k2, scale)
+        sched = _schedule_of(m, (zc, cu_k1, pq.cu, cu_k2, pq.pos, Hq, Hkv, 0, k1.shape[0], k2.shape[0]))
+        _, o = duo_attn_varlen(e_q, k1, v1, zc, cu_k1, q, k2, v2, pq.pos, pos_k2, pq.cu, cu_k2, scale, schedule=sched)
     return pq.unpack(o, Hq, D), None
+
+
+# Calls with at least this many (query row, kv head) pairs get a launch-order table: below it a launch has about
+# one workgroup per compute unit and the order does not matter.
+SCHEDULE_MIN_ROW_HEADS = 49152
+
+
+def _schedule_of(m: "DuoMask", args):
+    """The launch-order table of this mask's varlen calls: built at the first layer, shared by the others (the
+    boundaries of queries and cached keys are the same in every layer of a step) and by the backward pass."""
+    cu_q1, cu_k1, cu_q2, cu_k2, pos_q2, hq, hkv, tq1, tk1, tk2 = args
+    if (tq1 + pos_q2.shape[0]) * hkv < SCHEDULE_MIN_ROW_HEADS:
+        return None
+    key = (tq1, tk1, pos_q2.shape[0], tk2, hq, hkv, cu_k1.data_ptr(), cu_k2.data_ptr())
+    memo = getattr(m, "_sched", None)
+    if memo is None or memo[0] != key:
+        memo = (key, ops.duo_schedule(cu_q1, cu_k1, cu_q2, cu_k2, pos_q2, hq, hkv, tq1, tk1, tk2), (cu_k1, cu_k2))
+        m._sched = memo
+    return memo[1]
 
 
 def register_with_transformers(name: str = "tah_duo") -> str:

@@ -47,6 +47,7 @@ struct BwdParams {
     BwdStream s1, s2;
     int32_t nseq, hq, hkv;
     float scale, scale_log2e;
+    const int32_t* sched;  // launch-order table or nullptr
     // additive-mask mode only: mask[seq][head][query index][key index], strides in elements
     const void* mask;
     int64_t mask_sb, mask_sh, mask_sq, mask_sk;
@@ -104,12 +105,20 @@ __global__ __launch_bounds__(kDqThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dq_
     const int half = lane / 32, col = lane % 32;
     const int hk = blockIdx.x;
 
-    int slot = (int)(gridDim.y - 1 - blockIdx.y);
     int seq = 0, row0 = 0, row_end = 0;
     bool second = false;
-    if (!(p.s1.total_q > 0 && find_tile(p.s1.cu_q, p.nseq, BM, slot, seq, row0, row_end))) {
-        if (!(p.s2.total_q > 0 && find_tile(p.s2.cu_q, p.nseq, BM, slot, seq, row0, row_end))) return;
-        second = true;
+    const int listed = sched_lookup(p.sched, false, p.nseq, G, p.s1.total_q, p.s2.total_q, p.s1.total_k, p.s2.total_k,
+                                    (int)gridDim.y, (int)blockIdx.y, second, seq, row0);
+    if (listed < 0) return;
+    if (listed > 0) {  // the table's order: heaviest tile of the whole call first
+        const int hi = const_i32(second ? p.s2.cu_q : p.s1.cu_q, seq + 1);
+        row_end = row0 + BM < hi ? row0 + BM : hi;
+    } else {
+        int slot = (int)(gridDim.y - 1 - blockIdx.y);  // late (heavy) tiles of each sequence first
+        if (!(p.s1.total_q > 0 && find_tile(p.s1.cu_q, p.nseq, BM, slot, seq, row0, row_end))) {
+            if (!(p.s2.total_q > 0 && find_tile(p.s2.cu_q, p.nseq, BM, slot, seq, row0, row_end))) return;
+            second = true;
+        }
     }
     const BwdStream& qs = second ? p.s2 : p.s1;
     const int head = hk * G + wave % G;
@@ -310,6 +319,7 @@ __global__ __launch_bounds__(kDqThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dq_
 constexpr int kKvThreads = 512;                           // 8 waves = 4 key blocks x 2 query halves
 constexpr int kKB = 4;                                    // 32-key blocks per workgroup
 constexpr int kBK = 32 * kKB;                             // keys per workgroup
+static_assert(kBK == kSchedKeyTile, "the launch-order table lists key tiles of this size");
 constexpr int kBQ = 64;                                   // query rows per staged tile
 constexpr int kKvSlot = 2 * kTileBytes;                   // one stage: Q tile, dO tile (32 KiB)
 constexpr int kKvK = 2 * kKvSlot;                         // after the two stages: this workgroup's K tile (128 x 128 bf16) ...
@@ -329,12 +339,20 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
     const int kb = wave % kKB, qh = wave / kKB;  // 32-key block, 32-row half of the query tile
     const int hk = blockIdx.x;
 
-    int slot = (int)blockIdx.y;
     int seq = 0, key0 = 0, key_end = 0;
     bool second = false;
-    if (!(p.s1.total_k > 0 && find_tile(p.s1.cu_k, p.nseq, kBK, slot, seq, key0, key_end))) {
-        if (!(p.s2.total_k > 0 && find_tile(p.s2.cu_k, p.nseq, kBK, slot, seq, key0, key_end))) return;
-        second = true;
+    const int listed = sched_lookup(p.sched, true, p.nseq, G, p.s1.total_q, p.s2.total_q, p.s1.total_k, p.s2.total_k,
+                                    (int)gridDim.y, (int)blockIdx.y, second, seq, key0);
+    if (listed < 0) return;
+    if (listed > 0) {  // the table's order: the key tile seen by the most query rows first
+        const int hi = const_i32(second ? p.s2.cu_k : p.s1.cu_k, seq + 1);
+        key_end = key0 + kBK < hi ? key0 + kBK : hi;
+    } else {
+        int slot = (int)blockIdx.y;  // early (heavy) key tiles of each sequence first
+        if (!(p.s1.total_k > 0 && find_tile(p.s1.cu_k, p.nseq, kBK, slot, seq, key0, key_end))) {
+            if (!(p.s2.total_k > 0 && find_tile(p.s2.cu_k, p.nseq, kBK, slot, seq, key0, key_end))) return;
+            second = true;
+        }
     }
     const BwdStream& ks = second ? p.s2 : p.s1;
     const int k_lo = ks.cu_k[seq];
@@ -790,6 +808,7 @@ int dispatch_bwd(const tah_duo_bwd_args* a, const tah_additive_mask* m, tah_stre
     p.hkv = f.hkv;
     p.scale = f.scale;
     p.scale_log2e = f.scale * kLog2e;
+    p.sched = kDense ? nullptr : static_cast<const int32_t*>(f.schedule);
     p.mask = nullptr;
     p.mask_sb = p.mask_sh = p.mask_sq = p.mask_sk = 0;
     p.mask_f32 = 0;

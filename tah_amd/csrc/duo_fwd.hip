@@ -70,6 +70,7 @@ struct FwdParams {
     FwdStream s1, s2;
     int32_t nseq, hq, hkv;
     float scale_log2e;
+    const int32_t* sched;  // launch-order table or nullptr
     // additive-mask mode only: mask[seq][head][query index][key index], strides in elements
     const void* mask;
     int64_t mask_sb, mask_sh, mask_sq, mask_sk;
@@ -95,12 +96,20 @@ __global__ __launch_bounds__(kThreads) TAH_WAVES_PER_EU(2, 2) void duo_fwd_kerne
     const int hk = blockIdx.x;
 
     // ---- which tile am I ---------------------------------------------------
-    int slot = (int)(gridDim.y - 1 - blockIdx.y);  // heavy (late) tiles first
     int seq = 0, row0 = 0, row_end = 0;
     bool second = false;
-    if (!(p.s1.total_q > 0 && find_tile(p.s1.cu_q, p.nseq, BM, slot, seq, row0, row_end))) {
-        if (!(p.s2.total_q > 0 && find_tile(p.s2.cu_q, p.nseq, BM, slot, seq, row0, row_end))) return;
-        second = true;
+    const int listed = sched_lookup(p.sched, false, p.nseq, G, p.s1.total_q, p.s2.total_q, p.s1.total_k, p.s2.total_k,
+                                    (int)gridDim.y, (int)blockIdx.y, second, seq, row0);
+    if (listed < 0) return;
+    if (listed > 0) {  // the table's order: heaviest tile of the whole call first
+        const int hi = const_i32(second ? p.s2.cu_q : p.s1.cu_q, seq + 1);
+        row_end = row0 + BM < hi ? row0 + BM : hi;
+    } else {
+        int slot = (int)(gridDim.y - 1 - blockIdx.y);  // late (heavy) tiles of each sequence first
+        if (!(p.s1.total_q > 0 && find_tile(p.s1.cu_q, p.nseq, BM, slot, seq, row0, row_end))) {
+            if (!(p.s2.total_q > 0 && find_tile(p.s2.cu_q, p.nseq, BM, slot, seq, row0, row_end))) return;
+            second = true;
+        }
     }
     const FwdStream& qs = second ? p.s2 : p.s1;
 
@@ -565,6 +574,7 @@ int dispatch_fwd(const tah_duo_fwd_args* a, const tah_additive_mask* m, tah_stre
     p.hq = a->hq;
     p.hkv = a->hkv;
     p.scale_log2e = a->scale * kLog2e;
+    p.sched = kDense ? nullptr : static_cast<const int32_t*>(a->schedule);
     p.mask = nullptr;
     p.mask_sb = p.mask_sh = p.mask_sq = p.mask_sk = 0;
     p.mask_f32 = 0;

@@ -26,6 +26,8 @@ struct Api {
     decltype(&tah_duo_error_string) error_string = nullptr;
     decltype(&tah_duo_fwd_varlen) fwd_varlen = nullptr;
     decltype(&tah_duo_bwd_varlen) bwd_varlen = nullptr;
+    decltype(&tah_duo_schedule_bytes) schedule_bytes = nullptr;
+    decltype(&tah_duo_schedule_build) schedule_build = nullptr;
     decltype(&tah_duo_fwd_masked) fwd_masked = nullptr;
     decltype(&tah_duo_bwd_masked) bwd_masked = nullptr;
     decltype(&tah_duo_decode_workspace_bytes) decode_workspace_bytes = nullptr;
@@ -57,6 +59,8 @@ void load_library(const std::string& path, bool allow_host) {
     bind(g.error_string, "tah_duo_error_string");
     bind(g.fwd_varlen, "tah_duo_fwd_varlen");
     bind(g.bwd_varlen, "tah_duo_bwd_varlen");
+    bind(g.schedule_bytes, "tah_duo_schedule_bytes");
+    bind(g.schedule_build, "tah_duo_schedule_build");
     bind(g.fwd_masked, "tah_duo_fwd_masked");
     bind(g.bwd_masked, "tah_duo_bwd_masked");
     bind(g.decode_workspace_bytes, "tah_duo_decode_workspace_bytes");
@@ -122,15 +126,46 @@ void fill_stream(tah_duo_stream& s, const Tensor& q, const Tensor& k, const Tens
     s.total_q = (int32_t)q.size(0); s.total_k = (int32_t)k.size(0);
 }
 
+const void* schedule_ptr(const optional<Tensor>& schedule) {
+    if (!schedule.has_value()) return nullptr;
+    TORCH_CHECK(schedule->scalar_type() == at::kInt && schedule->is_contiguous(), "schedule must be the int32 tensor duo_schedule returned");
+    return ptr(*schedule);
+}
+
+// Launch-order table for the varlen calls that use these boundaries (tah_duo_schedule_build).
+Tensor duo_schedule(const Tensor& cu_q1, const Tensor& cu_k1, const Tensor& cu_q2, const Tensor& cu_k2, const Tensor& pos_q2,
+                    int64_t hq, int64_t hkv, int64_t total_q1, int64_t total_k1, int64_t total_k2) {
+    need_lib();
+    i32(cu_q1, "cu_q1"); i32(cu_k1, "cu_k1"); i32(cu_q2, "cu_q2"); i32(cu_k2, "cu_k2"); i32(pos_q2, "pos_q2");
+    Dev d;
+    for (const Tensor* t : {&cu_q1, &cu_k1, &cu_q2, &cu_k2, &pos_q2}) d.see(*t);
+    const int64_t nseq = cu_q1.numel() - 1;
+    TORCH_CHECK(cu_k1.numel() == nseq + 1 && cu_q2.numel() == nseq + 1 && cu_k2.numel() == nseq + 1,
+                "cu_seqlens tensors must all have nseq+1 entries");
+    tah_duo_schedule_args a{};
+    a.cu_q1 = static_cast<const int32_t*>(cu_q1.data_ptr()); a.cu_k1 = static_cast<const int32_t*>(cu_k1.data_ptr());
+    a.cu_q2 = static_cast<const int32_t*>(cu_q2.data_ptr()); a.cu_k2 = static_cast<const int32_t*>(cu_k2.data_ptr());
+    a.pos_q2 = static_cast<const int32_t*>(ptr(pos_q2));
+    a.nseq = (int32_t)nseq; a.hq = (int32_t)hq; a.hkv = (int32_t)hkv;
+    a.total_q1 = (int32_t)total_q1; a.total_k1 = (int32_t)total_k1; a.total_q2 = (int32_t)pos_q2.numel(); a.total_k2 = (int32_t)total_k2;
+    const size_t bytes = g.schedule_bytes(a.nseq, a.hq, a.hkv, a.total_q1, a.total_k1, a.total_q2, a.total_k2);
+    TORCH_CHECK(bytes > 0, "duo_schedule: unsupported sizes");
+    auto out = at::empty({(int64_t)(bytes / sizeof(int32_t))}, cu_q1.options());
+    a.schedule = out.data_ptr(); a.schedule_bytes = bytes;
+    check_rc(g.schedule_build(&a, d.stream()), "tah_duo_schedule_build");
+    return out;
+}
+
 std::tuple<Tensor, Tensor, Tensor, Tensor> duo_fwd_varlen(const Tensor& q1, const Tensor& k1, const Tensor& v1, const Tensor& cu_q1,
                                                           const Tensor& cu_k1, const Tensor& q2, const Tensor& k2, const Tensor& v2,
                                                           const Tensor& pos_q2, const Tensor& pos_k2, const Tensor& cu_q2,
-                                                          const Tensor& cu_k2, double scale) {
+                                                          const Tensor& cu_k2, double scale, const optional<Tensor>& schedule) {
     need_lib();
     thd(q1, "q1"); thd(k1, "k1"); thd(v1, "v1"); thd(q2, "q2"); thd(k2, "k2"); thd(v2, "v2");
     i32(cu_q1, "cu_q1"); i32(cu_k1, "cu_k1"); i32(cu_q2, "cu_q2"); i32(cu_k2, "cu_k2"); i32(pos_q2, "pos_q2"); i32(pos_k2, "pos_k2");
     Dev d;
     for (const Tensor* t : {&q1, &k1, &v1, &q2, &k2, &v2, &cu_q1, &cu_k1, &cu_q2, &cu_k2, &pos_q2, &pos_k2}) d.see(*t);
+    d.see(schedule);
     const int64_t nseq = cu_q1.numel() - 1;
     TORCH_CHECK(cu_k1.numel() == nseq + 1 && cu_q2.numel() == nseq + 1 && cu_k2.numel() == nseq + 1,
                 "cu_seqlens tensors must all have nseq+1 entries");
@@ -145,6 +180,7 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> duo_fwd_varlen(const Tensor& q1, cons
     fill_stream(a.s1, q1, k1, v1, o1, lse1, cu_q1, cu_k1, nullptr, nullptr);
     fill_stream(a.s2, q2, k2, v2, o2, lse2, cu_q2, cu_k2, &pos_q2, &pos_k2);
     a.nseq = (int32_t)nseq; a.hq = (int32_t)hq; a.hkv = (int32_t)k1.size(1); a.d = (int32_t)dd; a.scale = (float)scale;
+    a.schedule = schedule_ptr(schedule);
     check_rc(g.fwd_varlen(&a, d.stream()), "tah_duo_fwd_varlen");
     return {o1, lse1, o2, lse2};
 }
@@ -160,7 +196,8 @@ void fill_bwd_stream(tah_duo_bwd_stream& s, const Tensor& d_o, const Tensor& dq,
 std::vector<Tensor> duo_bwd_varlen(const Tensor& q1, const Tensor& k1, const Tensor& v1, const Tensor& o1, const Tensor& lse1,
                                    const Tensor& do1, const Tensor& cu_q1, const Tensor& cu_k1, const Tensor& q2, const Tensor& k2,
                                    const Tensor& v2, const Tensor& o2, const Tensor& lse2, const Tensor& do2, const Tensor& pos_q2,
-                                   const Tensor& pos_k2, const Tensor& cu_q2, const Tensor& cu_k2, double scale) {
+                                   const Tensor& pos_k2, const Tensor& cu_q2, const Tensor& cu_k2, double scale,
+                                   const optional<Tensor>& schedule) {
     need_lib();
     for (auto p : {std::make_pair(&q1, "q1"), {&k1, "k1"}, {&v1, "v1"}, {&o1, "o1"}, {&do1, "do1"}, {&q2, "q2"}, {&k2, "k2"},
                    {&v2, "v2"}, {&o2, "o2"}, {&do2, "do2"}})
@@ -169,6 +206,7 @@ std::vector<Tensor> duo_bwd_varlen(const Tensor& q1, const Tensor& k1, const Ten
     Dev d;
     for (const Tensor* t : {&q1, &k1, &v1, &o1, &lse1, &do1, &q2, &k2, &v2, &o2, &lse2, &do2, &cu_q1, &cu_k1, &cu_q2, &cu_k2, &pos_q2, &pos_k2})
         d.see(*t);
+    d.see(schedule);
     TORCH_CHECK(do1.sizes() == q1.sizes() && do2.sizes() == q2.sizes() && o1.sizes() == q1.sizes() && o2.sizes() == q2.sizes(),
                 "o / dO shapes must match q");
     TORCH_CHECK(lse1.scalar_type() == at::kFloat && lse2.scalar_type() == at::kFloat && lse1.is_contiguous() && lse2.is_contiguous(),
@@ -183,6 +221,7 @@ std::vector<Tensor> duo_bwd_varlen(const Tensor& q1, const Tensor& k1, const Ten
     fill_stream(a.fwd.s2, q2, k2, v2, o2, lse2, cu_q2, cu_k2, &pos_q2, &pos_k2);
     a.fwd.nseq = (int32_t)(cu_q1.numel() - 1); a.fwd.hq = (int32_t)hq; a.fwd.hkv = (int32_t)k1.size(1); a.fwd.d = (int32_t)q1.size(2);
     a.fwd.scale = (float)scale;
+    a.fwd.schedule = schedule_ptr(schedule);
     fill_bwd_stream(a.g1, do1, dq1, dk1, dv1, delta1);
     fill_bwd_stream(a.g2, do2, dq2, dk2, dv2, delta2);
     check_rc(g.bwd_varlen(&a, d.stream()), "tah_duo_bwd_varlen");
@@ -466,6 +505,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("load_library", &load_library, py::arg("path"), py::arg("allow_host") = false);
     m.def("loaded", [] { return g.handle != nullptr; });
     m.def("abi_version", [] { need_lib(); return g.abi_version(); });
+    m.def("duo_schedule", &duo_schedule);
     m.def("duo_fwd_varlen", &duo_fwd_varlen);
     m.def("duo_bwd_varlen", &duo_bwd_varlen);
     m.def("duo_fwd_masked", &duo_fwd_masked);

@@ -20,22 +20,39 @@ def _call(name: str, *args):
         raise _capi.TahDuoError(str(e).split("\nException raised from")[0]) from None
 
 
-def duo_fwd_varlen(q1, k1, v1, cu_q1, cu_k1, q2, k2, v2, pos_q2, pos_k2, cu_q2, cu_k2, scale: float
+MAX_SCHEDULE_SEQS = 4095
+
+
+def duo_schedule(cu_q1, cu_k1, cu_q2, cu_k2, pos_q2, hq: int, hkv: int, total_q1: int, total_k1: int, total_k2: int):
+    """Launch-order table for the varlen calls over these boundaries: every tile of both depths, heaviest first.
+
+    Built on the device from the boundary tensors (no read-back); pass it as ``schedule=`` to :func:`duo_fwd_varlen` /
+    :func:`duo_bwd_varlen` for as long as the boundaries, ``pos_q2`` and the row counts stay the same -- one table
+    serves every layer and the backward pass of a batch.  It only changes the order in which tiles are started.
+    Returns ``None`` for a single sequence (its tiles are already in that order) or more than 4095 sequences.
+    """
+    nseq = cu_q1.numel() - 1
+    if nseq <= 1 or nseq > MAX_SCHEDULE_SEQS:
+        return None
+    return _call("duo_schedule", cu_q1, cu_k1, cu_q2, cu_k2, pos_q2, int(hq), int(hkv), int(total_q1), int(total_k1), int(total_k2))
+
+
+def duo_fwd_varlen(q1, k1, v1, cu_q1, cu_k1, q2, k2, v2, pos_q2, pos_k2, cu_q2, cu_k2, scale: float, schedule=None
                    ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """Duo-causal attention forward on packed varlen bf16 tensors.
 
     q1 [T1q,Hq,D], k1/v1 [T1k,Hkv,D], cu_q1/cu_k1 int32 [nseq+1]: depth-0 stream.
     q2 [T2q,Hq,D], k2/v2 [T2k,Hkv,D], pos_q2/pos_k2 int32, cu_q2/cu_k2: depth-1 stream
-    (hard tokens).  Returns o1, lse1 [Hq,T1q], o2, lse2 [Hq,T2q].
+    (hard tokens).  ``schedule``: table from :func:`duo_schedule` or None.  Returns o1, lse1 [Hq,T1q], o2, lse2 [Hq,T2q].
     """
-    return _call("duo_fwd_varlen", q1, k1, v1, cu_q1, cu_k1, q2, k2, v2, pos_q2, pos_k2, cu_q2, cu_k2, float(scale))
+    return _call("duo_fwd_varlen", q1, k1, v1, cu_q1, cu_k1, q2, k2, v2, pos_q2, pos_k2, cu_q2, cu_k2, float(scale), schedule)
 
 
 def duo_bwd_varlen(q1, k1, v1, o1, lse1, do1, cu_q1, cu_k1, q2, k2, v2, o2, lse2, do2, pos_q2, pos_k2, cu_q2, cu_k2,
-                   scale: float):
+                   scale: float, schedule=None):
     """Backward of :func:`duo_fwd_varlen`; returns dq1, dk1, dv1, dq2, dk2, dv2 (bf16)."""
     return tuple(_call("duo_bwd_varlen", q1, k1, v1, o1, lse1, do1, cu_q1, cu_k1, q2, k2, v2, o2, lse2, do2, pos_q2, pos_k2,
-                       cu_q2, cu_k2, float(scale)))
+                       cu_q2, cu_k2, float(scale), schedule))
 
 
 def duo_fwd_masked(q, k, v, mask, nseq: int, scale: float):

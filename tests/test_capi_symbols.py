@@ -36,13 +36,27 @@ def test_torch_extension_loads_the_library_and_exposes_every_op():
         assert callable(getattr(ext, n))
 
 
-def test_struct_sizes_match_c_layout():
-    """ctypes mirrors must have the sizes the C compiler gives the structs (LP64)."""
+def test_struct_sizes_match_c_layout(tmp_path):
+    """ctypes mirrors must have the sizes the C compiler gives the structs of the header (gcc, LP64)."""
+    import shutil
+    import subprocess
+
     from tah_amd import _capi
+    pairs = {"tah_duo_stream": _capi.DuoStream, "tah_duo_fwd_args": _capi.DuoFwdArgs, "tah_duo_bwd_stream": _capi.DuoBwdStream,
+             "tah_duo_bwd_args": _capi.DuoBwdArgs, "tah_duo_schedule_args": _capi.DuoScheduleArgs, "tah_kv_segment": _capi.KvSegment,
+             "tah_duo_decode_args": _capi.DuoDecodeArgs, "tah_qk_prep_args": _capi.QkPrepArgs, "tah_topk_mix_args": _capi.TopkMixArgs,
+             "tah_kv_append_args": _capi.KvAppendArgs, "tah_additive_mask": _capi.AdditiveMask}
     assert ctypes.sizeof(_capi.DuoStream) == 9 * 8 + 8 * 8 + 2 * 4
-    assert ctypes.sizeof(_capi.DuoFwdArgs) == 2 * ctypes.sizeof(_capi.DuoStream) + 4 * 4 + 4 + 4
-    assert ctypes.sizeof(_capi.DuoBwdStream) == 5 * 8 + 8 * 8
-    assert ctypes.sizeof(_capi.KvSegment) == 5 * 8 + 4 * 8 + 2 * 4
+    if shutil.which("gcc") is None:
+        return
+    src = tmp_path / "sizes.c"
+    src.write_text('#include <stdio.h>\n#include "tah_duo.h"\nint main(void) {\n' +
+                   "".join(f'  printf("{n} %zu\\n", sizeof({n}));\n' for n in pairs) + "  return 0;\n}\n")
+    exe = tmp_path / "sizes"
+    subprocess.check_call(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)])
+    got = dict(line.split() for line in subprocess.check_output([str(exe)], text=True).splitlines())
+    for n, mirror in pairs.items():
+        assert int(got[n]) == ctypes.sizeof(mirror), n
 
 
 def test_product_ops_refuse_cpu_tensors():

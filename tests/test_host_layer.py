@@ -146,6 +146,24 @@ def _oracle_two_depths(c):
                                c["scale"], valid_mask=c["valid"])
 
 
+def test_forward_loop_with_launch_order_table(emu, monkeypatch):
+    """With the launch-order table switched on for every call size the loop returns what it returns without
+    it; one table is built per depth and the backward pass runs with it."""
+    from tah_amd import attention, ops
+    from tah_amd.cache import TaHDuoCache
+    c = make_dense_case(33, B=3, T=72, p_hard=0.25, Hq=2, Hkv=1, D=128, left_pad=[0, 10, 40])
+    _, w1, w2, _ = _forward_two_depths(c, TaHDuoCache())
+    built = []
+    real = ops.duo_schedule
+    monkeypatch.setattr(ops, "duo_schedule", lambda *a: built.append(1) or real(*a))
+    monkeypatch.setattr(attention, "SCHEDULE_MIN_ROW_HEADS", 0)
+    cache = TaHDuoCache()
+    t, o1, o2, _ = _forward_two_depths(c, cache, requires_grad=True)
+    assert len(built) == 2 and torch.equal(o1, w1) and torch.equal(o2, w2)
+    (o1.float().sum() + o2.float().sum()).backward()
+    assert all(t[k].grad is not None for k in ("q1", "k1", "v1"))
+
+
 @pytest.mark.parametrize("left_pad", [None, [0, 9]])
 def test_forward_loop_matches_dense_reference(emu, left_pad):
     from tah_amd.cache import TaHDuoCache
