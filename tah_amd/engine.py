@@ -249,10 +249,13 @@ class TaHDecodeEngine:
         zi = torch.zeros(0, dtype=torch.int32, device=dev)
         x = w.embed[ids]
         kv_tok = []
+        # launch order of the prompts' tiles, heaviest first across prompts: one table serves all layers of a depth
+        sched0 = ops.duo_schedule(cu, cu, zc, zc, zi, c.hq, c.hkv, N, N, 0)
         for l, L in enumerate(w.layers):
             q, k, v = self._split_qkv(self._rms(x, L["ln1"]) @ L["wqkv"].t())
             qo, ko = qk_norm_rope(q, k, L["qn"], L["kn"], cos, sin, c.rms_eps)
-            o1, _, _, _ = ops.duo_fwd_varlen(qo, ko, v, cu, cu, qo[:0], ko[:0], v[:0], zi, zi, zc, zc, self.scale)
+            o1, _, _, _ = ops.duo_fwd_varlen(qo, ko, v, cu, cu, qo[:0], ko[:0], v[:0], zi, zi, zc, zc, self.scale,
+                                             schedule=sched0)
             self.slabs0[l].append(ko, v, cu)
             kv_tok.append((ko, v))
             x = x + o1.view(N, -1) @ L["wo"].t()
@@ -275,11 +278,13 @@ class TaHDecodeEngine:
             x2 = ops.topk_mix(l0h, w.embed, c.topk)
             pos2 = pos[rows2].contiguous()
             cos2, sin2 = self.cos[pos2.long()], self.sin[pos2.long()]
+            sched1 = ops.duo_schedule(zc, cu, cu2, cu2, pos2, c.hq, c.hkv, 0, N, n2)
             for l, L in enumerate(w.layers):
                 q, k, v = self._split_qkv(self._rms(x2, L["ln1"]) @ L["wqkv"].t())
                 qo, ko = qk_norm_rope(q, k, L["qn"], L["kn"], cos2, sin2, c.rms_eps)
                 k1, v1 = kv_tok[l]
-                _, _, o2, _ = ops.duo_fwd_varlen(qo[:0], k1, v1, zc, cu, qo, ko, v, pos2, pos2, cu2, cu2, self.scale)
+                _, _, o2, _ = ops.duo_fwd_varlen(qo[:0], k1, v1, zc, cu, qo, ko, v, pos2, pos2, cu2, cu2, self.scale,
+                                                 schedule=sched1)
                 self.slabs1[l].append(ko, v, cu2, pos_new=pos2)
                 x2 = x2 + o2.view(n2, -1) @ L["wo"].t()
                 x2 = self._mlp(x2, L)

@@ -13,16 +13,19 @@ pytestmark = pytest.mark.skipif(not emu_util.have_host_clang(), reason="host cla
 NAMES = ("dq1", "dk1", "dv1", "dq2", "dk2", "dv2")
 
 
-def run_bwd(dev, seed):
-    """Forward + backward through tah_amd.ops; returns kernel grads and oracle grads (on the bf16-rounded inputs)."""
+def run_bwd(dev, seed, schedule=None):
+    """Forward + backward through tah_amd.ops; returns kernel grads and oracle grads (on the bf16-rounded inputs;
+    None when a launch-order table is given: that call is only compared with the one without)."""
     from tah_amd import ops
     g = torch.Generator().manual_seed(seed)
     mk = lambda t: torch.randn(t.shape, generator=g).to(torch.bfloat16).to(t.device)
     do1, do2 = mk(dev["q1"]), mk(dev["q2"])
-    o1, lse1, o2, lse2 = ops.duo_fwd_varlen(*varlen_args(dev))
+    o1, lse1, o2, lse2 = ops.duo_fwd_varlen(*varlen_args(dev), schedule=schedule)
     got = ops.duo_bwd_varlen(dev["q1"], dev["k1"], dev["v1"], o1, lse1, do1, dev["cu_q1"], dev["cu_k1"],
                              dev["q2"], dev["k2"], dev["v2"], o2, lse2, do2, dev["pos_q2"], dev["pos_k2"],
-                             dev["cu_q2"], dev["cu_k2"], dev["scale"])
+                             dev["cu_q2"], dev["cu_k2"], dev["scale"], schedule=schedule)
+    if schedule is not None:
+        return got, None
     host = [a.float().cpu().numpy() if torch.is_tensor(a) and a.is_floating_point() else
             (a.cpu().numpy() if torch.is_tensor(a) else a) for a in varlen_args(dev)]
     want = R.bwd(*host, do1.float().cpu().numpy(), do2.float().cpu().numpy())

@@ -42,6 +42,16 @@ def test_random_shape_forward_and_backward(seed):
     got, want = run_bwd(dev, seed + 1)
     torch.cuda.synchronize()
     check_grads(got, want)
+    # the same calls with the launch-order table of the batch: bit-identical outputs and gradients
+    sched = ops.duo_schedule(dev["cu_q1"], dev["cu_k1"], dev["cu_q2"], dev["cu_k2"], dev["pos_q2"], hq, hkv,
+                             dev["q1"].shape[0], dev["k1"].shape[0], dev["k2"].shape[0])
+    assert (sched is None) == (len(seqlens) == 1)
+    if sched is not None:
+        for a, b in zip(out, ops.duo_fwd_varlen(*varlen_args(dev), schedule=sched)):
+            assert torch.equal(a, b)
+        got2, _ = run_bwd(dev, seed + 1, schedule=sched)
+        for a, b in zip(got, got2):
+            assert torch.equal(a, b)
 
 
 def _draw_decode(seed):
