@@ -309,6 +309,31 @@ int tah_topk_mix(const tah_topk_mix_args* args, tah_stream_t stream);
 int tah_silu_mul(const void* gate_up, void* out, int32_t rows, int32_t inter, int64_t gate_up_row_stride,
                  int64_t out_row_stride, tah_stream_t stream);
 
+/* One greedy generation step after the logits exist: per row, the final logits (first-iteration logits, plus
+ * the second iteration's for rows that took one, summed in bf16 as the model's logits buffers are,
+ * tah/model/tah_model.py:543,628), their arg-max (the lower index among equals), and the generation loop's
+ * bookkeeping of tah/model/utils.py:228-262 without its per-row `.item()`: a row whose token is `eos` is finished
+ * and the token is not part of its output; finished rows write 0; positions advance for the rows that decoded.
+ * The final logits are never written out.  One launch instead of about thirty small ones per step. */
+typedef struct tah_greedy_step_args {
+    const void* logits0;      /* bf16 [rows, vocab] */
+    const void* logits1;      /* bf16 [rows, vocab] or NULL (then hard is NULL too) */
+    const uint8_t* hard;      /* [rows] nonzero: the row's logits are bf16(logits0 + logits1) */
+    int64_t row_stride0, row_stride1; /* elements, multiples of 8 */
+    int32_t rows, vocab;
+    int32_t eos;              /* end-of-sequence token id, < 0 for none */
+    int64_t* tok;             /* [rows] out: the token chosen, 0 for finished rows (input of the next step) */
+    uint8_t* finished;        /* [rows] in/out */
+    int32_t* pos;             /* [rows] += 1 for rows that were not finished */
+    int64_t* out_tokens;      /* [rows, out_stride] column step_idx[0] is written */
+    int64_t out_stride;
+    const int64_t* step_idx;  /* [1] */
+    int32_t* out_len;         /* [rows] += 1 for rows still unfinished after this step */
+    int64_t* n_hard;          /* += hard rows among those that decoded */
+    int64_t* n_steps;         /* += rows that decoded */
+} tah_greedy_step_args;
+int tah_greedy_step(const tah_greedy_step_args* args, tah_stream_t stream);
+
 /* Hard-token index build: stream compaction of a (B, S) byte mask in row-major
  * order.  Replaces the stable sort + nonzero of gather_active / scatter_back
  * (tah/model/tah_model.py:111-119, :160-167).  For the r-th True entry, at

@@ -142,6 +142,18 @@ class QkPrepArgs(C.Structure):
     ]
 
 
+class GreedyStepArgs(C.Structure):
+    """``tah_greedy_step_args``"""
+
+    _fields_ = [
+        ("logits0", c_void_p), ("logits1", c_void_p), ("hard", c_void_p),
+        ("row_stride0", c_int64), ("row_stride1", c_int64),
+        ("rows", c_int32), ("vocab", c_int32), ("eos", c_int32),
+        ("tok", c_void_p), ("finished", c_void_p), ("pos", c_void_p), ("out_tokens", c_void_p), ("out_stride", c_int64),
+        ("step_idx", c_void_p), ("out_len", c_void_p), ("n_hard", c_void_p), ("n_steps", c_void_p),
+    ]
+
+
 class TopkMixArgs(C.Structure):
     """``tah_topk_mix_args``"""
 
@@ -159,6 +171,7 @@ PROTOTYPES = {
     "tah_duo_bwd_varlen": (C.c_int, [C.POINTER(DuoBwdArgs), c_void_p]),
     "tah_duo_schedule_bytes": (C.c_size_t, [c_int32] * 7),
     "tah_duo_schedule_build": (C.c_int, [C.POINTER(DuoScheduleArgs), c_void_p]),
+    "tah_greedy_step": (C.c_int, [C.POINTER(GreedyStepArgs), c_void_p]),
     "tah_duo_fwd_masked": (C.c_int, [C.POINTER(DuoFwdArgs), C.POINTER(AdditiveMask), c_void_p]),
     "tah_duo_bwd_masked": (C.c_int, [C.POINTER(DuoBwdArgs), C.POINTER(AdditiveMask), c_void_p]),
     "tah_duo_decode_workspace_bytes": (C.c_size_t, [c_int32, c_int32, c_int32, c_int32]),

@@ -324,6 +324,7 @@ inline uint64_t emu_ds_read_tr16_b64(const void* p) {
 
 inline int atomicAdd(int* p, int v) { return __atomic_fetch_add(p, v, __ATOMIC_RELAXED); }
 inline unsigned atomicAdd(unsigned* p, unsigned v) { return __atomic_fetch_add(p, v, __ATOMIC_RELAXED); }
+inline unsigned long long atomicAdd(unsigned long long* p, unsigned long long v) { return __atomic_fetch_add(p, v, __ATOMIC_RELAXED); }
 inline float atomicAdd(float* p, float v) {
     float old, upd;
     __atomic_load(p, &old, __ATOMIC_RELAXED);

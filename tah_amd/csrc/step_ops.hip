@@ -36,8 +36,124 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const __bf16* gu, __bf16*
     *reinterpret_cast<u32x4*>(out + (int64_t)r * out_rs + i) = o;
 }
 
+// ---------------------------------------------------------------------------
+// Greedy step: final logits of a row (first iteration, plus the second for rows that took one, summed in
+// bf16 as the model's logits buffers are), their arg-max, and the generation loop's per-row bookkeeping.
+// One workgroup per row; the logits are read once (16-byte loads) and never written anywhere.
+// ---------------------------------------------------------------------------
+constexpr int kGreedyThreads = 1024;
+
+struct GreedyParams {
+    const __bf16 *l0, *l1;
+    const uint8_t* hard;
+    int64_t rs0, rs1;
+    int32_t vocab, eos;
+    int64_t* tok;
+    uint8_t* finished;
+    int32_t* pos;
+    int64_t* out_tokens;
+    int64_t out_stride;
+    const int64_t* step_idx;
+    int32_t* out_len;
+    unsigned long long *n_hard, *n_steps;
+};
+
+__device__ __forceinline__ void take_better(float& bv, int& bi, float v, int i) {
+    if (v > bv || (v == bv && i < bi)) {  // ties: the lower vocabulary index
+        bv = v;
+        bi = i;
+    }
+}
+
+__global__ __launch_bounds__(kGreedyThreads) void greedy_step_kernel(const GreedyParams p) {
+    __shared__ float wv[kGreedyThreads / kWave];
+    __shared__ int wi[kGreedyThreads / kWave];
+    const int row = blockIdx.x, tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    const bool active = p.finished[row] == 0;
+    const bool both = p.l1 != nullptr && p.hard != nullptr && p.hard[row] != 0;
+    float bv = -__builtin_inff();
+    int bi = 0x7fffffff;
+    if (active) {
+        const __bf16* a = p.l0 + (int64_t)row * p.rs0;
+        const __bf16* b = both ? p.l1 + (int64_t)row * p.rs1 : nullptr;
+        const int nvec = p.vocab / 8;
+        for (int c = tid; c < nvec; c += kGreedyThreads) {
+            const u32x4 x = *reinterpret_cast<const u32x4*>(a + 8 * c);
+            u32x4 y = {0u, 0u, 0u, 0u};
+            if (both) y = *reinterpret_cast<const u32x4*>(b + 8 * c);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                float lo = lo_f(x[q]), hi = hi_f(x[q]);
+                if (both) {  // the running sum of the iterations' logits lives in the model dtype
+                    const uint32_t s = pack2(lo + lo_f(y[q]), hi + hi_f(y[q]));
+                    lo = lo_f(s);
+                    hi = hi_f(s);
+                }
+                if (lo > bv) { bv = lo; bi = 8 * c + 2 * q; }          // indices ascend inside a thread:
+                if (hi > bv) { bv = hi; bi = 8 * c + 2 * q + 1; }      // strict > keeps the first of equals
+            }
+        }
+        for (int i = nvec * 8 + tid; i < p.vocab; i += kGreedyThreads) {  // a tail that is not a multiple of 8
+            float v = (float)a[i];
+            if (both) v = (float)(__bf16)(v + (float)b[i]);
+            take_better(bv, bi, v, i);
+        }
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) take_better(bv, bi, __shfl_xor(bv, m), __shfl_xor(bi, m));
+        if (lane == 0) {
+            wv[wave] = bv;
+            wi[wave] = bi;
+        }
+    }
+    __syncthreads();
+    if (tid != 0) return;
+    int64_t nxt = 0;
+    if (active) {
+        for (int w = 1; w < kGreedyThreads / kWave; ++w) take_better(bv, bi, wv[w], wi[w]);
+        nxt = bi == 0x7fffffff ? 0 : bi;
+    }
+    // the loop's bookkeeping for this row (tah/model/utils.py:228-262): a row ends with its end-of-sequence token,
+    // which is not part of its output; rows that have ended write zeros
+    bool done = !active;
+    if (active && p.eos >= 0 && nxt == p.eos) done = true;
+    p.finished[row] = done ? 1 : 0;
+    p.out_tokens[(int64_t)row * p.out_stride + p.step_idx[0]] = done ? 0 : nxt;
+    if (!done) p.out_len[row] += 1;
+    if (active) {
+        p.pos[row] += 1;
+        atomicAdd(p.n_steps, 1ull);
+        if (p.hard != nullptr && p.hard[row] != 0) atomicAdd(p.n_hard, 1ull);
+    }
+    p.tok[row] = nxt;
+}
+
 }  // namespace
 }  // namespace tah
+
+extern "C" int tah_greedy_step(const tah_greedy_step_args* a, tah_stream_t stream) {
+    using namespace tah;
+    if (!a) return TAH_E_NULL;
+    if (a->rows < 0 || a->vocab <= 0 || a->rows > 65535) return TAH_E_SHAPE;
+    if (a->rows == 0) return TAH_OK;
+    if (!a->logits0 || !a->tok || !a->finished || !a->pos || !a->out_tokens || !a->step_idx || !a->out_len || !a->n_hard || !a->n_steps)
+        return TAH_E_NULL;
+    if ((a->logits1 == nullptr) != (a->hard == nullptr)) return TAH_E_NULL;
+    if ((reinterpret_cast<uintptr_t>(a->logits0) & 15) || (reinterpret_cast<uintptr_t>(a->logits1) & 15) || a->row_stride0 % 8 ||
+        a->row_stride1 % 8)
+        return TAH_E_ALIGN;
+    GreedyParams p;
+    p.l0 = static_cast<const __bf16*>(a->logits0);
+    p.l1 = static_cast<const __bf16*>(a->logits1);
+    p.hard = a->hard;
+    p.rs0 = a->row_stride0; p.rs1 = a->row_stride1;
+    p.vocab = a->vocab; p.eos = a->eos;
+    p.tok = a->tok; p.finished = a->finished; p.pos = a->pos;
+    p.out_tokens = a->out_tokens; p.out_stride = a->out_stride; p.step_idx = a->step_idx; p.out_len = a->out_len;
+    p.n_hard = reinterpret_cast<unsigned long long*>(a->n_hard);
+    p.n_steps = reinterpret_cast<unsigned long long*>(a->n_steps);
+    hipLaunchKernelGGL(greedy_step_kernel, dim3(a->rows), dim3(kGreedyThreads), 0, static_cast<hipStream_t>(stream), p);
+    return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
+}
 
 extern "C" int tah_silu_mul(const void* gate_up, void* out, int32_t rows, int32_t inter, int64_t gate_up_row_stride,
                             int64_t out_row_stride, tah_stream_t stream) {

@@ -28,6 +28,7 @@ struct Api {
     decltype(&tah_duo_bwd_varlen) bwd_varlen = nullptr;
     decltype(&tah_duo_schedule_bytes) schedule_bytes = nullptr;
     decltype(&tah_duo_schedule_build) schedule_build = nullptr;
+    decltype(&tah_greedy_step) greedy_step = nullptr;
     decltype(&tah_duo_fwd_masked) fwd_masked = nullptr;
     decltype(&tah_duo_bwd_masked) bwd_masked = nullptr;
     decltype(&tah_duo_decode_workspace_bytes) decode_workspace_bytes = nullptr;
@@ -61,6 +62,7 @@ void load_library(const std::string& path, bool allow_host) {
     bind(g.bwd_varlen, "tah_duo_bwd_varlen");
     bind(g.schedule_bytes, "tah_duo_schedule_bytes");
     bind(g.schedule_build, "tah_duo_schedule_build");
+    bind(g.greedy_step, "tah_greedy_step");
     bind(g.fwd_masked, "tah_duo_fwd_masked");
     bind(g.bwd_masked, "tah_duo_bwd_masked");
     bind(g.decode_workspace_bytes, "tah_duo_decode_workspace_bytes");
@@ -498,6 +500,42 @@ Tensor silu_mul(const Tensor& gate_up) {
     return out;
 }
 
+// Arg-max of the step's final logits and the generation loop's per-row bookkeeping, in place (tah_greedy_step).
+void greedy_step(const Tensor& logits0, const optional<Tensor>& logits1, const optional<Tensor>& hard, int64_t eos, const Tensor& tok,
+                 const Tensor& finished, const Tensor& pos, const Tensor& out_tokens, const Tensor& step_idx, const Tensor& out_len,
+                 const Tensor& n_hard, const Tensor& n_steps) {
+    need_lib();
+    Dev d;
+    for (const Tensor* t : {&logits0, &tok, &finished, &pos, &out_tokens, &step_idx, &out_len, &n_hard, &n_steps}) d.see(*t);
+    d.see(logits1); d.see(hard);
+    const int64_t rows = logits0.size(0), vocab = logits0.size(1);
+    TORCH_CHECK(logits0.dim() == 2 && logits0.scalar_type() == at::kBFloat16 && logits0.stride(1) == 1, "greedy_step: logits0 must be bf16 [rows, vocab]");
+    TORCH_CHECK(logits1.has_value() == hard.has_value(), "greedy_step: logits1 and hard come together");
+    if (logits1.has_value()) {
+        TORCH_CHECK(logits1->sizes() == logits0.sizes() && logits1->scalar_type() == at::kBFloat16 && logits1->stride(1) == 1,
+                    "greedy_step: logits1 must match logits0");
+        TORCH_CHECK(hard->scalar_type() == at::kBool && hard->is_contiguous() && hard->numel() == rows, "greedy_step: hard must be bool [rows]");
+    }
+    TORCH_CHECK(tok.scalar_type() == at::kLong && tok.is_contiguous() && tok.numel() == rows, "greedy_step: tok must be int64 [rows]");
+    TORCH_CHECK(finished.scalar_type() == at::kBool && finished.is_contiguous() && finished.numel() == rows, "greedy_step: finished must be bool [rows]");
+    TORCH_CHECK(pos.scalar_type() == at::kInt && pos.is_contiguous() && pos.numel() == rows, "greedy_step: pos must be int32 [rows]");
+    TORCH_CHECK(out_len.scalar_type() == at::kInt && out_len.is_contiguous() && out_len.numel() == rows, "greedy_step: out_len must be int32 [rows]");
+    TORCH_CHECK(out_tokens.scalar_type() == at::kLong && out_tokens.dim() == 2 && out_tokens.size(0) == rows && out_tokens.stride(1) == 1,
+                "greedy_step: out_tokens must be int64 [rows, steps]");
+    for (const Tensor* t : {&step_idx, &n_hard, &n_steps})
+        TORCH_CHECK(t->scalar_type() == at::kLong && t->numel() == 1, "greedy_step: step_idx, n_hard and n_steps are int64 scalars");
+    tah_greedy_step_args a{};
+    a.logits0 = logits0.data_ptr(); a.logits1 = ptr(logits1); a.hard = static_cast<const uint8_t*>(ptr(hard));
+    a.row_stride0 = logits0.stride(0); a.row_stride1 = logits1.has_value() ? logits1->stride(0) : 0;
+    a.rows = (int32_t)rows; a.vocab = (int32_t)vocab; a.eos = (int32_t)eos;
+    a.tok = static_cast<int64_t*>(tok.data_ptr()); a.finished = static_cast<uint8_t*>(finished.data_ptr());
+    a.pos = static_cast<int32_t*>(pos.data_ptr()); a.out_tokens = static_cast<int64_t*>(out_tokens.data_ptr());
+    a.out_stride = out_tokens.stride(0); a.step_idx = static_cast<const int64_t*>(step_idx.data_ptr());
+    a.out_len = static_cast<int32_t*>(out_len.data_ptr());
+    a.n_hard = static_cast<int64_t*>(n_hard.data_ptr()); a.n_steps = static_cast<int64_t*>(n_steps.data_ptr());
+    check_rc(g.greedy_step(&a, d.stream()), "tah_greedy_step");
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -506,6 +544,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("loaded", [] { return g.handle != nullptr; });
     m.def("abi_version", [] { need_lib(); return g.abi_version(); });
     m.def("duo_schedule", &duo_schedule);
+    m.def("greedy_step", &greedy_step);
     m.def("duo_fwd_varlen", &duo_fwd_varlen);
     m.def("duo_bwd_varlen", &duo_bwd_varlen);
     m.def("duo_fwd_masked", &duo_fwd_masked);

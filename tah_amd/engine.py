@@ -142,6 +142,7 @@ class TaHDecodeEngine:
         self.minus1 = torch.full((batch,), -1, dtype=torch.int32, device=dev)
         self.zeros_i = torch.zeros(batch, dtype=torch.int32, device=dev)
         # generation state (all on the device)
+        self.fused_greedy = True  # arg-max + bookkeeping of a greedy step in one launch (tah_greedy_step)
         self.tok = torch.zeros(batch, dtype=torch.long, device=dev)       # token fed to the next step
         self.pos = torch.zeros(batch, dtype=torch.int32, device=dev)      # its position
         self.finished = torch.zeros(batch, dtype=torch.bool, device=dev)
@@ -205,26 +206,29 @@ class TaHDecodeEngine:
         Returns (final logits float32 [B, V], hard bool [B]).  ``force_hard`` replaces the decider's decision
         (tests drive both implementations with the same decisions).  Rows that are not ``active`` are neither
         cached nor attended; their logits are meaningless."""
+        l0, l1, hard = self._step_parts(tok, force_hard, active)
+        # running sum of the iterations' logits, rounded to the model dtype as the reference's buffers are
+        # (tah_model.py:543, 628)
+        return torch.where(hard[:, None], (l0 + l1).float(), l0.float()), hard
+
+    def _step_parts(self, tok: torch.Tensor, force_hard: Optional[torch.Tensor] = None, active: Optional[torch.Tensor] = None):
+        """Both latent iterations of one step: logits of the first and of the second iteration (model dtype [B, V];
+        the second are meaningless for rows that are not hard) and hard bool [B]."""
         B = self.B
         pos = self.pos
         act = active if active is not None else torch.ones(B, dtype=torch.bool, device=self.device)
         slot0 = torch.where(act, self.rows, self.minus1)
         qpos0 = torch.where(act, pos, self.minus1)
         h0 = self._pass_single(self.w.embed[tok], pos, 0, slot0, qpos0, self.zeros_i)
-        l0 = (h0 @ self.w.lm_head.t()).float()
+        l0 = h0 @ self.w.lm_head.t()
         hard = (self.decide(h0) > self.w.threshold) if force_hard is None else force_hard
         hard = hard & act
         # next-iteration input of the hard rows (tah_model.py:693-697); the other rows keep zeros
-        x1 = ops.topk_mix(l0.to(self.w.embed.dtype), self.w.embed, self.cfg.topk, row_enable=hard)
+        x1 = ops.topk_mix(l0, self.w.embed, self.cfg.topk, row_enable=hard)
         slot1 = torch.where(hard, self.rows, self.minus1)
         qpos1 = torch.where(hard, pos, self.minus1)
         h1 = self._pass_single(x1, pos, 1, slot1, qpos1, hard.to(torch.int32))
-        l1 = (h1 @ self.w.lm_head.t()).float()
-        # running sum of the iterations' logits, rounded to the model dtype as the reference's buffers are
-        # (tah_model.py:543, 628)
-        dt = self.w.embed.dtype
-        both = (l0.to(dt) + l1.to(dt)).float()
-        return torch.where(hard[:, None], both, l0.to(dt).float()), hard
+        return l0, h1 @ self.w.lm_head.t(), hard
 
     # ── prefill: packed prompts, both depths, through the varlen kernels ──
     @torch.no_grad()
@@ -330,6 +334,13 @@ class TaHDecodeEngine:
     def _step_inplace(self, temperature: float, eos: int, **filters):
         """One generated token for every unfinished row; every state change is an in-place device update."""
         act = ~self.finished
+        if temperature <= 0.0 and self.fused_greedy and self.w.embed.dtype == torch.bfloat16 and self.cfg.vocab % 8 == 0:
+            # arg-max of the final logits and the bookkeeping below in one launch; the final logits are not formed
+            l0, l1, hard = self._step_parts(self.tok, active=act)
+            ops.greedy_step(l0, l1, hard, eos, self.tok, self.finished, self.pos, self.out_tokens, self.step_idx, self.out_len,
+                            self.n_hard, self.n_steps)
+            self.step_idx += 1
+            return
         logits, hard = self.step_logits(self.tok, active=act)
         nxt = self.sample(logits, temperature, **filters)
         nxt = torch.where(act, nxt, torch.zeros_like(nxt))

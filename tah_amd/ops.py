@@ -107,3 +107,14 @@ def topk_mix(logits: torch.Tensor, embedding: torch.Tensor, topk: int, row_enabl
 def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
     """``silu(gate) * up`` of a fused gate|up projection, bf16 [rows, 2*I] -> [rows, I], in one launch."""
     return _call("silu_mul", gate_up)
+
+
+def greedy_step(logits0, logits1, hard, eos: int, tok, finished, pos, out_tokens, step_idx, out_len, n_hard, n_steps) -> None:
+    """One greedy generation step after the logits (``tah_greedy_step``), all updates in place on the device.
+
+    Per row: final logits = ``logits0`` (bf16 [rows, vocab]), or ``bf16(logits0 + logits1)`` where ``hard`` (bool
+    [rows]) is set; ``tok`` = their arg-max (0 for finished rows); a row whose token is ``eos`` (>= 0) becomes
+    ``finished`` and the token stays out of its output; ``out_tokens[:, step_idx]`` and ``out_len`` record the
+    output, ``pos`` advances for the rows that decoded, ``n_steps`` / ``n_hard`` count them.
+    """
+    _call("greedy_step", logits0, logits1, hard, int(eos), tok, finished, pos, out_tokens, step_idx, out_len, n_hard, n_steps)

@@ -106,3 +106,22 @@ def run(device, *, prompt=(9, 6, 12), steps=5, layers=2, seed=0, vocab=96, topk=
     n1 = [int(hard[b, Tm - n:].sum()) for b, n in enumerate(prompt)]
     assert all(sl.len.tolist() == n1 for sl in eng.slabs1)
     return out
+
+
+def run_greedy(device, *, fused, eos, B=3, T=9, new=7, vocab=64, seed=5, layers=2):
+    """Greedy generation with the fused arg-max + bookkeeping step on or off; returns everything the loop leaves
+    behind (tokens, lengths, positions, finished flags, counters, slab lengths)."""
+    from tah_amd.engine import EngineConfig, TaHDecodeEngine, Weights
+
+    cfg = EngineConfig(hidden=256, layers=layers, hq=4, hkv=2, head_dim=128, intermediate=512, vocab=vocab, decider_hidden=32)
+    w = Weights.random_init(cfg, device, seed=seed)
+    g = torch.Generator().manual_seed(seed + 1)
+    ids = torch.randint(0, vocab, (B * T,), generator=g).to(device)
+    cu = torch.arange(0, B * T + 1, T, dtype=torch.int32, device=device)
+    eng = TaHDecodeEngine(w, B, T + new + 2, device=device)
+    eng.fused_greedy = fused
+    first, _ = eng.prefill(ids, cu, calibrate=0.3)
+    toks = eng.generate(first, new, eos=eos, use_graph=False).clone()
+    return (toks.cpu(), eng.out_len.cpu(), eng.pos.cpu(), eng.finished.cpu(), int(eng.n_hard), int(eng.n_steps), eng.tok.cpu(),
+            [sl.len.tolist() for sl in eng.slabs0 + eng.slabs1])
+

@@ -19,6 +19,73 @@ def test_engine_matches_reference_loop_on_cpu_shim():
         _check(run("cpu", prompt=(7, 4), steps=4))
 
 
+def _same_greedy(device, **size):
+    from tests.engine_case import run_greedy
+    same = lambda a, b, e: [None for x, y in zip(a, b) if not (torch.equal(x, y) if torch.is_tensor(x) else x == y)] == [] or \
+        pytest.fail(f"fused and plain greedy steps differ (eos={e}): {a} vs {b}")
+    plain = run_greedy(device, fused=False, eos=-1, **size)
+    same(plain, run_greedy(device, fused=True, eos=-1, **size), -1)
+    # an end-of-sequence token that the run is known to produce part-way for some row: rows finish at different steps
+    eos = int(plain[0][0, 2])
+    a = run_greedy(device, fused=False, eos=eos, **size)
+    same(a, run_greedy(device, fused=True, eos=eos, **size), eos)
+    assert bool(a[3].any())  # some row did finish
+
+
+def _greedy_step_case(device, rows=6, vocab=200, seed=0):
+    """ops.greedy_step against the engine's own torch bookkeeping (engine.py:_step_inplace) on random logits with
+    ties, rows already finished, rows that hit the end-of-sequence token and rows that took a second iteration."""
+    from tah_amd import ops
+    g = torch.Generator().manual_seed(seed)
+    padded = (vocab + 7) // 8 * 8  # rows start on 16-byte boundaries; the vocabulary itself may be any size
+    l0p = (torch.randn(rows, padded, generator=g) * 3).to(torch.bfloat16)
+    l1p = (torch.randn(rows, padded, generator=g) * 3).to(torch.bfloat16)
+    l0, l1 = l0p[:, :vocab], l1p[:, :vocab]
+    l0[1, 7] = l0[1, 150] = 40.0               # a tie at the maximum: the lower index wins
+    hard = torch.tensor([False, False, True, True, False, True])[:rows]
+    finished = torch.tensor([False, False, False, True, False, False])[:rows]
+    final = torch.where(hard[:, None], (l0 + l1).float(), l0.float())
+    eos = int(final[4].argmax())               # row 4 produces the end-of-sequence token at this step
+    st = dict(tok=torch.full((rows,), 5, dtype=torch.long), finished=finished.clone(), pos=torch.arange(10, 10 + rows, dtype=torch.int32),
+              out_tokens=torch.zeros(rows, 4, dtype=torch.long), step_idx=torch.tensor([2]), out_len=torch.full((rows,), 2, dtype=torch.int32),
+              n_hard=torch.tensor(3), n_steps=torch.tensor(11))
+    dev = {k: v.clone().to(device) for k, v in st.items()}
+    ops.greedy_step(l0p.to(device)[:, :vocab], l1p.to(device)[:, :vocab], (hard & ~finished).to(device), eos, dev["tok"], dev["finished"], dev["pos"],
+                    dev["out_tokens"], dev["step_idx"], dev["out_len"], dev["n_hard"], dev["n_steps"])
+    # the same step as the unfused loop writes it
+    act = ~st["finished"]
+    nxt = torch.where(act, final.argmax(-1), torch.zeros(rows, dtype=torch.long))
+    assert int(nxt[1]) == 7
+    st["finished"] |= nxt == eos
+    keep = ~st["finished"]
+    st["out_tokens"][:, 2] = torch.where(keep, nxt, torch.zeros_like(nxt))
+    st["out_len"] += keep.to(torch.int32)
+    st["n_hard"] += (hard & act).sum()
+    st["n_steps"] += act.sum()
+    st["pos"] += act.to(torch.int32)
+    st["tok"] = nxt
+    for k in st:
+        assert torch.equal(dev[k].cpu(), st[k]), k
+
+
+@pytest.mark.skipif(not emu_util.have_host_clang(), reason="host clang++ not available")
+def test_greedy_step_kernel_on_cpu_shim():
+    with emu_util.emulated():
+        _greedy_step_case("cpu")
+        _greedy_step_case("cpu", vocab=203, seed=1)   # a vocabulary that is not a multiple of 8
+
+
+@pytest.mark.gpu
+def test_greedy_step_kernel_gpu():
+    _greedy_step_case("cuda", vocab=151936)
+    _greedy_step_case("cuda", vocab=1003, seed=2)
+
+
+@pytest.mark.gpu
+def test_fused_greedy_step_equals_the_torch_bookkeeping_gpu():
+    _same_greedy("cuda")
+
+
 @pytest.mark.gpu
 def test_engine_matches_reference_loop_gpu():
     from tests.engine_case import run
@@ -109,7 +176,7 @@ def test_generate_wrapper_returns_tokens_up_to_eos_gpu():
     import types
 
     from tah_amd.engine import EngineConfig, TaHDecodeEngine, Weights, generate
-    cfg = EngineConfig(hidden=256, layers=2, hq=4, hkv=2, head_dim=128, intermediate=512, vocab=300, decider_hidden=32)
+    cfg = EngineConfig(hidden=256, layers=2, hq=4, hkv=2, head_dim=128, intermediate=512, vocab=304, decider_hidden=32)
     w = Weights.random_init(cfg, "cuda", seed=5)
     B, T, new = 3, 20, 24
     g = torch.Generator().manual_seed(2)
