@@ -77,20 +77,35 @@ __global__ __launch_bounds__(kGreedyThreads) void greedy_step_kernel(const Greed
         const __bf16* a = p.l0 + (int64_t)row * p.rs0;
         const __bf16* b = both ? p.l1 + (int64_t)row * p.rs1 : nullptr;
         const int nvec = p.vocab / 8;
-        for (int c = tid; c < nvec; c += kGreedyThreads) {
-            const u32x4 x = *reinterpret_cast<const u32x4*>(a + 8 * c);
-            u32x4 y = {0u, 0u, 0u, 0u};
-            if (both) y = *reinterpret_cast<const u32x4*>(b + 8 * c);
+        // four 16-byte pieces per pass, all loaded before the first is looked at: 32 workgroups read 19 MB, and
+        // what a thread waits for is memory latency
+        constexpr int kAhead = 4;
+        for (int c0 = tid; c0 < nvec; c0 += kAhead * kGreedyThreads) {
+            u32x4 x[kAhead], y[kAhead];
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                float lo = lo_f(x[q]), hi = hi_f(x[q]);
-                if (both) {  // the running sum of the iterations' logits lives in the model dtype
-                    const uint32_t s = pack2(lo + lo_f(y[q]), hi + hi_f(y[q]));
-                    lo = lo_f(s);
-                    hi = hi_f(s);
+            for (int u = 0; u < kAhead; ++u) {
+                const int c = c0 + u * kGreedyThreads;
+                x[u] = y[u] = u32x4{0u, 0u, 0u, 0u};
+                if (c < nvec) {
+                    x[u] = *reinterpret_cast<const u32x4*>(a + 8 * c);
+                    if (both) y[u] = *reinterpret_cast<const u32x4*>(b + 8 * c);
                 }
-                if (lo > bv) { bv = lo; bi = 8 * c + 2 * q; }          // indices ascend inside a thread:
-                if (hi > bv) { bv = hi; bi = 8 * c + 2 * q + 1; }      // strict > keeps the first of equals
+            }
+#pragma unroll
+            for (int u = 0; u < kAhead; ++u) {
+                const int c = c0 + u * kGreedyThreads;
+                if (c >= nvec) break;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    float lo = lo_f(x[u][q]), hi = hi_f(x[u][q]);
+                    if (both) {  // the running sum of the iterations' logits lives in the model dtype
+                        const uint32_t s = pack2(lo + lo_f(y[u][q]), hi + hi_f(y[u][q]));
+                        lo = lo_f(s);
+                        hi = hi_f(s);
+                    }
+                    if (lo > bv) { bv = lo; bi = 8 * c + 2 * q; }          // indices ascend inside a thread:
+                    if (hi > bv) { bv = hi; bi = 8 * c + 2 * q + 1; }      // strict > keeps the first of equals
+                }
             }
         }
         for (int i = nvec * 8 + tid; i < p.vocab; i += kGreedyThreads) {  // a tail that is not a multiple of 8

@@ -3,8 +3,9 @@
 //   out[row] = sum_j softmax(top-k logits of the row)_j * embedding[index_j]
 //
 // One workgroup (1024 threads) per row.  The row's logits (bf16) are loaded once into registers as
-// order-preserving 16-bit keys; the k-th largest key is found by bisection on the 16-bit key space with a
-// block-wide count per step (no histogram atomics, no sort), ties at the threshold are broken towards the
+// order-preserving 16-bit keys; the keys that can be among the k largest (those at or above the k-th largest
+// thread maximum) are collected in LDS; the k-th largest key is found by bisection on the 16-bit key space with
+// a block-wide count per step (no histogram atomics, no sort), ties at the threshold are broken towards the
 // lower vocabulary index by a second bisection on the index, the <= k selected (index, value) pairs are
 // gathered into LDS and ordered by index (so that the float sums below have one fixed order), and the mix is
 // accumulated in float over bf16-rounded products, as the bf16 eager arithmetic it replaces rounds them.
@@ -19,6 +20,7 @@ namespace {
 constexpr int kMixThreads = 1024;
 constexpr int kMixWaves = kMixThreads / kWave;
 constexpr int kMaxTopk = 256;
+constexpr int kMaxCand = 2048;  // keys that reach the lower bound of the k-th largest (two per thread)
 constexpr int kMaxVec = 19;  // 16-byte pieces of the row per thread: vocabularies up to 19 * 8 * 1024 = 155648
 
 struct MixParams {
@@ -69,6 +71,9 @@ __global__ __launch_bounds__(kMixThreads) void topk_mix_kernel(const MixParams p
     __shared__ int ord_idx[kMaxTopk];
     __shared__ float ord_w[kMaxTopk];
     __shared__ int n_sel;
+    __shared__ uint16_t cand_key[kMaxCand];
+    __shared__ int cand_idx[kMaxCand];
+    __shared__ int n_cand;
     HIP_DYNAMIC_SHARED(unsigned char, dyn)  // float partial sums of the mix: [parts][hidden]
 
     const int row = blockIdx.x;
@@ -110,73 +115,179 @@ __global__ __launch_bounds__(kMixThreads) void topk_mix_kernel(const MixParams p
         }
         __builtin_amdgcn_sched_barrier(0);
     }
-    auto count_ge = [&](uint32_t t) {  // elements of this thread with key >= t
-        int c = 0;
+    // ---- candidates: the keys that can be among the k largest -------------------------------------------
+    // The k-th largest of the 1024 thread maxima, L, is a lower bound of the k-th largest key (k <= 256 threads
+    // hold a key >= L each), and on anything but a flat row only a few hundred keys reach it.  Those go to LDS
+    // with their indices, and the searches below run over them (two per thread) instead of over the whole row
+    // (152 per thread at the full vocabulary).  A row with more candidates than the list holds takes the
+    // searches over the whole row.
+    uint32_t tmax = 0u;
 #pragma unroll
-        for (int j = 0; j < NVEC; ++j) {
+    for (int j = 0; j < NVEC; ++j)
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                uint32_t w = keys[j][q];
-                TAH_OPAQUE1(w);  // the two halves are split here, every time: hoisted out of the bisection
-                                 // loop they would double the registers the row occupies
-                c += ((w & 0xffffu) >= t) + ((w >> 16) >= t);
-            }
-        }
-        return c;
-    };
-
-    // ---- largest key T with count(key >= T) >= k: bisection, invariant count(>= lo) >= k > count(>= hi) ----
-    uint32_t lo = 1u, hi = 0x10000u;  // key 0 only marks indices past the end
-    while (hi - lo > 1) {
-        const uint32_t mid = (lo + hi) >> 1;
-        if (block_sum(count_ge(mid), red, wave, lane) >= k) lo = mid;
-        else hi = mid;
-    }
-    const uint32_t T = lo;
-    const int n_gt = block_sum(count_ge(T + 1), red, wave, lane);
-    const int need_eq = k - n_gt;  // >= 1: that many elements with key == T are taken, lowest indices first
-    // ---- smallest index bound M with count(key == T and index < M) >= need_eq ----
-    auto count_eq_below = [&](int m) {
-        int c = 0;
-#pragma unroll
-        for (int j = 0; j < NVEC; ++j) {
-            int d = m - (j * kMixThreads + tid) * 8;  // index e of this piece is below the bound iff e < d
-            TAH_OPAQUE1(d);                           // (compared with constants: no per-element index registers)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                uint32_t w = keys[j][q];
-                TAH_OPAQUE1(w);
-                c += ((w & 0xffffu) == T) && (2 * q < d);
-                c += ((w >> 16) == T) && (2 * q + 1 < d);
-            }
-        }
-        return c;
-    };
-    int mlo = 0, mhi = V;  // invariant: count(< mlo) < need_eq <= count(< mhi)
-    while (mhi - mlo > 1) {
-        const int mid = (mlo + mhi) >> 1;
-        if (block_sum(count_eq_below(mid), red, wave, lane) >= need_eq) mhi = mid;
-        else mlo = mid;
-    }
-    const int M = mhi;
-
-    // ---- gather the k selected (index, value) pairs ----
-    if (tid == 0) n_sel = 0;
-    __syncthreads();
-#pragma unroll
-    for (int j = 0; j < NVEC; ++j) {
-        int i0 = (j * kMixThreads + tid) * 8;
-        TAH_OPAQUE1(i0);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            uint32_t w = keys[j][e / 2];
+        for (int q = 0; q < 4; ++q) {
+            uint32_t w = keys[j][q];
             TAH_OPAQUE1(w);
-            const uint32_t key = (w >> (16 * (e % 2))) & 0xffffu;
-            if (key > T || (key == T && e < M - i0)) {
-                const int s = atomicAdd(&n_sel, 1);
-                if (s < kMaxTopk) {
-                    sel_idx[s] = i0 + e;
-                    sel_val[s] = key_value(key);
+            const uint32_t a = w & 0xffffu, b = w >> 16;
+            tmax = tmax > a ? tmax : a;
+            tmax = tmax > b ? tmax : b;
+        }
+    uint32_t llo = 1u, lhi = 0x10000u;  // invariant: count(tmax >= llo) >= k > count(tmax >= lhi), or llo == 1
+    while (lhi - llo > 1) {
+        const uint32_t mid = (llo + lhi) >> 1;
+        if (block_sum(tmax >= mid ? 1 : 0, red, wave, lane) >= k) llo = mid;
+        else lhi = mid;
+    }
+    const uint32_t L = llo;
+    if (tid == 0) {
+        n_cand = 0;
+        n_sel = 0;
+    }
+    __syncthreads();
+    if (tmax >= L) {  // (most threads hold no candidate and skip their row)
+#pragma unroll
+        for (int j = 0; j < NVEC; ++j) {
+            int i0 = (j * kMixThreads + tid) * 8;
+            TAH_OPAQUE1(i0);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                uint32_t w = keys[j][e / 2];
+                TAH_OPAQUE1(w);
+                const uint32_t key = (w >> (16 * (e % 2))) & 0xffffu;
+                if (key >= L) {
+                    const int s_ = atomicAdd(&n_cand, 1);
+                    if (s_ < kMaxCand) {
+                        cand_key[s_] = (uint16_t)key;
+                        cand_idx[s_] = i0 + e;
+                    }
+                }
+            }
+        }
+    }
+    __syncthreads();
+    const int ncand = n_cand;
+    if (ncand <= kMaxCand) {
+        // this thread's candidates (key 0: none)
+        uint32_t ck[kMaxCand / kMixThreads];
+        int ci[kMaxCand / kMixThreads];
+#pragma unroll
+        for (int u = 0; u < kMaxCand / kMixThreads; ++u) {
+            const int c = tid + u * kMixThreads;
+            ck[u] = c < ncand ? cand_key[c] : 0u;
+            ci[u] = c < ncand ? cand_idx[c] : 0x7fffffff;
+        }
+        auto cnt_ge = [&](uint32_t t) {
+            int c = 0;
+#pragma unroll
+            for (int u = 0; u < kMaxCand / kMixThreads; ++u) c += ck[u] >= t;
+            return c;
+        };
+        // largest key T with count(key >= T) >= k; count(key >= L) = ncand >= k
+        uint32_t lo = L, hi = 0x10000u;
+        int n_ge = ncand;
+        while (hi - lo > 1) {
+            const uint32_t mid = (lo + hi) >> 1;
+            const int cnt = block_sum(cnt_ge(mid), red, wave, lane);
+            if (cnt >= k) { lo = mid; n_ge = cnt; }
+            else hi = mid;
+        }
+        const uint32_t T = lo;
+        const int n_gt = block_sum(cnt_ge(T + 1), red, wave, lane);
+        const int need_eq = k - n_gt;  // >= 1: that many keys == T are taken, lowest indices first
+        int mlo = 0, mhi = V;          // smallest bound M with count(key == T and index < M) >= need_eq
+        if (n_ge - n_gt > need_eq) {
+            while (mhi - mlo > 1) {
+                const int mid = (mlo + mhi) >> 1;
+                int c = 0;
+#pragma unroll
+                for (int u = 0; u < kMaxCand / kMixThreads; ++u) c += ck[u] == T && ci[u] < mid;
+                if (block_sum(c, red, wave, lane) >= need_eq) mhi = mid;
+                else mlo = mid;
+            }
+        }
+        const int M = mhi;
+#pragma unroll
+        for (int u = 0; u < kMaxCand / kMixThreads; ++u) {
+            if (ck[u] > T || (ck[u] == T && ci[u] < M)) {
+                const int s_ = atomicAdd(&n_sel, 1);
+                if (s_ < kMaxTopk) {
+                    sel_idx[s_] = ci[u];
+                    sel_val[s_] = key_value(ck[u]);
+                }
+            }
+        }
+    } else {
+        auto count_ge = [&](uint32_t t) {  // elements of this thread with key >= t
+            int c = 0;
+#pragma unroll
+            for (int j = 0; j < NVEC; ++j) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    uint32_t w = keys[j][q];
+                    TAH_OPAQUE1(w);  // the two halves are split here, every time: hoisted out of the bisection
+                                     // loop they would double the registers the row occupies
+                    c += ((w & 0xffffu) >= t) + ((w >> 16) >= t);
+                }
+            }
+            return c;
+        };
+
+        // ---- largest key T with count(key >= T) >= k: bisection, invariant count(>= lo) >= k > count(>= hi) ----
+        uint32_t lo = 1u, hi = 0x10000u;  // key 0 only marks indices past the end
+        int n_ge = V;                     // count(key >= lo): every real key is >= 1
+        while (hi - lo > 1) {
+            const uint32_t mid = (lo + hi) >> 1;
+            const int cnt = block_sum(count_ge(mid), red, wave, lane);
+            if (cnt >= k) { lo = mid; n_ge = cnt; }
+            else hi = mid;
+        }
+        const uint32_t T = lo;
+        const int n_gt = block_sum(count_ge(T + 1), red, wave, lane);
+        const int need_eq = k - n_gt;  // >= 1: that many elements with key == T are taken, lowest indices first
+        // ---- smallest index bound M with count(key == T and index < M) >= need_eq ----
+        auto count_eq_below = [&](int m) {
+            int c = 0;
+#pragma unroll
+            for (int j = 0; j < NVEC; ++j) {
+                int d = m - (j * kMixThreads + tid) * 8;  // index e of this piece is below the bound iff e < d
+                TAH_OPAQUE1(d);                           // (compared with constants: no per-element index registers)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    uint32_t w = keys[j][q];
+                    TAH_OPAQUE1(w);
+                    c += ((w & 0xffffu) == T) && (2 * q < d);
+                    c += ((w >> 16) == T) && (2 * q + 1 < d);
+                }
+            }
+            return c;
+        };
+        int mlo = 0, mhi = V;  // invariant: count(< mlo) < need_eq <= count(< mhi)
+        // (the usual case needs no search: every element with key == T is taken)
+        if (n_ge - n_gt > need_eq) {
+            while (mhi - mlo > 1) {
+                const int mid = (mlo + mhi) >> 1;
+                if (block_sum(count_eq_below(mid), red, wave, lane) >= need_eq) mhi = mid;
+                else mlo = mid;
+            }
+        }
+        const int M = mhi;
+
+        // ---- gather the k selected (index, value) pairs ----
+#pragma unroll
+        for (int j = 0; j < NVEC; ++j) {
+            int i0 = (j * kMixThreads + tid) * 8;
+            TAH_OPAQUE1(i0);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                uint32_t w = keys[j][e / 2];
+                TAH_OPAQUE1(w);
+                const uint32_t key = (w >> (16 * (e % 2))) & 0xffffu;
+                if (key > T || (key == T && e < M - i0)) {
+                    const int s = atomicAdd(&n_sel, 1);
+                    if (s < kMaxTopk) {
+                        sel_idx[s] = i0 + e;
+                        sel_val[s] = key_value(key);
+                    }
                 }
             }
         }
@@ -206,12 +317,26 @@ __global__ __launch_bounds__(kMixThreads) void topk_mix_kernel(const MixParams p
         const int cg = cg0 + (cgs >= kMixThreads ? tid : tid % cgs);
         float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         if (cg < cgs && part < parts) {
-            for (int i = part; i < n; i += parts) {
-                // probability rounded to bf16 (softmax output of the bf16 arithmetic), product rounded to bf16
-                const float pr = round_bf16(ord_w[i] * inv);
-                const bf16x8 e = *reinterpret_cast<const bf16x8*>(p.emb + (int64_t)ord_idx[i] * p.e_rs + cg * 8);
+            // eight embedding rows are fetched before the first of them is used (one workgroup per token: what
+            // this loop waits for is memory latency), and added in the same order as one by one
+            constexpr int kAhead = 8;
+            for (int i = part; i < n; i += parts * kAhead) {
+                bf16x8 e[kAhead];
 #pragma unroll
-                for (int c = 0; c < 8; ++c) acc[c] += round_bf16(pr * (float)e[c]);
+                for (int u = 0; u < kAhead; ++u) {
+                    const int ii = i + u * parts;
+                    if (ii < n) e[u] = *reinterpret_cast<const bf16x8*>(p.emb + (int64_t)ord_idx[ii] * p.e_rs + cg * 8);
+                }
+#pragma unroll
+                for (int u = 0; u < kAhead; ++u) {
+                    const int ii = i + u * parts;
+                    if (ii < n) {
+                        // probability rounded to bf16 (softmax output of the bf16 arithmetic), product rounded to bf16
+                        const float pr = round_bf16(ord_w[ii] * inv);
+#pragma unroll
+                        for (int c = 0; c < 8; ++c) acc[c] += round_bf16(pr * (float)e[u][c]);
+                    }
+                }
             }
 #pragma unroll
             for (int c = 0; c < 8; ++c) partial[(int64_t)part * H + cg * 8 + c] = acc[c];

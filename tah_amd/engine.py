@@ -179,12 +179,15 @@ class TaHDecodeEngine:
         return torch.sigmoid((h @ w.dec_w2.t() + w.dec_b2).float()).view(-1)
 
     # ── one token per sequence through all layers at one depth ───────────
-    def _pass_single(self, x, pos, depth: int, slot_of, q_pos, q_depth):
+    def _rope_rows(self, pos):
+        at = pos.long().clamp(0, self.max_len - 1)  # a position past the tables (a caller replaying beyond the
+        return self.cos[at], self.sin[at]           # capacity) must not read outside them
+
+    def _pass_single(self, x, pos, depth: int, slot_of, q_pos, q_depth, rope=None):
         """x [B, H]; appends this token's K/V to the depth's slabs (rows with slot_of < 0 are not cached) and
         attends with q_pos / q_depth per row (q_pos < 0: the row sees nothing and is dropped by the caller)."""
         c = self.cfg
-        at = pos.long().clamp(0, self.max_len - 1)  # a position past the tables (a caller replaying beyond the
-        cos, sin = self.cos[at], self.sin[at]       # capacity) must not read outside them
+        cos, sin = rope if rope is not None else self._rope_rows(pos)
         for l, L in enumerate(self.w.layers):
             qkv = self._rms(x, L["ln1"]) @ L["wqkv"].t()
             q, k, v = self._split_qkv(qkv)
@@ -219,7 +222,8 @@ class TaHDecodeEngine:
         act = active if active is not None else torch.ones(B, dtype=torch.bool, device=self.device)
         slot0 = torch.where(act, self.rows, self.minus1)
         qpos0 = torch.where(act, pos, self.minus1)
-        h0 = self._pass_single(self.w.embed[tok], pos, 0, slot0, qpos0, self.zeros_i)
+        rope = self._rope_rows(pos)  # both latent iterations of a token use its position
+        h0 = self._pass_single(self.w.embed[tok], pos, 0, slot0, qpos0, self.zeros_i, rope)
         l0 = h0 @ self.w.lm_head.t()
         hard = (self.decide(h0) > self.w.threshold) if force_hard is None else force_hard
         hard = hard & act
@@ -227,7 +231,7 @@ class TaHDecodeEngine:
         x1 = ops.topk_mix(l0, self.w.embed, self.cfg.topk, row_enable=hard)
         slot1 = torch.where(hard, self.rows, self.minus1)
         qpos1 = torch.where(hard, pos, self.minus1)
-        h1 = self._pass_single(x1, pos, 1, slot1, qpos1, hard.to(torch.int32))
+        h1 = self._pass_single(x1, pos, 1, slot1, qpos1, hard.to(torch.int32), rope)
         return l0, h1 @ self.w.lm_head.t(), hard
 
     # ── prefill: packed prompts, both depths, through the varlen kernels ──

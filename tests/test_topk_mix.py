@@ -29,6 +29,7 @@ def _run(device, seed, rows, V, H, k, **kw):
 @pytest.mark.parametrize("seed,rows,V,H,k,kw", [
     (0, 2, 700, 64, 100, {}), (1, 1, 9000, 32, 17, dict(ties=0.05)), (2, 2, 90, 16, 100, {}), (3, 1, 17000, 256, 100, {}),
     (4, 1, 1003, 8, 256, dict(ties=0.3)),
+    (5, 1, 17000, 16, 50, dict(ties=0.2)),   # 3400 equal logits at the threshold: more than the candidate list holds
 ])
 def test_topk_mix_on_cpu_shim(seed, rows, V, H, k, kw):
     with emu_util.emulated():
