@@ -274,6 +274,15 @@ typedef struct tah_qk_prep_args {
     /* != 0: the caller promises that every sequence brings at most one row and that the slots named are all
      * different (a decode step): the lengths are then advanced by the same launch instead of a second one */
     int32_t append_one_row_per_seq;
+    /* Optional: the layer's input RMSNorm folded in.  With `norm_input` set, q, k and v are projections of the
+     * un-normalised rows norm_input[rows, norm_cols] through weights that already carry the norm's weight
+     * (W' = W diag(g)), and every head is first multiplied by the row's rsqrt(mean(norm_input[row]^2) + norm_eps):
+     * the norm needs no launch of its own (Qwen3DecoderLayer.forward: input_layernorm, then q|k|v projections).
+     * V is then scaled as well (to v_out, or on its way into the slabs).  norm_cols % 8 == 0. */
+    const void* norm_input;
+    int64_t norm_input_row_stride;
+    int32_t norm_cols;
+    float norm_eps;
 } tah_qk_prep_args;
 
 /* Per-head RMSNorm of q and k, rotary embedding of both, and optionally the KV-cache append,
@@ -308,6 +317,12 @@ int tah_topk_mix(const tah_topk_mix_args* args, tah_stream_t stream);
  * tah/model/tah_model.py:616-623) on the output of one fused gate|up projection.  One launch instead of two. */
 int tah_silu_mul(const void* gate_up, void* out, int32_t rows, int32_t inter, int64_t gate_up_row_stride,
                  int64_t out_row_stride, tah_stream_t stream);
+/* The same with the MLP's input RMSNorm folded in (post_attention_layernorm, then gate|up projections): gate_up is the
+ * projection of the un-normalised rows norm_input[rows, norm_cols] through a weight that carries the norm's weight;
+ * gate and up are multiplied by the row's rsqrt(mean(norm_input[row]^2) + norm_eps) before the gate. */
+int tah_silu_mul_normed(const void* gate_up, void* out, int32_t rows, int32_t inter, int64_t gate_up_row_stride,
+                        int64_t out_row_stride, const void* norm_input, int64_t norm_input_row_stride, int32_t norm_cols,
+                        float norm_eps, tah_stream_t stream);
 
 /* One greedy generation step after the logits exist: per row, the final logits (first-iteration logits, plus
  * the second iteration's for rows that took one, summed in bf16 as the model's logits buffers are,

@@ -139,6 +139,7 @@ class QkPrepArgs(C.Structure):
         ("cache", KvSegment),
         ("overflow", c_void_p),
         ("append_one_row_per_seq", c_int32),
+        ("norm_input", c_void_p), ("norm_input_row_stride", c_int64), ("norm_cols", c_int32), ("norm_eps", C.c_float),
     ]
 
 
@@ -172,6 +173,8 @@ PROTOTYPES = {
     "tah_duo_schedule_bytes": (C.c_size_t, [c_int32] * 7),
     "tah_duo_schedule_build": (C.c_int, [C.POINTER(DuoScheduleArgs), c_void_p]),
     "tah_greedy_step": (C.c_int, [C.POINTER(GreedyStepArgs), c_void_p]),
+    "tah_silu_mul_normed": (C.c_int, [c_void_p, c_void_p, c_int32, c_int32, c_int64, c_int64, c_void_p, c_int64, c_int32, c_float,
+                                      c_void_p]),
     "tah_duo_fwd_masked": (C.c_int, [C.POINTER(DuoFwdArgs), C.POINTER(AdditiveMask), c_void_p]),
     "tah_duo_bwd_masked": (C.c_int, [C.POINTER(DuoBwdArgs), C.POINTER(AdditiveMask), c_void_p]),
     "tah_duo_decode_workspace_bytes": (C.c_size_t, [c_int32, c_int32, c_int32, c_int32]),

@@ -365,6 +365,10 @@ struct PrepParams {
     float eps;
     int32_t rows, hq, hkv, append;
     int32_t own_len;  // every sequence appends at most one row: the row's workgroup advances the length itself
+    const __bf16* xn;  // rows whose RMS the projections still have to be divided by (input norm folded in), or nullptr
+    int64_t xn_rs;
+    int32_t xn_cols;
+    float xn_eps;
     AppendParams a;  // destination slabs (append != 0); its k_new / v_new fields are not used
 };
 
@@ -406,6 +410,24 @@ __global__ __launch_bounds__(256) void qk_prep_kernel(const PrepParams p) {
     u32x4 ahead[kAhead];
 #pragma unroll
     for (int i = 0; i < kAhead; ++i) ahead[i] = load_item(16 * i + sub);
+    // input norm folded in: the factor the whole row is scaled by (1 when there is none)
+    float rin = 1.0f;
+    if (p.xn) {
+        __shared__ float xn_part[4];
+        const __bf16* xr = p.xn + (int64_t)r * p.xn_rs;
+        float ss = 0.f;
+        for (int c = threadIdx.x * 8; c < p.xn_cols; c += 256 * 8) {
+            const u32x4 x = *reinterpret_cast<const u32x4*>(xr + c);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) ss += bf16_lo(x[i]) * bf16_lo(x[i]) + bf16_hi(x[i]) * bf16_hi(x[i]);
+        }
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m);
+        if (lane == 0) xn_part[threadIdx.x / kWave] = ss;
+        __syncthreads();
+        ss = (xn_part[0] + xn_part[1]) + (xn_part[2] + xn_part[3]);
+        rin = __builtin_amdgcn_rsqf(ss / (float)p.xn_cols + p.xn_eps);
+    }
     const u32x4 cs = *reinterpret_cast<const u32x4*>(p.cos + (int64_t)r * p.cs_rs + 8 * j);
     const u32x4 sn = *reinterpret_cast<const u32x4*>(p.sin + (int64_t)r * p.cs_rs + 8 * j);
     const u32x4 qw = *reinterpret_cast<const u32x4*>(p.qw + 8 * j), kw = *reinterpret_cast<const u32x4*>(p.kw + 8 * j);
@@ -447,7 +469,11 @@ __global__ __launch_bounds__(256) void qk_prep_kernel(const PrepParams p) {
     for (int pass = 0; pass * 16 < items; ++pass) {
         const int it = pass * 16 + sub;
         const bool is_q = it < p.hq, is_k = !is_q && it < p.hq + p.hkv, is_v = !is_q && !is_k && it < items;
-        const u32x4 xin = pass == 0 ? ahead[0] : pass == 1 ? ahead[1] : load_item(it);
+        u32x4 xin = pass == 0 ? ahead[0] : pass == 1 ? ahead[1] : load_item(it);
+        if (p.xn) {  // the row's input-norm factor, applied where the eager modules have a normalised projection
+#pragma unroll
+            for (int i = 0; i < 4; ++i) xin[i] = pack_bf16(bf16_lo(xin[i]) * rin, bf16_hi(xin[i]) * rin);
+        }
         if (is_v && vdst)  // a V head: moved as it is
             *reinterpret_cast<u32x4*>(vdst + (int64_t)(it - p.hq - p.hkv) * vd_hs + 8 * j) = xin;
         const int h = is_q ? it : it - p.hq;
@@ -631,8 +657,9 @@ extern "C" int tah_qk_prep(const tah_qk_prep_args* a, tah_stream_t stream) {
     for (int64_t x : strides)
         if (x % 8 != 0) return TAH_E_ALIGN;  // every access is 16 bytes wide (eight elements)
     if (a->cos_sin_row_stride % 8 != 0) return TAH_E_ALIGN;
+    if (a->norm_input && (a->norm_cols <= 0 || a->norm_cols % 8 != 0 || a->norm_input_row_stride % 8 != 0)) return TAH_E_SHAPE;
     const void* ptrs[] = {a->q, a->k, a->v, a->q_out, a->k_out, a->v_out, a->q_weight, a->k_weight, a->cos, a->sin,
-                          a->append ? a->cache.k : nullptr, a->append ? a->cache.v : nullptr};
+                          a->append ? a->cache.k : nullptr, a->append ? a->cache.v : nullptr, a->norm_input};
     for (const void* q : ptrs)
         if (q && !aligned16(q)) return TAH_E_ALIGN;
     PrepParams p;
@@ -648,6 +675,8 @@ extern "C" int tah_qk_prep(const tah_qk_prep_args* a, tah_stream_t stream) {
     p.eps = a->eps;
     p.rows = a->rows; p.hq = a->hq; p.hkv = a->hkv; p.append = a->append ? 1 : 0;
     p.own_len = (a->append && a->append_one_row_per_seq) ? 1 : 0;
+    p.xn = static_cast<const __bf16*>(a->norm_input);
+    p.xn_rs = a->norm_input_row_stride; p.xn_cols = a->norm_cols; p.xn_eps = a->norm_eps;
     p.a = AppendParams{};
     if (a->append) {
         p.a.pos_new = a->pos_new; p.a.cu_new = a->cu_new; p.a.slot_of = a->slot_of;

@@ -20,16 +20,42 @@ __device__ __forceinline__ float lo_f(uint32_t w) { return __uint_as_float(w << 
 __device__ __forceinline__ float hi_f(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
 __device__ __forceinline__ float silu(float x) { return x / (1.0f + fast_exp2(-x * kLog2e)); }
 
-// out[r][i] = bf16(bf16(silu(gu[r][i])) * gu[r][inter + i]), eight elements per thread
-__global__ __launch_bounds__(256) void silu_mul_kernel(const __bf16* gu, __bf16* out, int inter, int64_t gu_rs, int64_t out_rs) {
+// out[r][i] = bf16(bf16(silu(gu[r][i])) * gu[r][inter + i]), eight elements per thread.  kNormed: gate and up are
+// first multiplied by rsqrt(mean(xn[r]^2) + eps) and rounded to bf16 (the MLP's input norm folded in: the projection
+// ran on the un-normalised row through a weight that carries the norm's weight); every workgroup of a row sums the
+// row's squares for itself (a few KB from L2).
+template <bool kNormed>
+__global__ __launch_bounds__(256) void silu_mul_kernel(const __bf16* gu, __bf16* out, int inter, int64_t gu_rs, int64_t out_rs,
+                                                       const __bf16* xn, int64_t xn_rs, int xn_cols, float xn_eps) {
     const int r = blockIdx.y;
     const int i = (blockIdx.x * 256 + threadIdx.x) * 8;
+    float rin = 1.0f;
+    if constexpr (kNormed) {
+        __shared__ float part[4];
+        const __bf16* xr = xn + (int64_t)r * xn_rs;
+        float ss = 0.f;
+        for (int c = threadIdx.x * 8; c < xn_cols; c += 256 * 8) {
+            const u32x4 x = *reinterpret_cast<const u32x4*>(xr + c);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) ss += lo_f(x[q]) * lo_f(x[q]) + hi_f(x[q]) * hi_f(x[q]);
+        }
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m);
+        if (threadIdx.x % kWave == 0) part[threadIdx.x / kWave] = ss;
+        __syncthreads();
+        ss = (part[0] + part[1]) + (part[2] + part[3]);
+        rin = __builtin_amdgcn_rsqf(ss / (float)xn_cols + xn_eps);
+    }
     if (i >= inter) return;
-    const u32x4 g = *reinterpret_cast<const u32x4*>(gu + (int64_t)r * gu_rs + i);
-    const u32x4 u = *reinterpret_cast<const u32x4*>(gu + (int64_t)r * gu_rs + inter + i);
+    u32x4 g = *reinterpret_cast<const u32x4*>(gu + (int64_t)r * gu_rs + i);
+    u32x4 u = *reinterpret_cast<const u32x4*>(gu + (int64_t)r * gu_rs + inter + i);
     u32x4 o;
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
+        if constexpr (kNormed) {
+            g[q] = pack2(lo_f(g[q]) * rin, hi_f(g[q]) * rin);
+            u[q] = pack2(lo_f(u[q]) * rin, hi_f(u[q]) * rin);
+        }
         const uint32_t s = pack2(silu(lo_f(g[q])), silu(hi_f(g[q])));  // the activation's own bf16 rounding
         o[q] = pack2(lo_f(s) * lo_f(u[q]), hi_f(s) * hi_f(u[q]));
     }
@@ -170,16 +196,29 @@ extern "C" int tah_greedy_step(const tah_greedy_step_args* a, tah_stream_t strea
     return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
 }
 
-extern "C" int tah_silu_mul(const void* gate_up, void* out, int32_t rows, int32_t inter, int64_t gate_up_row_stride,
-                            int64_t out_row_stride, tah_stream_t stream) {
+extern "C" int tah_silu_mul_normed(const void* gate_up, void* out, int32_t rows, int32_t inter, int64_t gate_up_row_stride,
+                                   int64_t out_row_stride, const void* norm_input, int64_t norm_input_row_stride,
+                                   int32_t norm_cols, float norm_eps, tah_stream_t stream) {
     using namespace tah;
     if (rows < 0 || inter < 0 || inter % 8 != 0 || rows > 65535) return TAH_E_SHAPE;
+    if (norm_input && (norm_cols <= 0 || norm_cols % 8 != 0 || norm_input_row_stride % 8 != 0)) return TAH_E_SHAPE;
     if (rows == 0 || inter == 0) return TAH_OK;
     if (!gate_up || !out) return TAH_E_NULL;
     if ((reinterpret_cast<uintptr_t>(gate_up) & 15) || (reinterpret_cast<uintptr_t>(out) & 15) || gate_up_row_stride % 8 ||
-        out_row_stride % 8)
+        out_row_stride % 8 || (reinterpret_cast<uintptr_t>(norm_input) & 15))
         return TAH_E_ALIGN;
-    hipLaunchKernelGGL(silu_mul_kernel, dim3((inter / 8 + 255) / 256, rows), dim3(256), 0, static_cast<hipStream_t>(stream),
-                       static_cast<const __bf16*>(gate_up), static_cast<__bf16*>(out), inter, gate_up_row_stride, out_row_stride);
+    const dim3 grid((inter / 8 + 255) / 256, rows);
+    const __bf16* xn = static_cast<const __bf16*>(norm_input);
+    if (xn)
+        hipLaunchKernelGGL(silu_mul_kernel<true>, grid, dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<const __bf16*>(gate_up),
+                           static_cast<__bf16*>(out), inter, gate_up_row_stride, out_row_stride, xn, norm_input_row_stride, norm_cols, norm_eps);
+    else
+        hipLaunchKernelGGL(silu_mul_kernel<false>, grid, dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<const __bf16*>(gate_up),
+                           static_cast<__bf16*>(out), inter, gate_up_row_stride, out_row_stride, xn, (int64_t)0, 0, 0.f);
     return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
+}
+
+extern "C" int tah_silu_mul(const void* gate_up, void* out, int32_t rows, int32_t inter, int64_t gate_up_row_stride,
+                            int64_t out_row_stride, tah_stream_t stream) {
+    return tah_silu_mul_normed(gate_up, out, rows, inter, gate_up_row_stride, out_row_stride, nullptr, 0, 0, 0.f, stream);
 }

@@ -29,6 +29,7 @@ struct Api {
     decltype(&tah_duo_schedule_bytes) schedule_bytes = nullptr;
     decltype(&tah_duo_schedule_build) schedule_build = nullptr;
     decltype(&tah_greedy_step) greedy_step = nullptr;
+    decltype(&tah_silu_mul_normed) silu_mul_normed = nullptr;
     decltype(&tah_duo_fwd_masked) fwd_masked = nullptr;
     decltype(&tah_duo_bwd_masked) bwd_masked = nullptr;
     decltype(&tah_duo_decode_workspace_bytes) decode_workspace_bytes = nullptr;
@@ -63,6 +64,7 @@ void load_library(const std::string& path, bool allow_host) {
     bind(g.schedule_bytes, "tah_duo_schedule_bytes");
     bind(g.schedule_build, "tah_duo_schedule_build");
     bind(g.greedy_step, "tah_greedy_step");
+    bind(g.silu_mul_normed, "tah_silu_mul_normed");
     bind(g.fwd_masked, "tah_duo_fwd_masked");
     bind(g.bwd_masked, "tah_duo_bwd_masked");
     bind(g.decode_workspace_bytes, "tah_duo_decode_workspace_bytes");
@@ -368,7 +370,8 @@ void qk_prep(const Tensor& q, const Tensor& k, const optional<Tensor>& v, const 
              const Tensor& q_weight, const Tensor& k_weight, const Tensor& cos, const Tensor& sin, double eps,
              const optional<Tensor>& ck, const optional<Tensor>& cv, const optional<Tensor>& cpos, const optional<Tensor>& start,
              const optional<Tensor>& len, const optional<Tensor>& overflow, const optional<Tensor>& cu_new,
-             const optional<Tensor>& pos_new, const optional<Tensor>& slot_of, bool one_row_per_seq) {
+             const optional<Tensor>& pos_new, const optional<Tensor>& slot_of, bool one_row_per_seq,
+             const optional<Tensor>& v_out, const optional<Tensor>& norm_input, double norm_eps) {
     need_lib();
     thd(q, "q"); thd(k, "k");
     Dev d; d.see(q); d.see(k); d.see(v); d.see(q_weight); d.see(k_weight); d.see(cos); d.see(sin); d.see(cu_new); d.see(pos_new);
@@ -409,6 +412,23 @@ void qk_prep(const Tensor& q, const Tensor& k, const optional<Tensor>& v, const 
         TORCH_CHECK(k_out.has_value(), "k_out is needed when nothing is appended");
         a.k_out = mptr(*k_out);
         a.k_out_row_stride = k_out->stride(0); a.k_out_head_stride = k_out->stride(1);
+        if (v_out.has_value()) {
+            TORCH_CHECK(v.has_value() && v_out->sizes() == v->sizes(), "v_out needs v, and its shape");
+            thd(*v_out, "v_out");
+            d.see(v_out);
+            a.v_out = mptr(*v_out);
+            a.v_out_row_stride = v_out->stride(0); a.v_out_head_stride = v_out->stride(1);
+        }
+    }
+    if (norm_input.has_value()) {
+        d.see(norm_input);
+        TORCH_CHECK(norm_input->dim() == 2 && norm_input->scalar_type() == at::kBFloat16 && norm_input->size(0) == q.size(0) &&
+                        norm_input->stride(1) == 1,
+                    "norm_input must be a bf16 [rows, hidden] tensor with unit inner stride");
+        a.norm_input = ptr(*norm_input);
+        a.norm_input_row_stride = norm_input->size(0) > 1 ? norm_input->stride(0) : norm_input->size(1);
+        a.norm_cols = (int32_t)norm_input->size(1);
+        a.norm_eps = (float)norm_eps;
     }
     check_rc(g.qk_prep(&a, d.stream()), "tah_qk_prep");
 }
@@ -488,13 +508,23 @@ Tensor topk_mix(const Tensor& logits, const Tensor& embedding, int64_t topk, con
     return out;
 }
 
-Tensor silu_mul(const Tensor& gate_up) {
+Tensor silu_mul(const Tensor& gate_up, const optional<Tensor>& norm_input, double norm_eps) {
     need_lib();
-    Dev d; d.see(gate_up);
+    Dev d; d.see(gate_up); d.see(norm_input);
     TORCH_CHECK(gate_up.dim() == 2 && gate_up.scalar_type() == at::kBFloat16 && gate_up.size(1) % 16 == 0 && gate_up.stride(1) == 1,
                 "silu_mul: gate_up must be bf16 [rows, 2*I] with I a multiple of 8 and a contiguous inner dimension");
     const int64_t rows = gate_up.size(0), inter = gate_up.size(1) / 2;
     auto out = at::empty({rows, inter}, gate_up.options());
+    if (norm_input.has_value()) {
+        TORCH_CHECK(norm_input->dim() == 2 && norm_input->scalar_type() == at::kBFloat16 && norm_input->size(0) == rows &&
+                        norm_input->stride(1) == 1,
+                    "silu_mul: norm_input must be a bf16 [rows, hidden] tensor with unit inner stride");
+        check_rc(g.silu_mul_normed(ptr(gate_up), mptr(out), (int32_t)rows, (int32_t)inter, rows > 1 ? gate_up.stride(0) : 2 * inter, inter,
+                                   ptr(*norm_input), rows > 1 ? norm_input->stride(0) : norm_input->size(1), (int32_t)norm_input->size(1),
+                                   (float)norm_eps, d.stream()),
+                 "tah_silu_mul_normed");
+        return out;
+    }
     check_rc(g.silu_mul(ptr(gate_up), mptr(out), (int32_t)rows, (int32_t)inter, rows > 1 ? gate_up.stride(0) : 2 * inter, inter, d.stream()),
              "tah_silu_mul");
     return out;

@@ -70,6 +70,19 @@ class Weights:
         self.dec_w2: torch.Tensor = None         # [1, Hd]
         self.dec_b2: torch.Tensor = None
         self.threshold: float = 0.5
+        self.norms_folded = False
+
+    def fold_norms(self) -> "Weights":
+        """Multiplies the input-norm weights into the projections that follow them (``wqkv *= ln1``, ``wgu *= ln2``,
+        column-wise, rounded to the model dtype once).  What is left of the two RMSNorms of a layer is a factor per
+        row, which ``tah_qk_prep`` and ``tah_silu_mul_normed`` apply: two launches per layer and latent iteration
+        less.  Done once, in place."""
+        if not self.norms_folded:
+            for L in self.layers:
+                L["wqkv"].mul_(L["ln1"][None, :])
+                L["wgu"].mul_(L["ln2"][None, :])
+            self.norms_folded = True
+        return self
 
     @staticmethod
     def random_init(cfg: EngineConfig, device, seed: int = 0, dtype=torch.bfloat16) -> "Weights":
@@ -126,10 +139,15 @@ def rope_tables(max_len: int, head_dim: int, theta: float, device, dtype=torch.b
 
 
 class TaHDecodeEngine:
-    def __init__(self, weights: Weights, batch: int, max_len: int, *, max_hard: Optional[int] = None, device="cuda"):
+    def __init__(self, weights: Weights, batch: int, max_len: int, *, max_hard: Optional[int] = None, device="cuda",
+                 fold_norms: bool = True):
+        """``fold_norms``: multiply the layers' input-norm weights into the projections behind them (in place in
+        ``weights``, once) so that the two RMSNorms of a layer cost no launch; needs hidden % 8 == 0 and bf16."""
         cfg = weights.cfg
         if cfg.head_dim != 128:
             raise TahDuoError("the kernels are built for head_dim 128")
+        if fold_norms and cfg.hidden % 8 == 0 and weights.embed.dtype == torch.bfloat16:
+            weights.fold_norms()
         self.w, self.cfg, self.B, self.max_len = weights, cfg, batch, max_len
         self.device = torch.device(device)
         self.max_hard = max_hard if max_hard is not None else max_len
@@ -163,8 +181,21 @@ class TaHDecodeEngine:
         return F.rms_norm(x, (x.shape[-1],), w, self.cfg.rms_eps)
 
     def _mlp(self, x, L):
-        gu = self._rms(x, L["ln2"]) @ L["wgu"].t()
-        return x.addmm_(ops.silu_mul(gu), L["wdown"].t())
+        if self.w.norms_folded:  # the norm's weight sits in wgu, its per-row factor is applied with the gate
+            h = ops.silu_mul(x @ L["wgu"].t(), norm_input=x, norm_eps=self.cfg.rms_eps)
+        else:
+            h = ops.silu_mul(self._rms(x, L["ln2"]) @ L["wgu"].t())
+        return x.addmm_(h, L["wdown"].t())
+
+    def _prefill_qkv(self, x, L, cos, sin):
+        """Prepared q, k and v of packed prompt rows (input norm, projections, q/k norm, rotary embedding)."""
+        c = self.cfg
+        if self.w.norms_folded:
+            q, k, v = self._split_qkv(x @ L["wqkv"].t())
+            return qk_norm_rope(q, k, L["qn"], L["kn"], cos, sin, c.rms_eps, v=v, norm_input=x, norm_eps=c.rms_eps)
+        q, k, v = self._split_qkv(self._rms(x, L["ln1"]) @ L["wqkv"].t())
+        qo, ko = qk_norm_rope(q, k, L["qn"], L["kn"], cos, sin, c.rms_eps)
+        return qo, ko, v
 
     def _split_qkv(self, qkv):
         c = self.cfg
@@ -188,15 +219,17 @@ class TaHDecodeEngine:
         attends with q_pos / q_depth per row (q_pos < 0: the row sees nothing and is dropped by the caller)."""
         c = self.cfg
         cos, sin = rope if rope is not None else self._rope_rows(pos)
+        folded = self.w.norms_folded
         for l, L in enumerate(self.w.layers):
-            qkv = self._rms(x, L["ln1"]) @ L["wqkv"].t()
+            qkv = (x if folded else self._rms(x, L["ln1"])) @ L["wqkv"].t()
             q, k, v = self._split_qkv(qkv)
             cache = self.slabs0[l] if depth == 0 else self.slabs1[l]
             if self.measure_without_attention:  # timing aid: the step minus its q/k preparation and decode kernels
                 o = q.contiguous()
             else:
                 qo, _ = qk_norm_rope(q, k, L["qn"], L["kn"], cos, sin, c.rms_eps, v=v, cache=cache, cu_new=self.cu_rows,
-                                     slot_of=slot_of, pos_new=pos if depth == 1 else None, one_row_per_seq=True)
+                                     slot_of=slot_of, pos_new=pos if depth == 1 else None, one_row_per_seq=True,
+                                     norm_input=x if folded else None, norm_eps=c.rms_eps)
                 o = _decode(qo, self.rows, q_pos, self.slabs0[l], self.slabs1[l], scale=self.scale, q_depth=q_depth,
                             static_scratch=self.static_scratch)
             x = x.addmm_(o.view(x.shape[0], c.hq * c.head_dim), L["wo"].t())  # residual add inside the GEMM, in place
@@ -260,8 +293,7 @@ class TaHDecodeEngine:
         # launch order of the prompts' tiles, heaviest first across prompts: one table serves all layers of a depth
         sched0 = ops.duo_schedule(cu, cu, zc, zc, zi, c.hq, c.hkv, N, N, 0)
         for l, L in enumerate(w.layers):
-            q, k, v = self._split_qkv(self._rms(x, L["ln1"]) @ L["wqkv"].t())
-            qo, ko = qk_norm_rope(q, k, L["qn"], L["kn"], cos, sin, c.rms_eps)
+            qo, ko, v = self._prefill_qkv(x, L, cos, sin)
             o1, _, _, _ = ops.duo_fwd_varlen(qo, ko, v, cu, cu, qo[:0], ko[:0], v[:0], zi, zi, zc, zc, self.scale,
                                              schedule=sched0)
             self.slabs0[l].append(ko, v, cu)
@@ -288,8 +320,7 @@ class TaHDecodeEngine:
             cos2, sin2 = self.cos[pos2.long()], self.sin[pos2.long()]
             sched1 = ops.duo_schedule(zc, cu, cu2, cu2, pos2, c.hq, c.hkv, 0, N, n2)
             for l, L in enumerate(w.layers):
-                q, k, v = self._split_qkv(self._rms(x2, L["ln1"]) @ L["wqkv"].t())
-                qo, ko = qk_norm_rope(q, k, L["qn"], L["kn"], cos2, sin2, c.rms_eps)
+                qo, ko, v = self._prefill_qkv(x2, L, cos2, sin2)
                 k1, v1 = kv_tok[l]
                 _, _, o2, _ = ops.duo_fwd_varlen(qo[:0], k1, v1, zc, cu, qo, ko, v, pos2, pos2, cu2, cu2, self.scale,
                                                  schedule=sched1)

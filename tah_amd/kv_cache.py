@@ -51,7 +51,8 @@ def qk_norm_rope(q: torch.Tensor, k: torch.Tensor, q_weight: torch.Tensor, k_wei
                  cos: torch.Tensor, sin: torch.Tensor, eps: float, *, v: Optional[torch.Tensor] = None,
                  cache: Optional[KvSlabs] = None, cu_new: Optional[torch.Tensor] = None,
                  pos_new: Optional[torch.Tensor] = None, slot_of: Optional[torch.Tensor] = None,
-                 in_place: bool = False, one_row_per_seq: bool = False):
+                 in_place: bool = False, one_row_per_seq: bool = False, norm_input: Optional[torch.Tensor] = None,
+                 norm_eps: float = 0.0):
     """Per-head RMSNorm of q and k, rotary embedding of both and, with ``cache``, the KV append, in one
     kernel: the steps of ``Qwen3Attention.forward`` between the projections and the attention call
     (``q_norm``, ``k_norm``, ``apply_rotary_pos_emb``, ``past_key_values.update``), with bf16 roundings
@@ -61,16 +62,25 @@ def qk_norm_rope(q: torch.Tensor, k: torch.Tensor, q_weight: torch.Tensor, k_wei
     weights ``[128]``, cos / sin ``[rows, 128]``, all bf16.  Returns ``(q_out, k_out)``; with ``cache``
     K and V go to the slabs (rows ``[cu_new[i], cu_new[i+1])`` to slot ``slot_of[i]``) and ``k_out`` is
     ``None``.  ``one_row_per_seq=True`` (a decode step: every sequence brings at most one row, all slots
-    different) lets the same launch advance the slab lengths."""
+    different) lets the same launch advance the slab lengths.
+
+    ``norm_input`` ``[rows, hidden]`` folds the layer's input RMSNorm in: q, k, v are then projections of these
+    un-normalised rows through weights that carry the norm's weight, and the kernel multiplies every head by the
+    row's ``rsqrt(mean(norm_input**2) + norm_eps)`` first.  Without a cache the scaled V comes back as a third
+    result."""
     q_out = q if in_place else torch.empty_like(q)
     if cache is not None:
         _call("qk_prep", q, k, v, q_out, None, q_weight, k_weight, cos, sin, float(eps), cache.k, cache.v, cache.pos,
-              cache.start, cache.len, cache.overflow, cu_new, pos_new, slot_of, bool(one_row_per_seq))
+              cache.start, cache.len, cache.overflow, cu_new, pos_new, slot_of, bool(one_row_per_seq), None, norm_input,
+              float(norm_eps))
         return q_out, None
     k_out = k if in_place else torch.empty_like(k)
+    v_out = None
+    if norm_input is not None and v is not None:
+        v_out = v if in_place else torch.empty_like(v)
     _call("qk_prep", q, k, v, q_out, k_out, q_weight, k_weight, cos, sin, float(eps), None, None, None, None, None, None,
-          None, None, None, False)
-    return q_out, k_out
+          None, None, None, False, v_out, norm_input, float(norm_eps))
+    return (q_out, k_out) if v_out is None else (q_out, k_out, v_out)
 
 
 _WORKSPACES = {}

@@ -104,9 +104,13 @@ def topk_mix(logits: torch.Tensor, embedding: torch.Tensor, topk: int, row_enabl
     return _call("topk_mix", logits, embedding, int(topk), row_enable, out)
 
 
-def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
-    """``silu(gate) * up`` of a fused gate|up projection, bf16 [rows, 2*I] -> [rows, I], in one launch."""
-    return _call("silu_mul", gate_up)
+def silu_mul(gate_up: torch.Tensor, norm_input: Optional[torch.Tensor] = None, norm_eps: float = 0.0) -> torch.Tensor:
+    """``silu(gate) * up`` of a fused gate|up projection, bf16 [rows, 2*I] -> [rows, I], in one launch.
+
+    ``norm_input`` [rows, hidden] folds the MLP's input RMSNorm in: ``gate_up`` is then the projection of these
+    un-normalised rows through a weight that carries the norm's weight, and gate and up are multiplied by the row's
+    ``rsqrt(mean(norm_input**2) + norm_eps)`` first."""
+    return _call("silu_mul", gate_up, norm_input, float(norm_eps))
 
 
 def greedy_step(logits0, logits1, hard, eos: int, tok, finished, pos, out_tokens, step_idx, out_len, n_hard, n_steps) -> None:

@@ -36,3 +36,18 @@ def assert_bf16_close(got: torch.Tensor, want: np.ndarray, what: str):
     worst = float(np.max(err / np.maximum(mag, 1e-30)))
     assert worst <= 2.0 ** -6 and exact >= 0.995, f"{what}: worst error / pair size {worst:.3e}, exact fraction {exact:.5f}"
     return exact
+
+
+def folded_norm_case(device, seed=50, rows=6, hq=4, hkv=2, hidden=512):
+    """Inputs for the input-norm-folded form and what the plain form gives on explicitly scaled projections:
+    returns (tensors, x, want_q, want_k, want_v) with want_* from the oracle on bf16(projection * r),
+    r = rsqrt(mean(x^2) + eps) per row."""
+    c = make_case(seed, rows, hq, hkv, scale=4.0)
+    g = np.random.default_rng(seed + 1)
+    x = R.bf16_round((g.standard_normal((rows, hidden)) * 7.0).astype(np.float32))
+    r = 1.0 / np.sqrt((x.astype(np.float64) ** 2).mean(-1) + 1e-6)
+    sc = lambda a: R.bf16_round((a.astype(np.float64) * r[:, None, None]).astype(np.float32))
+    wq, wk = R.qk_prep(sc(c["q"]), sc(c["k"]), c["qw"], c["kw"], c["cos"], c["sin"], c["eps"])
+    t = to_torch(c, device)
+    return c, t, torch.from_numpy(x).to(torch.bfloat16).to(device), wq, wk, sc(c["v"])
+

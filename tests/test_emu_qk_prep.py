@@ -22,6 +22,27 @@ def test_norm_rope_matches_oracle(rows, hq, hkv, scale):
     assert_bf16_close(k_out, wk, "k")
 
 
+def test_input_norm_folded_in_equals_scaling_the_projections_first():
+    from tah_amd.kv_cache import KvSlabs, qk_norm_rope
+    from tests.qk_prep_cases import folded_norm_case
+    c, t, x, wq, wk, wv = folded_norm_case("cpu")
+    with emu_util.emulated():
+        q_out, k_out, v_out = qk_norm_rope(t["q"], t["k"], t["qw"], t["kw"], t["cos"], t["sin"], c["eps"], v=t["v"],
+                                           norm_input=x, norm_eps=1e-6)
+        # and on the way into the slabs
+        rows = t["q"].shape[0]
+        slabs = KvSlabs(1, rows + 2, t["k"].shape[1], with_pos=False, device="cpu")
+        cu = torch.tensor([0, rows], dtype=torch.int32)
+        q2, _ = qk_norm_rope(t["q"], t["k"], t["qw"], t["kw"], t["cos"], t["sin"], c["eps"], v=t["v"], cache=slabs, cu_new=cu,
+                             norm_input=x, norm_eps=1e-6)
+    assert_bf16_close(q_out, wq, "q")
+    assert_bf16_close(k_out, wk, "k")
+    assert float((v_out.float() == torch.from_numpy(wv)).float().mean()) >= 0.99  # one bf16 step where r's last bit differs
+    assert torch.allclose(v_out.float(), torch.from_numpy(wv), rtol=2 ** -7, atol=0)
+    assert torch.equal(q2, q_out)
+    assert torch.equal(slabs.k[0, :, :rows].transpose(0, 1), k_out) and torch.equal(slabs.v[0, :, :rows].transpose(0, 1), v_out)
+
+
 def test_more_heads_than_one_pass_pair_and_empty_input():
     """48 head slots per row (three passes of 16; the first two are loaded up front), and a call with no rows."""
     from tah_amd.kv_cache import qk_norm_rope

@@ -80,3 +80,16 @@ def test_in_place_and_overflow():
                  cu_new=torch.tensor([0, 10, 40], dtype=torch.int32, device="cuda"))
     torch.cuda.synchronize()
     assert s.len.tolist() == [10, 16] and s.overflow.item() == 1
+
+
+def test_input_norm_folded_in_equals_scaling_the_projections_first_gpu():
+    from tah_amd.kv_cache import qk_norm_rope
+    from tests.qk_prep_cases import folded_norm_case
+    c, t, x, wq, wk, wv = folded_norm_case("cuda", seed=61, rows=300, hq=16, hkv=8, hidden=2048)
+    q_out, k_out, v_out = qk_norm_rope(t["q"], t["k"], t["qw"], t["kw"], t["cos"], t["sin"], c["eps"], v=t["v"],
+                                       norm_input=x, norm_eps=1e-6)
+    assert_bf16_close(q_out, wq, "q")
+    assert_bf16_close(k_out, wk, "k")
+    assert float((v_out.float().cpu() == torch.from_numpy(wv)).float().mean()) >= 0.99
+    assert torch.allclose(v_out.float().cpu(), torch.from_numpy(wv), rtol=2 ** -7, atol=0)
+

@@ -97,12 +97,28 @@ def _silu_mul_check(device):
     assert (got == want).float().mean() > 0.98
 
 
+def _silu_mul_normed_check(device):
+    """The MLP's input norm folded in: equals scaling gate and up by the row's rsqrt(mean(x^2) + eps) first."""
+    from tah_amd import ops
+    g = torch.Generator().manual_seed(4)
+    gu = (torch.randn(5, 2 * 1536, generator=g) * 9).to(torch.bfloat16)
+    x = (torch.randn(5, 640, generator=g) * 5).to(torch.bfloat16)
+    r = torch.rsqrt((x.double() ** 2).mean(-1, keepdim=True) + 1e-6)
+    scaled = (gu.double() * r).to(torch.bfloat16)
+    got = ops.silu_mul(gu.to(device), norm_input=x.to(device), norm_eps=1e-6).cpu()
+    want = ops.silu_mul(scaled.to(device)).cpu()
+    assert (got == want).float().mean() > 0.98   # one bf16 step where the last bit of r differs
+    assert torch.allclose(got.float(), want.float(), rtol=2.0 ** -6, atol=1e-30)
+
+
 @pytest.mark.skipif(not emu_util.have_host_clang(), reason="host clang++ not available")
 def test_silu_mul_on_cpu_shim():
     with emu_util.emulated():
         _silu_mul_check("cpu")
+        _silu_mul_normed_check("cpu")
 
 
 @pytest.mark.gpu
 def test_silu_mul_gpu():
     _silu_mul_check("cuda")
+    _silu_mul_normed_check("cuda")
