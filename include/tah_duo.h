@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define TAH_DUO_ABI_VERSION 3
+#define TAH_DUO_ABI_VERSION 4
 
 enum {
     TAH_OK = 0,
@@ -199,6 +199,8 @@ typedef struct tah_duo_decode_args {
     size_t workspace_bytes;
     int32_t nq, hq, hkv, d;
     float scale;
+    void* o_packed;          /* NULL, or bf16 [hq * d * 32]: the output once more as the rows operand of tah_linear_rows
+                              * (the o projection that follows), nq <= 32; rows nq .. 31 are left as they are */
 } tah_duo_decode_args;
 
 /* Bytes of split-K scratch tah_duo_decode needs for nq queries. */
@@ -323,6 +325,45 @@ int tah_silu_mul(const void* gate_up, void* out, int32_t rows, int32_t inter, in
 int tah_silu_mul_normed(const void* gate_up, void* out, int32_t rows, int32_t inter, int64_t gate_up_row_stride,
                         int64_t out_row_stride, const void* norm_input, int64_t norm_input_row_stride, int32_t norm_cols,
                         float norm_eps, tah_stream_t stream);
+
+/* Linear layers of a decode step: at most 32 rows (one token per sequence) against a weight of megabytes.  The work
+ * is streaming the weight once, so weight and rows are kept in the order the kernel reads them:
+ *   packed weight  tiles of 16 output columns x 32 k, the 64 16-byte operands of the lanes of one
+ *                  v_mfma_f32_16x16x32_bf16 step next to each other, a tile's k steps one after another;
+ *                  n * k elements (2 n * k for TAH_LINEAR_GATE_UP), made once by tah_linear_pack_weight;
+ *   packed rows    bf16 [k / 32][2][64][8]: unit (step, half, lane) holds row 16 half + lane % 16, columns
+ *                  32 step + 8 (lane / 16) ... + 8; always 32 rows, the rows past `rows` are zero.  Made by
+ *                  tah_linear_pack_rows, by tah_linear_rows (out_packed) and by tah_duo_decode (o_packed).
+ * Replaces, for the rows of a decode step, in Qwen3DecoderLayer.forward / Qwen3Attention.forward / Qwen3MLP.forward
+ * of the base model the reference runs (transformers/models/qwen3/modeling_qwen3.py, third party;
+ * tah/model/tah_model.py:616-623): the q|k|v projections, o_proj + residual add, gate|up projections +
+ * act_fn(gate) * up, down_proj + residual add.  Products accumulate in float32 in a fixed order (results do not
+ * vary from run to run) and are rounded to bf16 where the eager modules round. */
+enum { TAH_LINEAR_PLAIN = 0, TAH_LINEAR_GATE_UP = 1 };
+
+/* w bf16 [n, k] row-major (nn.Linear weight), or [2 n, k] = [gate; up] stacked for TAH_LINEAR_GATE_UP; k % 32 == 0,
+ * n % 16 == 0 (gate|up: n % 24 == 0 or n % 16 == 0).  packed: n * k (2 n * k) elements, 16-byte aligned. */
+int tah_linear_pack_weight(const void* w, int64_t w_row_stride, void* packed, int32_t n, int32_t k, int32_t kind,
+                           tah_stream_t stream);
+/* x bf16 [rows, k] row-major, rows <= 32 -> x_packed bf16 [32 * k] (rows past `rows` zero). */
+int tah_linear_pack_rows(const void* x, int64_t x_row_stride, void* x_packed, int32_t rows, int32_t k, tah_stream_t stream);
+
+typedef struct tah_linear_rows_args {
+    const void* w_packed;     /* from tah_linear_pack_weight(n, k, kind) */
+    const void* x_packed;     /* packed rows [32 * k] */
+    const void* residual;     /* bf16 [rows, n] added to the product, or NULL (TAH_LINEAR_PLAIN only); may be `out` */
+    void* out;                /* bf16 [rows, n] row-major, or NULL */
+    void* out_packed;         /* packed rows [32 * n] for the next layer (n % 32 == 0), or NULL; one of out / out_packed
+                               * is needed */
+    int64_t residual_row_stride, out_row_stride; /* elements */
+    int32_t rows, n, k;       /* rows <= 32 */
+    int32_t kind;             /* TAH_LINEAR_PLAIN: out = x W^T [+ residual]
+                               * TAH_LINEAR_GATE_UP: out = bf16(silu(g)) * u, g = bf16(r x Wg^T), u = bf16(r x Wu^T) */
+    int32_t input_norm;       /* TAH_LINEAR_GATE_UP: r = rsqrt(mean(x[row]^2) + norm_eps), the MLP's input RMSNorm whose
+                               * weight is already inside W (0: r = 1) */
+    float norm_eps;
+} tah_linear_rows_args;
+int tah_linear_rows(const tah_linear_rows_args* args, tah_stream_t stream);
 
 /* One greedy generation step after the logits exist: per row, the final logits (first-iteration logits, plus
  * the second iteration's for rows that took one, summed in bf16 as the model's logits buffers are,

@@ -8,7 +8,7 @@ from __future__ import annotations
 
 import ctypes as C
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 c_void_p, c_int32, c_int64, c_float = C.c_void_p, C.c_int32, C.c_int64, C.c_float
 
@@ -104,7 +104,22 @@ class DuoDecodeArgs(C.Structure):
         ("workspace", c_void_p), ("workspace_bytes", C.c_size_t),
         ("nq", c_int32), ("hq", c_int32), ("hkv", c_int32), ("d", c_int32),
         ("scale", c_float),
+        ("o_packed", c_void_p),
     ]
+
+
+class LinearRowsArgs(C.Structure):
+    """``tah_linear_rows_args``"""
+
+    _fields_ = [
+        ("w_packed", c_void_p), ("x_packed", c_void_p), ("residual", c_void_p), ("out", c_void_p), ("out_packed", c_void_p),
+        ("residual_row_stride", c_int64), ("out_row_stride", c_int64),
+        ("rows", c_int32), ("n", c_int32), ("k", c_int32), ("kind", c_int32), ("input_norm", c_int32), ("norm_eps", c_float),
+    ]
+
+
+LINEAR_PLAIN, LINEAR_GATE_UP = 0, 1
+LINEAR_MAX_ROWS = 32
 
 
 class KvAppendArgs(C.Structure):
@@ -180,6 +195,9 @@ PROTOTYPES = {
     "tah_duo_decode_workspace_bytes": (C.c_size_t, [c_int32, c_int32, c_int32, c_int32]),
     "tah_duo_decode": (C.c_int, [C.POINTER(DuoDecodeArgs), c_void_p]),
     "tah_duo_decode_static": (C.c_int, [C.POINTER(DuoDecodeArgs), c_void_p]),
+    "tah_linear_pack_weight": (C.c_int, [c_void_p, c_int64, c_void_p, c_int32, c_int32, c_int32, c_void_p]),
+    "tah_linear_pack_rows": (C.c_int, [c_void_p, c_int64, c_void_p, c_int32, c_int32, c_void_p]),
+    "tah_linear_rows": (C.c_int, [C.POINTER(LinearRowsArgs), c_void_p]),
     "tah_kv_append": (C.c_int, [C.POINTER(KvAppendArgs), c_void_p]),
     "tah_qk_prep": (C.c_int, [C.POINTER(QkPrepArgs), c_void_p]),
     "tah_topk_mix": (C.c_int, [C.POINTER(TopkMixArgs), c_void_p]),

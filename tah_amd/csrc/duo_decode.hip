@@ -54,6 +54,7 @@ struct Seg {
 struct DecParams {
     const __bf16* q;
     __bf16* o;
+    __bf16* op;  // the output once more in the rows form of the linear-layer kernels ([k / 32][2][64][8]), or null
     float* lse;
     int64_t q_rs, q_hs, o_rs, o_hs;
     const int32_t *q_slot, *q_pos, *q_depth;
@@ -280,7 +281,12 @@ __global__ __launch_bounds__(256) void duo_decode_merge_kernel(const DecParams p
 #pragma unroll
         for (int j = 0; j < 8; ++j) { o += red4[j][tid]; lt += red4[j][kD]; }
         const float inv = lt > 0.f ? 1.0f / lt : 0.f;
-        p.o[(int64_t)qi * p.o_rs + (int64_t)head * p.o_hs + tid] = (__bf16)(o * inv);
+        const __bf16 ob = (__bf16)(o * inv);
+        p.o[(int64_t)qi * p.o_rs + (int64_t)head * p.o_hs + tid] = ob;
+        if (p.op) {  // row qi, column k of the [nq, hq * d] matrix the o projection multiplies
+            const int k = head * kD + tid;
+            p.op[((((int64_t)(k / 32) * 2 + qi / 16) * 64) + (qi % 16) + 16 * ((k % 32) / 8)) * 8 + k % 8] = ob;
+        }
         if (p.lse && tid == 0) p.lse[(int64_t)qi * p.hq + head] = lt > 0.f ? (mx + fast_log2(lt)) * kLn2 : kNegInf;
     }
 }
@@ -571,6 +577,8 @@ int decode_impl(const tah_duo_decode_args* a, void* ws, size_t ws_bytes, int too
     if (a->nq > 65535 || a->hq > 65535) return TAH_E_SHAPE;
     if (!a->q || !a->o || !a->q_slot || !a->q_pos || !ws) return TAH_E_NULL;
     if (!aligned16(a->q) || !aligned16(ws) || a->q_row_stride % 8 || a->q_head_stride % 8) return TAH_E_ALIGN;
+    if (a->o_packed && a->nq > 32) return TAH_E_SHAPE;
+    if (!aligned16(a->o_packed)) return TAH_E_ALIGN;
     if (int rc = check_seg(a->c1, false)) return rc;
     const bool any_depth1 = a->q_depth != nullptr || a->depth >= 1;
     if (any_depth1)
@@ -580,6 +588,7 @@ int decode_impl(const tah_duo_decode_args* a, void* ws, size_t ws_bytes, int too
     DecParams p;
     p.q = static_cast<const __bf16*>(a->q);
     p.o = static_cast<__bf16*>(a->o);
+    p.op = static_cast<__bf16*>(a->o_packed);
     p.lse = a->lse;
     p.q_rs = a->q_row_stride; p.q_hs = a->q_head_stride;
     p.o_rs = a->o_row_stride; p.o_hs = a->o_head_stride;

@@ -30,6 +30,9 @@ struct Api {
     decltype(&tah_duo_schedule_build) schedule_build = nullptr;
     decltype(&tah_greedy_step) greedy_step = nullptr;
     decltype(&tah_silu_mul_normed) silu_mul_normed = nullptr;
+    decltype(&tah_linear_pack_weight) linear_pack_weight = nullptr;
+    decltype(&tah_linear_pack_rows) linear_pack_rows = nullptr;
+    decltype(&tah_linear_rows) linear_rows = nullptr;
     decltype(&tah_duo_fwd_masked) fwd_masked = nullptr;
     decltype(&tah_duo_bwd_masked) bwd_masked = nullptr;
     decltype(&tah_duo_decode_workspace_bytes) decode_workspace_bytes = nullptr;
@@ -65,6 +68,9 @@ void load_library(const std::string& path, bool allow_host) {
     bind(g.schedule_build, "tah_duo_schedule_build");
     bind(g.greedy_step, "tah_greedy_step");
     bind(g.silu_mul_normed, "tah_silu_mul_normed");
+    bind(g.linear_pack_weight, "tah_linear_pack_weight");
+    bind(g.linear_pack_rows, "tah_linear_pack_rows");
+    bind(g.linear_rows, "tah_linear_rows");
     bind(g.fwd_masked, "tah_duo_fwd_masked");
     bind(g.bwd_masked, "tah_duo_bwd_masked");
     bind(g.decode_workspace_bytes, "tah_duo_decode_workspace_bytes");
@@ -320,10 +326,14 @@ int64_t decode_workspace_bytes(int64_t nq, int64_t hq, int64_t cap1, int64_t cap
 void duo_decode(const Tensor& q, const Tensor& o, const optional<Tensor>& lse, const Tensor& q_slot, const Tensor& q_pos,
                 const optional<Tensor>& q_depth, int64_t depth, const Tensor& k1, const Tensor& v1, const Tensor& start1,
                 const Tensor& len1, const optional<Tensor>& k2, const optional<Tensor>& v2, const optional<Tensor>& pos2,
-                const optional<Tensor>& start2, const optional<Tensor>& len2, const optional<Tensor>& workspace, double scale) {
+                const optional<Tensor>& start2, const optional<Tensor>& len2, const optional<Tensor>& workspace, double scale,
+                const optional<Tensor>& o_packed) {
     need_lib();
     thd(q, "q"); i32(q_slot, "q_slot"); i32(q_pos, "q_pos");
-    Dev d; d.see(q); d.see(o); d.see(lse); d.see(q_slot); d.see(q_pos); d.see(q_depth); d.see(k1); d.see(workspace);
+    Dev d; d.see(q); d.see(o); d.see(lse); d.see(q_slot); d.see(q_pos); d.see(q_depth); d.see(k1); d.see(workspace); d.see(o_packed);
+    if (o_packed.has_value())
+        TORCH_CHECK(o_packed->scalar_type() == at::kBFloat16 && o_packed->is_contiguous() && o_packed->numel() == 32 * q.size(1) * q.size(2),
+                    "duo_decode: o_packed must be a contiguous bf16 tensor of 32 * Hq * D elements");
     const bool need2 = q_depth.has_value() || depth >= 1;
     TORCH_CHECK(!need2 || (k2.has_value() && v2.has_value() && pos2.has_value() && start2.has_value() && len2.has_value()),
                 "depth-1 queries need the depth-1 cache");
@@ -337,6 +347,7 @@ void duo_decode(const Tensor& q, const Tensor& o, const optional<Tensor>& lse, c
     a.c1 = segment(k1, v1, c10::nullopt, start1, len1);
     if (need2) a.c2 = segment(*k2, *v2, pos2, *start2, *len2);
     a.nq = (int32_t)q.size(0); a.hq = (int32_t)q.size(1); a.hkv = (int32_t)k1.size(1); a.d = (int32_t)q.size(2); a.scale = (float)scale;
+    a.o_packed = o_packed.has_value() ? o_packed->data_ptr() : nullptr;
     if (workspace.has_value()) {
         a.workspace = workspace->data_ptr();
         a.workspace_bytes = (size_t)workspace->numel() * workspace->element_size();
@@ -566,6 +577,69 @@ void greedy_step(const Tensor& logits0, const optional<Tensor>& logits1, const o
     check_rc(g.greedy_step(&a, d.stream()), "tah_greedy_step");
 }
 
+// ---- linear layers of a decode step (tah_linear_rows) ------------------------------------------------------
+bool packed_vec(const Tensor& t, int64_t numel) {
+    return t.scalar_type() == at::kBFloat16 && t.is_contiguous() && t.numel() == numel;
+}
+
+// w [n, k] (gate_up: [2 n, k], gate rows then up rows) -> the weight in the order tah_linear_rows reads it, [n * k] or [2 n * k]
+Tensor linear_pack_weight(const Tensor& w, bool gate_up) {
+    need_lib();
+    Dev d; d.see(w);
+    TORCH_CHECK(w.dim() == 2 && w.scalar_type() == at::kBFloat16 && w.stride(1) == 1, "linear_pack_weight: w must be a bf16 [N, K] matrix");
+    TORCH_CHECK(!gate_up || w.size(0) % 2 == 0, "linear_pack_weight: a stacked [gate; up] weight has an even number of rows");
+    const int64_t n = gate_up ? w.size(0) / 2 : w.size(0), k = w.size(1);
+    Tensor out = at::empty({w.size(0) * k}, w.options());
+    check_rc(g.linear_pack_weight(ptr(w), w.stride(0), mptr(out), (int32_t)n, (int32_t)k, gate_up ? TAH_LINEAR_GATE_UP : TAH_LINEAR_PLAIN, d.stream()),
+             "tah_linear_pack_weight");
+    return out;
+}
+
+// x [rows <= 32, k] -> packed rows [32 * k]
+Tensor linear_pack_rows(const Tensor& x, const optional<Tensor>& out) {
+    need_lib();
+    Dev d; d.see(x); d.see(out);
+    TORCH_CHECK(x.dim() == 2 && x.scalar_type() == at::kBFloat16 && (x.numel() == 0 || x.stride(1) == 1), "linear_pack_rows: x must be a bf16 [rows, K] matrix");
+    const int64_t rows = x.size(0), k = x.size(1);
+    Tensor xp = out.has_value() ? *out : at::empty({32 * k}, x.options());
+    TORCH_CHECK(packed_vec(xp, 32 * k), "linear_pack_rows: out must be a contiguous bf16 tensor of 32 * K elements");
+    check_rc(g.linear_pack_rows(ptr(x), rows > 1 ? x.stride(0) : k, mptr(xp), (int32_t)rows, (int32_t)k, d.stream()), "tah_linear_pack_rows");
+    return xp;
+}
+
+// out = x W^T [+ residual] or silu(gate) * up, from packed operands; returns the row-major result (or nothing when
+// only the packed result is asked for).
+optional<Tensor> linear_rows(const Tensor& w_packed, const Tensor& x_packed, int64_t rows, int64_t n, int64_t k, bool gate_up,
+                             const optional<Tensor>& residual, const optional<Tensor>& out, const optional<Tensor>& out_packed,
+                             bool want_out, bool input_norm, double norm_eps) {
+    need_lib();
+    Dev d; d.see(w_packed); d.see(x_packed); d.see(residual); d.see(out); d.see(out_packed);
+    TORCH_CHECK(rows >= 0 && n >= 0 && k >= 0, "linear_rows: negative size");
+    TORCH_CHECK(packed_vec(w_packed, (gate_up ? 2 : 1) * n * k), "linear_rows: w_packed must come from linear_pack_weight for these sizes");
+    TORCH_CHECK(packed_vec(x_packed, 32 * k), "linear_rows: x_packed must be a contiguous bf16 tensor of 32 * K elements");
+    optional<Tensor> y = out;
+    if (!y.has_value() && want_out) y = at::empty({rows, n}, x_packed.options());
+    if (y.has_value())
+        TORCH_CHECK(y->dim() == 2 && y->size(0) == rows && y->size(1) == n && y->scalar_type() == at::kBFloat16 && (y->numel() == 0 || y->stride(1) == 1),
+                    "linear_rows: out must be bf16 [rows, N]");
+    if (residual.has_value())
+        TORCH_CHECK(residual->dim() == 2 && residual->size(0) == rows && residual->size(1) == n && residual->scalar_type() == at::kBFloat16 &&
+                        (residual->numel() == 0 || residual->stride(1) == 1),
+                    "linear_rows: residual must be bf16 [rows, N]");
+    if (out_packed.has_value()) TORCH_CHECK(packed_vec(*out_packed, 32 * n), "linear_rows: out_packed must be a contiguous bf16 tensor of 32 * N elements");
+    TORCH_CHECK(y.has_value() || out_packed.has_value(), "linear_rows: nothing to write");
+    tah_linear_rows_args a{};
+    a.w_packed = w_packed.data_ptr(); a.x_packed = x_packed.data_ptr();
+    a.residual = ptr(residual); a.residual_row_stride = residual.has_value() ? (rows > 1 ? residual->stride(0) : n) : 0;
+    a.out = y.has_value() ? mptr(*y) : nullptr; a.out_row_stride = y.has_value() ? (rows > 1 ? y->stride(0) : n) : 0;
+    a.out_packed = out_packed.has_value() ? out_packed->data_ptr() : nullptr;
+    a.rows = (int32_t)rows; a.n = (int32_t)n; a.k = (int32_t)k;
+    a.kind = gate_up ? TAH_LINEAR_GATE_UP : TAH_LINEAR_PLAIN;
+    a.input_norm = input_norm ? 1 : 0; a.norm_eps = (float)norm_eps;
+    check_rc(g.linear_rows(&a, d.stream()), "tah_linear_rows");
+    return y;
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -588,4 +662,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("rows_copy", &rows_copy);
     m.def("topk_mix", &topk_mix);
     m.def("silu_mul", &silu_mul);
+    m.def("linear_pack_weight", &linear_pack_weight);
+    m.def("linear_pack_rows", &linear_pack_rows);
+    m.def("linear_rows", &linear_rows);
 }

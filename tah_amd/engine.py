@@ -16,8 +16,10 @@ new token per sequence -- with
 * batched sampling and end-of-sequence handling on the device;
 * the whole step captured once in a HIP graph and replayed per token.
 
-The linear layers are torch GEMMs (rocBLAS / hipBLASLt); everything between them that touches the cache is
-this library's kernels.  What is kept from the reference's forward loop, with the place it comes from:
+The linear layers of a decode step (at most 32 rows against weights of megabytes) run on weights re-ordered once
+for streaming (``tah_linear_rows``: residual adds and the MLP's gate in their epilogues, rows handed from kernel to
+kernel in the operand order of the matrix instruction); prefill, batches above 32 rows and the output head use torch
+GEMMs (rocBLAS / hipBLASLt).  What is kept from the reference's forward loop, with the place it comes from:
 depth-0 logits are the running sum (``additive_logits_update``, tah_model.py:78-83); the decider sees the
 last hidden state (a two-layer MLP, hidden -> 512 -> 1, sigmoid, threshold -- the form the end-to-end
 workload names; the reference's ``MLPIterDecider`` is a larger network over several layers,
@@ -71,6 +73,7 @@ class Weights:
         self.dec_b2: torch.Tensor = None
         self.threshold: float = 0.5
         self.norms_folded = False
+        self.linear_packed = False
 
     def fold_norms(self) -> "Weights":
         """Multiplies the input-norm weights into the projections that follow them (``wqkv *= ln1``, ``wgu *= ln2``,
@@ -82,6 +85,27 @@ class Weights:
                 L["wqkv"].mul_(L["ln1"][None, :])
                 L["wgu"].mul_(L["ln2"][None, :])
             self.norms_folded = True
+        return self
+
+    def can_pack_linear(self) -> bool:
+        c = self.cfg
+        qkv, o = (c.hq + 2 * c.hkv) * c.head_dim, c.hq * c.head_dim
+        return (self.norms_folded and self.embed.dtype == torch.bfloat16 and c.hidden % 32 == 0 and o % 32 == 0 and qkv % 16 == 0
+                and c.intermediate % 32 == 0 and (c.intermediate % 24 == 0 or c.intermediate % 16 == 0))
+
+    def pack_linear(self) -> "Weights":
+        """A second copy of every layer's four weights in the order ``ops.linear_rows`` streams them (``wqkv_p``,
+        ``wo_p``, ``wgu_p``, ``wdown_p``), made once; needs the input norms folded in (``wgu`` carries ln2).  The
+        row-major weights stay for prefill."""
+        if not self.linear_packed:
+            if not self.can_pack_linear():
+                raise TahDuoError("pack_linear: needs folded input norms, bf16 and sizes in whole MFMA steps")
+            for L in self.layers:
+                L["wqkv_p"] = ops.linear_pack_weight(L["wqkv"])
+                L["wo_p"] = ops.linear_pack_weight(L["wo"])
+                L["wgu_p"] = ops.linear_pack_weight(L["wgu"], gate_up=True)
+                L["wdown_p"] = ops.linear_pack_weight(L["wdown"])
+            self.linear_packed = True
         return self
 
     @staticmethod
@@ -140,14 +164,20 @@ def rope_tables(max_len: int, head_dim: int, theta: float, device, dtype=torch.b
 
 class TaHDecodeEngine:
     def __init__(self, weights: Weights, batch: int, max_len: int, *, max_hard: Optional[int] = None, device="cuda",
-                 fold_norms: bool = True):
+                 fold_norms: bool = True, packed_linear: bool = True):
         """``fold_norms``: multiply the layers' input-norm weights into the projections behind them (in place in
-        ``weights``, once) so that the two RMSNorms of a layer cost no launch; needs hidden % 8 == 0 and bf16."""
+        ``weights``, once) so that the two RMSNorms of a layer cost no launch; needs hidden % 8 == 0 and bf16.
+        ``packed_linear``: run the linear layers of a decode step on ``ops.linear_rows`` (a second, re-ordered copy
+        of the layers' weights is made once); needs ``fold_norms``, at most 32 rows and sizes in whole MFMA steps,
+        otherwise the step keeps torch GEMMs."""
         cfg = weights.cfg
         if cfg.head_dim != 128:
             raise TahDuoError("the kernels are built for head_dim 128")
         if fold_norms and cfg.hidden % 8 == 0 and weights.embed.dtype == torch.bfloat16:
             weights.fold_norms()
+        self.packed_linear = bool(packed_linear and batch <= ops.LINEAR_MAX_ROWS and weights.can_pack_linear())
+        if self.packed_linear:
+            weights.pack_linear()
         self.w, self.cfg, self.B, self.max_len = weights, cfg, batch, max_len
         self.device = torch.device(device)
         self.max_hard = max_hard if max_hard is not None else max_len
@@ -175,6 +205,9 @@ class TaHDecodeEngine:
         self._graph = None
         self.static_scratch = self.device.type == "cuda"
         self.measure_without_attention = False
+        if self.packed_linear:  # rows operands handed from kernel to kernel (32 rows each; rows past the batch stay zero)
+            z = lambda n: torch.zeros(32 * n, dtype=torch.bfloat16, device=dev)
+            self.xp, self.op, self.actp = z(cfg.hidden), z(cfg.hq * cfg.head_dim), z(cfg.intermediate)
 
     # ── model pieces ─────────────────────────────────────────────────────
     def _rms(self, x, w):
@@ -219,6 +252,8 @@ class TaHDecodeEngine:
         attends with q_pos / q_depth per row (q_pos < 0: the row sees nothing and is dropped by the caller)."""
         c = self.cfg
         cos, sin = rope if rope is not None else self._rope_rows(pos)
+        if self.packed_linear:
+            return self._pass_single_packed(x, pos, depth, slot_of, q_pos, q_depth, cos, sin)
         folded = self.w.norms_folded
         for l, L in enumerate(self.w.layers):
             qkv = (x if folded else self._rms(x, L["ln1"])) @ L["wqkv"].t()
@@ -234,6 +269,31 @@ class TaHDecodeEngine:
                             static_scratch=self.static_scratch)
             x = x.addmm_(o.view(x.shape[0], c.hq * c.head_dim), L["wo"].t())  # residual add inside the GEMM, in place
             x = self._mlp(x, L)
+        return self._rms(x, self.w.norm)
+
+    def _pass_single_packed(self, x, pos, depth: int, slot_of, q_pos, q_depth, cos, sin):
+        """The same pass with the four linear layers of a layer on ``ops.linear_rows``: seven launches per layer.  The
+        hidden state lives twice, row-major in ``x`` (updated in place; read by the q/k preparation for the norm
+        factor) and as rows operand in ``self.xp``; attention output and MLP activation exist as rows operands only."""
+        c = self.cfg
+        B, H, I = x.shape[0], c.hidden, c.intermediate
+        n_qkv, n_o = (c.hq + 2 * c.hkv) * c.head_dim, c.hq * c.head_dim
+        x = x.contiguous()
+        xp = ops.linear_pack_rows(x, out=self.xp)
+        for l, L in enumerate(self.w.layers):
+            q, k, v = self._split_qkv(ops.linear_rows(L["wqkv_p"], xp, B, n_qkv, H))
+            cache = self.slabs0[l] if depth == 0 else self.slabs1[l]
+            if self.measure_without_attention:  # timing aid: the step minus its q/k preparation and decode kernels
+                ops.linear_pack_rows(q.reshape(B, n_o), out=self.op)
+            else:
+                qo, _ = qk_norm_rope(q, k, L["qn"], L["kn"], cos, sin, c.rms_eps, v=v, cache=cache, cu_new=self.cu_rows,
+                                     slot_of=slot_of, pos_new=pos if depth == 1 else None, one_row_per_seq=True,
+                                     norm_input=x, norm_eps=c.rms_eps)
+                _decode(qo, self.rows, q_pos, self.slabs0[l], self.slabs1[l], scale=self.scale, q_depth=q_depth,
+                        static_scratch=self.static_scratch, out_packed=self.op)
+            ops.linear_rows(L["wo_p"], self.op, B, H, n_o, residual=x, out=x, out_packed=xp)
+            ops.linear_rows(L["wgu_p"], xp, B, I, H, gate_up=True, out_packed=self.actp, want_out=False, norm_eps=c.rms_eps)
+            ops.linear_rows(L["wdown_p"], self.actp, B, H, I, residual=x, out=x, out_packed=xp)
         return self._rms(x, self.w.norm)
 
     def step_logits(self, tok: torch.Tensor, force_hard: Optional[torch.Tensor] = None, active: Optional[torch.Tensor] = None):

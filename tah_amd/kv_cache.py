@@ -88,7 +88,8 @@ _WORKSPACES = {}
 
 def decode(q: torch.Tensor, q_slot: torch.Tensor, q_pos: torch.Tensor, c1: KvSlabs, c2: Optional[KvSlabs], *,
            scale: float, depth: int = 0, q_depth: Optional[torch.Tensor] = None, return_lse: bool = False,
-           out: Optional[torch.Tensor] = None, lse_out: Optional[torch.Tensor] = None, static_scratch: bool = False):
+           out: Optional[torch.Tensor] = None, lse_out: Optional[torch.Tensor] = None, static_scratch: bool = False,
+           out_packed: Optional[torch.Tensor] = None):
     """One decode step: q [nq, Hq, D] bf16, one row per (sequence, depth) being decoded.
 
     Row i belongs to cache slot q_slot[i], sits at position q_pos[i], and sees the
@@ -97,7 +98,8 @@ def decode(q: torch.Tensor, q_slot: torch.Tensor, q_pos: torch.Tensor, c1: KvSla
     ``out`` / ``lse_out`` take the results when given.  ``static_scratch=True`` calls
     ``tah_duo_decode_static``: the split-K partials go to the buffer the library holds on the GPU, so with
     ``out`` given the call allocates nothing (callers under graph capture); requests beyond
-    ``_capi.STATIC_SCRATCH_BYTES`` raise.
+    ``_capi.STATIC_SCRATCH_BYTES`` raise.  ``out_packed`` (bf16 [32 * Hq * D], nq <= 32) also receives the output as the
+    rows operand of ``ops.linear_rows`` for the o projection (rows nq .. 31 are not touched).
     """
     if q.dim() != 3:
         raise _capi.TahDuoError("decode: q must be [nq, Hq, D]")
@@ -118,5 +120,6 @@ def decode(q: torch.Tensor, q_slot: torch.Tensor, q_pos: torch.Tensor, c1: KvSla
             ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=q.device)
             _WORKSPACES[key] = ws
     two = (c2.k, c2.v, c2.pos, c2.start, c2.len) if need2 else (None,) * 5
-    _call("duo_decode", q, o, lse, q_slot, q_pos, q_depth, int(depth), c1.k, c1.v, c1.start, c1.len, *two, ws, float(scale))
+    _call("duo_decode", q, o, lse, q_slot, q_pos, q_depth, int(depth), c1.k, c1.v, c1.start, c1.len, *two, ws, float(scale),
+          out_packed)
     return (o, lse) if return_lse else o

@@ -113,6 +113,36 @@ def silu_mul(gate_up: torch.Tensor, norm_input: Optional[torch.Tensor] = None, n
     return _call("silu_mul", gate_up, norm_input, float(norm_eps))
 
 
+LINEAR_MAX_ROWS = 32
+
+
+def linear_pack_weight(w: torch.Tensor, gate_up: bool = False) -> torch.Tensor:
+    """A linear layer's weight, bf16 [N, K] (``gate_up``: [2N, K], gate rows then up rows), in the order
+    ``linear_rows`` streams it (``tah_linear_pack_weight``): flat bf16 of the same number of elements.  Done once per
+    weight.  K % 32 == 0, N % 16 == 0 (gate|up: N % 24 == 0 or N % 16 == 0)."""
+    return _call("linear_pack_weight", w, bool(gate_up))
+
+
+def linear_pack_rows(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Rows of a decode step, bf16 [rows <= 32, K], as the rows operand of ``linear_rows``: flat bf16 [32 * K], rows
+    past the last one zero (``tah_linear_pack_rows``)."""
+    return _call("linear_pack_rows", x, out)
+
+
+def linear_rows(w_packed: torch.Tensor, x_packed: torch.Tensor, rows: int, n: int, k: int, *, gate_up: bool = False,
+                residual: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+                out_packed: Optional[torch.Tensor] = None, want_out: bool = True, norm_eps: Optional[float] = None):
+    """A linear layer of a decode step on packed operands (``tah_linear_rows``), bf16, rows <= 32.
+
+    ``x @ w.T`` [rows, N], plus ``residual`` [rows, N] when given (``out=residual`` updates it in place); with
+    ``gate_up``, ``silu(x @ gate.T) * (x @ up.T)``, and with ``norm_eps`` gate and up are first multiplied by the row's
+    ``rsqrt(mean(x**2) + norm_eps)`` (the MLP's input RMSNorm whose weight sits in w).  ``out_packed`` [32 * N] also
+    receives the result as the next layer's rows operand; ``want_out=False`` with ``out_packed`` writes only that.
+    Returns the row-major result (None when it was not asked for)."""
+    return _call("linear_rows", w_packed, x_packed, int(rows), int(n), int(k), bool(gate_up), residual, out, out_packed,
+                 bool(want_out), norm_eps is not None, float(norm_eps or 0.0))
+
+
 def greedy_step(logits0, logits1, hard, eos: int, tok, finished, pos, out_tokens, step_idx, out_len, n_hard, n_steps) -> None:
     """One greedy generation step after the logits (``tah_greedy_step``), all updates in place on the device.
 

@@ -39,8 +39,13 @@ def test_decode_and_append_on_cpu_shim(hq, hkv, lens):
         o1, l1 = kv_cache.decode(c["q2"], hr, qpos[hr.long()], s1, s2, scale=c["scale"], depth=1, return_lse=True)
         # both depths in one launch
         qd = torch.tensor([0] * nseq + [1] * len(hr), dtype=torch.int32)
+        packed = torch.full((32 * hq * 128,), 3.0, dtype=torch.bfloat16)
         om = kv_cache.decode(torch.cat([c["q1"], c["q2"]]), torch.cat([slot, hr]), torch.cat([qpos, qpos[hr.long()]]),
-                             s1, s2, scale=c["scale"], q_depth=qd)
+                             s1, s2, scale=c["scale"], q_depth=qd, out_packed=packed)
+    # the same output as the rows operand of the o projection; rows past the last query are left alone
+    from tests.test_linear_rows import unpack_rows
+    rows = unpack_rows(packed, hq * 128)
+    assert torch.equal(rows[:om.shape[0]], om.reshape(om.shape[0], -1)) and (rows[om.shape[0]:] == 3.0).all()
     w0, wl0, w1, wl1 = oracle_decode(c)
     np.testing.assert_allclose(o0.float().numpy(), w0, atol=2e-2, rtol=2e-2)
     np.testing.assert_allclose(l0.numpy(), wl0, atol=2e-3, rtol=1e-3)

@@ -34,8 +34,14 @@ def run_decode(c, cap1, cap2, fused):
     q1, q2 = c["q1"].cuda(), c["q2"].cuda()
     if fused:
         qd = torch.tensor([0] * nseq + [1] * len(hr), dtype=torch.int32, device="cuda")
+        nq = nseq + len(hr)  # up to 32 queries the output is also written as the o projection's rows operand
+        packed = torch.zeros(32 * q1.shape[1] * q1.shape[2], dtype=torch.bfloat16, device="cuda") if nq <= 32 else None
         o, lse = kv_cache.decode(torch.cat([q1, q2]), torch.cat([slot, hr]), torch.cat([qpos, qpos[hr.long()]]), s1, s2,
-                                 scale=c["scale"], q_depth=qd, return_lse=True)
+                                 scale=c["scale"], q_depth=qd, return_lse=True, out_packed=packed)
+        if packed is not None:
+            from tests.test_linear_rows import unpack_rows
+            rows = unpack_rows(packed.cpu(), q1.shape[1] * q1.shape[2])
+            assert torch.equal(rows[:nq], o.cpu().reshape(nq, -1)) and not rows[nq:].any()
         out = o[:nseq], lse[:nseq], o[nseq:], lse[nseq:]
     else:
         o0, l0 = kv_cache.decode(q1, slot, qpos, s1, None, scale=c["scale"], depth=0, return_lse=True)
