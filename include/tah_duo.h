@@ -357,10 +357,10 @@ typedef struct tah_linear_rows_args {
                                * is needed */
     int64_t residual_row_stride, out_row_stride; /* elements */
     int32_t rows, n, k;       /* rows <= 32 */
-    int32_t kind;             /* TAH_LINEAR_PLAIN: out = x W^T [+ residual]
+    int32_t kind;             /* TAH_LINEAR_PLAIN: out = bf16(r x W^T) [+ residual]
                                * TAH_LINEAR_GATE_UP: out = bf16(silu(g)) * u, g = bf16(r x Wg^T), u = bf16(r x Wu^T) */
-    int32_t input_norm;       /* TAH_LINEAR_GATE_UP: r = rsqrt(mean(x[row]^2) + norm_eps), the MLP's input RMSNorm whose
-                               * weight is already inside W (0: r = 1) */
+    int32_t input_norm;       /* 1: r = rsqrt(mean(x[row]^2) + norm_eps), an RMSNorm of the rows whose weight is already
+                               * inside W (the MLP's input norm for gate|up, the final norm for an output head); 0: r = 1 */
     float norm_eps;
 } tah_linear_rows_args;
 int tah_linear_rows(const tah_linear_rows_args* args, tah_stream_t stream);

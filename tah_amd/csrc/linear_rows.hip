@@ -38,7 +38,7 @@ constexpr int kTileCols = 16;   // output columns of one weight tile
 constexpr int kStepK = 32;      // k of one MFMA step; a tile step is 16 x 32 bf16 = 1 KiB
 constexpr int kGroup24 = 24;    // gate|up: output columns per workgroup when n % 24 == 0 (256 workgroups for n = 6144)
 
-enum Epi { kPlain = 0, kGateUp16 = 2, kGateUp24 = 3 };
+enum Epi { kPlain = 0, kPlainNorm = 1, kGateUp16 = 2, kGateUp24 = 3 };  // kPlainNorm: plain with the rows' norm factor
 
 struct LinParams {
     const bf16x8* w;   // packed weight
@@ -50,6 +50,7 @@ struct LinParams {
     int32_t rows, n, k;
     float eps;
     int32_t norm;
+    int32_t groups;  // column groups (workgroups per row half)
 };
 
 __device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
@@ -62,13 +63,27 @@ __device__ __host__ __forceinline__ int64_t packed_rows_unit(int r, int k) {
 __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + fast_exp2(-x * kLog2e)); }
 
 // NC: weight tiles per workgroup (1 plain, 2 or 3 for gate|up).  CH: steps per chunk of loads.  PW: steps per wave
-// when K is known at compile time (K = 32 * 8 * PW), 0: any K % 32 == 0.
-template <int NC, int CH, int EPI, int PW>
+// when K is known at compile time (K = 32 * 8 * PW), 0: any K % 32 == 0.  NH: row halves per workgroup -- 2: all 32
+// rows; 1: sixteen rows, the grid holds a workgroup per (column group, half) (or only the first half when there
+// are at most 16 rows).  A layer with few column groups (n = 2048: 128) then fills the chip, and every compute
+// unit pulls half of the rows' operand; the second reader of a weight tile is placed on the same XCD, whose L2 has
+// it or is fetching it.
+template <int NC, int CH, int EPI, int PW, int NH>
 __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(const LinParams p) {
-    __shared__ __align__(16) float red[kLinWaves][NC][kLinRows][kTileCols];
-    __shared__ float ssq[kLinWaves][kLinRows];
+    __shared__ __align__(16) float red[kLinWaves][NC][16 * NH][kTileCols];
+    __shared__ float ssq[kLinWaves][16 * NH];
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const int c = lane % 16, kg = lane / 16;
+    int group = blockIdx.x, half = 0;
+    if (NH == 1 && (int)gridDim.x == 2 * p.groups) {
+        if (p.groups % 8 == 0) {  // workgroups go to the XCDs round robin: i and i + 8 share one
+            group = (blockIdx.x / 16) * 8 + blockIdx.x % 8;
+            half = (blockIdx.x / 8) % 2;
+        } else {
+            group = blockIdx.x / 2;
+            half = blockIdx.x % 2;
+        }
+    }
     const int steps = p.k / kStepK;
     const int per_wave = PW > 0 ? PW : (steps + kLinWaves - 1) / kLinWaves;
     int nst = steps - wave * per_wave;
@@ -76,15 +91,17 @@ __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(const LinParam
     const int s0 = nst > 0 ? wave * per_wave : 0;  // a wave without steps still points at valid memory
     const bf16x8* wb[NC];
 #pragma unroll
-    for (int t = 0; t < NC; ++t) wb[t] = p.w + ((int64_t)(blockIdx.x * NC + t) * steps + s0) * 64 + lane;
-    const bf16x8* xb = p.x + (int64_t)s0 * 128 + lane;
+    for (int t = 0; t < NC; ++t) wb[t] = p.w + ((int64_t)(group * NC + t) * steps + s0) * 64 + lane;
+    const bf16x8* xb = p.x + (int64_t)s0 * 128 + 64 * half + lane;
 
     struct Buf {
-        bf16x8 w[CH][NC], x[CH][2];
+        bf16x8 w[CH][NC], x[CH][NH];
     };
-    f32x4 acc[NC][2];
+    f32x4 acc[NC][NH];
 #pragma unroll
-    for (int t = 0; t < NC; ++t) acc[t][0] = acc[t][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < NC; ++t)
+#pragma unroll
+        for (int h = 0; h < NH; ++h) acc[t][h] = f32x4{0.f, 0.f, 0.f, 0.f};
     float ss0 = 0.f, ss1 = 0.f;
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
     // Loads of chunk ch.  Without a compile-time K a step past the wave's share reads step 0 of the wave's range
@@ -97,14 +114,14 @@ __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(const LinParam
 #pragma unroll
             for (int t = 0; t < NC; ++t) b.w[s][t] = __builtin_nontemporal_load(wb[t] + sti * 64);
             b.x[s][0] = xb[sti * 128];
-            b.x[s][1] = xb[sti * 128 + 64];
+            if constexpr (NH == 2) b.x[s][1] = xb[sti * 128 + 64];
         }
     };
     auto multiply = [&](int ch, Buf& b) __attribute__((always_inline)) {
 #pragma unroll
         for (int s = 0; s < CH; ++s) {
             const bool ok = PW > 0 || ch * CH + s < nst;
-            const bf16x8 a0 = ok ? b.x[s][0] : zero8, a1 = ok ? b.x[s][1] : zero8;
+            const bf16x8 a0 = ok ? b.x[s][0] : zero8, a1 = ok ? b.x[s][NH - 1] : zero8;
             if constexpr (EPI != kPlain) {
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
@@ -116,7 +133,7 @@ __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(const LinParam
 #pragma unroll
             for (int t = 0; t < NC; ++t) {
                 acc[t][0] = mfma16(a0, b.w[s][t], acc[t][0]);
-                acc[t][1] = mfma16(a1, b.w[s][t], acc[t][1]);
+                if constexpr (NH == 2) acc[t][1] = mfma16(a1, b.w[s][t], acc[t][1]);
             }
         }
     };
@@ -154,7 +171,7 @@ __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(const LinParam
 #pragma unroll
     for (int t = 0; t < NC; ++t)
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
+        for (int h = 0; h < NH; ++h)
 #pragma unroll
             for (int r = 0; r < 4; ++r) red[wave][t][16 * h + 4 * kg + r][c] = acc[t][h][r];
     if constexpr (EPI != kPlain) {
@@ -165,17 +182,19 @@ __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(const LinParam
         ss1 += __shfl_xor(ss1, 32);
         if (kg == 0) {
             ssq[wave][c] = ss0;
-            ssq[wave][16 + c] = ss1;
+            if constexpr (NH == 2) ssq[wave][16 + c] = ss1;
         }
     }
     __syncthreads();
 
     // ---- epilogue: one thread per (row, 8 output columns) -------------------------------------------------
-    constexpr int kUnits = EPI == kGateUp24 ? 3 : 2;  // 8-column units of output per row and workgroup
-    if (threadIdx.x >= kLinRows * kUnits) return;
-    const int row = threadIdx.x / kUnits, unit = threadIdx.x % kUnits;
+    constexpr bool kGate = EPI == kGateUp16 || EPI == kGateUp24;
+    constexpr int kUnits = EPI == kGateUp24 ? 3 : (kGate ? 2 : 2 * NC);  // 8-column units of output per row and workgroup
+    if (threadIdx.x >= 16 * NH * kUnits) return;
+    const int lrow = threadIdx.x / kUnits, unit = threadIdx.x % kUnits;  // row inside the workgroup's rows
+    const int row = 16 * half + lrow;
     // where the unit's gate (or plain) and up sums sit: tile and first column inside it
-    int gt = 0, gc = 8 * unit, ut = 1, uc = 8 * unit;
+    int gt = kGate ? 0 : unit / 2, gc = kGate ? 8 * unit : 8 * (unit % 2), ut = 1, uc = 8 * unit;
     if constexpr (EPI == kGateUp24) {  // tiles: gate 0-15 | gate 16-23, up 16-23 | up 0-15
         gt = unit == 2 ? 1 : 0;
         gc = unit == 1 ? 8 : 0;
@@ -187,16 +206,16 @@ __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(const LinParam
     for (int i = 0; i < 8; ++i) sg[i] = su[i] = 0.f;
 #pragma unroll
     for (int w = 0; w < kLinWaves; ++w) {
-        const f32x4 lo = *reinterpret_cast<const f32x4*>(&red[w][gt][row][gc]);
-        const f32x4 hi = *reinterpret_cast<const f32x4*>(&red[w][gt][row][gc + 4]);
+        const f32x4 lo = *reinterpret_cast<const f32x4*>(&red[w][gt][lrow][gc]);
+        const f32x4 hi = *reinterpret_cast<const f32x4*>(&red[w][gt][lrow][gc + 4]);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             sg[i] += lo[i];
             sg[4 + i] += hi[i];
         }
-        if constexpr (EPI != kPlain) {
-            const f32x4 ulo = *reinterpret_cast<const f32x4*>(&red[w][ut][row][uc]);
-            const f32x4 uhi = *reinterpret_cast<const f32x4*>(&red[w][ut][row][uc + 4]);
+        if constexpr (kGate) {
+            const f32x4 ulo = *reinterpret_cast<const f32x4*>(&red[w][ut][lrow][uc]);
+            const f32x4 uhi = *reinterpret_cast<const f32x4*>(&red[w][ut][lrow][uc + 4]);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 su[i] += ulo[i];
@@ -204,18 +223,20 @@ __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(const LinParam
             }
         }
     }
-    const int n0 = blockIdx.x * (EPI == kGateUp24 ? kGroup24 : kTileCols) + 8 * unit;
+    const int n0 = group * (EPI == kGateUp24 ? kGroup24 : (kGate ? kTileCols : NC * kTileCols)) + 8 * unit;
     const bool live = row < p.rows;
     bf16x8 out = zero8;
     if (live) {
+        float rin = 1.0f;
         if constexpr (EPI != kPlain) {
-            float rin = 1.0f;
             if (p.norm) {
                 float ss = 0.f;
 #pragma unroll
-                for (int w = 0; w < kLinWaves; ++w) ss += ssq[w][row];
+                for (int w = 0; w < kLinWaves; ++w) ss += ssq[w][lrow];
                 rin = __builtin_amdgcn_rsqf(ss / (float)p.k + p.eps);
             }
+        }
+        if constexpr (kGate) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 // the projections' own rounding to bf16, the activation's, the product's (Qwen3MLP.forward)
@@ -225,14 +246,17 @@ __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(const LinParam
         } else if (p.res) {
             const bf16x8 rv = *reinterpret_cast<const bf16x8*>(p.res + (int64_t)row * p.res_rs + n0);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) out[i] = (__bf16)((float)(__bf16)sg[i] + (float)rv[i]);
+            for (int i = 0; i < 8; ++i) out[i] = (__bf16)((float)(__bf16)(sg[i] * rin) + (float)rv[i]);
         } else {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) out[i] = (__bf16)sg[i];
+            for (int i = 0; i < 8; ++i) out[i] = (__bf16)(sg[i] * rin);
         }
         if (p.y) *reinterpret_cast<bf16x8*>(p.y + (int64_t)row * p.y_rs + n0) = out;
     }
-    if (p.yp) p.yp[packed_rows_unit(row, n0)] = out;  // rows past the last one stay zero for the next layer
+    if (p.yp) {
+        p.yp[packed_rows_unit(row, n0)] = out;  // rows past the last one stay zero for the next layer
+        if (NH == 1 && (int)gridDim.x == p.groups) p.yp[packed_rows_unit(16 + lrow, n0)] = zero8;  // nobody computes the second half
+    }
 }
 
 // ---- re-ordering -----------------------------------------------------------------------------------------
@@ -272,9 +296,20 @@ __global__ __launch_bounds__(256) void pack_rows_kernel(const __bf16* x, int64_t
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
+// Sixteen rows per workgroup when there are no more, or when the column groups alone would leave half of the
+// 256 compute units idle.
+constexpr int kSplitRowsBelowGroups = 129;
+constexpr int kWideFromCols = 16384;  // plain layers from this many output columns on take 32 columns per workgroup
+
 template <int NC, int CH, int EPI, int PW>
-void launch(const LinParams& p, int groups, hipStream_t st) {
-    hipLaunchKernelGGL((linear_rows_kernel<NC, CH, EPI, PW>), dim3(groups), dim3(kLinThreads), 0, st, p);
+void launch(LinParams& p, int groups, hipStream_t st) {
+    p.groups = groups;
+    if (p.rows <= 16)
+        hipLaunchKernelGGL((linear_rows_kernel<NC, CH, EPI, PW, 1>), dim3(groups), dim3(kLinThreads), 0, st, p);
+    else if (groups < kSplitRowsBelowGroups)
+        hipLaunchKernelGGL((linear_rows_kernel<NC, CH, EPI, PW, 1>), dim3(2 * groups), dim3(kLinThreads), 0, st, p);
+    else
+        hipLaunchKernelGGL((linear_rows_kernel<NC, CH, EPI, PW, 2>), dim3(groups), dim3(kLinThreads), 0, st, p);
 }
 
 }  // namespace
@@ -341,9 +376,22 @@ extern "C" int tah_linear_rows(const tah_linear_rows_args* a, tah_stream_t strea
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int steps = a->k / kStepK;
     const int pw = steps % kLinWaves == 0 ? steps / kLinWaves : 0;  // compile-time K for the sizes of the end-to-end model
-    if (!gate_up) {
+    if (!gate_up && a->n >= kWideFromCols && a->n % (2 * kTileCols) == 0) {
+        // an output head: two tiles per workgroup, the rows' operand is read half as often
+        const int groups = a->n / (2 * kTileCols);
+        if (p.norm) {
+            if (pw == 8) launch<2, 4, kPlainNorm, 8>(p, groups, st);
+            else launch<2, 2, kPlainNorm, 0>(p, groups, st);
+        } else {
+            if (pw == 8) launch<2, 4, kPlain, 8>(p, groups, st);
+            else launch<2, 2, kPlain, 0>(p, groups, st);
+        }
+    } else if (!gate_up) {
         const int groups = a->n / kTileCols;
-        if (pw == 8) launch<1, 8, kPlain, 8>(p, groups, st);
+        if (p.norm) {
+            if (pw == 8) launch<1, 8, kPlainNorm, 8>(p, groups, st);
+            else launch<1, 4, kPlainNorm, 0>(p, groups, st);
+        } else if (pw == 8) launch<1, 8, kPlain, 8>(p, groups, st);
         else if (pw == 24) launch<1, 8, kPlain, 24>(p, groups, st);
         else launch<1, 4, kPlain, 0>(p, groups, st);
     } else if (g24) {

@@ -74,6 +74,7 @@ class Weights:
         self.threshold: float = 0.5
         self.norms_folded = False
         self.linear_packed = False
+        self.lm_head_p: Optional[torch.Tensor] = None
 
     def fold_norms(self) -> "Weights":
         """Multiplies the input-norm weights into the projections that follow them (``wqkv *= ln1``, ``wgu *= ln2``,
@@ -105,6 +106,8 @@ class Weights:
                 L["wo_p"] = ops.linear_pack_weight(L["wo"])
                 L["wgu_p"] = ops.linear_pack_weight(L["wgu"], gate_up=True)
                 L["wdown_p"] = ops.linear_pack_weight(L["wdown"])
+            # the output head with the final norm's weight inside (a copy: the head may be the embedding itself)
+            self.lm_head_p = ops.linear_pack_weight(self.lm_head * self.norm[None, :]) if self.cfg.vocab % 16 == 0 else None
             self.linear_packed = True
         return self
 
@@ -249,7 +252,9 @@ class TaHDecodeEngine:
 
     def _pass_single(self, x, pos, depth: int, slot_of, q_pos, q_depth, rope=None):
         """x [B, H]; appends this token's K/V to the depth's slabs (rows with slot_of < 0 are not cached) and
-        attends with q_pos / q_depth per row (q_pos < 0: the row sees nothing and is dropped by the caller)."""
+        attends with q_pos / q_depth per row (q_pos < 0: the row sees nothing and is dropped by the caller).  Returns
+        the final-normed hidden state (with packed linear layers: the hidden state before the final norm, see
+        ``_head``)."""
         c = self.cfg
         cos, sin = rope if rope is not None else self._rope_rows(pos)
         if self.packed_linear:
@@ -294,7 +299,18 @@ class TaHDecodeEngine:
             ops.linear_rows(L["wo_p"], self.op, B, H, n_o, residual=x, out=x, out_packed=xp)
             ops.linear_rows(L["wgu_p"], xp, B, I, H, gate_up=True, out_packed=self.actp, want_out=False, norm_eps=c.rms_eps)
             ops.linear_rows(L["wdown_p"], self.actp, B, H, I, residual=x, out=x, out_packed=xp)
-        return self._rms(x, self.w.norm)
+        return x  # before the final norm; self.xp holds the same rows as operand
+
+    def _head(self, h):
+        """Logits [B, V] of what a pass returned: the final-normed rows through the head, or, with packed linear
+        layers, the rows operand the last layer left in ``self.xp`` through the head that carries the final norm's
+        weight, the norm's factor applied to the products."""
+        c = self.cfg
+        if not self.packed_linear:
+            return h @ self.w.lm_head.t()
+        if self.w.lm_head_p is None:
+            return self._rms(h, self.w.norm) @ self.w.lm_head.t()
+        return ops.linear_rows(self.w.lm_head_p, self.xp, h.shape[0], c.vocab, c.hidden, norm_eps=c.rms_eps)
 
     def step_logits(self, tok: torch.Tensor, force_hard: Optional[torch.Tensor] = None, active: Optional[torch.Tensor] = None):
         """The iteration loop of tah_model.py:580-706 for one new token per sequence, on ``self.pos``.
@@ -317,7 +333,9 @@ class TaHDecodeEngine:
         qpos0 = torch.where(act, pos, self.minus1)
         rope = self._rope_rows(pos)  # both latent iterations of a token use its position
         h0 = self._pass_single(self.w.embed[tok], pos, 0, slot0, qpos0, self.zeros_i, rope)
-        l0 = h0 @ self.w.lm_head.t()
+        l0 = self._head(h0)
+        if self.packed_linear:
+            h0 = self._rms(h0, self.w.norm)
         hard = (self.decide(h0) > self.w.threshold) if force_hard is None else force_hard
         hard = hard & act
         # next-iteration input of the hard rows (tah_model.py:693-697); the other rows keep zeros
@@ -325,7 +343,7 @@ class TaHDecodeEngine:
         slot1 = torch.where(hard, self.rows, self.minus1)
         qpos1 = torch.where(hard, pos, self.minus1)
         h1 = self._pass_single(x1, pos, 1, slot1, qpos1, hard.to(torch.int32), rope)
-        return l0, h1 @ self.w.lm_head.t(), hard
+        return l0, self._head(h1), hard
 
     # ── prefill: packed prompts, both depths, through the varlen kernels ──
     @torch.no_grad()

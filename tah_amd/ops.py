@@ -135,8 +135,9 @@ def linear_rows(w_packed: torch.Tensor, x_packed: torch.Tensor, rows: int, n: in
     """A linear layer of a decode step on packed operands (``tah_linear_rows``), bf16, rows <= 32.
 
     ``x @ w.T`` [rows, N], plus ``residual`` [rows, N] when given (``out=residual`` updates it in place); with
-    ``gate_up``, ``silu(x @ gate.T) * (x @ up.T)``, and with ``norm_eps`` gate and up are first multiplied by the row's
-    ``rsqrt(mean(x**2) + norm_eps)`` (the MLP's input RMSNorm whose weight sits in w).  ``out_packed`` [32 * N] also
+    ``gate_up``, ``silu(x @ gate.T) * (x @ up.T)``.  With ``norm_eps`` the products are first multiplied by the row's
+    ``rsqrt(mean(x**2) + norm_eps)``: an RMSNorm of the rows whose weight sits in w (the MLP's input norm for gate|up,
+    the final norm for an output head).  ``out_packed`` [32 * N] also
     receives the result as the next layer's rows operand; ``want_out=False`` with ``out_packed`` writes only that.
     Returns the row-major result (None when it was not asked for)."""
     return _call("linear_rows", w_packed, x_packed, int(rows), int(n), int(k), bool(gate_up), residual, out, out_packed,

@@ -64,11 +64,11 @@ def unpack_rows(packed, k):
 def reference(x, w, *, residual=None, gate_up=False, norm_eps=None):
     """float64 sums with the eager modules' bf16 roundings."""
     xd, wd = x.double(), w.double()
+    r = torch.rsqrt((xd ** 2).mean(-1, keepdim=True) + norm_eps) if norm_eps is not None else 1.0
     if not gate_up:
-        y = (xd @ wd.t()).to(BF)
+        y = (r * (xd @ wd.t())).to(BF)
         return y if residual is None else (y.double() + residual.double()).to(BF)
     n = w.shape[0] // 2
-    r = torch.rsqrt((xd ** 2).mean(-1, keepdim=True) + norm_eps) if norm_eps is not None else 1.0
     g = (r * (xd @ wd[:n].t())).to(BF).double()
     u = (r * (xd @ wd[n:].t())).to(BF).double()
     act = (g / (1.0 + torch.exp(-g))).to(BF).double()
@@ -109,6 +109,11 @@ CASES = [
     (9, 32, 2048, "gate_up_norm"),    # 16-column groups
     (32, 24, 320, "gate_up"),         # 24-column groups, any K, no norm
     (5, 16, 96, "gate_up_norm"),      # 16-column groups, any K
+    # more than 128 column groups: a workgroup takes all 32 rows (below, and up to 16 rows, it takes 16)
+    (20, 2080, 96, "residual"),
+    (32, 3120, 64, "gate_up_norm"),
+    (9, 48, 2048, "plain_norm"),      # an RMSNorm of the rows folded in (an output head behind the final norm)
+    (32, 32, 160, "plain_norm"),
 ]
 
 
@@ -118,7 +123,7 @@ def _linear_case(dev, rows, n, k, kind, seed=0):
     x = _rand((rows, k), 11 + seed, 1.5)
     w = _rand(((2 if gu else 1) * n, k), 12 + seed, k ** -0.5)
     res = _rand((rows, n), 13 + seed) if kind == "residual" else None
-    eps = 1e-6 if kind == "gate_up_norm" else None
+    eps = 1e-6 if kind.endswith("_norm") else None
     want = reference(x, w, residual=res, gate_up=gu, norm_eps=eps)
     wp = ops.linear_pack_weight(w.to(dev), gate_up=gu)
     xp = ops.linear_pack_rows(x.to(dev))
@@ -217,6 +222,7 @@ def test_packed_orders_gpu():
 @pytest.mark.parametrize("rows,n,k,kind", CASES + [
     (32, 4096, 2048, "plain"), (32, 2048, 2048, "residual"), (32, 6144, 2048, "gate_up_norm"), (32, 2048, 6144, "residual"),
     (13, 1024, 3072, "residual"), (32, 2560, 2560, "plain"), (32, 1600, 1024, "gate_up_norm"),
+    (32, 151936, 2048, "plain_norm"), (32, 16384, 512, "plain"), (20, 32000, 1024, "plain_norm"),   # output heads: 32 columns per workgroup
 ])
 def test_linear_rows_gpu(rows, n, k, kind):
     _linear_case("cuda", rows, n, k, kind, seed=n % 7)
