@@ -12,6 +12,8 @@
 // (Merging in the workgroup that finishes last would need device-scope fences,
 // which cost an L2 write-back per item across the eight XCDs; a persistent grid
 // striding over the items balanced worse than the hardware dispatcher.)
+// A call whose (query, kv head) pairs alone fill the chip, with slabs of at most 4096 rows, skips all that: one
+// workgroup per pair walks both segments and writes the finished output (duo_decode_whole_kernel).
 #include <hip/hip_runtime.h>
 
 #include <mutex>
@@ -63,6 +65,7 @@ struct DecParams {
     float* ws;
     int32_t nq, hq, hkv, nchunk1, nchunk2;
     int32_t chunk;  // rows per workgroup (kChunk or kChunkSmall)
+    int32_t whole;  // one workgroup per (query, kv head) over all rows, no partials (duo_decode_whole_kernel)
     float scale_log2e;
 };
 
@@ -70,6 +73,17 @@ struct DecParams {
 __host__ __device__ inline int chunk_rows(int nq, int hq, int capacity1) {
     const long big = (long)nq * hq * ((capacity1 + kChunk - 1) / kChunk);  // (query, head, chunk) triples at the large size
     return big < 4096 ? kChunkSmall : kChunk;
+}
+
+// One workgroup per (query, kv head) instead of split-K: when those pairs alone give every compute unit a workgroup
+// and no context can be long enough for their spread to matter.
+#ifndef TAH_DEC_WHOLE_MIN_PAIRS
+#define TAH_DEC_WHOLE_MIN_PAIRS 256  // the CPU execution build of the tests lowers it: 256 workgroups of 1024 threads are slow there
+#endif
+constexpr int kWholeMinPairs = TAH_DEC_WHOLE_MIN_PAIRS, kWholeMaxCapacity = 4096;
+constexpr int kWholeMaxGroup = 4;  // eight query heads per kv head do not fit the 128 registers of a 1024-thread workgroup
+inline bool whole_sequence(int nq, int hq, int hkv, int capacity1) {
+    return (long)nq * hkv >= kWholeMinPairs && capacity1 <= kWholeMaxCapacity && hq / hkv <= kWholeMaxGroup;
 }
 
 template <int CTRL>
@@ -101,6 +115,104 @@ __device__ __forceinline__ int visible_len(const DecParams& p, bool second, int 
         return qpos + 1 < n ? (qpos + 1 > 0 ? qpos + 1 : 0) : n;
     }
     return qdepth >= 1 ? p.c2.len[slot] : 0;
+}
+
+// Sixteen-lane groups of a wave each take one cache row per load (4 rows x 256 B = 1 KiB per instruction); U such
+// loads of K and of V are in flight per wave.  Scores, online softmax and the weighted sum of V for the 4 U rows
+// from r_it on (rows at or past row_end are masked; their loads are clamped into the slab), for the G query heads of
+// the kv head at once.  m / l / acc: running maximum (log2 domain), sum and un-normalised output of this lane's row
+// group, 8 values of d per lane.
+template <int G, int U>
+__device__ __forceinline__ void consume_rows(const Seg& sg, bool second, const __bf16* kbase, const __bf16* vbase, const int32_t* posbase,
+                                             int r_it, int row_end, int kq, int qpos, float scale_log2e, const u32x4 (&qv)[G],
+                                             float (&m_run)[G], float (&l_run)[G], float (&acc)[G][8]) {
+    u32x4 kreg[U], vreg[U];
+    int kpos[U];
+    bool ok[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int r = r_it + u * 4 + kq;
+        ok[u] = r < row_end;
+        const int rl = ok[u] ? r : row_end - 1;  // keep tail loads inside the slab
+#if TAH_DEC_NT
+        kreg[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kbase + (int64_t)rl * sg.k_rs));
+        vreg[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vbase + (int64_t)rl * sg.v_rs));
+#else
+        kreg[u] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)rl * sg.k_rs);
+        vreg[u] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)rl * sg.v_rs);
+#endif
+        kpos[u] = second ? posbase[rl] : 0;
+    }
+    float s[U][G];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const bool vis = ok[u] && (!second || kpos[u] <= qpos);
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            float d = 0.f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) d = dot2_acc(kreg[u][i], qv[g][i], d);
+            d = row16_sum(d) * scale_log2e;
+            s[u][g] = vis ? d : kNegInf;
+        }
+    }
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        float mx = m_run[g];
+#pragma unroll
+        for (int u = 0; u < U; ++u) mx = fmaxf(mx, s[u][g]);
+        const float m_use = mx == kNegInf ? 0.f : mx;
+        const float alpha = fast_exp2(m_run[g] - m_use);
+        m_run[g] = mx;
+        float pr[U], psum = 0.f;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            pr[u] = fast_exp2(s[u][g] - m_use);
+            psum += pr[u];
+        }
+        l_run[g] = l_run[g] * alpha + psum;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[g][i] *= alpha;
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc[g][2 * i] += pr[u] * bf16_lo(vreg[u][i]);
+                acc[g][2 * i + 1] += pr[u] * bf16_hi(vreg[u][i]);
+            }
+    }
+}
+
+// The 16 (wave, row group) partials of a workgroup into LDS: red[16][G][kPart].
+template <int G>
+__device__ __forceinline__ void park_partials(float (*red)[G][kPart], int grp, int dc, const float (&m_run)[G], const float (&l_run)[G],
+                                              const float (&acc)[G][8]) {
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) red[grp][g][dc * 8 + i] = acc[g][i];
+        if (dc == 0) {
+            red[grp][g][kD] = m_run[g];
+            red[grp][g][kD + 1] = l_run[g];
+        }
+    }
+}
+
+// Element d of head g merged over the 16 partials: un-normalised output, sum, maximum.
+template <int G>
+__device__ __forceinline__ void merge16(float (*red)[G][kPart], int g, int d, float& a, float& l, float& mx) {
+    mx = kNegInf;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) mx = fmaxf(mx, red[j][g][kD]);
+    const float m_use = mx == kNegInf ? 0.f : mx;
+    a = 0.f;
+    l = 0.f;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const float w = fast_exp2(red[j][g][kD] - m_use);
+        a += w * red[j][g][d];
+        l += w * red[j][g][kD + 1];
+    }
 }
 
 template <int G, int CH>
@@ -148,88 +260,16 @@ __global__ __launch_bounds__(kDecThreads) void duo_decode_split_kernel(const Dec
         for (int it = 0; it < kRowsPerWave / (4 * kUnroll); ++it) {
             const int r_it = wrow0 + it * 4 * kUnroll;
             if (r_it >= row_end) break;  // uniform per wave
-            u32x4 kreg[kUnroll], vreg[kUnroll];
-            int kpos[kUnroll];
-            bool ok[kUnroll];
-#pragma unroll
-            for (int u = 0; u < kUnroll; ++u) {
-                const int r = r_it + u * 4 + kq;
-                ok[u] = r < row_end;
-                const int rl = ok[u] ? r : row_end - 1;  // keep tail loads inside the slab
-#if TAH_DEC_NT
-                kreg[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kbase + (int64_t)rl * sg.k_rs));
-                vreg[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vbase + (int64_t)rl * sg.v_rs));
-#else
-                kreg[u] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)rl * sg.k_rs);
-                vreg[u] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)rl * sg.v_rs);
-#endif
-                kpos[u] = second ? posbase[rl] : 0;
-            }
-            float s[kUnroll][G];
-#pragma unroll
-            for (int u = 0; u < kUnroll; ++u) {
-                const bool vis = ok[u] && (!second || kpos[u] <= qpos);
-#pragma unroll
-                for (int g = 0; g < G; ++g) {
-                    float d = 0.f;
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) d = dot2_acc(kreg[u][i], qv[g][i], d);
-                    d = row16_sum(d) * p.scale_log2e;
-                    s[u][g] = vis ? d : kNegInf;
-                }
-            }
-#pragma unroll
-            for (int g = 0; g < G; ++g) {
-                float mx = m_run[g];
-#pragma unroll
-                for (int u = 0; u < kUnroll; ++u) mx = fmaxf(mx, s[u][g]);
-                const float m_use = mx == kNegInf ? 0.f : mx;
-                const float alpha = fast_exp2(m_run[g] - m_use);
-                m_run[g] = mx;
-                float pr[kUnroll], psum = 0.f;
-#pragma unroll
-                for (int u = 0; u < kUnroll; ++u) {
-                    pr[u] = fast_exp2(s[u][g] - m_use);
-                    psum += pr[u];
-                }
-                l_run[g] = l_run[g] * alpha + psum;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) acc[g][i] *= alpha;
-#pragma unroll
-                for (int u = 0; u < kUnroll; ++u)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        acc[g][2 * i] += pr[u] * bf16_lo(vreg[u][i]);
-                        acc[g][2 * i + 1] += pr[u] * bf16_hi(vreg[u][i]);
-                    }
-            }
+            consume_rows<G, kUnroll>(sg, second, kbase, vbase, posbase, r_it, row_end, kq, qpos, p.scale_log2e, qv, m_run, l_run, acc);
         }
 
         // ---- merge the 16 (wave, row group) partials of this workgroup ----------
-        const int grp = wave * 4 + kq;
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) red[grp][g][dc * 8 + i] = acc[g][i];
-            if (dc == 0) {
-                red[grp][g][kD] = m_run[g];
-                red[grp][g][kD + 1] = l_run[g];
-            }
-        }
+        park_partials<G>(red, wave * 4 + kq, dc, m_run, l_run, acc);
         __syncthreads();
         for (int e = tid; e < G * kD; e += kDecThreads) {
             const int g = e / kD, d = e % kD;
-            float mx = kNegInf;
-#pragma unroll
-            for (int j = 0; j < 16; ++j) mx = fmaxf(mx, red[j][g][kD]);
-            const float m_use = mx == kNegInf ? 0.f : mx;
-            float a = 0.f, l = 0.f;
-#pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                const float w = fast_exp2(red[j][g][kD] - m_use);
-                a += w * red[j][g][d];
-                l += w * red[j][g][kD + 1];
-            }
+            float a, l, mx;
+            merge16<G>(red, g, d, a, l, mx);
             float* out = p.ws + ((int64_t)(qi * p.hq + hk * G + g) * nslots + chunk) * kPart;
             out[d] = a;
             if (d == 0) {
@@ -238,6 +278,96 @@ __global__ __launch_bounds__(kDecThreads) void duo_decode_split_kernel(const Dec
             }
         }
 
+    }
+}
+
+// Element (query qi, head, d) of the finished output, row-major and, when asked for, once more in the rows form of
+// the linear-layer kernels ([k / 32][2][64][8] over the [nq, hq * d] matrix the o projection multiplies).
+__device__ __forceinline__ void store_output(const DecParams& p, int qi, int head, int d, float o) {
+    const __bf16 ob = (__bf16)o;
+    p.o[(int64_t)qi * p.o_rs + (int64_t)head * p.o_hs + d] = ob;
+    if (p.op) {
+        const int k = head * kD + d;
+        p.op[((((int64_t)(k / 32) * 2 + qi / 16) * 64) + (qi % 16) + 16 * ((k % 32) / 8)) * 8 + k % 8] = ob;
+    }
+}
+
+// The whole of a (query, kv head) in one workgroup, no partials and no merge launch: both segments one after the
+// other, sixteen waves taking 16-row blocks in turn (as many loads in flight per compute unit as three split-K
+// workgroups have).  For calls whose (query, kv head) pairs alone fill the chip and whose contexts are short enough
+// that their spread cannot unbalance it (a generation step of 32 sequences of a few thousand tokens): one launch
+// instead of two, and no partials through memory.
+constexpr int kWholeWaves = 16;
+constexpr int kWholeThreads = kWholeWaves * kWave;
+
+// The four row groups of a wave (lanes 16 apart hold the same slice of d) into one partial, left in every lane.
+template <int G>
+__device__ __forceinline__ void combine_row_groups(float (&m_run)[G], float (&l_run)[G], float (&acc)[G][8]) {
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        float mx = fmaxf(m_run[g], __shfl_xor(m_run[g], 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float w = fast_exp2(m_run[g] - (mx == kNegInf ? 0.f : mx));
+        float l = l_run[g] * w;
+        l += __shfl_xor(l, 16);
+        l += __shfl_xor(l, 32);
+        l_run[g] = l;
+        m_run[g] = mx;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float a = acc[g][i] * w;
+            a += __shfl_xor(a, 16);
+            a += __shfl_xor(a, 32);
+            acc[g][i] = a;
+        }
+    }
+}
+
+template <int G>
+__global__ __launch_bounds__(kWholeThreads) void duo_decode_whole_kernel(const DecParams p) {
+    HIP_DYNAMIC_SHARED(unsigned char, smem_raw)
+    float (*red)[G][kPart] = reinterpret_cast<float (*)[G][kPart]>(smem_raw);  // [16][G][kPart]: one partial per wave
+    const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+    const int kq = lane / 16, dc = lane % 16;
+    const int qi = blockIdx.x, hk = blockIdx.y;
+    const int slot = p.q_slot[qi];
+    const int qpos = p.q_pos[qi];
+    const int qdepth = p.q_depth ? p.q_depth[qi] : p.depth;
+    u32x4 qv[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+        qv[g] = *reinterpret_cast<const u32x4*>(p.q + (int64_t)qi * p.q_rs + (int64_t)(hk * G + g) * p.q_hs + dc * 8);
+    float m_run[G], l_run[G], acc[G][8];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        m_run[g] = kNegInf;
+        l_run[g] = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[g][i] = 0.f;
+    }
+    constexpr int kBlock = 4 * kUnroll;  // rows per wave and turn
+    for (int seg = 0; seg < 2; ++seg) {
+        const bool second = seg == 1;
+        const int nvis = visible_len(p, second, slot, qpos, qdepth);
+        if (nvis <= 0) continue;  // uniform per workgroup
+        const Seg& sg = second ? p.c2 : p.c1;
+        const int64_t base_row = sg.start[slot];
+        const __bf16* kbase = sg.k + base_row * sg.k_rs + (int64_t)hk * sg.k_hs + dc * 8;
+        const __bf16* vbase = sg.v + base_row * sg.v_rs + (int64_t)hk * sg.v_hs + dc * 8;
+        const int32_t* posbase = second ? sg.pos + (int64_t)slot * sg.capacity : nullptr;
+        for (int r_it = wave * kBlock; r_it < nvis; r_it += kWholeWaves * kBlock)
+            consume_rows<G, kUnroll>(sg, second, kbase, vbase, posbase, r_it, nvis, kq, qpos, p.scale_log2e, qv, m_run, l_run, acc);
+    }
+    combine_row_groups<G>(m_run, l_run, acc);
+    if (kq == 0) park_partials<G>(red, wave, dc, m_run, l_run, acc);
+    __syncthreads();
+    for (int e = tid; e < G * kD; e += kWholeThreads) {
+        const int g = e / kD, d = e % kD;
+        float a, l, mx;
+        merge16<G>(red, g, d, a, l, mx);
+        const int head = hk * G + g;
+        store_output(p, qi, head, d, l > 0.f ? a / l : 0.f);
+        if (p.lse && d == 0) p.lse[(int64_t)qi * p.hq + head] = l > 0.f ? (mx + fast_log2(l)) * kLn2 : kNegInf;
     }
 }
 
@@ -281,12 +411,7 @@ __global__ __launch_bounds__(256) void duo_decode_merge_kernel(const DecParams p
 #pragma unroll
         for (int j = 0; j < 8; ++j) { o += red4[j][tid]; lt += red4[j][kD]; }
         const float inv = lt > 0.f ? 1.0f / lt : 0.f;
-        const __bf16 ob = (__bf16)(o * inv);
-        p.o[(int64_t)qi * p.o_rs + (int64_t)head * p.o_hs + tid] = ob;
-        if (p.op) {  // row qi, column k of the [nq, hq * d] matrix the o projection multiplies
-            const int k = head * kD + tid;
-            p.op[((((int64_t)(k / 32) * 2 + qi / 16) * 64) + (qi % 16) + 16 * ((k % 32) / 8)) * 8 + k % 8] = ob;
-        }
+        store_output(p, qi, head, tid, o * inv);
         if (p.lse && tid == 0) p.lse[(int64_t)qi * p.hq + head] = lt > 0.f ? (mx + fast_log2(lt)) * kLn2 : kNegInf;
     }
 }
@@ -535,6 +660,12 @@ int check_seg(const tah_kv_segment& s, bool need_pos) {
 template <int G>
 int launch_decode(const DecParams& p, hipStream_t st) {
     constexpr int kRedBytes = 16 * G * kPart * (int)sizeof(float);  // 8.3 KB per query head of the group
+    if constexpr (G <= kWholeMaxGroup) {
+        if (p.whole) {
+            hipLaunchKernelGGL((duo_decode_whole_kernel<G>), dim3(p.nq, p.hkv), dim3(kWholeThreads), kRedBytes, st, p);
+            return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
+        }
+    }
     const dim3 grid(p.nchunk1 + p.nchunk2, p.nq, p.hkv);
     if (p.chunk == kChunk) {
         if (kRedBytes > 64 * 1024 &&
@@ -599,6 +730,7 @@ int decode_impl(const tah_duo_decode_args* a, void* ws, size_t ws_bytes, int too
     p.ws = static_cast<float*>(ws);
     p.nq = a->nq; p.hq = a->hq; p.hkv = a->hkv;
     p.chunk = chunk_rows(a->nq, a->hq, a->c1.capacity);
+    p.whole = whole_sequence(a->nq, a->hq, a->hkv, a->c1.capacity) ? 1 : 0;
     p.nchunk1 = (a->c1.capacity + p.chunk - 1) / p.chunk;
     p.nchunk2 = (cap2 + p.chunk - 1) / p.chunk;
     p.scale_log2e = a->scale * kLog2e;

@@ -23,7 +23,10 @@ def oracle_decode(c):
     return o0, l0, o1[hr], l1[hr]
 
 
-@pytest.mark.parametrize("hq,hkv,lens", [(2, 1, [700, 3, 513]), (4, 1, [40]), (2, 2, [1030]), (8, 1, [70, 5])])
+# The last case has 16 (query, kv head) pairs: in the CPU execution build such calls run one workgroup per pair over
+# both segments (duo_decode_whole_kernel; the MI355X build does from 256 pairs on, see the GPU tests).
+@pytest.mark.parametrize("hq,hkv,lens", [(2, 1, [700, 3, 513]), (4, 1, [40]), (2, 2, [1030]), (8, 1, [70, 5]),
+                                         (16, 8, [150, 37])])
 def test_decode_and_append_on_cpu_shim(hq, hkv, lens):
     from tah_amd import kv_cache
     c = make_decode_case(20 + hq, lens, 0.2, Hq=hq, Hkv=hkv, hard_new=[True] + [False] * (len(lens) - 1))
@@ -39,19 +42,24 @@ def test_decode_and_append_on_cpu_shim(hq, hkv, lens):
         o1, l1 = kv_cache.decode(c["q2"], hr, qpos[hr.long()], s1, s2, scale=c["scale"], depth=1, return_lse=True)
         # both depths in one launch
         qd = torch.tensor([0] * nseq + [1] * len(hr), dtype=torch.int32)
-        packed = torch.full((32 * hq * 128,), 3.0, dtype=torch.bfloat16)
+        packed = torch.full((32 * hq * 128,), 3.0, dtype=torch.bfloat16) if nseq + len(hr) <= 32 else None
         om = kv_cache.decode(torch.cat([c["q1"], c["q2"]]), torch.cat([slot, hr]), torch.cat([qpos, qpos[hr.long()]]),
                              s1, s2, scale=c["scale"], q_depth=qd, out_packed=packed)
     # the same output as the rows operand of the o projection; rows past the last query are left alone
-    from tests.test_linear_rows import unpack_rows
-    rows = unpack_rows(packed, hq * 128)
-    assert torch.equal(rows[:om.shape[0]], om.reshape(om.shape[0], -1)) and (rows[om.shape[0]:] == 3.0).all()
+    if packed is not None:
+        from tests.test_linear_rows import unpack_rows
+        rows = unpack_rows(packed, hq * 128)
+        assert torch.equal(rows[:om.shape[0]], om.reshape(om.shape[0], -1)) and (rows[om.shape[0]:] == 3.0).all()
     w0, wl0, w1, wl1 = oracle_decode(c)
     np.testing.assert_allclose(o0.float().numpy(), w0, atol=2e-2, rtol=2e-2)
     np.testing.assert_allclose(l0.numpy(), wl0, atol=2e-3, rtol=1e-3)
     np.testing.assert_allclose(o1.float().numpy(), w1, atol=2e-2, rtol=2e-2)
     np.testing.assert_allclose(l1.numpy(), wl1, atol=2e-3, rtol=1e-3)
-    assert torch.equal(om[:nseq], o0) and torch.equal(om[nseq:], o1)
+    assert torch.equal(om[:nseq], o0)
+    if nseq * hkv < 16:
+        assert torch.equal(om[nseq:], o1)
+    else:  # the depth-1 query alone went through split-K, in the joint call through the one-workgroup kernel: other sum order
+        np.testing.assert_allclose(om[nseq:].float().numpy(), o1.float().numpy(), atol=2e-2, rtol=2e-2)
 
 
 def test_append_is_exact_and_flags_overflow():

@@ -62,6 +62,11 @@ def run_decode(c, cap1, cap2, fused):
     (8, 8, [300], False),
     (16, 4, [777, 64], True),
     (16, 2, [1500, 33], True),   # group of 8 query heads per kv head
+    # 256 or more (query, kv head) pairs and slabs of at most 4096 rows: one workgroup per pair, no merge launch
+    (16, 8, [1 + (211 * i) % 2000 for i in range(32)], True),
+    (16, 8, [1 + (97 * i) % 1200 for i in range(40)], False),
+    (8, 8, [5 + (53 * i) % 700 for i in range(32)], True),
+    (32, 4, [1 + (151 * i) % 900 for i in range(64)], False),  # group of 8
 ])
 def test_decode_matches_oracle(hq, hkv, lens, fused):
     print(f"decode case hq={hq} hkv={hkv} lens={lens} fused={fused}", flush=True)
