@@ -313,6 +313,22 @@ typedef struct tah_topk_mix_args {
  * eager arithmetic rounds; sums are float32 in index order, so results do not vary from run to run. */
 int tah_topk_mix(const tah_topk_mix_args* args, tah_stream_t stream);
 
+/* tah_qk_prep (append, one row per sequence) and tah_duo_decode in one launch, for a generation step: the workgroup
+ * of a (query, kv head) prepares its query heads and the new K and V itself, stores K and V into the slabs and attends
+ * over the cached rows and the new one.  `prep` and `dec` mean what they mean for the two calls (prep->q_out / k_out,
+ * dec->q and the workspace are not used; prep->cache must be dec->c1 or dec->c2; row i of prep is query i of dec and
+ * prep->slot_of[i], where not negative, is dec->q_slot[i]); cache contents and lengths are bit for bit those of the
+ * two calls, the outputs too up to the last bit of a rare element (the same arithmetic in the same order, compiled
+ * twice).  append_at: int32 [rows], the number of rows sequence i's segment of prep->cache holds before the
+ * call, i.e. cache.len[slot] -- handed in because the workgroups of a sequence cannot read the length while one of
+ * them advances it (len[slot] becomes append_at[i] + 1).  Only for calls tah_duo_decode_step_supported() accepts (256
+ * or more (query, kv head) pairs, slabs of at most 4096 rows, one or two query heads per kv head: cases
+ * tah_duo_decode runs without split-K); others return TAH_E_SHAPE and the caller makes the two calls.  Replaces, with
+ * tah_qk_prep's and tah_duo_decode's lists, one more launch per layer and latent iteration. */
+int tah_duo_decode_step_supported(int32_t nq, int32_t hq, int32_t hkv, int32_t capacity1);
+int tah_duo_decode_step(const tah_qk_prep_args* prep, const tah_duo_decode_args* dec, const int32_t* append_at,
+                        tah_stream_t stream);
+
 /* Gate of the Qwen3 MLP for a decode step: out[r][i] = silu(gate_up[r][i]) * gate_up[r][inter + i], both
  * steps rounded to bf16 as the eager modules round them -- `act_fn(gate_proj(x)) * up_proj(x)` of Qwen3MLP.forward
  * (transformers/models/qwen3/modeling_qwen3.py, third party; the layer the reference's base model runs,

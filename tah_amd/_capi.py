@@ -200,6 +200,8 @@ PROTOTYPES = {
     "tah_linear_rows": (C.c_int, [C.POINTER(LinearRowsArgs), c_void_p]),
     "tah_kv_append": (C.c_int, [C.POINTER(KvAppendArgs), c_void_p]),
     "tah_qk_prep": (C.c_int, [C.POINTER(QkPrepArgs), c_void_p]),
+    "tah_duo_decode_step": (C.c_int, [C.POINTER(QkPrepArgs), C.POINTER(DuoDecodeArgs), c_void_p, c_void_p]),
+    "tah_duo_decode_step_supported": (C.c_int, [c_int32, c_int32, c_int32, c_int32]),
     "tah_topk_mix": (C.c_int, [C.POINTER(TopkMixArgs), c_void_p]),
     "tah_silu_mul": (C.c_int, [c_void_p, c_void_p, c_int32, c_int32, c_int64, c_int64, c_void_p]),
     "tah_hard_index_build": (C.c_int, [c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),

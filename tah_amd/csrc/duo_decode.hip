@@ -117,41 +117,66 @@ __device__ __forceinline__ int visible_len(const DecParams& p, bool second, int 
     return qdepth >= 1 ? p.c2.len[slot] : 0;
 }
 
-// Sixteen-lane groups of a wave each take one cache row per load (4 rows x 256 B = 1 KiB per instruction); U such
-// loads of K and of V are in flight per wave.  Scores, online softmax and the weighted sum of V for the 4 U rows
-// from r_it on (rows at or past row_end are masked; their loads are clamped into the slab), for the G query heads of
-// the kv head at once.  m / l / acc: running maximum (log2 domain), sum and un-normalised output of this lane's row
-// group, 8 values of d per lane.
-template <int G, int U>
-__device__ __forceinline__ void consume_rows(const Seg& sg, bool second, const __bf16* kbase, const __bf16* vbase, const int32_t* posbase,
-                                             int r_it, int row_end, int kq, int qpos, float scale_log2e, const u32x4 (&qv)[G],
-                                             float (&m_run)[G], float (&l_run)[G], float (&acc)[G][8]) {
-    u32x4 kreg[U], vreg[U];
-    int kpos[U];
+// kSub: row sub->row of the segment is not taken from memory but from sub->k / v / pos (the token the same
+// workgroup is appending while it attends: what the loads return for that row is discarded).
+struct SubRow {
+    int row;  // -1: none in this segment
+    int pos;
+    u32x4 k, v;
+};
+// The loads of 4 U rows from r_it on (one row per 16-lane group and load; rows at or past row_end are clamped into
+// the slab and flagged).
+template <int U>
+struct RowBlock {
+    u32x4 k[U], v[U];
+    int pos[U];
     bool ok[U];
+};
+template <int U>
+__device__ __forceinline__ void load_rows(RowBlock<U>& b, const Seg& sg, bool second, const __bf16* kbase, const __bf16* vbase,
+                                          const int32_t* posbase, int r_it, int row_end, int kq) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const int r = r_it + u * 4 + kq;
-        ok[u] = r < row_end;
-        const int rl = ok[u] ? r : row_end - 1;  // keep tail loads inside the slab
+        b.ok[u] = r < row_end;
+        const int rl = b.ok[u] ? r : row_end - 1;  // keep tail loads inside the slab
 #if TAH_DEC_NT
-        kreg[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kbase + (int64_t)rl * sg.k_rs));
-        vreg[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vbase + (int64_t)rl * sg.v_rs));
+        b.k[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kbase + (int64_t)rl * sg.k_rs));
+        b.v[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vbase + (int64_t)rl * sg.v_rs));
 #else
-        kreg[u] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)rl * sg.k_rs);
-        vreg[u] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)rl * sg.v_rs);
+        b.k[u] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)rl * sg.k_rs);
+        b.v[u] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)rl * sg.v_rs);
 #endif
-        kpos[u] = second ? posbase[rl] : 0;
+        b.pos[u] = second ? posbase[rl] : 0;
+    }
+}
+// Scores, online softmax and the weighted sum of V for a loaded block, for the G query heads of the kv head at
+// once.  m / l / acc: running maximum (log2 domain), sum and un-normalised output of this lane's row group, 8
+// values of d per lane.
+template <int G, int U, bool kSub = false>
+__device__ __forceinline__ void attend_rows(RowBlock<U>& b, bool second, int r_it, int kq, int qpos, float scale_log2e, const u32x4 (&qv)[G],
+                                            float (&m_run)[G], float (&l_run)[G], float (&acc)[G][8], const SubRow* sub = nullptr) {
+    if constexpr (kSub) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const bool hit = r_it + u * 4 + kq == sub->row;
+            b.pos[u] = hit ? sub->pos : b.pos[u];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                b.k[u][i] = hit ? sub->k[i] : b.k[u][i];
+                b.v[u][i] = hit ? sub->v[i] : b.v[u][i];
+            }
+        }
     }
     float s[U][G];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-        const bool vis = ok[u] && (!second || kpos[u] <= qpos);
+        const bool vis = b.ok[u] && (!second || b.pos[u] <= qpos);
 #pragma unroll
         for (int g = 0; g < G; ++g) {
             float d = 0.f;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) d = dot2_acc(kreg[u][i], qv[g][i], d);
+            for (int i = 0; i < 4; ++i) d = dot2_acc(b.k[u][i], qv[g][i], d);
             d = row16_sum(d) * scale_log2e;
             s[u][g] = vis ? d : kNegInf;
         }
@@ -177,10 +202,20 @@ __device__ __forceinline__ void consume_rows(const Seg& sg, bool second, const _
         for (int u = 0; u < U; ++u)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                acc[g][2 * i] += pr[u] * bf16_lo(vreg[u][i]);
-                acc[g][2 * i + 1] += pr[u] * bf16_hi(vreg[u][i]);
+                acc[g][2 * i] += pr[u] * bf16_lo(b.v[u][i]);
+                acc[g][2 * i + 1] += pr[u] * bf16_hi(b.v[u][i]);
             }
     }
+}
+// Sixteen-lane groups of a wave each take one cache row per load (4 rows x 256 B = 1 KiB per instruction); U such
+// loads of K and of V are in flight per wave: load, then attend.
+template <int G, int U, bool kSub = false>
+__device__ __forceinline__ void consume_rows(const Seg& sg, bool second, const __bf16* kbase, const __bf16* vbase, const int32_t* posbase,
+                                             int r_it, int row_end, int kq, int qpos, float scale_log2e, const u32x4 (&qv)[G],
+                                             float (&m_run)[G], float (&l_run)[G], float (&acc)[G][8], const SubRow* sub = nullptr) {
+    RowBlock<U> b;
+    load_rows<U>(b, sg, second, kbase, vbase, posbase, r_it, row_end, kq);
+    attend_rows<G, U, kSub>(b, second, r_it, kq, qpos, scale_log2e, qv, m_run, l_run, acc, sub);
 }
 
 // The 16 (wave, row group) partials of a workgroup into LDS: red[16][G][kPart].
@@ -517,6 +552,34 @@ __device__ __forceinline__ uint32_t mul_bf16x2(uint32_t a, uint32_t b) {
     return pack_bf16(bf16_lo(a) * bf16_lo(b), bf16_hi(a) * bf16_hi(b));
 }
 
+// One head's 16-byte piece (lane j of the head's 16 lanes) through RMSNorm, weight and rotary embedding, with the
+// roundings listed above; `sign`: 0x80008000 for the lower half of the head (j < 8), where the partner enters negated.
+__device__ __forceinline__ u32x4 prep_head_piece(u32x4 xin, const u32x4& w, const u32x4& cs, const u32x4& sn, uint32_t sign, float eps) {
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ss += bf16_lo(xin[i]) * bf16_lo(xin[i]) + bf16_hi(xin[i]) * bf16_hi(xin[i]);
+    ss = row16_sum(ss);
+    // hardware reciprocal square root (1 ulp): whether it or the order of the sum above decides
+    // the last bit of a normalised value before the bf16 rounding is the same kind of difference
+    const float rs = __builtin_amdgcn_rsqf(ss * (1.0f / 128.0f) + eps);
+    u32x4 yn, out;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) yn[i] = mul_bf16x2(w[i], pack_bf16(bf16_lo(xin[i]) * rs, bf16_hi(xin[i]) * rs));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        // the partner's normalised values: lane j^8 of this row (row rotation by 8)
+        const uint32_t pn = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)yn[i], 0x128, 0xf, 0xf, false) ^ sign;
+        const uint32_t a = mul_bf16x2(yn[i], cs[i]), b = mul_bf16x2(pn, sn[i]);
+        out[i] = pack_bf16(bf16_lo(a) + bf16_lo(b), bf16_hi(a) + bf16_hi(b));
+    }
+    return out;
+}
+__device__ __forceinline__ u32x4 scale_piece(u32x4 x, float f) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) x[i] = pack_bf16(bf16_lo(x[i]) * f, bf16_hi(x[i]) * f);
+    return x;
+}
+
 // One workgroup (4 waves) per token row.  A head is handled by 16 lanes, 8 elements (16 bytes) each, so
 // a wave takes 4 heads at a time and the workgroup 16: the mean of squares is a DPP reduction inside
 // the row of 16 lanes, and the rotary partner of lane j's elements (+-64) sits in lane j^8 of the
@@ -601,35 +664,150 @@ __global__ __launch_bounds__(256) void qk_prep_kernel(const PrepParams p) {
         const int it = pass * 16 + sub;
         const bool is_q = it < p.hq, is_k = !is_q && it < p.hq + p.hkv, is_v = !is_q && !is_k && it < items;
         u32x4 xin = pass == 0 ? ahead[0] : pass == 1 ? ahead[1] : load_item(it);
-        if (p.xn) {  // the row's input-norm factor, applied where the eager modules have a normalised projection
-#pragma unroll
-            for (int i = 0; i < 4; ++i) xin[i] = pack_bf16(bf16_lo(xin[i]) * rin, bf16_hi(xin[i]) * rin);
-        }
+        if (p.xn) xin = scale_piece(xin, rin);  // the row's input-norm factor, applied where the eager modules have a normalised projection
         if (is_v && vdst)  // a V head: moved as it is
             *reinterpret_cast<u32x4*>(vdst + (int64_t)(it - p.hq - p.hkv) * vd_hs + 8 * j) = xin;
         const int h = is_q ? it : it - p.hq;
         __bf16* y = is_q ? p.q_out + (int64_t)r * p.qo_rs + (int64_t)h * p.qo_hs
                          : (is_k && kdst ? kdst + (int64_t)h * kd_hs : nullptr);  // null: no head, or the row overflows its slab
-        float ss = 0.f;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) ss += bf16_lo(xin[i]) * bf16_lo(xin[i]) + bf16_hi(xin[i]) * bf16_hi(xin[i]);
-        ss = row16_sum(ss);
-        // hardware reciprocal square root (1 ulp): whether it or the order of the sum above decides
-        // the last bit of a normalised value before the bf16 rounding is the same kind of difference
-        const float rs = __builtin_amdgcn_rsqf(ss * (1.0f / 128.0f) + p.eps);
-        const u32x4 w = is_q ? qw : kw;
-        u32x4 yn, out;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            yn[i] = mul_bf16x2(w[i], pack_bf16(bf16_lo(xin[i]) * rs, bf16_hi(xin[i]) * rs));
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            // the partner's normalised values: lane j^8 of this row (row rotation by 8)
-            const uint32_t pn = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)yn[i], 0x128, 0xf, 0xf, false) ^ sign;
-            const uint32_t a = mul_bf16x2(yn[i], cs[i]), b = mul_bf16x2(pn, sn[i]);
-            out[i] = pack_bf16(bf16_lo(a) + bf16_lo(b), bf16_hi(a) + bf16_hi(b));
-        }
+        const u32x4 out = prep_head_piece(xin, is_q ? qw : kw, cs, sn, sign, p.eps);
         if (y) *reinterpret_cast<u32x4*>(y + 8 * j) = out;
+    }
+}
+
+// ---- q/k preparation, append and attention of a decode step in one launch --------------------------------
+// What qk_prep_kernel (one row per sequence, append) followed by duo_decode_whole_kernel do, for calls the latter
+// takes: the workgroup of (query, kv head) prepares the G query heads and the new K and V of its kv head itself
+// (every 16-lane group of every wave repeats the few dozen operations: the prepared pieces are then where the row
+// loop wants them), one group stores K and V into the slabs for the steps to come, and the row loop takes the new
+// row from registers instead of reading back what is being written.  The place of the new row comes from the
+// caller (append_at[], the segment's length before the call): the eight workgroups of a sequence cannot read
+// len[] while one of them advances it.  Same arithmetic in the same order as the two kernels: the slabs get the
+// same bits, the outputs too except where the compiler contracted a multiply-add in one kernel and not the other.
+constexpr int kStepMaxGroup = 2;  // with four query heads per kv head the preparation no longer fits the 128 registers
+struct StepParams {
+    PrepParams prep;
+    DecParams dec;
+    const int32_t* append_at;
+    int32_t append_second;  // the new K/V go to the depth-1 segment
+};
+
+template <int G>
+__global__ __launch_bounds__(kWholeThreads) void duo_decode_step_kernel(const StepParams sp) {
+    const PrepParams& pp = sp.prep;
+    const DecParams& p = sp.dec;
+    HIP_DYNAMIC_SHARED(unsigned char, smem_raw)
+    float (*red)[G][kPart] = reinterpret_cast<float (*)[G][kPart]>(smem_raw);
+    __shared__ float xn_part[kWholeWaves];
+    const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+    const int kq = lane / 16, dc = lane % 16;
+    const int qi = blockIdx.x, hk = blockIdx.y;
+    // the row's data first: the loads fly while the bookkeeping is looked up
+    u32x4 xq[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) xq[g] = *reinterpret_cast<const u32x4*>(pp.q + (int64_t)qi * pp.q_rs + (int64_t)(hk * G + g) * pp.q_hs + 8 * dc);
+    u32x4 xk = *reinterpret_cast<const u32x4*>(pp.k + (int64_t)qi * pp.k_rs + (int64_t)hk * pp.k_hs + 8 * dc);
+    u32x4 xv = *reinterpret_cast<const u32x4*>(pp.v + (int64_t)qi * pp.v_rs + (int64_t)hk * pp.v_hs + 8 * dc);
+    const u32x4 cs = *reinterpret_cast<const u32x4*>(pp.cos + (int64_t)qi * pp.cs_rs + 8 * dc);
+    const u32x4 sn = *reinterpret_cast<const u32x4*>(pp.sin + (int64_t)qi * pp.cs_rs + 8 * dc);
+    const u32x4 qw = *reinterpret_cast<const u32x4*>(pp.qw + 8 * dc), kw = *reinterpret_cast<const u32x4*>(pp.kw + 8 * dc);
+    const int slot = p.q_slot[qi];
+    const int qpos = p.q_pos[qi];
+    const int qdepth = p.q_depth ? p.q_depth[qi] : p.depth;
+    const int aslot = pp.a.slot_of ? pp.a.slot_of[qi] : qi;  // < 0: the row is not cached
+    const int dst = sp.append_at[qi];
+    const int pos_new = pp.a.pos_new ? pp.a.pos_new[qi] : 0;
+    const bool cached = aslot >= 0, fits = cached && dst < pp.a.capacity;
+    // rows of a segment: with the new row where this call appends (nobody may read len[] of that segment here)
+    auto visible = [&](int seg) {
+        const Seg& sg = seg ? p.c2 : p.c1;
+        if (seg && qdepth < 1) return 0;
+        const int n = (seg == sp.append_second && cached) ? (fits ? dst + 1 : (dst < pp.a.capacity ? dst : pp.a.capacity)) : sg.len[slot];
+        return seg ? n : (qpos + 1 < n ? (qpos + 1 > 0 ? qpos + 1 : 0) : n);
+    };
+    constexpr int kBlock = 4 * kUnroll;
+    // this wave's first block of cached rows goes on its way before the preparation below, which needs none of it
+    const int nvis0 = visible(0);
+    const int64_t base0 = p.c1.start[slot];
+    const __bf16* kbase0 = p.c1.k + base0 * p.c1.k_rs + (int64_t)hk * p.c1.k_hs + dc * 8;
+    const __bf16* vbase0 = p.c1.v + base0 * p.c1.v_rs + (int64_t)hk * p.c1.v_hs + dc * 8;
+    RowBlock<kUnroll> first;
+    const bool have_first = wave * kBlock < nvis0;  // uniform per wave
+    if (have_first) load_rows<kUnroll>(first, p.c1, false, kbase0, vbase0, nullptr, wave * kBlock, nvis0, kq);
+    float rin = 1.0f;
+    if (pp.xn) {
+        const __bf16* xr = pp.xn + (int64_t)qi * pp.xn_rs;
+        float ss = 0.f;
+        // summed as qk_prep_kernel's 256 threads sum it (same strides, same order), so that the factor has the same bits
+        if (tid < 256)
+            for (int c = tid * 8; c < pp.xn_cols; c += 256 * 8) {
+                const u32x4 x = *reinterpret_cast<const u32x4*>(xr + c);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) ss += bf16_lo(x[i]) * bf16_lo(x[i]) + bf16_hi(x[i]) * bf16_hi(x[i]);
+            }
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m);
+        if (lane == 0) xn_part[wave] = ss;
+        __syncthreads();
+        ss = (xn_part[0] + xn_part[1]) + (xn_part[2] + xn_part[3]);
+        rin = __builtin_amdgcn_rsqf(ss / (float)pp.xn_cols + pp.xn_eps);
+#pragma unroll
+        for (int g = 0; g < G; ++g) xq[g] = scale_piece(xq[g], rin);
+        xk = scale_piece(xk, rin);
+        xv = scale_piece(xv, rin);
+    }
+    const uint32_t sign = dc < 8 ? 0x80008000u : 0u;
+    u32x4 qv[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) qv[g] = prep_head_piece(xq[g], qw, cs, sn, sign, pp.eps);
+    SubRow sub;
+    sub.k = prep_head_piece(xk, kw, cs, sn, sign, pp.eps);
+    sub.v = xv;
+    sub.pos = pos_new;
+    if (cached && !fits && pp.a.overflow && tid == 0 && hk == 0) *pp.a.overflow = 1;
+    if (fits && wave == 0 && kq == 0) {
+        const int64_t drow = (int64_t)const_i32(pp.a.start, aslot) + dst;
+        *reinterpret_cast<u32x4*>(pp.a.ck + drow * pp.a.ck_rs + (int64_t)hk * pp.a.ck_hs + 8 * dc) = sub.k;
+        *reinterpret_cast<u32x4*>(pp.a.cv + drow * pp.a.cv_rs + (int64_t)hk * pp.a.cv_hs + 8 * dc) = sub.v;
+        if (dc == 0 && hk == 0) {
+            if (pp.a.cpos && pp.a.pos_new) pp.a.cpos[(int64_t)aslot * pp.a.capacity + dst] = pos_new;
+            pp.a.len[aslot] = dst + 1;
+        }
+    }
+    float m_run[G], l_run[G], acc[G][8];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        m_run[g] = kNegInf;
+        l_run[g] = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[g][i] = 0.f;
+    }
+    // depth-0 segment: the block loaded above, then the wave's other turns
+    sub.row = (sp.append_second == 0 && fits) ? dst : -1;
+    if (have_first) attend_rows<G, kUnroll, true>(first, false, wave * kBlock, kq, qpos, p.scale_log2e, qv, m_run, l_run, acc, &sub);
+    for (int r_it = (wave + kWholeWaves) * kBlock; r_it < nvis0; r_it += kWholeWaves * kBlock)
+        consume_rows<G, kUnroll, true>(p.c1, false, kbase0, vbase0, nullptr, r_it, nvis0, kq, qpos, p.scale_log2e, qv, m_run, l_run, acc, &sub);
+    // depth-1 segment
+    const int nvis1 = visible(1);
+    if (nvis1 > 0) {  // uniform per workgroup
+        sub.row = (sp.append_second == 1 && fits) ? dst : -1;
+        const int64_t base1 = p.c2.start[slot];
+        const __bf16* kbase1 = p.c2.k + base1 * p.c2.k_rs + (int64_t)hk * p.c2.k_hs + dc * 8;
+        const __bf16* vbase1 = p.c2.v + base1 * p.c2.v_rs + (int64_t)hk * p.c2.v_hs + dc * 8;
+        const int32_t* posbase = p.c2.pos + (int64_t)slot * p.c2.capacity;
+        for (int r_it = wave * kBlock; r_it < nvis1; r_it += kWholeWaves * kBlock)
+            consume_rows<G, kUnroll, true>(p.c2, true, kbase1, vbase1, posbase, r_it, nvis1, kq, qpos, p.scale_log2e, qv, m_run, l_run, acc, &sub);
+    }
+    combine_row_groups<G>(m_run, l_run, acc);
+    if (kq == 0) park_partials<G>(red, wave, dc, m_run, l_run, acc);
+    __syncthreads();
+    for (int e = tid; e < G * kD; e += kWholeThreads) {
+        const int g = e / kD, d = e % kD;
+        float a, l, mx;
+        merge16<G>(red, g, d, a, l, mx);
+        const int head = hk * G + g;
+        store_output(p, qi, head, d, l > 0.f ? a / l : 0.f);
+        if (p.lse && d == 0) p.lse[(int64_t)qi * p.hq + head] = l > 0.f ? (mx + fast_log2(l)) * kLn2 : kNegInf;
     }
 }
 
@@ -698,16 +876,20 @@ extern "C" size_t tah_duo_decode_workspace_bytes(int32_t nq, int32_t hq, int32_t
 namespace tah {
 namespace {
 
-// Shared by the two decode entry points: `ws` is the caller's workspace or the library's static scratch.
-int decode_impl(const tah_duo_decode_args* a, void* ws, size_t ws_bytes, int too_small, tah_stream_t stream) {
+// Argument checks of the decode entry points and the kernels' parameters.  `fused`: the call is the second half of
+// tah_duo_decode_step (no prepared q in memory, no workspace).  Returns 1 when there is nothing to do.
+int dec_fill(const tah_duo_decode_args* a, DecParams& p, bool fused, void* ws, size_t ws_bytes, int too_small) {
     if (!a) return TAH_E_NULL;
     if (a->d != kD || a->nq < 0 || a->hq <= 0 || a->hkv <= 0 || a->hq % a->hkv) return TAH_E_SHAPE;
     const int g = a->hq / a->hkv;
     if (g != 1 && g != 2 && g != 4 && g != 8) return TAH_E_SHAPE;
-    if (a->nq == 0) return TAH_OK;
+    if (a->nq == 0) return 1;
     if (a->nq > 65535 || a->hq > 65535) return TAH_E_SHAPE;
-    if (!a->q || !a->o || !a->q_slot || !a->q_pos || !ws) return TAH_E_NULL;
-    if (!aligned16(a->q) || !aligned16(ws) || a->q_row_stride % 8 || a->q_head_stride % 8) return TAH_E_ALIGN;
+    if (!a->o || !a->q_slot || !a->q_pos) return TAH_E_NULL;
+    if (!fused) {
+        if (!a->q || !ws) return TAH_E_NULL;
+        if (!aligned16(a->q) || !aligned16(ws) || a->q_row_stride % 8 || a->q_head_stride % 8) return TAH_E_ALIGN;
+    }
     if (a->o_packed && a->nq > 32) return TAH_E_SHAPE;
     if (!aligned16(a->o_packed)) return TAH_E_ALIGN;
     if (int rc = check_seg(a->c1, false)) return rc;
@@ -715,8 +897,7 @@ int decode_impl(const tah_duo_decode_args* a, void* ws, size_t ws_bytes, int too
     if (any_depth1)
         if (int rc = check_seg(a->c2, true)) return rc;
     const int cap2 = any_depth1 ? a->c2.capacity : 0;
-    if (ws_bytes < tah_duo_decode_workspace_bytes(a->nq, a->hq, a->c1.capacity, cap2)) return too_small;
-    DecParams p;
+    if (!fused && ws_bytes < tah_duo_decode_workspace_bytes(a->nq, a->hq, a->c1.capacity, cap2)) return too_small;
     p.q = static_cast<const __bf16*>(a->q);
     p.o = static_cast<__bf16*>(a->o);
     p.op = static_cast<__bf16*>(a->o_packed);
@@ -735,6 +916,14 @@ int decode_impl(const tah_duo_decode_args* a, void* ws, size_t ws_bytes, int too
     p.nchunk2 = (cap2 + p.chunk - 1) / p.chunk;
     p.scale_log2e = a->scale * kLog2e;
     if (p.nchunk1 + p.nchunk2 == 0) return TAH_E_SHAPE;
+    return TAH_OK;
+}
+
+// Shared by the two decode entry points: `ws` is the caller's workspace or the library's static scratch.
+int decode_impl(const tah_duo_decode_args* a, void* ws, size_t ws_bytes, int too_small, tah_stream_t stream) {
+    DecParams p;
+    if (int rc = dec_fill(a, p, false, ws, ws_bytes, too_small)) return rc < 0 ? rc : TAH_OK;
+    const int g = a->hq / a->hkv;
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (g) {
         case 1: return launch_decode<1>(p, st);
@@ -778,12 +967,17 @@ extern "C" int tah_duo_decode_static(const tah_duo_decode_args* a, tah_stream_t 
     return tah::decode_impl(a, ws, TAH_DUO_STATIC_SCRATCH_BYTES, TAH_E_SCRATCH, stream);
 }
 
-extern "C" int tah_qk_prep(const tah_qk_prep_args* a, tah_stream_t stream) {
-    using namespace tah;
+namespace tah {
+namespace {
+
+// Argument checks of tah_qk_prep and its kernel parameters.  `fused`: the call is the first half of
+// tah_duo_decode_step, which keeps the prepared heads in registers (q_out / k_out are not needed).
+// Returns 1 when there is nothing to do.
+int prep_fill(const tah_qk_prep_args* a, PrepParams& p, bool fused) {
     if (!a) return TAH_E_NULL;
     if (a->d != kD || a->rows < 0 || a->hq <= 0 || a->hkv <= 0) return TAH_E_SHAPE;
-    if (a->rows == 0) return TAH_OK;
-    if (!a->q || !a->k || !a->q_out || !a->q_weight || !a->k_weight || !a->cos || !a->sin) return TAH_E_NULL;
+    if (a->rows == 0) return 1;
+    if (!a->q || !a->k || (!fused && !a->q_out) || !a->q_weight || !a->k_weight || !a->cos || !a->sin) return TAH_E_NULL;
     if (a->append) {
         if (!a->v || !a->cu_new) return TAH_E_NULL;
         if (a->nseq <= 0 || a->cache.capacity <= 0) return TAH_E_SHAPE;
@@ -803,7 +997,6 @@ extern "C" int tah_qk_prep(const tah_qk_prep_args* a, tah_stream_t stream) {
                           a->append ? a->cache.k : nullptr, a->append ? a->cache.v : nullptr, a->norm_input};
     for (const void* q : ptrs)
         if (q && !aligned16(q)) return TAH_E_ALIGN;
-    PrepParams p;
     p.q = static_cast<const __bf16*>(a->q); p.k = static_cast<const __bf16*>(a->k); p.v = static_cast<const __bf16*>(a->v);
     p.q_out = static_cast<__bf16*>(a->q_out); p.k_out = static_cast<__bf16*>(a->k_out); p.v_out = static_cast<__bf16*>(a->v_out);
     p.q_rs = a->q_row_stride; p.q_hs = a->q_head_stride; p.k_rs = a->k_row_stride; p.k_hs = a->k_head_stride;
@@ -831,6 +1024,16 @@ extern "C" int tah_qk_prep(const tah_qk_prep_args* a, tah_stream_t stream) {
         p.a.capacity = a->cache.capacity; p.a.nseq = a->nseq; p.a.hkv = a->hkv;
         p.a.overflow = a->overflow;
     }
+    return TAH_OK;
+}
+
+}  // namespace
+}  // namespace tah
+
+extern "C" int tah_qk_prep(const tah_qk_prep_args* a, tah_stream_t stream) {
+    using namespace tah;
+    PrepParams p;
+    if (int rc = prep_fill(a, p, false)) return rc < 0 ? rc : TAH_OK;
     hipStream_t st = static_cast<hipStream_t>(stream);
     hipLaunchKernelGGL(qk_prep_kernel, dim3(a->rows), dim3(256), 0, st, p);
     if (a->append && !p.own_len) hipLaunchKernelGGL(kv_append_len_kernel, dim3((a->nseq + 63) / 64), dim3(64), 0, st, p.a);
@@ -866,4 +1069,43 @@ extern "C" int tah_kv_append(const tah_kv_append_args* a, tah_stream_t stream) {
     hipLaunchKernelGGL(kv_append_rows_kernel, dim3((a->total_new + 7) / 8), dim3(256), 0, st, p, a->total_new);
     hipLaunchKernelGGL(kv_append_len_kernel, dim3((a->nseq + 63) / 64), dim3(64), 0, st, p);
     return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
+}
+
+namespace tah {
+namespace {
+template <int G>
+int launch_step(const StepParams& sp, hipStream_t st) {
+    constexpr int kRedBytes = 16 * G * kPart * (int)sizeof(float);
+    hipLaunchKernelGGL((duo_decode_step_kernel<G>), dim3(sp.dec.nq, sp.dec.hkv), dim3(kWholeThreads), kRedBytes, st, sp);
+    return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
+}
+}  // namespace
+}  // namespace tah
+
+extern "C" int tah_duo_decode_step_supported(int32_t nq, int32_t hq, int32_t hkv, int32_t capacity1) {
+    if (nq <= 0 || hq <= 0 || hkv <= 0 || hq % hkv) return 0;
+    return tah::whole_sequence(nq, hq, hkv, capacity1) && hq / hkv <= tah::kStepMaxGroup ? 1 : 0;
+}
+
+extern "C" int tah_duo_decode_step(const tah_qk_prep_args* prep, const tah_duo_decode_args* dec, const int32_t* append_at,
+                                   tah_stream_t stream) {
+    using namespace tah;
+    if (!prep || !dec) return TAH_E_NULL;
+    StepParams sp;
+    const int rc_p = prep_fill(prep, sp.prep, true);
+    if (rc_p < 0) return rc_p;
+    const int rc_d = dec_fill(dec, sp.dec, true, nullptr, 0, TAH_E_WORKSPACE);
+    if (rc_d < 0) return rc_d;
+    if (rc_p == 1 && rc_d == 1) return TAH_OK;
+    // one row per sequence, appended to one of the two segments the queries read, in a call the one-workgroup kernel takes
+    if (rc_p == 1 || rc_d == 1 || prep->rows != dec->nq || prep->hq != dec->hq || prep->hkv != dec->hkv) return TAH_E_SHAPE;
+    if (!prep->append || !prep->append_one_row_per_seq || prep->nseq != prep->rows || !prep->v) return TAH_E_SHAPE;
+    if (!tah_duo_decode_step_supported(dec->nq, dec->hq, dec->hkv, dec->c1.capacity)) return TAH_E_SHAPE;
+    if (!append_at) return TAH_E_NULL;
+    if (prep->cache.k == dec->c1.k) sp.append_second = 0;
+    else if (prep->cache.k == dec->c2.k && (dec->q_depth != nullptr || dec->depth >= 1)) sp.append_second = 1;
+    else return TAH_E_SHAPE;
+    sp.append_at = append_at;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    return dec->hq / dec->hkv == 1 ? launch_step<1>(sp, st) : launch_step<2>(sp, st);
 }

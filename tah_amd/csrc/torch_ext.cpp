@@ -40,6 +40,8 @@ struct Api {
     decltype(&tah_duo_decode_static) decode_static = nullptr;
     decltype(&tah_kv_append) kv_append = nullptr;
     decltype(&tah_qk_prep) qk_prep = nullptr;
+    decltype(&tah_duo_decode_step) decode_step = nullptr;
+    decltype(&tah_duo_decode_step_supported) decode_step_supported = nullptr;
     decltype(&tah_topk_mix) topk_mix = nullptr;
     decltype(&tah_silu_mul) silu_mul = nullptr;
     decltype(&tah_hard_index_build) hard_index_build = nullptr;
@@ -78,6 +80,8 @@ void load_library(const std::string& path, bool allow_host) {
     bind(g.decode_static, "tah_duo_decode_static");
     bind(g.kv_append, "tah_kv_append");
     bind(g.qk_prep, "tah_qk_prep");
+    bind(g.decode_step, "tah_duo_decode_step");
+    bind(g.decode_step_supported, "tah_duo_decode_step_supported");
     bind(g.topk_mix, "tah_topk_mix");
     bind(g.silu_mul, "tah_silu_mul");
     bind(g.hard_index_build, "tah_hard_index_build");
@@ -323,31 +327,47 @@ int64_t decode_workspace_bytes(int64_t nq, int64_t hq, int64_t cap1, int64_t cap
     return (int64_t)g.decode_workspace_bytes((int32_t)nq, (int32_t)hq, (int32_t)cap1, (int32_t)cap2);
 }
 
-void duo_decode(const Tensor& q, const Tensor& o, const optional<Tensor>& lse, const Tensor& q_slot, const Tensor& q_pos,
-                const optional<Tensor>& q_depth, int64_t depth, const Tensor& k1, const Tensor& v1, const Tensor& start1,
-                const Tensor& len1, const optional<Tensor>& k2, const optional<Tensor>& v2, const optional<Tensor>& pos2,
-                const optional<Tensor>& start2, const optional<Tensor>& len2, const optional<Tensor>& workspace, double scale,
-                const optional<Tensor>& o_packed) {
-    need_lib();
-    thd(q, "q"); i32(q_slot, "q_slot"); i32(q_pos, "q_pos");
-    Dev d; d.see(q); d.see(o); d.see(lse); d.see(q_slot); d.see(q_pos); d.see(q_depth); d.see(k1); d.see(workspace); d.see(o_packed);
+// tah_duo_decode_args from tensors; q may be absent for the fused step (the queries are prepared inside the kernel).
+tah_duo_decode_args decode_args(Dev& d, const optional<Tensor>& q, const Tensor& o, const optional<Tensor>& lse, const Tensor& q_slot,
+                                const Tensor& q_pos, const optional<Tensor>& q_depth, int64_t depth, const Tensor& k1, const Tensor& v1,
+                                const Tensor& start1, const Tensor& len1, const optional<Tensor>& k2, const optional<Tensor>& v2,
+                                const optional<Tensor>& pos2, const optional<Tensor>& start2, const optional<Tensor>& len2, double scale,
+                                const optional<Tensor>& o_packed) {
+    thd(o, "o"); i32(q_slot, "q_slot"); i32(q_pos, "q_pos");
+    d.see(q); d.see(o); d.see(lse); d.see(q_slot); d.see(q_pos); d.see(q_depth); d.see(k1); d.see(o_packed);
     if (o_packed.has_value())
-        TORCH_CHECK(o_packed->scalar_type() == at::kBFloat16 && o_packed->is_contiguous() && o_packed->numel() == 32 * q.size(1) * q.size(2),
+        TORCH_CHECK(o_packed->scalar_type() == at::kBFloat16 && o_packed->is_contiguous() && o_packed->numel() == 32 * o.size(1) * o.size(2),
                     "duo_decode: o_packed must be a contiguous bf16 tensor of 32 * Hq * D elements");
     const bool need2 = q_depth.has_value() || depth >= 1;
     TORCH_CHECK(!need2 || (k2.has_value() && v2.has_value() && pos2.has_value() && start2.has_value() && len2.has_value()),
                 "depth-1 queries need the depth-1 cache");
     tah_duo_decode_args a{};
-    a.q = ptr(q); a.o = mptr(o); a.lse = lse.has_value() ? static_cast<float*>(lse->data_ptr()) : nullptr;
-    a.q_row_stride = q.stride(0); a.q_head_stride = q.stride(1); a.o_row_stride = o.stride(0); a.o_head_stride = o.stride(1);
+    a.o = mptr(o); a.lse = lse.has_value() ? static_cast<float*>(lse->data_ptr()) : nullptr;
+    a.o_row_stride = o.stride(0); a.o_head_stride = o.stride(1);
+    if (q.has_value()) {
+        thd(*q, "q");
+        TORCH_CHECK(q->sizes() == o.sizes(), "duo_decode: q and o must have the same shape");
+        a.q = ptr(*q); a.q_row_stride = q->stride(0); a.q_head_stride = q->stride(1);
+    }
     a.q_slot = static_cast<const int32_t*>(q_slot.data_ptr());
     a.q_pos = static_cast<const int32_t*>(q_pos.data_ptr());
     a.q_depth = q_depth.has_value() ? static_cast<const int32_t*>(q_depth->data_ptr()) : nullptr;
     a.depth = (int32_t)depth;
     a.c1 = segment(k1, v1, c10::nullopt, start1, len1);
     if (need2) a.c2 = segment(*k2, *v2, pos2, *start2, *len2);
-    a.nq = (int32_t)q.size(0); a.hq = (int32_t)q.size(1); a.hkv = (int32_t)k1.size(1); a.d = (int32_t)q.size(2); a.scale = (float)scale;
+    a.nq = (int32_t)o.size(0); a.hq = (int32_t)o.size(1); a.hkv = (int32_t)k1.size(1); a.d = (int32_t)o.size(2); a.scale = (float)scale;
     a.o_packed = o_packed.has_value() ? o_packed->data_ptr() : nullptr;
+    return a;
+}
+
+void duo_decode(const Tensor& q, const Tensor& o, const optional<Tensor>& lse, const Tensor& q_slot, const Tensor& q_pos,
+                const optional<Tensor>& q_depth, int64_t depth, const Tensor& k1, const Tensor& v1, const Tensor& start1,
+                const Tensor& len1, const optional<Tensor>& k2, const optional<Tensor>& v2, const optional<Tensor>& pos2,
+                const optional<Tensor>& start2, const optional<Tensor>& len2, const optional<Tensor>& workspace, double scale,
+                const optional<Tensor>& o_packed) {
+    need_lib();
+    Dev d; d.see(workspace);
+    tah_duo_decode_args a = decode_args(d, q, o, lse, q_slot, q_pos, q_depth, depth, k1, v1, start1, len1, k2, v2, pos2, start2, len2, scale, o_packed);
     if (workspace.has_value()) {
         a.workspace = workspace->data_ptr();
         a.workspace_bytes = (size_t)workspace->numel() * workspace->element_size();
@@ -376,16 +396,16 @@ void kv_append(const Tensor& k_new, const Tensor& v_new, const Tensor& cu_new, c
     check_rc(g.kv_append(&a, d.stream()), "tah_kv_append");
 }
 
-// q/k RMSNorm + rotary (+ append): returns nothing, the caller allocated q_out / k_out.
-void qk_prep(const Tensor& q, const Tensor& k, const optional<Tensor>& v, const Tensor& q_out, const optional<Tensor>& k_out,
-             const Tensor& q_weight, const Tensor& k_weight, const Tensor& cos, const Tensor& sin, double eps,
-             const optional<Tensor>& ck, const optional<Tensor>& cv, const optional<Tensor>& cpos, const optional<Tensor>& start,
-             const optional<Tensor>& len, const optional<Tensor>& overflow, const optional<Tensor>& cu_new,
-             const optional<Tensor>& pos_new, const optional<Tensor>& slot_of, bool one_row_per_seq,
-             const optional<Tensor>& v_out, const optional<Tensor>& norm_input, double norm_eps) {
-    need_lib();
+// tah_qk_prep_args from tensors; q_out may be absent for the fused step (the prepared heads stay in registers).
+tah_qk_prep_args prep_args(Dev& d, const Tensor& q, const Tensor& k, const optional<Tensor>& v, const optional<Tensor>& q_out,
+                           const optional<Tensor>& k_out, const Tensor& q_weight, const Tensor& k_weight, const Tensor& cos,
+                           const Tensor& sin, double eps, const optional<Tensor>& ck, const optional<Tensor>& cv,
+                           const optional<Tensor>& cpos, const optional<Tensor>& start, const optional<Tensor>& len,
+                           const optional<Tensor>& overflow, const optional<Tensor>& cu_new, const optional<Tensor>& pos_new,
+                           const optional<Tensor>& slot_of, bool one_row_per_seq, const optional<Tensor>& v_out,
+                           const optional<Tensor>& norm_input, double norm_eps) {
     thd(q, "q"); thd(k, "k");
-    Dev d; d.see(q); d.see(k); d.see(v); d.see(q_weight); d.see(k_weight); d.see(cos); d.see(sin); d.see(cu_new); d.see(pos_new);
+    d.see(q); d.see(k); d.see(v); d.see(q_weight); d.see(k_weight); d.see(cos); d.see(sin); d.see(cu_new); d.see(pos_new);
     d.see(slot_of); d.see(ck);
     const int64_t D = q.size(2);
     for (auto p : {std::make_pair(&q_weight, "q_weight"), {&k_weight, "k_weight"}})
@@ -398,10 +418,14 @@ void qk_prep(const Tensor& q, const Tensor& k, const optional<Tensor>& v, const 
     TORCH_CHECK(cos.stride(0) == sin.stride(0), "cos and sin must share their row stride");
     TORCH_CHECK(k.size(0) == q.size(0), "q and k must have one row per token");
     tah_qk_prep_args a{};
-    a.q = ptr(q); a.k = ptr(k); a.v = ptr(v); a.q_out = mptr(q_out);
+    a.q = ptr(q); a.k = ptr(k); a.v = ptr(v);
     a.q_row_stride = q.stride(0); a.q_head_stride = q.stride(1);
     a.k_row_stride = k.stride(0); a.k_head_stride = k.stride(1);
-    a.q_out_row_stride = q_out.stride(0); a.q_out_head_stride = q_out.stride(1);
+    if (q_out.has_value()) {
+        thd(*q_out, "q_out");
+        a.q_out = mptr(*q_out);
+        a.q_out_row_stride = q_out->stride(0); a.q_out_head_stride = q_out->stride(1);
+    }
     if (v.has_value()) { thd(*v, "v"); a.v_row_stride = v->stride(0); a.v_head_stride = v->stride(1); }
     a.q_weight = ptr(q_weight); a.k_weight = ptr(k_weight); a.cos = ptr(cos); a.sin = ptr(sin);
     a.cos_sin_row_stride = cos.stride(0);
@@ -441,7 +465,48 @@ void qk_prep(const Tensor& q, const Tensor& k, const optional<Tensor>& v, const 
         a.norm_cols = (int32_t)norm_input->size(1);
         a.norm_eps = (float)norm_eps;
     }
+    return a;
+}
+
+// q/k RMSNorm + rotary (+ append): returns nothing, the caller allocated q_out / k_out.
+void qk_prep(const Tensor& q, const Tensor& k, const optional<Tensor>& v, const Tensor& q_out, const optional<Tensor>& k_out,
+             const Tensor& q_weight, const Tensor& k_weight, const Tensor& cos, const Tensor& sin, double eps,
+             const optional<Tensor>& ck, const optional<Tensor>& cv, const optional<Tensor>& cpos, const optional<Tensor>& start,
+             const optional<Tensor>& len, const optional<Tensor>& overflow, const optional<Tensor>& cu_new,
+             const optional<Tensor>& pos_new, const optional<Tensor>& slot_of, bool one_row_per_seq,
+             const optional<Tensor>& v_out, const optional<Tensor>& norm_input, double norm_eps) {
+    need_lib();
+    Dev d;
+    const tah_qk_prep_args a = prep_args(d, q, k, v, q_out, k_out, q_weight, k_weight, cos, sin, eps, ck, cv, cpos, start, len, overflow,
+                                         cu_new, pos_new, slot_of, one_row_per_seq, v_out, norm_input, norm_eps);
     check_rc(g.qk_prep(&a, d.stream()), "tah_qk_prep");
+}
+
+bool duo_decode_step_supported(int64_t nq, int64_t hq, int64_t hkv, int64_t capacity1) {
+    need_lib();
+    return g.decode_step_supported((int32_t)nq, (int32_t)hq, (int32_t)hkv, (int32_t)capacity1) != 0;
+}
+
+// qk_prep (append, one row per sequence) + duo_decode in one launch (tah_duo_decode_step).  The slabs the new K/V go to
+// (ck, cv, ...) must be those of one of the two segments read.
+void duo_decode_step(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor& q_weight, const Tensor& k_weight,
+                     const Tensor& cos, const Tensor& sin, double eps, const Tensor& ck, const Tensor& cv,
+                     const optional<Tensor>& cpos, const Tensor& start, const Tensor& len, const optional<Tensor>& overflow,
+                     const Tensor& cu_new, const optional<Tensor>& pos_new, const optional<Tensor>& slot_of,
+                     const optional<Tensor>& norm_input, double norm_eps, const Tensor& append_at,
+                     const Tensor& o, const optional<Tensor>& lse, const Tensor& q_slot, const Tensor& q_pos,
+                     const optional<Tensor>& q_depth, int64_t depth, const Tensor& k1, const Tensor& v1, const Tensor& start1,
+                     const Tensor& len1, const optional<Tensor>& k2, const optional<Tensor>& v2, const optional<Tensor>& pos2,
+                     const optional<Tensor>& start2, const optional<Tensor>& len2, double scale, const optional<Tensor>& o_packed) {
+    need_lib();
+    Dev d; d.see(append_at);
+    i32(append_at, "append_at");
+    TORCH_CHECK(append_at.numel() == q.size(0), "duo_decode_step: append_at must have one entry per row");
+    const tah_qk_prep_args pa = prep_args(d, q, k, v, c10::nullopt, c10::nullopt, q_weight, k_weight, cos, sin, eps, ck, cv, cpos, start, len,
+                                          overflow, cu_new, pos_new, slot_of, true, c10::nullopt, norm_input, norm_eps);
+    const tah_duo_decode_args da = decode_args(d, c10::nullopt, o, lse, q_slot, q_pos, q_depth, depth, k1, v1, start1, len1, k2, v2, pos2,
+                                               start2, len2, scale, o_packed);
+    check_rc(g.decode_step(&pa, &da, static_cast<const int32_t*>(append_at.data_ptr()), d.stream()), "tah_duo_decode_step");
 }
 
 std::tuple<Tensor, Tensor, Tensor, Tensor> hard_index_build(const Tensor& mask) {
@@ -662,6 +727,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("rows_copy", &rows_copy);
     m.def("topk_mix", &topk_mix);
     m.def("silu_mul", &silu_mul);
+    m.def("duo_decode_step", &duo_decode_step);
+    m.def("duo_decode_step_supported", &duo_decode_step_supported);
     m.def("linear_pack_weight", &linear_pack_weight);
     m.def("linear_pack_rows", &linear_pack_rows);
     m.def("linear_rows", &linear_rows);

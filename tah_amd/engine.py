@@ -39,7 +39,7 @@ import torch.nn.functional as F
 
 from . import ops
 from ._capi import TahDuoError
-from .kv_cache import KvSlabs, decode as _decode, qk_norm_rope
+from .kv_cache import KvSlabs, decode as _decode, decode_step as _decode_step, decode_step_supported, qk_norm_rope
 
 
 @dataclasses.dataclass
@@ -208,6 +208,11 @@ class TaHDecodeEngine:
         self._graph = None
         self.static_scratch = self.device.type == "cuda"
         self.measure_without_attention = False
+        # depth-1 rows every sequence has cached (what each slabs1[l].len holds), kept once for the fused step kernel
+        self.hard_len = torch.zeros(batch, dtype=torch.int32, device=dev)
+        # q/k preparation, append and attention of a layer in one launch where the library takes the sizes
+        self.fused_step = bool(self.packed_linear and self.device.type == "cuda"
+                               and decode_step_supported(batch, cfg.hq, cfg.hkv, max_len))
         if self.packed_linear:  # rows operands handed from kernel to kernel (32 rows each; rows past the batch stay zero)
             z = lambda n: torch.zeros(32 * n, dtype=torch.bfloat16, device=dev)
             self.xp, self.op, self.actp = z(cfg.hidden), z(cfg.hq * cfg.head_dim), z(cfg.intermediate)
@@ -290,6 +295,12 @@ class TaHDecodeEngine:
             cache = self.slabs0[l] if depth == 0 else self.slabs1[l]
             if self.measure_without_attention:  # timing aid: the step minus its q/k preparation and decode kernels
                 ops.linear_pack_rows(q.reshape(B, n_o), out=self.op)
+            elif self.fused_step:
+                _decode_step(q, k, v, L["qn"], L["kn"], cos, sin, c.rms_eps, cache=cache, cu_new=self.cu_rows,
+                             append_at=pos if depth == 0 else self.hard_len, q_slot=self.rows, q_pos=q_pos,
+                             c1=self.slabs0[l], c2=self.slabs1[l], scale=self.scale, slot_of=slot_of,
+                             pos_new=pos if depth == 1 else None, norm_input=x, norm_eps=c.rms_eps, q_depth=q_depth,
+                             out_packed=self.op)
             else:
                 qo, _ = qk_norm_rope(q, k, L["qn"], L["kn"], cos, sin, c.rms_eps, v=v, cache=cache, cu_new=self.cu_rows,
                                      slot_of=slot_of, pos_new=pos if depth == 1 else None, one_row_per_seq=True,
@@ -342,7 +353,9 @@ class TaHDecodeEngine:
         x1 = ops.topk_mix(l0, self.w.embed, self.cfg.topk, row_enable=hard)
         slot1 = torch.where(hard, self.rows, self.minus1)
         qpos1 = torch.where(hard, pos, self.minus1)
-        h1 = self._pass_single(x1, pos, 1, slot1, qpos1, hard.to(torch.int32), rope)
+        hard_i = hard.to(torch.int32)
+        h1 = self._pass_single(x1, pos, 1, slot1, qpos1, hard_i, rope)
+        self.hard_len += hard_i  # after all layers appended at the old count
         return l0, self._head(h1), hard
 
     # ── prefill: packed prompts, both depths, through the varlen kernels ──
@@ -414,6 +427,7 @@ class TaHDecodeEngine:
                 logits_last[which] = both[is_last]
             self.host_hard_rows = int(counts.max())
         self.pos.copy_(torch.tensor(lens, dtype=torch.int32))
+        self.hard_len.copy_(self.slabs1[0].len)
         self.host_positions = max(lens)
         self.finished.zero_()
         return logits_last.float(), hard
@@ -470,7 +484,8 @@ class TaHDecodeEngine:
         self.tok.copy_(nxt)
 
     def _state(self):
-        return (self.tok, self.pos, self.finished, self.n_hard, self.n_steps, self.step_idx, self.out_tokens, self.out_len)
+        return (self.tok, self.pos, self.finished, self.n_hard, self.n_steps, self.step_idx, self.out_tokens, self.out_len,
+                self.hard_len)
 
     @torch.no_grad()
     def generate(self, first_logits: torch.Tensor, max_new_tokens: int, *, temperature: float = 0.0, eos: int = -1,

@@ -86,6 +86,37 @@ def qk_norm_rope(q: torch.Tensor, k: torch.Tensor, q_weight: torch.Tensor, k_wei
 _WORKSPACES = {}
 
 
+def decode_step_supported(nq: int, hq: int, hkv: int, capacity1: int) -> bool:
+    """Whether :func:`decode_step` takes a call of these sizes (``tah_duo_decode_step_supported``)."""
+    return bool(_call("duo_decode_step_supported", int(nq), int(hq), int(hkv), int(capacity1)))
+
+
+def decode_step(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_weight: torch.Tensor, k_weight: torch.Tensor,
+                cos: torch.Tensor, sin: torch.Tensor, eps: float, *, cache: KvSlabs, cu_new: torch.Tensor,
+                append_at: torch.Tensor, q_slot: torch.Tensor, q_pos: torch.Tensor, c1: KvSlabs, c2: Optional[KvSlabs],
+                scale: float, slot_of: Optional[torch.Tensor] = None, pos_new: Optional[torch.Tensor] = None,
+                norm_input: Optional[torch.Tensor] = None, norm_eps: float = 0.0, depth: int = 0,
+                q_depth: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+                out_packed: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``qk_norm_rope(..., cache=cache, one_row_per_seq=True)`` followed by ``decode(...)`` in one launch
+    (``tah_duo_decode_step``), for a generation step: q ``[B, Hq, 128]``, k / v ``[B, Hkv, 128]`` are the projections
+    of one new token per sequence, ``cache`` (``c1`` or ``c2``) receives the prepared K and V, and row i attends as
+    query i.  ``append_at`` int32 [B]: the rows sequence i's segment of ``cache`` holds before the call (the caller's
+    own copy of ``cache.len``: the kernel cannot read the lengths while it advances them).  Same cache contents and
+    lengths as the two calls, bit for bit, and the same outputs up to the last bit of a rare element.  Only for sizes :func:`decode_step_supported` accepts."""
+    if q.dim() != 3:
+        raise _capi.TahDuoError("decode_step: q must be [B, Hq, D]")
+    need2 = q_depth is not None or depth >= 1
+    if need2 and c2 is None:
+        raise _capi.TahDuoError("depth-1 queries need the depth-1 cache")
+    o = out if out is not None else torch.empty_like(q)
+    two = (c2.k, c2.v, c2.pos, c2.start, c2.len) if need2 else (None,) * 5
+    _call("duo_decode_step", q, k, v, q_weight, k_weight, cos, sin, float(eps), cache.k, cache.v, cache.pos, cache.start,
+          cache.len, cache.overflow, cu_new, pos_new, slot_of, norm_input, float(norm_eps), append_at,
+          o, None, q_slot, q_pos, q_depth, int(depth), c1.k, c1.v, c1.start, c1.len, *two, float(scale), out_packed)
+    return o
+
+
 def decode(q: torch.Tensor, q_slot: torch.Tensor, q_pos: torch.Tensor, c1: KvSlabs, c2: Optional[KvSlabs], *,
            scale: float, depth: int = 0, q_depth: Optional[torch.Tensor] = None, return_lse: bool = False,
            out: Optional[torch.Tensor] = None, lse_out: Optional[torch.Tensor] = None, static_scratch: bool = False,

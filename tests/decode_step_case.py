@@ -1,0 +1,78 @@
+"""One generation step's attention, fused (tah_duo_decode_step) against the two calls it replaces (tah_qk_prep with
+append + tah_duo_decode): cache contents, positions and lengths have to agree bit for bit; the outputs as well, up to
+the last bit of a rare element (same arithmetic in the same order, but two kernels: the compiler may contract a
+multiply and an add into one instruction in one of them and not in the other)."""
+import copy
+
+import torch
+
+BF = torch.bfloat16
+
+
+def _slabs(B, cap, hkv, lens, with_pos, g, dev):
+    from tah_amd.kv_cache import KvSlabs
+    s = KvSlabs(B, cap, hkv, 128, with_pos=with_pos, device=dev)
+    s.k.copy_(torch.randn(s.k.shape, generator=g).to(BF))
+    s.v.copy_(torch.randn(s.v.shape, generator=g).to(BF))
+    s.len.copy_(torch.tensor(lens, dtype=torch.int32))
+    return s
+
+
+def run(dev, *, B, hq, hkv, seed=0, max_len=90, hidden=256, cap1=128, cap2=64):
+    from tah_amd import kv_cache
+    g = torch.Generator().manual_seed(seed)
+    lens1 = torch.randint(1, max_len, (B,), generator=g).tolist()
+    lens2 = [int(torch.randint(0, min(l, cap2 - 1) + 1, (1,), generator=g)) for l in lens1]
+    c1 = _slabs(B, cap1, hkv, lens1, False, g, dev)
+    c2 = _slabs(B, cap2, hkv, lens2, True, g, dev)
+    for b in range(B):  # depth-1 rows sit at increasing positions below the sequence's length
+        c2.pos[b, :lens2[b]] = torch.sort(torch.randperm(lens1[b], generator=g)[:lens2[b]]).values.to(torch.int32)
+    rn = lambda *s: torch.randn(*s, generator=g).to(BF).to(dev)
+    q, k, v = rn(B, hq, 128) * 3, rn(B, hkv, 128) * 3, rn(B, hkv, 128)
+    qw, kw = (1 + 0.1 * torch.randn(128, generator=g)).to(BF).to(dev), (1 + 0.1 * torch.randn(128, generator=g)).to(BF).to(dev)
+    x = rn(B, hidden) * 2
+    rows = torch.arange(B, dtype=torch.int32, device=dev)
+    cu = torch.arange(B + 1, dtype=torch.int32, device=dev)
+    pos = torch.tensor(lens1, dtype=torch.int32, device=dev)
+    ang = torch.randn(B, 128, generator=g)
+    cos, sin = ang.cos().to(BF).to(dev), ang.sin().to(BF).to(dev)
+    active = torch.ones(B, dtype=torch.bool)
+    active[B // 3] = False        # a finished row: not cached, sees nothing
+    hard = torch.rand(B, generator=g) < 0.4
+    hard[0], hard[B // 3] = True, False
+    active, hard = active.to(dev), hard.to(dev)
+    minus1 = torch.full((B,), -1, dtype=torch.int32, device=dev)
+    scale = 128 ** -0.5
+    results = {}
+    for depth in (0, 1):
+        sel = active if depth == 0 else hard
+        slot_of = torch.where(sel, rows, minus1)
+        q_pos = torch.where(sel, pos, minus1)
+        q_depth = torch.zeros(B, dtype=torch.int32, device=dev) if depth == 0 else hard.to(torch.int32)
+        out = []
+        for fused in (False, True):
+            a1, a2 = copy.deepcopy(c1), copy.deepcopy(c2)
+            tgt = a1 if depth == 0 else a2
+            packed = torch.zeros(32 * hq * 128, dtype=BF, device=dev) if B <= 32 else None
+            common = dict(cache=tgt, cu_new=cu, slot_of=slot_of, pos_new=pos if depth == 1 else None, norm_input=x, norm_eps=1e-6)
+            if fused:
+                o = kv_cache.decode_step(q, k, v, qw, kw, cos, sin, 1e-6, append_at=tgt.len.clone(), q_slot=rows, q_pos=q_pos,
+                                         c1=a1, c2=a2, scale=scale, q_depth=q_depth, out_packed=packed, **common)
+            else:
+                qo, _ = kv_cache.qk_norm_rope(q, k, qw, kw, cos, sin, 1e-6, v=v, one_row_per_seq=True, **common)
+                o = kv_cache.decode(qo, rows, q_pos, a1, a2, scale=scale, q_depth=q_depth, out_packed=packed)
+            out.append((o, packed, a1, a2))
+        (oa, pa, a1, a2), (ob, pb, b1, b2) = out
+        assert torch.allclose(oa.float(), ob.float(), rtol=2.0 ** -7, atol=2.0 ** -12), f"depth {depth}: outputs differ"
+        assert (oa != ob).float().mean() < 1e-3, f"depth {depth}: more than a rare last bit differs"
+        from tests.test_linear_rows import unpack_rows
+        assert pb is None or torch.equal(unpack_rows(pb.cpu(), hq * 128)[:B], ob.cpu().reshape(B, -1))
+        for sa, sb in ((a1, b1), (a2, b2)):
+            assert torch.equal(sa.k, sb.k) and torch.equal(sa.v, sb.v) and torch.equal(sa.len, sb.len)
+            assert int(sa.overflow) == int(sb.overflow) == 0
+        assert torch.equal(a2.pos, b2.pos)
+        tgt_a, src = (a1, c1) if depth == 0 else (a2, c2)
+        assert torch.equal(tgt_a.len.cpu(), src.len.cpu() + sel.cpu().to(torch.int32))  # the step did append
+        assert oa[B // 3].abs().max() == 0                                              # the finished row saw nothing
+        results[depth] = oa
+    return results

@@ -79,3 +79,13 @@ def test_append_is_exact_and_flags_overflow():
         s.append(k[:3], v[:3], torch.tensor([0, 3], dtype=torch.int32), pos_new=pos[:3], slot_of=torch.tensor([0], dtype=torch.int32))
         assert s.len.tolist() == [5, 0, 2] and int(s.overflow) == 1
         assert torch.equal(s.k[0, :, 4], k[0])
+
+
+def test_fused_decode_step_equals_prep_then_decode_on_cpu_shim():
+    """16 (query, kv head) pairs: the CPU execution build takes such calls in one launch."""
+    from tests import decode_step_case
+    from tah_amd import kv_cache
+    with emu_util.emulated():
+        assert kv_cache.decode_step_supported(2, 16, 8, 128) and not kv_cache.decode_step_supported(1, 16, 8, 128)
+        assert not kv_cache.decode_step_supported(2, 32, 8, 128)  # four query heads per kv head
+        decode_step_case.run("cpu", B=3, hq=16, hkv=8, seed=5)

@@ -198,3 +198,45 @@ def test_generate_wrapper_returns_tokens_up_to_eos_gpu():
         stop = free[b].index(tok.eos_token_id) if tok.eos_token_id in free[b] else new
         assert cut[b] == free[b][:stop], b
     assert len(cut[0]) <= 5
+
+
+@pytest.mark.gpu
+def test_engine_with_fused_layer_attention_equals_the_separate_launches_gpu():
+    """32 sequences x 8 kv heads: the engine runs q/k preparation, append and attention of a layer in one launch
+    (tah_duo_decode_step).  Driven with the same tokens and hard decisions, it gives the logits of the separate
+    launches (to the last bits of bf16: the two kernels are compiled separately) and exactly their cache lengths; its
+    captured step gives exactly the tokens of its eager step."""
+    from tah_amd.engine import EngineConfig, TaHDecodeEngine, Weights
+    cfg = EngineConfig(hidden=256, layers=2, hq=16, hkv=8, head_dim=128, intermediate=768, vocab=4096, decider_hidden=32)
+    w = Weights.random_init(cfg, "cuda", seed=6)
+    B, T, steps = 32, 21, 5
+    g = torch.Generator().manual_seed(10)
+    ids = torch.randint(0, cfg.vocab, (B * T,), generator=g).cuda()
+    toks = torch.randint(0, cfg.vocab, (steps, B), generator=g).cuda()
+    hards = (torch.rand(steps, B, generator=g) < 0.3).cuda()
+    hards[1], hards[2] = False, True
+    cu = torch.arange(0, B * T + 1, T, dtype=torch.int32, device="cuda")
+    runs = []
+    for fused in (False, True):
+        eng = TaHDecodeEngine(w, B, T + steps + 12, device="cuda")
+        assert eng.fused_step and eng.packed_linear
+        eng.fused_step = fused
+        eng.prefill(ids, cu, calibrate=0.2)
+        logits = []
+        for s in range(steps):
+            got, h = eng.step_logits(toks[s], force_hard=hards[s])
+            eng.pos += 1
+            logits.append(got)
+        runs.append((logits, [sl.len.tolist() for sl in eng.slabs0 + eng.slabs1], eng.hard_len.tolist()))
+    for a, b in zip(runs[0][0], runs[1][0]):
+        assert (a - b).abs().max().item() <= 2e-2 * max(a.abs().max().item(), 1.0)
+    assert runs[0][1:] == runs[1][1:]
+    assert runs[1][2] == runs[1][1][cfg.layers]  # the engine's own count of depth-1 rows is what the slabs hold
+    # the fused step under the graph: the tokens of its eager run
+    out = []
+    for use_graph in (False, True):
+        eng = TaHDecodeEngine(w, B, T + 12, device="cuda")
+        first, _ = eng.prefill(ids, cu, calibrate=0.2)
+        out.append((eng.generate(first, 10, eos=7, use_graph=use_graph).clone(), int(eng.n_hard), eng.hard_len.tolist(),
+                    [sl.len.tolist() for sl in eng.slabs0 + eng.slabs1]))
+    assert torch.equal(out[0][0], out[1][0]) and out[0][1:] == out[1][1:] and out[0][1] > 0

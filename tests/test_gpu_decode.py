@@ -119,3 +119,14 @@ def test_decode_rejects_small_workspace_and_bad_shapes():
     a.d = 128
     assert lib.tah_duo_decode(ctypes.byref(a), None) == -1
     assert lib.tah_duo_decode_workspace_bytes(64, 16, 16384, 2048) == 64 * 16 * (16 + 2) * 130 * 4
+
+
+@pytest.mark.parametrize("B,hq,hkv", [(32, 16, 8), (40, 8, 8), (64, 8, 4)])
+def test_fused_decode_step_equals_prep_then_decode(B, hq, hkv):
+    """tah_duo_decode_step against tah_qk_prep + tah_duo_decode: bit for bit (outputs, cache rows, positions, lengths)."""
+    from tests import decode_step_case
+    from tah_amd import kv_cache
+    print(f"fused decode step B={B} hq={hq} hkv={hkv}", flush=True)
+    assert kv_cache.decode_step_supported(B, hq, hkv, 4096) and not kv_cache.decode_step_supported(B, hq, hkv, 4097)
+    assert not kv_cache.decode_step_supported(B, 4 * hkv, hkv, 4096)  # four query heads per kv head: the two calls
+    decode_step_case.run("cuda", B=B, hq=hq, hkv=hkv, seed=B + hq, max_len=3000, hidden=2048, cap1=4096, cap2=1024)
