@@ -355,7 +355,7 @@ def bench_e2e_decode(new_tokens: int, B: int = 32, prompt_len: int = 512):
             "hard_fraction_decode": frac_hard, "hard_fraction_prompt": float(hard.float().mean()),
             "attention_ms_per_step": attn_ms, "attention_share_of_step": attn_ms / step_ms,
             "step_ms_without_attention_kernels": without_ms,
-            "attention_kernels": "qk_prep_kernel + duo_decode_whole_kernel<2>, 28 layers x 2 iterations",
+            "attention_kernels": "duo_decode_step_kernel<2> (q/k preparation + append + attention), 28 layers x 2 iterations",
             "attention_cache_bytes_per_step": attn_bytes, "attention_cache_gbs": attn_bytes / (attn_ms * 1e-3) / 1e9,
             "host_enqueue_ms_per_replay": sorted(enqueue)[n_enqueue // 2] * 1e3, "host_ms_per_step_in_loop": host_s / n * 1e3,
             "eager_ms_per_step": eager_s * 1e3,
