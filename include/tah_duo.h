@@ -300,9 +300,12 @@ typedef struct tah_topk_mix_args {
     const void* logits;        /* bf16 [rows, vocab], vocab contiguous */
     const void* embedding;     /* bf16 [vocab, hidden], 16-byte aligned rows */
     void* out;                 /* bf16 [rows, hidden] */
-    const uint8_t* row_enable; /* optional, one byte per row: rows whose byte is 0 are skipped (out untouched) */
+    const uint8_t* row_enable; /* optional, one byte per row: rows whose byte is 0 are skipped (out untouched, or zeroed) */
     int64_t logits_row_stride, embedding_row_stride, out_row_stride; /* elements */
     int32_t rows, vocab, hidden, topk; /* topk <= 256, vocab <= 155648, hidden a multiple of 8 */
+    void* out_packed;          /* optional: the rows once more as the rows operand of tah_linear_rows, bf16 [32 * hidden]
+                                * (rows <= 32, hidden % 32 == 0; rows past `rows` are not touched) */
+    int32_t zero_disabled;     /* != 0: rows whose row_enable byte is 0 are written as zeros instead of left alone */
 } tah_topk_mix_args;
 
 /* Next-iteration input of hard tokens: softmax over each row's top-k logits, then the probability-weighted
@@ -373,11 +376,14 @@ typedef struct tah_linear_rows_args {
                                * is needed */
     int64_t residual_row_stride, out_row_stride; /* elements */
     int32_t rows, n, k;       /* rows <= 32 */
-    int32_t kind;             /* TAH_LINEAR_PLAIN: out = bf16(r x W^T) [+ residual]
+    int32_t kind;             /* TAH_LINEAR_PLAIN: out = bf16(r x W^T) [+ bias] [+ residual] [relu]
                                * TAH_LINEAR_GATE_UP: out = bf16(silu(g)) * u, g = bf16(r x Wg^T), u = bf16(r x Wu^T) */
     int32_t input_norm;       /* 1: r = rsqrt(mean(x[row]^2) + norm_eps), an RMSNorm of the rows whose weight is already
                                * inside W (the MLP's input norm for gate|up, the final norm for an output head); 0: r = 1 */
     float norm_eps;
+    const void* bias;         /* TAH_LINEAR_PLAIN: bf16 [n] added to the product (after its rounding to bf16, before the
+                               * residual), or NULL */
+    int32_t relu;             /* TAH_LINEAR_PLAIN: != 0: max(., 0) last (a two-layer MLP's first layer) */
 } tah_linear_rows_args;
 int tah_linear_rows(const tah_linear_rows_args* args, tah_stream_t stream);
 
@@ -405,6 +411,53 @@ typedef struct tah_greedy_step_args {
     int64_t* n_steps;         /* += rows that decoded */
 } tah_greedy_step_args;
 int tah_greedy_step(const tah_greedy_step_args* args, tah_stream_t stream);
+
+/* Start of a generation step (one token per sequence), in one launch: for row i, active[i] = !finished[i]; slot[i] = i
+ * and q_pos[i] = pos[i] for active rows, -1 for finished ones (nothing cached, nothing seen); the rotary rows of
+ * position pos[i] (clamped into the tables); and the embedding row of tok[i], row-major and, when x_packed is given
+ * (rows <= 32, hidden % 32 == 0), in the rows form of tah_linear_rows (rows past `rows` are not touched).  Replaces the
+ * embed_tokens lookup of the base model and the rotary lookup (Qwen3Model.forward / Qwen3RotaryEmbedding, third party)
+ * for the generation loop of tah/model/utils.py:228-262, plus the masks a fixed-shape step needs. */
+typedef struct tah_step_begin_args {
+    const int64_t* tok;       /* [rows] */
+    const int32_t* pos;       /* [rows] */
+    const uint8_t* finished;  /* [rows] */
+    const void* embed;        /* bf16 [vocab, hidden] */
+    int64_t embed_row_stride;
+    const void* cos_table;    /* bf16 [table_rows, 128] */
+    const void* sin_table;
+    int32_t rows, vocab, hidden, table_rows;
+    void* x;                  /* bf16 [rows, hidden] out */
+    int64_t x_row_stride;
+    void* x_packed;           /* bf16 [32 * hidden] out, or NULL */
+    void* cos_rows;           /* bf16 [rows, 128] out */
+    void* sin_rows;
+    int32_t* slot;            /* [rows] out */
+    int32_t* q_pos;           /* [rows] out */
+    uint8_t* active;          /* [rows] out */
+} tah_step_begin_args;
+int tah_step_begin(const tah_step_begin_args* args, tah_stream_t stream);
+
+/* Second layer of a two-layer decider MLP and the decision, in one launch: hard[i] = sigmoid(bf16(bf16(hidden[i] . w2) +
+ * b2)) > threshold and active[i] (the roundings of the eager `h @ w2.T + b2` in bf16, then .float().sigmoid()), and for
+ * the second latent iteration hard_i32[i] (0/1), slot[i] = i and q_pos[i] = pos[i] for hard rows, -1 otherwise (each
+ * optional).  The first layer is a tah_linear_rows call with bias and relu.  The decider of the end-to-end workload
+ * (hidden -> 512 -> 1); the reference's MLPIterDecider (tah/model/iter_decider.py:193-301) is a larger network. */
+typedef struct tah_decider_tail_args {
+    const void* hidden;       /* bf16 [rows, width], after the first layer's ReLU */
+    int64_t hidden_row_stride;
+    const void* w2;           /* bf16 [width] */
+    const void* b2;           /* bf16 [1] or NULL */
+    float threshold;
+    int32_t rows, width;      /* width % 8 == 0 */
+    const uint8_t* active;    /* [rows] or NULL (all) */
+    const int32_t* pos;       /* [rows]; needed with q_pos */
+    uint8_t* hard;            /* [rows] out */
+    int32_t* hard_i32;        /* [rows] out or NULL */
+    int32_t* slot;            /* [rows] out or NULL */
+    int32_t* q_pos;           /* [rows] out or NULL */
+} tah_decider_tail_args;
+int tah_decider_tail(const tah_decider_tail_args* args, tah_stream_t stream);
 
 /* Hard-token index build: stream compaction of a (B, S) byte mask in row-major
  * order.  Replaces the stable sort + nonzero of gather_active / scatter_back

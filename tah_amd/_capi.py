@@ -115,6 +115,29 @@ class LinearRowsArgs(C.Structure):
         ("w_packed", c_void_p), ("x_packed", c_void_p), ("residual", c_void_p), ("out", c_void_p), ("out_packed", c_void_p),
         ("residual_row_stride", c_int64), ("out_row_stride", c_int64),
         ("rows", c_int32), ("n", c_int32), ("k", c_int32), ("kind", c_int32), ("input_norm", c_int32), ("norm_eps", c_float),
+        ("bias", c_void_p), ("relu", c_int32),
+    ]
+
+
+class StepBeginArgs(C.Structure):
+    """``tah_step_begin_args``"""
+
+    _fields_ = [
+        ("tok", c_void_p), ("pos", c_void_p), ("finished", c_void_p), ("embed", c_void_p), ("embed_row_stride", c_int64),
+        ("cos_table", c_void_p), ("sin_table", c_void_p),
+        ("rows", c_int32), ("vocab", c_int32), ("hidden", c_int32), ("table_rows", c_int32),
+        ("x", c_void_p), ("x_row_stride", c_int64), ("x_packed", c_void_p), ("cos_rows", c_void_p), ("sin_rows", c_void_p),
+        ("slot", c_void_p), ("q_pos", c_void_p), ("active", c_void_p),
+    ]
+
+
+class DeciderTailArgs(C.Structure):
+    """``tah_decider_tail_args``"""
+
+    _fields_ = [
+        ("hidden", c_void_p), ("hidden_row_stride", c_int64), ("w2", c_void_p), ("b2", c_void_p), ("threshold", c_float),
+        ("rows", c_int32), ("width", c_int32), ("active", c_void_p), ("pos", c_void_p), ("hard", c_void_p),
+        ("hard_i32", c_void_p), ("slot", c_void_p), ("q_pos", c_void_p),
     ]
 
 
@@ -177,6 +200,7 @@ class TopkMixArgs(C.Structure):
         ("logits", c_void_p), ("embedding", c_void_p), ("out", c_void_p), ("row_enable", c_void_p),
         ("logits_row_stride", c_int64), ("embedding_row_stride", c_int64), ("out_row_stride", c_int64),
         ("rows", c_int32), ("vocab", c_int32), ("hidden", c_int32), ("topk", c_int32),
+        ("out_packed", c_void_p), ("zero_disabled", c_int32),
     ]
 
 
@@ -195,6 +219,8 @@ PROTOTYPES = {
     "tah_duo_decode_workspace_bytes": (C.c_size_t, [c_int32, c_int32, c_int32, c_int32]),
     "tah_duo_decode": (C.c_int, [C.POINTER(DuoDecodeArgs), c_void_p]),
     "tah_duo_decode_static": (C.c_int, [C.POINTER(DuoDecodeArgs), c_void_p]),
+    "tah_step_begin": (C.c_int, [C.POINTER(StepBeginArgs), c_void_p]),
+    "tah_decider_tail": (C.c_int, [C.POINTER(DeciderTailArgs), c_void_p]),
     "tah_linear_pack_weight": (C.c_int, [c_void_p, c_int64, c_void_p, c_int32, c_int32, c_int32, c_void_p]),
     "tah_linear_pack_rows": (C.c_int, [c_void_p, c_int64, c_void_p, c_int32, c_int32, c_void_p]),
     "tah_linear_rows": (C.c_int, [C.POINTER(LinearRowsArgs), c_void_p]),

@@ -44,6 +44,8 @@ struct LinParams {
     const bf16x8* w;   // packed weight
     const bf16x8* x;   // packed rows
     const __bf16* res; // row-major residual or null
+    const __bf16* bias; // [n] added to the product (rounded to bf16 first, as a GEMM's output is) or null
+    int32_t relu;
     __bf16* y;         // row-major result or null
     bf16x8* yp;        // packed result or null
     int64_t res_rs, y_rs;
@@ -243,13 +245,23 @@ __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(const LinParam
                 const float g = (float)(__bf16)(sg[i] * rin), u = (float)(__bf16)(su[i] * rin);
                 out[i] = (__bf16)((float)(__bf16)silu_f(g) * u);
             }
-        } else if (p.res) {
-            const bf16x8 rv = *reinterpret_cast<const bf16x8*>(p.res + (int64_t)row * p.res_rs + n0);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) out[i] = (__bf16)((float)(__bf16)(sg[i] * rin) + (float)rv[i]);
         } else {
 #pragma unroll
             for (int i = 0; i < 8; ++i) out[i] = (__bf16)(sg[i] * rin);
+            if (p.bias) {
+                const bf16x8 bv = *reinterpret_cast<const bf16x8*>(p.bias + n0);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) out[i] = (__bf16)((float)out[i] + (float)bv[i]);
+            }
+            if (p.res) {
+                const bf16x8 rv = *reinterpret_cast<const bf16x8*>(p.res + (int64_t)row * p.res_rs + n0);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) out[i] = (__bf16)((float)out[i] + (float)rv[i]);
+            }
+            if (p.relu) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) out[i] = (float)out[i] > 0.f ? out[i] : (__bf16)0.f;
+            }
         }
         if (p.y) *reinterpret_cast<bf16x8*>(p.y + (int64_t)row * p.y_rs + n0) = out;
     }
@@ -352,11 +364,12 @@ extern "C" int tah_linear_rows(const tah_linear_rows_args* a, tah_stream_t strea
     const bool gate_up = a->kind == TAH_LINEAR_GATE_UP;
     const bool g24 = gate_up && a->n % kGroup24 == 0;
     if (!g24 && a->n % kTileCols != 0) return TAH_E_SHAPE;
-    if (gate_up && a->residual) return TAH_E_SHAPE;
+    if (gate_up && (a->residual || a->bias || a->relu)) return TAH_E_SHAPE;
     if (a->out_packed && a->n % kStepK != 0) return TAH_E_SHAPE;  // the packed rows form holds whole steps of 32 columns
     if (a->n == 0 || a->k == 0 || (a->rows == 0 && !a->out_packed)) return TAH_OK;
     if (!a->w_packed || !a->x_packed || (!a->out && !a->out_packed)) return TAH_E_NULL;
     if (!aligned16(a->w_packed) || !aligned16(a->x_packed) || !aligned16(a->out) || !aligned16(a->out_packed) || !aligned16(a->residual) ||
+        !aligned16(a->bias) ||
         (a->out && a->out_row_stride % 8 != 0) || (a->residual && a->residual_row_stride % 8 != 0))
         return TAH_E_ALIGN;
     if ((a->out && a->out_row_stride < a->n) || (a->residual && a->residual_row_stride < a->n)) return TAH_E_SHAPE;
@@ -364,6 +377,8 @@ extern "C" int tah_linear_rows(const tah_linear_rows_args* a, tah_stream_t strea
     p.w = static_cast<const bf16x8*>(a->w_packed);
     p.x = static_cast<const bf16x8*>(a->x_packed);
     p.res = static_cast<const __bf16*>(a->residual);
+    p.bias = static_cast<const __bf16*>(a->bias);
+    p.relu = a->relu ? 1 : 0;
     p.y = static_cast<__bf16*>(a->out);
     p.yp = static_cast<bf16x8*>(a->out_packed);
     p.res_rs = a->residual_row_stride;

@@ -168,6 +168,84 @@ __global__ __launch_bounds__(kGreedyThreads) void greedy_step_kernel(const Greed
     p.tok[row] = nxt;
 }
 
+
+// ---------------------------------------------------------------------------
+// Glue of a generation step that would otherwise be a dozen element-wise launches each.
+// step_begin: per row, whether it is still active, the cache slot and position it appends and attends at (-1 for
+// finished rows), the rotary rows of its position, and its token's embedding row, row-major and in the rows form
+// of the linear-layer kernels.  decider_tail: the second layer of the two-layer decider (width -> 1), sigmoid,
+// threshold, and the same per-row bookkeeping for the second latent iteration.
+// ---------------------------------------------------------------------------
+struct StepBeginParams {
+    const int64_t* tok;
+    const int32_t* pos;
+    const uint8_t* finished;
+    const __bf16 *embed, *cos_table, *sin_table;
+    int64_t embed_rs;
+    int32_t vocab, hidden, table_rows;
+    __bf16 *x, *x_packed, *cos_rows, *sin_rows;
+    int64_t x_rs;
+    int32_t *slot, *q_pos;
+    uint8_t* active;
+};
+
+__global__ __launch_bounds__(256) void step_begin_kernel(const StepBeginParams p) {
+    const int row = blockIdx.x, tid = threadIdx.x;
+    const bool act = p.finished[row] == 0;
+    const int pos = p.pos[row];
+    if (tid == 0) {
+        p.slot[row] = act ? row : -1;
+        p.q_pos[row] = act ? pos : -1;
+        p.active[row] = act ? 1 : 0;
+    }
+    const int at = pos < 0 ? 0 : (pos >= p.table_rows ? p.table_rows - 1 : pos);  // a position past the tables reads their last row
+    if (tid < 16) *reinterpret_cast<u32x4*>(p.cos_rows + (int64_t)row * 128 + 8 * tid) = *reinterpret_cast<const u32x4*>(p.cos_table + (int64_t)at * 128 + 8 * tid);
+    else if (tid < 32) *reinterpret_cast<u32x4*>(p.sin_rows + (int64_t)row * 128 + 8 * (tid - 16)) = *reinterpret_cast<const u32x4*>(p.sin_table + (int64_t)at * 128 + 8 * (tid - 16));
+    int64_t t = p.tok[row];
+    t = t < 0 ? 0 : (t >= p.vocab ? p.vocab - 1 : t);
+    const __bf16* e = p.embed + t * p.embed_rs;
+    for (int c = 8 * tid; c < p.hidden; c += 8 * 256) {
+        const u32x4 v = *reinterpret_cast<const u32x4*>(e + c);
+        *reinterpret_cast<u32x4*>(p.x + (int64_t)row * p.x_rs + c) = v;
+        // unit (step c / 32, half row / 16, lane row % 16 + 16 ((c % 32) / 8)) of the packed rows form
+        if (p.x_packed) reinterpret_cast<u32x4*>(p.x_packed)[((int64_t)(c / 32) * 2 + row / 16) * 64 + (row % 16) + 16 * ((c % 32) / 8)] = v;
+    }
+}
+
+struct DeciderTailParams {
+    const __bf16 *h, *w2, *b2;
+    int64_t h_rs;
+    int32_t width;
+    float threshold;
+    const uint8_t* active;
+    const int32_t* pos;
+    uint8_t* hard;
+    int32_t *hard_i, *slot, *q_pos;
+};
+
+// One wave per row.  z = bf16(h . w2) (float32 sum), + b2 in bf16, sigmoid in float32, > threshold, and active.
+__global__ __launch_bounds__(64) void decider_tail_kernel(const DeciderTailParams p) {
+    const int row = blockIdx.x, lane = threadIdx.x;
+    float s = 0.f;
+    for (int c = 8 * lane; c < p.width; c += 8 * 64) {
+        const u32x4 a = *reinterpret_cast<const u32x4*>(p.h + (int64_t)row * p.h_rs + c);
+        const u32x4 b = *reinterpret_cast<const u32x4*>(p.w2 + c);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) s += lo_f(a[q]) * lo_f(b[q]) + hi_f(a[q]) * hi_f(b[q]);
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) s += __shfl_xor(s, m);
+    if (lane != 0) return;
+    float z = lo_f(pack2(s, 0.f));
+    if (p.b2) z = lo_f(pack2(z + (float)p.b2[0], 0.f));
+    const float prob = 1.0f / (1.0f + fast_exp2(-z * kLog2e));
+    const bool hard = prob > p.threshold && (p.active == nullptr || p.active[row] != 0);
+    p.hard[row] = hard ? 1 : 0;
+    if (p.hard_i) p.hard_i[row] = hard ? 1 : 0;
+    if (p.slot) p.slot[row] = hard ? row : -1;
+    if (p.q_pos) p.q_pos[row] = hard ? p.pos[row] : -1;
+}
+
 }  // namespace
 }  // namespace tah
 
@@ -221,4 +299,44 @@ extern "C" int tah_silu_mul_normed(const void* gate_up, void* out, int32_t rows,
 extern "C" int tah_silu_mul(const void* gate_up, void* out, int32_t rows, int32_t inter, int64_t gate_up_row_stride,
                             int64_t out_row_stride, tah_stream_t stream) {
     return tah_silu_mul_normed(gate_up, out, rows, inter, gate_up_row_stride, out_row_stride, nullptr, 0, 0, 0.f, stream);
+}
+
+extern "C" int tah_step_begin(const tah_step_begin_args* a, tah_stream_t stream) {
+    using namespace tah;
+    if (!a) return TAH_E_NULL;
+    if (a->rows < 0 || a->rows > 65535 || a->vocab <= 0 || a->hidden <= 0 || a->hidden % 8 != 0 || a->table_rows <= 0) return TAH_E_SHAPE;
+    if (a->x_packed && (a->rows > 32 || a->hidden % 32 != 0)) return TAH_E_SHAPE;
+    if (a->rows == 0) return TAH_OK;
+    if (!a->tok || !a->pos || !a->finished || !a->embed || !a->cos_table || !a->sin_table || !a->x || !a->cos_rows || !a->sin_rows ||
+        !a->slot || !a->q_pos || !a->active)
+        return TAH_E_NULL;
+    const void* ptrs[] = {a->embed, a->cos_table, a->sin_table, a->x, a->x_packed, a->cos_rows, a->sin_rows};
+    for (const void* q : ptrs)
+        if (reinterpret_cast<uintptr_t>(q) & 15) return TAH_E_ALIGN;
+    if (a->embed_row_stride % 8 != 0 || a->x_row_stride % 8 != 0) return TAH_E_ALIGN;
+    StepBeginParams p;
+    p.tok = a->tok; p.pos = a->pos; p.finished = a->finished;
+    p.embed = static_cast<const __bf16*>(a->embed);
+    p.cos_table = static_cast<const __bf16*>(a->cos_table); p.sin_table = static_cast<const __bf16*>(a->sin_table);
+    p.embed_rs = a->embed_row_stride; p.vocab = a->vocab; p.hidden = a->hidden; p.table_rows = a->table_rows;
+    p.x = static_cast<__bf16*>(a->x); p.x_packed = static_cast<__bf16*>(a->x_packed);
+    p.cos_rows = static_cast<__bf16*>(a->cos_rows); p.sin_rows = static_cast<__bf16*>(a->sin_rows);
+    p.x_rs = a->x_row_stride; p.slot = a->slot; p.q_pos = a->q_pos; p.active = a->active;
+    hipLaunchKernelGGL(step_begin_kernel, dim3(a->rows), dim3(256), 0, static_cast<hipStream_t>(stream), p);
+    return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
+}
+
+extern "C" int tah_decider_tail(const tah_decider_tail_args* a, tah_stream_t stream) {
+    using namespace tah;
+    if (!a) return TAH_E_NULL;
+    if (a->rows < 0 || a->rows > 65535 || a->width <= 0 || a->width % 8 != 0) return TAH_E_SHAPE;
+    if (a->rows == 0) return TAH_OK;
+    if (!a->hidden || !a->w2 || !a->hard || (a->q_pos && !a->pos)) return TAH_E_NULL;
+    if ((reinterpret_cast<uintptr_t>(a->hidden) & 15) || (reinterpret_cast<uintptr_t>(a->w2) & 15) || a->hidden_row_stride % 8 != 0) return TAH_E_ALIGN;
+    DeciderTailParams p;
+    p.h = static_cast<const __bf16*>(a->hidden); p.w2 = static_cast<const __bf16*>(a->w2); p.b2 = static_cast<const __bf16*>(a->b2);
+    p.h_rs = a->hidden_row_stride; p.width = a->width; p.threshold = a->threshold;
+    p.active = a->active; p.pos = a->pos; p.hard = a->hard; p.hard_i = a->hard_i32; p.slot = a->slot; p.q_pos = a->q_pos;
+    hipLaunchKernelGGL(decider_tail_kernel, dim3(a->rows), dim3(64), 0, static_cast<hipStream_t>(stream), p);
+    return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
 }

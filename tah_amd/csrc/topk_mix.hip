@@ -27,6 +27,8 @@ struct MixParams {
     const __bf16* logits;
     const __bf16* emb;
     __bf16* out;
+    bf16x8* outp;  // the rows form of the linear-layer kernels ([hidden / 32][2][64][8]) or null
+    int32_t zero_disabled;
     const uint8_t* row_enable;
     int64_t l_rs, e_rs, o_rs;
     int32_t rows, vocab, hidden, topk;
@@ -77,8 +79,17 @@ __global__ __launch_bounds__(kMixThreads) void topk_mix_kernel(const MixParams p
     HIP_DYNAMIC_SHARED(unsigned char, dyn)  // float partial sums of the mix: [parts][hidden]
 
     const int row = blockIdx.x;
-    if (p.row_enable && !p.row_enable[row]) return;  // uniform per workgroup
     const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    if (p.row_enable && !p.row_enable[row]) {  // uniform per workgroup
+        if (p.zero_disabled) {
+            const bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+            for (int cg = tid; cg < p.hidden / 8; cg += kMixThreads) {
+                *reinterpret_cast<bf16x8*>(p.out + (int64_t)row * p.o_rs + cg * 8) = z;
+                if (p.outp) p.outp[((int64_t)(cg / 4) * 2 + row / 16) * 64 + (row % 16) + 16 * (cg % 4)] = z;
+            }
+        }
+        return;
+    }
     const int V = p.vocab;
     const int k = p.topk < V ? p.topk : V;
     const __bf16* lrow = p.logits + (int64_t)row * p.l_rs;
@@ -351,6 +362,8 @@ __global__ __launch_bounds__(kMixThreads) void topk_mix_kernel(const MixParams p
                 o[c] = (__bf16)s;
             }
             *reinterpret_cast<bf16x8*>(p.out + (int64_t)row * p.o_rs + cg * 8) = o;
+            // columns 8 cg ... of row `row`: step cg / 4, lane row % 16 + 16 (cg % 4) of the packed rows form
+            if (p.outp) p.outp[((int64_t)(cg / 4) * 2 + row / 16) * 64 + (row % 16) + 16 * (cg % 4)] = o;
         }
         __syncthreads();
     }
@@ -364,8 +377,10 @@ extern "C" int tah_topk_mix(const tah_topk_mix_args* a, tah_stream_t stream) {
     if (!a) return TAH_E_NULL;
     if (a->rows < 0 || a->vocab <= 0 || a->hidden <= 0 || a->topk <= 0) return TAH_E_SHAPE;
     if (a->topk > kMaxTopk || a->vocab > kMaxVec * 8 * kMixThreads || a->hidden % 8 != 0) return TAH_E_SHAPE;
+    if (a->out_packed && (a->rows > 32 || a->hidden % 32 != 0)) return TAH_E_SHAPE;
     if (a->rows == 0) return TAH_OK;
     if (!a->logits || !a->embedding || !a->out) return TAH_E_NULL;
+    if (reinterpret_cast<uintptr_t>(a->out_packed) & 15) return TAH_E_ALIGN;
     if ((reinterpret_cast<uintptr_t>(a->embedding) & 15) || (reinterpret_cast<uintptr_t>(a->out) & 15) ||
         (reinterpret_cast<uintptr_t>(a->logits) & 1) || a->embedding_row_stride % 8 || a->out_row_stride % 8)
         return TAH_E_ALIGN;
@@ -373,6 +388,8 @@ extern "C" int tah_topk_mix(const tah_topk_mix_args* a, tah_stream_t stream) {
     p.logits = static_cast<const __bf16*>(a->logits);
     p.emb = static_cast<const __bf16*>(a->embedding);
     p.out = static_cast<__bf16*>(a->out);
+    p.outp = static_cast<bf16x8*>(a->out_packed);
+    p.zero_disabled = a->zero_disabled ? 1 : 0;
     p.row_enable = a->row_enable;
     p.l_rs = a->logits_row_stride; p.e_rs = a->embedding_row_stride; p.o_rs = a->out_row_stride;
     p.rows = a->rows; p.vocab = a->vocab; p.hidden = a->hidden; p.topk = a->topk;

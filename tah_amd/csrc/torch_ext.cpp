@@ -30,6 +30,8 @@ struct Api {
     decltype(&tah_duo_schedule_build) schedule_build = nullptr;
     decltype(&tah_greedy_step) greedy_step = nullptr;
     decltype(&tah_silu_mul_normed) silu_mul_normed = nullptr;
+    decltype(&tah_step_begin) step_begin = nullptr;
+    decltype(&tah_decider_tail) decider_tail = nullptr;
     decltype(&tah_linear_pack_weight) linear_pack_weight = nullptr;
     decltype(&tah_linear_pack_rows) linear_pack_rows = nullptr;
     decltype(&tah_linear_rows) linear_rows = nullptr;
@@ -70,6 +72,8 @@ void load_library(const std::string& path, bool allow_host) {
     bind(g.schedule_build, "tah_duo_schedule_build");
     bind(g.greedy_step, "tah_greedy_step");
     bind(g.silu_mul_normed, "tah_silu_mul_normed");
+    bind(g.step_begin, "tah_step_begin");
+    bind(g.decider_tail, "tah_decider_tail");
     bind(g.linear_pack_weight, "tah_linear_pack_weight");
     bind(g.linear_pack_rows, "tah_linear_pack_rows");
     bind(g.linear_rows, "tah_linear_rows");
@@ -558,15 +562,21 @@ void rows_copy(const Tensor& src, const optional<Tensor>& src_rows, const Tensor
              "tah_rows_copy");
 }
 
-Tensor topk_mix(const Tensor& logits, const Tensor& embedding, int64_t topk, const optional<Tensor>& row_enable, const optional<Tensor>& out_) {
+Tensor topk_mix(const Tensor& logits, const Tensor& embedding, int64_t topk, const optional<Tensor>& row_enable, const optional<Tensor>& out_,
+                const optional<Tensor>& out_packed, bool zero_disabled) {
     need_lib();
-    Dev d; d.see(logits); d.see(embedding); d.see(row_enable); d.see(out_);
+    Dev d; d.see(logits); d.see(embedding); d.see(row_enable); d.see(out_); d.see(out_packed);
     TORCH_CHECK(logits.dim() == 2 && embedding.dim() == 2 && logits.scalar_type() == at::kBFloat16 && embedding.scalar_type() == at::kBFloat16,
                 "topk_mix: logits [rows, V] and embedding [V, H] must be bf16");
     TORCH_CHECK(logits.size(1) == embedding.size(0) && logits.stride(1) == 1 && embedding.stride(1) == 1,
                 "topk_mix: vocabulary sizes differ or the inner dimension is not contiguous");
     const int64_t rows = logits.size(0), H = embedding.size(1);
+    // rows that are not enabled: zeros in a fresh tensor (it is zero-filled); in the caller's tensor they keep their
+    // contents unless zero_disabled asks the kernel to write zeros
     Tensor out = out_.has_value() ? *out_ : (row_enable.has_value() ? at::zeros({rows, H}, embedding.options()) : at::empty({rows, H}, embedding.options()));
+    if (out_packed.has_value())
+        TORCH_CHECK(out_packed->scalar_type() == at::kBFloat16 && out_packed->is_contiguous() && out_packed->numel() == 32 * H,
+                    "topk_mix: out_packed must be a contiguous bf16 tensor of 32 * H elements");
     TORCH_CHECK(out.dim() == 2 && out.size(0) == rows && out.size(1) == H && out.scalar_type() == embedding.scalar_type() && out.stride(1) == 1,
                 "topk_mix: out must be bf16 [rows, H]");
     if (row_enable.has_value())
@@ -580,6 +590,8 @@ Tensor topk_mix(const Tensor& logits, const Tensor& embedding, int64_t topk, con
     a.embedding_row_stride = embedding.stride(0);
     a.out_row_stride = rows > 1 ? out.stride(0) : H;
     a.rows = (int32_t)rows; a.vocab = (int32_t)logits.size(1); a.hidden = (int32_t)H; a.topk = (int32_t)topk;
+    a.out_packed = out_packed.has_value() ? out_packed->data_ptr() : nullptr;
+    a.zero_disabled = zero_disabled ? 1 : 0;
     check_rc(g.topk_mix(&a, d.stream()), "tah_topk_mix");
     return out;
 }
@@ -642,6 +654,70 @@ void greedy_step(const Tensor& logits0, const optional<Tensor>& logits1, const o
     check_rc(g.greedy_step(&a, d.stream()), "tah_greedy_step");
 }
 
+// ---- glue of a generation step ---------------------------------------------------------------------------
+bool vec_of(const Tensor& t, at::ScalarType ty, int64_t n) { return t.scalar_type() == ty && t.is_contiguous() && t.numel() == n; }
+
+// tah_step_begin: everything a step needs before its first layer, written into the caller's tensors.
+void step_begin(const Tensor& tok, const Tensor& pos, const Tensor& finished, const Tensor& embed, const Tensor& cos_table,
+                const Tensor& sin_table, const Tensor& x, const optional<Tensor>& x_packed, const Tensor& cos_rows,
+                const Tensor& sin_rows, const Tensor& slot, const Tensor& q_pos, const Tensor& active) {
+    need_lib();
+    Dev d;
+    for (const Tensor* t : {&tok, &pos, &finished, &embed, &cos_table, &sin_table, &x, &cos_rows, &sin_rows, &slot, &q_pos, &active}) d.see(*t);
+    d.see(x_packed);
+    const int64_t rows = tok.numel(), hidden = embed.size(1);
+    TORCH_CHECK(vec_of(tok, at::kLong, rows) && vec_of(pos, at::kInt, rows) && vec_of(finished, at::kBool, rows) &&
+                    vec_of(slot, at::kInt, rows) && vec_of(q_pos, at::kInt, rows) && vec_of(active, at::kBool, rows),
+                "step_begin: tok int64, pos / slot / q_pos int32, finished / active bool, all [rows]");
+    TORCH_CHECK(embed.dim() == 2 && embed.scalar_type() == at::kBFloat16 && embed.stride(1) == 1, "step_begin: embed must be bf16 [V, H]");
+    for (const Tensor* t : {&cos_table, &sin_table})
+        TORCH_CHECK(t->dim() == 2 && t->size(1) == 128 && t->scalar_type() == at::kBFloat16 && t->is_contiguous() && t->size(0) == cos_table.size(0),
+                    "step_begin: the rotary tables must be contiguous bf16 [L, 128]");
+    TORCH_CHECK(x.dim() == 2 && x.size(0) == rows && x.size(1) == hidden && x.scalar_type() == at::kBFloat16 && (rows == 0 || x.stride(1) == 1),
+                "step_begin: x must be bf16 [rows, H]");
+    for (const Tensor* t : {&cos_rows, &sin_rows}) TORCH_CHECK(vec_of(*t, at::kBFloat16, rows * 128), "step_begin: cos_rows / sin_rows must be contiguous bf16 [rows, 128]");
+    if (x_packed.has_value()) TORCH_CHECK(vec_of(*x_packed, at::kBFloat16, 32 * hidden), "step_begin: x_packed must be a contiguous bf16 tensor of 32 * H elements");
+    tah_step_begin_args a{};
+    a.tok = static_cast<const int64_t*>(tok.data_ptr()); a.pos = static_cast<const int32_t*>(pos.data_ptr());
+    a.finished = static_cast<const uint8_t*>(finished.data_ptr());
+    a.embed = embed.data_ptr(); a.embed_row_stride = embed.stride(0);
+    a.cos_table = cos_table.data_ptr(); a.sin_table = sin_table.data_ptr();
+    a.rows = (int32_t)rows; a.vocab = (int32_t)embed.size(0); a.hidden = (int32_t)hidden; a.table_rows = (int32_t)cos_table.size(0);
+    a.x = x.data_ptr(); a.x_row_stride = rows > 1 ? x.stride(0) : hidden;
+    a.x_packed = x_packed.has_value() ? x_packed->data_ptr() : nullptr;
+    a.cos_rows = cos_rows.data_ptr(); a.sin_rows = sin_rows.data_ptr();
+    a.slot = static_cast<int32_t*>(slot.data_ptr()); a.q_pos = static_cast<int32_t*>(q_pos.data_ptr());
+    a.active = static_cast<uint8_t*>(active.data_ptr());
+    check_rc(g.step_begin(&a, d.stream()), "tah_step_begin");
+}
+
+// tah_decider_tail: second layer of the decider, the decision, and the second iteration's per-row bookkeeping.
+void decider_tail(const Tensor& hidden, const Tensor& w2, const optional<Tensor>& b2, double threshold, const optional<Tensor>& active,
+                  const optional<Tensor>& pos, const Tensor& hard, const optional<Tensor>& hard_i32, const optional<Tensor>& slot,
+                  const optional<Tensor>& q_pos) {
+    need_lib();
+    Dev d; d.see(hidden); d.see(w2); d.see(b2); d.see(active); d.see(pos); d.see(hard); d.see(hard_i32); d.see(slot); d.see(q_pos);
+    TORCH_CHECK(hidden.dim() == 2 && hidden.scalar_type() == at::kBFloat16 && (hidden.numel() == 0 || hidden.stride(1) == 1), "decider_tail: hidden must be bf16 [rows, width]");
+    const int64_t rows = hidden.size(0), width = hidden.size(1);
+    TORCH_CHECK(vec_of(w2, at::kBFloat16, width), "decider_tail: w2 must be a contiguous bf16 tensor of `width` elements");
+    if (b2.has_value()) TORCH_CHECK(vec_of(*b2, at::kBFloat16, 1), "decider_tail: b2 must be a bf16 scalar");
+    TORCH_CHECK(vec_of(hard, at::kBool, rows), "decider_tail: hard must be bool [rows]");
+    if (active.has_value()) TORCH_CHECK(vec_of(*active, at::kBool, rows), "decider_tail: active must be bool [rows]");
+    for (const optional<Tensor>* t : {&pos, &hard_i32, &slot, &q_pos})
+        if (t->has_value()) TORCH_CHECK(vec_of(**t, at::kInt, rows), "decider_tail: pos, hard_i32, slot and q_pos are int32 [rows]");
+    tah_decider_tail_args a{};
+    a.hidden = hidden.data_ptr(); a.hidden_row_stride = rows > 1 ? hidden.stride(0) : width;
+    a.w2 = w2.data_ptr(); a.b2 = b2.has_value() ? b2->data_ptr() : nullptr;
+    a.threshold = (float)threshold; a.rows = (int32_t)rows; a.width = (int32_t)width;
+    a.active = active.has_value() ? static_cast<const uint8_t*>(active->data_ptr()) : nullptr;
+    a.pos = pos.has_value() ? static_cast<const int32_t*>(pos->data_ptr()) : nullptr;
+    a.hard = static_cast<uint8_t*>(hard.data_ptr());
+    a.hard_i32 = hard_i32.has_value() ? static_cast<int32_t*>(hard_i32->data_ptr()) : nullptr;
+    a.slot = slot.has_value() ? static_cast<int32_t*>(slot->data_ptr()) : nullptr;
+    a.q_pos = q_pos.has_value() ? static_cast<int32_t*>(q_pos->data_ptr()) : nullptr;
+    check_rc(g.decider_tail(&a, d.stream()), "tah_decider_tail");
+}
+
 // ---- linear layers of a decode step (tah_linear_rows) ------------------------------------------------------
 bool packed_vec(const Tensor& t, int64_t numel) {
     return t.scalar_type() == at::kBFloat16 && t.is_contiguous() && t.numel() == numel;
@@ -676,9 +752,10 @@ Tensor linear_pack_rows(const Tensor& x, const optional<Tensor>& out) {
 // only the packed result is asked for).
 optional<Tensor> linear_rows(const Tensor& w_packed, const Tensor& x_packed, int64_t rows, int64_t n, int64_t k, bool gate_up,
                              const optional<Tensor>& residual, const optional<Tensor>& out, const optional<Tensor>& out_packed,
-                             bool want_out, bool input_norm, double norm_eps) {
+                             bool want_out, bool input_norm, double norm_eps, const optional<Tensor>& bias, bool relu) {
     need_lib();
-    Dev d; d.see(w_packed); d.see(x_packed); d.see(residual); d.see(out); d.see(out_packed);
+    Dev d; d.see(w_packed); d.see(x_packed); d.see(residual); d.see(out); d.see(out_packed); d.see(bias);
+    if (bias.has_value()) TORCH_CHECK(packed_vec(*bias, n), "linear_rows: bias must be a contiguous bf16 [N] tensor");
     TORCH_CHECK(rows >= 0 && n >= 0 && k >= 0, "linear_rows: negative size");
     TORCH_CHECK(packed_vec(w_packed, (gate_up ? 2 : 1) * n * k), "linear_rows: w_packed must come from linear_pack_weight for these sizes");
     TORCH_CHECK(packed_vec(x_packed, 32 * k), "linear_rows: x_packed must be a contiguous bf16 tensor of 32 * K elements");
@@ -701,6 +778,7 @@ optional<Tensor> linear_rows(const Tensor& w_packed, const Tensor& x_packed, int
     a.rows = (int32_t)rows; a.n = (int32_t)n; a.k = (int32_t)k;
     a.kind = gate_up ? TAH_LINEAR_GATE_UP : TAH_LINEAR_PLAIN;
     a.input_norm = input_norm ? 1 : 0; a.norm_eps = (float)norm_eps;
+    a.bias = bias.has_value() ? bias->data_ptr() : nullptr; a.relu = relu ? 1 : 0;
     check_rc(g.linear_rows(&a, d.stream()), "tah_linear_rows");
     return y;
 }
@@ -729,6 +807,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("silu_mul", &silu_mul);
     m.def("duo_decode_step", &duo_decode_step);
     m.def("duo_decode_step_supported", &duo_decode_step_supported);
+    m.def("step_begin", &step_begin);
+    m.def("decider_tail", &decider_tail);
     m.def("linear_pack_weight", &linear_pack_weight);
     m.def("linear_pack_rows", &linear_pack_rows);
     m.def("linear_rows", &linear_rows);

@@ -75,6 +75,7 @@ class Weights:
         self.norms_folded = False
         self.linear_packed = False
         self.lm_head_p: Optional[torch.Tensor] = None
+        self.dec_w1_p: Optional[torch.Tensor] = None
 
     def fold_norms(self) -> "Weights":
         """Multiplies the input-norm weights into the projections that follow them (``wqkv *= ln1``, ``wgu *= ln2``,
@@ -108,6 +109,9 @@ class Weights:
                 L["wdown_p"] = ops.linear_pack_weight(L["wdown"])
             # the output head with the final norm's weight inside (a copy: the head may be the embedding itself)
             self.lm_head_p = ops.linear_pack_weight(self.lm_head * self.norm[None, :]) if self.cfg.vocab % 16 == 0 else None
+            # the decider's first layer behind the final norm, the same way
+            self.dec_w1_p = (ops.linear_pack_weight(self.dec_w1 * self.norm[None, :])
+                             if self.dec_w1 is not None and self.dec_w1.shape[0] % 16 == 0 else None)
             self.linear_packed = True
         return self
 
@@ -194,6 +198,7 @@ class TaHDecodeEngine:
         self.zeros_i = torch.zeros(batch, dtype=torch.int32, device=dev)
         # generation state (all on the device)
         self.fused_greedy = True  # arg-max + bookkeeping of a greedy step in one launch (tah_greedy_step)
+        self.use_fused_glue = True  # (tests switch it off to compare with the torch glue)
         self.tok = torch.zeros(batch, dtype=torch.long, device=dev)       # token fed to the next step
         self.pos = torch.zeros(batch, dtype=torch.int32, device=dev)      # its position
         self.finished = torch.zeros(batch, dtype=torch.bool, device=dev)
@@ -216,6 +221,19 @@ class TaHDecodeEngine:
         if self.packed_linear:  # rows operands handed from kernel to kernel (32 rows each; rows past the batch stay zero)
             z = lambda n: torch.zeros(32 * n, dtype=torch.bfloat16, device=dev)
             self.xp, self.op, self.actp = z(cfg.hidden), z(cfg.hq * cfg.head_dim), z(cfg.intermediate)
+        # the step's element-wise glue in two launches (tah_step_begin, tah_decider_tail) and the decider's first layer
+        # on the linear-layer kernel, instead of some twenty torch launches; needs the packed rows
+        self.fused_glue = bool(self.packed_linear and weights.dec_w1_p is not None and weights.lm_head_p is not None
+                               and cfg.decider_hidden % 8 == 0)
+        if self.fused_glue:
+            i32 = lambda: torch.zeros(batch, dtype=torch.int32, device=dev)
+            self.x0 = torch.zeros(batch, cfg.hidden, dtype=torch.bfloat16, device=dev)
+            self.x1 = torch.zeros_like(self.x0)
+            self.cos_rows = torch.zeros(batch, cfg.head_dim, dtype=torch.bfloat16, device=dev)
+            self.sin_rows = torch.zeros_like(self.cos_rows)
+            self.slot0, self.qpos0, self.slot1, self.qpos1, self.hard_i = i32(), i32(), i32(), i32(), i32()
+            self.act = torch.zeros(batch, dtype=torch.bool, device=dev)
+            self.hard = torch.zeros(batch, dtype=torch.bool, device=dev)
 
     # ── model pieces ─────────────────────────────────────────────────────
     def _rms(self, x, w):
@@ -281,7 +299,7 @@ class TaHDecodeEngine:
             x = self._mlp(x, L)
         return self._rms(x, self.w.norm)
 
-    def _pass_single_packed(self, x, pos, depth: int, slot_of, q_pos, q_depth, cos, sin):
+    def _pass_single_packed(self, x, pos, depth: int, slot_of, q_pos, q_depth, cos, sin, rows_packed: bool = False):
         """The same pass with the four linear layers of a layer on ``ops.linear_rows``: seven launches per layer.  The
         hidden state lives twice, row-major in ``x`` (updated in place; read by the q/k preparation for the norm
         factor) and as rows operand in ``self.xp``; attention output and MLP activation exist as rows operands only."""
@@ -289,7 +307,7 @@ class TaHDecodeEngine:
         B, H, I = x.shape[0], c.hidden, c.intermediate
         n_qkv, n_o = (c.hq + 2 * c.hkv) * c.head_dim, c.hq * c.head_dim
         x = x.contiguous()
-        xp = ops.linear_pack_rows(x, out=self.xp)
+        xp = self.xp if rows_packed else ops.linear_pack_rows(x, out=self.xp)  # rows_packed: self.xp already holds x
         for l, L in enumerate(self.w.layers):
             q, k, v = self._split_qkv(ops.linear_rows(L["wqkv_p"], xp, B, n_qkv, H))
             cache = self.slabs0[l] if depth == 0 else self.slabs1[l]
@@ -357,6 +375,32 @@ class TaHDecodeEngine:
         h1 = self._pass_single(x1, pos, 1, slot1, qpos1, hard_i, rope)
         self.hard_len += hard_i  # after all layers appended at the old count
         return l0, self._head(h1), hard
+
+    def _step_parts_device(self):
+        """``_step_parts(self.tok, active=~self.finished)`` with the element-wise glue in two launches and the decider's
+        first layer on the linear-layer kernel (the final norm folded into it, as into the output head): the decider sees
+        the same numbers up to bf16 rounding order."""
+        c, w, B = self.cfg, self.w, self.B
+        ops.step_begin(self.tok, self.pos, self.finished, w.embed, self.cos, self.sin, x=self.x0, x_packed=self.xp,
+                       cos_rows=self.cos_rows, sin_rows=self.sin_rows, slot=self.slot0, q_pos=self.qpos0, active=self.act)
+        self._pass_single_packed(self.x0, self.pos, 0, self.slot0, self.qpos0, self.zeros_i, self.cos_rows, self.sin_rows,
+                                 rows_packed=True)
+        l0 = self._head(self.x0)
+        hr = ops.linear_rows(w.dec_w1_p, self.xp, B, c.decider_hidden, c.hidden, norm_eps=c.rms_eps, bias=w.dec_b1, relu=True)
+        ops.decider_tail(hr, w.dec_w2.reshape(-1), w.dec_b2, w.threshold, hard=self.hard, active=self.act, pos=self.pos,
+                         hard_i32=self.hard_i, slot=self.slot1, q_pos=self.qpos1)
+        ops.topk_mix(l0, w.embed, c.topk, row_enable=self.hard, out=self.x1, out_packed=self.xp, zero_disabled=True)
+        h1 = self._pass_single_packed(self.x1, self.pos, 1, self.slot1, self.qpos1, self.hard_i, self.cos_rows, self.sin_rows,
+                                      rows_packed=True)
+        self.hard_len += self.hard_i  # after all layers appended at the old count
+        return l0, self._head(h1), self.hard
+
+    def _parts(self):
+        """Both iterations of a step on the engine's own state: (logits0, logits1, hard, active)."""
+        if self.fused_glue and self.use_fused_glue:
+            return self._step_parts_device() + (self.act,)
+        act = ~self.finished
+        return self._step_parts(self.tok, active=act) + (act,)
 
     # ── prefill: packed prompts, both depths, through the varlen kernels ──
     @torch.no_grad()
@@ -460,15 +504,14 @@ class TaHDecodeEngine:
 
     def _step_inplace(self, temperature: float, eos: int, **filters):
         """One generated token for every unfinished row; every state change is an in-place device update."""
-        act = ~self.finished
+        l0, l1, hard, act = self._parts()
         if temperature <= 0.0 and self.fused_greedy and self.w.embed.dtype == torch.bfloat16 and self.cfg.vocab % 8 == 0:
             # arg-max of the final logits and the bookkeeping below in one launch; the final logits are not formed
-            l0, l1, hard = self._step_parts(self.tok, active=act)
             ops.greedy_step(l0, l1, hard, eos, self.tok, self.finished, self.pos, self.out_tokens, self.step_idx, self.out_len,
                             self.n_hard, self.n_steps)
             self.step_idx += 1
             return
-        logits, hard = self.step_logits(self.tok, active=act)
+        logits = torch.where(hard[:, None], (l0 + l1).float(), l0.float())  # as step_logits forms them
         nxt = self.sample(logits, temperature, **filters)
         nxt = torch.where(act, nxt, torch.zeros_like(nxt))
         if eos >= 0:

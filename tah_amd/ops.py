@@ -97,11 +97,14 @@ def rows_copy(src: torch.Tensor, src_rows: Optional[torch.Tensor], dst: torch.Te
 
 
 def topk_mix(logits: torch.Tensor, embedding: torch.Tensor, topk: int, row_enable: Optional[torch.Tensor] = None,
-             out: Optional[torch.Tensor] = None) -> torch.Tensor:
+             out: Optional[torch.Tensor] = None, out_packed: Optional[torch.Tensor] = None,
+             zero_disabled: bool = False) -> torch.Tensor:
     """Soft input embedding of hard tokens (tah_model.py:57-75): logits bf16 [rows, V] -> bf16 [rows, H], the
     softmax over each row's top-k logits times the matching rows of ``embedding`` [V, H].  ``row_enable``
-    (bool/uint8 [rows]): rows with 0 are skipped and keep what ``out`` held (zeros when ``out`` is not given)."""
-    return _call("topk_mix", logits, embedding, int(topk), row_enable, out)
+    (bool/uint8 [rows]): rows with 0 are skipped and keep what ``out`` held (zeros when ``out`` is not given, or with
+    ``zero_disabled``).  ``out_packed`` (bf16 [32 * H], rows <= 32) also receives the rows as the rows operand of
+    ``linear_rows``."""
+    return _call("topk_mix", logits, embedding, int(topk), row_enable, out, out_packed, bool(zero_disabled))
 
 
 def silu_mul(gate_up: torch.Tensor, norm_input: Optional[torch.Tensor] = None, norm_eps: float = 0.0) -> torch.Tensor:
@@ -111,6 +114,21 @@ def silu_mul(gate_up: torch.Tensor, norm_input: Optional[torch.Tensor] = None, n
     un-normalised rows through a weight that carries the norm's weight, and gate and up are multiplied by the row's
     ``rsqrt(mean(norm_input**2) + norm_eps)`` first."""
     return _call("silu_mul", gate_up, norm_input, float(norm_eps))
+
+
+def step_begin(tok, pos, finished, embed, cos_table, sin_table, *, x, x_packed, cos_rows, sin_rows, slot, q_pos, active) -> None:
+    """Start of a generation step in one launch (``tah_step_begin``), results written into the keyword tensors: per
+    row ``active = ~finished``; ``slot`` = row index and ``q_pos`` = ``pos`` for active rows, -1 otherwise; the rotary
+    rows of ``pos`` (clamped into the tables) in ``cos_rows`` / ``sin_rows`` [rows, 128]; the embedding row of ``tok`` in
+    ``x`` [rows, H] and, when given, in ``x_packed`` [32 * H] (the rows operand of ``linear_rows``)."""
+    _call("step_begin", tok, pos, finished, embed, cos_table, sin_table, x, x_packed, cos_rows, sin_rows, slot, q_pos, active)
+
+
+def decider_tail(hidden, w2, b2, threshold: float, *, hard, active=None, pos=None, hard_i32=None, slot=None, q_pos=None) -> None:
+    """Second layer of a two-layer decider and the decision (``tah_decider_tail``): ``hard = sigmoid(hidden @ w2 + b2) >
+    threshold`` (``& active``), with the eager bf16 roundings, written into ``hard`` (bool [rows]); optionally
+    ``hard_i32`` (0/1), ``slot`` (row index or -1) and ``q_pos`` (``pos`` or -1) for the second latent iteration."""
+    _call("decider_tail", hidden, w2, b2, float(threshold), active, pos, hard, hard_i32, slot, q_pos)
 
 
 LINEAR_MAX_ROWS = 32
@@ -131,17 +149,19 @@ def linear_pack_rows(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> tor
 
 def linear_rows(w_packed: torch.Tensor, x_packed: torch.Tensor, rows: int, n: int, k: int, *, gate_up: bool = False,
                 residual: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
-                out_packed: Optional[torch.Tensor] = None, want_out: bool = True, norm_eps: Optional[float] = None):
+                out_packed: Optional[torch.Tensor] = None, want_out: bool = True, norm_eps: Optional[float] = None,
+                bias: Optional[torch.Tensor] = None, relu: bool = False):
     """A linear layer of a decode step on packed operands (``tah_linear_rows``), bf16, rows <= 32.
 
     ``x @ w.T`` [rows, N], plus ``residual`` [rows, N] when given (``out=residual`` updates it in place); with
     ``gate_up``, ``silu(x @ gate.T) * (x @ up.T)``.  With ``norm_eps`` the products are first multiplied by the row's
     ``rsqrt(mean(x**2) + norm_eps)``: an RMSNorm of the rows whose weight sits in w (the MLP's input norm for gate|up,
-    the final norm for an output head).  ``out_packed`` [32 * N] also
+    the final norm for an output head).  ``bias`` [N] is added to the rounded product and ``relu`` applied last (the first
+    layer of a small MLP; not with ``gate_up``).  ``out_packed`` [32 * N] also
     receives the result as the next layer's rows operand; ``want_out=False`` with ``out_packed`` writes only that.
     Returns the row-major result (None when it was not asked for)."""
     return _call("linear_rows", w_packed, x_packed, int(rows), int(n), int(k), bool(gate_up), residual, out, out_packed,
-                 bool(want_out), norm_eps is not None, float(norm_eps or 0.0))
+                 bool(want_out), norm_eps is not None, float(norm_eps or 0.0), bias, bool(relu))
 
 
 def greedy_step(logits0, logits1, hard, eos: int, tok, finished, pos, out_tokens, step_idx, out_len, n_hard, n_steps) -> None:

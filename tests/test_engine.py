@@ -240,3 +240,33 @@ def test_engine_with_fused_layer_attention_equals_the_separate_launches_gpu():
         out.append((eng.generate(first, 10, eos=7, use_graph=use_graph).clone(), int(eng.n_hard), eng.hard_len.tolist(),
                     [sl.len.tolist() for sl in eng.slabs0 + eng.slabs1]))
     assert torch.equal(out[0][0], out[1][0]) and out[0][1:] == out[1][1:] and out[0][1] > 0
+
+
+@pytest.mark.gpu
+def test_engine_fused_glue_agrees_with_the_torch_glue_gpu():
+    """One step from the same state through tah_step_begin / the decider on the linear-layer kernel / tah_decider_tail
+    and through the torch operations they replace: the first iteration's logits are the same launches on the same
+    inputs (equal), the decisions agree except where a probability sits within rounding of the threshold, and the
+    second iteration's logits agree for rows both call hard."""
+    from tah_amd.engine import EngineConfig, TaHDecodeEngine, Weights
+    cfg = EngineConfig(hidden=256, layers=2, hq=4, hkv=2, head_dim=128, intermediate=512, vocab=4096, decider_hidden=32)
+    w = Weights.random_init(cfg, "cuda", seed=8)
+    B, T = 16, 19
+    g = torch.Generator().manual_seed(12)
+    ids = torch.randint(0, cfg.vocab, (B * T,), generator=g).cuda()
+    cu = torch.arange(0, B * T + 1, T, dtype=torch.int32, device="cuda")
+    outs = []
+    for fused in (True, False):
+        eng = TaHDecodeEngine(w, B, T + 8, device="cuda")
+        assert eng.fused_glue
+        eng.use_fused_glue = fused
+        first, _ = eng.prefill(ids, cu, calibrate=0.3)
+        eng.tok.copy_(first.argmax(-1))
+        eng.finished[3] = True
+        l0, l1, hard, _ = eng._parts()
+        outs.append((l0.float().clone(), l1.float().clone(), hard.clone(), [sl.len.tolist() for sl in eng.slabs0]))
+    (a0, a1, ha, la), (b0, b1, hb, lb) = outs
+    assert torch.equal(a0, b0) and la == lb
+    assert (ha == hb).float().mean() >= 0.9 and ha.any() and not ha[3]
+    both = ha & hb
+    assert (a1[both] - b1[both]).abs().max().item() <= 2e-2 * max(b1[both].abs().max().item(), 1.0)

@@ -151,7 +151,7 @@ def test_forward_loop_with_launch_order_table(emu, monkeypatch):
     it; one table is built per depth and the backward pass runs with it."""
     from tah_amd import attention, ops
     from tah_amd.cache import TaHDuoCache
-    c = make_dense_case(33, B=3, T=72, p_hard=0.25, Hq=2, Hkv=1, D=128, left_pad=[0, 10, 40])
+    c = make_dense_case(33, B=3, T=40, p_hard=0.25, Hq=2, Hkv=1, D=128, left_pad=[0, 6, 22])
     _, w1, w2, _ = _forward_two_depths(c, TaHDuoCache())
     built = []
     real = ops.duo_schedule

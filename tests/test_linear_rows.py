@@ -61,13 +61,17 @@ def unpack_rows(packed, k):
     return x
 
 
-def reference(x, w, *, residual=None, gate_up=False, norm_eps=None):
+def reference(x, w, *, residual=None, gate_up=False, norm_eps=None, bias=None, relu=False):
     """float64 sums with the eager modules' bf16 roundings."""
     xd, wd = x.double(), w.double()
     r = torch.rsqrt((xd ** 2).mean(-1, keepdim=True) + norm_eps) if norm_eps is not None else 1.0
     if not gate_up:
         y = (r * (xd @ wd.t())).to(BF)
-        return y if residual is None else (y.double() + residual.double()).to(BF)
+        if bias is not None:
+            y = (y.double() + bias.double()).to(BF)
+        if residual is not None:
+            y = (y.double() + residual.double()).to(BF)
+        return torch.relu(y) if relu else y
     n = w.shape[0] // 2
     g = (r * (xd @ wd[:n].t())).to(BF).double()
     u = (r * (xd @ wd[n:].t())).to(BF).double()
@@ -114,6 +118,8 @@ CASES = [
     (32, 3120, 64, "gate_up_norm"),
     (9, 48, 2048, "plain_norm"),      # an RMSNorm of the rows folded in (an output head behind the final norm)
     (32, 32, 160, "plain_norm"),
+    (11, 32, 2048, "bias_relu_norm"),  # first layer of a small MLP behind a folded norm (the decider)
+    (32, 48, 96, "bias_relu"),
 ]
 
 
@@ -124,7 +130,10 @@ def _linear_case(dev, rows, n, k, kind, seed=0):
     w = _rand(((2 if gu else 1) * n, k), 12 + seed, k ** -0.5)
     res = _rand((rows, n), 13 + seed) if kind == "residual" else None
     eps = 1e-6 if kind.endswith("_norm") else None
-    want = reference(x, w, residual=res, gate_up=gu, norm_eps=eps)
+    bias = _rand((n,), 14 + seed) if kind.startswith("bias") else None
+    relu = "relu" in kind
+    want = reference(x, w, residual=res, gate_up=gu, norm_eps=eps, bias=bias, relu=relu)
+    extra = dict(bias=bias.to(dev), relu=relu) if bias is not None else {}
     wp = ops.linear_pack_weight(w.to(dev), gate_up=gu)
     xp = ops.linear_pack_rows(x.to(dev))
     yp = torch.full((32 * n,), 7.0, dtype=BF, device=dev) if n % 32 == 0 else None  # the packed form holds whole steps of 32
@@ -133,7 +142,9 @@ def _linear_case(dev, rows, n, k, kind, seed=0):
         got = ops.linear_rows(wp, xp, rows, n, k, residual=h, out=h, out_packed=yp)
         assert got.data_ptr() == h.data_ptr()
     else:
-        got = ops.linear_rows(wp, xp, rows, n, k, gate_up=gu, out_packed=yp, norm_eps=eps)
+        got = ops.linear_rows(wp, xp, rows, n, k, gate_up=gu, out_packed=yp, norm_eps=eps, **extra)
+        if relu:
+            assert (got.float() >= 0).all() and (got == 0).any()
     got = got.cpu()
     _close(got, want)
     if yp is not None:
@@ -142,10 +153,10 @@ def _linear_case(dev, rows, n, k, kind, seed=0):
         # packed result only
         yp2 = torch.empty_like(yp)
         h2 = res.clone().to(dev) if res is not None else None
-        assert ops.linear_rows(wp, xp, rows, n, k, gate_up=gu, residual=h2, out_packed=yp2, want_out=False, norm_eps=eps) is None
+        assert ops.linear_rows(wp, xp, rows, n, k, gate_up=gu, residual=h2, out_packed=yp2, want_out=False, norm_eps=eps, **extra) is None
         assert torch.equal(yp2, yp)
     # twice the same: sums run in a fixed order
-    again = ops.linear_rows(wp, xp, rows, n, k, gate_up=gu, residual=res.to(dev) if res is not None else None, norm_eps=eps)
+    again = ops.linear_rows(wp, xp, rows, n, k, gate_up=gu, residual=res.to(dev) if res is not None else None, norm_eps=eps, **extra)
     assert torch.equal(again.cpu(), got)
 
 

@@ -28,7 +28,7 @@ def _run(device, seed, rows, V, H, k, **kw):
 @pytest.mark.skipif(not emu_util.have_host_clang(), reason="host clang++ not available")
 @pytest.mark.parametrize("seed,rows,V,H,k,kw", [
     (0, 2, 700, 64, 100, {}), (1, 1, 9000, 32, 17, dict(ties=0.05)), (2, 2, 90, 16, 100, {}), (3, 1, 17000, 256, 100, {}),
-    (4, 1, 1003, 8, 256, dict(ties=0.3)),
+    (4, 1, 1003, 8, 200, dict(ties=0.3)),
     (5, 1, 17000, 16, 50, dict(ties=0.2)),   # 3400 equal logits at the threshold: more than the candidate list holds
 ])
 def test_topk_mix_on_cpu_shim(seed, rows, V, H, k, kw):
@@ -46,7 +46,18 @@ def test_topk_mix_golden_and_row_enable_on_cpu_shim():
         en = torch.tensor([1, 0, 1], dtype=torch.uint8)
         keep = torch.full((3, z["emb"].shape[1]), 7.0, dtype=torch.bfloat16)
         ops.topk_mix(to_torch(z["logits"], "cpu"), to_torch(z["emb"], "cpu"), int(z["k"]), row_enable=en, out=keep)
+        # rows that are not enabled written as zeros, and the rows once more in the linear-layer kernels' operand order
+        H = z["emb"].shape[1]
+        zeroed = torch.full((3, H), 7.0, dtype=torch.bfloat16)
+        packed = torch.full((32 * H,), 5.0, dtype=torch.bfloat16) if H % 32 == 0 else None
+        ops.topk_mix(to_torch(z["logits"], "cpu"), to_torch(z["emb"], "cpu"), int(z["k"]), row_enable=en, out=zeroed, out_packed=packed,
+                     zero_disabled=True)
     assert np.array_equal(keep[0].float().numpy(), z["out"][0]) and (keep[1] == 7).all()
+    assert torch.equal(zeroed[0], keep[0]) and torch.equal(zeroed[2], keep[2]) and not zeroed[1].any()
+    if packed is not None:
+        from tests.test_linear_rows import unpack_rows
+        rows = unpack_rows(packed, H)
+        assert torch.equal(rows[:3], zeroed) and (rows[3:] == 5).all()
 
 
 def test_oracle_reproduces_golden():
@@ -111,14 +122,32 @@ def _silu_mul_normed_check(device):
     assert torch.allclose(got.float(), want.float(), rtol=2.0 ** -6, atol=1e-30)
 
 
+def _packed_rows_check(device):
+    """The rows once more in the operand order of the linear-layer kernels, rows that are not enabled as zeros."""
+    from tah_amd import ops
+    from tests.test_linear_rows import unpack_rows
+    g = torch.Generator().manual_seed(8)
+    logits = torch.randn(5, 300, generator=g).to(torch.bfloat16).to(device)
+    emb = torch.randn(300, 64, generator=g).to(torch.bfloat16).to(device)
+    en = torch.tensor([1, 1, 0, 1, 0], dtype=torch.bool, device=device)
+    want = ops.topk_mix(logits, emb, 20, row_enable=en)
+    out = torch.full((5, 64), 3.0, dtype=torch.bfloat16, device=device)
+    packed = torch.full((32 * 64,), 3.0, dtype=torch.bfloat16, device=device)
+    ops.topk_mix(logits, emb, 20, row_enable=en, out=out, out_packed=packed, zero_disabled=True)
+    rows = unpack_rows(packed.cpu(), 64)
+    assert torch.equal(out, want) and not out[2].any() and torch.equal(rows[:5], out.cpu()) and (rows[5:] == 3).all()
+
+
 @pytest.mark.skipif(not emu_util.have_host_clang(), reason="host clang++ not available")
 def test_silu_mul_on_cpu_shim():
     with emu_util.emulated():
         _silu_mul_check("cpu")
         _silu_mul_normed_check("cpu")
+        _packed_rows_check("cpu")
 
 
 @pytest.mark.gpu
 def test_silu_mul_gpu():
     _silu_mul_check("cuda")
     _silu_mul_normed_check("cuda")
+    _packed_rows_check("cuda")
