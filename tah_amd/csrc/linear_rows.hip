@@ -395,10 +395,10 @@ extern "C" int tah_linear_rows(const tah_linear_rows_args* a, tah_stream_t strea
         // an output head: two tiles per workgroup, the rows' operand is read half as often
         const int groups = a->n / (2 * kTileCols);
         if (p.norm) {
-            if (pw == 8) launch<2, 4, kPlainNorm, 8>(p, groups, st);
+            if (pw == 8) launch<2, 2, kPlainNorm, 8>(p, groups, st);
             else launch<2, 2, kPlainNorm, 0>(p, groups, st);
         } else {
-            if (pw == 8) launch<2, 4, kPlain, 8>(p, groups, st);
+            if (pw == 8) launch<2, 2, kPlain, 8>(p, groups, st);
             else launch<2, 2, kPlain, 0>(p, groups, st);
         }
     } else if (!gate_up) {

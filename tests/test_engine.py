@@ -270,3 +270,28 @@ def test_engine_fused_glue_agrees_with_the_torch_glue_gpu():
     assert (ha == hb).float().mean() >= 0.9 and ha.any() and not ha[3]
     both = ha & hb
     assert (a1[both] - b1[both]).abs().max().item() <= 2e-2 * max(b1[both].abs().max().item(), 1.0)
+
+
+@pytest.mark.gpu
+def test_engine_beyond_32_rows_falls_back_to_library_gemms_gpu():
+    """33 sequences: the linear-layer kernels take at most 32 rows, so the step runs on torch GEMMs and the torch glue;
+    the captured step still gives the eager step's tokens, and the first 32 rows' prefill logits do not depend on the
+    33rd sequence being there."""
+    from tah_amd.engine import EngineConfig, TaHDecodeEngine, Weights
+    cfg = EngineConfig(hidden=256, layers=2, hq=4, hkv=2, head_dim=128, intermediate=512, vocab=2048, decider_hidden=32)
+    w = Weights.random_init(cfg, "cuda", seed=9)
+    B, T, new = 33, 17, 6
+    g = torch.Generator().manual_seed(13)
+    ids = torch.randint(0, cfg.vocab, (B * T,), generator=g).cuda()
+    cu = torch.arange(0, B * T + 1, T, dtype=torch.int32, device="cuda")
+    out = []
+    for use_graph in (False, True):
+        eng = TaHDecodeEngine(w, B, T + new + 2, device="cuda")
+        assert not eng.packed_linear and not eng.fused_glue and not eng.fused_step
+        first, _ = eng.prefill(ids, cu, calibrate=0.3)
+        out.append((first.clone(), eng.generate(first, new, use_graph=use_graph).clone(), int(eng.n_hard)))
+    assert torch.equal(out[0][1], out[1][1]) and out[0][2] == out[1][2] and out[0][2] > 0
+    small = TaHDecodeEngine(w, 32, T + new + 2, device="cuda")
+    assert small.packed_linear
+    first32, _ = small.prefill(ids[:32 * T], cu[:33])
+    assert torch.allclose(first32, out[0][0][:32], atol=2e-2 * float(first32.abs().max()))
