@@ -16,8 +16,8 @@
 //    factor (the norm's weight is expected inside W): the sum of squares of a row comes from the operands the
 //    waves load anyway.  Results are written row-major and/or in the packed rows form for the next layer.
 //
-// Measured at 32 rows inside a captured step (MI355X): q|k|v 16 MB 6.0 us, o 8 MB 5.7 us, gate|up + SiLU 50 MB
-// 12.8 us, down 25 MB 12.1 us, against 14 / 8.4 / 16 + 5 / 15 us for the library GEMMs and the SiLU kernel.  What
+// Measured at 32 rows inside a captured step (MI355X): q|k|v 16 MB 6.0 us, o 8 MB 5.1 us, gate|up + SiLU 50 MB
+// 12.3 us, down 25 MB 9.6 us, against 14 / 8.4 / 16 + 5 / 15 us for the library GEMMs and the SiLU kernel.  What
 // is left besides the weight stream (7.5 TB/s once started) is about 4 us of launch, first-byte latency and
 // reduction per kernel, and the rows' operand: every workgroup reads all 32 x K of it from L2, which the
 // per-CU L1 fill rate (about 100 GB/s) makes 1 us per 128 KB.  Splitting K over workgroups would cut that, but
@@ -109,14 +109,22 @@ __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(const LinParam
     // Loads of chunk ch.  Without a compile-time K a step past the wave's share reads step 0 of the wave's range
     // (valid memory) and is multiplied by rows of zeros: no branch sits between the loads.
     auto issue = [&](int ch, Buf& b) __attribute__((always_inline)) {
+        // the rows' operand first: it comes from L2 and is there long before the weights are, and a wave's loads
+        // return in order -- behind the weight loads it would only arrive after their trip to HBM (down 11.2 -> 9.6 us)
+#pragma unroll
+        for (int s = 0; s < CH; ++s) {
+            const int st = ch * CH + s;
+            const int64_t sti = (PW > 0 || st < nst) ? st : 0;
+            b.x[s][0] = xb[sti * 128];
+            if constexpr (NH == 2) b.x[s][1] = xb[sti * 128 + 64];
+        }
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int s = 0; s < CH; ++s) {
             const int st = ch * CH + s;
             const int64_t sti = (PW > 0 || st < nst) ? st : 0;
 #pragma unroll
             for (int t = 0; t < NC; ++t) b.w[s][t] = __builtin_nontemporal_load(wb[t] + sti * 64);
-            b.x[s][0] = xb[sti * 128];
-            if constexpr (NH == 2) b.x[s][1] = xb[sti * 128 + 64];
         }
     };
     auto multiply = [&](int ch, Buf& b) __attribute__((always_inline)) {
