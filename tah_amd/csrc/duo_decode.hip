@@ -135,19 +135,28 @@ struct RowBlock {
 template <int U>
 __device__ __forceinline__ void load_rows(RowBlock<U>& b, const Seg& sg, bool second, const __bf16* kbase, const __bf16* vbase,
                                           const int32_t* posbase, int r_it, int row_end, int kq) {
+    // all of K (and the positions) before V: a wave's loads return in order, and the scores need K only
+    int rl[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const int r = r_it + u * 4 + kq;
         b.ok[u] = r < row_end;
-        const int rl = b.ok[u] ? r : row_end - 1;  // keep tail loads inside the slab
+        rl[u] = b.ok[u] ? r : row_end - 1;  // keep tail loads inside the slab
 #if TAH_DEC_NT
-        b.k[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kbase + (int64_t)rl * sg.k_rs));
-        b.v[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vbase + (int64_t)rl * sg.v_rs));
+        b.k[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kbase + (int64_t)rl[u] * sg.k_rs));
 #else
-        b.k[u] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)rl * sg.k_rs);
-        b.v[u] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)rl * sg.v_rs);
+        b.k[u] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)rl[u] * sg.k_rs);
 #endif
-        b.pos[u] = second ? posbase[rl] : 0;
+        b.pos[u] = second ? posbase[rl[u]] : 0;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#if TAH_DEC_NT
+        b.v[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vbase + (int64_t)rl[u] * sg.v_rs));
+#else
+        b.v[u] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)rl[u] * sg.v_rs);
+#endif
     }
 }
 // Scores, online softmax and the weighted sum of V for a loaded block, for the G query heads of the kv head at
