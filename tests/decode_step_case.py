@@ -18,10 +18,15 @@ def _slabs(B, cap, hkv, lens, with_pos, g, dev):
     return s
 
 
-def run(dev, *, B, hq, hkv, seed=0, max_len=90, hidden=256, cap1=128, cap2=64):
+def run(dev, *, B, hq, hkv, seed=0, max_len=90, hidden=256, cap1=128, cap2=64, full_slab=False):
+    """full_slab: the depth-0 slabs hold exactly the longest sequence, so that sequence's new row does not fit: both
+    paths have to raise the overflow flag, leave slab and length alone and attend over what is cached."""
     from tah_amd import kv_cache
     g = torch.Generator().manual_seed(seed)
     lens1 = torch.randint(1, max_len, (B,), generator=g).tolist()
+    if full_slab:
+        lens1[1] = max(lens1) + 1   # one longest sequence, active
+        cap1 = lens1[1]
     lens2 = [int(torch.randint(0, min(l, cap2 - 1) + 1, (1,), generator=g)) for l in lens1]
     c1 = _slabs(B, cap1, hkv, lens1, False, g, dev)
     c2 = _slabs(B, cap2, hkv, lens2, True, g, dev)
@@ -69,10 +74,14 @@ def run(dev, *, B, hq, hkv, seed=0, max_len=90, hidden=256, cap1=128, cap2=64):
         assert pb is None or torch.equal(unpack_rows(pb.cpu(), hq * 128)[:B], ob.cpu().reshape(B, -1))
         for sa, sb in ((a1, b1), (a2, b2)):
             assert torch.equal(sa.k, sb.k) and torch.equal(sa.v, sb.v) and torch.equal(sa.len, sb.len)
-            assert int(sa.overflow) == int(sb.overflow) == 0
+        over = 1 if (full_slab and depth == 0) else 0
+        assert int(a1.overflow) == int(b1.overflow) == over and int(a2.overflow) == int(b2.overflow) == 0
         assert torch.equal(a2.pos, b2.pos)
         tgt_a, src = (a1, c1) if depth == 0 else (a2, c2)
-        assert torch.equal(tgt_a.len.cpu(), src.len.cpu() + sel.cpu().to(torch.int32))  # the step did append
+        grew = sel.cpu().to(torch.int32)
+        if over:
+            grew[1] = 0   # the row that did not fit
+        assert torch.equal(tgt_a.len.cpu(), src.len.cpu() + grew)  # the step did append
         assert oa[B // 3].abs().max() == 0                                              # the finished row saw nothing
         results[depth] = oa
     return results

@@ -16,7 +16,7 @@ def _check(outs):
 def test_engine_matches_reference_loop_on_cpu_shim():
     from tests.engine_case import run
     with emu_util.emulated():
-        _check(run("cpu", prompt=(7, 4), steps=4))
+        _check(run("cpu", prompt=(7, 4), steps=3))  # one hard row and a pad row, nobody, everybody
 
 
 def _same_greedy(device, **size):
