@@ -418,6 +418,14 @@ class TaHDecodeEngine:
         N = int(cu_h[-1])
         if max(lens) > self.max_len:
             raise TahDuoError("prompt longer than the cache capacity")
+        # a new batch: whatever an earlier generation left in the slabs is forgotten
+        for sl in self.slabs0 + self.slabs1:
+            sl.len.zero_()
+            sl.overflow.zero_()
+        self.n_hard.zero_()
+        self.n_steps.zero_()
+        self.host_hard_rows = 0
+        self._graph = None  # (its warm-up step belongs to the old batch's state)
         seq = torch.repeat_interleave(torch.arange(B, device=dev), torch.tensor(lens, device=dev))
         pos = (torch.arange(N, device=dev) - cu.long()[seq]).to(torch.int32)
         cos, sin = self.cos[pos.long()], self.sin[pos.long()]

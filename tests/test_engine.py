@@ -295,3 +295,26 @@ def test_engine_beyond_32_rows_falls_back_to_library_gemms_gpu():
     assert small.packed_linear
     first32, _ = small.prefill(ids[:32 * T], cu[:33])
     assert torch.allclose(first32, out[0][0][:32], atol=2e-2 * float(first32.abs().max()))
+
+
+@pytest.mark.gpu
+def test_engine_can_be_used_for_a_second_batch_gpu():
+    """prefill() starts from empty slabs: a second generation on the same engine equals the first one and a fresh
+    engine's."""
+    from tah_amd.engine import EngineConfig, TaHDecodeEngine, Weights
+    cfg = EngineConfig(hidden=256, layers=2, hq=4, hkv=2, head_dim=128, intermediate=512, vocab=2048, decider_hidden=32)
+    w = Weights.random_init(cfg, "cuda", seed=11)
+    B, T, new = 4, 15, 8
+    g = torch.Generator().manual_seed(14)
+    ids = torch.randint(0, cfg.vocab, (2, B * T), generator=g).cuda()
+    cu = torch.arange(0, B * T + 1, T, dtype=torch.int32, device="cuda")
+    eng = TaHDecodeEngine(w, B, T + new + 2, device="cuda")
+    runs = []
+    for which in (0, 1, 0):
+        first, _ = eng.prefill(ids[which], cu, calibrate=None)
+        runs.append((eng.generate(first, new).clone(), int(eng.n_hard), [sl.len.tolist() for sl in eng.slabs0 + eng.slabs1]))
+    assert torch.equal(runs[0][0], runs[2][0]) and runs[0][1:] == runs[2][1:]
+    assert not torch.equal(runs[0][0], runs[1][0])
+    fresh = TaHDecodeEngine(w, B, T + new + 2, device="cuda")
+    first, _ = fresh.prefill(ids[1], cu)
+    assert torch.equal(fresh.generate(first, new), runs[1][0])
