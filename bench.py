@@ -290,77 +290,73 @@ def bench_e2e_decode(new_tokens: int, B: int = 32, prompt_len: int = 512):
     first, hard = eng.prefill(ids, cu, calibrate=0.06)
     torch.cuda.synchronize()
     prefill_s = time.perf_counter() - t0
-    # eager steps (every kernel launched from Python): what the host layer costs without the graph
-    n_eager = 8
-    eng.generate(first, 1, use_graph=False)
+    # the generation: greedy, rows at different latent iterations share a batch (one captured tick per replay; a row's
+    # token costs it one tick, or two when it is hard), the host looks every 8 ticks whether all rows have their tokens
+    eng.capture_ticks(-1, new_tokens)  # (graph capture is set-up, like the engine's buffers)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(n_eager):
-        eng._step_inplace(0.0, -1)
-    host_eager = (time.perf_counter() - t0) / n_eager
+    toks = eng.generate(first, new_tokens, use_graph=True)
     torch.cuda.synchronize()
-    eager_s = (time.perf_counter() - t0) / n_eager
-    eng.host_positions += n_eager
-    eng.host_hard_rows += n_eager
-    # graph replays
-    gr = eng.capture(0.0, -1)
-    # what a replay costs the host when the queue is empty (in the loop below the host runs ahead of the GPU until
-    # the queue is full and then waits for it, so its time per replay there is the GPU's)
-    left = new_tokens - 1 - n_eager
-    if left < 2:
-        raise SystemExit(f"--e2e-tokens must be at least {n_eager + 3}")
-    n_enqueue = 5 if left >= 20 else 1
-    enqueue = []
-    for _ in range(n_enqueue):
+    gen_s = time.perf_counter() - t0
+    ticks = eng.ticks
+    n_tokens = int(eng.n_steps)
+    assert n_tokens == B * (new_tokens - 1) and int(eng.out_len.min()) == new_tokens
+    frac_hard = int(eng.n_hard) / max(n_tokens, 1)
+    step_ms = gen_s * 1e3 / ticks
+    ctx = float(eng.pos.float().mean())
+    # one tick at the final context, with and without the attention launches, all rows busy; and launched from Python
+    eng.finished.zero_()
+    eng.out_len.zero_()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    n_probe = (extra_steps - 10) // 3
+
+    def ticks_ms(without_attention: bool, graph: bool):
+        eng.measure_without_attention = without_attention
+        eng._tick_graphs = None
+        graphs = eng.capture_ticks(-1, eng.max_len) if graph else None
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        gr.replay()
+        e0.record()
+        for i in range(n_probe):
+            if graphs is not None:
+                graphs[i % 2].replay()
+            else:
+                eng._tick(i % 2, -1, eng.max_len)
+        e1.record()
+        host = (time.perf_counter() - t0) / n_probe
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n_probe, host * 1e3
+
+    with_ms, _ = ticks_ms(False, True)
+    # what a replay costs the host when the queue is empty
+    enqueue = []
+    for i in range(5):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        eng._tick_graphs[i % 2].replay()
         enqueue.append(time.perf_counter() - t0)
-    hard0, steps0 = int(eng.n_hard), int(eng.n_steps)
-    n = new_tokens - 1 - n_eager - n_enqueue
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    e0.record()
-    for _ in range(n):
-        gr.replay()
-    e1.record()
-    host_s = time.perf_counter() - t0
-    torch.cuda.synchronize()
-    step_ms = e0.elapsed_time(e1) / n
-    frac_hard = (int(eng.n_hard) - hard0) / max(int(eng.n_steps) - steps0, 1)
-    # the duo-causal attention part of a step: the same captured step with the q/k preparation and decode
-    # kernels of all layers and both latent iterations left out, replayed on the final cache; the difference
-    # is what those kernels cost inside the step
-    eng.measure_without_attention = True
-    eng._graph = None
-    g0 = eng.capture(0.0, -1)
-    torch.cuda.synchronize()
-    e0.record()
-    for _ in range(extra_steps - 10):
-        g0.replay()
-    e1.record()
-    torch.cuda.synchronize()
-    without_ms = e0.elapsed_time(e1) / (extra_steps - 10)
+    eager_ms, host_eager_ms = ticks_ms(False, False)
+    without_ms, _ = ticks_ms(True, True)
     eng.measure_without_attention = False
-    eng._graph = None
-    attn_ms = max(step_ms - without_ms, 0.0)
-    ctx = float(eng.pos.float().mean())
+    eng._tick_graphs = None
+    attn_ms = max(with_ms - without_ms, 0.0)
     attn_bytes = cfg.layers * B * ctx * 2 * cfg.hkv * cfg.head_dim * 2
     params = sum(t.numel() for L in w.layers for k, t in L.items() if not k.endswith("_p")) + w.embed.numel() + w.norm.numel()
-    return {"workload": f"configs[4]: end-to-end TaH decode, Qwen3-1.7B architecture (28 layers, hidden 2048, 16/8 heads, "
+    return {"workload": "configs[4]: end-to-end TaH decode, Qwen3-1.7B architecture (28 layers, hidden 2048, 16/8 heads, "
                         f"vocab 151936), random weights, B={B}, {prompt_len}-token prompts, {new_tokens} generated tokens, "
                         "greedy sampling, MLP decider 2048->512->1 thresholded at the 94th percentile of the prompt tokens",
-            "tokens_per_s": B / (step_ms * 1e-3), "ms_per_step": step_ms, "steps_timed": n,
+            "tokens_per_s": n_tokens / gen_s, "ms_per_step": step_ms, "steps_timed": ticks,
+            "schedule": "every replay is one pass of all rows, each at the latent iteration its own token needs next "
+                        "(a hard token costs its row two passes, any other one); the loop that keeps the batch in step "
+                        "costs two passes per token",
+            "tokens_per_pass": n_tokens / ticks, "passes_per_token_of_the_slowest_row": ticks / (new_tokens - 1),
             "hard_fraction_decode": frac_hard, "hard_fraction_prompt": float(hard.float().mean()),
-            "attention_ms_per_step": attn_ms, "attention_share_of_step": attn_ms / step_ms,
-            "step_ms_without_attention_kernels": without_ms,
-            "attention_kernels": "duo_decode_step_kernel<2> (q/k preparation + append + attention), 28 layers x 2 iterations",
-            "attention_cache_bytes_per_step": attn_bytes, "attention_cache_gbs": attn_bytes / (attn_ms * 1e-3) / 1e9,
-            "host_enqueue_ms_per_replay": sorted(enqueue)[n_enqueue // 2] * 1e3, "host_ms_per_step_in_loop": host_s / n * 1e3,
-            "eager_ms_per_step": eager_s * 1e3,
-            "host_ms_per_step_eager": host_eager * 1e3, "prefill_s": prefill_s,
-            "weight_bytes": params * 2, "mean_context_at_end": ctx}
+            "pass_ms_at_final_context": with_ms, "attention_ms_per_pass_at_final_context": attn_ms,
+            "attention_share_of_pass_at_final_context": attn_ms / with_ms, "pass_ms_without_attention_kernels": without_ms,
+            "attention_kernels": "duo_decode_step_kernel<2> (q/k preparation + append + attention), 28 layers",
+            "attention_cache_bytes_per_pass_at_final_context": attn_bytes, "attention_cache_gbs": attn_bytes / (attn_ms * 1e-3) / 1e9,
+            "host_enqueue_ms_per_replay": sorted(enqueue)[2] * 1e3, "eager_ms_per_pass": eager_ms, "host_ms_per_pass_eager": host_eager_ms,
+            "prefill_s": prefill_s, "weight_bytes": params * 2, "mean_context_at_end": ctx}
 
 
 def main() -> int:

@@ -326,11 +326,14 @@ int tah_topk_mix(const tah_topk_mix_args* args, tah_stream_t stream);
  * call, i.e. cache.len[slot] -- handed in because the workgroups of a sequence cannot read the length while one of
  * them advances it (len[slot] becomes append_at[i] + 1).  Only for calls tah_duo_decode_step_supported() accepts (256
  * or more (query, kv head) pairs, slabs of at most 4096 rows, one or two query heads per kv head: cases
- * tah_duo_decode runs without split-K); others return TAH_E_SHAPE and the caller makes the two calls.  Replaces, with
+ * tah_duo_decode runs without split-K); others return TAH_E_SHAPE and the caller makes the two calls.  append_depth: NULL,
+ * or int32 [rows], 0 / 1 per row: the segment (dec->c1 / dec->c2) that row's K and V go to, for a batch whose rows are at
+ * different latent iterations (append_at[i] then counts the rows of that segment, and prep->cache only has to be one of
+ * the two).  Replaces, with
  * tah_qk_prep's and tah_duo_decode's lists, one more launch per layer and latent iteration. */
 int tah_duo_decode_step_supported(int32_t nq, int32_t hq, int32_t hkv, int32_t capacity1);
 int tah_duo_decode_step(const tah_qk_prep_args* prep, const tah_duo_decode_args* dec, const int32_t* append_at,
-                        tah_stream_t stream);
+                        const int32_t* append_depth, tah_stream_t stream);
 
 /* Gate of the Qwen3 MLP for a decode step: out[r][i] = silu(gate_up[r][i]) * gate_up[r][inter + i], both
  * steps rounded to bf16 as the eager modules round them -- `act_fn(gate_proj(x)) * up_proj(x)` of Qwen3MLP.forward
@@ -435,6 +438,17 @@ typedef struct tah_step_begin_args {
     int32_t* slot;            /* [rows] out */
     int32_t* q_pos;           /* [rows] out */
     uint8_t* active;          /* [rows] out */
+    /* Optional, for a batch whose rows are at different latent iterations (tah_greedy_tick): phase[i] != 0 means row i
+     * runs the second iteration of its token -- its input is x_alt[i] (the top-k mix the previous tick left there)
+     * instead of the embedding row; q_depth[i] = phase[i]; append_at[i] = hard_len[i] for such rows, pos[i] for the
+     * others (the row count of the segment the row appends to); eligible[i] = active and at the first iteration. */
+    const int32_t* phase;     /* [rows] or NULL */
+    const void* x_alt;        /* bf16 [rows, hidden]; needed with phase */
+    int64_t x_alt_row_stride;
+    const int32_t* hard_len;  /* [rows]; needed with append_at */
+    int32_t* q_depth;         /* [rows] out or NULL */
+    int32_t* append_at;       /* [rows] out or NULL */
+    uint8_t* eligible;        /* [rows] out or NULL */
 } tah_step_begin_args;
 int tah_step_begin(const tah_step_begin_args* args, tah_stream_t stream);
 
@@ -458,6 +472,36 @@ typedef struct tah_decider_tail_args {
     int32_t* q_pos;           /* [rows] out or NULL */
 } tah_decider_tail_args;
 int tah_decider_tail(const tah_decider_tail_args* args, tah_stream_t stream);
+
+/* End of a tick of a generation loop in which every row advances by one latent iteration of its own token, so that a
+ * row whose token needs no second iteration does not wait for those that do (the reference's loop,
+ * tah/model/tah_model.py:580-706 + tah/model/utils.py:228-262, keeps the batch in step; per row the computation and its
+ * result are the same).  phase[i]: 0 = row i just ran the first iteration of a token, 1 = the second.  Rows with
+ * phase 0 and hard_now[i] set only move to phase 1.  Every other unfinished row gets its token -- the arg-max of
+ * `logits`, or of bf16(logits_prev + logits) at phase 1 (logits_prev: what the previous tick's launch left there, the
+ * row's first iteration) -- written to out_tokens[i, out_len[i]]; out_len, pos, tok, finished (end-of-sequence, which is
+ * not written, or `limit` tokens reached), phase = 0, hard_len += 1 and n_hard += 1 after a second iteration,
+ * n_steps += 1. */
+typedef struct tah_greedy_tick_args {
+    const void* logits;       /* bf16 [rows, vocab]: this tick's */
+    const void* logits_prev;  /* bf16 [rows, vocab]: the previous tick's */
+    int64_t row_stride, row_stride_prev; /* elements, multiples of 8 */
+    int32_t rows, vocab;
+    int32_t eos;              /* end-of-sequence token id, < 0 for none */
+    int32_t limit;            /* a row is finished when out_len reaches it */
+    const uint8_t* hard_now;  /* [rows] */
+    int32_t* phase;           /* [rows] in/out */
+    int64_t* tok;             /* [rows] out */
+    uint8_t* finished;        /* [rows] in/out */
+    int32_t* pos;             /* [rows] in/out */
+    int64_t* out_tokens;      /* [rows, out_stride] */
+    int64_t out_stride;
+    int32_t* out_len;         /* [rows] in/out */
+    int32_t* hard_len;        /* [rows] in/out */
+    int64_t* n_hard;
+    int64_t* n_steps;
+} tah_greedy_tick_args;
+int tah_greedy_tick(const tah_greedy_tick_args* args, tah_stream_t stream);
 
 /* Hard-token index build: stream compaction of a (B, S) byte mask in row-major
  * order.  Replaces the stable sort + nonzero of gather_active / scatter_back

@@ -128,6 +128,20 @@ class StepBeginArgs(C.Structure):
         ("rows", c_int32), ("vocab", c_int32), ("hidden", c_int32), ("table_rows", c_int32),
         ("x", c_void_p), ("x_row_stride", c_int64), ("x_packed", c_void_p), ("cos_rows", c_void_p), ("sin_rows", c_void_p),
         ("slot", c_void_p), ("q_pos", c_void_p), ("active", c_void_p),
+        ("phase", c_void_p), ("x_alt", c_void_p), ("x_alt_row_stride", c_int64), ("hard_len", c_void_p),
+        ("q_depth", c_void_p), ("append_at", c_void_p), ("eligible", c_void_p),
+    ]
+
+
+class GreedyTickArgs(C.Structure):
+    """``tah_greedy_tick_args``"""
+
+    _fields_ = [
+        ("logits", c_void_p), ("logits_prev", c_void_p), ("row_stride", c_int64), ("row_stride_prev", c_int64),
+        ("rows", c_int32), ("vocab", c_int32), ("eos", c_int32), ("limit", c_int32),
+        ("hard_now", c_void_p), ("phase", c_void_p), ("tok", c_void_p), ("finished", c_void_p), ("pos", c_void_p),
+        ("out_tokens", c_void_p), ("out_stride", c_int64), ("out_len", c_void_p), ("hard_len", c_void_p),
+        ("n_hard", c_void_p), ("n_steps", c_void_p),
     ]
 
 
@@ -220,13 +234,14 @@ PROTOTYPES = {
     "tah_duo_decode": (C.c_int, [C.POINTER(DuoDecodeArgs), c_void_p]),
     "tah_duo_decode_static": (C.c_int, [C.POINTER(DuoDecodeArgs), c_void_p]),
     "tah_step_begin": (C.c_int, [C.POINTER(StepBeginArgs), c_void_p]),
+    "tah_greedy_tick": (C.c_int, [C.POINTER(GreedyTickArgs), c_void_p]),
     "tah_decider_tail": (C.c_int, [C.POINTER(DeciderTailArgs), c_void_p]),
     "tah_linear_pack_weight": (C.c_int, [c_void_p, c_int64, c_void_p, c_int32, c_int32, c_int32, c_void_p]),
     "tah_linear_pack_rows": (C.c_int, [c_void_p, c_int64, c_void_p, c_int32, c_int32, c_void_p]),
     "tah_linear_rows": (C.c_int, [C.POINTER(LinearRowsArgs), c_void_p]),
     "tah_kv_append": (C.c_int, [C.POINTER(KvAppendArgs), c_void_p]),
     "tah_qk_prep": (C.c_int, [C.POINTER(QkPrepArgs), c_void_p]),
-    "tah_duo_decode_step": (C.c_int, [C.POINTER(QkPrepArgs), C.POINTER(DuoDecodeArgs), c_void_p, c_void_p]),
+    "tah_duo_decode_step": (C.c_int, [C.POINTER(QkPrepArgs), C.POINTER(DuoDecodeArgs), c_void_p, c_void_p, c_void_p]),
     "tah_duo_decode_step_supported": (C.c_int, [c_int32, c_int32, c_int32, c_int32]),
     "tah_topk_mix": (C.c_int, [C.POINTER(TopkMixArgs), c_void_p]),
     "tah_silu_mul": (C.c_int, [c_void_p, c_void_p, c_int32, c_int32, c_int64, c_int64, c_void_p]),

@@ -697,8 +697,10 @@ constexpr int kStepMaxGroup = 2;  // with four query heads per kv head the prepa
 struct StepParams {
     PrepParams prep;
     DecParams dec;
+    AppendParams app[2];           // where a new row goes in the depth-0 / depth-1 segment (slabs, positions, lengths)
     const int32_t* append_at;
-    int32_t append_second;  // the new K/V go to the depth-1 segment
+    const int32_t* append_depth;   // per row 0 / 1, or null: every row appends to segment `append_second`
+    int32_t append_second;
 };
 
 template <int G>
@@ -726,12 +728,14 @@ __global__ __launch_bounds__(kWholeThreads) void duo_decode_step_kernel(const St
     const int aslot = pp.a.slot_of ? pp.a.slot_of[qi] : qi;  // < 0: the row is not cached
     const int dst = sp.append_at[qi];
     const int pos_new = pp.a.pos_new ? pp.a.pos_new[qi] : 0;
-    const bool cached = aslot >= 0, fits = cached && dst < pp.a.capacity;
+    const int adepth = sp.append_depth ? (sp.append_depth[qi] != 0 ? 1 : 0) : sp.append_second;  // uniform per workgroup
+    const AppendParams& ap = sp.app[adepth];
+    const bool cached = aslot >= 0, fits = cached && dst < ap.capacity;
     // rows of a segment: with the new row where this call appends (nobody may read len[] of that segment here)
     auto visible = [&](int seg) {
         const Seg& sg = seg ? p.c2 : p.c1;
         if (seg && qdepth < 1) return 0;
-        const int n = (seg == sp.append_second && cached) ? (fits ? dst + 1 : (dst < pp.a.capacity ? dst : pp.a.capacity)) : sg.len[slot];
+        const int n = (seg == adepth && cached) ? (fits ? dst + 1 : (dst < ap.capacity ? dst : ap.capacity)) : sg.len[slot];
         return seg ? n : (qpos + 1 < n ? (qpos + 1 > 0 ? qpos + 1 : 0) : n);
     };
     constexpr int kBlock = 4 * kUnroll;
@@ -775,12 +779,12 @@ __global__ __launch_bounds__(kWholeThreads) void duo_decode_step_kernel(const St
     sub.pos = pos_new;
     if (cached && !fits && pp.a.overflow && tid == 0 && hk == 0) *pp.a.overflow = 1;
     if (fits && wave == 0 && kq == 0) {
-        const int64_t drow = (int64_t)const_i32(pp.a.start, aslot) + dst;
-        *reinterpret_cast<u32x4*>(pp.a.ck + drow * pp.a.ck_rs + (int64_t)hk * pp.a.ck_hs + 8 * dc) = sub.k;
-        *reinterpret_cast<u32x4*>(pp.a.cv + drow * pp.a.cv_rs + (int64_t)hk * pp.a.cv_hs + 8 * dc) = sub.v;
+        const int64_t drow = (int64_t)const_i32(ap.start, aslot) + dst;
+        *reinterpret_cast<u32x4*>(ap.ck + drow * ap.ck_rs + (int64_t)hk * ap.ck_hs + 8 * dc) = sub.k;
+        *reinterpret_cast<u32x4*>(ap.cv + drow * ap.cv_rs + (int64_t)hk * ap.cv_hs + 8 * dc) = sub.v;
         if (dc == 0 && hk == 0) {
-            if (pp.a.cpos && pp.a.pos_new) pp.a.cpos[(int64_t)aslot * pp.a.capacity + dst] = pos_new;
-            pp.a.len[aslot] = dst + 1;
+            if (ap.cpos && pp.a.pos_new) ap.cpos[(int64_t)aslot * ap.capacity + dst] = pos_new;
+            ap.len[aslot] = dst + 1;
         }
     }
     float m_run[G], l_run[G], acc[G][8];
@@ -792,14 +796,14 @@ __global__ __launch_bounds__(kWholeThreads) void duo_decode_step_kernel(const St
         for (int i = 0; i < 8; ++i) acc[g][i] = 0.f;
     }
     // depth-0 segment: the block loaded above, then the wave's other turns
-    sub.row = (sp.append_second == 0 && fits) ? dst : -1;
+    sub.row = (adepth == 0 && fits) ? dst : -1;
     if (have_first) attend_rows<G, kUnroll, true>(first, false, wave * kBlock, kq, qpos, p.scale_log2e, qv, m_run, l_run, acc, &sub);
     for (int r_it = (wave + kWholeWaves) * kBlock; r_it < nvis0; r_it += kWholeWaves * kBlock)
         consume_rows<G, kUnroll, true>(p.c1, false, kbase0, vbase0, nullptr, r_it, nvis0, kq, qpos, p.scale_log2e, qv, m_run, l_run, acc, &sub);
     // depth-1 segment
     const int nvis1 = visible(1);
     if (nvis1 > 0) {  // uniform per workgroup
-        sub.row = (sp.append_second == 1 && fits) ? dst : -1;
+        sub.row = (adepth == 1 && fits) ? dst : -1;
         const int64_t base1 = p.c2.start[slot];
         const __bf16* kbase1 = p.c2.k + base1 * p.c2.k_rs + (int64_t)hk * p.c2.k_hs + dc * 8;
         const __bf16* vbase1 = p.c2.v + base1 * p.c2.v_rs + (int64_t)hk * p.c2.v_hs + dc * 8;
@@ -1096,8 +1100,24 @@ extern "C" int tah_duo_decode_step_supported(int32_t nq, int32_t hq, int32_t hkv
     return tah::whole_sequence(nq, hq, hkv, capacity1) && hq / hkv <= tah::kStepMaxGroup ? 1 : 0;
 }
 
+namespace tah {
+namespace {
+AppendParams append_target(const tah_kv_segment& c) {
+    AppendParams a{};
+    a.ck = static_cast<__bf16*>(c.k);
+    a.cv = static_cast<__bf16*>(c.v);
+    a.cpos = c.pos;
+    a.start = c.start;
+    a.len = c.len;
+    a.ck_rs = c.k_row_stride; a.ck_hs = c.k_head_stride; a.cv_rs = c.v_row_stride; a.cv_hs = c.v_head_stride;
+    a.capacity = c.capacity;
+    return a;
+}
+}  // namespace
+}  // namespace tah
+
 extern "C" int tah_duo_decode_step(const tah_qk_prep_args* prep, const tah_duo_decode_args* dec, const int32_t* append_at,
-                                   tah_stream_t stream) {
+                                   const int32_t* append_depth, tah_stream_t stream) {
     using namespace tah;
     if (!prep || !dec) return TAH_E_NULL;
     StepParams sp;
@@ -1111,10 +1131,15 @@ extern "C" int tah_duo_decode_step(const tah_qk_prep_args* prep, const tah_duo_d
     if (!prep->append || !prep->append_one_row_per_seq || prep->nseq != prep->rows || !prep->v) return TAH_E_SHAPE;
     if (!tah_duo_decode_step_supported(dec->nq, dec->hq, dec->hkv, dec->c1.capacity)) return TAH_E_SHAPE;
     if (!append_at) return TAH_E_NULL;
+    const bool have2 = dec->q_depth != nullptr || dec->depth >= 1;
     if (prep->cache.k == dec->c1.k) sp.append_second = 0;
-    else if (prep->cache.k == dec->c2.k && (dec->q_depth != nullptr || dec->depth >= 1)) sp.append_second = 1;
+    else if (prep->cache.k == dec->c2.k && have2) sp.append_second = 1;
     else return TAH_E_SHAPE;
+    if (append_depth && !have2) return TAH_E_SHAPE;  // rows that append to the depth-1 segment need it
+    sp.app[0] = append_target(dec->c1);
+    sp.app[1] = have2 ? append_target(dec->c2) : AppendParams{};
     sp.append_at = append_at;
+    sp.append_depth = append_depth;
     hipStream_t st = static_cast<hipStream_t>(stream);
     return dec->hq / dec->hkv == 1 ? launch_step<1>(sp, st) : launch_step<2>(sp, st);
 }

@@ -91,68 +91,71 @@ __device__ __forceinline__ void take_better(float& bv, int& bi, float v, int i) 
     }
 }
 
+// Arg-max over a row of logits a[0 .. vocab) -- of bf16(a + b) when b is given (the running sum of the iterations'
+// logits lives in the model dtype) -- by the whole workgroup; the lower index among equals.  Valid in thread 0.
+__device__ __forceinline__ int row_argmax(const __bf16* a, const __bf16* b, int vocab, float* wv, int* wi) {
+    const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    const bool both = b != nullptr;
+    float bv = -__builtin_inff();
+    int bi = 0x7fffffff;
+    const int nvec = vocab / 8;
+    // four 16-byte pieces per pass, all loaded before the first is looked at: 32 workgroups read 19 MB, and
+    // what a thread waits for is memory latency
+    constexpr int kAhead = 4;
+    for (int c0 = tid; c0 < nvec; c0 += kAhead * kGreedyThreads) {
+        u32x4 x[kAhead], y[kAhead];
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+            const int c = c0 + u * kGreedyThreads;
+            x[u] = y[u] = u32x4{0u, 0u, 0u, 0u};
+            if (c < nvec) {
+                x[u] = *reinterpret_cast<const u32x4*>(a + 8 * c);
+                if (both) y[u] = *reinterpret_cast<const u32x4*>(b + 8 * c);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+            const int c = c0 + u * kGreedyThreads;
+            if (c >= nvec) break;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                float lo = lo_f(x[u][q]), hi = hi_f(x[u][q]);
+                if (both) {
+                    const uint32_t s = pack2(lo + lo_f(y[u][q]), hi + hi_f(y[u][q]));
+                    lo = lo_f(s);
+                    hi = hi_f(s);
+                }
+                if (lo > bv) { bv = lo; bi = 8 * c + 2 * q; }          // indices ascend inside a thread:
+                if (hi > bv) { bv = hi; bi = 8 * c + 2 * q + 1; }      // strict > keeps the first of equals
+            }
+        }
+    }
+    for (int i = nvec * 8 + tid; i < vocab; i += kGreedyThreads) {  // a tail that is not a multiple of 8
+        float v = (float)a[i];
+        if (both) v = (float)(__bf16)(v + (float)b[i]);
+        take_better(bv, bi, v, i);
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) take_better(bv, bi, __shfl_xor(bv, m), __shfl_xor(bi, m));
+    if (lane == 0) {
+        wv[wave] = bv;
+        wi[wave] = bi;
+    }
+    __syncthreads();
+    if (tid != 0) return 0;
+    for (int w = 1; w < kGreedyThreads / kWave; ++w) take_better(bv, bi, wv[w], wi[w]);
+    return bi == 0x7fffffff ? 0 : bi;
+}
+
 __global__ __launch_bounds__(kGreedyThreads) void greedy_step_kernel(const GreedyParams p) {
     __shared__ float wv[kGreedyThreads / kWave];
     __shared__ int wi[kGreedyThreads / kWave];
-    const int row = blockIdx.x, tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
-    const bool active = p.finished[row] == 0;
+    const int row = blockIdx.x, tid = threadIdx.x;
+    const bool active = p.finished[row] == 0;  // uniform per workgroup
     const bool both = p.l1 != nullptr && p.hard != nullptr && p.hard[row] != 0;
-    float bv = -__builtin_inff();
-    int bi = 0x7fffffff;
-    if (active) {
-        const __bf16* a = p.l0 + (int64_t)row * p.rs0;
-        const __bf16* b = both ? p.l1 + (int64_t)row * p.rs1 : nullptr;
-        const int nvec = p.vocab / 8;
-        // four 16-byte pieces per pass, all loaded before the first is looked at: 32 workgroups read 19 MB, and
-        // what a thread waits for is memory latency
-        constexpr int kAhead = 4;
-        for (int c0 = tid; c0 < nvec; c0 += kAhead * kGreedyThreads) {
-            u32x4 x[kAhead], y[kAhead];
-#pragma unroll
-            for (int u = 0; u < kAhead; ++u) {
-                const int c = c0 + u * kGreedyThreads;
-                x[u] = y[u] = u32x4{0u, 0u, 0u, 0u};
-                if (c < nvec) {
-                    x[u] = *reinterpret_cast<const u32x4*>(a + 8 * c);
-                    if (both) y[u] = *reinterpret_cast<const u32x4*>(b + 8 * c);
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < kAhead; ++u) {
-                const int c = c0 + u * kGreedyThreads;
-                if (c >= nvec) break;
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    float lo = lo_f(x[u][q]), hi = hi_f(x[u][q]);
-                    if (both) {  // the running sum of the iterations' logits lives in the model dtype
-                        const uint32_t s = pack2(lo + lo_f(y[u][q]), hi + hi_f(y[u][q]));
-                        lo = lo_f(s);
-                        hi = hi_f(s);
-                    }
-                    if (lo > bv) { bv = lo; bi = 8 * c + 2 * q; }          // indices ascend inside a thread:
-                    if (hi > bv) { bv = hi; bi = 8 * c + 2 * q + 1; }      // strict > keeps the first of equals
-                }
-            }
-        }
-        for (int i = nvec * 8 + tid; i < p.vocab; i += kGreedyThreads) {  // a tail that is not a multiple of 8
-            float v = (float)a[i];
-            if (both) v = (float)(__bf16)(v + (float)b[i]);
-            take_better(bv, bi, v, i);
-        }
-#pragma unroll
-        for (int m = 32; m >= 1; m >>= 1) take_better(bv, bi, __shfl_xor(bv, m), __shfl_xor(bi, m));
-        if (lane == 0) {
-            wv[wave] = bv;
-            wi[wave] = bi;
-        }
-    }
-    __syncthreads();
-    if (tid != 0) return;
     int64_t nxt = 0;
-    if (active) {
-        for (int w = 1; w < kGreedyThreads / kWave; ++w) take_better(bv, bi, wv[w], wi[w]);
-        nxt = bi == 0x7fffffff ? 0 : bi;
-    }
+    if (active) nxt = row_argmax(p.l0 + (int64_t)row * p.rs0, both ? p.l1 + (int64_t)row * p.rs1 : nullptr, p.vocab, wv, wi);
+    if (tid != 0) return;
     // the loop's bookkeeping for this row (tah/model/utils.py:228-262): a row ends with its end-of-sequence token,
     // which is not part of its output; rows that have ended write zeros
     bool done = !active;
@@ -168,6 +171,60 @@ __global__ __launch_bounds__(kGreedyThreads) void greedy_step_kernel(const Greed
     p.tok[row] = nxt;
 }
 
+
+// ---------------------------------------------------------------------------
+// End of a tick of the generation loop in which every row advances by one latent iteration of its own token
+// (rows at different iterations share a batch).  phase[row]: 0 = the row just ran the first iteration of a token,
+// 1 = the second.  A row whose first iteration was called hard only moves to phase 1; every other active row gets
+// its token (arg-max of the first iteration's logits, or of bf16(first + second), the first being the logits the
+// previous tick left in `prev`) and the bookkeeping of greedy_step_kernel, with the row's own output column.
+// ---------------------------------------------------------------------------
+struct TickParams {
+    const __bf16 *cur, *prev;
+    int64_t rs_cur, rs_prev;
+    int32_t vocab, eos, limit;
+    const uint8_t* hard_now;
+    int32_t* phase;
+    int64_t* tok;
+    uint8_t* finished;
+    int32_t *pos, *out_len, *hard_len;
+    int64_t* out_tokens;
+    int64_t out_stride;
+    unsigned long long *n_hard, *n_steps;
+};
+
+__global__ __launch_bounds__(kGreedyThreads) void greedy_tick_kernel(const TickParams p) {
+    __shared__ float wv[kGreedyThreads / kWave];
+    __shared__ int wi[kGreedyThreads / kWave];
+    const int row = blockIdx.x, tid = threadIdx.x;
+    if (p.finished[row] != 0) return;  // uniform per workgroup
+    const int ph = p.phase[row];
+    if (ph == 0 && p.hard_now[row] != 0) {  // the token takes a second iteration: next tick
+        if (tid == 0) p.phase[row] = 1;
+        return;
+    }
+    const bool both = ph != 0;
+    const int64_t nxt = row_argmax(p.cur + (int64_t)row * p.rs_cur, both ? p.prev + (int64_t)row * p.rs_prev : nullptr, p.vocab, wv, wi);
+    if (tid != 0) return;
+    // a row ends with its end-of-sequence token, which is not part of its output (tah/model/utils.py:228-262),
+    // or when it has `limit` tokens
+    bool done = p.eos >= 0 && nxt == p.eos;
+    if (!done) {
+        const int col = p.out_len[row];
+        p.out_tokens[(int64_t)row * p.out_stride + col] = nxt;
+        p.out_len[row] = col + 1;
+        done = col + 1 >= p.limit;
+    }
+    p.finished[row] = done ? 1 : 0;
+    p.pos[row] += 1;
+    p.tok[row] = nxt;
+    p.phase[row] = 0;
+    atomicAdd(p.n_steps, 1ull);
+    if (both) {
+        p.hard_len[row] += 1;  // the second iteration's K/V went into the depth-1 slabs during this tick
+        atomicAdd(p.n_hard, 1ull);
+    }
+}
 
 // ---------------------------------------------------------------------------
 // Glue of a generation step that would otherwise be a dozen element-wise launches each.
@@ -187,23 +244,33 @@ struct StepBeginParams {
     int64_t x_rs;
     int32_t *slot, *q_pos;
     uint8_t* active;
+    // rows at their second latent iteration (phase[row] != 0) take their input from x_alt instead of the embedding
+    const int32_t *phase, *hard_len;
+    const __bf16* x_alt;
+    int64_t x_alt_rs;
+    int32_t *q_depth, *append_at;
+    uint8_t* eligible;
 };
 
 __global__ __launch_bounds__(256) void step_begin_kernel(const StepBeginParams p) {
     const int row = blockIdx.x, tid = threadIdx.x;
     const bool act = p.finished[row] == 0;
     const int pos = p.pos[row];
+    const int ph = p.phase ? (p.phase[row] != 0 ? 1 : 0) : 0;
     if (tid == 0) {
         p.slot[row] = act ? row : -1;
         p.q_pos[row] = act ? pos : -1;
         p.active[row] = act ? 1 : 0;
+        if (p.q_depth) p.q_depth[row] = ph;
+        if (p.append_at) p.append_at[row] = ph ? p.hard_len[row] : pos;
+        if (p.eligible) p.eligible[row] = act && ph == 0 ? 1 : 0;
     }
     const int at = pos < 0 ? 0 : (pos >= p.table_rows ? p.table_rows - 1 : pos);  // a position past the tables reads their last row
     if (tid < 16) *reinterpret_cast<u32x4*>(p.cos_rows + (int64_t)row * 128 + 8 * tid) = *reinterpret_cast<const u32x4*>(p.cos_table + (int64_t)at * 128 + 8 * tid);
     else if (tid < 32) *reinterpret_cast<u32x4*>(p.sin_rows + (int64_t)row * 128 + 8 * (tid - 16)) = *reinterpret_cast<const u32x4*>(p.sin_table + (int64_t)at * 128 + 8 * (tid - 16));
     int64_t t = p.tok[row];
     t = t < 0 ? 0 : (t >= p.vocab ? p.vocab - 1 : t);
-    const __bf16* e = p.embed + t * p.embed_rs;
+    const __bf16* e = ph ? p.x_alt + (int64_t)row * p.x_alt_rs : p.embed + t * p.embed_rs;
     for (int c = 8 * tid; c < p.hidden; c += 8 * 256) {
         const u32x4 v = *reinterpret_cast<const u32x4*>(e + c);
         *reinterpret_cast<u32x4*>(p.x + (int64_t)row * p.x_rs + c) = v;
@@ -322,6 +389,10 @@ extern "C" int tah_step_begin(const tah_step_begin_args* a, tah_stream_t stream)
     p.x = static_cast<__bf16*>(a->x); p.x_packed = static_cast<__bf16*>(a->x_packed);
     p.cos_rows = static_cast<__bf16*>(a->cos_rows); p.sin_rows = static_cast<__bf16*>(a->sin_rows);
     p.x_rs = a->x_row_stride; p.slot = a->slot; p.q_pos = a->q_pos; p.active = a->active;
+    p.phase = a->phase; p.hard_len = a->hard_len; p.x_alt = static_cast<const __bf16*>(a->x_alt); p.x_alt_rs = a->x_alt_row_stride;
+    p.q_depth = a->q_depth; p.append_at = a->append_at; p.eligible = a->eligible;
+    if (p.phase && (!p.x_alt || (p.append_at && !p.hard_len))) return TAH_E_NULL;
+    if ((reinterpret_cast<uintptr_t>(a->x_alt) & 15) || a->x_alt_row_stride % 8 != 0) return TAH_E_ALIGN;
     hipLaunchKernelGGL(step_begin_kernel, dim3(a->rows), dim3(256), 0, static_cast<hipStream_t>(stream), p);
     return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
 }
@@ -338,5 +409,28 @@ extern "C" int tah_decider_tail(const tah_decider_tail_args* a, tah_stream_t str
     p.h_rs = a->hidden_row_stride; p.width = a->width; p.threshold = a->threshold;
     p.active = a->active; p.pos = a->pos; p.hard = a->hard; p.hard_i = a->hard_i32; p.slot = a->slot; p.q_pos = a->q_pos;
     hipLaunchKernelGGL(decider_tail_kernel, dim3(a->rows), dim3(64), 0, static_cast<hipStream_t>(stream), p);
+    return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
+}
+
+extern "C" int tah_greedy_tick(const tah_greedy_tick_args* a, tah_stream_t stream) {
+    using namespace tah;
+    if (!a) return TAH_E_NULL;
+    if (a->rows < 0 || a->vocab <= 0 || a->rows > 65535 || a->limit < 0) return TAH_E_SHAPE;
+    if (a->rows == 0) return TAH_OK;
+    if (!a->logits || !a->logits_prev || !a->hard_now || !a->phase || !a->tok || !a->finished || !a->pos || !a->out_tokens || !a->out_len ||
+        !a->hard_len || !a->n_hard || !a->n_steps)
+        return TAH_E_NULL;
+    if ((reinterpret_cast<uintptr_t>(a->logits) & 15) || (reinterpret_cast<uintptr_t>(a->logits_prev) & 15) || a->row_stride % 8 ||
+        a->row_stride_prev % 8)
+        return TAH_E_ALIGN;
+    TickParams p;
+    p.cur = static_cast<const __bf16*>(a->logits); p.prev = static_cast<const __bf16*>(a->logits_prev);
+    p.rs_cur = a->row_stride; p.rs_prev = a->row_stride_prev;
+    p.vocab = a->vocab; p.eos = a->eos; p.limit = a->limit;
+    p.hard_now = a->hard_now; p.phase = a->phase; p.tok = a->tok; p.finished = a->finished; p.pos = a->pos;
+    p.out_len = a->out_len; p.hard_len = a->hard_len; p.out_tokens = a->out_tokens; p.out_stride = a->out_stride;
+    p.n_hard = reinterpret_cast<unsigned long long*>(a->n_hard);
+    p.n_steps = reinterpret_cast<unsigned long long*>(a->n_steps);
+    hipLaunchKernelGGL(greedy_tick_kernel, dim3(a->rows), dim3(kGreedyThreads), 0, static_cast<hipStream_t>(stream), p);
     return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
 }

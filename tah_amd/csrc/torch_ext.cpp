@@ -31,6 +31,7 @@ struct Api {
     decltype(&tah_greedy_step) greedy_step = nullptr;
     decltype(&tah_silu_mul_normed) silu_mul_normed = nullptr;
     decltype(&tah_step_begin) step_begin = nullptr;
+    decltype(&tah_greedy_tick) greedy_tick = nullptr;
     decltype(&tah_decider_tail) decider_tail = nullptr;
     decltype(&tah_linear_pack_weight) linear_pack_weight = nullptr;
     decltype(&tah_linear_pack_rows) linear_pack_rows = nullptr;
@@ -73,6 +74,7 @@ void load_library(const std::string& path, bool allow_host) {
     bind(g.greedy_step, "tah_greedy_step");
     bind(g.silu_mul_normed, "tah_silu_mul_normed");
     bind(g.step_begin, "tah_step_begin");
+    bind(g.greedy_tick, "tah_greedy_tick");
     bind(g.decider_tail, "tah_decider_tail");
     bind(g.linear_pack_weight, "tah_linear_pack_weight");
     bind(g.linear_pack_rows, "tah_linear_pack_rows");
@@ -498,19 +500,25 @@ void duo_decode_step(const Tensor& q, const Tensor& k, const Tensor& v, const Te
                      const optional<Tensor>& cpos, const Tensor& start, const Tensor& len, const optional<Tensor>& overflow,
                      const Tensor& cu_new, const optional<Tensor>& pos_new, const optional<Tensor>& slot_of,
                      const optional<Tensor>& norm_input, double norm_eps, const Tensor& append_at,
-                     const Tensor& o, const optional<Tensor>& lse, const Tensor& q_slot, const Tensor& q_pos,
+                     const optional<Tensor>& append_depth, const Tensor& o, const optional<Tensor>& lse, const Tensor& q_slot, const Tensor& q_pos,
                      const optional<Tensor>& q_depth, int64_t depth, const Tensor& k1, const Tensor& v1, const Tensor& start1,
                      const Tensor& len1, const optional<Tensor>& k2, const optional<Tensor>& v2, const optional<Tensor>& pos2,
                      const optional<Tensor>& start2, const optional<Tensor>& len2, double scale, const optional<Tensor>& o_packed) {
     need_lib();
-    Dev d; d.see(append_at);
+    Dev d; d.see(append_at); d.see(append_depth);
     i32(append_at, "append_at");
     TORCH_CHECK(append_at.numel() == q.size(0), "duo_decode_step: append_at must have one entry per row");
+    if (append_depth.has_value()) {
+        i32(*append_depth, "append_depth");
+        TORCH_CHECK(append_depth->numel() == q.size(0), "duo_decode_step: append_depth must have one entry per row");
+    }
     const tah_qk_prep_args pa = prep_args(d, q, k, v, c10::nullopt, c10::nullopt, q_weight, k_weight, cos, sin, eps, ck, cv, cpos, start, len,
                                           overflow, cu_new, pos_new, slot_of, true, c10::nullopt, norm_input, norm_eps);
     const tah_duo_decode_args da = decode_args(d, c10::nullopt, o, lse, q_slot, q_pos, q_depth, depth, k1, v1, start1, len1, k2, v2, pos2,
                                                start2, len2, scale, o_packed);
-    check_rc(g.decode_step(&pa, &da, static_cast<const int32_t*>(append_at.data_ptr()), d.stream()), "tah_duo_decode_step");
+    check_rc(g.decode_step(&pa, &da, static_cast<const int32_t*>(append_at.data_ptr()),
+                           append_depth.has_value() ? static_cast<const int32_t*>(append_depth->data_ptr()) : nullptr, d.stream()),
+             "tah_duo_decode_step");
 }
 
 std::tuple<Tensor, Tensor, Tensor, Tensor> hard_index_build(const Tensor& mask) {
@@ -660,11 +668,13 @@ bool vec_of(const Tensor& t, at::ScalarType ty, int64_t n) { return t.scalar_typ
 // tah_step_begin: everything a step needs before its first layer, written into the caller's tensors.
 void step_begin(const Tensor& tok, const Tensor& pos, const Tensor& finished, const Tensor& embed, const Tensor& cos_table,
                 const Tensor& sin_table, const Tensor& x, const optional<Tensor>& x_packed, const Tensor& cos_rows,
-                const Tensor& sin_rows, const Tensor& slot, const Tensor& q_pos, const Tensor& active) {
+                const Tensor& sin_rows, const Tensor& slot, const Tensor& q_pos, const Tensor& active, const optional<Tensor>& phase,
+                const optional<Tensor>& x_alt, const optional<Tensor>& hard_len, const optional<Tensor>& q_depth,
+                const optional<Tensor>& append_at, const optional<Tensor>& eligible) {
     need_lib();
     Dev d;
     for (const Tensor* t : {&tok, &pos, &finished, &embed, &cos_table, &sin_table, &x, &cos_rows, &sin_rows, &slot, &q_pos, &active}) d.see(*t);
-    d.see(x_packed);
+    d.see(x_packed); d.see(phase); d.see(x_alt); d.see(hard_len); d.see(q_depth); d.see(append_at); d.see(eligible);
     const int64_t rows = tok.numel(), hidden = embed.size(1);
     TORCH_CHECK(vec_of(tok, at::kLong, rows) && vec_of(pos, at::kInt, rows) && vec_of(finished, at::kBool, rows) &&
                     vec_of(slot, at::kInt, rows) && vec_of(q_pos, at::kInt, rows) && vec_of(active, at::kBool, rows),
@@ -688,7 +698,52 @@ void step_begin(const Tensor& tok, const Tensor& pos, const Tensor& finished, co
     a.cos_rows = cos_rows.data_ptr(); a.sin_rows = sin_rows.data_ptr();
     a.slot = static_cast<int32_t*>(slot.data_ptr()); a.q_pos = static_cast<int32_t*>(q_pos.data_ptr());
     a.active = static_cast<uint8_t*>(active.data_ptr());
+    for (const optional<Tensor>* t : {&phase, &hard_len, &q_depth, &append_at})
+        if (t->has_value()) TORCH_CHECK(vec_of(**t, at::kInt, rows), "step_begin: phase, hard_len, q_depth and append_at are int32 [rows]");
+    if (eligible.has_value()) TORCH_CHECK(vec_of(*eligible, at::kBool, rows), "step_begin: eligible must be bool [rows]");
+    if (x_alt.has_value())
+        TORCH_CHECK(x_alt->dim() == 2 && x_alt->size(0) == rows && x_alt->size(1) == hidden && x_alt->scalar_type() == at::kBFloat16 &&
+                        (rows == 0 || x_alt->stride(1) == 1),
+                    "step_begin: x_alt must be bf16 [rows, H]");
+    a.phase = phase.has_value() ? static_cast<const int32_t*>(phase->data_ptr()) : nullptr;
+    a.x_alt = x_alt.has_value() ? x_alt->data_ptr() : nullptr;
+    a.x_alt_row_stride = x_alt.has_value() ? (rows > 1 ? x_alt->stride(0) : hidden) : 0;
+    a.hard_len = hard_len.has_value() ? static_cast<const int32_t*>(hard_len->data_ptr()) : nullptr;
+    a.q_depth = q_depth.has_value() ? static_cast<int32_t*>(q_depth->data_ptr()) : nullptr;
+    a.append_at = append_at.has_value() ? static_cast<int32_t*>(append_at->data_ptr()) : nullptr;
+    a.eligible = eligible.has_value() ? static_cast<uint8_t*>(eligible->data_ptr()) : nullptr;
     check_rc(g.step_begin(&a, d.stream()), "tah_step_begin");
+}
+
+// tah_greedy_tick: tokens and bookkeeping at the end of a tick whose rows are at different latent iterations.
+void greedy_tick(const Tensor& logits, const Tensor& logits_prev, int64_t eos, int64_t limit, const Tensor& hard_now, const Tensor& phase,
+                 const Tensor& tok, const Tensor& finished, const Tensor& pos, const Tensor& out_tokens, const Tensor& out_len,
+                 const Tensor& hard_len, const Tensor& n_hard, const Tensor& n_steps) {
+    need_lib();
+    Dev d;
+    for (const Tensor* t : {&logits, &logits_prev, &hard_now, &phase, &tok, &finished, &pos, &out_tokens, &out_len, &hard_len, &n_hard, &n_steps}) d.see(*t);
+    const int64_t rows = logits.size(0), vocab = logits.size(1);
+    for (const Tensor* t : {&logits, &logits_prev})
+        TORCH_CHECK(t->dim() == 2 && t->size(0) == rows && t->size(1) == vocab && t->scalar_type() == at::kBFloat16 && t->stride(1) == 1,
+                    "greedy_tick: logits and logits_prev must be bf16 [rows, vocab]");
+    TORCH_CHECK(vec_of(hard_now, at::kBool, rows) && vec_of(finished, at::kBool, rows), "greedy_tick: hard_now and finished are bool [rows]");
+    for (const Tensor* t : {&phase, &pos, &out_len, &hard_len}) TORCH_CHECK(vec_of(*t, at::kInt, rows), "greedy_tick: phase, pos, out_len and hard_len are int32 [rows]");
+    TORCH_CHECK(vec_of(tok, at::kLong, rows), "greedy_tick: tok must be int64 [rows]");
+    TORCH_CHECK(out_tokens.scalar_type() == at::kLong && out_tokens.dim() == 2 && out_tokens.size(0) == rows && out_tokens.stride(1) == 1 &&
+                    out_tokens.size(1) >= limit,
+                "greedy_tick: out_tokens must be int64 [rows, >= limit]");
+    for (const Tensor* t : {&n_hard, &n_steps}) TORCH_CHECK(t->scalar_type() == at::kLong && t->numel() == 1, "greedy_tick: n_hard and n_steps are int64 scalars");
+    tah_greedy_tick_args a{};
+    a.logits = logits.data_ptr(); a.logits_prev = logits_prev.data_ptr();
+    a.row_stride = rows > 1 ? logits.stride(0) : vocab; a.row_stride_prev = rows > 1 ? logits_prev.stride(0) : vocab;
+    a.rows = (int32_t)rows; a.vocab = (int32_t)vocab; a.eos = (int32_t)eos; a.limit = (int32_t)limit;
+    a.hard_now = static_cast<const uint8_t*>(hard_now.data_ptr()); a.phase = static_cast<int32_t*>(phase.data_ptr());
+    a.tok = static_cast<int64_t*>(tok.data_ptr()); a.finished = static_cast<uint8_t*>(finished.data_ptr());
+    a.pos = static_cast<int32_t*>(pos.data_ptr()); a.out_tokens = static_cast<int64_t*>(out_tokens.data_ptr());
+    a.out_stride = out_tokens.stride(0); a.out_len = static_cast<int32_t*>(out_len.data_ptr());
+    a.hard_len = static_cast<int32_t*>(hard_len.data_ptr());
+    a.n_hard = static_cast<int64_t*>(n_hard.data_ptr()); a.n_steps = static_cast<int64_t*>(n_steps.data_ptr());
+    check_rc(g.greedy_tick(&a, d.stream()), "tah_greedy_tick");
 }
 
 // tah_decider_tail: second layer of the decider, the decision, and the second iteration's per-row bookkeeping.
@@ -808,6 +863,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("duo_decode_step", &duo_decode_step);
     m.def("duo_decode_step_supported", &duo_decode_step_supported);
     m.def("step_begin", &step_begin);
+    m.def("greedy_tick", &greedy_tick);
     m.def("decider_tail", &decider_tail);
     m.def("linear_pack_weight", &linear_pack_weight);
     m.def("linear_pack_rows", &linear_pack_rows);

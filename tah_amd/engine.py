@@ -234,6 +234,16 @@ class TaHDecodeEngine:
             self.slot0, self.qpos0, self.slot1, self.qpos1, self.hard_i = i32(), i32(), i32(), i32(), i32()
             self.act = torch.zeros(batch, dtype=torch.bool, device=dev)
             self.hard = torch.zeros(batch, dtype=torch.bool, device=dev)
+        # Rows at different latent iterations in one batch (generate(..., continuous=True)): a row whose token takes no
+        # second iteration goes on to its next token while others run theirs.  Needs the fused attention launch (it
+        # appends per row to the depth-0 or depth-1 slabs) and the fused glue.
+        self.can_run_continuous = bool(self.fused_glue and self.fused_step)
+        self.phase = torch.zeros(batch, dtype=torch.int32, device=dev)   # 1: the row's next pass is a second iteration
+        if self.can_run_continuous:
+            self.q_depth_rows, self.append_at = i32(), i32()
+            self.eligible = torch.zeros(batch, dtype=torch.bool, device=dev)
+            self.logits2 = [torch.zeros(batch, cfg.vocab, dtype=torch.bfloat16, device=dev) for _ in range(2)]
+        self._tick_graphs = None
 
     # ── model pieces ─────────────────────────────────────────────────────
     def _rms(self, x, w):
@@ -310,9 +320,14 @@ class TaHDecodeEngine:
         xp = self.xp if rows_packed else ops.linear_pack_rows(x, out=self.xp)  # rows_packed: self.xp already holds x
         for l, L in enumerate(self.w.layers):
             q, k, v = self._split_qkv(ops.linear_rows(L["wqkv_p"], xp, B, n_qkv, H))
-            cache = self.slabs0[l] if depth == 0 else self.slabs1[l]
+            cache = self.slabs1[l] if depth == 1 else self.slabs0[l]
             if self.measure_without_attention:  # timing aid: the step minus its q/k preparation and decode kernels
                 ops.linear_pack_rows(q.reshape(B, n_o), out=self.op)
+            elif depth is None:  # every row at its own iteration (q_depth): it appends to that depth's slabs
+                _decode_step(q, k, v, L["qn"], L["kn"], cos, sin, c.rms_eps, cache=self.slabs1[l], cu_new=self.cu_rows,
+                             append_at=self.append_at, append_depth=q_depth, q_slot=self.rows, q_pos=q_pos,
+                             c1=self.slabs0[l], c2=self.slabs1[l], scale=self.scale, slot_of=slot_of, pos_new=pos,
+                             norm_input=x, norm_eps=c.rms_eps, q_depth=q_depth, out_packed=self.op)
             elif self.fused_step:
                 _decode_step(q, k, v, L["qn"], L["kn"], cos, sin, c.rms_eps, cache=cache, cu_new=self.cu_rows,
                              append_at=pos if depth == 0 else self.hard_len, q_slot=self.rows, q_pos=q_pos,
@@ -426,6 +441,8 @@ class TaHDecodeEngine:
         self.n_steps.zero_()
         self.host_hard_rows = 0
         self._graph = None  # (its warm-up step belongs to the old batch's state)
+        self._tick_graphs = None
+        self.phase.zero_()
         seq = torch.repeat_interleave(torch.arange(B, device=dev), torch.tensor(lens, device=dev))
         pos = (torch.arange(N, device=dev) - cu.long()[seq]).to(torch.int32)
         cos, sin = self.cos[pos.long()], self.sin[pos.long()]
@@ -536,17 +553,28 @@ class TaHDecodeEngine:
 
     def _state(self):
         return (self.tok, self.pos, self.finished, self.n_hard, self.n_steps, self.step_idx, self.out_tokens, self.out_len,
-                self.hard_len)
+                self.hard_len, self.phase)
 
     @torch.no_grad()
     def generate(self, first_logits: torch.Tensor, max_new_tokens: int, *, temperature: float = 0.0, eos: int = -1,
-                 use_graph: bool = True, check_every: int = 64, **filters):
+                 use_graph: bool = True, check_every: int = 64, continuous: Optional[bool] = None, **filters):
         """Continues after :meth:`prefill`.  Returns tokens int64 [B, max_new_tokens]; a row's tokens end before its
         end-of-sequence token and are 0 from there on (``self.out_len`` holds each row's count).  With ``eos`` the
-        loop looks every ``check_every`` steps whether all rows are done (the only host synchronisation)."""
+        loop looks every ``check_every`` steps whether all rows are done (the only host synchronisation).
+
+        ``continuous`` (greedy decoding only; default: whenever the engine can): rows do not wait for each other's
+        second latent iterations -- see :meth:`_generate_ticks`.  Same tokens per row."""
         if self.host_positions + max_new_tokens > self.max_len or self.host_hard_rows + max_new_tokens > self.max_hard:
             raise TahDuoError("generation would outgrow the KV slabs: construct the engine with a larger max_len / max_hard")
         dev = self.device
+        greedy_fused = temperature <= 0.0 and self.fused_greedy and self.cfg.vocab % 8 == 0
+        if continuous is None:
+            continuous = self.can_run_continuous and greedy_fused and self.use_fused_glue and not self.measure_without_attention
+        if continuous:
+            if not (self.can_run_continuous and greedy_fused):
+                raise TahDuoError("continuous generation needs greedy decoding and the fused attention and glue launches "
+                                  "(at most 32 rows, 256 (row, kv head) pairs, slabs of at most 4096 rows)")
+            return self._generate_ticks(first_logits, max_new_tokens, eos, use_graph and dev.type == "cuda")
         self.out_tokens.zero_()
         self.out_len.zero_()
         self.step_idx.zero_()
@@ -571,6 +599,92 @@ class TaHDecodeEngine:
                 break
         self.host_positions += done
         self.host_hard_rows += done
+        return self.out_tokens[:, :max_new_tokens]
+
+    # ── rows at different latent iterations in one batch ─────────────────
+    def _tick(self, parity: int, eos: int, limit: int):
+        """Every unfinished row advances by one latent iteration of its own token: the first iteration of its next
+        token (phase 0), or the second iteration of the token whose first the previous tick ran (phase 1).  The
+        logits go to ``self.logits2[parity]``; a row at phase 1 finds its first iteration's logits in the other one."""
+        c, w, B = self.cfg, self.w, self.B
+        ops.step_begin(self.tok, self.pos, self.finished, w.embed, self.cos, self.sin, x=self.x0, x_packed=self.xp,
+                       cos_rows=self.cos_rows, sin_rows=self.sin_rows, slot=self.slot0, q_pos=self.qpos0, active=self.act,
+                       phase=self.phase, x_alt=self.x1, hard_len=self.hard_len, q_depth=self.q_depth_rows,
+                       append_at=self.append_at, eligible=self.eligible)
+        self._pass_single_packed(self.x0, self.pos, None, self.slot0, self.qpos0, self.q_depth_rows, self.cos_rows,
+                                 self.sin_rows, rows_packed=True)
+        logits = ops.linear_rows(w.lm_head_p, self.xp, B, c.vocab, c.hidden, norm_eps=c.rms_eps, out=self.logits2[parity])
+        hr = ops.linear_rows(w.dec_w1_p, self.xp, B, c.decider_hidden, c.hidden, norm_eps=c.rms_eps, bias=w.dec_b1, relu=True)
+        ops.decider_tail(hr, w.dec_w2.reshape(-1), w.dec_b2, w.threshold, hard=self.hard, active=self.eligible)
+        ops.topk_mix(logits, w.embed, c.topk, row_enable=self.hard, out=self.x1)  # (other rows of x1 are not read)
+        ops.greedy_tick(logits, self.logits2[1 - parity], eos, limit, hard_now=self.hard, phase=self.phase, tok=self.tok,
+                        finished=self.finished, pos=self.pos, out_tokens=self.out_tokens, out_len=self.out_len,
+                        hard_len=self.hard_len, n_hard=self.n_hard, n_steps=self.n_steps)
+
+    def capture_ticks(self, eos: int, limit: int):
+        """The tick as two HIP graphs, one per logits buffer, after a warm-up tick whose state changes are undone."""
+        key = (eos, limit, self.w.threshold)
+        if self._tick_graphs is not None and self._tick_key == key:
+            return self._tick_graphs
+        state = [t.clone() for t in self._state()]
+        lens = [sl.len.clone() for sl in self.slabs0 + self.slabs1]
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            self._tick(0, eos, limit)
+        torch.cuda.current_stream().wait_stream(s)
+        torch.cuda.synchronize()
+        for t, old in zip(self._state(), state):
+            t.copy_(old)
+        for sl, ln in zip(self.slabs0 + self.slabs1, lens):
+            sl.len.copy_(ln)
+        graphs = []
+        for parity in (0, 1):
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                self._tick(parity, eos, limit)
+            graphs.append(g)
+        self._tick_graphs, self._tick_key = graphs, key
+        return graphs
+
+    def _generate_ticks(self, first_logits: torch.Tensor, max_new_tokens: int, eos: int, use_graph: bool, check_every: int = 8):
+        """Greedy generation in ticks.  The reference's loop (tah_model.py:580-706 inside utils.py:228-262) keeps the
+        batch in step: every token costs the batch a first iteration and, if any row calls it hard, a second one --
+        here a full pass over the weights for the one row in twelve that needs it.  Rows do not interact, so each row
+        can run its own sequence of passes: a tick is one pass in which every row does the next iteration it needs.  A
+        token costs its row 1 + [hard] ticks instead of 2, and the tokens are the ones the step-wise loop produces.
+        The host looks every ``check_every`` ticks, once the fastest possible row could be done, whether all are."""
+        B = self.B
+        self.out_tokens.zero_()
+        self.out_len.zero_()
+        self.phase.zero_()
+        first = self.sample(first_logits, 0.0)
+        if eos >= 0:
+            self.finished |= first == eos
+        keep = ~self.finished
+        self.out_tokens[:, 0] = torch.where(keep, first, torch.zeros_like(first))
+        self.out_len += keep.to(torch.int32)
+        self.tok.copy_(first)
+        limit = max_new_tokens
+        reached = self.out_len >= limit
+        self.finished |= reached
+        n_min = max_new_tokens - 1
+        graphs = self.capture_ticks(eos, limit) if (use_graph and n_min > 0) else None
+        ticks = 0
+        while n_min > 0:
+            if graphs is not None:
+                graphs[ticks % 2].replay()
+            else:
+                self._tick(ticks % 2, eos, limit)
+            ticks += 1
+            if ticks >= n_min and (ticks - n_min) % check_every == 0 and bool(self.finished.all()):
+                break
+            if ticks > 2 * n_min + check_every:
+                raise TahDuoError("generation did not finish within two passes per token")
+        self.ticks = ticks
+        self.finished &= self.out_len < limit  # rows stopped by the limit have not ended
+        self.host_positions += n_min
+        self.host_hard_rows += n_min
         return self.out_tokens[:, :max_new_tokens]
 
     def capture(self, temperature: float = 0.0, eos: int = -1, **filters):

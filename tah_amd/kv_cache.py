@@ -97,13 +97,15 @@ def decode_step(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_weight: tor
                 scale: float, slot_of: Optional[torch.Tensor] = None, pos_new: Optional[torch.Tensor] = None,
                 norm_input: Optional[torch.Tensor] = None, norm_eps: float = 0.0, depth: int = 0,
                 q_depth: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
-                out_packed: Optional[torch.Tensor] = None) -> torch.Tensor:
+                out_packed: Optional[torch.Tensor] = None, append_depth: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``qk_norm_rope(..., cache=cache, one_row_per_seq=True)`` followed by ``decode(...)`` in one launch
     (``tah_duo_decode_step``), for a generation step: q ``[B, Hq, 128]``, k / v ``[B, Hkv, 128]`` are the projections
     of one new token per sequence, ``cache`` (``c1`` or ``c2``) receives the prepared K and V, and row i attends as
     query i.  ``append_at`` int32 [B]: the rows sequence i's segment of ``cache`` holds before the call (the caller's
     own copy of ``cache.len``: the kernel cannot read the lengths while it advances them).  Same cache contents and
-    lengths as the two calls, bit for bit, and the same outputs up to the last bit of a rare element.  Only for sizes :func:`decode_step_supported` accepts."""
+    lengths as the two calls, bit for bit, and the same outputs up to the last bit of a rare element.  ``append_depth``
+    (int32 [B], 0 / 1): per row the segment (``c1`` / ``c2``) its K and V go to, for a batch whose rows are at different
+    latent iterations; ``append_at`` then counts that segment's rows.  Only for sizes :func:`decode_step_supported` accepts."""
     if q.dim() != 3:
         raise _capi.TahDuoError("decode_step: q must be [B, Hq, D]")
     need2 = q_depth is not None or depth >= 1
@@ -112,7 +114,7 @@ def decode_step(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_weight: tor
     o = out if out is not None else torch.empty_like(q)
     two = (c2.k, c2.v, c2.pos, c2.start, c2.len) if need2 else (None,) * 5
     _call("duo_decode_step", q, k, v, q_weight, k_weight, cos, sin, float(eps), cache.k, cache.v, cache.pos, cache.start,
-          cache.len, cache.overflow, cu_new, pos_new, slot_of, norm_input, float(norm_eps), append_at,
+          cache.len, cache.overflow, cu_new, pos_new, slot_of, norm_input, float(norm_eps), append_at, append_depth,
           o, None, q_slot, q_pos, q_depth, int(depth), c1.k, c1.v, c1.start, c1.len, *two, float(scale), out_packed)
     return o
 

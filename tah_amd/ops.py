@@ -116,12 +116,28 @@ def silu_mul(gate_up: torch.Tensor, norm_input: Optional[torch.Tensor] = None, n
     return _call("silu_mul", gate_up, norm_input, float(norm_eps))
 
 
-def step_begin(tok, pos, finished, embed, cos_table, sin_table, *, x, x_packed, cos_rows, sin_rows, slot, q_pos, active) -> None:
+def step_begin(tok, pos, finished, embed, cos_table, sin_table, *, x, x_packed, cos_rows, sin_rows, slot, q_pos, active,
+               phase=None, x_alt=None, hard_len=None, q_depth=None, append_at=None, eligible=None) -> None:
     """Start of a generation step in one launch (``tah_step_begin``), results written into the keyword tensors: per
     row ``active = ~finished``; ``slot`` = row index and ``q_pos`` = ``pos`` for active rows, -1 otherwise; the rotary
     rows of ``pos`` (clamped into the tables) in ``cos_rows`` / ``sin_rows`` [rows, 128]; the embedding row of ``tok`` in
-    ``x`` [rows, H] and, when given, in ``x_packed`` [32 * H] (the rows operand of ``linear_rows``)."""
-    _call("step_begin", tok, pos, finished, embed, cos_table, sin_table, x, x_packed, cos_rows, sin_rows, slot, q_pos, active)
+    ``x`` [rows, H] and, when given, in ``x_packed`` [32 * H] (the rows operand of ``linear_rows``).
+
+    For a batch whose rows are at different latent iterations (``greedy_tick``): ``phase`` (int32 [rows]) != 0 marks rows at
+    their second iteration, whose input is ``x_alt[row]`` instead of the embedding row; ``q_depth`` receives the phase,
+    ``append_at`` ``hard_len`` for such rows and ``pos`` for the others, ``eligible`` active rows at their first iteration."""
+    _call("step_begin", tok, pos, finished, embed, cos_table, sin_table, x, x_packed, cos_rows, sin_rows, slot, q_pos, active,
+          phase, x_alt, hard_len, q_depth, append_at, eligible)
+
+
+def greedy_tick(logits, logits_prev, eos: int, limit: int, *, hard_now, phase, tok, finished, pos, out_tokens, out_len, hard_len,
+                n_hard, n_steps) -> None:
+    """End of a tick in which every row advanced by one latent iteration of its own token (``tah_greedy_tick``), all
+    updates in place: rows at phase 0 with ``hard_now`` move to phase 1; every other unfinished row gets its token (arg-max
+    of ``logits``, or of ``bf16(logits_prev + logits)`` at phase 1) in ``out_tokens[row, out_len[row]]`` and the loop's
+    bookkeeping; a row is finished at its end-of-sequence token or with ``limit`` tokens."""
+    _call("greedy_tick", logits, logits_prev, int(eos), int(limit), hard_now, phase, tok, finished, pos, out_tokens, out_len,
+          hard_len, n_hard, n_steps)
 
 
 def decider_tail(hidden, w2, b2, threshold: float, *, hard, active=None, pos=None, hard_i32=None, slot=None, q_pos=None) -> None:

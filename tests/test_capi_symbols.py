@@ -47,7 +47,8 @@ def test_struct_sizes_match_c_layout(tmp_path):
              "tah_duo_decode_args": _capi.DuoDecodeArgs, "tah_qk_prep_args": _capi.QkPrepArgs, "tah_topk_mix_args": _capi.TopkMixArgs,
              "tah_kv_append_args": _capi.KvAppendArgs, "tah_additive_mask": _capi.AdditiveMask,
              "tah_greedy_step_args": _capi.GreedyStepArgs, "tah_linear_rows_args": _capi.LinearRowsArgs,
-             "tah_step_begin_args": _capi.StepBeginArgs, "tah_decider_tail_args": _capi.DeciderTailArgs}
+             "tah_step_begin_args": _capi.StepBeginArgs, "tah_decider_tail_args": _capi.DeciderTailArgs,
+             "tah_greedy_tick_args": _capi.GreedyTickArgs}
     assert ctypes.sizeof(_capi.DuoStream) == 9 * 8 + 8 * 8 + 2 * 4
     if shutil.which("gcc") is None:
         return

@@ -318,3 +318,34 @@ def test_engine_can_be_used_for_a_second_batch_gpu():
     fresh = TaHDecodeEngine(w, B, T + new + 2, device="cuda")
     first, _ = fresh.prefill(ids[1], cu)
     assert torch.equal(fresh.generate(first, new), runs[1][0])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("eos", [-1, 7])
+def test_continuous_generation_gives_the_tokens_of_the_stepwise_loop_gpu(eos):
+    """Rows at different latent iterations in one batch (generate(continuous=True)) against the loop that keeps the
+    batch in step: rows do not interact, so tokens, lengths, counters and cache lengths have to be the same; the ticks
+    needed are fewer than two per token."""
+    from tah_amd.engine import EngineConfig, TaHDecodeEngine, Weights
+    cfg = EngineConfig(hidden=256, layers=2, hq=16, hkv=8, head_dim=128, intermediate=768, vocab=4096, decider_hidden=32)
+    w = Weights.random_init(cfg, "cuda", seed=6)
+    B, T, new = 32, 21, 24
+    g = torch.Generator().manual_seed(10)
+    ids = torch.randint(0, cfg.vocab, (B * T,), generator=g).cuda()
+    cu = torch.arange(0, B * T + 1, T, dtype=torch.int32, device="cuda")
+    runs = []
+    for continuous, use_graph in ((False, True), (True, False), (True, True)):
+        eng = TaHDecodeEngine(w, B, T + new + 2, device="cuda")
+        assert eng.can_run_continuous
+        first, _ = eng.prefill(ids, cu, calibrate=0.25)
+        toks = eng.generate(first, new, eos=eos, continuous=continuous, use_graph=use_graph).clone()
+        n_out = eng.out_len.clone()
+        live = torch.arange(new, device="cuda")[None, :] < n_out[:, None]
+        runs.append((torch.where(live, toks, torch.zeros_like(toks)).cpu(), n_out.cpu(), eng.finished.cpu(), int(eng.n_hard),
+                     [sl.len.tolist() for sl in eng.slabs1], getattr(eng, "ticks", None)))
+    ref = runs[0]
+    assert 0 < ref[3]
+    for r in runs[1:]:
+        assert torch.equal(r[0], ref[0]) and torch.equal(r[1], ref[1]) and torch.equal(r[2], ref[2])
+        assert r[3] == ref[3] and r[4] == ref[4]
+        assert new - 1 <= r[5] <= 2 * (new - 1) + 8  # (the host looks every 8 ticks)
