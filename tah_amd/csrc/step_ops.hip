@@ -197,9 +197,12 @@ __global__ __launch_bounds__(kGreedyThreads) void greedy_tick_kernel(const TickP
     __shared__ float wv[kGreedyThreads / kWave];
     __shared__ int wi[kGreedyThreads / kWave];
     const int row = blockIdx.x, tid = threadIdx.x;
-    if (p.finished[row] != 0) return;  // uniform per workgroup
+    const bool ended = p.finished[row] != 0;
     const int ph = p.phase[row];
-    if (ph == 0 && p.hard_now[row] != 0) {  // the token takes a second iteration: next tick
+    const bool again = ph == 0 && p.hard_now[row] != 0;
+    __syncthreads();  // every thread has read the row's state before thread 0 changes it: the branches below are uniform
+    if (ended) return;
+    if (again) {  // the token takes a second iteration: next tick
         if (tid == 0) p.phase[row] = 1;
         return;
     }

@@ -85,3 +85,54 @@ def run(dev, *, B, hq, hkv, seed=0, max_len=90, hidden=256, cap1=128, cap2=64, f
         assert oa[B // 3].abs().max() == 0                                              # the finished row saw nothing
         results[depth] = oa
     return results
+
+
+def run_mixed(dev, *, B, hq, hkv, seed=0, max_len=90, hidden=256, cap1=128, cap2=64):
+    """Rows at different latent iterations in one call (append_depth): rows at depth 0 append to the depth-0 slabs and
+    see them, rows at depth 1 append to the depth-1 slabs (with their position) and see both.  Against two tah_qk_prep
+    calls, one per depth with the other depth's rows masked out, followed by one tah_duo_decode."""
+    from tah_amd import kv_cache
+    g = torch.Generator().manual_seed(seed)
+    lens1 = torch.randint(2, max_len, (B,), generator=g).tolist()
+    lens2 = [int(torch.randint(0, min(l, cap2 - 1), (1,), generator=g)) for l in lens1]
+    c1 = _slabs(B, cap1, hkv, lens1, False, g, dev)
+    c2 = _slabs(B, cap2, hkv, lens2, True, g, dev)
+    for b in range(B):
+        c2.pos[b, :lens2[b]] = torch.sort(torch.randperm(lens1[b] - 1, generator=g)[:lens2[b]]).values.to(torch.int32)
+    rn = lambda *s: torch.randn(*s, generator=g).to(BF).to(dev)
+    q, k, v = rn(B, hq, 128) * 3, rn(B, hkv, 128) * 3, rn(B, hkv, 128)
+    qw, kw = (1 + 0.1 * torch.randn(128, generator=g)).to(BF).to(dev), (1 + 0.1 * torch.randn(128, generator=g)).to(BF).to(dev)
+    x = rn(B, hidden) * 2
+    rows = torch.arange(B, dtype=torch.int32, device=dev)
+    cu = torch.arange(B + 1, dtype=torch.int32, device=dev)
+    ang = torch.randn(B, 128, generator=g)
+    cos, sin = ang.cos().to(BF).to(dev), ang.sin().to(BF).to(dev)
+    active = torch.ones(B, dtype=torch.bool)
+    active[B // 3] = False
+    depth = (torch.rand(B, generator=g) < 0.5)
+    depth[0], depth[1] = True, False
+    active, depth = active.to(dev), depth.to(dev)
+    minus1 = torch.full((B,), -1, dtype=torch.int32, device=dev)
+    # a row at depth 1 has its depth-0 K/V in the slabs already: its position is the last cached one
+    pos = torch.tensor(lens1, dtype=torch.int32, device=dev) - depth.to(torch.int32)
+    q_pos = torch.where(active, pos, minus1)
+    q_depth = depth.to(torch.int32)
+    slot_all = torch.where(active, rows, minus1)
+    scale = 128 ** -0.5
+    a1, a2 = copy.deepcopy(c1), copy.deepcopy(c2)
+    common = dict(cu_new=cu, norm_input=x, norm_eps=1e-6)
+    qo, _ = kv_cache.qk_norm_rope(q, k, qw, kw, cos, sin, 1e-6, v=v, one_row_per_seq=True, cache=a1,
+                                  slot_of=torch.where(active & ~depth, rows, minus1), **common)
+    kv_cache.qk_norm_rope(q, k, qw, kw, cos, sin, 1e-6, v=v, one_row_per_seq=True, cache=a2, pos_new=pos,
+                          slot_of=torch.where(active & depth, rows, minus1), **common)
+    oa = kv_cache.decode(qo, rows, q_pos, a1, a2, scale=scale, q_depth=q_depth)
+    b1, b2 = copy.deepcopy(c1), copy.deepcopy(c2)
+    append_at = torch.where(depth, b2.len, b1.len)
+    ob = kv_cache.decode_step(q, k, v, qw, kw, cos, sin, 1e-6, cache=b2, append_at=append_at, append_depth=q_depth, q_slot=rows,
+                              q_pos=q_pos, c1=b1, c2=b2, scale=scale, slot_of=slot_all, pos_new=pos, q_depth=q_depth, **common)
+    assert torch.allclose(oa.float(), ob.float(), rtol=2.0 ** -7, atol=2.0 ** -12) and (oa != ob).float().mean() < 1e-3
+    for sa, sb in ((a1, b1), (a2, b2)):
+        assert torch.equal(sa.k, sb.k) and torch.equal(sa.v, sb.v) and torch.equal(sa.len, sb.len) and int(sa.overflow) == int(sb.overflow) == 0
+    assert torch.equal(a2.pos, b2.pos)
+    assert torch.equal(b1.len.cpu(), c1.len.cpu() + (active & ~depth).cpu().to(torch.int32))
+    assert torch.equal(b2.len.cpu(), c2.len.cpu() + (active & depth).cpu().to(torch.int32))

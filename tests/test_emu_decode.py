@@ -90,3 +90,4 @@ def test_fused_decode_step_equals_prep_then_decode_on_cpu_shim():
         assert not kv_cache.decode_step_supported(2, 32, 8, 128)  # four query heads per kv head
         decode_step_case.run("cpu", B=3, hq=16, hkv=8, seed=5)
         decode_step_case.run("cpu", B=2, hq=8, hkv=8, seed=6, full_slab=True)
+        decode_step_case.run_mixed("cpu", B=4, hq=8, hkv=8, seed=7)

@@ -131,3 +131,4 @@ def test_fused_decode_step_equals_prep_then_decode(B, hq, hkv):
     assert not kv_cache.decode_step_supported(B, 4 * hkv, hkv, 4096)  # four query heads per kv head: the two calls
     decode_step_case.run("cuda", B=B, hq=hq, hkv=hkv, seed=B + hq, max_len=3000, hidden=2048, cap1=4096, cap2=1024)
     decode_step_case.run("cuda", B=B, hq=hq, hkv=hkv, seed=B + hq + 1, max_len=500, hidden=512, cap2=512, full_slab=True)
+    decode_step_case.run_mixed("cuda", B=B, hq=hq, hkv=hkv, seed=B + hq + 2, max_len=3000, hidden=2048, cap1=4096, cap2=1024)
