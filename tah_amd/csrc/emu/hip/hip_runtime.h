@@ -193,6 +193,7 @@ inline unsigned long long __ballot(int pred) {
     emu::wave_sync();
     return all;
 }
+inline int __popcll(unsigned long long x) { return __builtin_popcountll(x); }
 inline int emu_readfirstlane(int v) { return emu::exchange(v, 0); }
 #define __builtin_amdgcn_readfirstlane emu_readfirstlane
 #define __builtin_amdgcn_ballot_w64(p) __ballot(p)

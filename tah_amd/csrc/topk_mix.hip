@@ -36,6 +36,13 @@ struct MixParams {
 
 // bf16 bits -> unsigned key with the same order as the values (negative values reversed below the positive ones)
 __device__ __forceinline__ uint32_t order_key(uint32_t bits) { return (bits & 0x8000u) ? (~bits & 0xffffu) : (bits | 0x8000u); }
+// the same for the two bf16 halves of a dword at once: bits ^ 0xffff where negative, bits ^ 0x8000 where not
+typedef short i16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t order_keys2(uint32_t w) {
+    const i16x2 fifteen = {15, 15};
+    const i16x2 neg = __builtin_bit_cast(i16x2, w) >> fifteen;  // 0xffff per negative half
+    return w ^ (__builtin_bit_cast(uint32_t, neg) | 0x80008000u);
+}
 __device__ __forceinline__ float key_value(uint32_t key) {
     const uint32_t bits = (key & 0x8000u) ? (key & 0x7fffu) : (~key & 0xffffu);
     return __uint_as_float(bits << 16);
@@ -54,7 +61,53 @@ __device__ __forceinline__ int block_sum(int x, int* red, int wave, int lane) {
     return t;
 }
 
+// Number of threads of the workgroup for which `pred` holds, returned to every thread: one ballot per wave instead of
+// block_sum's six exchanges.
+__device__ __forceinline__ int block_count(bool pred, int* red, int wave, int lane) {
+    const int c = __popcll(__ballot(pred));
+    __syncthreads();  // earlier readers of red are done
+    if (lane == 0) red[wave] = c;
+    __syncthreads();
+    int t = 0;
+#pragma unroll
+    for (int w = 0; w < kMixWaves; ++w) t += red[w];
+    return t;
+}
+
+constexpr int kSearchRows = 6;
+template <int NU, class Pred>
+__device__ __forceinline__ uint32_t search_kth(uint32_t lo, uint32_t hi, int k, int (*tot)[16], int lane, Pred pred) {
+    int round = 0;
+    while (hi - lo > 1 && round < kSearchRows) {
+        const uint32_t step = (hi - lo + 15u) / 16u;
+        auto threshold = [&](int i) { return lo + i * step < hi ? lo + i * step : hi; };  // (scalar arithmetic)
+        int* t = tot[round++];
+        int mine = 0;  // lane i: this wave's count for threshold i
+#pragma unroll
+        for (int i = 1; i < 16; ++i) {
+            const uint32_t th = threshold(i);
+            int c = 0;
+#pragma unroll
+            for (int u = 0; u < NU; ++u) c += __popcll(__ballot(pred(th, u)));
+            mine = lane == i ? c : mine;
+        }
+        if (lane < 16 && mine != 0) atomicAdd(&t[lane], mine);
+        __syncthreads();
+        const unsigned long long ge = __ballot(t[lane & 15] >= k) & 0xfffeull;
+        if (ge == 0ull) {
+            hi = threshold(1);
+        } else {
+            const int i = 63 - __builtin_clzll(ge);
+            const uint32_t nlo = threshold(i), nhi = i == 15 ? hi : threshold(i + 1);
+            lo = nlo;
+            hi = nhi;
+        }
+    }
+    return lo;
+}
+
 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2e __attribute__((ext_vector_type(2)));
 // x rounded to bfloat16 (nearest even), as a float.  Through the packed conversion on purpose: a scalar
@@ -68,6 +121,7 @@ __device__ __forceinline__ float round_bf16(float x) {
 template <int NVEC>
 __global__ __launch_bounds__(kMixThreads) void topk_mix_kernel(const MixParams p) {
     __shared__ int red[kMixWaves];
+    __shared__ int tot[3 * kSearchRows][16];
     __shared__ int sel_idx[kMaxTopk];
     __shared__ float sel_val[kMaxTopk];
     __shared__ int ord_idx[kMaxTopk];
@@ -93,6 +147,8 @@ __global__ __launch_bounds__(kMixThreads) void topk_mix_kernel(const MixParams p
     const int V = p.vocab;
     const int k = p.topk < V ? p.topk : V;
     const __bf16* lrow = p.logits + (int64_t)row * p.l_rs;
+    if (tid < 3 * kSearchRows * 16) (&tot[0][0])[tid] = 0;  // the searches' counters
+    __syncthreads();
 
     // ---- the row as keys: piece j of thread t covers indices (j * 1024 + t) * 8 .. + 7 (coalesced loads) ----
     uint32_t keys[NVEC][4];  // two keys per dword, low half = even index
@@ -115,13 +171,18 @@ __global__ __launch_bounds__(kMixThreads) void topk_mix_kernel(const MixParams p
                     w[e / 2] |= b << (16 * (e % 2));
                 }
             }
+            if ((j + 1) * kMixThreads * 8 <= V) {  // (uniform) the whole piece lies inside the row, for every thread
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                uint32_t lo = order_key(w[q] & 0xffffu), hi = order_key(w[q] >> 16);
-                // indices past the end get key 0 (below every real key) so that they are never selected
-                if (i0 + 2 * q >= V) lo = 0u;
-                if (i0 + 2 * q + 1 >= V) hi = 0u;
-                keys[j][q] = lo | (hi << 16);
+                for (int q = 0; q < 4; ++q) keys[j][q] = order_keys2(w[q]);
+            } else {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    uint32_t lo = order_key(w[q] & 0xffffu), hi = order_key(w[q] >> 16);
+                    // indices past the end get key 0 (below every real key) so that they are never selected
+                    if (i0 + 2 * q >= V) lo = 0u;
+                    if (i0 + 2 * q + 1 >= V) hi = 0u;
+                    keys[j][q] = lo | (hi << 16);
+                }
             }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -132,32 +193,32 @@ __global__ __launch_bounds__(kMixThreads) void topk_mix_kernel(const MixParams p
     // with their indices, and the searches below run over them (two per thread) instead of over the whole row
     // (152 per thread at the full vocabulary).  A row with more candidates than the list holds takes the
     // searches over the whole row.
-    uint32_t tmax = 0u;
+    u16x2 tmax2 = {0, 0};  // the larger key per half, then the larger of the two
 #pragma unroll
     for (int j = 0; j < NVEC; ++j)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            uint32_t w = keys[j][q];
-            TAH_OPAQUE1(w);
-            const uint32_t a = w & 0xffffu, b = w >> 16;
-            tmax = tmax > a ? tmax : a;
-            tmax = tmax > b ? tmax : b;
-        }
-    uint32_t llo = 1u, lhi = 0x10000u;  // invariant: count(tmax >= llo) >= k > count(tmax >= lhi), or llo == 1
-    while (lhi - llo > 1) {
-        const uint32_t mid = (llo + lhi) >> 1;
-        if (block_sum(tmax >= mid ? 1 : 0, red, wave, lane) >= k) llo = mid;
-        else lhi = mid;
-    }
-    const uint32_t L = llo;
+        for (int q = 0; q < 4; ++q) tmax2 = __builtin_elementwise_max(tmax2, __builtin_bit_cast(u16x2, keys[j][q]));
+    const uint32_t tmax = tmax2.x > tmax2.y ? tmax2.x : tmax2.y;
+    // count(tmax >= 1) >= k unless fewer than k threads hold an element (then L = 1), count(tmax >= 0x10000) = 0
+    const uint32_t L = search_kth<1>(1u, 0x10000u, k, tot, lane, [&](uint32_t t, int) { return tmax >= t; });
     if (tid == 0) {
         n_cand = 0;
         n_sel = 0;
     }
     __syncthreads();
     if (tmax >= L) {  // (most threads hold no candidate and skip their row)
+        const uint32_t below = (L - 1u) | ((L - 1u) << 16);  // key >= L  <=>  max(key, L - 1) != L - 1, two keys per dword
 #pragma unroll
         for (int j = 0; j < NVEC; ++j) {
+            uint32_t any = 0u;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                uint32_t w = keys[j][q];
+                TAH_OPAQUE1(w);
+                const u16x2 m = __builtin_elementwise_max(__builtin_bit_cast(u16x2, w), __builtin_bit_cast(u16x2, below));
+                any |= __builtin_bit_cast(uint32_t, m) ^ below;
+            }
+            if (any == 0u) continue;  // none of this piece's eight keys reaches L
             int i0 = (j * kMixThreads + tid) * 8;
             TAH_OPAQUE1(i0);
 #pragma unroll
@@ -194,29 +255,17 @@ __global__ __launch_bounds__(kMixThreads) void topk_mix_kernel(const MixParams p
             return c;
         };
         // largest key T with count(key >= T) >= k; count(key >= L) = ncand >= k
-        uint32_t lo = L, hi = 0x10000u;
-        int n_ge = ncand;
-        while (hi - lo > 1) {
-            const uint32_t mid = (lo + hi) >> 1;
-            const int cnt = block_sum(cnt_ge(mid), red, wave, lane);
-            if (cnt >= k) { lo = mid; n_ge = cnt; }
-            else hi = mid;
-        }
-        const uint32_t T = lo;
+        const uint32_t T = search_kth<kMaxCand / kMixThreads>(L, 0x10000u, k, tot + kSearchRows, lane, [&](uint32_t t, int u) { return ck[u] >= t; });
+        const int n_ge = block_sum(cnt_ge(T), red, wave, lane);
         const int n_gt = block_sum(cnt_ge(T + 1), red, wave, lane);
         const int need_eq = k - n_gt;  // >= 1: that many keys == T are taken, lowest indices first
-        int mlo = 0, mhi = V;          // smallest bound M with count(key == T and index < M) >= need_eq
-        if (n_ge - n_gt > need_eq) {
-            while (mhi - mlo > 1) {
-                const int mid = (mlo + mhi) >> 1;
-                int c = 0;
-#pragma unroll
-                for (int u = 0; u < kMaxCand / kMixThreads; ++u) c += ck[u] == T && ci[u] < mid;
-                if (block_sum(c, red, wave, lane) >= need_eq) mhi = mid;
-                else mlo = mid;
-            }
-        }
-        const int M = mhi;
+        // smallest bound M with count(key == T and index < M) >= need_eq.  More keys == T than needed is the usual
+        // case on a full vocabulary (16-bit keys), so this is the same 16-way search, for the need_eq-th largest
+        // of V - index over the keys == T (empty slots have key 0 < T)
+        int M = V;
+        if (n_ge - n_gt > need_eq)
+            M = V + 1 - (int)search_kth<kMaxCand / kMixThreads>(1u, (uint32_t)V + 1u, need_eq, tot + 2 * kSearchRows, lane,
+                                                                [&](uint32_t t, int u) { return ck[u] == T && (uint32_t)(V - ci[u]) >= t; });
 #pragma unroll
         for (int u = 0; u < kMaxCand / kMixThreads; ++u) {
             if (ck[u] > T || (ck[u] == T && ci[u] < M)) {
@@ -328,9 +377,9 @@ __global__ __launch_bounds__(kMixThreads) void topk_mix_kernel(const MixParams p
         const int cg = cg0 + (cgs >= kMixThreads ? tid : tid % cgs);
         float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         if (cg < cgs && part < parts) {
-            // eight embedding rows are fetched before the first of them is used (one workgroup per token: what
+            // thirteen embedding rows are fetched before the first of them is used (one workgroup per token: what
             // this loop waits for is memory latency), and added in the same order as one by one
-            constexpr int kAhead = 8;
+            constexpr int kAhead = 13;
             for (int i = part; i < n; i += parts * kAhead) {
                 bf16x8 e[kAhead];
 #pragma unroll
