@@ -10,7 +10,7 @@ from tests.qk_prep_cases import assert_bf16_close, make_case, to_torch
 pytestmark = pytest.mark.skipif(not emu_util.have_host_clang(), reason="host clang++ not available")
 
 
-@pytest.mark.parametrize("rows,hq,hkv,scale", [(5, 4, 2, 1.0), (3, 2, 2, 20.0), (4, 8, 1, 0.03)])
+@pytest.mark.parametrize("rows,hq,hkv,scale", [(5, 4, 2, 1.0), (3, 2, 2, 20.0), (4, 8, 1, 0.03), (7, 4, 2, 1.0), (12, 2, 2, 5.0)])
 def test_norm_rope_matches_oracle(rows, hq, hkv, scale):
     from tah_amd.kv_cache import qk_norm_rope
     c = make_case(10 + rows, rows, hq, hkv, scale=scale)
