@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define TAH_DUO_ABI_VERSION 4
+#define TAH_DUO_ABI_VERSION 5
 
 enum {
     TAH_OK = 0,
@@ -306,6 +306,12 @@ typedef struct tah_topk_mix_args {
     void* out_packed;          /* optional: the rows once more as the rows operand of tah_linear_rows, bf16 [32 * hidden]
                                 * (rows <= 32, hidden % 32 == 0; rows past `rows` are not touched) */
     int32_t zero_disabled;     /* != 0: rows whose row_enable byte is 0 are written as zeros instead of left alone */
+    /* Optional: the row's top-k logits themselves, largest first: bf16 [rows, min(topk, vocab)], what
+     * torch.topk(logits, topk).values holds (equal values make the choice among ties invisible here).  The input of
+     * MLPIterDecider's logits_projection (tah/model/iter_decider.py:281).  With values_out set, `out` may be NULL:
+     * then only the values are produced (`embedding`, `hidden` are not used). */
+    void* values_out;
+    int64_t values_row_stride; /* elements */
 } tah_topk_mix_args;
 
 /* Next-iteration input of hard tokens: softmax over each row's top-k logits, then the probability-weighted

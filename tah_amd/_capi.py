@@ -8,7 +8,7 @@ from __future__ import annotations
 
 import ctypes as C
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 c_void_p, c_int32, c_int64, c_float = C.c_void_p, C.c_int32, C.c_int64, C.c_float
 
@@ -215,6 +215,7 @@ class TopkMixArgs(C.Structure):
         ("logits_row_stride", c_int64), ("embedding_row_stride", c_int64), ("out_row_stride", c_int64),
         ("rows", c_int32), ("vocab", c_int32), ("hidden", c_int32), ("topk", c_int32),
         ("out_packed", c_void_p), ("zero_disabled", c_int32),
+        ("values_out", c_void_p), ("values_row_stride", c_int64),
     ]
 
 

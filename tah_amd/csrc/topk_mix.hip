@@ -29,6 +29,8 @@ struct MixParams {
     __bf16* out;
     bf16x8* outp;  // the rows form of the linear-layer kernels ([hidden / 32][2][64][8]) or null
     int32_t zero_disabled;
+    __bf16* vals;  // the selected logits themselves, largest first ([rows, v_rs]), or null
+    int64_t v_rs;
     const uint8_t* row_enable;
     int64_t l_rs, e_rs, o_rs;
     int32_t rows, vocab, hidden, topk;
@@ -135,7 +137,7 @@ __global__ __launch_bounds__(kMixThreads) void topk_mix_kernel(const MixParams p
     const int row = blockIdx.x;
     const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
     if (p.row_enable && !p.row_enable[row]) {  // uniform per workgroup
-        if (p.zero_disabled) {
+        if (p.zero_disabled && p.out) {
             const bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
             for (int cg = tid; cg < p.hidden / 8; cg += kMixThreads) {
                 *reinterpret_cast<bf16x8*>(p.out + (int64_t)row * p.o_rs + cg * 8) = z;
@@ -354,6 +356,15 @@ __global__ __launch_bounds__(kMixThreads) void topk_mix_kernel(const MixParams p
     }
     __syncthreads();
     const int n = n_sel < kMaxTopk ? n_sel : kMaxTopk;  // == k
+    if (p.vals && tid < n) {
+        // largest first: place = how many selected values are larger, equal ones in the order they were collected
+        // (equal values: any order gives the same row)
+        const float mine = sel_val[tid];
+        int place = 0;
+        for (int i = 0; i < n; ++i) place += (sel_val[i] > mine) || (sel_val[i] == mine && i < tid);
+        p.vals[(int64_t)row * p.v_rs + place] = (__bf16)mine;  // (exact: the value came from a bf16)
+    }
+    if (!p.out) return;  // only the values were asked for (uniform)
     // order by index (all distinct): rank = number of selected entries with a smaller index
     float vmax = kNegInf;
     for (int i = 0; i < n; ++i) vmax = fmaxf(vmax, sel_val[i]);
@@ -424,11 +435,14 @@ __global__ __launch_bounds__(kMixThreads) void topk_mix_kernel(const MixParams p
 extern "C" int tah_topk_mix(const tah_topk_mix_args* a, tah_stream_t stream) {
     using namespace tah;
     if (!a) return TAH_E_NULL;
-    if (a->rows < 0 || a->vocab <= 0 || a->hidden <= 0 || a->topk <= 0) return TAH_E_SHAPE;
-    if (a->topk > kMaxTopk || a->vocab > kMaxVec * 8 * kMixThreads || a->hidden % 8 != 0) return TAH_E_SHAPE;
-    if (a->out_packed && (a->rows > 32 || a->hidden % 32 != 0)) return TAH_E_SHAPE;
+    const bool mix = a->out != nullptr;  // without `out` only values_out is produced
+    if (a->rows < 0 || a->vocab <= 0 || a->topk <= 0 || (mix && a->hidden <= 0)) return TAH_E_SHAPE;
+    if (a->topk > kMaxTopk || a->vocab > kMaxVec * 8 * kMixThreads || (mix && a->hidden % 8 != 0)) return TAH_E_SHAPE;
+    if (a->out_packed && (!mix || a->rows > 32 || a->hidden % 32 != 0)) return TAH_E_SHAPE;
+    if (a->values_out && a->values_row_stride < (a->topk < a->vocab ? a->topk : a->vocab)) return TAH_E_SHAPE;
     if (a->rows == 0) return TAH_OK;
-    if (!a->logits || !a->embedding || !a->out) return TAH_E_NULL;
+    if (!a->logits || (!mix && !a->values_out) || (mix && !a->embedding)) return TAH_E_NULL;
+    if (reinterpret_cast<uintptr_t>(a->values_out) & 1) return TAH_E_ALIGN;
     if (reinterpret_cast<uintptr_t>(a->out_packed) & 15) return TAH_E_ALIGN;
     if ((reinterpret_cast<uintptr_t>(a->embedding) & 15) || (reinterpret_cast<uintptr_t>(a->out) & 15) ||
         (reinterpret_cast<uintptr_t>(a->logits) & 1) || a->embedding_row_stride % 8 || a->out_row_stride % 8)
@@ -439,12 +453,14 @@ extern "C" int tah_topk_mix(const tah_topk_mix_args* a, tah_stream_t stream) {
     p.out = static_cast<__bf16*>(a->out);
     p.outp = static_cast<bf16x8*>(a->out_packed);
     p.zero_disabled = a->zero_disabled ? 1 : 0;
+    p.vals = static_cast<__bf16*>(a->values_out);
+    p.v_rs = a->values_row_stride;
     p.row_enable = a->row_enable;
     p.l_rs = a->logits_row_stride; p.e_rs = a->embedding_row_stride; p.o_rs = a->out_row_stride;
     p.rows = a->rows; p.vocab = a->vocab; p.hidden = a->hidden; p.topk = a->topk;
-    const int cgs = a->hidden / 8;
+    const int cgs = mix ? a->hidden / 8 : 1;
     const int parts = cgs >= kMixThreads ? 1 : kMixThreads / cgs;
-    const size_t smem = (size_t)parts * a->hidden * sizeof(float);
+    const size_t smem = mix ? (size_t)parts * a->hidden * sizeof(float) : 0;
     if (smem > 48 * 1024) return TAH_E_SHAPE;  // (32 KiB whenever hidden < 8192)
     const int nvec = (a->vocab + 8 * kMixThreads - 1) / (8 * kMixThreads);
     const dim3 grid(a->rows), block(kMixThreads);

@@ -571,9 +571,9 @@ void rows_copy(const Tensor& src, const optional<Tensor>& src_rows, const Tensor
 }
 
 Tensor topk_mix(const Tensor& logits, const Tensor& embedding, int64_t topk, const optional<Tensor>& row_enable, const optional<Tensor>& out_,
-                const optional<Tensor>& out_packed, bool zero_disabled) {
+                const optional<Tensor>& out_packed, bool zero_disabled, const optional<Tensor>& values_out) {
     need_lib();
-    Dev d; d.see(logits); d.see(embedding); d.see(row_enable); d.see(out_); d.see(out_packed);
+    Dev d; d.see(logits); d.see(embedding); d.see(row_enable); d.see(out_); d.see(out_packed); d.see(values_out);
     TORCH_CHECK(logits.dim() == 2 && embedding.dim() == 2 && logits.scalar_type() == at::kBFloat16 && embedding.scalar_type() == at::kBFloat16,
                 "topk_mix: logits [rows, V] and embedding [V, H] must be bf16");
     TORCH_CHECK(logits.size(1) == embedding.size(0) && logits.stride(1) == 1 && embedding.stride(1) == 1,
@@ -600,8 +600,33 @@ Tensor topk_mix(const Tensor& logits, const Tensor& embedding, int64_t topk, con
     a.rows = (int32_t)rows; a.vocab = (int32_t)logits.size(1); a.hidden = (int32_t)H; a.topk = (int32_t)topk;
     a.out_packed = out_packed.has_value() ? out_packed->data_ptr() : nullptr;
     a.zero_disabled = zero_disabled ? 1 : 0;
+    if (values_out.has_value()) {
+        TORCH_CHECK(values_out->dim() == 2 && values_out->size(0) == rows && values_out->size(1) == std::min<int64_t>(topk, logits.size(1)) &&
+                        values_out->scalar_type() == at::kBFloat16 && values_out->stride(1) == 1,
+                    "topk_mix: values_out must be bf16 [rows, min(topk, V)]");
+        a.values_out = values_out->data_ptr();
+        a.values_row_stride = rows > 1 ? values_out->stride(0) : values_out->size(1);
+    }
     check_rc(g.topk_mix(&a, d.stream()), "tah_topk_mix");
     return out;
+}
+
+// the top-k logits of every row, largest first (tah_topk_mix with values_out only)
+Tensor topk_values(const Tensor& logits, int64_t topk) {
+    need_lib();
+    Dev d; d.see(logits);
+    TORCH_CHECK(logits.dim() == 2 && logits.scalar_type() == at::kBFloat16 && logits.stride(1) == 1 && topk >= 1,
+                "topk_values: logits must be bf16 [rows, V] with a contiguous inner dimension");
+    const int64_t rows = logits.size(0), k = std::min<int64_t>(topk, logits.size(1));
+    Tensor vals = at::empty({rows, k}, logits.options());
+    tah_topk_mix_args a{};
+    a.logits = ptr(logits);
+    a.logits_row_stride = rows > 1 ? logits.stride(0) : logits.size(1);
+    a.rows = (int32_t)rows; a.vocab = (int32_t)logits.size(1); a.hidden = 8; a.topk = (int32_t)topk;
+    a.values_out = vals.data_ptr();
+    a.values_row_stride = k;
+    check_rc(g.topk_mix(&a, d.stream()), "tah_topk_mix");
+    return vals;
 }
 
 Tensor silu_mul(const Tensor& gate_up, const optional<Tensor>& norm_input, double norm_eps) {
@@ -859,6 +884,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("pad_rows_build", &pad_rows_build);
     m.def("rows_copy", &rows_copy);
     m.def("topk_mix", &topk_mix);
+    m.def("topk_values", &topk_values);
     m.def("silu_mul", &silu_mul);
     m.def("duo_decode_step", &duo_decode_step);
     m.def("duo_decode_step_supported", &duo_decode_step_supported);

@@ -98,13 +98,20 @@ def rows_copy(src: torch.Tensor, src_rows: Optional[torch.Tensor], dst: torch.Te
 
 def topk_mix(logits: torch.Tensor, embedding: torch.Tensor, topk: int, row_enable: Optional[torch.Tensor] = None,
              out: Optional[torch.Tensor] = None, out_packed: Optional[torch.Tensor] = None,
-             zero_disabled: bool = False) -> torch.Tensor:
+             zero_disabled: bool = False, values_out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Soft input embedding of hard tokens (tah_model.py:57-75): logits bf16 [rows, V] -> bf16 [rows, H], the
     softmax over each row's top-k logits times the matching rows of ``embedding`` [V, H].  ``row_enable``
     (bool/uint8 [rows]): rows with 0 are skipped and keep what ``out`` held (zeros when ``out`` is not given, or with
     ``zero_disabled``).  ``out_packed`` (bf16 [32 * H], rows <= 32) also receives the rows as the rows operand of
-    ``linear_rows``."""
-    return _call("topk_mix", logits, embedding, int(topk), row_enable, out, out_packed, bool(zero_disabled))
+    ``linear_rows``.  ``values_out`` (bf16 [rows, min(topk, V)]) also receives the top-k logits themselves, largest
+    first, as ``torch.topk(logits, topk).values`` holds them."""
+    return _call("topk_mix", logits, embedding, int(topk), row_enable, out, out_packed, bool(zero_disabled), values_out)
+
+
+def topk_values(logits: torch.Tensor, topk: int) -> torch.Tensor:
+    """``torch.topk(logits, min(topk, V), dim=-1).values`` for bf16 logits [rows, V] (``tah_topk_mix`` producing only
+    its ``values_out``): the logit features of the iteration decider (tah/model/iter_decider.py:281)."""
+    return _call("topk_values", logits, int(topk))
 
 
 def silu_mul(gate_up: torch.Tensor, norm_input: Optional[torch.Tensor] = None, norm_eps: float = 0.0) -> torch.Tensor:

@@ -94,6 +94,40 @@ def test_topk_mix_gpu_vs_torch_ops_on_device_and_strided_logits():
     assert np.array_equal(out.float().cpu().numpy(), z["out"])
 
 
+def _values_check(device, V=3000, rows=3, k=100):
+    """The top-k logits themselves, largest first, equal torch.topk's values to the bit (ties make the indices a
+    matter of choice, the values not): alone and next to the mix; more places than vocabulary entries."""
+    from tah_amd import ops
+    g = torch.Generator().manual_seed(V + rows)
+    logits = (torch.randn(rows, V, generator=g) * 3).to(torch.bfloat16)
+    logits[0, ::7] = logits[0, 0]                      # a plateau
+    logits[-1] = torch.randint(-2, 3, (V,), generator=g).to(torch.bfloat16)   # five distinct values: ties everywhere
+    emb = torch.randn(V, 64, generator=g).to(torch.bfloat16)
+    want = torch.topk(logits.float(), min(k, V), dim=-1).values.to(torch.bfloat16)
+    ld, ed = logits.to(device), emb.to(device)
+    got = ops.topk_values(ld, k)
+    assert got.shape == want.shape and torch.equal(got.cpu(), want)
+    vals = torch.zeros(rows, min(k, V), dtype=torch.bfloat16, device=device)
+    mix = ops.topk_mix(ld, ed, k, values_out=vals)
+    assert torch.equal(vals.cpu(), want) and torch.equal(mix, ops.topk_mix(ld, ed, k))
+    small = ops.topk_values(ld[:, :40].contiguous(), 100)   # more places than entries: every entry, sorted
+    assert torch.equal(small.cpu(), torch.sort(logits[:, :40].float(), dim=-1, descending=True).values.to(torch.bfloat16))
+
+
+@pytest.mark.skipif(not emu_util.have_host_clang(), reason="host clang++ not available")
+def test_topk_values_on_cpu_shim():
+    with emu_util.emulated():
+        _values_check("cpu")
+        _values_check("cpu", V=9000, rows=2, k=17)
+
+
+@pytest.mark.gpu
+def test_topk_values_gpu():
+    _values_check("cuda")
+    _values_check("cuda", V=151936, rows=40, k=100)
+    _values_check("cuda", V=151936, rows=2, k=256)
+
+
 def _silu_mul_check(device):
     """tah_silu_mul against torch's own silu and product in bf16 (the eager modules' arithmetic; a library routine)."""
     import torch.nn.functional as F
