@@ -487,7 +487,8 @@ int tah_decider_tail(const tah_decider_tail_args* args, tah_stream_t stream);
  * `logits`, or of bf16(logits_prev + logits) at phase 1 (logits_prev: what the previous tick's launch left there, the
  * row's first iteration) -- written to out_tokens[i, out_len[i]]; out_len, pos, tok, finished (end-of-sequence, which is
  * not written, or `limit` tokens reached), phase = 0, hard_len += 1 and n_hard += 1 after a second iteration,
- * n_steps += 1. */
+ * n_steps += 1.  With `chosen` set the token of row i is chosen[i] instead of the arg-max (a sampled token, drawn by the
+ * caller from the same final logits); the logits are then not read and may be NULL. */
 typedef struct tah_greedy_tick_args {
     const void* logits;       /* bf16 [rows, vocab]: this tick's */
     const void* logits_prev;  /* bf16 [rows, vocab]: the previous tick's */
@@ -506,6 +507,7 @@ typedef struct tah_greedy_tick_args {
     int32_t* hard_len;        /* [rows] in/out */
     int64_t* n_hard;
     int64_t* n_steps;
+    const int64_t* chosen;    /* [rows] or NULL: take these tokens instead of the arg-max */
 } tah_greedy_tick_args;
 int tah_greedy_tick(const tah_greedy_tick_args* args, tah_stream_t stream);
 

@@ -141,7 +141,7 @@ class GreedyTickArgs(C.Structure):
         ("rows", c_int32), ("vocab", c_int32), ("eos", c_int32), ("limit", c_int32),
         ("hard_now", c_void_p), ("phase", c_void_p), ("tok", c_void_p), ("finished", c_void_p), ("pos", c_void_p),
         ("out_tokens", c_void_p), ("out_stride", c_int64), ("out_len", c_void_p), ("hard_len", c_void_p),
-        ("n_hard", c_void_p), ("n_steps", c_void_p),
+        ("n_hard", c_void_p), ("n_steps", c_void_p), ("chosen", c_void_p),
     ]
 
 

@@ -191,6 +191,7 @@ struct TickParams {
     int64_t* out_tokens;
     int64_t out_stride;
     unsigned long long *n_hard, *n_steps;
+    const int64_t* chosen;
 };
 
 __global__ __launch_bounds__(kGreedyThreads) void greedy_tick_kernel(const TickParams p) {
@@ -207,7 +208,8 @@ __global__ __launch_bounds__(kGreedyThreads) void greedy_tick_kernel(const TickP
         return;
     }
     const bool both = ph != 0;
-    const int64_t nxt = row_argmax(p.cur + (int64_t)row * p.rs_cur, both ? p.prev + (int64_t)row * p.rs_prev : nullptr, p.vocab, wv, wi);
+    const int64_t nxt = p.chosen ? p.chosen[row]  // (uniform)
+                                 : row_argmax(p.cur + (int64_t)row * p.rs_cur, both ? p.prev + (int64_t)row * p.rs_prev : nullptr, p.vocab, wv, wi);
     if (tid != 0) return;
     // a row ends with its end-of-sequence token, which is not part of its output (tah/model/utils.py:228-262),
     // or when it has `limit` tokens
@@ -420,7 +422,7 @@ extern "C" int tah_greedy_tick(const tah_greedy_tick_args* a, tah_stream_t strea
     if (!a) return TAH_E_NULL;
     if (a->rows < 0 || a->vocab <= 0 || a->rows > 65535 || a->limit < 0) return TAH_E_SHAPE;
     if (a->rows == 0) return TAH_OK;
-    if (!a->logits || !a->logits_prev || !a->hard_now || !a->phase || !a->tok || !a->finished || !a->pos || !a->out_tokens || !a->out_len ||
+    if ((!a->chosen && (!a->logits || !a->logits_prev)) || !a->hard_now || !a->phase || !a->tok || !a->finished || !a->pos || !a->out_tokens || !a->out_len ||
         !a->hard_len || !a->n_hard || !a->n_steps)
         return TAH_E_NULL;
     if ((reinterpret_cast<uintptr_t>(a->logits) & 15) || (reinterpret_cast<uintptr_t>(a->logits_prev) & 15) || a->row_stride % 8 ||
@@ -434,6 +436,7 @@ extern "C" int tah_greedy_tick(const tah_greedy_tick_args* a, tah_stream_t strea
     p.out_len = a->out_len; p.hard_len = a->hard_len; p.out_tokens = a->out_tokens; p.out_stride = a->out_stride;
     p.n_hard = reinterpret_cast<unsigned long long*>(a->n_hard);
     p.n_steps = reinterpret_cast<unsigned long long*>(a->n_steps);
+    p.chosen = a->chosen;
     hipLaunchKernelGGL(greedy_tick_kernel, dim3(a->rows), dim3(kGreedyThreads), 0, static_cast<hipStream_t>(stream), p);
     return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
 }

@@ -743,10 +743,11 @@ void step_begin(const Tensor& tok, const Tensor& pos, const Tensor& finished, co
 // tah_greedy_tick: tokens and bookkeeping at the end of a tick whose rows are at different latent iterations.
 void greedy_tick(const Tensor& logits, const Tensor& logits_prev, int64_t eos, int64_t limit, const Tensor& hard_now, const Tensor& phase,
                  const Tensor& tok, const Tensor& finished, const Tensor& pos, const Tensor& out_tokens, const Tensor& out_len,
-                 const Tensor& hard_len, const Tensor& n_hard, const Tensor& n_steps) {
+                 const Tensor& hard_len, const Tensor& n_hard, const Tensor& n_steps, const optional<Tensor>& chosen) {
     need_lib();
     Dev d;
     for (const Tensor* t : {&logits, &logits_prev, &hard_now, &phase, &tok, &finished, &pos, &out_tokens, &out_len, &hard_len, &n_hard, &n_steps}) d.see(*t);
+    d.see(chosen);
     const int64_t rows = logits.size(0), vocab = logits.size(1);
     for (const Tensor* t : {&logits, &logits_prev})
         TORCH_CHECK(t->dim() == 2 && t->size(0) == rows && t->size(1) == vocab && t->scalar_type() == at::kBFloat16 && t->stride(1) == 1,
@@ -768,6 +769,10 @@ void greedy_tick(const Tensor& logits, const Tensor& logits_prev, int64_t eos, i
     a.out_stride = out_tokens.stride(0); a.out_len = static_cast<int32_t*>(out_len.data_ptr());
     a.hard_len = static_cast<int32_t*>(hard_len.data_ptr());
     a.n_hard = static_cast<int64_t*>(n_hard.data_ptr()); a.n_steps = static_cast<int64_t*>(n_steps.data_ptr());
+    if (chosen.has_value()) {
+        TORCH_CHECK(vec_of(*chosen, at::kLong, rows), "greedy_tick: chosen must be int64 [rows]");
+        a.chosen = static_cast<const int64_t*>(chosen->data_ptr());
+    }
     check_rc(g.greedy_tick(&a, d.stream()), "tah_greedy_tick");
 }
 

@@ -562,19 +562,22 @@ class TaHDecodeEngine:
         end-of-sequence token and are 0 from there on (``self.out_len`` holds each row's count).  With ``eos`` the
         loop looks every ``check_every`` steps whether all rows are done (the only host synchronisation).
 
-        ``continuous`` (greedy decoding only; default: whenever the engine can): rows do not wait for each other's
-        second latent iterations -- see :meth:`_generate_ticks`.  Same tokens per row."""
+        ``continuous`` (default: whenever the engine can): rows do not wait for each other's second latent iterations
+        -- see :meth:`_generate_ticks`.  Greedy decoding gives the same tokens per row either way; sampled tokens come from
+        the same per-row distributions but from other random draws (a tick draws for every row, a step once per token)."""
         if self.host_positions + max_new_tokens > self.max_len or self.host_hard_rows + max_new_tokens > self.max_hard:
             raise TahDuoError("generation would outgrow the KV slabs: construct the engine with a larger max_len / max_hard")
         dev = self.device
         greedy_fused = temperature <= 0.0 and self.fused_greedy and self.cfg.vocab % 8 == 0
+        can_tick = self.can_run_continuous and self.fused_greedy and self.cfg.vocab % 8 == 0
         if continuous is None:
-            continuous = self.can_run_continuous and greedy_fused and self.use_fused_glue and not self.measure_without_attention
+            continuous = can_tick and self.use_fused_glue and not self.measure_without_attention
         if continuous:
-            if not (self.can_run_continuous and greedy_fused):
-                raise TahDuoError("continuous generation needs greedy decoding and the fused attention and glue launches "
+            if not can_tick:
+                raise TahDuoError("continuous generation needs the fused attention and glue launches "
                                   "(at most 32 rows, 256 (row, kv head) pairs, slabs of at most 4096 rows)")
-            return self._generate_ticks(first_logits, max_new_tokens, eos, use_graph and dev.type == "cuda")
+            return self._generate_ticks(first_logits, max_new_tokens, eos, use_graph and dev.type == "cuda",
+                                        temperature=temperature, **filters)
         self.out_tokens.zero_()
         self.out_len.zero_()
         self.step_idx.zero_()
@@ -602,7 +605,7 @@ class TaHDecodeEngine:
         return self.out_tokens[:, :max_new_tokens]
 
     # ── rows at different latent iterations in one batch ─────────────────
-    def _tick(self, parity: int, eos: int, limit: int):
+    def _tick(self, parity: int, eos: int, limit: int, temperature: float = 0.0, **filters):
         """Every unfinished row advances by one latent iteration of its own token: the first iteration of its next
         token (phase 0), or the second iteration of the token whose first the previous tick ran (phase 1).  The
         logits go to ``self.logits2[parity]``; a row at phase 1 finds its first iteration's logits in the other one."""
@@ -617,13 +620,20 @@ class TaHDecodeEngine:
         hr = ops.linear_rows(w.dec_w1_p, self.xp, B, c.decider_hidden, c.hidden, norm_eps=c.rms_eps, bias=w.dec_b1, relu=True)
         ops.decider_tail(hr, w.dec_w2.reshape(-1), w.dec_b2, w.threshold, hard=self.hard, active=self.eligible)
         ops.topk_mix(logits, w.embed, c.topk, row_enable=self.hard, out=self.x1)  # (other rows of x1 are not read)
+        chosen = None
+        if temperature > 0.0:
+            # one draw per row from the final logits as the step-wise loop forms them (first iteration, plus the second
+            # where there was one, summed in bf16); rows that only move on to their second iteration ignore theirs
+            prev = self.logits2[1 - parity]
+            final = torch.where((self.phase != 0)[:, None], (prev + logits).float(), logits.float())
+            chosen = self.sample(final, temperature, **filters).contiguous()
         ops.greedy_tick(logits, self.logits2[1 - parity], eos, limit, hard_now=self.hard, phase=self.phase, tok=self.tok,
                         finished=self.finished, pos=self.pos, out_tokens=self.out_tokens, out_len=self.out_len,
-                        hard_len=self.hard_len, n_hard=self.n_hard, n_steps=self.n_steps)
+                        hard_len=self.hard_len, n_hard=self.n_hard, n_steps=self.n_steps, chosen=chosen)
 
-    def capture_ticks(self, eos: int, limit: int):
+    def capture_ticks(self, eos: int, limit: int, temperature: float = 0.0, **filters):
         """The tick as two HIP graphs, one per logits buffer, after a warm-up tick whose state changes are undone."""
-        key = (eos, limit, self.w.threshold)
+        key = (eos, limit, self.w.threshold, temperature, tuple(sorted(filters.items())))
         if self._tick_graphs is not None and self._tick_key == key:
             return self._tick_graphs
         state = [t.clone() for t in self._state()]
@@ -631,7 +641,7 @@ class TaHDecodeEngine:
         s = torch.cuda.Stream()
         s.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(s):
-            self._tick(0, eos, limit)
+            self._tick(0, eos, limit, temperature, **filters)
         torch.cuda.current_stream().wait_stream(s)
         torch.cuda.synchronize()
         for t, old in zip(self._state(), state):
@@ -642,13 +652,14 @@ class TaHDecodeEngine:
         for parity in (0, 1):
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g):
-                self._tick(parity, eos, limit)
+                self._tick(parity, eos, limit, temperature, **filters)
             graphs.append(g)
         self._tick_graphs, self._tick_key = graphs, key
         return graphs
 
-    def _generate_ticks(self, first_logits: torch.Tensor, max_new_tokens: int, eos: int, use_graph: bool, check_every: int = 8):
-        """Greedy generation in ticks.  The reference's loop (tah_model.py:580-706 inside utils.py:228-262) keeps the
+    def _generate_ticks(self, first_logits: torch.Tensor, max_new_tokens: int, eos: int, use_graph: bool, check_every: int = 8,
+                        temperature: float = 0.0, **filters):
+        """Generation in ticks.  The reference's loop (tah_model.py:580-706 inside utils.py:228-262) keeps the
         batch in step: every token costs the batch a first iteration and, if any row calls it hard, a second one --
         here a full pass over the weights for the one row in twelve that needs it.  Rows do not interact, so each row
         can run its own sequence of passes: a tick is one pass in which every row does the next iteration it needs.  A
@@ -658,7 +669,7 @@ class TaHDecodeEngine:
         self.out_tokens.zero_()
         self.out_len.zero_()
         self.phase.zero_()
-        first = self.sample(first_logits, 0.0)
+        first = self.sample(first_logits, temperature, **filters)
         if eos >= 0:
             self.finished |= first == eos
         keep = ~self.finished
@@ -669,13 +680,13 @@ class TaHDecodeEngine:
         reached = self.out_len >= limit
         self.finished |= reached
         n_min = max_new_tokens - 1
-        graphs = self.capture_ticks(eos, limit) if (use_graph and n_min > 0) else None
+        graphs = self.capture_ticks(eos, limit, temperature, **filters) if (use_graph and n_min > 0) else None
         ticks = 0
         while n_min > 0:
             if graphs is not None:
                 graphs[ticks % 2].replay()
             else:
-                self._tick(ticks % 2, eos, limit)
+                self._tick(ticks % 2, eos, limit, temperature, **filters)
             ticks += 1
             if ticks >= n_min and (ticks - n_min) % check_every == 0 and bool(self.finished.all()):
                 break

@@ -138,13 +138,14 @@ def step_begin(tok, pos, finished, embed, cos_table, sin_table, *, x, x_packed, 
 
 
 def greedy_tick(logits, logits_prev, eos: int, limit: int, *, hard_now, phase, tok, finished, pos, out_tokens, out_len, hard_len,
-                n_hard, n_steps) -> None:
+                n_hard, n_steps, chosen=None) -> None:
     """End of a tick in which every row advanced by one latent iteration of its own token (``tah_greedy_tick``), all
     updates in place: rows at phase 0 with ``hard_now`` move to phase 1; every other unfinished row gets its token (arg-max
     of ``logits``, or of ``bf16(logits_prev + logits)`` at phase 1) in ``out_tokens[row, out_len[row]]`` and the loop's
-    bookkeeping; a row is finished at its end-of-sequence token or with ``limit`` tokens."""
+    bookkeeping; a row is finished at its end-of-sequence token or with ``limit`` tokens.  ``chosen`` (int64 [rows]):
+    tokens to take instead of the arg-max (sampled from the same final logits by the caller)."""
     _call("greedy_tick", logits, logits_prev, int(eos), int(limit), hard_now, phase, tok, finished, pos, out_tokens, out_len,
-          hard_len, n_hard, n_steps)
+          hard_len, n_hard, n_steps, chosen)
 
 
 def decider_tail(hidden, w2, b2, threshold: float, *, hard, active=None, pos=None, hard_i32=None, slot=None, q_pos=None) -> None:

@@ -349,3 +349,41 @@ def test_continuous_generation_gives_the_tokens_of_the_stepwise_loop_gpu(eos):
         assert torch.equal(r[0], ref[0]) and torch.equal(r[1], ref[1]) and torch.equal(r[2], ref[2])
         assert r[3] == ref[3] and r[4] == ref[4]
         assert new - 1 <= r[5] <= 2 * (new - 1) + 8  # (the host looks every 8 ticks)
+
+
+@pytest.mark.gpu
+def test_continuous_generation_with_sampling_gpu():
+    """Sampled tokens in ticks.  With a stand-in for the draw that is a function of the final logits alone (their
+    second-largest entry) the tokens have to be those of the step-wise loop, eager and captured; with the real draw the
+    generation runs to its length and every row gets its tokens."""
+    from tah_amd.engine import EngineConfig, TaHDecodeEngine, Weights
+    cfg = EngineConfig(hidden=256, layers=2, hq=16, hkv=8, head_dim=128, intermediate=768, vocab=4096, decider_hidden=32)
+    w = Weights.random_init(cfg, "cuda", seed=7)
+    B, T, new = 32, 17, 20
+    g = torch.Generator().manual_seed(11)
+    ids = torch.randint(0, cfg.vocab, (B * T,), generator=g).cuda()
+    cu = torch.arange(0, B * T + 1, T, dtype=torch.int32, device="cuda")
+
+    def second_best(logits, temperature=0.0, **_):
+        return torch.topk(logits, 2, dim=-1).indices[:, 1] if temperature > 0.0 else torch.argmax(logits, dim=-1)
+
+    runs = []
+    for continuous, use_graph in ((False, True), (True, False), (True, True)):
+        eng = TaHDecodeEngine(w, B, T + new + 2, device="cuda")
+        eng.sample = second_best
+        first, _ = eng.prefill(ids, cu, calibrate=0.25)
+        toks = eng.generate(first, new, temperature=0.7, eos=-1, continuous=continuous, use_graph=use_graph).clone()
+        runs.append((toks.cpu(), eng.out_len.cpu(), int(eng.n_hard), [sl.len.tolist() for sl in eng.slabs1]))
+    assert 0 < runs[0][2] and (runs[0][1] == new).all()
+    for r in runs[1:]:
+        assert torch.equal(r[0], runs[0][0]) and torch.equal(r[1], runs[0][1]) and r[2] == runs[0][2] and r[3] == runs[0][3]
+    greedy = TaHDecodeEngine(w, B, T + new + 2, device="cuda")
+    first, _ = greedy.prefill(ids, cu, calibrate=0.25)
+    assert not torch.equal(greedy.generate(first, new).cpu(), runs[0][0])   # (the stand-in was really used)
+    eng = TaHDecodeEngine(w, B, T + new + 2, device="cuda")
+    first, _ = eng.prefill(ids, cu, calibrate=0.25)
+    toks = eng.generate(first, new, temperature=0.8, top_p=0.9, top_k=50, eos=-1)   # ticks by default, captured
+    assert eng.ticks >= new - 1 and (eng.out_len == new).all() and int(eng.n_steps) == B * (new - 1)
+    assert int(toks.min()) >= 0 and int(toks.max()) < cfg.vocab
+    top50 = torch.topk(first, 50, dim=-1).indices
+    assert (toks[:, :1] == top50).any(dim=-1).all()                          # the first draw obeys the top-k filter

@@ -122,6 +122,16 @@ def _greedy_tick_case(dev, B=7, V=304, limit=5, eos=11):
     for r, col in ((2, 3), (3, 1), (4, 2), (6, limit - 1)):
         want_out[r, col] = want_tok[r]
     assert torch.equal(got["out_tokens"], want_out)
+    # tokens handed in instead of the arg-max (a sampled token): the same bookkeeping around them
+    st = dict(hard_now=d(hard), phase=d(phase), tok=d(tok), finished=d(fin), pos=d(pos), out_tokens=d(out), out_len=d(out_len),
+              hard_len=d(hlen), n_hard=d(n_hard), n_steps=d(n_steps))
+    chosen = torch.tensor([70, 71, 72, 73, eos, 75, 76])
+    ops.greedy_tick(d(cur), d(prev), eos, limit, chosen=d(chosen), **st)
+    got = {k: v.cpu() for k, v in st.items()}
+    assert got["tok"].tolist() == [99, 99, 72, 73, eos, 75, 76] and got["phase"].tolist() == [1, 0, 0, 0, 0, 0, 0]
+    assert got["finished"].tolist() == [False, True, False, False, True, False, True]
+    assert got["out_len"].tolist() == [1, 2, 4, 2, 2, 3, limit] and got["hard_len"].tolist() == [0, 1, 2, 4, 5, 5, 6]
+    assert got["out_tokens"][2, 3] == 72 and got["out_tokens"][3, 1] == 73 and got["out_tokens"][5, 2] == 75 and got["out_tokens"][6, limit - 1] == 76
 
 
 @pytest.mark.skipif(not emu_util.have_host_clang(), reason="host clang++ not available")
