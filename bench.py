@@ -269,7 +269,7 @@ def bench_qk_prep(steps: int, warmup: int):
             "tokens_per_s": rows / (ms * 1e-3)}
 
 
-def bench_e2e_decode(new_tokens: int, B: int = 32, prompt_len: int = 512):
+def bench_e2e_decode(new_tokens: int, B: int = 32, prompt_len: int = 512, temperature: float = 0.0, top_p: float = 0.95):
     """BASELINE configs[4]: end-to-end TaH decode, Qwen3-1.7B architecture with random weights, a two-layer MLP
     decider whose threshold is set so that about 6 % of the prompt tokens iterate, batch 32, 512-token prompts.
     One HIP graph replay per generated token (both latent iterations, sampling included)."""
@@ -292,10 +292,11 @@ def bench_e2e_decode(new_tokens: int, B: int = 32, prompt_len: int = 512):
     prefill_s = time.perf_counter() - t0
     # the generation: greedy, rows at different latent iterations share a batch (one captured tick per replay; a row's
     # token costs it one tick, or two when it is hard), the host looks every 8 ticks whether all rows have their tokens
-    eng.capture_ticks(-1, new_tokens)  # (graph capture is set-up, like the engine's buffers)
+    draw = dict(temperature=temperature, top_p=top_p) if temperature > 0.0 else {}
+    eng.capture_ticks(-1, new_tokens, **draw)  # (graph capture is set-up, like the engine's buffers)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    toks = eng.generate(first, new_tokens, use_graph=True)
+    toks = eng.generate(first, new_tokens, use_graph=True, **draw)
     torch.cuda.synchronize()
     gen_s = time.perf_counter() - t0
     ticks = eng.ticks
@@ -344,7 +345,8 @@ def bench_e2e_decode(new_tokens: int, B: int = 32, prompt_len: int = 512):
     params = sum(t.numel() for L in w.layers for k, t in L.items() if not k.endswith("_p")) + w.embed.numel() + w.norm.numel()
     return {"workload": "configs[4]: end-to-end TaH decode, Qwen3-1.7B architecture (28 layers, hidden 2048, 16/8 heads, "
                         f"vocab 151936), random weights, B={B}, {prompt_len}-token prompts, {new_tokens} generated tokens, "
-                        "greedy sampling, MLP decider 2048->512->1 thresholded at the 94th percentile of the prompt tokens",
+                        + (f"sampling at temperature {temperature}, top-p {top_p}" if temperature > 0.0 else "greedy sampling")
+                        + ", MLP decider 2048->512->1 thresholded at the 94th percentile of the prompt tokens",
             "tokens_per_s": n_tokens / gen_s, "ms_per_step": step_ms, "steps_timed": ticks,
             "schedule": "every replay is one pass of all rows, each at the latent iteration its own token needs next "
                         "(a hard token costs its row two passes, any other one); the loop that keeps the batch in step "
@@ -366,6 +368,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--e2e-tokens", type=int, default=1024, help="generated tokens of the end-to-end decode leg")
+    ap.add_argument("--e2e-temperature", type=float, default=0.0,
+                    help="end-to-end decode leg: sample at this temperature with top-p 0.95 instead of greedy decoding")
     ap.add_argument("--spinup", type=int, default=200,
                     help="untimed launches of the headline kernel before its warm-up steps (the GPU's clock needs tens of "
                          "milliseconds of work to leave its idle state)")
@@ -416,7 +420,7 @@ def main() -> int:
     if args.only in ("all", "qk_prep"):
         legs.append(("qk_prep_prefill", bench_qk_prep(args.steps, args.warmup)))
     if args.only in ("all", "e2e"):
-        legs.append(("e2e_decode", bench_e2e_decode(args.e2e_tokens)))
+        legs.append(("e2e_decode", bench_e2e_decode(args.e2e_tokens, temperature=args.e2e_temperature)))
     for _, leg in legs:
         next(leg)  # runs the leg up to its `yield`: inputs built and resident
     sched = launch_order(ops, dev)
