@@ -269,7 +269,7 @@ def bench_qk_prep(steps: int, warmup: int):
             "tokens_per_s": rows / (ms * 1e-3)}
 
 
-def bench_e2e_decode(new_tokens: int, B: int = 32, prompt_len: int = 512, temperature: float = 0.0, top_p: float = 0.95):
+def bench_e2e_decode(new_tokens: int, B: int = 32, prompt_len: int = 512, temperature: float = 0.0, top_p: float = 0.95, top_k: int = 0):
     """BASELINE configs[4]: end-to-end TaH decode, Qwen3-1.7B architecture with random weights, a two-layer MLP
     decider whose threshold is set so that about 6 % of the prompt tokens iterate, batch 32, 512-token prompts.
     One HIP graph replay per generated token (both latent iterations, sampling included)."""
@@ -292,7 +292,7 @@ def bench_e2e_decode(new_tokens: int, B: int = 32, prompt_len: int = 512, temper
     prefill_s = time.perf_counter() - t0
     # the generation: greedy, rows at different latent iterations share a batch (one captured tick per replay; a row's
     # token costs it one tick, or two when it is hard), the host looks every 8 ticks whether all rows have their tokens
-    draw = dict(temperature=temperature, top_p=top_p) if temperature > 0.0 else {}
+    draw = dict(temperature=temperature, top_p=top_p, top_k=top_k) if temperature > 0.0 else {}
     eng.capture_ticks(-1, new_tokens, **draw)  # (graph capture is set-up, like the engine's buffers)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -345,7 +345,7 @@ def bench_e2e_decode(new_tokens: int, B: int = 32, prompt_len: int = 512, temper
     params = sum(t.numel() for L in w.layers for k, t in L.items() if not k.endswith("_p")) + w.embed.numel() + w.norm.numel()
     return {"workload": "configs[4]: end-to-end TaH decode, Qwen3-1.7B architecture (28 layers, hidden 2048, 16/8 heads, "
                         f"vocab 151936), random weights, B={B}, {prompt_len}-token prompts, {new_tokens} generated tokens, "
-                        + (f"sampling at temperature {temperature}, top-p {top_p}" if temperature > 0.0 else "greedy sampling")
+                        + (f"sampling at temperature {temperature}, top-p {top_p}, top-k {top_k}" if temperature > 0.0 else "greedy sampling")
                         + ", MLP decider 2048->512->1 thresholded at the 94th percentile of the prompt tokens",
             "tokens_per_s": n_tokens / gen_s, "ms_per_step": step_ms, "steps_timed": ticks,
             "schedule": "every replay is one pass of all rows, each at the latent iteration its own token needs next "
@@ -370,6 +370,7 @@ def main() -> int:
     ap.add_argument("--e2e-tokens", type=int, default=1024, help="generated tokens of the end-to-end decode leg")
     ap.add_argument("--e2e-temperature", type=float, default=0.0,
                     help="end-to-end decode leg: sample at this temperature with top-p 0.95 instead of greedy decoding")
+    ap.add_argument("--e2e-top-k", type=int, default=0, help="with --e2e-temperature: top-k filter (0: none)")
     ap.add_argument("--spinup", type=int, default=200,
                     help="untimed launches of the headline kernel before its warm-up steps (the GPU's clock needs tens of "
                          "milliseconds of work to leave its idle state)")
@@ -420,7 +421,7 @@ def main() -> int:
     if args.only in ("all", "qk_prep"):
         legs.append(("qk_prep_prefill", bench_qk_prep(args.steps, args.warmup)))
     if args.only in ("all", "e2e"):
-        legs.append(("e2e_decode", bench_e2e_decode(args.e2e_tokens, temperature=args.e2e_temperature)))
+        legs.append(("e2e_decode", bench_e2e_decode(args.e2e_tokens, temperature=args.e2e_temperature, top_k=args.e2e_top_k)))
     for _, leg in legs:
         next(leg)  # runs the leg up to its `yield`: inputs built and resident
     sched = launch_order(ops, dev)

@@ -312,6 +312,9 @@ typedef struct tah_topk_mix_args {
      * then only the values are produced (`embedding`, `hidden` are not used). */
     void* values_out;
     int64_t values_row_stride; /* elements */
+    /* Optional, with values_out: the vocabulary index of each of those values, int32 [rows, values_row_stride]; equal
+     * values in ascending index order (among equal values at the k-th place the lower indices are the ones taken). */
+    int32_t* indices_out;
 } tah_topk_mix_args;
 
 /* Next-iteration input of hard tokens: softmax over each row's top-k logits, then the probability-weighted

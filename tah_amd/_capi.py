@@ -215,7 +215,7 @@ class TopkMixArgs(C.Structure):
         ("logits_row_stride", c_int64), ("embedding_row_stride", c_int64), ("out_row_stride", c_int64),
         ("rows", c_int32), ("vocab", c_int32), ("hidden", c_int32), ("topk", c_int32),
         ("out_packed", c_void_p), ("zero_disabled", c_int32),
-        ("values_out", c_void_p), ("values_row_stride", c_int64),
+        ("values_out", c_void_p), ("values_row_stride", c_int64), ("indices_out", c_void_p),
     ]
 
 

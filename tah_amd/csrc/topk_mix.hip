@@ -30,6 +30,7 @@ struct MixParams {
     bf16x8* outp;  // the rows form of the linear-layer kernels ([hidden / 32][2][64][8]) or null
     int32_t zero_disabled;
     __bf16* vals;  // the selected logits themselves, largest first ([rows, v_rs]), or null
+    int32_t* idxs;  // their vocabulary indices ([rows, v_rs]), or null
     int64_t v_rs;
     const uint8_t* row_enable;
     int64_t l_rs, e_rs, o_rs;
@@ -357,12 +358,13 @@ __global__ __launch_bounds__(kMixThreads) void topk_mix_kernel(const MixParams p
     __syncthreads();
     const int n = n_sel < kMaxTopk ? n_sel : kMaxTopk;  // == k
     if (p.vals && tid < n) {
-        // largest first: place = how many selected values are larger, equal ones in the order they were collected
-        // (equal values: any order gives the same row)
+        // largest first, equal values by ascending index: place = how many selected entries come before this one
         const float mine = sel_val[tid];
+        const int mine_idx = sel_idx[tid];
         int place = 0;
-        for (int i = 0; i < n; ++i) place += (sel_val[i] > mine) || (sel_val[i] == mine && i < tid);
+        for (int i = 0; i < n; ++i) place += (sel_val[i] > mine) || (sel_val[i] == mine && sel_idx[i] < mine_idx);
         p.vals[(int64_t)row * p.v_rs + place] = (__bf16)mine;  // (exact: the value came from a bf16)
+        if (p.idxs) p.idxs[(int64_t)row * p.v_rs + place] = mine_idx;
     }
     if (!p.out) return;  // only the values were asked for (uniform)
     // order by index (all distinct): rank = number of selected entries with a smaller index
@@ -443,6 +445,8 @@ extern "C" int tah_topk_mix(const tah_topk_mix_args* a, tah_stream_t stream) {
     if (a->rows == 0) return TAH_OK;
     if (!a->logits || (!mix && !a->values_out) || (mix && !a->embedding)) return TAH_E_NULL;
     if (reinterpret_cast<uintptr_t>(a->values_out) & 1) return TAH_E_ALIGN;
+    if (a->indices_out && !a->values_out) return TAH_E_NULL;
+    if (reinterpret_cast<uintptr_t>(a->indices_out) & 3) return TAH_E_ALIGN;
     if (reinterpret_cast<uintptr_t>(a->out_packed) & 15) return TAH_E_ALIGN;
     if ((reinterpret_cast<uintptr_t>(a->embedding) & 15) || (reinterpret_cast<uintptr_t>(a->out) & 15) ||
         (reinterpret_cast<uintptr_t>(a->logits) & 1) || a->embedding_row_stride % 8 || a->out_row_stride % 8)
@@ -454,6 +458,7 @@ extern "C" int tah_topk_mix(const tah_topk_mix_args* a, tah_stream_t stream) {
     p.outp = static_cast<bf16x8*>(a->out_packed);
     p.zero_disabled = a->zero_disabled ? 1 : 0;
     p.vals = static_cast<__bf16*>(a->values_out);
+    p.idxs = a->indices_out;
     p.v_rs = a->values_row_stride;
     p.row_enable = a->row_enable;
     p.l_rs = a->logits_row_stride; p.e_rs = a->embedding_row_stride; p.o_rs = a->out_row_stride;

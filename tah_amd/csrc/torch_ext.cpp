@@ -611,8 +611,8 @@ Tensor topk_mix(const Tensor& logits, const Tensor& embedding, int64_t topk, con
     return out;
 }
 
-// the top-k logits of every row, largest first (tah_topk_mix with values_out only)
-Tensor topk_values(const Tensor& logits, int64_t topk) {
+// the top-k logits of every row, largest first (tah_topk_mix with values_out only), optionally with their indices
+Tensor topk_values(const Tensor& logits, int64_t topk, const optional<Tensor>& indices) {
     need_lib();
     Dev d; d.see(logits);
     TORCH_CHECK(logits.dim() == 2 && logits.scalar_type() == at::kBFloat16 && logits.stride(1) == 1 && topk >= 1,
@@ -625,6 +625,12 @@ Tensor topk_values(const Tensor& logits, int64_t topk) {
     a.rows = (int32_t)rows; a.vocab = (int32_t)logits.size(1); a.hidden = 8; a.topk = (int32_t)topk;
     a.values_out = vals.data_ptr();
     a.values_row_stride = k;
+    if (indices.has_value()) {
+        d.see(*indices);
+        TORCH_CHECK(indices->scalar_type() == at::kInt && indices->dim() == 2 && indices->size(0) == rows && indices->size(1) == k && indices->is_contiguous(),
+                    "topk_values: indices must be a contiguous int32 [rows, min(topk, V)] tensor");
+        a.indices_out = static_cast<int32_t*>(indices->data_ptr());
+    }
     check_rc(g.topk_mix(&a, d.stream()), "tah_topk_mix");
     return vals;
 }

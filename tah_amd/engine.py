@@ -511,6 +511,12 @@ class TaHDecodeEngine:
         captured in a graph."""
         if temperature <= 0.0:
             return torch.argmax(logits, dim=-1)
+        probs = TaHDecodeEngine.filtered_probs(logits, temperature, top_p=top_p, top_k=top_k, min_p=min_p)
+        return torch.argmax(probs / torch.empty_like(probs).exponential_(), dim=-1)
+
+    @staticmethod
+    def filtered_probs(logits: torch.Tensor, temperature: float, *, top_p: float = 1.0, top_k: int = 0, min_p: float = 0.0) -> torch.Tensor:
+        """The distribution ``sample`` draws from: [rows, V], zero outside the filters."""
         probs = F.softmax(logits / temperature if temperature != 1.0 else logits, dim=-1)
         if min_p > 0.0:
             probs = torch.where(probs >= min_p * probs.max(dim=-1, keepdim=True).values, probs, torch.zeros_like(probs))
@@ -525,7 +531,45 @@ class TaHDecodeEngine:
             remove = torch.cat([torch.zeros_like(remove[..., :1]), remove[..., :-1]], dim=-1)  # keep the one that crosses
             probs = torch.where(torch.zeros_like(remove).scatter_(-1, si, remove), torch.zeros_like(probs), probs)
             probs = probs / probs.sum(dim=-1, keepdim=True)
-        return torch.argmax(probs / torch.empty_like(probs).exponential_(), dim=-1)
+        return probs
+
+    # With a top-k filter (0 < top_k <= 256) nothing outside the k largest logits can be drawn, and every filter compares
+    # probabilities with each other, never with the softmax's denominator: the whole of ``sample`` can run on the
+    # [rows, k] values that one ``tah_topk_mix`` launch returns (largest first, with their vocabulary indices) instead
+    # of on [rows, V] -- no sort over the vocabulary, about a millisecond less per step at 32 x 151 936.  One
+    # difference: logits equal to the k-th largest beyond the k-th place stay out (the lower indices are taken),
+    # where ``torch.where(probs < kth, 0, probs)`` (utils.py:113) keeps them all.
+    TOPK_SAMPLING_MAX = 256
+
+    @staticmethod
+    def topk_filtered_probs(vals: torch.Tensor, temperature: float, *, top_p: float = 1.0, min_p: float = 0.0) -> torch.Tensor:
+        """``filtered_probs`` on the k largest logits of every row, ``vals`` [rows, k] sorted largest first."""
+        x = vals.float()
+        probs = F.softmax(x / temperature if temperature != 1.0 else x, dim=-1)
+        if min_p > 0.0:
+            probs = torch.where(probs >= min_p * probs[..., :1], probs, torch.zeros_like(probs))
+            probs = probs / probs.sum(dim=-1, keepdim=True)
+        if top_p < 1.0:
+            remove = torch.cumsum(probs, dim=-1) > top_p
+            remove = torch.cat([torch.zeros_like(remove[..., :1]), remove[..., :-1]], dim=-1)  # keep the one that crosses
+            probs = torch.where(remove, torch.zeros_like(probs), probs)
+            probs = probs / probs.sum(dim=-1, keepdim=True)
+        return probs
+
+    @staticmethod
+    def sample_topk(logits: torch.Tensor, temperature: float, *, top_p: float = 1.0, top_k: int, min_p: float = 0.0) -> torch.Tensor:
+        """``sample`` for bf16 logits [rows, V] and 0 < top_k <= TOPK_SAMPLING_MAX."""
+        vals, idx = ops.topk(logits, top_k)
+        probs = TaHDecodeEngine.topk_filtered_probs(vals, temperature, top_p=top_p, min_p=min_p)
+        j = torch.argmax(probs / torch.empty_like(probs).exponential_(), dim=-1, keepdim=True)
+        return torch.gather(idx, 1, j).squeeze(1).to(torch.int64)
+
+    def _draw(self, final_bf16: torch.Tensor, temperature: float, **filters) -> torch.Tensor:
+        """One token per row from final logits in bf16: on the top-k values when there is a top-k filter, else on the row."""
+        k = int(filters.get("top_k", 0))
+        if 0 < k <= self.TOPK_SAMPLING_MAX and final_bf16.dtype == torch.bfloat16 and final_bf16.size(-1) <= 155648:
+            return self.sample_topk(final_bf16, temperature, **filters)
+        return self.sample(final_bf16.float(), temperature, **filters)
 
     def _step_inplace(self, temperature: float, eos: int, **filters):
         """One generated token for every unfinished row; every state change is an in-place device update."""
@@ -536,8 +580,8 @@ class TaHDecodeEngine:
                             self.n_hard, self.n_steps)
             self.step_idx += 1
             return
-        logits = torch.where(hard[:, None], (l0 + l1).float(), l0.float())  # as step_logits forms them
-        nxt = self.sample(logits, temperature, **filters)
+        logits = torch.where(hard[:, None], l0 + l1, l0)  # as step_logits forms them (the sum in the logits' dtype)
+        nxt = self._draw(logits, temperature, **filters) if temperature > 0.0 else self.sample(logits.float(), 0.0)
         nxt = torch.where(act, nxt, torch.zeros_like(nxt))
         if eos >= 0:
             self.finished |= nxt == eos
@@ -625,8 +669,8 @@ class TaHDecodeEngine:
             # one draw per row from the final logits as the step-wise loop forms them (first iteration, plus the second
             # where there was one, summed in bf16); rows that only move on to their second iteration ignore theirs
             prev = self.logits2[1 - parity]
-            final = torch.where((self.phase != 0)[:, None], (prev + logits).float(), logits.float())
-            chosen = self.sample(final, temperature, **filters).contiguous()
+            final = torch.where((self.phase != 0)[:, None], prev + logits, logits)
+            chosen = self._draw(final, temperature, **filters).contiguous()
         ops.greedy_tick(logits, self.logits2[1 - parity], eos, limit, hard_now=self.hard, phase=self.phase, tok=self.tok,
                         finished=self.finished, pos=self.pos, out_tokens=self.out_tokens, out_len=self.out_len,
                         hard_len=self.hard_len, n_hard=self.n_hard, n_steps=self.n_steps, chosen=chosen)

@@ -111,7 +111,15 @@ def topk_mix(logits: torch.Tensor, embedding: torch.Tensor, topk: int, row_enabl
 def topk_values(logits: torch.Tensor, topk: int) -> torch.Tensor:
     """``torch.topk(logits, min(topk, V), dim=-1).values`` for bf16 logits [rows, V] (``tah_topk_mix`` producing only
     its ``values_out``): the logit features of the iteration decider (tah/model/iter_decider.py:281)."""
-    return _call("topk_values", logits, int(topk))
+    return _call("topk_values", logits, int(topk), None)
+
+
+def topk(logits: torch.Tensor, k: int):
+    """``(values, indices)`` of the k largest entries of every row of bf16 logits [rows, V], largest first, equal values by
+    ascending index (``torch.topk`` leaves the order and the choice among equal values open): values bf16, indices int32.
+    k <= 256."""
+    idx = torch.empty(logits.size(0), min(int(k), logits.size(1)), dtype=torch.int32, device=logits.device)
+    return _call("topk_values", logits, int(k), idx), idx
 
 
 def silu_mul(gate_up: torch.Tensor, norm_input: Optional[torch.Tensor] = None, norm_eps: float = 0.0) -> torch.Tensor:

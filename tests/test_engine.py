@@ -387,3 +387,46 @@ def test_continuous_generation_with_sampling_gpu():
     assert int(toks.min()) >= 0 and int(toks.max()) < cfg.vocab
     top50 = torch.topk(first, 50, dim=-1).indices
     assert (toks[:, :1] == top50).any(dim=-1).all()                          # the first draw obeys the top-k filter
+
+
+def _topk_sampling_case(device, V, rows=6, draws=True):
+    """The distribution over the k largest logits that sample_topk draws from against the one the reference's filters
+    leave on the whole row (utils.py:84-125), on rows without equal values; and the draws land where it is not zero."""
+    from tah_amd import ops
+    from tah_amd.engine import TaHDecodeEngine as E
+    g = torch.Generator().manual_seed(V)
+    # 300 different values from the bf16 grid of [1, 8) at random places (every filter's boundary falls among them),
+    # the rest of the row below them
+    grid = torch.arange(0x3F80, 0x4100, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    logits = (torch.rand(rows, V, generator=g) * 4 - 3.2).to(torch.bfloat16)
+    for r in range(rows):
+        logits[r, torch.randperm(V, generator=g)[:300]] = grid[torch.randperm(grid.numel(), generator=g)[:300]]
+    logits = logits.to(device)
+    for T, top_p, top_k, min_p in ((0.6, 0.95, 20, 0.0), (1.0, 1.0, 50, 0.0), (0.8, 0.7, 256, 0.05), (1.3, 0.9, 1, 0.0))[:4 if draws else 3]:
+        want = E.filtered_probs(logits.float(), T, top_p=top_p, top_k=top_k, min_p=min_p)
+        vals, idx = ops.topk(logits, top_k)
+        got = torch.zeros_like(want).scatter_(1, idx.long(), E.topk_filtered_probs(vals, T, top_p=top_p, min_p=min_p))
+        assert torch.allclose(got, want, rtol=1e-4, atol=1e-7), float((got - want).abs().max())
+        assert torch.equal(got > 0, want > 0)
+        for _ in range(3 if draws else 1):
+            tok = E.sample_topk(logits, T, top_p=top_p, top_k=top_k, min_p=min_p)
+            assert tok.dtype == torch.int64 and (torch.gather(want, 1, tok[:, None]) > 0).all()
+    if not draws:
+        return
+    # a draw follows the distribution: two tokens at 3:1
+    two = torch.full((1, V), -30.0, dtype=torch.bfloat16, device=device)
+    two[0, 5], two[0, 9] = 1.0986, 0.0
+    draws = torch.stack([E.sample_topk(two.expand(64, V).contiguous(), 1.0, top_k=4) for _ in range(40)]).flatten()
+    assert set(draws.tolist()) == {5, 9} and 0.70 < float((draws == 5).float().mean()) < 0.80
+
+
+@pytest.mark.skipif(not emu_util.have_host_clang(), reason="host clang++ not available")
+def test_sampling_on_the_topk_values_on_cpu_shim():
+    with emu_util.emulated():
+        _topk_sampling_case("cpu", 3000, rows=2, draws=False)
+
+
+@pytest.mark.gpu
+def test_sampling_on_the_topk_values_gpu():
+    _topk_sampling_case("cuda", 20000)
+

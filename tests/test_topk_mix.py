@@ -110,6 +110,15 @@ def _values_check(device, V=3000, rows=3, k=100):
     vals = torch.zeros(rows, min(k, V), dtype=torch.bfloat16, device=device)
     mix = ops.topk_mix(ld, ed, k, values_out=vals)
     assert torch.equal(vals.cpu(), want) and torch.equal(mix, ops.topk_mix(ld, ed, k))
+    v2, i2 = ops.topk(ld, k)                                # with the indices: the values sit there, equal ones by ascending index
+    assert torch.equal(v2.cpu(), want) and torch.equal(torch.gather(logits, 1, i2.cpu().long()), want)
+    for r in range(rows):
+        vv, ii = want[r].float(), i2[r].cpu()
+        assert all(vv[j] > vv[j + 1] or ii[j] < ii[j + 1] for j in range(len(ii) - 1))
+        kth = vv[-1]
+        taken = set(ii[vv == kth].tolist())
+        ties = (logits[r].float() == kth).nonzero().flatten().tolist()
+        assert taken == set(ties[:len(taken)])               # at the k-th place the lower indices
     small = ops.topk_values(ld[:, :40].contiguous(), 100)   # more places than entries: every entry, sorted
     assert torch.equal(small.cpu(), torch.sort(logits[:, :40].float(), dim=-1, descending=True).values.to(torch.bfloat16))
 
