@@ -114,3 +114,29 @@ def test_argument_checks_run_before_any_device_work():
         g.do_row_stride = g.dq_row_stride = g.dk_row_stride = g.dv_row_stride = 1024
         g.do_head_stride = g.dq_head_stride = g.dk_head_stride = g.dv_head_stride = 128
     assert lib.tah_duo_bwd_varlen(ctypes.byref(b), None) == _capi.TAH_E_SHAPE
+
+
+def test_topk_mix_argument_checks():
+    """tah_topk_mix with its optional outputs: what has to be there, in which shape, before anything is launched."""
+    from tah_amd import _capi, _lib
+    lib = _capi.bind(ctypes.CDLL(_lib.LIB_PATH))
+
+    def args(**kw):
+        a = _capi.TopkMixArgs()
+        a.logits, a.embedding, a.out = 0x10000, 0x20000, 0x30000
+        a.logits_row_stride, a.embedding_row_stride, a.out_row_stride = 4096, 64, 64
+        a.rows, a.vocab, a.hidden, a.topk = 2, 4096, 64, 100
+        for k, v in kw.items():
+            setattr(a, k, v)
+        return a
+
+    call = lambda a: lib.tah_topk_mix(ctypes.byref(a), None)
+    assert call(args(topk=257)) == _capi.TAH_E_SHAPE                                       # more places than the kernel holds
+    assert call(args(out=0)) == _capi.TAH_E_NULL                                           # neither the mix nor the values
+    assert call(args(out=0, indices_out=0x50000)) == _capi.TAH_E_NULL                      # indices without values
+    assert call(args(values_out=0x40000, values_row_stride=99)) == _capi.TAH_E_SHAPE       # rows of values would overlap
+    assert call(args(values_out=0x40001, values_row_stride=100)) == _capi.TAH_E_ALIGN
+    assert call(args(values_out=0x40000, values_row_stride=100, indices_out=0x50002)) == _capi.TAH_E_ALIGN
+    assert call(args(out=0, values_out=0x40000, values_row_stride=100, out_packed=0x60000)) == _capi.TAH_E_SHAPE  # packed rows need the mix
+    assert call(args(rows=0)) == _capi.TAH_OK
+
