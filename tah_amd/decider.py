@@ -94,12 +94,20 @@ class MLPIterDecider(nn.Module):
     @torch.no_grad()
     def forward(self, logits: torch.Tensor, iter_depth: int, all_hidden_states: Optional[torch.Tensor] = None, **_) -> Tuple[torch.Tensor, torch.Tensor]:
         lead = tuple(logits.shape[:-1])
+        if iter_depth >= self.max_iter:
+            return self.decide_selected(logits, iter_depth, None)
+        return self.decide_selected(logits, iter_depth, self.hidden_features(all_hidden_states, lead, logits))
+
+    @torch.no_grad()
+    def decide_selected(self, logits: torch.Tensor, iter_depth: int, feats: Optional[torch.Tensor]) -> Tuple[torch.Tensor, torch.Tensor]:
+        """``forward`` for a caller that kept only the configured layers: ``feats`` ``(*lead, n * H)``, those layers' hidden
+        states side by side in the configured order (what ``hidden_features`` returns)."""
+        lead = tuple(logits.shape[:-1])
         if iter_depth >= self.max_iter:  # cap reached: nobody continues (iter_decider.py:273-274)
             return (torch.zeros(lead, dtype=torch.bool, device=logits.device),
                     torch.full(lead, STOP_LOGIT, dtype=logits.dtype, device=logits.device))
         if logits.dtype != torch.bfloat16:
             raise TypeError(f"MLPIterDecider: bf16 logits expected, got {logits.dtype} (the top-k kernel reads bf16; there is no other path)")
-        feats = self.hidden_features(all_hidden_states, lead, logits)
         flat = logits.reshape(-1, logits.size(-1))
         top = ops.topk_values(flat if flat.stride(-1) == 1 else flat.contiguous(), self.topk).view(*lead, -1)
         work = self.combined_projection.weight.dtype  # (bf16 as released; a float32 copy of the decider works too)

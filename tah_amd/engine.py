@@ -171,12 +171,16 @@ def rope_tables(max_len: int, head_dim: int, theta: float, device, dtype=torch.b
 
 class TaHDecodeEngine:
     def __init__(self, weights: Weights, batch: int, max_len: int, *, max_hard: Optional[int] = None, device="cuda",
-                 fold_norms: bool = True, packed_linear: bool = True):
+                 fold_norms: bool = True, packed_linear: bool = True, decider=None):
         """``fold_norms``: multiply the layers' input-norm weights into the projections behind them (in place in
         ``weights``, once) so that the two RMSNorms of a layer cost no launch; needs hidden % 8 == 0 and bf16.
         ``packed_linear``: run the linear layers of a decode step on ``ops.linear_rows`` (a second, re-ordered copy
         of the layers' weights is made once); needs ``fold_norms``, at most 32 rows and sizes in whole MFMA steps,
-        otherwise the step keeps torch GEMMs."""
+        otherwise the step keeps torch GEMMs.  ``decider``: a ``tah_amd.decider.MLPIterDecider`` (the reference's learned
+        decider, iter_decider.py:193-301) to decide with instead of the two-layer MLP in ``weights``: it sees each token's
+        first-iteration logits and the hidden states of its configured layers, counted as Hugging Face's
+        ``output_hidden_states`` counts them (0: the embeddings, i: after layer i, the last one after the final norm;
+        tah_model.py:434-441, 615-642)."""
         cfg = weights.cfg
         if cfg.head_dim != 128:
             raise TahDuoError("the kernels are built for head_dim 128")
@@ -223,8 +227,8 @@ class TaHDecodeEngine:
             self.xp, self.op, self.actp = z(cfg.hidden), z(cfg.hq * cfg.head_dim), z(cfg.intermediate)
         # the step's element-wise glue in two launches (tah_step_begin, tah_decider_tail) and the decider's first layer
         # on the linear-layer kernel, instead of some twenty torch launches; needs the packed rows
-        self.fused_glue = bool(self.packed_linear and weights.dec_w1_p is not None and weights.lm_head_p is not None
-                               and cfg.decider_hidden % 8 == 0)
+        self.fused_glue = bool(self.packed_linear and weights.lm_head_p is not None and
+                               (decider is not None or (weights.dec_w1_p is not None and cfg.decider_hidden % 8 == 0)))
         if self.fused_glue:
             i32 = lambda: torch.zeros(batch, dtype=torch.int32, device=dev)
             self.x0 = torch.zeros(batch, cfg.hidden, dtype=torch.bfloat16, device=dev)
@@ -244,6 +248,34 @@ class TaHDecodeEngine:
             self.eligible = torch.zeros(batch, dtype=torch.bool, device=dev)
             self.logits2 = [torch.zeros(batch, cfg.vocab, dtype=torch.bfloat16, device=dev) for _ in range(2)]
         self._tick_graphs = None
+        self.decider = decider
+        if decider is not None:
+            if decider.hidden_states_size != cfg.hidden:
+                raise TahDuoError("the decider's hidden_states_size differs from the model's hidden size")
+            self.hs_pick = list(decider.hidden_states_layer_nums) or [cfg.layers]
+            if min(self.hs_pick) < 0 or max(self.hs_pick) > cfg.layers:
+                raise TahDuoError("the decider's hidden_states_layer_nums do not fit the model's layers")
+            # what the last single-token pass left: [B, picked layers, H], and the decision logits of the last decision
+            self.hs_buf = torch.zeros(batch, len(self.hs_pick), cfg.hidden, dtype=weights.embed.dtype, device=dev)
+            self.decision_logits = None
+
+    def _keep_hidden(self, index: int, x: torch.Tensor, into: Optional[list] = None):
+        """Called with the hidden state after ``index`` layers (before the final norm): keeps it if the decider wants it."""
+        if self.decider is None or index not in self.hs_pick:
+            return
+        h = self._rms(x, self.w.norm) if index == self.cfg.layers else x
+        for j, want in enumerate(self.hs_pick):
+            if want == index:
+                if into is None:
+                    self.hs_buf[:, j].copy_(h)
+                else:
+                    into[j] = h
+
+    def _decide_rows(self, logits: torch.Tensor, hidden_states: torch.Tensor):
+        """The learned decider after a token's first iteration (iter_depth 1 of at most 2: tah_model.py:625-642)."""
+        mask, z = self.decider.decide_selected(logits, 1, hidden_states.reshape(hidden_states.shape[0], -1))
+        self.decision_logits = z
+        return mask
 
     # ── model pieces ─────────────────────────────────────────────────────
     def _rms(self, x, w):
@@ -293,6 +325,7 @@ class TaHDecodeEngine:
         if self.packed_linear:
             return self._pass_single_packed(x, pos, depth, slot_of, q_pos, q_depth, cos, sin)
         folded = self.w.norms_folded
+        self._keep_hidden(0, x)
         for l, L in enumerate(self.w.layers):
             qkv = (x if folded else self._rms(x, L["ln1"])) @ L["wqkv"].t()
             q, k, v = self._split_qkv(qkv)
@@ -307,6 +340,7 @@ class TaHDecodeEngine:
                             static_scratch=self.static_scratch)
             x = x.addmm_(o.view(x.shape[0], c.hq * c.head_dim), L["wo"].t())  # residual add inside the GEMM, in place
             x = self._mlp(x, L)
+            self._keep_hidden(l + 1, x)
         return self._rms(x, self.w.norm)
 
     def _pass_single_packed(self, x, pos, depth: int, slot_of, q_pos, q_depth, cos, sin, rows_packed: bool = False):
@@ -318,6 +352,7 @@ class TaHDecodeEngine:
         n_qkv, n_o = (c.hq + 2 * c.hkv) * c.head_dim, c.hq * c.head_dim
         x = x.contiguous()
         xp = self.xp if rows_packed else ops.linear_pack_rows(x, out=self.xp)  # rows_packed: self.xp already holds x
+        self._keep_hidden(0, x)
         for l, L in enumerate(self.w.layers):
             q, k, v = self._split_qkv(ops.linear_rows(L["wqkv_p"], xp, B, n_qkv, H))
             cache = self.slabs1[l] if depth == 1 else self.slabs0[l]
@@ -343,6 +378,7 @@ class TaHDecodeEngine:
             ops.linear_rows(L["wo_p"], self.op, B, H, n_o, residual=x, out=x, out_packed=xp)
             ops.linear_rows(L["wgu_p"], xp, B, I, H, gate_up=True, out_packed=self.actp, want_out=False, norm_eps=c.rms_eps)
             ops.linear_rows(L["wdown_p"], self.actp, B, H, I, residual=x, out=x, out_packed=xp)
+            self._keep_hidden(l + 1, x)
         return x  # before the final norm; self.xp holds the same rows as operand
 
     def _head(self, h):
@@ -380,7 +416,14 @@ class TaHDecodeEngine:
         l0 = self._head(h0)
         if self.packed_linear:
             h0 = self._rms(h0, self.w.norm)
-        hard = (self.decide(h0) > self.w.threshold) if force_hard is None else force_hard
+        if force_hard is not None:
+            hard = force_hard
+            if self.decider is not None:
+                self._decide_rows(l0, self.hs_buf)  # (kept for inspection: decision_logits)
+        elif self.decider is not None:
+            hard = self._decide_rows(l0, self.hs_buf)
+        else:
+            hard = self.decide(h0) > self.w.threshold
         hard = hard & act
         # next-iteration input of the hard rows (tah_model.py:693-697); the other rows keep zeros
         x1 = ops.topk_mix(l0, self.w.embed, self.cfg.topk, row_enable=hard)
@@ -401,9 +444,15 @@ class TaHDecodeEngine:
         self._pass_single_packed(self.x0, self.pos, 0, self.slot0, self.qpos0, self.zeros_i, self.cos_rows, self.sin_rows,
                                  rows_packed=True)
         l0 = self._head(self.x0)
-        hr = ops.linear_rows(w.dec_w1_p, self.xp, B, c.decider_hidden, c.hidden, norm_eps=c.rms_eps, bias=w.dec_b1, relu=True)
-        ops.decider_tail(hr, w.dec_w2.reshape(-1), w.dec_b2, w.threshold, hard=self.hard, active=self.act, pos=self.pos,
-                         hard_i32=self.hard_i, slot=self.slot1, q_pos=self.qpos1)
+        if self.decider is not None:
+            torch.logical_and(self._decide_rows(l0, self.hs_buf), self.act, out=self.hard)
+            self.hard_i.copy_(self.hard)
+            torch.where(self.hard, self.rows, self.minus1, out=self.slot1)
+            torch.where(self.hard, self.pos, self.minus1, out=self.qpos1)
+        else:
+            hr = ops.linear_rows(w.dec_w1_p, self.xp, B, c.decider_hidden, c.hidden, norm_eps=c.rms_eps, bias=w.dec_b1, relu=True)
+            ops.decider_tail(hr, w.dec_w2.reshape(-1), w.dec_b2, w.threshold, hard=self.hard, active=self.act, pos=self.pos,
+                             hard_i32=self.hard_i, slot=self.slot1, q_pos=self.qpos1)
         ops.topk_mix(l0, w.embed, c.topk, row_enable=self.hard, out=self.x1, out_packed=self.xp, zero_disabled=True)
         h1 = self._pass_single_packed(self.x1, self.pos, 1, self.slot1, self.qpos1, self.hard_i, self.cos_rows, self.sin_rows,
                                       rows_packed=True)
@@ -450,6 +499,8 @@ class TaHDecodeEngine:
         zi = torch.zeros(0, dtype=torch.int32, device=dev)
         x = w.embed[ids]
         kv_tok = []
+        hs_sel = [None] * len(self.hs_pick) if self.decider is not None else None
+        self._keep_hidden(0, x, hs_sel)
         # launch order of the prompts' tiles, heaviest first across prompts: one table serves all layers of a depth
         sched0 = ops.duo_schedule(cu, cu, zc, zc, zi, c.hq, c.hkv, N, N, 0)
         for l, L in enumerate(w.layers):
@@ -460,11 +511,26 @@ class TaHDecodeEngine:
             kv_tok.append((ko, v))
             x = x + o1.view(N, -1) @ L["wo"].t()
             x = self._mlp(x, L)
+            self._keep_hidden(l + 1, x, hs_sel)
         h0 = self._rms(x, w.norm)
-        prob = self.decide(h0)
-        if calibrate is not None:
-            w.threshold = float(torch.quantile(prob, 1.0 - calibrate))
-        hard = (prob > w.threshold) if force_hard is None else force_hard
+        if self.decider is not None:
+            # the decider wants every prompt token's logits: a thousand rows of the vocabulary at a time
+            zs = []
+            for a in range(0, N, 1024):
+                b = min(a + 1024, N)
+                self._decide_rows(h0[a:b] @ w.lm_head.t(), torch.stack([h[a:b] for h in hs_sel], dim=1))
+                zs.append(self.decision_logits)
+            z = self.decision_logits = torch.cat(zs)
+            prob = torch.sigmoid(z)  # in the logits' dtype, as the decider compares it (iter_decider.py:299)
+            if calibrate is not None:
+                with torch.no_grad():
+                    self.decider.threshold.fill_(float(torch.quantile(prob.float(), 1.0 - calibrate)))
+            hard = (prob > self.decider.threshold.to(z.dtype)) if force_hard is None else force_hard
+        else:
+            prob = self.decide(h0)
+            if calibrate is not None:
+                w.threshold = float(torch.quantile(prob, 1.0 - calibrate))
+            hard = (prob > w.threshold) if force_hard is None else force_hard
         last = (cu[1:] - 1).long()
         logits_last = (h0[last] @ w.lm_head.t())  # model dtype, like the reference's logits buffers
         rows2 = torch.nonzero(hard).flatten()
@@ -661,8 +727,11 @@ class TaHDecodeEngine:
         self._pass_single_packed(self.x0, self.pos, None, self.slot0, self.qpos0, self.q_depth_rows, self.cos_rows,
                                  self.sin_rows, rows_packed=True)
         logits = ops.linear_rows(w.lm_head_p, self.xp, B, c.vocab, c.hidden, norm_eps=c.rms_eps, out=self.logits2[parity])
-        hr = ops.linear_rows(w.dec_w1_p, self.xp, B, c.decider_hidden, c.hidden, norm_eps=c.rms_eps, bias=w.dec_b1, relu=True)
-        ops.decider_tail(hr, w.dec_w2.reshape(-1), w.dec_b2, w.threshold, hard=self.hard, active=self.eligible)
+        if self.decider is not None:  # (rows at their second iteration are not eligible: what they left in hs_buf is not used)
+            torch.logical_and(self._decide_rows(logits, self.hs_buf), self.eligible, out=self.hard)
+        else:
+            hr = ops.linear_rows(w.dec_w1_p, self.xp, B, c.decider_hidden, c.hidden, norm_eps=c.rms_eps, bias=w.dec_b1, relu=True)
+            ops.decider_tail(hr, w.dec_w2.reshape(-1), w.dec_b2, w.threshold, hard=self.hard, active=self.eligible)
         ops.topk_mix(logits, w.embed, c.topk, row_enable=self.hard, out=self.x1)  # (other rows of x1 are not read)
         chosen = None
         if temperature > 0.0:

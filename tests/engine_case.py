@@ -20,17 +20,21 @@ class _Cache(O.OracleCache):
         return cache_position.shape[0] + self.get_seq_length(layer_idx), 0
 
 
-def _ref_forward(model, embed, cache, ids, valid, hard, topk):
-    """tah_model.py:495-706 for max_iter = 2 with the decider's decisions given: returns final logits (B, T, V)."""
+def _ref_forward(model, embed, cache, ids, valid, hard, topk, decide=None):
+    """tah_model.py:495-706 for max_iter = 2 with the decider's decisions given: returns final logits (B, T, V).
+    ``decide(logits, stacked hidden states (B, T, L + 1, H))``, when given, is called as the loop calls its decider after
+    the first iteration (tah_model.py:434-441, 636-642) and its result returned as well."""
     B, T = ids.shape
     x = embed[ids]
     cached_valid = cache.get_valid_mask_upto_iter(0, 0, B)
     pos = (torch.cumsum(torch.cat((cached_valid, valid), -1), -1)[:, -T:] - 1).clamp(min=0)  # tah_model.py:555-561
     m0 = O.build_attention_mask(pos, valid, cache, 0, torch.float32)
     cache.current_iter_depth, cache.position_ids_to_cache, cache.valid_mask_to_cache = 0, pos, valid
-    h = model(inputs_embeds=x, attention_mask={"full_attention": m0}, position_ids=pos, past_key_values=cache,
-              use_cache=True).last_hidden_state
+    out0 = model(inputs_embeds=x, attention_mask={"full_attention": m0}, position_ids=pos, past_key_values=cache,
+                 use_cache=True, output_hidden_states=decide is not None)
+    h = out0.last_hidden_state
     cum = h @ embed.t()
+    decided = decide(cum, torch.stack(list(out0.hidden_states), dim=0).permute(1, 2, 0, 3)) if decide is not None else None
     final = cum.clone()
     cur = hard & (valid == 1)
     if cur.any():
@@ -43,7 +47,7 @@ def _ref_forward(model, embed, cache, ids, valid, hard, topk):
         h1 = model(inputs_embeds=a_x, attention_mask={"full_attention": m1}, position_ids=a_pos, past_key_values=cache,
                    use_cache=True).last_hidden_state
         final = O.scatter_back(cur, a_cum + h1 @ embed.t(), final)  # additive_logits_update, tah_model.py:78-83
-    return final
+    return final if decide is None else (final, decided)
 
 
 def run(device, *, prompt=(9, 6, 12), steps=5, layers=2, seed=0, vocab=96, topk=100):
@@ -124,4 +128,67 @@ def run_greedy(device, *, fused, eos, B=3, T=9, new=7, vocab=64, seed=5, layers=
     toks = eng.generate(first, new, eos=eos, use_graph=False).clone()
     return (toks.cpu(), eng.out_len.cpu(), eng.pos.cpu(), eng.finished.cpu(), int(eng.n_hard), int(eng.n_steps), eng.tok.cpu(),
             [sl.len.tolist() for sl in eng.slabs0 + eng.slabs1])
+
+
+def run_with_decider(device, *, prompt=(9, 6, 12), steps=4, layers=3, seed=2, vocab=96):
+    """The engine deciding with tah_amd.decider.MLPIterDecider: the decision logits it computes in prefill (every
+    prompt token) and in every decode step against oracle/decider_ref.py fed with the Hugging Face model's own
+    logits and ``output_hidden_states`` (float32), both sides driven by the same tokens and decisions.  Returns
+    pairs (engine's decision logits, oracle's) per call."""
+    pytest.importorskip("transformers.models.qwen3.modeling_qwen3")
+    from transformers import Qwen3Config, Qwen3Model
+
+    from oracle import decider_ref as R
+    from tah_amd.decider import MLPIterDecider
+    from tah_amd.engine import EngineConfig, TaHDecodeEngine, Weights
+    from tests import decider_case as D
+
+    torch.manual_seed(seed)
+    hf = Qwen3Config(hidden_size=256, num_attention_heads=4, num_key_value_heads=2, head_dim=128,
+                     num_hidden_layers=layers, intermediate_size=512, vocab_size=vocab, rope_theta=1e6,
+                     attention_dropout=0.0, rms_norm_eps=1e-6)
+    hf._attn_implementation = "sdpa"
+    ref = Qwen3Model(hf).to(torch.bfloat16).float().eval()
+    cfg = EngineConfig(hidden=256, layers=layers, hq=4, hkv=2, head_dim=128, intermediate=512, vocab=vocab,
+                       decider_hidden=32, topk=100)
+
+    class _LM:
+        model = ref
+        lm_head = type("H", (), {"weight": ref.embed_tokens.weight})
+    w = Weights.from_hf(_LM, cfg, device)
+    picks = (1, layers)   # after the first layer, and the last one (after the final norm)
+    dec = D.make(device, torch.bfloat16, seed=seed + 3, topk=10, hidden_states_size=256, hidden_states_layer_nums=picks,
+                 hidden_dims=(16, 32, 16), expansion_factor=2)
+    p64 = D.state64(dec)
+
+    def decide(logits, stack):
+        return torch.from_numpy(R.decide(p64, logits.numpy(), 1, stack.numpy(), topk=10, hidden_size=256, layer_nums=picks,
+                                         n_blocks=3, max_iter=3)[1])
+
+    g = torch.Generator().manual_seed(seed + 1)
+    B, Tm = len(prompt), max(prompt)
+    eng = TaHDecodeEngine(w, B, Tm + steps + 4, device=device, decider=dec)
+    ids = torch.randint(0, vocab, (B, Tm + steps), generator=g)
+    valid = torch.zeros(B, Tm, dtype=torch.long)
+    for b, n in enumerate(prompt):
+        valid[b, Tm - n:] = 1
+    hard = torch.rand(B, Tm + steps, generator=g) < 0.35
+    embed = ref.embed_tokens.weight.detach()
+    out = []
+    with torch.no_grad():
+        cache = _Cache()
+        _, z = _ref_forward(ref, embed, cache, ids[:, :Tm], valid, hard[:, :Tm], 100, decide)
+        packed = torch.cat([ids[b, Tm - n:Tm] for b, n in enumerate(prompt)]).to(device)
+        hard_packed = torch.cat([hard[b, Tm - n:Tm] for b, n in enumerate(prompt)]).to(device)
+        cu = torch.tensor([0] + list(torch.tensor(prompt).cumsum(0)), dtype=torch.int32, device=device)
+        eng.prefill(packed, cu, force_hard=hard_packed)
+        out.append((eng.decision_logits.float().cpu(), torch.cat([z[b, Tm - n:] for b, n in enumerate(prompt)])))
+        one = torch.ones(B, 1, dtype=torch.long)
+        for s_ in range(steps):
+            t = Tm + s_
+            _, z = _ref_forward(ref, embed, cache, ids[:, t:t + 1], one, hard[:, t:t + 1], 100, decide)
+            eng.step_logits(ids[:, t].to(device), force_hard=hard[:, t].to(device))
+            eng.pos += 1
+            out.append((eng.decision_logits.float().cpu(), z[:, 0]))
+    return out
 

@@ -430,3 +430,47 @@ def test_sampling_on_the_topk_values_on_cpu_shim():
 def test_sampling_on_the_topk_values_gpu():
     _topk_sampling_case("cuda", 20000)
 
+
+def _decider_wiring_check(device, **size):
+    from tests import engine_case
+    for got, want in engine_case.run_with_decider(device, **size):
+        want = want.float()
+        assert got.shape == want.shape
+        err = (got - want).abs()
+        assert float((err / (0.25 + 0.06 * want.abs())).max()) <= 1.0, (float(err.max()), float(want.abs().max()))
+        assert float(err.mean()) <= 0.06 * float(want.abs().mean()) + 0.05
+
+
+@pytest.mark.skipif(not emu_util.have_host_clang(), reason="host clang++ not available")
+def test_engine_with_the_learned_decider_on_cpu_shim():
+    """The hidden states and logits the engine hands tah_amd.decider.MLPIterDecider are the ones the Hugging Face
+    model reports with output_hidden_states (embeddings, after each layer, the last after the final norm)."""
+    with emu_util.emulated():
+        _decider_wiring_check("cpu", prompt=(3, 2), steps=1, layers=2)
+
+
+@pytest.mark.gpu
+def test_engine_with_the_learned_decider_gpu():
+    _decider_wiring_check("cuda")
+    # and deciding by itself: ticks (eager and captured) give the step-wise loop's tokens
+    from tah_amd.engine import EngineConfig, TaHDecodeEngine, Weights
+    from tests import decider_case as D
+    cfg = EngineConfig(hidden=256, layers=3, hq=16, hkv=8, head_dim=128, intermediate=768, vocab=4096, decider_hidden=32)
+    w = Weights.random_init(cfg, "cuda", seed=8)
+    dec = D.make("cuda", torch.bfloat16, seed=12, topk=10, hidden_states_size=256, hidden_states_layer_nums=(1, 2, 3),
+                 hidden_dims=(16, 32, 16), expansion_factor=2)
+    B, T, new = 32, 19, 18
+    g = torch.Generator().manual_seed(13)
+    ids = torch.randint(0, cfg.vocab, (B * T,), generator=g).cuda()
+    cu = torch.arange(0, B * T + 1, T, dtype=torch.int32, device="cuda")
+    runs = []
+    for continuous, use_graph in ((False, False), (False, True), (True, False), (True, True)):
+        eng = TaHDecodeEngine(w, B, T + new + 2, device="cuda", decider=dec)
+        assert eng.can_run_continuous
+        first, hard = eng.prefill(ids, cu, calibrate=0.25)
+        toks = eng.generate(first, new, continuous=continuous, use_graph=use_graph).clone()
+        runs.append((toks.cpu(), int(eng.n_hard), [sl.len.tolist() for sl in eng.slabs1], int(hard.sum())))
+    assert 0 < runs[0][1] < B * (new - 1) and 0 < runs[0][3] < B * T
+    for r in runs[1:]:
+        assert torch.equal(r[0], runs[0][0]) and r[1:] == runs[0][1:]
+
