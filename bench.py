@@ -269,6 +269,45 @@ def bench_qk_prep(steps: int, warmup: int):
             "tokens_per_s": rows / (ms * 1e-3)}
 
 
+def bench_topk_mix(steps: int, warmup: int, rows: int = 1024, vocab: int = 151936, hidden: int = 2048, topk: int = 100):
+    """Next-iteration input of hard tokens (tah_model.py:57-75): top-100 softmax mix of embedding rows for `rows` rows of
+    the full vocabulary, and the top-k logit values alone (the decider's features, iter_decider.py:281) next to
+    torch.topk on the same rows.  Per row the kernel reads the logits once and k embedding rows."""
+    import torch
+
+    from tah_amd import ops
+
+    g = torch.Generator().manual_seed(1241)
+    logits = [(torch.randn(rows, vocab, generator=g) * 3).to(torch.bfloat16).cuda() for _ in range(2)]  # two sets in rotation
+    emb = (torch.randn(vocab, hidden, generator=g) * 0.02).to(torch.bfloat16).cuda()
+    out = torch.empty(rows, hidden, dtype=torch.bfloat16, device="cuda")
+    yield
+
+    def timed(f):
+        for i in range(warmup):
+            f(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(steps):
+            f(i)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps
+
+    mix_ms = timed(lambda i: ops.topk_mix(logits[i % 2], emb, topk, out=out))
+    val_ms = timed(lambda i: ops.topk_values(logits[i % 2], topk))
+    torch_ms = timed(lambda i: torch.topk(logits[i % 2], topk, dim=-1))
+    nbytes = rows * (vocab * 2 + topk * hidden * 2 + hidden * 2)
+    gbs = nbytes / (mix_ms * 1e-3) / 1e9
+    return {"workload": f"top-{topk} softmax mix of embedding rows, {rows} rows of {vocab} bf16 logits, hidden {hidden} "
+                        "(two sets of logits in rotation)",
+            "ms_per_step": mix_ms, "algorithmic_bytes": nbytes, "hbm_gbs": gbs,
+            "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
+                         "traffic": None, "kernels": "topk_mix_kernel<19>"},
+            "topk_values_ms": val_ms, "torch_topk_ms": torch_ms, "rows_per_s": rows / (mix_ms * 1e-3)}
+
+
 def bench_e2e_decode(new_tokens: int, B: int = 32, prompt_len: int = 512, temperature: float = 0.0, top_p: float = 0.95, top_k: int = 0):
     """BASELINE configs[4]: end-to-end TaH decode, Qwen3-1.7B architecture with random weights, a two-layer MLP
     decider whose threshold is set so that about 6 % of the prompt tokens iterate, batch 32, 512-token prompts.
@@ -374,7 +413,7 @@ def main() -> int:
     ap.add_argument("--spinup", type=int, default=200,
                     help="untimed launches of the headline kernel before its warm-up steps (the GPU's clock needs tens of "
                          "milliseconds of work to leave its idle state)")
-    ap.add_argument("--only", choices=["all", "fwd", "decode", "fwd_bwd", "qk_prep", "e2e"], default="all",
+    ap.add_argument("--only", choices=["all", "fwd", "decode", "fwd_bwd", "qk_prep", "topk_mix", "e2e"], default="all",
                     help="profiling aid: run only one leg (the JSON line then lacks the other legs)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="profiling aid: also run one plain 256 MiB device copy (known traffic for counter scaling)")
@@ -420,6 +459,8 @@ def main() -> int:
         legs.append(("decode", bench_decode(args.steps, args.warmup)))
     if args.only in ("all", "qk_prep"):
         legs.append(("qk_prep_prefill", bench_qk_prep(args.steps, args.warmup)))
+    if args.only in ("all", "topk_mix"):
+        legs.append(("topk_mix", bench_topk_mix(args.steps, args.warmup)))
     if args.only in ("all", "e2e"):
         legs.append(("e2e_decode", bench_e2e_decode(args.e2e_tokens, temperature=args.e2e_temperature, top_k=args.e2e_top_k)))
     for _, leg in legs:
