@@ -64,19 +64,13 @@ __device__ __forceinline__ int block_sum(int x, int* red, int wave, int lane) {
     return t;
 }
 
-// Number of threads of the workgroup for which `pred` holds, returned to every thread: one ballot per wave instead of
-// block_sum's six exchanges.
-__device__ __forceinline__ int block_count(bool pred, int* red, int wave, int lane) {
-    const int c = __popcll(__ballot(pred));
-    __syncthreads();  // earlier readers of red are done
-    if (lane == 0) red[wave] = c;
-    __syncthreads();
-    int t = 0;
-#pragma unroll
-    for (int w = 0; w < kMixWaves; ++w) t += red[w];
-    return t;
-}
-
+// Largest T in [lo, hi) with count(key >= T) >= k, given count(key >= lo) >= k > count(key >= hi) (if even `lo` has
+// fewer, `lo` comes back).  A 16-way search: every step counts the keys at or above fifteen thresholds spread over the
+// interval, each count one ballot per wave and element slot (`pred(t, u)`: this thread's element u, u < NU, has a key
+// >= t); lane i of every wave adds its wave's count for threshold i into row `round` of `tot` (zero on entry, every
+// row used once), and after one barrier a ballot over that row tells which thresholds still have k keys at or above
+// them.  The bounds stay in scalar registers.  Four steps for 16 bits, five for a vocabulary index; kSearchRows
+// rows of `tot` per search.
 constexpr int kSearchRows = 6;
 template <int NU, class Pred>
 __device__ __forceinline__ uint32_t search_kth(uint32_t lo, uint32_t hi, int k, int (*tot)[16], int lane, Pred pred) {
