@@ -71,7 +71,7 @@ def test_decider_gpu_released_sizes():
     m32 = D.make("cuda", torch.float32, seed=8)
     D.check(m32, logits, hs, atol=1e-3, rtol=1e-3)
     m = D.make("cuda", torch.bfloat16, seed=9, normalize_input=True)
-    D.check(m, logits, hs, atol=0.15, rtol=0.06)
+    D.check(m, logits, hs, atol=0.06, rtol=0.03)     # bf16 layers: measured 0.022 at most on logits up to 3
     # the same weights through a state dict, as a released decider would arrive
     from tah_amd.decider import MLPIterDecider
     again = MLPIterDecider(normalize_input=True).to("cuda")

@@ -437,8 +437,10 @@ def _decider_wiring_check(device, **size):
         want = want.float()
         assert got.shape == want.shape
         err = (got - want).abs()
-        assert float((err / (0.25 + 0.06 * want.abs())).max()) <= 1.0, (float(err.max()), float(want.abs().max()))
-        assert float(err.mean()) <= 0.06 * float(want.abs().mean()) + 0.05
+        # (bf16 model and decider against float32 / float64: measured 0.03 at most, 0.02 on average, on logits of size 2;
+        # a wrong layer or a missing final norm moves them by their own size)
+        assert float((err / (0.08 + 0.03 * want.abs())).max()) <= 1.0, (float(err.max()), float(want.abs().max()))
+        assert float(err.mean()) <= 0.02 * float(want.abs().mean()) + 0.02
 
 
 @pytest.mark.skipif(not emu_util.have_host_clang(), reason="host clang++ not available")
