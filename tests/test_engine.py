@@ -387,6 +387,13 @@ def test_continuous_generation_with_sampling_gpu():
     assert int(toks.min()) >= 0 and int(toks.max()) < cfg.vocab
     top50 = torch.topk(first, 50, dim=-1).indices
     assert (toks[:, :1] == top50).any(dim=-1).all()                          # the first draw obeys the top-k filter
+    # the same prompt in every row: the captured tick must draw anew at every replay and for every row
+    same = ids[:T].repeat(B)
+    eng = TaHDecodeEngine(w, B, T + new + 2, device="cuda")
+    first, _ = eng.prefill(same, cu, calibrate=0.25)
+    toks = eng.generate(first, new, temperature=1.0, top_k=50, eos=-1)
+    assert len({tuple(r.tolist()) for r in toks}) > B // 2
+    assert min(len(set(toks[:, j].tolist())) for j in range(1, new)) > B // 4
 
 
 def _topk_sampling_case(device, V, rows=6, draws=True):
