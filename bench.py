@@ -28,6 +28,7 @@ PEAK_HBM_GBS = 8000.0
 TRAFFIC_FWD_BYTES = 203.3e6 + 72.2e6
 TRAFFIC_DECODE_BYTES = 2.329e9 + 5.1e6 + 5.2e6 + 0.3e6
 TRAFFIC_QK_PREP_BYTES = 142.7e6 + 134.2e6
+TRAFFIC_TOPK_MIX_BYTES = 729.3e6 + 8.4e6  # (profiles/topk_mix_kernel_1024_rows_counters.md)
 # forward + backward legs, all kernels of one step (forward, two delta kernels, dQ, dK/dV): bytes fetched + written
 # (profiles/duo_fwd_bwd_seq8192_and_4docs_counters.md)
 TRAFFIC_FWD_BWD_SEQ8192_BYTES = 610.5e6 + 113.2e6
@@ -304,7 +305,8 @@ def bench_topk_mix(steps: int, warmup: int, rows: int = 1024, vocab: int = 15193
                         "(two sets of logits in rotation)",
             "ms_per_step": mix_ms, "algorithmic_bytes": nbytes, "hbm_gbs": gbs,
             "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
-                         "traffic": None, "kernels": "topk_mix_kernel<19>"},
+                         "traffic": TRAFFIC_TOPK_MIX_BYTES if (rows, vocab, hidden, topk) == (1024, 151936, 2048, 100) else None,
+                         "kernels": "topk_mix_kernel<19>"},
             "topk_values_ms": val_ms, "torch_topk_ms": torch_ms, "rows_per_s": rows / (mix_ms * 1e-3)}
 
 
