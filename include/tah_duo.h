@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define TAH_DUO_ABI_VERSION 5
+#define TAH_DUO_ABI_VERSION 6
 
 enum {
     TAH_OK = 0,
@@ -138,7 +138,7 @@ typedef struct tah_duo_bwd_stream {
     void* dq;               /* bf16 [total_q, Hq,  D] */
     void* dk;               /* bf16 [total_k, Hkv, D] */
     void* dv;               /* bf16 [total_k, Hkv, D] */
-    float* delta;           /* f32  [Hq, total_q] scratch (rowsum(dO*O)), written by the call */
+    float* delta;           /* f32  [2, Hq, total_q] scratch written by the call: rowsum(dO*O), then lse * log2(e) */
     int64_t do_row_stride, do_head_stride;
     int64_t dq_row_stride, dq_head_stride;
     int64_t dk_row_stride, dk_head_stride;
@@ -149,14 +149,28 @@ typedef struct tah_duo_bwd_args {
     tah_duo_fwd_args fwd;   /* the forward call's tensors; o and lse are inputs here */
     tah_duo_bwd_stream g1;  /* depth 0 */
     tah_duo_bwd_stream g2;  /* depth 1 */
+    void* ds_workspace;         /* NULL, or >= tah_duo_bwd_workspace_bytes(...) bytes, 16-byte aligned; contents need no
+                                 * initialisation and mean nothing after the call */
+    size_t ds_workspace_bytes;
+    int32_t max_seqlen_k1;      /* upper bound on one sequence's depth-0 key rows, 0: unknown (total_k is used) */
+    int32_t max_seqlen_k2;      /* same for depth 1 */
 } tah_duo_bwd_args;
 
 /* Backward of tah_duo_fwd_varlen: dQ, dK, dV of both depths.  Replaces torch
  * autograd through SDPA + torch.cat + repeat_kv on this path; the reference
  * keeps cached K/V attached to the graph (tah/model/causal_cache.py:92-93), so
  * depth-0 dK/dV collect the contributions of depth-0 and depth-1 queries, summed
- * over the query heads of each kv head.  Deterministic (no atomics). */
+ * over the query heads of each kv head.  Deterministic (no atomics).
+ *
+ * Without `ds_workspace`: three kernels, dQ and dK/dV each recompute the scores (7 matrix products per
+ * visible (query tile, key tile) pair).  With it (hq / hkv <= 4): the dK/dV kernel also writes
+ * dS = P o (dP - delta) in bf16, one 16 KiB block per (64 query rows, head, 128 keys), and dQ = scale * dS K
+ * reads it back (5 products per pair; the workspace is written and read once).  Both give the same dK / dV
+ * to the bit; dQ then uses the dS the dK product uses.  The bound the size function returns covers every
+ * (64-row query tile, 128-key tile) pair of the call: about total_q * max_seqlen_k * hq * 2 bytes. */
 int tah_duo_bwd_varlen(const tah_duo_bwd_args* args, tah_stream_t stream);
+size_t tah_duo_bwd_workspace_bytes(int32_t nseq, int32_t hq, int32_t hkv, int32_t total_q1, int32_t total_k1,
+                                   int32_t total_q2, int32_t total_k2, int32_t max_seqlen_k1, int32_t max_seqlen_k2);
 
 /* Backward of tah_duo_fwd_masked (same additive mask; no gradient is formed for
  * the mask itself, which the reference builds from integers).  Replaces torch

@@ -8,7 +8,7 @@ from __future__ import annotations
 
 import ctypes as C
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 c_void_p, c_int32, c_int64, c_float = C.c_void_p, C.c_int32, C.c_int64, C.c_float
 
@@ -69,7 +69,9 @@ class DuoBwdStream(C.Structure):
 class DuoBwdArgs(C.Structure):
     """``tah_duo_bwd_args``"""
 
-    _fields_ = [("fwd", DuoFwdArgs), ("g1", DuoBwdStream), ("g2", DuoBwdStream)]
+    _fields_ = [("fwd", DuoFwdArgs), ("g1", DuoBwdStream), ("g2", DuoBwdStream),
+                ("ds_workspace", c_void_p), ("ds_workspace_bytes", C.c_size_t),
+                ("max_seqlen_k1", c_int32), ("max_seqlen_k2", c_int32)]
 
 
 class AdditiveMask(C.Structure):
@@ -224,6 +226,7 @@ PROTOTYPES = {
     "tah_duo_error_string": (C.c_char_p, [C.c_int]),
     "tah_duo_fwd_varlen": (C.c_int, [C.POINTER(DuoFwdArgs), c_void_p]),
     "tah_duo_bwd_varlen": (C.c_int, [C.POINTER(DuoBwdArgs), c_void_p]),
+    "tah_duo_bwd_workspace_bytes": (C.c_size_t, [c_int32] * 9),
     "tah_duo_schedule_bytes": (C.c_size_t, [c_int32] * 7),
     "tah_duo_schedule_build": (C.c_int, [C.POINTER(DuoScheduleArgs), c_void_p]),
     "tah_greedy_step": (C.c_int, [C.POINTER(GreedyStepArgs), c_void_p]),

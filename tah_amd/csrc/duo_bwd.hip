@@ -53,7 +53,36 @@ struct BwdParams {
     int64_t mask_sb, mask_sh, mask_sq, mask_sk;
     int32_t mask_f32;  // element type: 1 = float, 0 = bf16
     float inv_scale;   // 1 / scale: the mask is added to raw scores as mask / scale
+    // dS exchange between the key-tile kernel and the dQ kernel that reads it back (see ds_block)
+    unsigned char* ds_ws;
+    int32_t ds_q1slots, ds_kt1, ds_kt;
 };
+
+// ---------------------------------------------------------------------------
+// dS exchange.  With a workspace the key-tile kernel (which forms S, P, dP and dS for dK / dV anyway) also
+// writes dS, and dQ = scale * dS K becomes one product that reads it back instead of a second pass that
+// recomputes S and dP: 5 products per (query tile, key tile) pair instead of 7.
+// The workspace is a table of 16 KiB blocks, one per (64 query rows, query head, 128 keys):
+//   block = ((qslot * hq + head) * ds_kt + ktile)
+//   qslot = cu_q1[seq] / 64 + seq + tile                  depth-0 query rows  (ds_q1slots slots)
+//           ds_q1slots + cu_q2[seq] / 64 + seq + tile     depth-1 query rows
+//   ktile = key tile inside its sequence (depth 0), ds_kt1 + key tile (depth 1)
+// (cu / 64 + seq numbers the 64-row tiles of successive sequences without collisions and needs no prefix
+// sum over tile counts.)  Inside a block wave w = 4 * (query half) + (32-key block) of the key-tile kernel
+// owns 2 KiB: its bf16 dS registers as they are, 16 bytes (four query rows of one key, twice) per lane,
+// placed so that the reader's transpose reads of one half-wave cover 256 contiguous bytes:
+//   16-byte piece (a2 = register / 8, key k = lane % 32, hf = lane / 32)  ->  ((k/4)*16 + a2*8 + hf*4 + k%4) * 16
+// and holds rows 16*a2 + 8*j + 4*hf + 0..3 (j = 0, 1 in the piece's two halves) of the wave's 32 query rows.
+// ---------------------------------------------------------------------------
+constexpr int kDsBlockBytes = 64 * 128 * 2;
+constexpr int kDsWaveBytes = 2048;
+__device__ __forceinline__ int ds_piece_off(int a2, int k, int hf) { return (((k >> 2) << 4) + (a2 << 3) + (hf << 2) + (k & 3)) << 4; }
+inline __host__ __device__ int ds_key_slots(int total_k, int max_k) {
+    const int m = (max_k > 0 && max_k < total_k) ? max_k : total_k;
+    return total_k > 0 ? (m + 127) / 128 : 0;
+}
+inline __host__ __device__ int ds_query_slots(int total_q, int nseq) { return total_q > 0 ? total_q / 64 + nseq : 0; }
+
 
 __device__ __forceinline__ float mask_value(const BwdParams& p, const unsigned char* row, int64_t k) {
     return p.mask_f32 ? reinterpret_cast<const float*>(row)[k * p.mask_sk]
@@ -61,7 +90,8 @@ __device__ __forceinline__ float mask_value(const BwdParams& p, const unsigned c
 }
 
 // ---------------------------------------------------------------------------
-// delta = rowsum(dO * O): 16 lanes per (row, head), 8 elements each
+// delta = rowsum(dO * O): 16 lanes per (row, head), 8 elements each; behind the Hq * total_q deltas the same
+// launch leaves lse * log2(e), the form in which the dK/dV kernel subtracts it from the scaled scores
 // ---------------------------------------------------------------------------
 template <int CTRL>
 __device__ __forceinline__ float dpp_add(float x) {
@@ -83,7 +113,10 @@ __global__ __launch_bounds__(256) void duo_bwd_delta_kernel(const BwdStream s, i
     acc = dpp_add<0x4E>(acc);
     acc = dpp_add<0x141>(acc);
     acc = dpp_add<0x140>(acc);
-    if (dc == 0 && item < total) s.delta[(int64_t)head * s.total_q + row] = acc;
+    if (dc == 0 && item < total) {
+        s.delta[(int64_t)head * s.total_q + row] = acc;
+        s.delta[total + (int64_t)head * s.total_q + row] = s.lse[(int64_t)head * s.total_q + row] * kLog2e;
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -330,9 +363,11 @@ constexpr int kKvSmem = kKvMeta + 2 * kKvMetaBytes;
 constexpr int kKvRed = kKB * 128 * 64 * 4;                // final reduction: [key block][128 regs][64 lanes] f32, reuses the front
 static_assert(kKvRed <= kKvSmem, "reduction buffer must fit");
 
-template <int G, bool kDense>
+// kExport: dS of every item is also written to the exchange workspace (p.ds_ws), for duo_bwd_dq_from_ds_kernel.
+template <int G, bool kDense, bool kExport>
 __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkdv_kernel(const BwdParams p) {
-    HIP_DYNAMIC_SHARED(unsigned char, smem)
+    HIP_DYNAMIC_SHARED(unsigned char, smem_array)
+    TAH_LDS_ZERO_BASED(smem, smem_array);
     const int tid = threadIdx.x, lane = tid % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);  // wave-uniform: lives in a scalar register
     const int half = lane / 32, col = lane % 32;
@@ -423,6 +458,21 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
         for (int r = 0; r < 16; ++r) { dkacc[i][r] = 0.f; dvacc[i][r] = 0.f; }
     const float c = p.scale_log2e;
 
+    // dS exchange: my two 16-byte pieces inside the wave's 2 KiB of an item's block, and the block of item 0 of
+    // each query stream (blocks of successive query tiles are hq * ds_kt blocks apart, heads ds_kt)
+    [[maybe_unused]] const int ds_lane_off = ds_piece_off(0, col, half);
+    [[maybe_unused]] int64_t ds_base1 = 0, ds_base2 = 0;
+    if constexpr (kExport) {
+        const int ktile = (second ? p.ds_kt1 : 0) + kl0 / kBK;
+        const int slot1 = q1_lo / kBQ + seq + t1_begin;
+        const int slot2 = p.ds_q1slots + q2_lo / kBQ + seq;
+        ds_base1 = ((int64_t)slot1 * p.hq * p.ds_kt + ktile) * kDsBlockBytes + wave * kDsWaveBytes;
+        ds_base2 = ((int64_t)slot2 * p.hq * p.ds_kt + ktile) * kDsBlockBytes + wave * kDsWaveBytes;
+    }
+    // An item's dS leaves at the start of the next item: a store issued where dS is complete would still be on its
+    // way at the barrier that ends the item, whose wait for the staged tiles (vmcnt) counts stores as well.
+    [[maybe_unused]] bf16x8 ds_keep[2] = {};
+
     // item = (query tile, query head): rows [r0, r_end) of stream q2s, head `head`
     auto item_rows = [&](int item, bool& q2s, int& r0, int& r_end, int& head) {
         const int t = item / G;
@@ -448,7 +498,7 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
     // that every wave would sit through right after the barrier).
     struct ItemSrc {
         const __bf16 *q, *g;
-        const float *lse, *delta;
+        const float *lse, *delta;  // lse: the log2-scaled copy behind the deltas
         const int32_t* pos;
         uint32_t qrs2, grs2;
         int64_t q_hs, g_hs;
@@ -457,7 +507,7 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
     auto stream_src = [&](bool q2s) {
         const BwdStream& qs = q2s ? p.s2 : p.s1;
         ItemSrc r;
-        r.q = qs.q; r.g = qs.d_o; r.lse = qs.lse; r.delta = qs.delta; r.pos = qs.pos_q;
+        r.q = qs.q; r.g = qs.d_o; r.lse = qs.delta + (int64_t)p.hq * qs.total_q; r.delta = qs.delta; r.pos = qs.pos_q;
         r.qrs2 = (uint32_t)(qs.q_rs * 2) & 0xffffffu;
         r.grs2 = (uint32_t)(qs.do_rs * 2) & 0xffffffu;
         r.q_hs = qs.q_hs; r.g_hs = qs.do_hs;
@@ -473,9 +523,9 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
         const bool q2s = src.tile0 != 0 || nt1 == 0;
         const int r0 = src.row_lo + (t - src.tile0) * kBQ;
         const int r_end = r0 + kBQ < src.row_end ? r0 + kBQ : src.row_end;
-        unsigned char* qt = smem + buf * kKvSlot;
-        unsigned char* gt = qt + kTileBytes;
-        float* meta = reinterpret_cast<float*>(smem + kKvMeta + buf * kKvMetaBytes);
+        auto* qt = smem + buf * kKvSlot;
+        auto* gt = qt + kTileBytes;
+        auto* meta = TAH_LDS_CAST(float, smem + kKvMeta + buf * kKvMetaBytes);
         const int last = r_end - 1 - r0;
         const uint32_t l0 = (uint32_t)(my_lrow < last ? my_lrow : last) & 63u;
         const uint32_t l1 = (uint32_t)(my_lrow + 4 < last ? my_lrow + 4 : last) & 63u;
@@ -495,6 +545,16 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
         TAH_WAIT_VMEM();
         __syncthreads();
         if (item + 1 == nt1 * G) src = stream_src(true);  // the next item is the first of the depth-1 stream
+    };
+    // this wave's 2 KiB of an item's dS block (wave-uniform), and the store of the dS kept from that item
+    [[maybe_unused]] auto ds_store = [&](int item) __attribute__((always_inline)) {
+        const int t = item / G;
+        const int64_t blk = t >= nt1 ? ds_base2 + (int64_t)((t - nt1) * p.hq + hk * G + item % G) * p.ds_kt * kDsBlockBytes
+                                     : ds_base1 + (int64_t)(t * p.hq + hk * G + item % G) * p.ds_kt * kDsBlockBytes;
+        unsigned char* dst = p.ds_ws + blk;
+        // (streaming stores: 1 GB of dS per call should not push the Q / dO / K / V tiles out of the L2)
+        __builtin_nontemporal_store(ds_keep[0], reinterpret_cast<bf16x8*>(dst + ds_lane_off));
+        __builtin_nontemporal_store(ds_keep[1], reinterpret_cast<bf16x8*>(dst + ds_lane_off + 128));
     };
 
     // per-lane LDS read offsets inside a tile, computed once
@@ -521,13 +581,13 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
         constexpr bool kMasked = decltype(mask_tag)::value;
         constexpr int kStage = decltype(stage_tag)::value;  // 0 / 1: stage known at compile time; -1: item & 1
         const int stage = kStage >= 0 ? kStage : (item & 1);
-        const unsigned char* qt = smem + stage * kKvSlot;
-        const unsigned char* gt = qt + kTileBytes;
-        const float* meta = reinterpret_cast<const float*>(smem + kKvMeta + stage * kKvMetaBytes);
+        const auto* qt = smem + stage * kKvSlot;
+        const auto* gt = qt + kTileBytes;
+        const auto* meta = TAH_LDS_CAST(const float, smem + kKvMeta + stage * kKvMetaBytes);
 
         [[maybe_unused]] bool q2s = false;
         [[maybe_unused]] int nvalid = kBQ, pos0 = 0;
-        [[maybe_unused]] const int* qposs = reinterpret_cast<const int*>(meta) + 2 * kBQ;
+        [[maybe_unused]] const auto* qposs = TAH_LDS_CAST(const int, meta) + 2 * kBQ;
         [[maybe_unused]] int dense_head = 0, dense_q0 = 0;
         if constexpr (kMasked) {
             int r0, r_end, head;
@@ -554,12 +614,12 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
         [[maybe_unused]] int mrow_m = mrow, kpos_m = kpos;
         if constexpr (kMasked) TAH_OPAQUE2(mrow_m, kpos_m);
         auto load_ab = [&](int n) __attribute__((always_inline)) {
-            ra[n % 3] = *reinterpret_cast<const bf16x8*>((n < 8 ? qt : gt) + (abase ^ (32 * (n % 8))));
-            rb[n % 3] = *reinterpret_cast<const bf16x8*>(smem + (n < 8 ? 0 : kKvV - kKvK) + (bbase ^ (32 * (n % 8))));
+            ra[n % 3] = *TAH_LDS_CAST(const bf16x8, (n < 8 ? qt : gt) + (abase ^ (32 * (n % 8))));
+            rb[n % 3] = *TAH_LDS_CAST(const bf16x8, smem + (n < 8 ? 0 : kKvV - kKvK) + (bbase ^ (32 * (n % 8))));
         };
         // B operand of tail slot m: dO columns (dV, m < 8) or Q columns (dK) of my 32 query rows
         auto load_t = [&](int m) __attribute__((always_inline)) {
-            const unsigned char* t = m < 8 ? gt : qt;
+            const auto* t = m < 8 ? gt : qt;
             const int st = (m % 8) / 4, dt = m % 4;
             const bf16x4 lo = lds_read_tr16(t + (tlo ^ (64 * dt)) + st * 4096);
             const bf16x4 hi = lds_read_tr16(t + (thi ^ (64 * dt)) + st * 4096);
@@ -572,7 +632,7 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
             for (int u = 0; u < 2; ++u) {
                 const int rr = r + u, j = rr / 4, b4 = rr % 4;
                 const float lse = lse4[j % 2][b4];
-                pr[u] = fast_exp2(sacc[rr] * c - lse * kLog2e);
+                pr[u] = fast_exp2(sacc[rr] * c - lse);
                 if constexpr (kMasked && !kDense) {
                     const int qr = mrow_m + 8 * j + b4;
                     const int qp = q2s ? qposs[qr] : pos0 + qr;
@@ -586,7 +646,7 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
                     const float mv = mask_value(p, static_cast<const unsigned char*>(p.mask) + e * (p.mask_f32 ? 4 : 2),
                                                 ok ? kl0 + 32 * kb + col : 0);
                     const float lse_row = lse == kNegInf ? -kNegInf : lse;  // all keys hidden: P = 0
-                    pr[u] = ok ? fast_exp2((sacc[rr] + mv * p.inv_scale) * c - lse_row * kLog2e) : 0.f;
+                    pr[u] = ok ? fast_exp2((sacc[rr] + mv * p.inv_scale) * c - lse_row) : 0.f;
                 }
             }
             const f32x2 pr2 = {pr[0], pr[1]};
@@ -604,10 +664,10 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
             dsfr[r / 8][r % 8 + 1] = pk[1];
         };
         auto load_lse = [&](int j) __attribute__((always_inline)) {
-            lse4[j % 2] = *reinterpret_cast<const f32x4*>(meta + mrow + 8 * j);
+            lse4[j % 2] = *TAH_LDS_CAST(const f32x4, meta + mrow + 8 * j);
         };
         auto load_del = [&](int j) __attribute__((always_inline)) {
-            del4[j % 2] = *reinterpret_cast<const f32x4*>(meta + kBQ + mrow + 8 * j);
+            del4[j % 2] = *TAH_LDS_CAST(const f32x4, meta + kBQ + mrow + 8 * j);
         };
 
         load_ab(0);
@@ -640,6 +700,10 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
                 // dK += dS^T Q (contraction over my 32 queries)
                 dkacc[n % 4] = mfma32(dsfr[(n - 24) / 4], rt[n % 4], dkacc[n % 4]);
             }
+            if constexpr (kExport) {
+                if (n == 0 && item > 0) ds_store(item - 1);  // the previous item's dS (before this item's copies are issued)
+                if (n == 31) { ds_keep[0] = dsfr[0]; ds_keep[1] = dsfr[1]; }
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -671,10 +735,13 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
     run(t_vis * G, t_whole * G, Plain{});
     run(t_whole * G, nitems, Masked{});
 
+    if constexpr (kExport) {
+        if (nitems > 0) ds_store(nitems - 1);
+    }
     // ---- add the two query halves and store ---------------------------------
     TAH_WAIT_VMEM();  // no copy may still be on its way into the memory the reduction reuses
     __syncthreads();
-    float* red = reinterpret_cast<float*>(smem);  // [key block][128 regs][64 lanes]
+    auto* red = TAH_LDS_CAST(float, smem);  // [key block][128 regs][64 lanes]
     if (qh == 1) {
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt)
@@ -697,6 +764,195 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
                 if (krow < key_end) {
                     ks.dk[(int64_t)krow * ks.dk_rs + (int64_t)hk * ks.dk_hs + 32 * dt + col] = (__bf16)dkv;
                     ks.dv[(int64_t)krow * ks.dv_rs + (int64_t)hk * ks.dv_hs + 32 * dt + col] = (__bf16)dvv;
+                }
+            }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// dQ from the exchanged dS: dQ = scale * dS K, one product per (query tile, key tile) pair
+// ---------------------------------------------------------------------------
+// One workgroup = the query tile of the forward / dQ kernels (256 / G rows, the G heads of one kv head), i.e.
+// four units of (64 query rows, one head); waves 2u and 2u + 1 own unit u and split the head dimension.
+// Per step of 64 keys the workgroup stages the K rows (row-major, swizzled, as everywhere) and every unit's
+// 8 KiB of dS in LDS with asynchronous copies, three steps deep (the kernel streams dS from HBM and does one
+// MFMA per 512 bytes of it, so what matters is the number of bytes on their way); a wave then forms
+// dQ[64 rows x 64 d] += dS[64 x 64 keys] K[64 keys x 64 d] from transpose reads of both (dS lies key-major,
+// K row-major, and both operands want the keys along a lane's registers): 16 MFMAs.
+constexpr int kLqThreads = 512;
+constexpr int kLqUnits = 4;
+constexpr int kLqStageDs = kLqUnits * 8192;            // per unit: 64 rows x 64 keys of dS
+constexpr int kLqStage = kTileBytes + kLqStageDs;      // K rows of the step + dS
+constexpr int kLqStages = 3;
+constexpr int kLqSmem = kLqStages * kLqStage;
+constexpr int kLqCopies = 6;                           // asynchronous copies per wave and step
+
+template <int G>
+__global__ __launch_bounds__(kLqThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dq_from_ds_kernel(const BwdParams p) {
+    static_assert(G == 1 || G == 2 || G == 4, "four (64-row tile, head) units per workgroup");
+    constexpr int BM = 32 * (8 / G);
+    HIP_DYNAMIC_SHARED(unsigned char, smem_array)
+    TAH_LDS_ZERO_BASED(smem, smem_array);
+    const int tid = threadIdx.x, lane = tid % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int half = lane / 32, col = lane % 32;
+    const int hk = blockIdx.x;
+
+    int seq = 0, row0 = 0, row_end = 0;
+    bool second = false;
+    const int listed = sched_lookup(p.sched, false, p.nseq, G, p.s1.total_q, p.s2.total_q, p.s1.total_k, p.s2.total_k,
+                                    (int)gridDim.y, (int)blockIdx.y, second, seq, row0);
+    if (listed < 0) return;
+    if (listed > 0) {
+        const int hi = const_i32(second ? p.s2.cu_q : p.s1.cu_q, seq + 1);
+        row_end = row0 + BM < hi ? row0 + BM : hi;
+    } else {
+        int slot = (int)(gridDim.y - 1 - blockIdx.y);  // late (heavy) tiles of each sequence first
+        if (!(p.s1.total_q > 0 && find_tile(p.s1.cu_q, p.nseq, BM, slot, seq, row0, row_end))) {
+            if (!(p.s2.total_q > 0 && find_tile(p.s2.cu_q, p.nseq, BM, slot, seq, row0, row_end))) return;
+            second = true;
+        }
+    }
+    const BwdStream& qs = second ? p.s2 : p.s1;
+    const int q_lo = const_i32(qs.cu_q, seq);
+    const int k1_lo = const_i32(p.s1.cu_k, seq);
+    const int lk1 = const_i32(p.s1.cu_k, seq + 1) - k1_lo;
+    const int lq1 = p.s1.total_q > 0 ? const_i32(p.s1.cu_q, seq + 1) - const_i32(p.s1.cu_q, seq) : 0;
+    const int off = lk1 - lq1;  // position of depth-0 query row i of the sequence is i + off
+    const __bf16* k1p = p.s1.k + (int64_t)k1_lo * p.s1.k_rs + (int64_t)hk * p.s1.k_hs;
+    const int left1 = p.s1.total_k - k1_lo;
+    int lk2 = 0, left2 = 0;
+    const __bf16* k2p = nullptr;
+    if (second) {
+        const int k2_lo = const_i32(p.s2.cu_k, seq);
+        lk2 = const_i32(p.s2.cu_k, seq + 1) - k2_lo;
+        k2p = p.s2.k + (int64_t)k2_lo * p.s2.k_rs + (int64_t)hk * p.s2.k_hs;
+        left2 = p.s2.total_k - k2_lo;
+    }
+
+    // my unit: 64-row tile `tile` of the sequence's query rows (all wave-uniform)
+    const int unit = wave / 2, dh = wave % 2;
+    const int utile = unit / G, uhead = hk * G + unit % G;
+    const int tile0 = (row0 - q_lo) / kBN;                 // first 64-row tile of the workgroup
+    const int ntiles_wg = (row_end - row0 + kBN - 1) / kBN;  // tiles of the workgroup that exist (>= 1)
+    const bool unit_ok = utile < ntiles_wg;
+    // 64-key steps that hold a key visible to some row of 64-row tile t (depth-0 rows see positions <= row + off)
+    auto steps_of = [&](int t) {
+        if (second) return (lk1 + kBN - 1) / kBN;
+        const int last = 64 * t + 63 + off < lk1 - 1 ? 64 * t + 63 + off : lk1 - 1;
+        return last >= 0 ? last / kBN + 1 : 0;
+    };
+    const int my_n1 = __builtin_amdgcn_readfirstlane(unit_ok ? steps_of(tile0 + utile) : 0);
+    const int n1 = __builtin_amdgcn_readfirstlane(steps_of(tile0 + ntiles_wg - 1));  // the workgroup's last tile sees the most
+    const int n2 = second ? (lk2 + kBN - 1) / kBN : 0;
+    const int nsteps = n1 + n2;
+
+    // where my unit's blocks start: (qslot, head), key tile 0.  A unit without a tile copies the first unit's
+    // blocks (memory that exists; never used).
+    const int qslot = (second ? p.ds_q1slots : 0) + q_lo / kBN + seq + tile0 + (unit_ok ? utile : 0);
+    const unsigned char* ds_unit = p.ds_ws + (int64_t)(qslot * p.hq + uhead) * p.ds_kt * kDsBlockBytes;
+
+    // asynchronous copies of one step: K rows as in the dQ kernel (4 rows per copy, two copies per wave), then four
+    // 1 KiB pieces of my unit's dS: piece pi = 4 * dh + j covers the key-tile kernel's wave (pi / 4, 2 * hh + (pi % 4) / 2)
+    const int my_lrow = 8 * wave + (lane >> 4);
+    const uint32_t my_chunk0 = (uint32_t)(((lane & 15) ^ row_swizzle(my_lrow)) * 16);
+    const uint32_t my_chunk1 = (uint32_t)(((lane & 15) ^ row_swizzle(my_lrow + 4)) * 16);
+    auto issue_step = [&](int s, int stage) {
+        const bool s0 = s < n1;
+        const int ks = s0 ? s : s - n1;  // 64-key step inside its segment
+        const int64_t krs = s0 ? p.s1.k_rs : p.s2.k_rs;
+        const __bf16* kt0 = (s0 ? k1p : k2p) + (int64_t)ks * kBN * krs;
+        const int last = (s0 ? left1 : left2) - 1 - ks * kBN;
+        auto* kt = smem + stage * kLqStage;
+        const uint32_t r0 = (uint32_t)(my_lrow < last ? my_lrow : last) & 63u;
+        const uint32_t r1 = (uint32_t)(my_lrow + 4 < last ? my_lrow + 4 : last) & 63u;
+        const uint32_t krs2 = (uint32_t)(krs * 2) & 0xffffffu;
+        async_copy_16B(kt0, r0 * krs2 + my_chunk0, kt + (2 * wave) * 1024);
+        async_copy_16B(kt0, r1 * krs2 + my_chunk1, kt + (2 * wave + 1) * 1024);
+        const int ktile = (s0 ? 0 : p.ds_kt1) + ks / 2, hh = ks % 2;
+        const unsigned char* blk = ds_unit + (int64_t)ktile * kDsBlockBytes;
+        auto* dst = kt + kTileBytes + unit * 8192 + dh * 4096;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            // piece pi = 4 * dh + j: query half pi / 4 = dh, key block 2 * hh + j / 2, KiB j % 2 of that wave's 2 KiB
+            const uint32_t src = (uint32_t)((4 * dh + 2 * hh + j / 2) * kDsWaveBytes + (j % 2) * 1024 + lane * 16);
+            async_copy_16B_stream(blk, src, dst + j * 1024);
+        }
+    };
+
+    // per-lane LDS read offsets
+    // dS operand (A: rows = my 32 query rows of block qb, 8 keys 16*ks4 + 8*half + 0..7): two transpose reads;
+    // lane f of a 16-lane group points at the four rows 16*a2 + 4*(f%4) + 0..3 of key k0 + f/4
+    const int f16 = lane & 15, a2 = (lane >> 4) & 1;
+    const int ds_lane = ds_piece_off(a2, 8 * half + (f16 >> 2), f16 & 1) + 8 * ((f16 >> 1) & 1);
+    // K operand (B: columns = d, same 8 keys): rows 16*ks4 + 8*half + f/4 (+4), columns 64*dh + 32*dt + 16*a2 + 4*(f%4)
+    int k_lane[2][2];
+#pragma unroll
+    for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int r = 8 * half + 4 * u + (f16 >> 2), cc = 64 * dh + 32 * dt + 16 * a2 + 4 * (f16 & 3);
+            k_lane[dt][u] = rowmajor128_off(r, cc >> 3) + (cc & 7) * 2;
+        }
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[qb][dt][r] = 0.f;
+
+    auto compute = [&](int stage) __attribute__((always_inline)) {
+        const auto* kt = smem + stage * kLqStage;
+        const auto* ds = kt + kTileBytes + unit * 8192;
+#pragma unroll
+        for (int ks4 = 0; ks4 < 4; ++ks4) {
+            bf16x8 a[2], b[2];
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb) {
+                // query half qb, key block ks4 / 2 of the step: the copied piece layout is [qb][key block][2 KiB]
+                const auto* w = ds + qb * 4096 + (ks4 / 2) * 2048 + (ks4 % 2) * 1024 + ds_lane;
+                const bf16x4 lo = lds_read_tr16(w), hi = lds_read_tr16(w + 256);
+                a[qb] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            }
+#pragma unroll
+            for (int dt = 0; dt < 2; ++dt) {
+                const bf16x4 lo = lds_read_tr16(kt + k_lane[dt][0] + ks4 * 4096), hi = lds_read_tr16(kt + k_lane[dt][1] + ks4 * 4096);
+                b[dt] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            }
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+                for (int dt = 0; dt < 2; ++dt) acc[qb][dt] = mfma32(a[qb], b[dt], acc[qb][dt]);
+        }
+    };
+
+    if (nsteps > 0) issue_step(0, 0);
+    if (nsteps > 1) issue_step(1, 1);
+    int stage = 0;
+    for (int s = 0; s < nsteps; ++s) {
+        // the copies of step s are in; those of step s + 1 (the last kLqCopies this wave issued) may still be on their way
+        if (s + 1 < nsteps) TAH_WAIT_VMEM_N(kLqCopies); else TAH_WAIT_VMEM();
+        __syncthreads();
+        if (s + 2 < nsteps) issue_step(s + 2, stage == 0 ? 2 : stage - 1);
+        if (s >= n1 ? unit_ok : s < my_n1) compute(stage);
+        stage = stage == 2 ? 0 : stage + 1;
+    }
+
+    if (unit_ok) {
+        // accumulator (qb, dt, reg r, lane): row 32*qb + acc_row(half, r) of my tile, d = 64*dh + 32*dt + col
+        const int trow0 = row0 + utile * kBN;
+        const int tend = qs.cu_q[seq + 1];
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = trow0 + 32 * qb + acc_row(half, r);
+                if (row < tend) {
+                    __bf16* drow = qs.dq + (int64_t)row * qs.dq_rs + (int64_t)uhead * qs.dq_hs + 64 * dh + col;
+                    drow[0] = (__bf16)(acc[qb][0][r] * p.scale);
+                    drow[32] = (__bf16)(acc[qb][1][r] * p.scale);
                 }
             }
     }
@@ -766,6 +1022,23 @@ int launch_bwd(const BwdParams& p, hipStream_t st) {
     if (p.s2.total_q > 0) qtiles += p.s2.total_q / BM + p.nseq;
     if (p.s1.total_k > 0) ktiles += p.s1.total_k / kBK + p.nseq;
     if (p.s2.total_k > 0) ktiles += p.s2.total_k / kBK + p.nseq;
+    if constexpr (!kDense && G <= 4) {
+        if (p.ds_ws) {  // dS exchange: the key-tile kernel writes dS, dQ is one product that reads it back
+            if (ktiles > 0) {
+                if (hipFuncSetAttribute(reinterpret_cast<const void*>(&duo_bwd_dkdv_kernel<G, false, true>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, kKvSmem) != hipSuccess)
+                    return TAH_E_LAUNCH;
+                hipLaunchKernelGGL((duo_bwd_dkdv_kernel<G, false, true>), dim3(p.hkv, ktiles), dim3(kKvThreads), kKvSmem, st, p);
+            }
+            if (qtiles > 0) {
+                if (hipFuncSetAttribute(reinterpret_cast<const void*>(&duo_bwd_dq_from_ds_kernel<G>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLqSmem) != hipSuccess)
+                    return TAH_E_LAUNCH;
+                hipLaunchKernelGGL((duo_bwd_dq_from_ds_kernel<G>), dim3(p.hkv, qtiles), dim3(kLqThreads), kLqSmem, st, p);
+            }
+            return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
+        }
+    }
     if (qtiles > 0) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(&duo_bwd_dq_kernel<G, kDense>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kDqSmem) != hipSuccess)
@@ -773,10 +1046,10 @@ int launch_bwd(const BwdParams& p, hipStream_t st) {
         hipLaunchKernelGGL((duo_bwd_dq_kernel<G, kDense>), dim3(p.hkv, qtiles), dim3(kDqThreads), kDqSmem, st, p);
     }
     if (ktiles > 0) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&duo_bwd_dkdv_kernel<G, kDense>),
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&duo_bwd_dkdv_kernel<G, kDense, false>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kKvSmem) != hipSuccess)
             return TAH_E_LAUNCH;
-        hipLaunchKernelGGL((duo_bwd_dkdv_kernel<G, kDense>), dim3(p.hkv, ktiles), dim3(kKvThreads), kKvSmem, st, p);
+        hipLaunchKernelGGL((duo_bwd_dkdv_kernel<G, kDense, false>), dim3(p.hkv, ktiles), dim3(kKvThreads), kKvSmem, st, p);
     }
     return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
 }
@@ -809,6 +1082,18 @@ int dispatch_bwd(const tah_duo_bwd_args* a, const tah_additive_mask* m, tah_stre
     p.scale = f.scale;
     p.scale_log2e = f.scale * kLog2e;
     p.sched = kDense ? nullptr : static_cast<const int32_t*>(f.schedule);
+    p.ds_ws = nullptr;
+    p.ds_q1slots = p.ds_kt1 = p.ds_kt = 0;
+    if (!kDense && a->ds_workspace && g <= 4) {
+        if (reinterpret_cast<uintptr_t>(a->ds_workspace) & 15) return TAH_E_ALIGN;
+        const size_t need = tah_duo_bwd_workspace_bytes(f.nseq, f.hq, f.hkv, f.s1.total_q, f.s1.total_k, f.s2.total_q, f.s2.total_k,
+                                                        a->max_seqlen_k1, a->max_seqlen_k2);
+        if (a->ds_workspace_bytes < need) return TAH_E_WORKSPACE;
+        p.ds_ws = static_cast<unsigned char*>(a->ds_workspace);
+        p.ds_q1slots = ds_query_slots(f.s1.total_q, f.nseq);
+        p.ds_kt1 = ds_key_slots(f.s1.total_k, a->max_seqlen_k1);
+        p.ds_kt = p.ds_kt1 + ds_key_slots(f.s2.total_k, a->max_seqlen_k2);
+    }
     p.mask = nullptr;
     p.mask_sb = p.mask_sh = p.mask_sq = p.mask_sk = 0;
     p.mask_f32 = 0;
@@ -829,6 +1114,14 @@ int dispatch_bwd(const tah_duo_bwd_args* a, const tah_additive_mask* m, tah_stre
 }
 }  // namespace
 }  // namespace tah
+
+extern "C" size_t tah_duo_bwd_workspace_bytes(int32_t nseq, int32_t hq, int32_t hkv, int32_t total_q1, int32_t total_k1,
+                                              int32_t total_q2, int32_t total_k2, int32_t max_seqlen_k1, int32_t max_seqlen_k2) {
+    if (nseq <= 0 || hq <= 0 || hkv <= 0 || hq % hkv != 0 || hq / hkv > 4) return 0;
+    const size_t qslots = (size_t)tah::ds_query_slots(total_q1, nseq) + (size_t)tah::ds_query_slots(total_q2, nseq);
+    const size_t kslots = (size_t)tah::ds_key_slots(total_k1, max_seqlen_k1) + (size_t)tah::ds_key_slots(total_k2, max_seqlen_k2);
+    return qslots * (size_t)hq * kslots * (size_t)tah::kDsBlockBytes;
+}
 
 extern "C" int tah_duo_bwd_varlen(const tah_duo_bwd_args* a, tah_stream_t stream) {
     return tah::dispatch_bwd<false>(a, nullptr, stream);

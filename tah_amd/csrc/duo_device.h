@@ -11,6 +11,26 @@ typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 
+// LDS addressed through pointers that carry the LDS address space and start at LDS address 0.  A kernel that
+// declares no static LDS object has its dynamic LDS at address 0; a pointer made from that integer (instead of
+// the extern array's symbol, whose zero the compiler only learns after instruction selection) lets constant
+// parts of an offset fold into the instructions' immediate fields -- no `v_add_u32 v, 0, v` per access -- and
+// needs no generic-to-LDS conversion (a compare and a select each) where an address goes into m0.
+#ifdef TAH_CPU_EMU
+typedef unsigned char lds_byte;
+typedef float lds_float;
+typedef int lds_int;
+#define TAH_LDS_ZERO_BASED(name, decl) unsigned char* const name = decl
+#define TAH_LDS_CAST(T, p) (reinterpret_cast<T*>(p))
+#else
+typedef __attribute__((address_space(3))) unsigned char lds_byte;
+typedef __attribute__((address_space(3))) float lds_float;
+typedef __attribute__((address_space(3))) int lds_int;
+#define TAH_LDS_ZERO_BASED(name, decl) \
+    tah::lds_byte* const name = reinterpret_cast<tah::lds_byte*>(static_cast<uintptr_t>(0)); (void)decl
+#define TAH_LDS_CAST(T, p) (reinterpret_cast<__attribute__((address_space(3))) T*>(p))
+#endif
+
 constexpr int kWave = 64;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
@@ -79,6 +99,29 @@ __device__ __forceinline__ void async_copy_16B(const void* gsrc, unsigned char* 
 __device__ __forceinline__ void async_copy_16B(const void* sbase, uint32_t voff, unsigned char* lds_wave_base) {
     TAH_ASYNC_COPY_16B_SO(sbase, voff, lds_wave_base);
 }
+// The same copy for data that is read once (streaming: the lines are not kept in the L2).
+#ifndef TAH_ASYNC_COPY_16B_SO_NT
+#define TAH_ASYNC_COPY_16B_SO_NT(sbase, voff, lds_wave_base)                                                       \
+    do {                                                                                                           \
+        const unsigned tah_m0_ = __builtin_amdgcn_readfirstlane(                                                   \
+            (unsigned)(uintptr_t)(__attribute__((address_space(3))) void*)(lds_wave_base));                        \
+        const uint64_t tah_b_ = (uint64_t)(uintptr_t)(sbase);                                                      \
+        const uint64_t tah_sb_ = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((unsigned)tah_b_) |            \
+                                 ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((unsigned)(tah_b_ >> 32)) << 32); \
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"                           \
+                     :                                                                                             \
+                     : "s"(tah_m0_), "v"(voff), "s"(tah_sb_)                                                       \
+                     : "memory");                                                                                  \
+    } while (0)
+#endif
+__device__ __forceinline__ void async_copy_16B_stream(const void* sbase, uint32_t voff, unsigned char* lds_wave_base) {
+    TAH_ASYNC_COPY_16B_SO_NT(sbase, voff, lds_wave_base);
+}
+#ifndef TAH_CPU_EMU
+__device__ __forceinline__ void async_copy_16B_stream(const void* sbase, uint32_t voff, lds_byte* lds_wave_base) {
+    TAH_ASYNC_COPY_16B_SO_NT(sbase, voff, lds_wave_base);
+}
+#endif
 // Same with 4 bytes per lane (global_load_lds_dword): lane l's dword lands at lds_wave_base + 4*l.
 #ifndef TAH_ASYNC_COPY_4B
 #define TAH_ASYNC_COPY_4B(gsrc, lds_wave_base)                                                                     \
@@ -112,6 +155,15 @@ __device__ __forceinline__ void async_copy_4B(const void* gsrc, void* lds_wave_b
 __device__ __forceinline__ void async_copy_4B(const void* sbase, uint32_t voff, void* lds_wave_base) {
     TAH_ASYNC_COPY_4B_SO(sbase, voff, lds_wave_base);
 }
+#ifndef TAH_CPU_EMU
+// the same copies with the destination given as an LDS-address-space pointer
+__device__ __forceinline__ void async_copy_16B(const void* sbase, uint32_t voff, lds_byte* lds_wave_base) {
+    TAH_ASYNC_COPY_16B_SO(sbase, voff, lds_wave_base);
+}
+__device__ __forceinline__ void async_copy_4B(const void* sbase, uint32_t voff, lds_float* lds_wave_base) {
+    TAH_ASYNC_COPY_4B_SO(sbase, voff, lds_wave_base);
+}
+#endif
 // acc (16 floats of an MFMA accumulator) *= a, executed only if the wave-uniform `cond` is non-zero.
 // The branch lives inside the assembly so that the compiler sees one unconditional in-place update:
 // a C++ `if` around accumulator updates makes it keep two copies of the accumulators.
@@ -167,6 +219,10 @@ __device__ __forceinline__ void async_copy_4B(const void* sbase, uint32_t voff, 
 // bookkeeping also learns that no ordinary load is pending past this point.
 #define TAH_WAIT_VMEM() __builtin_amdgcn_s_waitcnt(0x0F70)
 #endif
+#ifndef TAH_WAIT_VMEM_N
+// s_waitcnt vmcnt(n), n <= 15: all but the n most recently issued loads / asynchronous copies have landed
+#define TAH_WAIT_VMEM_N(n) __builtin_amdgcn_s_waitcnt(0x0F70 | (n))
+#endif
 
 // LDS tile of R rows x 128 bf16 (256 B per row, 16 chunks of 16 B).  The chunk index is XORed
 // with a 4-bit function of the row that (a) takes 16 different values over 16 consecutive rows,
@@ -188,6 +244,12 @@ __device__ __forceinline__ bf16x4 lds_read_tr16(const unsigned char* p) {
     typedef __attribute__((address_space(3))) bf16x4 lds_bf16x4;
     return __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)p);
 }
+#ifndef TAH_CPU_EMU
+__device__ __forceinline__ bf16x4 lds_read_tr16(const lds_byte* p) {
+    typedef __attribute__((address_space(3))) bf16x4 lds_bf16x4;
+    return __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)p);
+}
+#endif
 
 // MFMA operand whose contraction index runs over the ROWS of a row-major [rows][128] bf16 LDS
 // tile (rowmajor128_off layout): returns, for this lane, the 8 values

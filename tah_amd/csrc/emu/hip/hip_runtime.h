@@ -31,6 +31,7 @@
 #define TAH_CPU_EMU 1
 #define TAH_MUL_INPLACE(x, a) ((x) *= (a))
 #define TAH_WAIT_VMEM() ((void)0)
+#define TAH_WAIT_VMEM_N(n) ((void)0)
 #define TAH_KEEP_HERE4(a, b, c, d) ((void)0)
 #define TAH_OPAQUE2(a, b) ((void)0)
 #define TAH_OPAQUE1(a) ((void)0)
@@ -40,6 +41,7 @@
     memcpy((unsigned char*)(lds_wave_base) + 16 * emu::t_lane, (const void*)(gsrc), 16)
 #define TAH_ASYNC_COPY_16B_SO(sbase, voff, lds_wave_base) \
     memcpy((unsigned char*)(lds_wave_base) + 16 * emu::t_lane, (const unsigned char*)(sbase) + (voff), 16)
+#define TAH_ASYNC_COPY_16B_SO_NT(sbase, voff, lds_wave_base) TAH_ASYNC_COPY_16B_SO(sbase, voff, lds_wave_base)
 #define TAH_ASYNC_COPY_4B_SO(sbase, voff, lds_wave_base) \
     memcpy((unsigned char*)(lds_wave_base) + 4 * emu::t_lane, (const unsigned char*)(sbase) + (voff), 4)
 #define TAH_ASYNC_COPY_4B(gsrc, lds_wave_base) \

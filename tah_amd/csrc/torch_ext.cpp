@@ -26,6 +26,7 @@ struct Api {
     decltype(&tah_duo_error_string) error_string = nullptr;
     decltype(&tah_duo_fwd_varlen) fwd_varlen = nullptr;
     decltype(&tah_duo_bwd_varlen) bwd_varlen = nullptr;
+    decltype(&tah_duo_bwd_workspace_bytes) bwd_workspace_bytes = nullptr;
     decltype(&tah_duo_schedule_bytes) schedule_bytes = nullptr;
     decltype(&tah_duo_schedule_build) schedule_build = nullptr;
     decltype(&tah_greedy_step) greedy_step = nullptr;
@@ -69,6 +70,7 @@ void load_library(const std::string& path, bool allow_host) {
     bind(g.error_string, "tah_duo_error_string");
     bind(g.fwd_varlen, "tah_duo_fwd_varlen");
     bind(g.bwd_varlen, "tah_duo_bwd_varlen");
+    bind(g.bwd_workspace_bytes, "tah_duo_bwd_workspace_bytes");
     bind(g.schedule_bytes, "tah_duo_schedule_bytes");
     bind(g.schedule_build, "tah_duo_schedule_build");
     bind(g.greedy_step, "tah_greedy_step");
@@ -217,7 +219,8 @@ std::vector<Tensor> duo_bwd_varlen(const Tensor& q1, const Tensor& k1, const Ten
                                    const Tensor& do1, const Tensor& cu_q1, const Tensor& cu_k1, const Tensor& q2, const Tensor& k2,
                                    const Tensor& v2, const Tensor& o2, const Tensor& lse2, const Tensor& do2, const Tensor& pos_q2,
                                    const Tensor& pos_k2, const Tensor& cu_q2, const Tensor& cu_k2, double scale,
-                                   const optional<Tensor>& schedule) {
+                                   const optional<Tensor>& schedule, const optional<Tensor>& ds_workspace,
+                                   int64_t max_seqlen_k1, int64_t max_seqlen_k2) {
     need_lib();
     for (auto p : {std::make_pair(&q1, "q1"), {&k1, "k1"}, {&v1, "v1"}, {&o1, "o1"}, {&do1, "do1"}, {&q2, "q2"}, {&k2, "k2"},
                    {&v2, "v2"}, {&o2, "o2"}, {&do2, "do2"}})
@@ -234,8 +237,8 @@ std::vector<Tensor> duo_bwd_varlen(const Tensor& q1, const Tensor& k1, const Ten
     const int64_t hq = q1.size(1);
     auto dq1 = at::empty(q1.sizes(), q1.options()), dk1 = at::empty(k1.sizes(), k1.options()), dv1 = at::empty(v1.sizes(), v1.options());
     auto dq2 = at::empty(q2.sizes(), q2.options()), dk2 = at::empty(k2.sizes(), k2.options()), dv2 = at::empty(v2.sizes(), v2.options());
-    auto delta1 = at::empty({hq, q1.size(0)}, q1.options().dtype(at::kFloat));
-    auto delta2 = at::empty({hq, q2.size(0)}, q1.options().dtype(at::kFloat));
+    auto delta1 = at::empty({2, hq, q1.size(0)}, q1.options().dtype(at::kFloat));
+    auto delta2 = at::empty({2, hq, q2.size(0)}, q1.options().dtype(at::kFloat));
     tah_duo_bwd_args a{};
     fill_stream(a.fwd.s1, q1, k1, v1, o1, lse1, cu_q1, cu_k1, nullptr, nullptr);
     fill_stream(a.fwd.s2, q2, k2, v2, o2, lse2, cu_q2, cu_k2, &pos_q2, &pos_k2);
@@ -244,6 +247,14 @@ std::vector<Tensor> duo_bwd_varlen(const Tensor& q1, const Tensor& k1, const Ten
     a.fwd.schedule = schedule_ptr(schedule);
     fill_bwd_stream(a.g1, do1, dq1, dk1, dv1, delta1);
     fill_bwd_stream(a.g2, do2, dq2, dk2, dv2, delta2);
+    if (ds_workspace && ds_workspace->defined() && ds_workspace->numel() > 0) {
+        d.see(*ds_workspace);
+        TORCH_CHECK(ds_workspace->is_contiguous(), "ds_workspace must be contiguous");
+        a.ds_workspace = ds_workspace->data_ptr();
+        a.ds_workspace_bytes = (size_t)ds_workspace->numel() * ds_workspace->element_size();
+        a.max_seqlen_k1 = (int32_t)max_seqlen_k1;
+        a.max_seqlen_k2 = (int32_t)max_seqlen_k2;
+    }
     check_rc(g.bwd_varlen(&a, d.stream()), "tah_duo_bwd_varlen");
     return {dq1, dk1, dv1, dq2, dk2, dv2};
 }
@@ -297,10 +308,10 @@ std::vector<Tensor> duo_bwd_masked(const Tensor& q, const Tensor& k, const Tenso
     TORCH_CHECK(lse.scalar_type() == at::kFloat && lse.is_contiguous(), "lse must be contiguous float32 [Hq, rows]");
     const int64_t tq = q.size(0) / nseq, tk = k.size(0) / nseq, hq = q.size(1);
     auto dq = at::empty(q.sizes(), q.options()), dk = at::empty(k.sizes(), k.options()), dv = at::empty(v.sizes(), v.options());
-    auto delta = at::empty({hq, q.size(0)}, q.options().dtype(at::kFloat));
+    auto delta = at::empty({2, hq, q.size(0)}, q.options().dtype(at::kFloat));
     auto cu_q = dense_cu(q, nseq, tq), cu_k = dense_cu(q, nseq, tk);
     auto zc = at::zeros({nseq + 1}, q.options().dtype(at::kInt));
-    auto e = q.narrow(0, 0, 0), ek = k.narrow(0, 0, 0), el = lse.narrow(1, 0, 0), ed = delta.narrow(1, 0, 0);
+    auto e = q.narrow(0, 0, 0), ek = k.narrow(0, 0, 0), el = lse.narrow(1, 0, 0), ed = delta.narrow(2, 0, 0);
     tah_duo_bwd_args a{};
     fill_stream(a.fwd.s1, q, k, v, o, lse, cu_q, cu_k, nullptr, nullptr);
     fill_stream(a.fwd.s2, e, ek, ek, e, el, zc, zc, nullptr, nullptr);
@@ -885,6 +896,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("greedy_step", &greedy_step);
     m.def("duo_fwd_varlen", &duo_fwd_varlen);
     m.def("duo_bwd_varlen", &duo_bwd_varlen);
+    m.def("duo_bwd_workspace_bytes", [](int64_t nseq, int64_t hq, int64_t hkv, int64_t tq1, int64_t tk1, int64_t tq2, int64_t tk2,
+                                        int64_t mk1, int64_t mk2) {
+        need_lib();
+        return (int64_t)g.bwd_workspace_bytes((int32_t)nseq, (int32_t)hq, (int32_t)hkv, (int32_t)tq1, (int32_t)tk1, (int32_t)tq2,
+                                              (int32_t)tk2, (int32_t)mk1, (int32_t)mk2);
+    });
     m.def("duo_fwd_masked", &duo_fwd_masked);
     m.def("duo_bwd_masked", &duo_bwd_masked);
     m.def("decode_workspace_bytes", &decode_workspace_bytes);

@@ -48,11 +48,50 @@ def duo_fwd_varlen(q1, k1, v1, cu_q1, cu_k1, q2, k2, v2, pos_q2, pos_k2, cu_q2, 
     return _call("duo_fwd_varlen", q1, k1, v1, cu_q1, cu_k1, q2, k2, v2, pos_q2, pos_k2, cu_q2, cu_k2, float(scale), schedule)
 
 
+# The backward pass can hand dS from the dK/dV kernel to the dQ kernel through a workspace instead of computing the
+# scores twice (``tah_duo_bwd_varlen`` with ``ds_workspace``): 5 matrix products per tile pair instead of 7.  The
+# workspace holds about total_q * max_seqlen_k * Hq * 2 bytes; calls that would need more than DS_EXCHANGE_MAX_BYTES
+# (or Hq / Hkv > 4) run the three-kernel backward.  One buffer per device is kept and grown on demand: the calls of
+# a backward pass run one after another on one stream and nothing in it outlives a call.
+DS_EXCHANGE = True
+DS_EXCHANGE_MAX_BYTES = 24 << 30
+_ds_workspaces = {}
+
+
+def duo_bwd_workspace_bytes(nseq: int, hq: int, hkv: int, total_q1: int, total_k1: int, total_q2: int, total_k2: int,
+                            max_seqlen_k1: int = 0, max_seqlen_k2: int = 0) -> int:
+    """Bytes of ``ds_workspace`` for a backward call of these sizes (0: the call cannot use one)."""
+    return int(_call("duo_bwd_workspace_bytes", int(nseq), int(hq), int(hkv), int(total_q1), int(total_k1), int(total_q2),
+                     int(total_k2), int(max_seqlen_k1), int(max_seqlen_k2)))
+
+
+def _ds_workspace(device, nbytes: int):
+    buf = _ds_workspaces.get(device)
+    if buf is None or buf.numel() < nbytes:
+        _ds_workspaces[device] = None  # release the old one before the larger one is requested
+        buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        _ds_workspaces[device] = buf
+    return buf
+
+
 def duo_bwd_varlen(q1, k1, v1, o1, lse1, do1, cu_q1, cu_k1, q2, k2, v2, o2, lse2, do2, pos_q2, pos_k2, cu_q2, cu_k2,
-                   scale: float, schedule=None):
-    """Backward of :func:`duo_fwd_varlen`; returns dq1, dk1, dv1, dq2, dk2, dv2 (bf16)."""
+                   scale: float, schedule=None, ds_workspace=None, max_seqlen_k1: int = 0, max_seqlen_k2: int = 0):
+    """Backward of :func:`duo_fwd_varlen`; returns dq1, dk1, dv1, dq2, dk2, dv2 (bf16).
+
+    ``ds_workspace``: a uint8 tensor of at least :func:`duo_bwd_workspace_bytes` bytes, ``False`` for the three-kernel
+    backward, or None: the package's own buffer when ``DS_EXCHANGE`` is on and the call fits ``DS_EXCHANGE_MAX_BYTES``.
+    ``max_seqlen_k1`` / ``max_seqlen_k2``: upper bounds on one sequence's key rows per depth (0: unknown); they only
+    make the workspace smaller.
+    """
+    if ds_workspace is None and DS_EXCHANGE:
+        need = duo_bwd_workspace_bytes(cu_q1.numel() - 1, q1.shape[1], k1.shape[1], q1.shape[0], k1.shape[0], q2.shape[0],
+                                       k2.shape[0], max_seqlen_k1, max_seqlen_k2)
+        if 0 < need <= DS_EXCHANGE_MAX_BYTES:
+            ds_workspace = _ds_workspace(q1.device, need)
+    if ds_workspace is False:
+        ds_workspace = None
     return tuple(_call("duo_bwd_varlen", q1, k1, v1, o1, lse1, do1, cu_q1, cu_k1, q2, k2, v2, o2, lse2, do2, pos_q2, pos_k2,
-                       cu_q2, cu_k2, float(scale), schedule))
+                       cu_q2, cu_k2, float(scale), schedule, ds_workspace, int(max_seqlen_k1), int(max_seqlen_k2)))
 
 
 def duo_fwd_masked(q, k, v, mask, nseq: int, scale: float):

@@ -30,12 +30,43 @@ def test_bwd_matches_oracle(hq, hkv, seqlens, p, seed, kw):
     print(check_grads(got, want), flush=True)
 
 
-def test_bwd_is_deterministic():
+@pytest.mark.parametrize("ds_workspace", [None, False], ids=["ds-exchange", "three-kernel"])
+def test_bwd_is_deterministic(ds_workspace):
     dev = to_device(make_varlen_case(21, [900, 200], 0.1))
-    a, _ = run_bwd(dev, 1)
-    b, _ = run_bwd(dev, 1)
+    a, _ = run_bwd(dev, 1, ds_workspace=ds_workspace, want_oracle=False)
+    b, _ = run_bwd(dev, 1, ds_workspace=ds_workspace, want_oracle=False)
     for x, y in zip(a, b):
         assert torch.equal(x, y)
+
+
+@pytest.mark.parametrize("hq,hkv,seqlens,p,seed,kw", [
+    (16, 8, [300, 1000, 17, 129], 0.10, 2, {}),
+    (8, 8, [257, 64], 0.2, 3, {}),
+    (16, 4, [700], 0.3, 4, {}),
+    (16, 8, [40, 1, 300], 0.3, 11, dict(seqlens_k=[500, 900, 300], extra_k2=100)),
+    (16, 8, [2500], 0.06, 12, {}),
+])
+def test_ds_exchange_against_three_kernel_backward(hq, hkv, seqlens, p, seed, kw):
+    """Both backward paths on the same inputs: dK / dV equal to the bit (same kernel arithmetic), dQ of both within
+    the tolerance of the oracle; the exchange path with a caller's workspace sized by the per-sequence bounds and
+    pre-filled with NaN patterns (a block read before it was written would show) gives the default path's bits."""
+    from tah_amd import ops
+    print(f"ds exchange case hq={hq} hkv={hkv} seqlens={seqlens} p={p} seed={seed} {kw}", flush=True)
+    dev = to_device(make_varlen_case(seed, seqlens, p, Hq=hq, Hkv=hkv, D=128, **kw))
+    old, want = run_bwd(dev, seed + 100, ds_workspace=False)
+    new, _ = run_bwd(dev, seed + 100, want_oracle=False)
+    mk1 = int(np.diff(dev["cu_k1"].cpu().numpy()).max())
+    mk2 = int(np.diff(dev["cu_k2"].cpu().numpy()).max()) if dev["k2"].shape[0] else 0
+    need = ops.duo_bwd_workspace_bytes(len(seqlens), hq, hkv, dev["q1"].shape[0], dev["k1"].shape[0], dev["q2"].shape[0],
+                                       dev["k2"].shape[0], mk1, mk2)
+    ws = torch.full((need,), 0xFF, dtype=torch.uint8, device="cuda")
+    tight, _ = run_bwd(dev, seed + 100, ds_workspace=ws, want_oracle=False, max_seqlen_k1=mk1, max_seqlen_k2=mk2)
+    torch.cuda.synchronize()
+    print(check_grads(new, want), flush=True)
+    for i, n in enumerate(NAMES):
+        assert torch.equal(new[i], tight[i]), n
+        if n[1] != "q":
+            assert torch.equal(new[i], old[i]), n
 
 
 def test_bwd_full_size_training_config_vs_torch_fp32():
