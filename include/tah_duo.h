@@ -14,7 +14,11 @@
  * index j has position j, and a depth-0 query at local index i has position
  * i + (Lk1 - Lq1) (queries are the newest rows of the sequence).  Depth-1
  * ("iteration 2") rows exist only for hard tokens and carry their position
- * explicitly (pos_q2 / pos_k2, int32).
+ * explicitly (pos_q2 / pos_k2, int32).  Inside a sequence the depth-1 query rows
+ * come in ascending position (pos_q2 non-decreasing between cu_q2[b] and
+ * cu_q2[b+1]), the order in which gather_active packs hard tokens
+ * (tah/model/tah_model.py:114-117): the backward pass skips depth-1 query tiles
+ * by the position of their last row.
  *
  * Visibility (tah/model/tah_model.py:788): key (pos_k, depth_k) is visible to
  * query (pos_q, depth_q) iff pos_k <= pos_q and depth_k <= depth_q.

@@ -436,7 +436,23 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
         nt1 = (lq1 + kBQ - 1) / kBQ - t1_begin;
         if (nt1 < 0) nt1 = 0;
     }
-    const int nt2 = (lq2 + kBQ - 1) / kBQ;
+    // Depth-1 query tiles: rows of a sequence come in ascending position, so the tiles that can see a depth-0
+    // key tile are a suffix -- those whose last row has a position >= the tile's first key.  One lane per tile
+    // looks its last row up; every wave does the same and gets the same answer.
+    int t2_begin = 0;
+    const int nt2_all = (lq2 + kBQ - 1) / kBQ;
+    if (!second && !kDense && nt2_all > 0) {
+        t2_begin = nt2_all;
+        for (int t0 = 0; t0 < nt2_all; t0 += kWave) {
+            const int t = t0 + lane;
+            const int last = q2_lo + (t * kBQ + kBQ - 1 < lq2 - 1 ? t * kBQ + kBQ - 1 : lq2 - 1);
+            const bool sees = t < nt2_all && p.s2.pos_q[last] >= kl0;
+            const unsigned long long m = __builtin_amdgcn_ballot_w64(sees);
+            if (m) { t2_begin = t0 + __builtin_ctzll(m); break; }
+        }
+    }
+    const int q2_first = q2_lo + t2_begin * kBQ;  // first depth-1 query row staged by this workgroup
+    const int nt2 = nt2_all - t2_begin;
     const int nitems = (nt1 + nt2) * G;
     // Depth-0 query tiles [t_vis, t_whole) (relative to t1_begin) need no mask for this wave: all 64 rows
     // exist and the first row of my half already sees the last key of my block.
@@ -465,7 +481,7 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
     if constexpr (kExport) {
         const int ktile = (second ? p.ds_kt1 : 0) + kl0 / kBK;
         const int slot1 = q1_lo / kBQ + seq + t1_begin;
-        const int slot2 = p.ds_q1slots + q2_lo / kBQ + seq;
+        const int slot2 = p.ds_q1slots + q2_lo / kBQ + seq + t2_begin;
         ds_base1 = ((int64_t)slot1 * p.hq * p.ds_kt + ktile) * kDsBlockBytes + wave * kDsWaveBytes;
         ds_base2 = ((int64_t)slot2 * p.hq * p.ds_kt + ktile) * kDsBlockBytes + wave * kDsWaveBytes;
     }
@@ -482,7 +498,7 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
             r0 = q1_lo + (t1_begin + t) * kBQ;
             r_end = q1_lo + lq1;
         } else {
-            r0 = q2_lo + (t - nt1) * kBQ;
+            r0 = q2_first + (t - nt1) * kBQ;
             r_end = q2_lo + lq2;
         }
         r_end = r0 + kBQ < r_end ? r0 + kBQ : r_end;
@@ -512,7 +528,7 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
         r.grs2 = (uint32_t)(qs.do_rs * 2) & 0xffffffu;
         r.q_hs = qs.q_hs; r.g_hs = qs.do_hs;
         r.total_q = qs.total_q;
-        r.row_lo = q2s ? q2_lo : q1_lo + t1_begin * kBQ;
+        r.row_lo = q2s ? q2_first : q1_lo + t1_begin * kBQ;
         r.row_end = q2s ? q2_lo + lq2 : q1_lo + lq1;
         r.tile0 = q2s ? nt1 : 0;
         return r;
@@ -837,9 +853,15 @@ __global__ __launch_bounds__(kLqThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dq_
     const int ntiles_wg = (row_end - row0 + kBN - 1) / kBN;  // tiles of the workgroup that exist (>= 1)
     const bool unit_ok = utile < ntiles_wg;
     // 64-key steps that hold a key visible to some row of 64-row tile t (depth-0 rows see positions <= row + off)
+    // (the position of depth-1 row: pos_q, ascending inside a sequence, so a tile's last row has its largest)
+    const int q_end = const_i32(qs.cu_q, seq + 1);
     auto steps_of = [&](int t) {
-        if (second) return (lk1 + kBN - 1) / kBN;
-        const int last = 64 * t + 63 + off < lk1 - 1 ? 64 * t + 63 + off : lk1 - 1;
+        int reach = 64 * t + 63 + off;  // largest position a row of the tile has
+        if (second) {
+            const int r = q_lo + 64 * t + 63;
+            reach = const_i32(qs.pos_q, r < q_end - 1 ? r : q_end - 1);
+        }
+        const int last = reach < lk1 - 1 ? reach : lk1 - 1;
         return last >= 0 ? last / kBN + 1 : 0;
     };
     const int my_n1 = __builtin_amdgcn_readfirstlane(unit_ok ? steps_of(tile0 + utile) : 0);
@@ -943,7 +965,7 @@ __global__ __launch_bounds__(kLqThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dq_
     if (unit_ok) {
         // accumulator (qb, dt, reg r, lane): row 32*qb + acc_row(half, r) of my tile, d = 64*dh + 32*dt + col
         const int trow0 = row0 + utile * kBN;
-        const int tend = qs.cu_q[seq + 1];
+        const int tend = q_end;
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb)
 #pragma unroll
