@@ -351,7 +351,9 @@ int tah_topk_mix(const tah_topk_mix_args* args, tah_stream_t stream);
  * two calls, the outputs too up to the last bit of a rare element (the same arithmetic in the same order, compiled
  * twice).  append_at: int32 [rows], the number of rows sequence i's segment of prep->cache holds before the
  * call, i.e. cache.len[slot] -- handed in because the workgroups of a sequence cannot read the length while one of
- * them advances it (len[slot] becomes append_at[i] + 1).  Only for calls tah_duo_decode_step_supported() accepts (256
+ * them advances it (len[slot] becomes append_at[i] + 1; a row whose append_at differs from the length sets
+ * *prep->overflow to 2 where that flag is given: the slab then has a gap or an overwritten row; one query row per
+ * slot and call).  Only for calls tah_duo_decode_step_supported() accepts (256
  * or more (query, kv head) pairs, slabs of at most 4096 rows, one or two query heads per kv head: cases
  * tah_duo_decode runs without split-K); others return TAH_E_SHAPE and the caller makes the two calls.  append_depth: NULL,
  * or int32 [rows], 0 / 1 per row: the segment (dec->c1 / dec->c2) that row's K and V go to, for a batch whose rows are at
@@ -436,6 +438,8 @@ typedef struct tah_greedy_step_args {
     int64_t* out_tokens;      /* [rows, out_stride] column step_idx[0] is written */
     int64_t out_stride;
     const int64_t* step_idx;  /* [1] */
+    int32_t out_cols;         /* columns of out_tokens: with step_idx[0] >= out_cols (a captured step replayed more often
+                               * than the buffer has columns) nothing is stored and the row is marked finished */
     int32_t* out_len;         /* [rows] += 1 for rows still unfinished after this step */
     int64_t* n_hard;          /* += hard rows among those that decoded */
     int64_t* n_steps;         /* += rows that decoded */

@@ -205,7 +205,7 @@ class GreedyStepArgs(C.Structure):
         ("row_stride0", c_int64), ("row_stride1", c_int64),
         ("rows", c_int32), ("vocab", c_int32), ("eos", c_int32),
         ("tok", c_void_p), ("finished", c_void_p), ("pos", c_void_p), ("out_tokens", c_void_p), ("out_stride", c_int64),
-        ("step_idx", c_void_p), ("out_len", c_void_p), ("n_hard", c_void_p), ("n_steps", c_void_p),
+        ("step_idx", c_void_p), ("out_cols", c_int32), ("out_len", c_void_p), ("n_hard", c_void_p), ("n_steps", c_void_p),
     ]
 
 

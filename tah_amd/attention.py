@@ -198,6 +198,10 @@ class _Packed:
     def __init__(self, valid: Optional[torch.Tensor], pos: Optional[torch.Tensor], B: int, T: int, device):
         self.B, self.T = B, T
         self.n_dev = None
+        if valid is not None and tuple(valid.shape) != (B, T):
+            raise TahDuoError(f"valid mask of shape {tuple(valid.shape)} for a block of {B} x {T} rows")
+        if pos is not None and pos.numel() != B * T:
+            raise TahDuoError(f"positions of shape {tuple(pos.shape)} for a block of {B} x {T} rows")
         all_valid = valid is None
         if not all_valid:
             idx = HardIndex(valid)

@@ -45,6 +45,7 @@ class TaHDuoCache:
         self.batch_size: Optional[int] = None
         self.return_concat = return_concat
         self._rows: Dict[_Slot, int] = {}       # rows written per slot (pad rows included), the reference's length
+        self._meta_memo: Dict[Tuple[int, int, int], Tuple[int, torch.Tensor]] = {}  # folded positions / valid flags per slot
         self._kv_dropped: Dict[_Slot, bool] = {}  # K/V of the slot live in the slabs only
         self._device: Optional[torch.device] = None
         self._dtype: Optional[torch.dtype] = None
@@ -201,7 +202,15 @@ class TaHDuoCache:
         for d in range(upto_iter_idx + 1):
             ts = store.get((layer_idx, d), [])
             if len(ts) > 1 and all(t is not None for t in ts):
-                ts[:] = [torch.cat(ts, dim=-1)]  # fold the per-step pieces once, so a long generation stays cheap
+                # The per-step pieces are folded in a memo of their own (a long generation stays cheap: one
+                # concatenation of the folded part and the new pieces per call).  The lists themselves stay one
+                # entry per write: chunks() pairs them with the K/V chunks entry by entry.
+                key = (id(store), layer_idx, d)
+                n, folded = self._meta_memo.get(key, (0, None))
+                if n != len(ts):
+                    folded = torch.cat(([folded] if n else []) + ts[n:], dim=-1) if n < len(ts) else torch.cat(ts, dim=-1)
+                    self._meta_memo[key] = (len(ts), folded)
+                ts = [folded]
             parts += ts
         if not parts:
             return torch.empty((init_batch_size, 0), device=self.device, dtype=torch.long)
@@ -279,6 +288,7 @@ class TaHDuoCache:
             raise TahDuoError("cannot move a cache whose slabs are already allocated")
         mv = lambda t, with_dtype: t if t is None else t.to(**({"device": device} if device is not None else {}),
                                                             **({"dtype": dtype} if dtype is not None and with_dtype else {}))
+        self._meta_memo.clear()
         for store, with_dtype in ((self._k, True), (self._v, True), (self._pos, False), (self._valid, False)):
             for slot, ts in store.items():
                 store[slot] = [mv(t, with_dtype) for t in ts]

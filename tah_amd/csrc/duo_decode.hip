@@ -784,6 +784,9 @@ __global__ __launch_bounds__(kWholeThreads) void duo_decode_step_kernel(const St
         *reinterpret_cast<u32x4*>(ap.cv + drow * ap.cv_rs + (int64_t)hk * ap.cv_hs + 8 * dc) = sub.v;
         if (dc == 0 && hk == 0) {
             if (ap.cpos && pp.a.pos_new) ap.cpos[(int64_t)aslot * ap.capacity + dst] = pos_new;
+            // (only this workgroup touches the length of the segment the row appends to)  A row placed anywhere but
+            // at the end of its slab leaves a gap of stale rows or overwrites cached ones: reported, not repaired.
+            if (ap.len[aslot] != dst && pp.a.overflow) *pp.a.overflow = 2;
             ap.len[aslot] = dst + 1;
         }
     }

@@ -80,6 +80,7 @@ struct GreedyParams {
     int64_t* out_tokens;
     int64_t out_stride;
     const int64_t* step_idx;
+    int32_t out_cols;
     int32_t* out_len;
     unsigned long long *n_hard, *n_steps;
 };
@@ -160,8 +161,11 @@ __global__ __launch_bounds__(kGreedyThreads) void greedy_step_kernel(const Greed
     // which is not part of its output; rows that have ended write zeros
     bool done = !active;
     if (active && p.eos >= 0 && nxt == p.eos) done = true;
+    const int64_t column = p.step_idx[0];
+    const bool room = column >= 0 && column < p.out_cols;  // a step beyond the buffer ends the row instead of writing
+    if (!room) done = true;
     p.finished[row] = done ? 1 : 0;
-    p.out_tokens[(int64_t)row * p.out_stride + p.step_idx[0]] = done ? 0 : nxt;
+    if (room) p.out_tokens[(int64_t)row * p.out_stride + column] = done ? 0 : nxt;
     if (!done) p.out_len[row] += 1;
     if (active) {
         p.pos[row] += 1;
@@ -324,7 +328,7 @@ __global__ __launch_bounds__(64) void decider_tail_kernel(const DeciderTailParam
 extern "C" int tah_greedy_step(const tah_greedy_step_args* a, tah_stream_t stream) {
     using namespace tah;
     if (!a) return TAH_E_NULL;
-    if (a->rows < 0 || a->vocab <= 0 || a->rows > 65535) return TAH_E_SHAPE;
+    if (a->rows < 0 || a->vocab <= 0 || a->rows > 65535 || a->out_cols < 0 || a->out_cols > a->out_stride) return TAH_E_SHAPE;
     if (a->rows == 0) return TAH_OK;
     if (!a->logits0 || !a->tok || !a->finished || !a->pos || !a->out_tokens || !a->step_idx || !a->out_len || !a->n_hard || !a->n_steps)
         return TAH_E_NULL;
@@ -340,6 +344,7 @@ extern "C" int tah_greedy_step(const tah_greedy_step_args* a, tah_stream_t strea
     p.vocab = a->vocab; p.eos = a->eos;
     p.tok = a->tok; p.finished = a->finished; p.pos = a->pos;
     p.out_tokens = a->out_tokens; p.out_stride = a->out_stride; p.step_idx = a->step_idx; p.out_len = a->out_len;
+    p.out_cols = a->out_cols;
     p.n_hard = reinterpret_cast<unsigned long long*>(a->n_hard);
     p.n_steps = reinterpret_cast<unsigned long long*>(a->n_steps);
     hipLaunchKernelGGL(greedy_step_kernel, dim3(a->rows), dim3(kGreedyThreads), 0, static_cast<hipStream_t>(stream), p);

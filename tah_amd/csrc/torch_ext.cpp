@@ -699,6 +699,7 @@ void greedy_step(const Tensor& logits0, const optional<Tensor>& logits1, const o
     a.tok = static_cast<int64_t*>(tok.data_ptr()); a.finished = static_cast<uint8_t*>(finished.data_ptr());
     a.pos = static_cast<int32_t*>(pos.data_ptr()); a.out_tokens = static_cast<int64_t*>(out_tokens.data_ptr());
     a.out_stride = out_tokens.stride(0); a.step_idx = static_cast<const int64_t*>(step_idx.data_ptr());
+    a.out_cols = (int32_t)out_tokens.size(1);
     a.out_len = static_cast<int32_t*>(out_len.data_ptr());
     a.n_hard = static_cast<int64_t*>(n_hard.data_ptr()); a.n_steps = static_cast<int64_t*>(n_steps.data_ptr());
     check_rc(g.greedy_step(&a, d.stream()), "tah_greedy_step");

@@ -744,9 +744,15 @@ class TaHDecodeEngine:
                         finished=self.finished, pos=self.pos, out_tokens=self.out_tokens, out_len=self.out_len,
                         hard_len=self.hard_len, n_hard=self.n_hard, n_steps=self.n_steps, chosen=chosen)
 
+    def _launch_switches(self):
+        """Every attribute that changes which kernels a captured step launches: part of both graph keys, so that
+        flipping one between two generate() calls on the same prefill captures again instead of replaying a graph
+        of the old path."""
+        return (self.use_fused_glue, self.fused_greedy, self.static_scratch, self.measure_without_attention, id(self.decider))
+
     def capture_ticks(self, eos: int, limit: int, temperature: float = 0.0, **filters):
         """The tick as two HIP graphs, one per logits buffer, after a warm-up tick whose state changes are undone."""
-        key = (eos, limit, self.w.threshold, temperature, tuple(sorted(filters.items())))
+        key = (eos, limit, self.w.threshold, temperature, tuple(sorted(filters.items()))) + self._launch_switches()
         if self._tick_graphs is not None and self._tick_key == key:
             return self._tick_graphs
         state = [t.clone() for t in self._state()]
@@ -814,7 +820,7 @@ class TaHDecodeEngine:
     def capture(self, temperature: float = 0.0, eos: int = -1, **filters):
         """Captures one generation step in a HIP graph (after a warm-up step run on a side stream whose state
         changes are undone, so that library workspaces exist before the capture)."""
-        key = (temperature, eos, tuple(sorted(filters.items())), self.measure_without_attention)
+        key = (temperature, eos, tuple(sorted(filters.items()))) + self._launch_switches()
         if self._graph is not None and self._graph_key == key:
             return self._graph
         state = [t.clone() for t in self._state()]

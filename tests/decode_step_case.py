@@ -84,6 +84,15 @@ def run(dev, *, B, hq, hkv, seed=0, max_len=90, hidden=256, cap1=128, cap2=64, f
         assert torch.equal(tgt_a.len.cpu(), src.len.cpu() + grew)  # the step did append
         assert oa[B // 3].abs().max() == 0                                              # the finished row saw nothing
         results[depth] = oa
+    if not full_slab:  # a row told to append below its slab's end: the step reports it (flag value 2)
+        a1, a2 = copy.deepcopy(c1), copy.deepcopy(c2)
+        at = a1.len.clone()
+        victim = next(b for b in range(B) if bool(active[b]) and lens1[b] >= 2)
+        at[victim] -= 1
+        kv_cache.decode_step(q, k, v, qw, kw, cos, sin, 1e-6, append_at=at, q_slot=rows, q_pos=torch.where(active, pos, minus1),
+                             c1=a1, c2=a2, scale=scale, q_depth=torch.zeros(B, dtype=torch.int32, device=dev), cache=a1, cu_new=cu,
+                             slot_of=torch.where(active, rows, minus1), pos_new=None, norm_input=x, norm_eps=1e-6)
+        assert int(a1.overflow) == 2 and int(a1.len[victim]) == lens1[victim]
     return results
 
 

@@ -114,6 +114,17 @@ def test_argument_checks_run_before_any_device_work():
         g.do_row_stride = g.dq_row_stride = g.dk_row_stride = g.dv_row_stride = 1024
         g.do_head_stride = g.dq_head_stride = g.dk_head_stride = g.dv_head_stride = 128
     assert lib.tah_duo_bwd_varlen(ctypes.byref(b), None) == _capi.TAH_E_SHAPE
+    # the dS workspace: refused when misaligned or smaller than the size function says (before any launch)
+    b.fwd.s1.v_row_stride = 1024
+    b.fwd.s2.cu_q = b.fwd.s2.cu_k = 0x30000
+    need = lib.tah_duo_bwd_workspace_bytes(1, 8, 8, 64, 64, 0, 0, 0, 0)
+    assert need == 2 * 8 * 1 * 16384  # (64 / 64 + 1) query slots x 8 heads x one 128-key slot x 16 KiB
+    assert lib.tah_duo_bwd_workspace_bytes(1, 8, 8, 64, 4096, 0, 0, 300, 0) == 2 * 8 * 3 * 16384  # bounded by max_seqlen_k
+    assert lib.tah_duo_bwd_workspace_bytes(1, 8, 1, 64, 64, 0, 0, 0, 0) == 0                         # 8 query heads per kv head
+    b.ds_workspace, b.ds_workspace_bytes = 0x60008, need
+    assert lib.tah_duo_bwd_varlen(ctypes.byref(b), None) == _capi.TAH_E_ALIGN
+    b.ds_workspace, b.ds_workspace_bytes = 0x60000, need - 1
+    assert lib.tah_duo_bwd_varlen(ctypes.byref(b), None) == _capi.TAH_E_WORKSPACE
 
 
 def test_topk_mix_argument_checks():

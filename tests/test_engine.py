@@ -66,6 +66,13 @@ def _greedy_step_case(device, rows=6, vocab=200, seed=0):
     st["tok"] = nxt
     for k in st:
         assert torch.equal(dev[k].cpu(), st[k]), k
+    # a step beyond the last column of out_tokens (a captured step replayed too often) stores nothing and ends the rows
+    dev["step_idx"].fill_(4)
+    before = dev["out_tokens"].clone()
+    ops.greedy_step(l0p.to(device)[:, :vocab], None, None, -1, dev["tok"], dev["finished"], dev["pos"],
+                    dev["out_tokens"], dev["step_idx"], dev["out_len"], dev["n_hard"], dev["n_steps"])
+    assert torch.equal(dev["out_tokens"], before) and bool(dev["finished"].all())
+    assert torch.equal(dev["out_len"].cpu(), st["out_len"])
 
 
 @pytest.mark.skipif(not emu_util.have_host_clang(), reason="host clang++ not available")

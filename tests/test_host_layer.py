@@ -384,3 +384,30 @@ def test_reorder_cache_chunks_only():
     K, V = c.get_cache_upto_iter(0, 0)
     assert torch.equal(K, k[beam]) and torch.equal(V, v[beam])
     assert torch.equal(c.get_position_id_upto_iter(0, 0), pos)
+
+
+def test_metadata_getters_leave_the_chunk_lists_alone():
+    """The getters fold positions / valid flags of many writes in a memo of their own; the per-write lists that
+    chunks() pairs with the K/V chunks keep one entry per write, before and after (and between) getter calls."""
+    from tah_amd.attention import _Packed
+    from tah_amd.cache import TaHDuoCache
+    from tah_amd import TahDuoError
+    cache = TaHDuoCache()
+    B, H, D = 2, 2, 8
+    widths = [4, 1, 3]
+    for i, T in enumerate(widths):
+        cache.current_iter_depth = 0
+        cache.position_ids_to_cache = torch.arange(T).repeat(B, 1) + 10 * i
+        cache.valid_mask_to_cache = torch.ones(B, T, dtype=torch.long)
+        cache.update(torch.randn(B, H, T, D), torch.randn(B, H, T, D), 0)
+        pos = cache.get_position_id_upto_iter(0, 0)
+        assert pos.shape == (B, sum(widths[: i + 1]))
+        assert cache.get_valid_mask_upto_iter(0, 0).shape == pos.shape
+    want = torch.cat([torch.arange(T).repeat(B, 1) + 10 * i for i, T in enumerate(widths)], dim=-1)
+    assert torch.equal(cache.get_position_id_upto_iter(0, 0), want)
+    ch = cache.chunks(0, 0)
+    assert len(ch) == len(widths)
+    for (k, v, pos, valid), T in zip(ch, widths):
+        assert k.shape[-2] == v.shape[-2] == pos.shape[-1] == valid.shape[-1] == T
+    with pytest.raises(TahDuoError):  # a valid mask of another width than the block it is said to describe
+        _Packed(torch.ones(B, 5, dtype=torch.long), None, B, 4, torch.device("cpu"))
