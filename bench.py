@@ -23,16 +23,20 @@ if ROOT not in sys.path:
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, vendor figure
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a plain copy of
-# known size (profiles/*_counters.md); valid for the default workloads only.
-TRAFFIC_FWD_BYTES = 203.3e6 + 72.2e6
-TRAFFIC_DECODE_BYTES = 2.329e9 + 5.1e6 + 5.2e6 + 0.3e6
-TRAFFIC_QK_PREP_BYTES = 142.7e6 + 134.2e6
-TRAFFIC_TOPK_MIX_BYTES = 729.3e6 + 8.4e6  # (profiles/topk_mix_kernel_1024_rows_counters.md)
-# forward + backward legs, all kernels of one step (forward, two delta kernels, dQ, dK/dV): bytes fetched + written
-# (profiles/duo_fwd_bwd_seq8192_and_4docs_counters.md)
-TRAFFIC_FWD_BWD_SEQ8192_BYTES = 610.5e6 + 113.2e6
-TRAFFIC_FWD_BWD_4DOCS_BYTES = 439.6e6 + 116.9e6
+
+
+def measured_traffic(leg: str):
+    """HBM bytes per launch (per step for the forward+backward legs) of a default workload, as the rocprofv3 --pmc
+    FETCH_SIZE / WRITE_SIZE runs measured them: profiles/traffic.json holds the figures (fetched + written, each
+    scaled by what the same counter reads for a plain copy of known size) next to the summary file they come from.
+    None for a leg the file does not list."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            entry = json.load(f)["legs"].get(leg)
+    except (OSError, ValueError, KeyError):
+        return None
+    return None if entry is None else float(entry["fetch_bytes"]) + float(entry["write_bytes"])
+
 
 
 def visible_pairs(case):
@@ -69,12 +73,49 @@ def cpu_baseline(seed: int, T: int, p: float, reps: int = 3):
             O.duo_prefill_dense(c0["q1"], c0["k1"], c0["v1"], c0["q2"], c0["k2"], c0["v2"], c0["hard"], c0["scale"])
             t0s.append(time.perf_counter() - t0)
     tc0 = sorted(t0s[1:])[5]
+    # configs[2], the reference's way: per sequence one Tq = 1 SDPA call over the repeated-head cache with a
+    # (1, 1, 1, L) additive mask, fp32; sample: the first 8 of the 64 sequences (same seeded context lengths)
+    g = torch.Generator().manual_seed(1236)
+    lens = torch.randint(1024, 16385, (64,), generator=g).tolist()[:8]
+    dec_in = [(torch.randn(1, 16, 1, 128, generator=g), torch.randn(1, 8, L, 128, generator=g), torch.randn(1, 8, L, 128, generator=g),
+               torch.zeros(1, 1, 1, L)) for L in lens]
+    tds = []
+    with torch.no_grad():
+        for _ in range(4):
+            t0 = time.perf_counter()
+            for q, k, v, m in dec_in:
+                O.sdpa_dense(q, k, v, m, 128 ** -0.5)
+            tds.append(time.perf_counter() - t0)
+    td = sorted(tds[1:])[1]
+    dec_bytes = sum(lens) * 2 * 8 * 128 * 2  # the bytes the metric counts for these rows (bf16 K and V)
+    del dec_in
+    # configs[3], down-scaled: one document of 1024 tokens (the shortest of the four), p = 0.10, forward + backward
+    # through torch autograd over the same dense formulation
+    c3 = make_dense_case(1237, B=1, T=1024, p_hard=0.10)
+    f3 = 3.5 * 4.0 * 128 * 16 * visible_pairs(dense_to_varlen(c3))
+    leaves = {k: (c3[k] * 0.5).requires_grad_(True) for k in ("q1", "k1", "v1", "q2", "k2", "v2")}
+    t3s = []
+    for _ in range(4):
+        t0 = time.perf_counter()
+        o1, o2, _ = O.duo_prefill_dense(leaves["q1"], leaves["k1"], leaves["v1"], leaves["q2"], leaves["k2"], leaves["v2"],
+                                        c3["hard"], c3["scale"])
+        (o1.sum() + o2.sum()).backward()
+        t3s.append(time.perf_counter() - t0)
+        for t_ in leaves.values():
+            t_.grad = None
+    t3 = sorted(t3s[1:])[1]
     return {
         "value": flops / t / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
         "sample": f"1 of 4 sequences (B=1, T={T}, p={p}), fp32 dense mask + SDPA restatement, median of {reps}, "
                   f"{t * 1e3:.1f} ms, os.cpu_count()={os.cpu_count()}",
         "configs0": {"workload": "configs[0]: B=1, T=512, Hq=16, Hkv=8, D=128, fp32, p_hard=0.06, as stated",
                      "ms": tc0 * 1e3, "tflops": f0 / tc0 / 1e12, "flop": f0, "median_of": 10},
+        "decode": {"workload": "configs[2] as the reference runs it: one Tq=1 SDPA per sequence (repeat_kv + additive mask), fp32",
+                   "sample": f"8 of the 64 sequences (context lengths {lens}): 1/8 of the step's sequences, depth-0 queries only",
+                   "ms": td * 1e3, "gbs_of_the_metrics_bytes": dec_bytes / td / 1e9, "median_of": 3},
+        "configs3": {"workload": "configs[3] down-scaled: forward + backward (torch autograd) over the dense formulation, fp32",
+                     "sample": "one document of 1024 tokens, p_hard=0.10: 1/8 of the tokens, about 1/40 of the step's visible pairs",
+                     "ms": t3 * 1e3, "tflops": f3 / t3 / 1e12, "flop": f3, "median_of": 3},
     }
 
 
@@ -119,7 +160,7 @@ def bench_decode(steps: int, warmup: int):
                         "(three copies of the cache read in rotation)",
             "ms_per_step": ms, "visible_rows": rows, "algorithmic_bytes": nbytes, "hbm_gbs": gbs,
             "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
-                         "traffic": TRAFFIC_DECODE_BYTES, "kernels": "duo_decode_split_kernel<2> + duo_decode_merge_kernel"},
+                         "traffic": measured_traffic("decode"), "kernels": "duo_decode_split_kernel<2> + duo_decode_merge_kernel"},
             "tokens_per_s": nseq / (ms * 1e-3)}
 
 
@@ -160,28 +201,34 @@ def bench_fwd_bwd(name: str, seqlens, p_hard: float, seed: int, steps: int, warm
     pairs = visible_pairs(case)
     fwd_flops = 4.0 * 128 * 16 * pairs
     sched = launch_order(ops, dev)
+    mk = max(seqlens)  # what a caller knows of the batch: no sequence is longer (sizes the backward's dS workspace)
+    ws_bytes = ops.duo_bwd_workspace_bytes(len(seqlens), 16, 8, dev["q1"].shape[0], dev["k1"].shape[0], dev["q2"].shape[0],
+                                           dev["k2"].shape[0], mk, mk)
+
+    def bwd(o1, lse1, o2, lse2, schedule, ds_workspace=None):
+        return ops.duo_bwd_varlen(dev["q1"], dev["k1"], dev["v1"], o1, lse1, do1, dev["cu_q1"], dev["cu_k1"],
+                                  dev["q2"], dev["k2"], dev["v2"], o2, lse2, do2, dev["pos_q2"], dev["pos_k2"],
+                                  dev["cu_q2"], dev["cu_k2"], dev["scale"], schedule=schedule, ds_workspace=ds_workspace,
+                                  max_seqlen_k1=mk, max_seqlen_k2=mk)
+
+    bwd(*ops.duo_fwd_varlen(*a, schedule=sched), sched)  # (allocates the package's dS workspace outside the timed steps)
     yield  # inputs are resident; everything below runs when main() resumes the leg
-    def in_sequence_order():  # the same step with the tiles in sequence order (no table), for comparison
+    def other_way(schedule, ds_workspace):  # the same step in sequence order (no table) / with the three-kernel backward
         t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         for i in range(warmup + steps):
             if i == warmup:
                 t0.record()
-            o1, lse1, o2, lse2 = ops.duo_fwd_varlen(*a)
-            ops.duo_bwd_varlen(dev["q1"], dev["k1"], dev["v1"], o1, lse1, do1, dev["cu_q1"], dev["cu_k1"],
-                               dev["q2"], dev["k2"], dev["v2"], o2, lse2, do2, dev["pos_q2"], dev["pos_k2"],
-                               dev["cu_q2"], dev["cu_k2"], dev["scale"])
+            bwd(*ops.duo_fwd_varlen(*a, schedule=schedule), schedule, ds_workspace)
         t1.record()
         torch.cuda.synchronize()
         return t0.elapsed_time(t1) / steps
+    in_sequence_order = lambda: other_way(None, None)
 
     if sched is not None:
         in_sequence_order()  # (measured again after the timed steps, so that neither order runs on a colder GPU)
 
     def step():
-        o1, lse1, o2, lse2 = ops.duo_fwd_varlen(*a, schedule=sched)
-        ops.duo_bwd_varlen(dev["q1"], dev["k1"], dev["v1"], o1, lse1, do1, dev["cu_q1"], dev["cu_k1"],
-                           dev["q2"], dev["k2"], dev["v2"], o2, lse2, do2, dev["pos_q2"], dev["pos_k2"],
-                           dev["cu_q2"], dev["cu_k2"], dev["scale"], schedule=sched)
+        bwd(*ops.duo_fwd_varlen(*a, schedule=sched), sched)
 
     for _ in range(warmup):
         step()
@@ -201,27 +248,118 @@ def bench_fwd_bwd(name: str, seqlens, p_hard: float, seed: int, steps: int, warm
         ev[0].record()
         ops.duo_fwd_varlen(*a, schedule=sched)
         ev[1].record()
-        ops.duo_bwd_varlen(dev["q1"], dev["k1"], dev["v1"], o1, lse1, do1, dev["cu_q1"], dev["cu_k1"],
-                           dev["q2"], dev["k2"], dev["v2"], o2, lse2, do2, dev["pos_q2"], dev["pos_k2"],
-                           dev["cu_q2"], dev["cu_k2"], dev["scale"], schedule=sched)
+        bwd(o1, lse1, o2, lse2, sched)
         ev[2].record()
         torch.cuda.synchronize()
         half["fwd"] += ev[0].elapsed_time(ev[1]) / steps
         half["bwd"] += ev[1].elapsed_time(ev[2]) / steps
     tf = 3.5 * fwd_flops / (ms * 1e-3) / 1e12
+    ms_three = other_way(sched, False)
     order = None
     if sched is not None:  # what one table costs to build (once per batch)
         order = {"table": "heaviest tile first across documents, built once per batch outside the timed region",
                  "table_build_ms": time_schedule_build(ops, dev), "ms_per_step_in_sequence_order": in_sequence_order()}
     return {"workload": name, "ms_per_step": ms, "launch_order": order, "visible_pairs_per_head": pairs, "flop_per_step": 3.5 * fwd_flops,
+            "backward": {"path": "dS exchange: dK/dV kernel writes dS (bf16), dQ = scale * dS K reads it back (5 products per "
+                                 "tile pair)", "ds_workspace_bytes": ws_bytes,
+                         "ms_per_step_with_three_kernel_backward": ms_three,
+                         "three_kernel_backward": "dQ and dK/dV each recompute S and dP (7 products per tile pair), no workspace"},
             "tflops": tf, "roofline": {"bound": "mfma", "achieved": tf, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                                        "frac": tf / PEAK_BF16_TFLOPS, "traffic": traffic,
-                                       "kernels": "duo_fwd_kernel + duo_bwd_delta/dq/dkdv kernels",
+                                       "kernels": "duo_fwd_kernel + duo_bwd_delta_kernel x2 + duo_bwd_dkdv_kernel (dS export) + "
+                                                  "duo_bwd_dq_from_ds_kernel",
                                        "kernel_ms": {"forward (duo_fwd_kernel)": half["fwd"],
-                                                     "backward (delta x2, dq, dkdv)": half["bwd"]},
+                                                     "backward (delta x2, dkdv + dS export, dq from dS)": half["bwd"]},
                                        "frac_forward": fwd_flops / (half["fwd"] * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
                                        "frac_backward": 2.5 * fwd_flops / (half["bwd"] * 1e-3) / 1e12 / PEAK_BF16_TFLOPS},
             "tokens_per_s": sum(seqlens) / (ms * 1e-3)}
+
+
+def bench_host_layer_train_step(seqlens, p_hard: float, seed: int, steps: int, warmup: int, layers: int = 4):
+    """The path a maintainer of the reference runs in training (tah_model.py:580-623 around HF attention layers): per
+    decoder layer and latent iteration `build_attention_mask` (once per iteration) -> `TaHDuoCache.update` ->
+    `duo_attention_forward`, both iterations, then `.backward()`, on configs[3]'s documents as a batch of padded rows
+    with a valid mask -- against the bare packed-varlen launches (`ops.duo_fwd_varlen` + `ops.duo_bwd_varlen`) of the
+    same rows."""
+    import types
+
+    import torch
+
+    from tah_amd import ops
+    from tah_amd.attention import build_attention_mask, duo_attention_forward
+    from tah_amd.cache import TaHDuoCache
+    from tah_amd.pack import gather_active
+    from tests.cases import make_varlen_case, varlen_args
+    from tests.gpu_util import to_device
+
+    B, T, Hq, Hkv, D = len(seqlens), max(seqlens), 16, 8, 128
+    g = torch.Generator().manual_seed(seed)
+    valid = torch.zeros(B, T, dtype=torch.long)
+    for b, n in enumerate(seqlens):
+        valid[b, :n] = 1  # right-padded rows
+    hard = (torch.rand(B, T, generator=g) < p_hard) & valid.bool()
+    mk = lambda h: [(torch.randn(B, T, h, D, generator=g) * 0.5).to(torch.bfloat16).cuda().requires_grad_(True) for _ in range(layers)]
+    q1, k1, v1, q2, k2, v2 = mk(Hq), mk(Hkv), mk(Hkv), mk(Hq), mk(Hkv), mk(Hkv)
+    valid, hard = valid.cuda(), hard.cuda()
+    pos = (torch.cumsum(valid, -1) - 1).clamp(min=0)
+    w1 = torch.randn(B, T, Hq, D, generator=g).to(torch.bfloat16).cuda()
+    mods = [types.SimpleNamespace(layer_idx=l, num_key_value_groups=Hq // Hkv) for l in range(layers)]
+    scale = D ** -0.5
+    # the bare launches on the same rows, packed (one call serves both iterations)
+    case = make_varlen_case(seed, list(seqlens), p_hard, std=0.5)
+    dev = to_device(case)
+    a = varlen_args(dev)
+    do1 = torch.randn(dev["q1"].shape, generator=g).to(torch.bfloat16).cuda()
+    do2 = torch.randn(dev["q2"].shape, generator=g).to(torch.bfloat16).cuda()
+    sched = launch_order(ops, dev)
+    yield
+
+    def host_step():
+        cache = TaHDuoCache()
+        m0 = build_attention_mask(pos, valid, cache, 0, dtype=torch.bfloat16)
+        cache.current_iter_depth, cache.position_ids_to_cache, cache.valid_mask_to_cache = 0, pos, valid
+        outs = []
+        for l in range(layers):
+            k, v = cache.update(k1[l].transpose(1, 2), v1[l].transpose(1, 2), l)
+            outs.append(duo_attention_forward(mods[l], q1[l].transpose(1, 2), k, v, m0, scaling=scale)[0])
+        # second iteration: the hard tokens, packed per row (one index for all layers, as the model's loop has it)
+        packed = gather_active(hard, pos, valid, *q2, *k2, *v2)
+        pos2, val2 = packed[1], packed[2]
+        gq, gk, gv = packed[3:3 + layers], packed[3 + layers:3 + 2 * layers], packed[3 + 2 * layers:]
+        m1 = build_attention_mask(pos2, val2, cache, 1, dtype=torch.bfloat16)
+        cache.current_iter_depth, cache.position_ids_to_cache, cache.valid_mask_to_cache = 1, pos2, val2
+        for l in range(layers):
+            k, v = cache.update(gk[l].transpose(1, 2), gv[l].transpose(1, 2), l)
+            outs.append(duo_attention_forward(mods[l], gq[l].transpose(1, 2), k, v, m1, scaling=scale)[0])
+        torch.autograd.backward(outs, [w1[:, : o.shape[1]] for o in outs])  # upstream gradients as given (no loss arithmetic)
+        for t in q1 + k1 + v1 + q2 + k2 + v2:
+            t.grad = None
+
+    def bare_step():
+        for _ in range(layers):
+            o1, lse1, o2, lse2 = ops.duo_fwd_varlen(*a, schedule=sched)
+            ops.duo_bwd_varlen(dev["q1"], dev["k1"], dev["v1"], o1, lse1, do1, dev["cu_q1"], dev["cu_k1"],
+                               dev["q2"], dev["k2"], dev["v2"], o2, lse2, do2, dev["pos_q2"], dev["pos_k2"],
+                               dev["cu_q2"], dev["cu_k2"], dev["scale"], schedule=sched, max_seqlen_k1=T, max_seqlen_k2=T)
+
+    def timed(f):
+        for _ in range(max(2, warmup // 2)):
+            f()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            f()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps
+
+    host_ms, bare_ms = timed(host_step), timed(bare_step)
+    return {"workload": f"configs[3] as the host layer sees it: {B} rows padded to {T}, valid lengths {list(seqlens)}, "
+                        f"p_hard={p_hard}, {layers} attention layers x 2 latent iterations, forward + backward",
+            "path": "build_attention_mask -> TaHDuoCache.update -> duo_attention_forward (both iterations) -> loss.backward(); "
+                    "wall clock, includes the packing of valid / hard rows and autograd's own kernels",
+            "ms_per_step": host_ms, "ms_per_layer": host_ms / layers,
+            "bare_launches_ms_per_step": bare_ms, "bare_launches_ms_per_layer": bare_ms / layers,
+            "ratio_to_bare_launches": host_ms / bare_ms, "layers": layers}
 
 
 def bench_qk_prep(steps: int, warmup: int):
@@ -266,7 +404,7 @@ def bench_qk_prep(steps: int, warmup: int):
                         "Hq=16, Hkv=8, D=128 (fresh slabs every step)",
             "ms_per_step": ms, "algorithmic_bytes": nbytes, "hbm_gbs": gbs,
             "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
-                         "traffic": TRAFFIC_QK_PREP_BYTES, "kernels": "qk_prep_kernel + kv_append_len_kernel"},
+                         "traffic": measured_traffic("qk_prep_prefill"), "kernels": "qk_prep_kernel + kv_append_len_kernel"},
             "tokens_per_s": rows / (ms * 1e-3)}
 
 
@@ -305,7 +443,7 @@ def bench_topk_mix(steps: int, warmup: int, rows: int = 1024, vocab: int = 15193
                         "(two sets of logits in rotation)",
             "ms_per_step": mix_ms, "algorithmic_bytes": nbytes, "hbm_gbs": gbs,
             "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
-                         "traffic": TRAFFIC_TOPK_MIX_BYTES if (rows, vocab, hidden, topk) == (1024, 151936, 2048, 100) else None,
+                         "traffic": measured_traffic("topk_mix") if (rows, vocab, hidden, topk) == (1024, 151936, 2048, 100) else None,
                          "kernels": "topk_mix_kernel<19>"},
             "topk_values_ms": val_ms, "torch_topk_ms": torch_ms, "rows_per_s": rows / (mix_ms * 1e-3)}
 
@@ -415,7 +553,7 @@ def main() -> int:
     ap.add_argument("--spinup", type=int, default=200,
                     help="untimed launches of the headline kernel before its warm-up steps (the GPU's clock needs tens of "
                          "milliseconds of work to leave its idle state)")
-    ap.add_argument("--only", choices=["all", "fwd", "decode", "fwd_bwd", "qk_prep", "topk_mix", "e2e"], default="all",
+    ap.add_argument("--only", choices=["all", "fwd", "decode", "fwd_bwd", "host_layer", "qk_prep", "topk_mix", "e2e"], default="all",
                     help="profiling aid: run only one leg (the JSON line then lacks the other legs)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="profiling aid: also run one plain 256 MiB device copy (known traffic for counter scaling)")
@@ -453,10 +591,13 @@ def main() -> int:
     if args.only in ("all", "fwd_bwd"):
         legs.append(("fwd_bwd_seq8192_p06", bench_fwd_bwd(
             "north-star headline: fwd+bwd, one sequence of 8192, p_hard=0.06, Hq=16, Hkv=8, D=128", [8192], 0.06, 1238,
-            args.steps, args.warmup, TRAFFIC_FWD_BWD_SEQ8192_BYTES)))
+            args.steps, args.warmup, measured_traffic("fwd_bwd_seq8192_p06"))))
         legs.append(("fwd_bwd_4docs_p10", bench_fwd_bwd(
             "configs[3]: fwd+bwd, 8192 packed tokens in 4 documents, p_hard=0.10", [1397, 3210, 2561, 1024], 0.10, 1237,
-            args.steps, args.warmup, TRAFFIC_FWD_BWD_4DOCS_BYTES)))
+            args.steps, args.warmup, measured_traffic("fwd_bwd_4docs_p10"))))
+    if args.only in ("all", "host_layer"):
+        legs.append(("host_layer_train_step", bench_host_layer_train_step([1397, 3210, 2561, 1024], 0.10, 1237,
+                                                                          max(3, args.steps // 4), args.warmup)))
     if args.only in ("all", "decode"):
         legs.append(("decode", bench_decode(args.steps, args.warmup)))
     if args.only in ("all", "qk_prep"):
@@ -496,8 +637,10 @@ def main() -> int:
     ev1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    ms = ev0.elapsed_time(ev1) / fwd_steps  # events on the stream the kernel is launched on
+    ms_wall = wall * 1e3 / fwd_steps           # the K timed steps between two synchronisations: `ms_per_step` and `value`
+    ms = ev0.elapsed_time(ev1) / fwd_steps    # the same launches by HIP events on their stream: the roofline's kernel time
     tflops = flops / (ms * 1e-3) / 1e12
+    value = flops / (ms_wall * 1e-3) / 1e12
     ms_sequence_order = in_sequence_order()
     sustained = None
     if args.only in ("all", "fwd"):
@@ -520,17 +663,21 @@ def main() -> int:
 
     out = {
         "metric": "duo-causal attn TFLOP/s (% bf16 MFMA peak) prefill; decode HBM GB/s",
-        "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": wall * 1e3 / fwd_steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_wall, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
+        "timing": {"value_and_ms_per_step": "wall clock of the timed steps between two device synchronisations",
+                   "roofline": "HIP events on the launch stream around the same steps (kernel_ms)",
+                   "untimed_launches_before_the_timed_steps": spinup + 2 * fwd_warmup + fwd_steps,
+                   "of_which": {"spinup": spinup, "warmup": fwd_warmup, "same_kernel_in_sequence_order": fwd_warmup + fwd_steps}},
         "config": {"workload": "configs[1]: duo-causal prefill forward, B=4, T=4096, Hq=16, Hkv=8, D=128, p_hard=0.06",
-                   "visible_pairs_per_head": pairs, "flop_per_step": flops, "tokens_per_s": B * T / (ms * 1e-3),
+                   "visible_pairs_per_head": pairs, "flop_per_step": flops, "tokens_per_s": B * T / (ms_wall * 1e-3),
                    "launch_order": {"table": "heaviest tile first across the 4 sequences (tah_duo_schedule_build), built once "
                                              "per batch outside the timed region: one table serves all 28 layers",
                                     "table_build_ms": table_build_ms, "ms_per_step_in_sequence_order": ms_sequence_order},
                    "spinup_launches": spinup, "sustained": sustained},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_FWD_BYTES, "kernel": "duo_fwd_kernel<2>",
+                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": measured_traffic("prefill_fwd"), "kernel": "duo_fwd_kernel<2>",
                      "kernel_ms": ms},
     }
     out["extra"] = extra

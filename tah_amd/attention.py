@@ -34,12 +34,14 @@ from .pack import HardIndex
 
 class _DuoAttnVarlen(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, q1, k1, v1, q2, k2, v2, cu_q1, cu_k1, pos_q2, pos_k2, cu_q2, cu_k2, scale, schedule=None):
+    def forward(ctx, q1, k1, v1, q2, k2, v2, cu_q1, cu_k1, pos_q2, pos_k2, cu_q2, cu_k2, scale, schedule=None,
+                max_seqlen_k1=0, max_seqlen_k2=0):
         o1, lse1, o2, lse2 = ops.duo_fwd_varlen(q1, k1, v1, cu_q1, cu_k1, q2, k2, v2, pos_q2, pos_k2, cu_q2, cu_k2, scale,
                                                 schedule)
         ctx.save_for_backward(q1, k1, v1, o1, lse1, q2, k2, v2, o2, lse2, cu_q1, cu_k1, pos_q2, pos_k2, cu_q2, cu_k2)
         ctx.scale = scale
         ctx.schedule = schedule
+        ctx.max_k = (int(max_seqlen_k1), int(max_seqlen_k2))
         ctx.mark_non_differentiable(lse1, lse2)
         return o1, o2, lse1, lse2
 
@@ -49,12 +51,12 @@ class _DuoAttnVarlen(torch.autograd.Function):
         c = lambda g, like: (torch.zeros_like(like) if g is None else g.contiguous())
         dq1, dk1, dv1, dq2, dk2, dv2 = ops.duo_bwd_varlen(
             q1, k1, v1, o1, lse1, c(do1, o1), cu_q1, cu_k1, q2, k2, v2, o2, lse2, c(do2, o2),
-            pos_q2, pos_k2, cu_q2, cu_k2, ctx.scale, ctx.schedule)
-        return dq1, dk1, dv1, dq2, dk2, dv2, None, None, None, None, None, None, None, None
+            pos_q2, pos_k2, cu_q2, cu_k2, ctx.scale, ctx.schedule, max_seqlen_k1=ctx.max_k[0], max_seqlen_k2=ctx.max_k[1])
+        return dq1, dk1, dv1, dq2, dk2, dv2, None, None, None, None, None, None, None, None, None, None
 
 
 def duo_attn_varlen(q1, k1, v1, cu_q1, cu_k1, q2, k2, v2, pos_q2, pos_k2, cu_q2, cu_k2, scale: float,
-                    return_lse: bool = False, schedule=None):
+                    return_lse: bool = False, schedule=None, max_seqlen_k1: int = 0, max_seqlen_k2: int = 0):
     """Duo-causal attention on packed varlen bf16 tensors, differentiable.
 
     Depth-0 stream: q1 [T1q,Hq,D], k1/v1 [T1k,Hkv,D], cu_q1/cu_k1 int32 [nseq+1].
@@ -62,10 +64,12 @@ def duo_attn_varlen(q1, k1, v1, cu_q1, cu_k1, q2, k2, v2, pos_q2, pos_k2, cu_q2,
     pos_q2/pos_k2 and cu_q2/cu_k2.  Key (pos_k, depth_k) is visible to query
     (pos_q, depth_q) iff pos_k <= pos_q and depth_k <= depth_q.  ``schedule``: the launch-order table
     :func:`tah_amd.ops.duo_schedule` built for these boundaries (forward and backward use it), or None.
+    ``max_seqlen_k1`` / ``max_seqlen_k2``: upper bounds on one sequence's key rows per depth (0: unknown); they only
+    make the backward pass's dS workspace smaller (:func:`tah_amd.ops.duo_bwd_varlen`).
     Returns (o1, o2).
     """
     o1, o2, lse1, lse2 = _DuoAttnVarlen.apply(q1, k1, v1, q2, k2, v2, cu_q1, cu_k1, pos_q2, pos_k2, cu_q2, cu_k2,
-                                              float(scale), schedule)
+                                              float(scale), schedule, max_seqlen_k1, max_seqlen_k2)
     return (o1, o2, lse1, lse2) if return_lse else (o1, o2)
 
 
@@ -371,12 +375,14 @@ def duo_attention_forward(module, query: torch.Tensor, key: torch.Tensor, value:
         e_q = q[:0]
         e_k = k1[:0]
         sched = _schedule_of(m, (pq.cu, cu_k1, zc, zc, zi, Hq, Hkv, q.shape[0], k1.shape[0], 0))
-        o, _ = duo_attn_varlen(q, k1, v1, pq.cu, cu_k1, e_q, e_k, e_k, zi, zi, zc, zc, scale, schedule=sched)
+        o, _ = duo_attn_varlen(q, k1, v1, pq.cu, cu_k1, e_q, e_k, e_k, zi, zi, zc, zc, scale, schedule=sched,
+                               max_seqlen_k1=cache.get_cache_length(layer, 0))
     else:
         k2, v2, cu_k2, pos_k2 = _segment(cache, layer, 1, B, with_pos=True)
         e_q = q[:0]
         sched = _schedule_of(m, (zc, cu_k1, pq.cu, cu_k2, pq.pos, Hq, Hkv, 0, k1.shape[0], k2.shape[0]))
-        _, o = duo_attn_varlen(e_q, k1, v1, zc, cu_k1, q, k2, v2, pq.pos, pos_k2, pq.cu, cu_k2, scale, schedule=sched)
+        _, o = duo_attn_varlen(e_q, k1, v1, zc, cu_k1, q, k2, v2, pq.pos, pos_k2, pq.cu, cu_k2, scale, schedule=sched,
+                               max_seqlen_k1=cache.get_cache_length(layer, 0), max_seqlen_k2=cache.get_cache_length(layer, 1))
     return pq.unpack(o, Hq, D), None
 
 

@@ -20,7 +20,7 @@ class _Cache(O.OracleCache):
         return cache_position.shape[0] + self.get_seq_length(layer_idx), 0
 
 
-def _ref_forward(model, embed, cache, ids, valid, hard, topk, decide=None):
+def _ref_forward(model, embed, cache, ids, valid, hard, topk, decide=None, mix_from_bf16_logits=False):
     """tah_model.py:495-706 for max_iter = 2 with the decider's decisions given: returns final logits (B, T, V).
     ``decide(logits, stacked hidden states (B, T, L + 1, H))``, when given, is called as the loop calls its decider after
     the first iteration (tah_model.py:434-441, 636-642) and its result returned as well."""
@@ -40,7 +40,8 @@ def _ref_forward(model, embed, cache, ids, valid, hard, topk, decide=None):
     if cur.any():
         pad, a_cum, a_pos, a_valid = O.gather_active(cur, cum, pos, valid)
         k = min(topk, a_cum.shape[-1])
-        tv, ti = torch.topk(a_cum, k=k, dim=-1)
+        # (mix_from_bf16_logits: the first iteration's logits as a bf16 model holds them, for the top-k mix only)
+        tv, ti = torch.topk(a_cum.to(torch.bfloat16).float() if mix_from_bf16_logits else a_cum, k=k, dim=-1)
         a_x = torch.sum(torch.softmax(tv, -1).unsqueeze(-1) * embed[ti], dim=-2)  # tah_model.py:57-75
         m1 = O.build_attention_mask(a_pos, a_valid, cache, 1, torch.float32)
         cache.current_iter_depth, cache.position_ids_to_cache, cache.valid_mask_to_cache = 1, a_pos, a_valid
@@ -50,29 +51,41 @@ def _ref_forward(model, embed, cache, ids, valid, hard, topk, decide=None):
     return final if decide is None else (final, decided)
 
 
-def run(device, *, prompt=(9, 6, 12), steps=5, layers=2, seed=0, vocab=96, topk=100):
+def run(device, *, prompt=(9, 6, 12), steps=5, layers=2, seed=0, vocab=96, topk=100, hidden=256, hq=4, hkv=2,
+        intermediate=512, decider_hidden=32, ref_device="cpu", with_hard=False, p_hard=0.35):
+    """``ref_device``: where the float32 reference model and its dense logits live (the host by default; the
+    end-to-end workload's own shape -- 28 layers, hidden 2048, 151 936 tokens -- wants the device).  ``with_hard``: every
+    stage comes back as (engine logits, reference logits, which rows took the second iteration)."""
     pytest.importorskip("transformers.models.qwen3.modeling_qwen3")
     from transformers import Qwen3Config, Qwen3Model
 
     from tah_amd.engine import EngineConfig, TaHDecodeEngine, Weights
 
     torch.manual_seed(seed)
-    hf = Qwen3Config(hidden_size=256, num_attention_heads=4, num_key_value_heads=2, head_dim=128,
-                     num_hidden_layers=layers, intermediate_size=512, vocab_size=vocab, rope_theta=1e6,
+    hf = Qwen3Config(hidden_size=hidden, num_attention_heads=hq, num_key_value_heads=hkv, head_dim=128,
+                     num_hidden_layers=layers, intermediate_size=intermediate, vocab_size=vocab, rope_theta=1e6,
                      attention_dropout=0.0, rms_norm_eps=1e-6)
     hf._attn_implementation = "sdpa"
-    ref = Qwen3Model(hf).to(torch.bfloat16).float().eval()  # bf16-representable weights, float32 arithmetic
-    cfg = EngineConfig(hidden=256, layers=layers, hq=4, hkv=2, head_dim=128, intermediate=512, vocab=vocab,
-                       decider_hidden=32, topk=topk)
+    with torch.device(ref_device):
+        ref = Qwen3Model(hf)
+    inv_freq = ref.rotary_emb.inv_freq.clone()
+    ref = ref.to(torch.bfloat16).float().eval()  # bf16-representable weights, float32 arithmetic
+    # (the round trip also rounds the rotary frequencies, a float32 buffer of the module, to bf16: angles would then be
+    # off in proportion to the position -- 0.5 rad at position 480 -- which a short prompt hides and a long one does not)
+    ref.rotary_emb.inv_freq.copy_(inv_freq)
+    if hasattr(ref.rotary_emb, "original_inv_freq"):
+        ref.rotary_emb.original_inv_freq = inv_freq.clone()
+    cfg = EngineConfig(hidden=hidden, layers=layers, hq=hq, hkv=hkv, head_dim=128, intermediate=intermediate, vocab=vocab,
+                       decider_hidden=decider_hidden, topk=topk)
 
     class _LM:  # the pieces Weights.from_hf reads: tied output head
         model = ref
         lm_head = type("H", (), {"weight": ref.embed_tokens.weight})
     w = Weights.from_hf(_LM, cfg, device)
     g = torch.Generator().manual_seed(seed + 1)
-    w.dec_w1 = torch.randn(32, 256, generator=g).to(torch.bfloat16).to(device)
-    w.dec_b1 = torch.zeros(32, dtype=torch.bfloat16, device=device)
-    w.dec_w2 = torch.randn(1, 32, generator=g).to(torch.bfloat16).to(device)
+    w.dec_w1 = torch.randn(decider_hidden, hidden, generator=g).to(torch.bfloat16).to(device)
+    w.dec_b1 = torch.zeros(decider_hidden, dtype=torch.bfloat16, device=device)
+    w.dec_w2 = torch.randn(1, decider_hidden, generator=g).to(torch.bfloat16).to(device)
     w.dec_b2 = torch.zeros(1, dtype=torch.bfloat16, device=device)
 
     B, Tm = len(prompt), max(prompt)
@@ -81,30 +94,33 @@ def run(device, *, prompt=(9, 6, 12), steps=5, layers=2, seed=0, vocab=96, topk=
     valid = torch.zeros(B, Tm, dtype=torch.long)
     for b, n in enumerate(prompt):
         valid[b, Tm - n:] = 1  # left padding, as the reference batches prompts
-    hard = torch.rand(B, Tm + steps, generator=g) < 0.35
+    hard = torch.rand(B, Tm + steps, generator=g) < p_hard
     hard[:, Tm] = torch.tensor([True] + [False] * (B - 1))   # first decode step: one hard row, the rest pad rows
     hard[:, Tm + 1] = False                                  # second: nobody iterates
     hard[:, Tm + 2] = True                                   # third: every row does
     hard[0, Tm - 1] = True                                   # a prompt whose last token is hard
     embed = ref.embed_tokens.weight.detach()
+    rd = lambda t: t.to(ref_device)
 
     out = []
     with torch.no_grad():
         cache = _Cache()
-        want = _ref_forward(ref, embed, cache, ids[:, :Tm], valid, hard[:, :Tm], topk)[:, -1]
+        with torch.device(ref_device):  # (the oracle's helpers create their tensors on the default device)
+            want = _ref_forward(ref, embed, cache, rd(ids[:, :Tm]), rd(valid), rd(hard[:, :Tm]), topk)[:, -1].cpu()
         packed = torch.cat([ids[b, Tm - n:Tm] for b, n in enumerate(prompt)]).to(device)
         hard_packed = torch.cat([hard[b, Tm - n:Tm] for b, n in enumerate(prompt)]).to(device)
         cu = torch.tensor([0] + list(torch.tensor(prompt).cumsum(0)), dtype=torch.int32, device=device)
         got, _ = eng.prefill(packed, cu, force_hard=hard_packed)
-        out.append((got.cpu(), want))
-        one = torch.ones(B, 1, dtype=torch.long)
+        out.append((got.cpu(), want) + ((hard[:, Tm - 1].clone(),) if with_hard else ()))
+        one = rd(torch.ones(B, 1, dtype=torch.long))
         for s in range(steps):
             t = Tm + s
-            want = _ref_forward(ref, embed, cache, ids[:, t:t + 1], one, hard[:, t:t + 1], topk)[:, 0]
+            with torch.device(ref_device):
+                want = _ref_forward(ref, embed, cache, rd(ids[:, t:t + 1]), one, rd(hard[:, t:t + 1]), topk)[:, 0].cpu()
             got, h = eng.step_logits(ids[:, t].to(device), force_hard=hard[:, t].to(device))
             eng.pos += 1
             assert torch.equal(h.cpu(), hard[:, t])
-            out.append((got.cpu(), want))
+            out.append((got.cpu(), want) + ((hard[:, t].clone(),) if with_hard else ()))
     lens0 = [n + steps for n in prompt]
     assert all(sl.len.tolist() == lens0 for sl in eng.slabs0)
     n1 = [int(hard[b, Tm - n:].sum()) for b, n in enumerate(prompt)]
@@ -148,7 +164,10 @@ def run_with_decider(device, *, prompt=(9, 6, 12), steps=4, layers=3, seed=2, vo
                      num_hidden_layers=layers, intermediate_size=512, vocab_size=vocab, rope_theta=1e6,
                      attention_dropout=0.0, rms_norm_eps=1e-6)
     hf._attn_implementation = "sdpa"
-    ref = Qwen3Model(hf).to(torch.bfloat16).float().eval()
+    ref = Qwen3Model(hf)
+    inv_freq = ref.rotary_emb.inv_freq.clone()
+    ref = ref.to(torch.bfloat16).float().eval()
+    ref.rotary_emb.inv_freq.copy_(inv_freq)  # (a float32 buffer the round trip must not round, see run())
     cfg = EngineConfig(hidden=256, layers=layers, hq=4, hkv=2, head_dim=128, intermediate=512, vocab=vocab,
                        decider_hidden=32, topk=100)
 
@@ -172,7 +191,7 @@ def run_with_decider(device, *, prompt=(9, 6, 12), steps=4, layers=3, seed=2, vo
     valid = torch.zeros(B, Tm, dtype=torch.long)
     for b, n in enumerate(prompt):
         valid[b, Tm - n:] = 1
-    hard = torch.rand(B, Tm + steps, generator=g) < 0.35
+    hard = torch.rand(B, Tm + steps, generator=g) < p_hard
     embed = ref.embed_tokens.weight.detach()
     out = []
     with torch.no_grad():

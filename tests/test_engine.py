@@ -486,3 +486,54 @@ def test_engine_with_the_learned_decider_gpu():
     for r in runs[1:]:
         assert torch.equal(r[0], runs[0][0]) and r[1:] == runs[0][1:]
 
+
+
+@pytest.mark.gpu
+def test_engine_at_the_end_to_end_shape_gpu():
+    """The end-to-end workload's own shape (``EngineConfig()``: 28 layers, hidden 2048, 16 / 8 heads, 151 936 tokens;
+    32 prompts of 512 tokens), where the other engine tests use a model a hundred times smaller:
+    (a) greedy generation in captured ticks, in eager ticks and in the captured step-wise loop gives the same tokens,
+    lengths, hard counts and slab lengths;
+    (b) the prefill's and three decode steps' final logits (a step with a single hard row and pad rows, one with none, one
+    where every row iterates) against the reference's loop around a float32 transformers ``Qwen3Model`` with dense masks
+    and a concatenating cache, same tokens and hard decisions on both sides.  Rows that take one iteration: within 3e-2 of
+    the logits' range, the bound of the small-model tests (bf16 weights, activations and logits through 28 layers on one
+    side, float32 on the other).  Rows that take the second iteration get a loose bound (mean 6e-2, largest 0.4 of the
+    range): their input is a softmax over the top-100 first-iteration logits, which turns a logit difference of one bf16
+    step into a few per cent of weight, and 28 randomly initialised layers carry that on -- the float32 reference alone
+    moves by 0.3 (hidden 2048, two layers, range 12.8) when only its own logits are rounded to bf16 before the mix."""
+    from tah_amd.engine import EngineConfig, TaHDecodeEngine, Weights
+    from tests.engine_case import run
+    cfg = EngineConfig()
+    w = Weights.random_init(cfg, "cuda", seed=11)
+    B, T, new = 32, 512, 6
+    g = torch.Generator().manual_seed(12)
+    ids = torch.randint(0, cfg.vocab, (B * T,), generator=g).cuda()
+    cu = torch.arange(0, B * T + 1, T, dtype=torch.int32, device="cuda")
+    runs = []
+    for continuous, use_graph in ((False, True), (True, False), (True, True)):
+        eng = TaHDecodeEngine(w, B, T + new + 2, device="cuda")
+        assert eng.can_run_continuous
+        first, _ = eng.prefill(ids, cu, calibrate=0.25)
+        toks = eng.generate(first, new, continuous=continuous, use_graph=use_graph).clone()
+        runs.append((toks.cpu(), eng.out_len.cpu(), int(eng.n_hard), [sl.len.tolist() for sl in eng.slabs0 + eng.slabs1]))
+        del eng
+    assert 0 < runs[0][2] and (runs[0][1] == new).all()
+    for r in runs[1:]:
+        assert torch.equal(r[0], runs[0][0]) and torch.equal(r[1], runs[0][1]) and r[2] == runs[0][2] and r[3] == runs[0][3]
+    del w, runs
+    torch.cuda.empty_cache()
+    prompts = tuple([512] * 29 + [500, 384, 77])
+    plain, second = 0.0, (0.0, 0.0)
+    for got, want, hard in run("cuda", prompt=prompts, steps=3, layers=cfg.layers, seed=13, vocab=cfg.vocab, topk=cfg.topk, hidden=cfg.hidden,
+                               hq=cfg.hq, hkv=cfg.hkv, intermediate=cfg.intermediate, decider_hidden=cfg.decider_hidden, ref_device="cuda",
+                               with_hard=True):
+        rng = max(want.max().item() - want.min().item(), 1e-6)
+        d = (got.float() - want).abs()
+        if (~hard).any():
+            plain = max(plain, d[~hard].max().item() / rng)
+        if hard.any():
+            second = (max(second[0], d[hard].max().item() / rng), max(second[1], d[hard].mean().item() / rng))
+    print(f"end-to-end shape, error / logit range: rows with one iteration max {plain:.3e}; rows with two: max {second[0]:.3e}, "
+          f"mean {second[1]:.3e}", flush=True)
+    assert plain <= 3e-2 and second[0] <= 0.4 and second[1] <= 6e-2
