@@ -191,7 +191,7 @@ def run_with_decider(device, *, prompt=(9, 6, 12), steps=4, layers=3, seed=2, vo
     valid = torch.zeros(B, Tm, dtype=torch.long)
     for b, n in enumerate(prompt):
         valid[b, Tm - n:] = 1
-    hard = torch.rand(B, Tm + steps, generator=g) < p_hard
+    hard = torch.rand(B, Tm + steps, generator=g) < 0.35
     embed = ref.embed_tokens.weight.detach()
     out = []
     with torch.no_grad():
