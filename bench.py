@@ -362,6 +362,88 @@ def bench_host_layer_train_step(seqlens, p_hard: float, seed: int, steps: int, w
             "ratio_to_bare_launches": host_ms / bare_ms, "layers": layers}
 
 
+def device_clock():
+    """Shader clock the device reports right now (rocm-smi), or None where the tool is not there."""
+    import subprocess
+    try:
+        out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=20).stdout
+    except (OSError, subprocess.SubprocessError):
+        return None
+    for line in out.splitlines():
+        if "sclk" in line and "(" in line:
+            return line.split("(")[-1].split(")")[0]
+    return None
+
+
+def bench_device_context(steps: int):
+    """What the 2.5 PFLOP/s figure means on the device at hand.  The shader clock follows the power the work draws,
+    and that depends on the data: the same instruction stream runs faster on zeros than on random values.  This leg
+    times (a) the library's own bf16 GEMM (8192^3, torch.matmul: no softmax, no masks, nothing but the matrix pipe
+    and its operand traffic) and (b) the duo-causal forward and backward kernels of the headline shape, each on random
+    data and on zeros, and reads the clock the device reports while each of them runs."""
+    import threading
+
+    import torch
+
+    from tah_amd import ops
+    from tests.cases import make_varlen_case, varlen_args
+    from tests.gpu_util import to_device
+
+    dev = to_device(make_varlen_case(1238, [8192], 0.06, std=0.5))
+    g = torch.Generator().manual_seed(3)
+    do1 = torch.randn(dev["q1"].shape, generator=g).to(torch.bfloat16).cuda()
+    do2 = torch.randn(dev["q2"].shape, generator=g).to(torch.bfloat16).cuda()
+    zero = dict(dev)
+    for k in ("q1", "k1", "v1", "q2", "k2", "v2"):
+        zero[k] = torch.zeros_like(dev[k])
+    n = 8192
+    mats = {"random": (torch.randn(n, n, device="cuda").to(torch.bfloat16), torch.randn(n, n, device="cuda").to(torch.bfloat16)),
+            "zeros": (torch.zeros(n, n, device="cuda", dtype=torch.bfloat16), torch.zeros(n, n, device="cuda", dtype=torch.bfloat16))}
+    yield
+
+    def attention_calls(d, g1, g2):
+        a = varlen_args(d)
+        o1, lse1, o2, lse2 = ops.duo_fwd_varlen(*a)
+        return (lambda: ops.duo_fwd_varlen(*a),
+                lambda: ops.duo_bwd_varlen(d["q1"], d["k1"], d["v1"], o1, lse1, g1, d["cu_q1"], d["cu_k1"], d["q2"], d["k2"], d["v2"], o2,
+                                           lse2, g2, d["pos_q2"], d["pos_k2"], d["cu_q2"], d["cu_k2"], d["scale"], max_seqlen_k1=8192,
+                                           max_seqlen_k2=8192))
+
+    def measure(fn):
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / steps
+        seen = {}
+        th = threading.Thread(target=lambda: seen.setdefault("sclk", device_clock()))
+        th.start()
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < 2.0:  # keep the device at this work while the clock is read
+            for _ in range(20):
+                fn()
+            torch.cuda.synchronize()
+        th.join()
+        return ms, seen.get("sclk")
+
+    out = {"what": "the same kernels on random data and on zeros, with the shader clock the device reports meanwhile; "
+                   "2.5 PFLOP/s assumes 2.4 GHz", "library_bf16_gemm_8192": {}, "duo_fwd_seq8192": {}, "duo_bwd_seq8192": {}}
+    for name, (a, b) in mats.items():
+        ms, clk = measure(lambda: a @ b)
+        out["library_bf16_gemm_8192"][name] = {"ms": ms, "tflops": 2.0 * n ** 3 / (ms * 1e-3) / 1e12, "sclk": clk}
+    for name, (d, g1, g2) in {"random": (dev, do1, do2), "zeros": (zero, torch.zeros_like(do1), torch.zeros_like(do2))}.items():
+        fwd, bwd = attention_calls(d, g1, g2)
+        for key, fn in (("duo_fwd_seq8192", fwd), ("duo_bwd_seq8192", bwd)):
+            ms, clk = measure(fn)
+            out[key][name] = {"ms": ms, "sclk": clk}
+    return out
+
+
 def bench_qk_prep(steps: int, warmup: int):
     """q/k RMSNorm + rotary embedding + KV append for the prefill rows of configs[1] (B=4, T=4096): the
     step before the attention call.  HBM-bound: every q, k, v row is read and written once."""
@@ -553,7 +635,7 @@ def main() -> int:
     ap.add_argument("--spinup", type=int, default=200,
                     help="untimed launches of the headline kernel before its warm-up steps (the GPU's clock needs tens of "
                          "milliseconds of work to leave its idle state)")
-    ap.add_argument("--only", choices=["all", "fwd", "decode", "fwd_bwd", "host_layer", "qk_prep", "topk_mix", "e2e"], default="all",
+    ap.add_argument("--only", choices=["all", "fwd", "decode", "fwd_bwd", "host_layer", "context", "qk_prep", "topk_mix", "e2e"], default="all",
                     help="profiling aid: run only one leg (the JSON line then lacks the other legs)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="profiling aid: also run one plain 256 MiB device copy (known traffic for counter scaling)")
@@ -600,6 +682,8 @@ def main() -> int:
                                                                           max(3, args.steps // 4), args.warmup)))
     if args.only in ("all", "decode"):
         legs.append(("decode", bench_decode(args.steps, args.warmup)))
+    if args.only in ("all", "context"):
+        legs.append(("device_context", bench_device_context(args.steps)))
     if args.only in ("all", "qk_prep"):
         legs.append(("qk_prep_prefill", bench_qk_prep(args.steps, args.warmup)))
     if args.only in ("all", "topk_mix"):

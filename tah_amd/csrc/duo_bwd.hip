@@ -482,8 +482,8 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
         const int ktile = (second ? p.ds_kt1 : 0) + kl0 / kBK;
         const int slot1 = q1_lo / kBQ + seq + t1_begin;
         const int slot2 = p.ds_q1slots + q2_lo / kBQ + seq + t2_begin;
-        ds_base1 = ((int64_t)slot1 * p.hq * p.ds_kt + ktile) * kDsBlockBytes + wave * kDsWaveBytes;
-        ds_base2 = ((int64_t)slot2 * p.hq * p.ds_kt + ktile) * kDsBlockBytes + wave * kDsWaveBytes;
+        ds_base1 = (((int64_t)slot1 * p.hq + hk * G) * p.ds_kt + ktile) * kDsBlockBytes + wave * kDsWaveBytes;
+        ds_base2 = (((int64_t)slot2 * p.hq + hk * G) * p.ds_kt + ktile) * kDsBlockBytes + wave * kDsWaveBytes;
     }
     // An item's dS leaves at the start of the next item: a store issued where dS is complete would still be on its
     // way at the barrier that ends the item, whose wait for the staged tiles (vmcnt) counts stores as well.
@@ -563,11 +563,18 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
         if (item + 1 == nt1 * G) src = stream_src(true);  // the next item is the first of the depth-1 stream
     };
     // this wave's 2 KiB of an item's dS block (wave-uniform), and the store of the dS kept from that item
-    [[maybe_unused]] auto ds_store = [&](int item) __attribute__((always_inline)) {
-        const int t = item / G;
-        const int64_t blk = t >= nt1 ? ds_base2 + (int64_t)((t - nt1) * p.hq + hk * G + item % G) * p.ds_kt * kDsBlockBytes
-                                     : ds_base1 + (int64_t)(t * p.hq + hk * G + item % G) * p.ds_kt * kDsBlockBytes;
-        unsigned char* dst = p.ds_ws + blk;
+    // Items follow one another head by head, tile by tile: the block offsets of the current and the previous item are
+    // carried along (two additions per item) instead of being formed from the item number (64-bit multiplies).
+    [[maybe_unused]] const int64_t ds_head_step = (int64_t)p.ds_kt * kDsBlockBytes;
+    [[maybe_unused]] const int64_t ds_tile_step = (int64_t)(p.hq - (G - 1)) * p.ds_kt * kDsBlockBytes;  // last head of a tile -> first of the next
+    [[maybe_unused]] int64_t ds_cur = nt1 > 0 ? ds_base1 : ds_base2, ds_prev = 0;
+    [[maybe_unused]] auto ds_advance = [&](int item) __attribute__((always_inline)) {  // from `item` to `item + 1`
+        ds_prev = ds_cur;
+        ds_cur += (item + 1) % G != 0 ? ds_head_step : ds_tile_step;
+        if (item + 1 == nt1 * G) ds_cur = ds_base2;
+    };
+    [[maybe_unused]] auto ds_store = [&]() __attribute__((always_inline)) {
+        unsigned char* dst = p.ds_ws + ds_prev;
         // (streaming stores: 1 GB of dS per call should not push the Q / dO / K / V tiles out of the L2)
         __builtin_nontemporal_store(ds_keep[0], reinterpret_cast<bf16x8*>(dst + ds_lane_off));
         __builtin_nontemporal_store(ds_keep[1], reinterpret_cast<bf16x8*>(dst + ds_lane_off + 128));
@@ -717,8 +724,8 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
                 dkacc[n % 4] = mfma32(dsfr[(n - 24) / 4], rt[n % 4], dkacc[n % 4]);
             }
             if constexpr (kExport) {
-                if (n == 0 && item > 0) ds_store(item - 1);  // the previous item's dS (before this item's copies are issued)
-                if (n == 31) { ds_keep[0] = dsfr[0]; ds_keep[1] = dsfr[1]; }
+                if (n == 0 && item > 0) ds_store();  // the previous item's dS (before this item's copies are issued)
+                if (n == 31) { ds_keep[0] = dsfr[0]; ds_keep[1] = dsfr[1]; ds_advance(item); }
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -752,7 +759,7 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
     run(t_whole * G, nitems, Masked{});
 
     if constexpr (kExport) {
-        if (nitems > 0) ds_store(nitems - 1);
+        if (nitems > 0) ds_store();
     }
     // ---- add the two query halves and store ---------------------------------
     TAH_WAIT_VMEM();  // no copy may still be on its way into the memory the reduction reuses
