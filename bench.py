@@ -420,16 +420,21 @@ def bench_device_context(steps: int):
         e1.record()
         torch.cuda.synchronize()
         ms = e0.elapsed_time(e1) / steps
-        seen = {}
-        th = threading.Thread(target=lambda: seen.setdefault("sclk", device_clock()))
+        seen = []
+
+        def sample():  # four readings, half a second apart (one reading is a snapshot of a clock that moves)
+            for _ in range(4):
+                seen.append(device_clock())
+                time.sleep(0.5)
+
+        th = threading.Thread(target=sample)
         th.start()
-        t0 = time.perf_counter()
-        while time.perf_counter() - t0 < 2.0:  # keep the device at this work while the clock is read
+        while th.is_alive():  # keep the device at this work while the clock is read
             for _ in range(20):
                 fn()
             torch.cuda.synchronize()
         th.join()
-        return ms, seen.get("sclk")
+        return ms, seen
 
     out = {"what": "the same kernels on random data and on zeros, with the shader clock the device reports meanwhile; "
                    "2.5 PFLOP/s assumes 2.4 GHz", "library_bf16_gemm_8192": {}, "duo_fwd_seq8192": {}, "duo_bwd_seq8192": {}}
