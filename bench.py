@@ -766,7 +766,7 @@ def main() -> int:
                                     "table_build_ms": table_build_ms, "ms_per_step_in_sequence_order": ms_sequence_order},
                    "spinup_launches": spinup, "sustained": sustained},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": measured_traffic("prefill_fwd"), "kernel": "duo_fwd_kernel<2>",
+                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": measured_traffic("prefill_fwd"), "kernel": "duo_fwd_kernel<2, false, 4>",
                      "kernel_ms": ms},
     }
     out["extra"] = extra
