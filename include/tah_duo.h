@@ -343,6 +343,33 @@ typedef struct tah_topk_mix_args {
  * eager arithmetic rounds; sums are float32 in index order, so results do not vary from run to run. */
 int tah_topk_mix(const tah_topk_mix_args* args, tah_stream_t stream);
 
+typedef struct tah_sample_rows_args {
+    const void* logits;        /* bf16 [rows, vocab], vocab contiguous */
+    const void* logits_prev;   /* optional bf16 [rows, vocab]: see add_prev */
+    const int32_t* add_prev;   /* optional int32 [rows]: a row whose entry is not 0 draws from logits_prev + logits, the sum
+                                * rounded to bf16 (the final logits of a token that took a second latent iteration) */
+    const uint8_t* row_enable; /* optional, one byte per row: rows whose byte is 0 are skipped (outputs untouched) */
+    const float* uniforms;     /* float32 [rows], each in [0, 1): the caller's random numbers, one per row and call */
+    int64_t* tokens;           /* optional int64 [rows]: the drawn vocabulary index */
+    float* probs;              /* optional float32 [rows, probs_row_stride]: the distribution drawn from (0 outside the filters) */
+    int64_t logits_row_stride, prev_row_stride, probs_row_stride; /* elements */
+    int32_t rows, vocab;       /* vocab <= 155648 */
+    float temperature;         /* > 0 */
+    float top_p;               /* in (0, 1]; 1: no filter */
+    float min_p;               /* in [0, 1]; 0: no filter */
+} tah_sample_rows_args;
+
+/* One token per row by temperature sampling with the min_p and top_p filters, in one launch and without a sort over
+ * the vocabulary.  Replaces sample_next_token (tah/model/utils.py:84-125) for do_sample=True and top_k == 0:
+ * softmax(logits / temperature); tokens below min_p times the largest probability dropped, renormalised; tokens
+ * dropped once the probability mass before them, in descending order, exceeds top_p, renormalised; one draw.  Tokens
+ * of equal probability are ordered by vocabulary index, lower first (a stable descending sort; torch.sort leaves it
+ * open).  The draw is the inverse-CDF draw over that same order with the caller's uniform number u: the first token
+ * at which the kept mass passes u times the kept total (torch.multinomial draws from the same distribution with its
+ * own generator).  Sums are float32; the row maximum must be finite.  `probs`, when given, receives the filtered and
+ * renormalised distribution itself. */
+int tah_sample_rows(const tah_sample_rows_args* args, tah_stream_t stream);
+
 /* tah_qk_prep (append, one row per sequence) and tah_duo_decode in one launch, for a generation step: the workgroup
  * of a (query, kv head) prepares its query heads and the new K and V itself, stores K and V into the slabs and attends
  * over the cached rows and the new one.  `prep` and `dec` mean what they mean for the two calls (prep->q_out / k_out,

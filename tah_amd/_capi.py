@@ -221,6 +221,17 @@ class TopkMixArgs(C.Structure):
     ]
 
 
+class SampleRowsArgs(C.Structure):
+    """``tah_sample_rows_args``"""
+
+    _fields_ = [
+        ("logits", c_void_p), ("logits_prev", c_void_p), ("add_prev", c_void_p), ("row_enable", c_void_p), ("uniforms", c_void_p),
+        ("tokens", c_void_p), ("probs", c_void_p),
+        ("logits_row_stride", c_int64), ("prev_row_stride", c_int64), ("probs_row_stride", c_int64),
+        ("rows", c_int32), ("vocab", c_int32), ("temperature", c_float), ("top_p", c_float), ("min_p", c_float),
+    ]
+
+
 PROTOTYPES = {
     "tah_duo_abi_version": (C.c_int, []),
     "tah_duo_error_string": (C.c_char_p, [C.c_int]),
@@ -248,6 +259,7 @@ PROTOTYPES = {
     "tah_duo_decode_step": (C.c_int, [C.POINTER(QkPrepArgs), C.POINTER(DuoDecodeArgs), c_void_p, c_void_p, c_void_p]),
     "tah_duo_decode_step_supported": (C.c_int, [c_int32, c_int32, c_int32, c_int32]),
     "tah_topk_mix": (C.c_int, [C.POINTER(TopkMixArgs), c_void_p]),
+    "tah_sample_rows": (C.c_int, [C.POINTER(SampleRowsArgs), c_void_p]),
     "tah_silu_mul": (C.c_int, [c_void_p, c_void_p, c_int32, c_int32, c_int64, c_int64, c_void_p]),
     "tah_hard_index_build": (C.c_int, [c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "tah_pad_rows_build": (C.c_int, [c_void_p, c_void_p, c_int32, c_void_p, c_int32, c_void_p, c_void_p, c_void_p]),

@@ -47,6 +47,7 @@ struct Api {
     decltype(&tah_duo_decode_step) decode_step = nullptr;
     decltype(&tah_duo_decode_step_supported) decode_step_supported = nullptr;
     decltype(&tah_topk_mix) topk_mix = nullptr;
+    decltype(&tah_sample_rows) sample_rows = nullptr;
     decltype(&tah_silu_mul) silu_mul = nullptr;
     decltype(&tah_hard_index_build) hard_index_build = nullptr;
     decltype(&tah_pad_rows_build) pad_rows_build = nullptr;
@@ -91,6 +92,7 @@ void load_library(const std::string& path, bool allow_host) {
     bind(g.decode_step, "tah_duo_decode_step");
     bind(g.decode_step_supported, "tah_duo_decode_step_supported");
     bind(g.topk_mix, "tah_topk_mix");
+    bind(g.sample_rows, "tah_sample_rows");
     bind(g.silu_mul, "tah_silu_mul");
     bind(g.hard_index_build, "tah_hard_index_build");
     bind(g.pad_rows_build, "tah_pad_rows_build");
@@ -646,6 +648,65 @@ Tensor topk_values(const Tensor& logits, int64_t topk, const optional<Tensor>& i
     return vals;
 }
 
+// one token per row by temperature / min_p / top_p sampling (tah_sample_rows); returns tokens int64 [rows], and fills
+// `probs_out` (float32 [rows, V]) with the distribution drawn from when it is given; without `uniforms` only that
+void sample_rows(const Tensor& logits, const optional<Tensor>& logits_prev, const optional<Tensor>& add_prev,
+                 const optional<Tensor>& uniforms, const optional<Tensor>& tokens_out, const optional<Tensor>& probs_out,
+                 const optional<Tensor>& row_enable, double temperature, double top_p, double min_p) {
+    need_lib();
+    Dev d; d.see(logits);
+    TORCH_CHECK(logits.dim() == 2 && logits.scalar_type() == at::kBFloat16 && logits.stride(1) == 1,
+                "sample_rows: logits must be bf16 [rows, V] with a contiguous inner dimension");
+    const int64_t rows = logits.size(0), V = logits.size(1);
+    tah_sample_rows_args a{};
+    a.logits = ptr(logits);
+    a.logits_row_stride = rows > 1 ? logits.stride(0) : V;
+    if (logits_prev.has_value()) {
+        d.see(*logits_prev);
+        TORCH_CHECK(logits_prev->sizes() == logits.sizes() && logits_prev->scalar_type() == at::kBFloat16 && logits_prev->stride(1) == 1,
+                    "sample_rows: logits_prev must be bf16 [rows, V] like logits");
+        TORCH_CHECK(add_prev.has_value(), "sample_rows: logits_prev needs add_prev");
+        a.logits_prev = ptr(*logits_prev);
+        a.prev_row_stride = rows > 1 ? logits_prev->stride(0) : V;
+    }
+    if (add_prev.has_value()) {
+        d.see(*add_prev);
+        TORCH_CHECK(add_prev->scalar_type() == at::kInt && add_prev->is_contiguous() && add_prev->numel() == rows,
+                    "sample_rows: add_prev must be a contiguous int32 [rows] tensor");
+        TORCH_CHECK(logits_prev.has_value(), "sample_rows: add_prev needs logits_prev");
+        a.add_prev = static_cast<const int32_t*>(add_prev->data_ptr());
+    }
+    if (uniforms.has_value()) {
+        d.see(*uniforms);
+        TORCH_CHECK(uniforms->scalar_type() == at::kFloat && uniforms->is_contiguous() && uniforms->numel() == rows && tokens_out.has_value(),
+                    "sample_rows: uniforms must be a contiguous float32 [rows] tensor, given together with tokens_out");
+        d.see(*tokens_out);
+        TORCH_CHECK(tokens_out->scalar_type() == at::kLong && tokens_out->is_contiguous() && tokens_out->numel() == rows,
+                    "sample_rows: tokens_out must be a contiguous int64 [rows] tensor");
+        a.uniforms = static_cast<const float*>(uniforms->data_ptr());
+        a.tokens = static_cast<int64_t*>(tokens_out->data_ptr());
+    }
+    if (probs_out.has_value()) {
+        d.see(*probs_out);
+        TORCH_CHECK(probs_out->scalar_type() == at::kFloat && probs_out->dim() == 2 && probs_out->size(0) == rows && probs_out->size(1) == V &&
+                        probs_out->stride(1) == 1,
+                    "sample_rows: probs_out must be float32 [rows, V] with a contiguous inner dimension");
+        a.probs = static_cast<float*>(probs_out->data_ptr());
+        a.probs_row_stride = rows > 1 ? probs_out->stride(0) : V;
+    }
+    TORCH_CHECK(a.tokens || a.probs, "sample_rows: nothing to produce (give uniforms and tokens_out, or probs_out)");
+    if (row_enable.has_value()) {
+        d.see(*row_enable);
+        TORCH_CHECK((row_enable->scalar_type() == at::kBool || row_enable->scalar_type() == at::kByte) && row_enable->is_contiguous() &&
+                        row_enable->numel() == rows,
+                    "sample_rows: row_enable must be a contiguous bool/uint8 [rows] tensor");
+        a.row_enable = static_cast<const uint8_t*>(row_enable->data_ptr());
+    }
+    a.rows = (int32_t)rows; a.vocab = (int32_t)V;
+    a.temperature = (float)temperature; a.top_p = (float)top_p; a.min_p = (float)min_p;
+    check_rc(g.sample_rows(&a, d.stream()), "tah_sample_rows");
+}
+
 Tensor silu_mul(const Tensor& gate_up, const optional<Tensor>& norm_input, double norm_eps) {
     need_lib();
     Dev d; d.see(gate_up); d.see(norm_input);
@@ -913,6 +974,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("pad_rows_build", &pad_rows_build);
     m.def("rows_copy", &rows_copy);
     m.def("topk_mix", &topk_mix);
+    m.def("sample_rows", &sample_rows);
     m.def("topk_values", &topk_values);
     m.def("silu_mul", &silu_mul);
     m.def("duo_decode_step", &duo_decode_step);

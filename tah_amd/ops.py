@@ -161,6 +161,29 @@ def topk(logits: torch.Tensor, k: int):
     return _call("topk_values", logits, int(k), idx), idx
 
 
+def sample_rows(logits: torch.Tensor, uniforms: torch.Tensor, temperature: float, *, top_p: float = 1.0, min_p: float = 0.0,
+                logits_prev: Optional[torch.Tensor] = None, add_prev: Optional[torch.Tensor] = None,
+                row_enable: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One token per row of bf16 logits [rows, V] by temperature sampling with the min_p and top_p filters of
+    ``sample_next_token`` (tah/model/utils.py:84-125, ``top_k == 0``), in one launch and without a sort over the vocabulary
+    (``tah_sample_rows``).  ``uniforms`` float32 [rows] in [0, 1): the row's random number (``torch.rand``); the draw is the
+    inverse-CDF draw over the tokens in descending order of probability, equal ones by ascending index.  Rows whose
+    ``add_prev`` entry (int32 [rows]) is not 0 draw from ``logits_prev + logits`` (summed in bf16).  Returns int64 [rows]."""
+    if out is None:
+        out = torch.zeros(logits.size(0), dtype=torch.int64, device=logits.device)
+    _call("sample_rows", logits, logits_prev, add_prev, uniforms, out, None, row_enable, float(temperature), float(top_p), float(min_p))
+    return out
+
+
+def sample_probs(logits: torch.Tensor, temperature: float, *, top_p: float = 1.0, min_p: float = 0.0,
+                 logits_prev: Optional[torch.Tensor] = None, add_prev: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The distribution :func:`sample_rows` draws from, float32 [rows, V]: softmax(logits / temperature), then min_p and
+    top_p, each renormalised; zero outside the filters."""
+    probs = torch.empty(logits.shape, dtype=torch.float32, device=logits.device)
+    _call("sample_rows", logits, logits_prev, add_prev, None, None, probs, None, float(temperature), float(top_p), float(min_p))
+    return probs
+
+
 def silu_mul(gate_up: torch.Tensor, norm_input: Optional[torch.Tensor] = None, norm_eps: float = 0.0) -> torch.Tensor:
     """``silu(gate) * up`` of a fused gate|up projection, bf16 [rows, 2*I] -> [rows, I], in one launch.
 
