@@ -78,7 +78,7 @@ __device__ __forceinline__ T wave_incl_scan(T x, int lane) {
     return x;
 }
 
-template <int NVEC>
+template <int NVEC, bool kProbs>
 __global__ __launch_bounds__(kSmpThreads) void sample_rows_kernel(const SampleParams p) {
     __shared__ float wtot[kSmpWaves];
     __shared__ int wv[kSmpMaxVec][kSmpWaves];  // per piece and wave: tokens equal to the key looked for
@@ -185,18 +185,19 @@ __global__ __launch_bounds__(kSmpThreads) void sample_rows_kernel(const SamplePa
         for (int i = 0; i < kBinsPerThread + 1; ++i) mine[i] = 0u;  // (33 words per thread cover the padded array)
         __syncthreads();
         const uint32_t span = dmax - wbase < (uint32_t)kWinKeys - 1u ? dmax - wbase : (uint32_t)kWinKeys - 1u;  // rel <= span
+        // rel = kmax - wbase - key, both halves of a dword at once in 16-bit arithmetic: keys above the window wrap to
+        // 32768 and more, keys below it (and key 0, past the end of the row) stay above span as they are
+        const uint32_t kb2 = ((kmax - wbase) & 0xffffu) * 0x10001u;
 #pragma unroll
         for (int j = 0; j < NVEC; ++j) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 uint32_t w = keys[j][q];
                 TAH_OPAQUE1(w);
-#pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    const uint32_t key = h ? (w >> 16) : (w & 0xffffu);
-                    const uint32_t rel = kmax - key - wbase;  // (key 0: kmax - wbase, past dmax - wbase)
-                    if (rel <= span && key != 0u) atomicAdd(&hist[rel + (rel >> 5)], 1u);
-                }
+                const uint32_t r2 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(u16x2, kb2) - __builtin_bit_cast(u16x2, w));
+                const uint32_t r0 = r2 & 0xffffu, r1 = r2 >> 16;
+                if (r0 <= span) atomicAdd(&hist[r0 + (r0 >> 5)], 1u);
+                if (r1 <= span) atomicAdd(&hist[r1 + (r1 >> 5)], 1u);
             }
         }
         __syncthreads();
@@ -440,7 +441,7 @@ __global__ __launch_bounds__(kSmpThreads) void sample_rows_kernel(const SamplePa
     }
 
     // ---- optionally the distribution itself: softmax, min_p, top_p, each renormalised ------------------------
-    if (p.probs) {
+    if constexpr (kProbs) {
         float* orow = p.probs + (int64_t)row * p.pr_rs;
         const float inv = Z > 0.f ? 1.f / Z : 0.f;
         const uint32_t kcut = dcut <= dmax ? kmax - dcut : 0u;  // key of the partly kept tokens (0: none)
@@ -517,10 +518,11 @@ extern "C" int tah_sample_rows(const tah_sample_rows_args* a, tah_stream_t strea
     hipStream_t st = static_cast<hipStream_t>(stream);
 #define TAH_SAMPLE_LAUNCH(N)                                                                                                  \
     do {                                                                                                                      \
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&sample_rows_kernel<N>), hipFuncAttributeMaxDynamicSharedMemorySize, \
+        auto* kern = a->probs ? &sample_rows_kernel<N, true> : &sample_rows_kernel<N, false>;                                 \
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,              \
                                 (int)kSmpSmem) != hipSuccess)                                                                 \
             return TAH_E_LAUNCH;                                                                                              \
-        hipLaunchKernelGGL(sample_rows_kernel<N>, grid, block, kSmpSmem, st, p);                                              \
+        hipLaunchKernelGGL(kern, grid, block, kSmpSmem, st, p);                                                               \
     } while (0)
     if (nvec <= 2) TAH_SAMPLE_LAUNCH(2);
     else if (nvec <= 8) TAH_SAMPLE_LAUNCH(8);

@@ -202,6 +202,7 @@ class TaHDecodeEngine:
         self.zeros_i = torch.zeros(batch, dtype=torch.int32, device=dev)
         # generation state (all on the device)
         self.fused_greedy = True  # arg-max + bookkeeping of a greedy step in one launch (tah_greedy_step)
+        self.fused_sampling = True  # draws without a top-k filter in one launch (tah_sample_rows) instead of a sort in torch
         self.use_fused_glue = True  # (tests switch it off to compare with the torch glue)
         self.tok = torch.zeros(batch, dtype=torch.long, device=dev)       # token fed to the next step
         self.pos = torch.zeros(batch, dtype=torch.int32, device=dev)      # its position
@@ -630,12 +631,24 @@ class TaHDecodeEngine:
         j = torch.argmax(probs / torch.empty_like(probs).exponential_(), dim=-1, keepdim=True)
         return torch.gather(idx, 1, j).squeeze(1).to(torch.int64)
 
-    def _draw(self, final_bf16: torch.Tensor, temperature: float, **filters) -> torch.Tensor:
-        """One token per row from final logits in bf16: on the top-k values when there is a top-k filter, else on the row."""
+    # Without a top-k filter the draw is one ``tah_sample_rows`` launch on the bf16 logits (no sort over the vocabulary);
+    # with one of at most 256 places it runs on the k largest logits; anything else takes the torch formulation.
+    SAMPLE_ROWS_MAX_VOCAB = 155648
+
+    def _draw(self, logits: torch.Tensor, temperature: float, prev: Optional[torch.Tensor] = None,
+              add_prev: Optional[torch.Tensor] = None, **filters) -> torch.Tensor:
+        """One token per row from final logits in bf16.  ``prev`` / ``add_prev`` (int32 [rows]): rows whose entry is not 0
+        draw from ``prev + logits``, summed in bf16 as the step-wise loop forms the final logits of a hard token."""
         k = int(filters.get("top_k", 0))
-        if 0 < k <= self.TOPK_SAMPLING_MAX and final_bf16.dtype == torch.bfloat16 and final_bf16.size(-1) <= 155648:
-            return self.sample_topk(final_bf16, temperature, **filters)
-        return self.sample(final_bf16.float(), temperature, **filters)
+        fits = logits.dtype == torch.bfloat16 and logits.size(-1) <= self.SAMPLE_ROWS_MAX_VOCAB
+        if k == 0 and fits and self.fused_sampling:
+            u = torch.rand(logits.size(0), dtype=torch.float32, device=logits.device)
+            return ops.sample_rows(logits, u, temperature, top_p=float(filters.get("top_p", 1.0)), min_p=float(filters.get("min_p", 0.0)),
+                                   logits_prev=prev, add_prev=add_prev)
+        final = logits if prev is None else torch.where((add_prev != 0)[:, None], prev + logits, logits)
+        if 0 < k <= self.TOPK_SAMPLING_MAX and fits:
+            return self.sample_topk(final, temperature, **filters)
+        return self.sample(final.float(), temperature, **filters)
 
     def _step_inplace(self, temperature: float, eos: int, **filters):
         """One generated token for every unfinished row; every state change is an in-place device update."""
@@ -646,8 +659,10 @@ class TaHDecodeEngine:
                             self.n_hard, self.n_steps)
             self.step_idx += 1
             return
-        logits = torch.where(hard[:, None], l0 + l1, l0)  # as step_logits forms them (the sum in the logits' dtype)
-        nxt = self._draw(logits, temperature, **filters) if temperature > 0.0 else self.sample(logits.float(), 0.0)
+        if temperature > 0.0:  # final logits as step_logits forms them: l0, plus l1 for hard tokens (the sum in the logits' dtype)
+            nxt = self._draw(l0, temperature, prev=l1, add_prev=hard.to(torch.int32), **filters)
+        else:
+            nxt = self.sample(torch.where(hard[:, None], l0 + l1, l0).float(), 0.0)
         nxt = torch.where(act, nxt, torch.zeros_like(nxt))
         if eos >= 0:
             self.finished |= nxt == eos
@@ -737,9 +752,7 @@ class TaHDecodeEngine:
         if temperature > 0.0:
             # one draw per row from the final logits as the step-wise loop forms them (first iteration, plus the second
             # where there was one, summed in bf16); rows that only move on to their second iteration ignore theirs
-            prev = self.logits2[1 - parity]
-            final = torch.where((self.phase != 0)[:, None], prev + logits, logits)
-            chosen = self._draw(final, temperature, **filters).contiguous()
+            chosen = self._draw(logits, temperature, prev=self.logits2[1 - parity], add_prev=self.phase, **filters).contiguous()
         ops.greedy_tick(logits, self.logits2[1 - parity], eos, limit, hard_now=self.hard, phase=self.phase, tok=self.tok,
                         finished=self.finished, pos=self.pos, out_tokens=self.out_tokens, out_len=self.out_len,
                         hard_len=self.hard_len, n_hard=self.n_hard, n_steps=self.n_steps, chosen=chosen)
@@ -748,7 +761,7 @@ class TaHDecodeEngine:
         """Every attribute that changes which kernels a captured step launches: part of both graph keys, so that
         flipping one between two generate() calls on the same prefill captures again instead of replaying a graph
         of the old path."""
-        return (self.use_fused_glue, self.fused_greedy, self.static_scratch, self.measure_without_attention, id(self.decider))
+        return (self.use_fused_glue, self.fused_greedy, self.fused_sampling, self.static_scratch, self.measure_without_attention, id(self.decider))
 
     def capture_ticks(self, eos: int, limit: int, temperature: float = 0.0, **filters):
         """The tick as two HIP graphs, one per logits buffer, after a warm-up tick whose state changes are undone."""

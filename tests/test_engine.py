@@ -378,6 +378,7 @@ def test_continuous_generation_with_sampling_gpu():
     for continuous, use_graph in ((False, True), (True, False), (True, True)):
         eng = TaHDecodeEngine(w, B, T + new + 2, device="cuda")
         eng.sample = second_best
+        eng.fused_sampling = False  # (draws without a top-k filter go through ``sample``)
         first, _ = eng.prefill(ids, cu, calibrate=0.25)
         toks = eng.generate(first, new, temperature=0.7, eos=-1, continuous=continuous, use_graph=use_graph).clone()
         runs.append((toks.cpu(), eng.out_len.cpu(), int(eng.n_hard), [sl.len.tolist() for sl in eng.slabs1]))
@@ -399,6 +400,22 @@ def test_continuous_generation_with_sampling_gpu():
     eng = TaHDecodeEngine(w, B, T + new + 2, device="cuda")
     first, _ = eng.prefill(same, cu, calibrate=0.25)
     toks = eng.generate(first, new, temperature=1.0, top_k=50, eos=-1)
+    assert len({tuple(r.tolist()) for r in toks}) > B // 2
+    assert min(len(set(toks[:, j].tolist())) for j in range(1, new)) > B // 4
+    # without a top-k filter the draw is one tah_sample_rows launch on the tick's and the previous tick's logits.  With
+    # top_p so small that only the largest token survives, it has to reproduce the greedy generation, step-wise and in ticks
+    want = greedy.out_tokens[:, :new].cpu()
+    for continuous in (False, True):
+        eng = TaHDecodeEngine(w, B, T + new + 2, device="cuda")
+        first, _ = eng.prefill(ids, cu, calibrate=0.25)
+        toks = eng.generate(first, new, temperature=0.9, top_p=1e-6, eos=-1, continuous=continuous)
+        assert torch.equal(toks.cpu(), want), continuous
+    # and with real filters: every row gets its tokens, equal rows draw apart, at every replay
+    eng = TaHDecodeEngine(w, B, T + new + 2, device="cuda")
+    first, _ = eng.prefill(same, cu, calibrate=0.25)
+    toks = eng.generate(first, new, temperature=1.0, top_p=0.95, min_p=0.001, eos=-1)
+    assert eng.ticks >= new - 1 and (eng.out_len == new).all()
+    assert int(toks.min()) >= 0 and int(toks.max()) < cfg.vocab
     assert len({tuple(r.tolist()) for r in toks}) > B // 2
     assert min(len(set(toks[:, j].tolist())) for j in range(1, new)) > B // 4
 
