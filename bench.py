@@ -535,6 +535,46 @@ def bench_topk_mix(steps: int, warmup: int, rows: int = 1024, vocab: int = 15193
             "topk_values_ms": val_ms, "torch_topk_ms": torch_ms, "rows_per_s": rows / (mix_ms * 1e-3)}
 
 
+def bench_sample_rows(steps: int, warmup: int, vocab: int = 151936, temperature: float = 0.6, top_p: float = 0.95):
+    """The draw of a generation step without a top-k filter (tah/model/utils.py:84-125): one tah_sample_rows launch over the
+    32 rows of the end-to-end workload, next to the torch formulation it replaces (softmax, sort over the vocabulary,
+    cumulative sum, scatter, renormalisation, draw), and over 1024 rows against the bytes of the logits."""
+    import torch
+
+    from tah_amd import ops
+    from tah_amd.engine import TaHDecodeEngine
+
+    g = torch.Generator().manual_seed(1242)
+    logits = [(torch.randn(1024, vocab, generator=g) * 3).to(torch.bfloat16).cuda() for _ in range(2)]  # two sets in rotation
+    u = torch.rand(1024, generator=g).cuda()
+    out = torch.zeros(1024, dtype=torch.int64, device="cuda")
+    yield
+
+    def timed(f, n):
+        for i in range(warmup):
+            f(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(n):
+            f(i)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n
+
+    ms32 = timed(lambda i: ops.sample_rows(logits[i % 2][:32], u[:32], temperature, top_p=top_p, out=out[:32]), steps)
+    torch32 = timed(lambda i: TaHDecodeEngine.sample(logits[i % 2][:32].float(), temperature, top_p=top_p), max(3, steps // 4))
+    ms1024 = timed(lambda i: ops.sample_rows(logits[i % 2], u, temperature, top_p=top_p, out=out), steps)
+    nbytes = 1024 * vocab * 2
+    gbs = nbytes / (ms1024 * 1e-3) / 1e9
+    return {"workload": f"temperature {temperature} / top_p {top_p} draw without a top-k filter, rows of {vocab} bf16 logits",
+            "ms_per_step_32_rows": ms32, "torch_ms_per_step_32_rows": torch32,
+            "ms_per_step": ms1024, "rows": 1024, "algorithmic_bytes": nbytes, "hbm_gbs": gbs,
+            "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
+                         "traffic": None, "kernels": "sample_rows_kernel<19, false>"},
+            "rows_per_s": 1024 / (ms1024 * 1e-3)}
+
+
 def bench_e2e_decode(new_tokens: int, B: int = 32, prompt_len: int = 512, temperature: float = 0.0, top_p: float = 0.95, top_k: int = 0):
     """BASELINE configs[4]: end-to-end TaH decode, Qwen3-1.7B architecture with random weights, a two-layer MLP
     decider whose threshold is set so that about 6 % of the prompt tokens iterate, batch 32, 512-token prompts.
@@ -640,7 +680,7 @@ def main() -> int:
     ap.add_argument("--spinup", type=int, default=200,
                     help="untimed launches of the headline kernel before its warm-up steps (the GPU's clock needs tens of "
                          "milliseconds of work to leave its idle state)")
-    ap.add_argument("--only", choices=["all", "fwd", "decode", "fwd_bwd", "host_layer", "context", "qk_prep", "topk_mix", "e2e"], default="all",
+    ap.add_argument("--only", choices=["all", "fwd", "decode", "fwd_bwd", "host_layer", "context", "qk_prep", "topk_mix", "sample_rows", "e2e"], default="all",
                     help="profiling aid: run only one leg (the JSON line then lacks the other legs)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="profiling aid: also run one plain 256 MiB device copy (known traffic for counter scaling)")
@@ -693,6 +733,8 @@ def main() -> int:
         legs.append(("qk_prep_prefill", bench_qk_prep(args.steps, args.warmup)))
     if args.only in ("all", "topk_mix"):
         legs.append(("topk_mix", bench_topk_mix(args.steps, args.warmup)))
+    if args.only in ("all", "sample_rows"):
+        legs.append(("sample_rows", bench_sample_rows(args.steps, args.warmup)))
     if args.only in ("all", "e2e"):
         legs.append(("e2e_decode", bench_e2e_decode(args.e2e_tokens, temperature=args.e2e_temperature, top_k=args.e2e_top_k)))
     for _, leg in legs:
