@@ -21,7 +21,11 @@
  * by the position of their last row.
  *
  * Visibility (tah/model/tah_model.py:788): key (pos_k, depth_k) is visible to
- * query (pos_q, depth_q) iff pos_k <= pos_q and depth_k <= depth_q.
+ * query (pos_q, depth_q) iff pos_k <= pos_q and depth_k <= depth_q.  The two
+ * streams are what that rule needs for any depth: queries at depth d >= 2 go
+ * where depth-1 queries go, with the keys of depths 1 .. d together as their
+ * position-carrying key stream (rows of a sequence in any order; all of them
+ * satisfy depth_k <= depth_q).
  * GQA: query head h reads kv head h / (Hq / Hkv)
  * (transformers/integrations/sdpa_attention.py:15-24, repeat_kv).
  */

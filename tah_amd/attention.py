@@ -111,6 +111,7 @@ class DuoMask:
         self.position_ids, self.valid_mask, self.cache, self.iter_depth = position_ids, valid_mask, cache, iter_depth
         self._packed = None  # per-step packing metadata, shared by all decoder layers
         self._sched = None   # launch-order table of the step's varlen calls, likewise
+        self._merge = None   # where the rows of depths 1 .. iter_depth go in their common packing (depth >= 2)
 
     def dense(self, dtype: torch.dtype = torch.float32) -> Optional[torch.Tensor]:
         """The (B,1,Tq,Tkv) additive mask the reference would have built (for inspection only)."""
@@ -147,11 +148,10 @@ def build_attention_mask(active_position_ids, active_valid_mask, cache, iter_dep
 
 
 def _check_depth(iter_depth: int) -> None:
-    """The kernels know two latent iterations; the reference's mask handles any depth (tah_model.py:788) and
-    its deciders accept ``max_iter`` 3, so a deeper call must fail here and not be computed as depth 1."""
-    if not 0 <= int(iter_depth) <= 1:
-        raise TahDuoError(f"iter_depth = {iter_depth}: duo-causal attention is implemented for depths 0 and 1 "
-                          "(max_iter = 2, as in every shipped recipe)")
+    """Any latent depth is accepted, as the reference's mask accepts it (tah_model.py:788): a query at depth d sees the
+    keys at or before its position of every depth <= d."""
+    if int(iter_depth) < 0:
+        raise TahDuoError(f"iter_depth = {iter_depth}: a latent iteration depth cannot be negative")
 
 
 # Debug switch: verify on the device (one host sync per model step) that the positions handed in are the
@@ -305,6 +305,52 @@ def _segment(cache: TaHDuoCache, layer_idx: int, depth: int, B: int, with_pos: b
     return pk.pack(k), pk.pack(v), pk.cu, pk.pos
 
 
+def _merge_plan(m: "DuoMask", segs, B: int):
+    """Where the rows of several packed segments go when they are packed together, sequence by sequence (inside a
+    sequence: the first segment's rows, then the second's, ...): (dest int64 [sum of rows], cu int32 [B+1], pos int32).
+    Built on the device from the segments' boundaries, once per step (every layer caches the same boundaries).  Rows
+    past a segment's cu[B] (packing by upper bounds) go past the merged cu[B]."""
+    key = tuple((sg[2].data_ptr(), sg[0].shape[0]) for sg in segs)
+    memo = getattr(m, "_merge", None)
+    if memo is not None and memo[0] == key:
+        return memo[1:]
+    dev = segs[0][2].device
+    cus = [sg[2].long() for sg in segs]
+    cu_m = torch.stack(cus).sum(0)
+    off = torch.zeros(B, dtype=torch.long, device=dev)
+    tail = cu_m[B]
+    dests = []
+    for cu, sg in zip(cus, segs):
+        n = sg[0].shape[0]
+        r = torch.arange(n, dtype=torch.long, device=dev)
+        seq = torch.searchsorted(cu[1:].contiguous(), r, right=True)
+        sq = seq.clamp(max=B - 1)
+        dests.append(torch.where(seq < B, cu_m[sq] + off[sq] + (r - cu[sq]), tail + (r - cu[B])))
+        off = off + (cu[1:] - cu[:-1])
+        tail = tail + (n - cu[B])
+    dest = torch.cat(dests)
+    pos = torch.zeros(dest.shape[0], dtype=torch.int32, device=dev).index_copy_(0, dest, torch.cat([sg[3] for sg in segs]))
+    m._merge = (key, dest, cu_m.to(torch.int32), pos)
+    return m._merge[1:]
+
+
+def _sparse_keys(m: "DuoMask", cache: TaHDuoCache, layer: int, depth: int, B: int):
+    """The keys a query at ``depth`` >= 1 sees beside the depth-0 ones: every row cached at depths 1 .. depth, packed per
+    sequence with their positions -- (k, v, cu, pos, upper bound of a sequence's rows).  The kernels tell depth-0 keys
+    (position = index) from keys that carry a position, and among the latter a query sees those at or before its own
+    position whatever their depth (tah_model.py:788 with depth_k <= depth_q for all of them), so deeper calls hand the
+    kernels the union of these depths as the one sparse key stream; one depth needs no copy."""
+    segs = [_segment(cache, layer, d, B, with_pos=True) for d in range(1, depth + 1) if cache.has_rows(layer, d)]
+    if not segs:
+        raise TahDuoError(f"no keys cached for layer {layer} at depths 1..{depth}")
+    bound = sum(cache.get_cache_length(layer, d) for d in range(1, depth + 1))
+    if len(segs) == 1:
+        return segs[0] + (bound,)
+    dest, cu, pos = _merge_plan(m, segs, B)
+    kcat, vcat = torch.cat([sg[0] for sg in segs]), torch.cat([sg[1] for sg in segs])
+    return torch.zeros_like(kcat).index_copy(0, dest, kcat), torch.zeros_like(vcat).index_copy(0, dest, vcat), cu, pos, bound
+
+
 def duo_attention_forward(module, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
                           attention_mask, dropout: float = 0.0, scaling: Optional[float] = None,
                           is_causal: Optional[bool] = None, **kwargs) -> Tuple[torch.Tensor, None]:
@@ -348,7 +394,7 @@ def duo_attention_forward(module, query: torch.Tensor, key: torch.Tensor, value:
 
     # decode fast path: one query row per sequence, slabs hold every cached row (incl. this step's)
     s1 = cache.slabs(layer, 0)
-    if Tq == 1 and s1 is not None and not (torch.is_grad_enabled() and query.requires_grad):
+    if Tq == 1 and s1 is not None and depth <= 1 and not (torch.is_grad_enabled() and query.requires_grad):
         # every batch row is a query row; a row that is not valid (a pad row of the depth-1 pack, tah_model.py:116-118)
         # gets position -1, sees nothing and comes back as zeros -- no index to build, nothing read back
         if m._packed is None:
@@ -378,11 +424,11 @@ def duo_attention_forward(module, query: torch.Tensor, key: torch.Tensor, value:
         o, _ = duo_attn_varlen(q, k1, v1, pq.cu, cu_k1, e_q, e_k, e_k, zi, zi, zc, zc, scale, schedule=sched,
                                max_seqlen_k1=cache.get_cache_length(layer, 0))
     else:
-        k2, v2, cu_k2, pos_k2 = _segment(cache, layer, 1, B, with_pos=True)
+        k2, v2, cu_k2, pos_k2, bound_k2 = _sparse_keys(m, cache, layer, depth, B)
         e_q = q[:0]
         sched = _schedule_of(m, (zc, cu_k1, pq.cu, cu_k2, pq.pos, Hq, Hkv, 0, k1.shape[0], k2.shape[0]))
         _, o = duo_attn_varlen(e_q, k1, v1, zc, cu_k1, q, k2, v2, pq.pos, pos_k2, pq.cu, cu_k2, scale, schedule=sched,
-                               max_seqlen_k1=cache.get_cache_length(layer, 0), max_seqlen_k2=cache.get_cache_length(layer, 1))
+                               max_seqlen_k1=cache.get_cache_length(layer, 0), max_seqlen_k2=bound_k2)
     return pq.unpack(o, Hq, D), None
 
 

@@ -147,9 +147,11 @@ class TaHDuoCache:
             assert key_states.shape[0] == self.batch_size, (
                 f"batch size mismatch: cached {self.batch_size}, got {key_states.shape[0]}")
         self._device, self._dtype = key_states.device, key_states.dtype
-        if not 0 <= int(self.current_iter_depth) <= 1:
-            raise TahDuoError(f"current_iter_depth = {self.current_iter_depth}: the kernels implement two latent "
-                              "iterations (depth 0 and depth 1), as every shipped recipe uses (max_iter = 2)")
+        if int(self.current_iter_depth) < 0:
+            raise TahDuoError(f"current_iter_depth = {self.current_iter_depth}: a latent iteration depth cannot be negative")
+        if int(self.current_iter_depth) > 1 and self._slab_cfg is not None:
+            raise TahDuoError(f"current_iter_depth = {self.current_iter_depth}: the KV slabs of the decode path hold two latent "
+                              "iterations (depth 0 and depth 1); deeper iterations run without enable_slabs()")
         slot = (layer_idx, self.current_iter_depth)
         to_slabs = self._slab_cfg is not None and not (torch.is_grad_enabled() and key_states.requires_grad)
         if to_slabs:
@@ -176,6 +178,10 @@ class TaHDuoCache:
     def _slabs_cover(self, slot: _Slot) -> bool:
         """True when every row ever written to the slot also went to its slabs."""
         return slot in self._slabs and self._slab_rows.get(slot, 0) == self._rows.get(slot, 0)
+
+    def has_rows(self, layer_idx: int, depth: int) -> bool:
+        """Whether anything was written at (layer, depth)."""
+        return self._rows.get((layer_idx, depth), 0) > 0
 
     # ── chunk access for the attention callable ───────────────────────────
     def chunks(self, layer_idx: int, depth: int):

@@ -5,7 +5,8 @@ import torch
 
 from oracle import duo_oracle as O
 from tests.cases import make_dense_case
-from tests.test_host_layer import _forward_two_depths, _forward_two_depths_reference_style, _oracle_two_depths
+from tests.test_host_layer import (_deeper_levels, _forward_two_depths, _forward_two_depths_reference_style, _loops_over_depths,
+                                   _oracle_two_depths, check_depth_gradients, check_depth_outputs)
 
 pytestmark = pytest.mark.gpu
 
@@ -111,3 +112,13 @@ def test_forward_loop_without_host_sync_gpu():
     reference's loop has there)."""
     from tests.sync_free_case import run
     assert run("cuda", B=3, T=300, p=0.1, left_pad=(0, 37, 150), Hq=16, Hkv=8)
+
+
+@pytest.mark.parametrize("B,T,p,left_pad,n_deeper", [(2, 300, 0.3, [0, 41], 1), (1, 600, 0.25, None, 2)])
+def test_forward_loop_over_more_than_two_depths_gpu(B, T, p, left_pad, n_deeper):
+    """Latent depths 2 and 3 (tah_model.py:788 takes any): outputs and gradients against the dense restatement."""
+    c = make_dense_case(70 + B, B=B, T=T, p_hard=p, left_pad=left_pad)
+    deeper = _deeper_levels(c, 71, n_deeper)
+    outs, leaves, rleaves = _loops_over_depths(c, deeper, requires_grad=True, device="cuda")
+    check_depth_outputs(c, outs)
+    check_depth_gradients(c, outs, leaves, rleaves)

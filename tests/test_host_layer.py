@@ -275,23 +275,121 @@ def test_slab_overflow_raises_through_cache_update(emu):
     assert int(cache.slabs(0, 0).overflow) == 0 and cache.slabs(0, 0).len.tolist() == [6]
 
 
-def test_depth_two_is_refused(emu):
-    """The reference's mask and cache take any depth (tah_model.py:788); this build has two and says so."""
+def _loops_over_depths(c, deeper, requires_grad=False, device="cpu"):
+    """The reference's forward loop (tah_model.py:580-623) over more than two latent iterations, run twice on the same
+    bf16 inputs: through this package (TaHDuoCache, DuoMask, duo_attention_forward) and through the dense restatement
+    (list cache, dense mask, softmax in float64).  ``deeper``: [(active mask (B, T), q, k, v dense (B, H, T, D)), ...]
+    for depths 2, 3, ...; depth 1 uses c["hard"] and q2 / k2 / v2.  Returns per depth (ours, reference, pad mask), and
+    the leaves of both runs."""
+    from tah_amd.attention import build_attention_mask, duo_attention_forward
+    from tah_amd.cache import TaHDuoCache
+    from tah_amd.pack import gather_active
+    cache, ocache = TaHDuoCache(), O.OracleCache()
+    valid = c["valid"]
+    pos = (torch.cumsum(valid, -1) - 1).clamp(min=0)
+    levels = [(None, c["q1"], c["k1"], c["v1"]), (c["hard"], c["q2"], c["k2"], c["v2"])] + list(deeper)
+    tok = lambda x: x.transpose(1, 2)
+    leaves, rleaves, outs = [], [], []
+    for depth, (active, q, k, v) in enumerate(levels):
+        t = [x.to(torch.bfloat16).to(device).requires_grad_(requires_grad) for x in (q, k, v)]
+        r = [x.to(torch.bfloat16).double().requires_grad_(requires_grad) for x in (q, k, v)]
+        leaves.append(t)
+        rleaves.append(r)
+        if active is None:
+            (tq, tk, tv), (rq, rk, rv), p, vl, rp, rvl, pad = t, r, pos.to(device), valid.to(device), pos, valid, None
+        else:
+            pad, tq, tk, tv, p, vl = gather_active(active.to(device), tok(t[0]), tok(t[1]), tok(t[2]), pos.to(device), valid.to(device))
+            rpad, rq, rk, rv, rp, rvl = O.gather_active(active, tok(r[0]), tok(r[1]), tok(r[2]), pos, valid)
+            pad = pad.cpu()
+            assert torch.equal(pad, rpad) and torch.equal(p.cpu(), rp) and torch.equal(vl.cpu(), rvl)
+            tq, tk, tv, rq, rk, rv = (tok(x) for x in (tq, tk, tv, rq, rk, rv))
+        m = build_attention_mask(p, vl, cache, depth, dtype=torch.bfloat16)
+        om = O.build_attention_mask(rp, rvl, ocache, depth, torch.float64)
+        assert torch.equal(m.dense(torch.float64).cpu(), om)
+        cache.current_iter_depth, cache.position_ids_to_cache, cache.valid_mask_to_cache = depth, p, vl
+        ocache.current_iter_depth, ocache.position_ids_to_cache, ocache.valid_mask_to_cache = depth, rp, rvl
+        kk, vv = cache.update(tk, tv, 0)
+        o, _ = duo_attention_forward(_layer(), tq, kk, vv, m, scaling=c["scale"])
+        K, V = ocache.update(rk, rv, 0)
+        outs.append((o, O.sdpa_dense(rq, K, V, om, c["scale"]), pad))
+    assert cache.get_cache_iter_index_upto_iter(0, len(levels) - 1).tolist() == ocache.get_cache_iter_index_upto_iter(0, len(levels) - 1).tolist()
+    return outs, leaves, rleaves
+
+
+def _deeper_levels(c, seed, n):
+    """n more latent iterations over shrinking subsets of the hard tokens, with projections of their own."""
+    g = torch.Generator().manual_seed(seed)
+    B, Hq, T, D = c["q1"].shape
+    Hkv = c["k1"].shape[1]
+    active, out = c["hard"], []
+    for _ in range(n):
+        active = active & (torch.rand(B, T, generator=g) < 0.6)
+        out.append((active, torch.randn(B, Hq, T, D, generator=g), torch.randn(B, Hkv, T, D, generator=g),
+                    torch.randn(B, Hkv, T, D, generator=g)))
+    return out
+
+
+@pytest.mark.parametrize("left_pad,n_deeper", [(None, 1), ([0, 7], 2)])
+def test_forward_loop_over_three_and_four_depths_matches_dense_reference(emu, left_pad, n_deeper):
+    """The reference's mask and cache take any depth (tah_model.py:788, causal_cache.py:101-158; both deciders default
+    to max_iter = 3): a query at depth d sees the keys of depths 0..d at or before its position."""
+    c = make_dense_case(41, B=2, T=44, p_hard=0.5, Hq=4, Hkv=2, D=128, left_pad=left_pad)
+    deeper = _deeper_levels(c, 42, n_deeper)
+    assert all(int(lv[0].sum()) > 0 for lv in deeper)
+    check_depth_outputs(c, _loops_over_depths(c, deeper)[0])
+
+
+def check_depth_outputs(c, outs):
+    valid = c["valid"].bool()
+    for depth, (o, w, pad) in enumerate(outs):
+        o, w = o.detach().cpu(), w.detach()
+        keep = valid if pad is None else ~pad
+        np.testing.assert_allclose(o[keep].float().numpy(), w[keep].float().numpy(), atol=2e-2, rtol=2e-2, err_msg=f"depth {depth}")
+        assert (o[~keep] == 0).all()
+
+
+def test_forward_loop_over_three_depths_gradients(emu):
+    c = make_dense_case(43, B=2, T=30, p_hard=0.5, Hq=2, Hkv=1, D=128, left_pad=[0, 5])
+    deeper = _deeper_levels(c, 44, 1)
+    check_depth_gradients(c, *_loops_over_depths(c, deeper, requires_grad=True))
+
+
+def check_depth_gradients(c, outs, leaves, rleaves):
+    g = torch.Generator().manual_seed(2)
+    loss = rloss = 0.0
+    for o, w, pad in outs:
+        wt = torch.randn(o.shape, generator=g).to(torch.bfloat16)
+        if pad is not None:
+            wt = torch.where(pad[..., None, None], torch.zeros_like(wt), wt)   # (pad rows: zeros here, anything there)
+        else:
+            wt = torch.where(c["valid"].bool()[..., None, None], wt, torch.zeros_like(wt))
+        loss = loss + (o.float() * wt.float().to(o.device)).sum()
+        rloss = rloss + (w * wt.double()).sum()
+    loss.backward()
+    rloss.backward()
+    for depth, (t, r) in enumerate(zip(leaves, rleaves)):
+        for name, a, b in zip("qkv", t, r):
+            err = (a.grad.float().cpu() - b.grad.float()).abs().max() / b.grad.abs().max().clamp_min(1e-6).float()
+            assert err < 3e-2, (depth, name, float(err))
+
+
+def test_depth_limits(emu):
+    """Negative depths are refused; with the decode path's slabs enabled a cache holds two depths and says so."""
     from tah_amd import TahDuoError
-    from tah_amd.attention import DuoMask, build_attention_mask, duo_attention_forward
+    from tah_amd.attention import build_attention_mask
     from tah_amd.cache import TaHDuoCache
     cache = TaHDuoCache()
     pos, one = torch.arange(4)[None], torch.ones(1, 4, dtype=torch.long)
     with pytest.raises(TahDuoError, match="depth"):
-        build_attention_mask(pos, one, cache, 2)
+        build_attention_mask(pos, one, cache, -1)
     k = torch.zeros(1, 1, 4, 128, dtype=torch.bfloat16)
-    cache.current_iter_depth, cache.position_ids_to_cache, cache.valid_mask_to_cache = 2, pos, one
+    cache.current_iter_depth, cache.position_ids_to_cache, cache.valid_mask_to_cache = -1, pos, one
     with pytest.raises(TahDuoError, match="depth"):
         cache.update(k, k, 0)
-    cache.current_iter_depth = 0
-    cache.update(k, k, 0)
-    with pytest.raises(TahDuoError, match="depth"):
-        duo_attention_forward(_layer(), torch.zeros(1, 2, 4, 128, dtype=torch.bfloat16), k, k, DuoMask(pos, one, cache, 2))
+    slabbed = TaHDuoCache().enable_slabs(8, 8)
+    slabbed.current_iter_depth, slabbed.position_ids_to_cache, slabbed.valid_mask_to_cache = 2, pos, one
+    with pytest.raises(TahDuoError, match="slabs"):
+        slabbed.update(k, k, 0)
 
 
 def test_position_check_switch(emu):
