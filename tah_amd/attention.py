@@ -160,6 +160,15 @@ def _check_depth(iter_depth: int) -> None:
 # ``position_ids`` is None (tah_model.py:555-561); a caller that passes its own position_ids can turn this on.
 CHECK_POSITIONS = False
 
+# What the positions handed to ``build_attention_mask`` are.  True: the rank of a valid token inside its sequence, which
+# the model's forward computes when ``position_ids`` is None (tah_model.py:555-561); depth-0 keys then need no
+# position (it is their index) and the kernels skip the key tiles behind a query tile.  False: plain numbers that the
+# caller chose (tah_model.py:499 hands ``position_ids`` through and :788 compares them as they are): every key then
+# carries its position -- depth-0 rows go through the position-carrying stream as well, any order and any repeats,
+# at the price of visiting every (query tile, key tile) pair of a sequence.  Packed path only: the decode path's
+# depth-0 slabs keep no positions.
+POSITION_IDS_ARE_RANKS = True
+
 
 def _assert_rank_positions(m: "DuoMask") -> None:
     c, B = m.cache, m.position_ids.shape[0]
@@ -178,7 +187,8 @@ def _assert_rank_positions(m: "DuoMask") -> None:
         bad = (((m.position_ids < 0) | (m.position_ids >= total0)) & v).any()
     if bool(bad):
         raise TahDuoError("position_ids are not the valid tokens' ranks inside their sequence; the kernels take the "
-                          "depth-0 position of a token from its index among the valid tokens")
+                          "depth-0 position of a token from its index among the valid tokens "
+                          "(tah_amd.attention.POSITION_IDS_ARE_RANKS = False makes every key carry its position instead)")
 
 
 # ---------------------------------------------------------------------------
@@ -334,16 +344,17 @@ def _merge_plan(m: "DuoMask", segs, B: int):
     return m._merge[1:]
 
 
-def _sparse_keys(m: "DuoMask", cache: TaHDuoCache, layer: int, depth: int, B: int):
-    """The keys a query at ``depth`` >= 1 sees beside the depth-0 ones: every row cached at depths 1 .. depth, packed per
+def _sparse_keys(m: "DuoMask", cache: TaHDuoCache, layer: int, depth: int, B: int, first: int = 1):
+    """The keys a query at ``depth`` >= 1 sees beside the depth-0 ones: every row cached at depths 1 .. depth (``first``
+    = 0: with the depth-0 rows, for positions that are not ranks), packed per
     sequence with their positions -- (k, v, cu, pos, upper bound of a sequence's rows).  The kernels tell depth-0 keys
     (position = index) from keys that carry a position, and among the latter a query sees those at or before its own
     position whatever their depth (tah_model.py:788 with depth_k <= depth_q for all of them), so deeper calls hand the
     kernels the union of these depths as the one sparse key stream; one depth needs no copy."""
-    segs = [_segment(cache, layer, d, B, with_pos=True) for d in range(1, depth + 1) if cache.has_rows(layer, d)]
+    segs = [_segment(cache, layer, d, B, with_pos=True) for d in range(first, depth + 1) if cache.has_rows(layer, d)]
     if not segs:
-        raise TahDuoError(f"no keys cached for layer {layer} at depths 1..{depth}")
-    bound = sum(cache.get_cache_length(layer, d) for d in range(1, depth + 1))
+        raise TahDuoError(f"no keys cached for layer {layer} at depths {first}..{depth}")
+    bound = sum(cache.get_cache_length(layer, d) for d in range(first, depth + 1))
     if len(segs) == 1:
         return segs[0] + (bound,)
     dest, cu, pos = _merge_plan(m, segs, B)
@@ -383,7 +394,7 @@ def duo_attention_forward(module, query: torch.Tensor, key: torch.Tensor, value:
     m = attention_mask
     cache, depth = m.cache, m.iter_depth
     _check_depth(depth)
-    if CHECK_POSITIONS and m._packed is None:
+    if CHECK_POSITIONS and POSITION_IDS_ARE_RANKS and m._packed is None:
         _assert_rank_positions(m)
     if cache is None:
         raise TahDuoError("the DuoMask carries no cache; pass the cache that update() was called on")
@@ -394,6 +405,10 @@ def duo_attention_forward(module, query: torch.Tensor, key: torch.Tensor, value:
 
     # decode fast path: one query row per sequence, slabs hold every cached row (incl. this step's)
     s1 = cache.slabs(layer, 0)
+    ranks = POSITION_IDS_ARE_RANKS
+    if s1 is not None and not ranks:
+        raise TahDuoError("POSITION_IDS_ARE_RANKS = False: position ids of the caller's choosing run on the packed path only "
+                          "(the decode path's depth-0 slabs keep no positions); use a cache without enable_slabs()")
     if Tq == 1 and s1 is not None and depth <= 1 and not (torch.is_grad_enabled() and query.requires_grad):
         # every batch row is a query row; a row that is not valid (a pad row of the depth-1 pack, tah_model.py:116-118)
         # gets position -1, sees nothing and comes back as zeros -- no index to build, nothing read back
@@ -408,27 +423,32 @@ def duo_attention_forward(module, query: torch.Tensor, key: torch.Tensor, value:
 
     # general path: packed varlen forward (+ backward through autograd)
     if m._packed is None:
-        m._packed = _Packed(m.valid_mask, m.position_ids if depth >= 1 else None, B, Tq, dev)
+        m._packed = _Packed(m.valid_mask, m.position_ids if (depth >= 1 or not ranks) else None, B, Tq, dev)
     pq = m._packed
     if not isinstance(pq, _Packed):
         raise TahDuoError("a DuoMask cannot be shared between the decode path and the varlen path")
     q = pq.pack(query)
     zc = torch.zeros(B + 1, dtype=torch.int32, device=dev)
     zi = torch.zeros(0, dtype=torch.int32, device=dev)
-    k1, v1, cu_k1, _ = _segment(cache, layer, 0, B, with_pos=False)
-    Hkv = k1.shape[1]
-    if depth == 0:
-        e_q = q[:0]
+    e_q = q[:0]
+    if depth == 0 and ranks:
+        k1, v1, cu_k1, _ = _segment(cache, layer, 0, B, with_pos=False)
+        Hkv = k1.shape[1]
         e_k = k1[:0]
         sched = _schedule_of(m, (pq.cu, cu_k1, zc, zc, zi, Hq, Hkv, q.shape[0], k1.shape[0], 0))
         o, _ = duo_attn_varlen(q, k1, v1, pq.cu, cu_k1, e_q, e_k, e_k, zi, zi, zc, zc, scale, schedule=sched,
                                max_seqlen_k1=cache.get_cache_length(layer, 0))
     else:
-        k2, v2, cu_k2, pos_k2, bound_k2 = _sparse_keys(m, cache, layer, depth, B)
-        e_q = q[:0]
+        k2, v2, cu_k2, pos_k2, bound_k2 = _sparse_keys(m, cache, layer, depth, B, first=1 if ranks else 0)
+        Hkv = k2.shape[1]
+        if ranks:
+            k1, v1, cu_k1, _ = _segment(cache, layer, 0, B, with_pos=False)
+            bound_k1 = cache.get_cache_length(layer, 0)
+        else:  # no key without a position of its own
+            k1, v1, cu_k1, bound_k1 = k2[:0], v2[:0], zc, 0
         sched = _schedule_of(m, (zc, cu_k1, pq.cu, cu_k2, pq.pos, Hq, Hkv, 0, k1.shape[0], k2.shape[0]))
         _, o = duo_attn_varlen(e_q, k1, v1, zc, cu_k1, q, k2, v2, pq.pos, pos_k2, pq.cu, cu_k2, scale, schedule=sched,
-                               max_seqlen_k1=cache.get_cache_length(layer, 0), max_seqlen_k2=bound_k2)
+                               max_seqlen_k1=bound_k1, max_seqlen_k2=bound_k2)
     return pq.unpack(o, Hq, D), None
 
 

@@ -5,7 +5,7 @@ import torch
 
 from oracle import duo_oracle as O
 from tests.cases import make_dense_case
-from tests.test_host_layer import (_deeper_levels, _forward_two_depths, _forward_two_depths_reference_style, _loops_over_depths,
+from tests.test_host_layer import (_deeper_levels, caller_position_ids, _forward_two_depths, _forward_two_depths_reference_style, _loops_over_depths,
                                    _oracle_two_depths, check_depth_gradients, check_depth_outputs)
 
 pytestmark = pytest.mark.gpu
@@ -120,5 +120,17 @@ def test_forward_loop_over_more_than_two_depths_gpu(B, T, p, left_pad, n_deeper)
     c = make_dense_case(70 + B, B=B, T=T, p_hard=p, left_pad=left_pad)
     deeper = _deeper_levels(c, 71, n_deeper)
     outs, leaves, rleaves = _loops_over_depths(c, deeper, requires_grad=True, device="cuda")
+    check_depth_outputs(c, outs)
+    check_depth_gradients(c, outs, leaves, rleaves)
+
+
+@pytest.mark.parametrize("kind", ["documents", "shuffled"])
+def test_forward_loop_with_position_ids_of_the_callers_choosing_gpu(monkeypatch, kind):
+    """POSITION_IDS_ARE_RANKS off: every key carries its position (tah_model.py:499, :788 with plain numbers)."""
+    import tah_amd.attention as A
+    monkeypatch.setattr(A, "POSITION_IDS_ARE_RANKS", False)
+    c = make_dense_case(80, B=2, T=330, p_hard=0.3, left_pad=[0, 50])
+    ids = caller_position_ids(c, 81, kind)
+    outs, leaves, rleaves = _loops_over_depths(c, _deeper_levels(c, 82, 1), requires_grad=True, device="cuda", position_ids=ids)
     check_depth_outputs(c, outs)
     check_depth_gradients(c, outs, leaves, rleaves)

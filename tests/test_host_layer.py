@@ -275,7 +275,7 @@ def test_slab_overflow_raises_through_cache_update(emu):
     assert int(cache.slabs(0, 0).overflow) == 0 and cache.slabs(0, 0).len.tolist() == [6]
 
 
-def _loops_over_depths(c, deeper, requires_grad=False, device="cpu"):
+def _loops_over_depths(c, deeper, requires_grad=False, device="cpu", position_ids=None):
     """The reference's forward loop (tah_model.py:580-623) over more than two latent iterations, run twice on the same
     bf16 inputs: through this package (TaHDuoCache, DuoMask, duo_attention_forward) and through the dense restatement
     (list cache, dense mask, softmax in float64).  ``deeper``: [(active mask (B, T), q, k, v dense (B, H, T, D)), ...]
@@ -286,7 +286,7 @@ def _loops_over_depths(c, deeper, requires_grad=False, device="cpu"):
     from tah_amd.pack import gather_active
     cache, ocache = TaHDuoCache(), O.OracleCache()
     valid = c["valid"]
-    pos = (torch.cumsum(valid, -1) - 1).clamp(min=0)
+    pos = (torch.cumsum(valid, -1) - 1).clamp(min=0) if position_ids is None else position_ids
     levels = [(None, c["q1"], c["k1"], c["v1"]), (c["hard"], c["q2"], c["k2"], c["v2"])] + list(deeper)
     tok = lambda x: x.transpose(1, 2)
     leaves, rleaves, outs = [], [], []
@@ -371,6 +371,37 @@ def check_depth_gradients(c, outs, leaves, rleaves):
         for name, a, b in zip("qkv", t, r):
             err = (a.grad.float().cpu() - b.grad.float()).abs().max() / b.grad.abs().max().clamp_min(1e-6).float()
             assert err < 3e-2, (depth, name, float(err))
+
+
+def caller_position_ids(c, seed, kind):
+    """Position ids that are not the tokens' ranks: ``documents``: several documents packed into one row, positions
+    starting again at 0 in each; ``shuffled``: a random permutation of the ranks with an offset; ``coarse``: many
+    tokens sharing a position."""
+    g = torch.Generator().manual_seed(seed)
+    B, T = c["valid"].shape
+    rank = (torch.cumsum(c["valid"], -1) - 1).clamp(min=0)
+    if kind == "documents":
+        starts = torch.rand(B, T, generator=g) < 0.08
+        starts[:, 0] = True
+        doc_start = torch.cummax(torch.where(starts, rank, torch.zeros_like(rank)), dim=-1).values
+        return rank - doc_start
+    if kind == "shuffled":
+        return torch.stack([torch.randperm(T, generator=g) for _ in range(B)]) + 5
+    return rank // 7
+
+
+@pytest.mark.parametrize("kind", ["documents", "shuffled", "coarse"])
+def test_forward_loop_with_position_ids_of_the_callers_choosing(emu, monkeypatch, kind):
+    """tah_model.py:499 hands position_ids through and :788 compares them as plain numbers: with
+    POSITION_IDS_ARE_RANKS off every key carries its position and the loop gives what the dense restatement gives
+    with the same ids, over three depths, outputs and gradients."""
+    import tah_amd.attention as A
+    monkeypatch.setattr(A, "POSITION_IDS_ARE_RANKS", False)
+    c = make_dense_case(47, B=2, T=40, p_hard=0.4, Hq=2, Hkv=1, D=128, left_pad=[0, 6])
+    ids = caller_position_ids(c, 48, kind)
+    outs, leaves, rleaves = _loops_over_depths(c, _deeper_levels(c, 49, 1), requires_grad=True, position_ids=ids)
+    check_depth_outputs(c, outs)
+    check_depth_gradients(c, outs, leaves, rleaves)
 
 
 def test_depth_limits(emu):
