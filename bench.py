@@ -484,6 +484,19 @@ def bench_qk_prep(steps: int, warmup: int):
     e1.record()
     torch.cuda.synchronize()
     ms = e0.elapsed_time(e1) / steps
+    # the backward of the preparation (training; no append): q, k and the two output gradients read, dq and dk written
+    from tah_amd import _lib
+    gq, gk = torch.randn_like(t["q"]), torch.randn_like(t["k"])
+    bwd = lambda: _lib.lib().qk_prep_bwd(t["q"], t["k"], gq, gk, t["qw"], t["kw"], t["cos"], t["sin"], c["eps"], 4096)
+    for _ in range(warmup):
+        bwd()
+    e0.record()
+    for _ in range(steps):
+        bwd()
+    e1.record()
+    torch.cuda.synchronize()
+    bwd_ms = e0.elapsed_time(e1) / steps
+    bwd_bytes = rows * (3 * (hq + hkv) * 256 + 2 * 256)
     # per token row: q, k, v read and q, K, V written (256 B per head), cos and sin rows read
     nbytes = rows * (2 * (hq + 2 * hkv) * 256 + 2 * 256)
     gbs = nbytes / (ms * 1e-3) / 1e9
@@ -492,6 +505,8 @@ def bench_qk_prep(steps: int, warmup: int):
             "ms_per_step": ms, "algorithmic_bytes": nbytes, "hbm_gbs": gbs,
             "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
                          "traffic": measured_traffic("qk_prep_prefill"), "kernels": "qk_prep_kernel + kv_append_len_kernel"},
+            "backward": {"kernel": "qk_prep_bwd_kernel", "ms_per_step": bwd_ms, "algorithmic_bytes": bwd_bytes,
+                         "hbm_gbs": bwd_bytes / (bwd_ms * 1e-3) / 1e9, "frac": bwd_bytes / (bwd_ms * 1e-3) / 1e9 / PEAK_HBM_GBS},
             "tokens_per_s": rows / (ms * 1e-3)}
 
 

@@ -318,6 +318,37 @@ typedef struct tah_qk_prep_args {
  * head_dim 128 only.  In-place use (q_out == q, k_out == k) is allowed. */
 int tah_qk_prep(const tah_qk_prep_args* args, tah_stream_t stream);
 
+typedef struct tah_qk_prep_bwd_args {
+    const void* q;           /* bf16 [rows, Hq, D]: what tah_qk_prep was given */
+    const void* k;           /* bf16 [rows, Hkv, D] */
+    const void* dq_out;      /* bf16 [rows, Hq, D]: gradient of tah_qk_prep's q_out */
+    const void* dk_out;      /* bf16 [rows, Hkv, D]: gradient of its k_out */
+    void* dq;                /* bf16 [rows, Hq, D]: gradient of q; may alias dq_out */
+    void* dk;                /* bf16 [rows, Hkv, D]; may alias dk_out */
+    int64_t q_row_stride, q_head_stride, k_row_stride, k_head_stride;
+    int64_t dq_out_row_stride, dq_out_head_stride, dk_out_row_stride, dk_out_head_stride;
+    int64_t dq_row_stride, dq_head_stride, dk_row_stride, dk_head_stride;
+    const void* q_weight;    /* bf16 [D] */
+    const void* k_weight;    /* bf16 [D] */
+    const void* cos;         /* bf16 [rows, D] */
+    const void* sin;         /* bf16 [rows, D] */
+    int64_t cos_sin_row_stride;
+    float eps;
+    int32_t rows, hq, hkv, d;
+    /* float32 [n_partial, 2, D]: row i holds the sums, over the token rows i, i + n_partial, ... and over the heads, of
+     * the gradients of q_weight ([i, 0, :]) and k_weight ([i, 1, :]); every row is written (zeros when n_partial > rows).
+     * The caller adds the rows up (a fixed order: results do not vary from run to run). */
+    float* dw_partial;
+    int32_t n_partial;       /* workgroups to launch, >= 1; a few per compute unit is enough */
+} tah_qk_prep_bwd_args;
+
+/* Backward of tah_qk_prep without append and without a folded input norm: gradients of the projected q and k and of
+ * the two RMSNorm weights, given the gradients of the prepared q and k (V passes through tah_qk_prep unchanged, so
+ * its gradient is the caller's already).  Differentiates Qwen3RMSNorm.forward and apply_rotary_pos_emb
+ * (transformers/models/qwen3/modeling_qwen3.py; third party, pinned 4.52.4 by the reference) in float32 on the bf16
+ * inputs.  head_dim 128 only. */
+int tah_qk_prep_bwd(const tah_qk_prep_bwd_args* args, tah_stream_t stream);
+
 typedef struct tah_topk_mix_args {
     const void* logits;        /* bf16 [rows, vocab], vocab contiguous */
     const void* embedding;     /* bf16 [vocab, hidden], 16-byte aligned rows */

@@ -17,6 +17,9 @@ Pinned in tests/test_oracle_qk_prep.py against the installed transformers' own `
 float32 summation order in the mean), and by what the mathematics fixes: unit weights give rows of
 RMS 1 before the rotation, the rotation keeps the norm of every (i, i + 64) pair up to rounding,
 position 0 (cos = 1, sin = 0) is the identity.
+
+``qk_prep_backward`` is the analytic gradient of the same two steps (no intermediate rounding), float64; pinned in the
+same file against autograd through the installed transformers modules run in float64 and against finite differences.
 """
 import numpy as np
 
@@ -57,3 +60,28 @@ def rotary_tables(positions: np.ndarray, d: int = 128, theta: float = 1e6):
     f = positions.astype(np.float32)[:, None] * inv[None, :]
     emb = np.concatenate([f, f], axis=-1)
     return bf16_round(np.cos(emb).astype(np.float32)), bf16_round(np.sin(emb).astype(np.float32))
+
+
+def qk_prep_backward(q, k, q_weight, k_weight, cos, sin, eps, dq_out, dk_out):
+    """Gradients of ``qk_prep`` (taken as the real-valued function: RMSNorm, weight, rotation): float64
+    ``(dq, dk, dq_weight, dk_weight)`` for output gradients ``dq_out`` [rows, Hq, D], ``dk_out`` [rows, Hkv, D].
+
+    With y = w * xh, xh = x * rs, rs = (mean(x^2) + eps)^(-1/2) and out = y cos + rotate_half(y) sin:
+    dy = g cos + rotate_half^T(g sin) where rotate_half^T(u) = cat(u[64:], -u[:64]); dw = sum dy * xh;
+    dx = rs * (dy w - xh * mean(dy w xh))."""
+    c, s = cos[:, None, :].astype(np.float64), sin[:, None, :].astype(np.float64)
+
+    def one(x, w, g):
+        x, w, g = x.astype(np.float64), w.astype(np.float64), g.astype(np.float64)
+        half = x.shape[-1] // 2
+        rs = 1.0 / np.sqrt(np.mean(x * x, axis=-1, keepdims=True) + eps)
+        xh = x * rs
+        u = g * s
+        dy = g * c + np.concatenate([u[..., half:], -u[..., :half]], axis=-1)
+        dxh = dy * w
+        dx = rs * (dxh - xh * np.mean(dxh * xh, axis=-1, keepdims=True))
+        return dx, (dy * xh).sum(axis=(0, 1))
+
+    dq, dqw = one(q, q_weight, dq_out)
+    dk, dkw = one(k, k_weight, dk_out)
+    return dq, dk, dqw, dkw

@@ -232,6 +232,20 @@ class SampleRowsArgs(C.Structure):
     ]
 
 
+class QkPrepBwdArgs(C.Structure):
+    """``tah_qk_prep_bwd_args``"""
+
+    _fields_ = [
+        ("q", c_void_p), ("k", c_void_p), ("dq_out", c_void_p), ("dk_out", c_void_p), ("dq", c_void_p), ("dk", c_void_p),
+        ("q_row_stride", c_int64), ("q_head_stride", c_int64), ("k_row_stride", c_int64), ("k_head_stride", c_int64),
+        ("dq_out_row_stride", c_int64), ("dq_out_head_stride", c_int64), ("dk_out_row_stride", c_int64), ("dk_out_head_stride", c_int64),
+        ("dq_row_stride", c_int64), ("dq_head_stride", c_int64), ("dk_row_stride", c_int64), ("dk_head_stride", c_int64),
+        ("q_weight", c_void_p), ("k_weight", c_void_p), ("cos", c_void_p), ("sin", c_void_p), ("cos_sin_row_stride", c_int64),
+        ("eps", c_float), ("rows", c_int32), ("hq", c_int32), ("hkv", c_int32), ("d", c_int32),
+        ("dw_partial", c_void_p), ("n_partial", c_int32),
+    ]
+
+
 PROTOTYPES = {
     "tah_duo_abi_version": (C.c_int, []),
     "tah_duo_error_string": (C.c_char_p, [C.c_int]),
@@ -259,6 +273,7 @@ PROTOTYPES = {
     "tah_duo_decode_step": (C.c_int, [C.POINTER(QkPrepArgs), C.POINTER(DuoDecodeArgs), c_void_p, c_void_p, c_void_p]),
     "tah_duo_decode_step_supported": (C.c_int, [c_int32, c_int32, c_int32, c_int32]),
     "tah_topk_mix": (C.c_int, [C.POINTER(TopkMixArgs), c_void_p]),
+    "tah_qk_prep_bwd": (C.c_int, [C.POINTER(QkPrepBwdArgs), c_void_p]),
     "tah_sample_rows": (C.c_int, [C.POINTER(SampleRowsArgs), c_void_p]),
     "tah_silu_mul": (C.c_int, [c_void_p, c_void_p, c_int32, c_int32, c_int64, c_int64, c_void_p]),
     "tah_hard_index_build": (C.c_int, [c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),

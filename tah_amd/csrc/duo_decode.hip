@@ -684,6 +684,106 @@ __global__ __launch_bounds__(256) void qk_prep_kernel(const PrepParams p) {
     }
 }
 
+// ---- backward of the q/k preparation ----------------------------------------------------------------------
+// out = rope(w * x * rsqrt(mean(x^2) + eps)) per head.  With g the gradient of out:
+//   dyn = g cos + partner(g sin), the partner entering with the opposite sign of the forward's (+ for the lower
+//         half of the head, - for the upper one: the transpose of rotate_half);
+//   dw += dyn * xh, xh = x * rs (summed over rows and heads);
+//   dx  = rs * (dyn w - xh * mean(dyn w xh)).
+// Evaluated in float32 on the bf16 inputs (the forward's intermediate roundings are not differentiated through, as
+// in any bf16 backward).  Same lane layout as the forward: 16 lanes per head, partner in lane j ^ 8.  A workgroup
+// walks rows blockIdx.x, blockIdx.x + gridDim.x, ... and leaves its sums of the two weight gradients in its own row
+// of dw_partial (float32 [gridDim.x, 2, 128]): no atomics, the caller adds the rows up.
+struct PrepBwdParams {
+    const __bf16 *q, *k, *dqo, *dko;
+    __bf16 *dq, *dk;
+    int64_t q_rs, q_hs, k_rs, k_hs, dqo_rs, dqo_hs, dko_rs, dko_hs, dq_rs, dq_hs, dk_rs, dk_hs;
+    const __bf16 *qw, *kw, *cos, *sin;
+    int64_t cs_rs;
+    float eps;
+    int32_t rows, hq, hkv;
+    float* dw_partial;
+};
+
+__global__ __launch_bounds__(256) void qk_prep_bwd_kernel(const PrepBwdParams p) {
+    __shared__ float red[2][16][128];
+    const int lane = threadIdx.x % kWave;
+    const int sub = threadIdx.x / 16, j = lane % 16;
+    const int items = p.hq + p.hkv;
+    const u32x4 qw = *reinterpret_cast<const u32x4*>(p.qw + 8 * j), kw = *reinterpret_cast<const u32x4*>(p.kw + 8 * j);
+    float dwq[8], dwk[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dwq[i] = dwk[i] = 0.f;
+    const float psign = j < 8 ? 1.f : -1.f;
+    for (int r = blockIdx.x; r < p.rows; r += gridDim.x) {
+        const u32x4 cs = *reinterpret_cast<const u32x4*>(p.cos + (int64_t)r * p.cs_rs + 8 * j);
+        const u32x4 sn = *reinterpret_cast<const u32x4*>(p.sin + (int64_t)r * p.cs_rs + 8 * j);
+        // (every lane of a wave walks the same number of passes and takes part in every lane exchange)
+        for (int pass = 0; pass * 16 < items; ++pass) {
+            const int it = pass * 16 + sub;
+            const bool is_q = it < p.hq, live = it < items;
+            const int h = is_q ? it : it - p.hq;
+            u32x4 xin = {0u, 0u, 0u, 0u}, gin = {0u, 0u, 0u, 0u};
+            if (live) {
+                xin = *reinterpret_cast<const u32x4*>(is_q ? p.q + (int64_t)r * p.q_rs + (int64_t)h * p.q_hs + 8 * j
+                                                            : p.k + (int64_t)r * p.k_rs + (int64_t)h * p.k_hs + 8 * j);
+                gin = *reinterpret_cast<const u32x4*>(is_q ? p.dqo + (int64_t)r * p.dqo_rs + (int64_t)h * p.dqo_hs + 8 * j
+                                                            : p.dko + (int64_t)r * p.dko_rs + (int64_t)h * p.dko_hs + 8 * j);
+            }
+            const u32x4& w = is_q ? qw : kw;
+            float x[8], g[8], u[8];
+            float ss = 0.f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                x[2 * i] = bf16_lo(xin[i]);
+                x[2 * i + 1] = bf16_hi(xin[i]);
+                g[2 * i] = bf16_lo(gin[i]);
+                g[2 * i + 1] = bf16_hi(gin[i]);
+                u[2 * i] = g[2 * i] * bf16_lo(sn[i]);
+                u[2 * i + 1] = g[2 * i + 1] * bf16_hi(sn[i]);
+                ss += x[2 * i] * x[2 * i] + x[2 * i + 1] * x[2 * i + 1];
+            }
+            ss = row16_sum(ss);
+            const float rs = __builtin_amdgcn_rsqf(ss * (1.0f / 128.0f) + p.eps);
+            float dxh[8], xh[8];
+            float dot = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                // the partner's g sin: lane j ^ 8 of this row of 16 lanes (row rotation by 8)
+                const float pu = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(u[i]), 0x128, 0xf, 0xf, false));
+                const float c = (i % 2) ? bf16_hi(cs[i / 2]) : bf16_lo(cs[i / 2]);
+                const float wi = (i % 2) ? bf16_hi(w[i / 2]) : bf16_lo(w[i / 2]);
+                const float dyn = g[i] * c + psign * pu;
+                xh[i] = x[i] * rs;
+                if (is_q) dwq[i] += dyn * xh[i];
+                else dwk[i] += dyn * xh[i];
+                dxh[i] = dyn * wi;
+                dot += dxh[i] * xh[i];
+            }
+            dot = row16_sum(dot) * (1.0f / 128.0f);
+            u32x4 out;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                out[i] = pack_bf16(rs * (dxh[2 * i] - xh[2 * i] * dot), rs * (dxh[2 * i + 1] - xh[2 * i + 1] * dot));
+            if (live) {
+                __bf16* y = is_q ? p.dq + (int64_t)r * p.dq_rs + (int64_t)h * p.dq_hs : p.dk + (int64_t)r * p.dk_rs + (int64_t)h * p.dk_hs;
+                *reinterpret_cast<u32x4*>(y + 8 * j) = out;
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        red[0][sub][8 * j + i] = dwq[i];
+        red[1][sub][8 * j + i] = dwk[i];
+    }
+    __syncthreads();
+    const int which = threadIdx.x / 128, d = threadIdx.x % 128;
+    float t = 0.f;
+#pragma unroll
+    for (int s_ = 0; s_ < 16; ++s_) t += red[which][s_][d];
+    p.dw_partial[((int64_t)blockIdx.x * 2 + which) * 128 + d] = t;
+}
+
 // ---- q/k preparation, append and attention of a decode step in one launch --------------------------------
 // What qk_prep_kernel (one row per sequence, append) followed by duo_decode_whole_kernel do, for calls the latter
 // takes: the workgroup of (query, kv head) prepares the G query heads and the new K and V of its kv head itself
@@ -1053,6 +1153,40 @@ extern "C" int tah_qk_prep(const tah_qk_prep_args* a, tah_stream_t stream) {
     hipStream_t st = static_cast<hipStream_t>(stream);
     hipLaunchKernelGGL(qk_prep_kernel, dim3(a->rows), dim3(256), 0, st, p);
     if (a->append && !p.own_len) hipLaunchKernelGGL(kv_append_len_kernel, dim3((a->nseq + 63) / 64), dim3(64), 0, st, p.a);
+    return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
+}
+
+extern "C" int tah_qk_prep_bwd(const tah_qk_prep_bwd_args* a, tah_stream_t stream) {
+    using namespace tah;
+    if (!a) return TAH_E_NULL;
+    if (a->d != kD || a->rows < 0 || a->hq <= 0 || a->hkv <= 0 || a->n_partial <= 0) return TAH_E_SHAPE;
+    if (!a->dw_partial) return TAH_E_NULL;
+    if (reinterpret_cast<uintptr_t>(a->dw_partial) & 3) return TAH_E_ALIGN;
+    if (a->rows > 0) {
+        if (!a->q || !a->k || !a->dq_out || !a->dk_out || !a->dq || !a->dk || !a->q_weight || !a->k_weight || !a->cos || !a->sin)
+            return TAH_E_NULL;
+        for (const void* ptr : {a->q, a->k, a->dq_out, a->dk_out, (const void*)a->dq, (const void*)a->dk, a->q_weight, a->k_weight,
+                                a->cos, a->sin})
+            if (!aligned16(ptr)) return TAH_E_ALIGN;
+        for (int64_t st : {a->q_row_stride, a->q_head_stride, a->k_row_stride, a->k_head_stride, a->dq_out_row_stride,
+                           a->dq_out_head_stride, a->dk_out_row_stride, a->dk_out_head_stride, a->dq_row_stride, a->dq_head_stride,
+                           a->dk_row_stride, a->dk_head_stride, a->cos_sin_row_stride})
+            if (st % 8) return TAH_E_ALIGN;
+    }
+    PrepBwdParams p;
+    p.q = static_cast<const __bf16*>(a->q); p.k = static_cast<const __bf16*>(a->k);
+    p.dqo = static_cast<const __bf16*>(a->dq_out); p.dko = static_cast<const __bf16*>(a->dk_out);
+    p.dq = static_cast<__bf16*>(a->dq); p.dk = static_cast<__bf16*>(a->dk);
+    p.q_rs = a->q_row_stride; p.q_hs = a->q_head_stride; p.k_rs = a->k_row_stride; p.k_hs = a->k_head_stride;
+    p.dqo_rs = a->dq_out_row_stride; p.dqo_hs = a->dq_out_head_stride; p.dko_rs = a->dk_out_row_stride; p.dko_hs = a->dk_out_head_stride;
+    p.dq_rs = a->dq_row_stride; p.dq_hs = a->dq_head_stride; p.dk_rs = a->dk_row_stride; p.dk_hs = a->dk_head_stride;
+    p.qw = static_cast<const __bf16*>(a->q_weight); p.kw = static_cast<const __bf16*>(a->k_weight);
+    p.cos = static_cast<const __bf16*>(a->cos); p.sin = static_cast<const __bf16*>(a->sin);
+    p.cs_rs = a->cos_sin_row_stride;
+    p.eps = a->eps;
+    p.rows = a->rows; p.hq = a->hq; p.hkv = a->hkv;
+    p.dw_partial = a->dw_partial;
+    hipLaunchKernelGGL(qk_prep_bwd_kernel, dim3(a->n_partial), dim3(256), 0, static_cast<hipStream_t>(stream), p);
     return hipGetLastError() == hipSuccess ? TAH_OK : TAH_E_LAUNCH;
 }
 

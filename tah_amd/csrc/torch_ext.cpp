@@ -47,6 +47,7 @@ struct Api {
     decltype(&tah_duo_decode_step) decode_step = nullptr;
     decltype(&tah_duo_decode_step_supported) decode_step_supported = nullptr;
     decltype(&tah_topk_mix) topk_mix = nullptr;
+    decltype(&tah_qk_prep_bwd) qk_prep_bwd = nullptr;
     decltype(&tah_sample_rows) sample_rows = nullptr;
     decltype(&tah_silu_mul) silu_mul = nullptr;
     decltype(&tah_hard_index_build) hard_index_build = nullptr;
@@ -93,6 +94,7 @@ void load_library(const std::string& path, bool allow_host) {
     bind(g.decode_step_supported, "tah_duo_decode_step_supported");
     bind(g.topk_mix, "tah_topk_mix");
     bind(g.sample_rows, "tah_sample_rows");
+    bind(g.qk_prep_bwd, "tah_qk_prep_bwd");
     bind(g.silu_mul, "tah_silu_mul");
     bind(g.hard_index_build, "tah_hard_index_build");
     bind(g.pad_rows_build, "tah_pad_rows_build");
@@ -499,6 +501,43 @@ void qk_prep(const Tensor& q, const Tensor& k, const optional<Tensor>& v, const 
     const tah_qk_prep_args a = prep_args(d, q, k, v, q_out, k_out, q_weight, k_weight, cos, sin, eps, ck, cv, cpos, start, len, overflow,
                                          cu_new, pos_new, slot_of, one_row_per_seq, v_out, norm_input, norm_eps);
     check_rc(g.qk_prep(&a, d.stream()), "tah_qk_prep");
+}
+
+// backward of qk_prep (no append, no folded input norm): returns dq, dk (bf16) and the per-workgroup partial sums of the
+// two weight gradients, float32 [n_partial, 2, D]
+std::vector<Tensor> qk_prep_bwd(const Tensor& q, const Tensor& k, const Tensor& dq_out, const Tensor& dk_out, const Tensor& q_weight,
+                                const Tensor& k_weight, const Tensor& cos, const Tensor& sin, double eps, int64_t n_partial) {
+    need_lib();
+    Dev d;
+    thd(q, "q"); thd(k, "k"); thd(dq_out, "dq_out"); thd(dk_out, "dk_out");
+    d.see(q); d.see(k); d.see(dq_out); d.see(dk_out); d.see(q_weight); d.see(k_weight); d.see(cos); d.see(sin);
+    const int64_t D = q.size(2), rows = q.size(0);
+    TORCH_CHECK(dq_out.sizes() == q.sizes() && dk_out.sizes() == k.sizes() && k.size(0) == rows, "qk_prep_bwd: gradient shapes must match q and k");
+    for (auto p : {std::make_pair(&q_weight, "q_weight"), {&k_weight, "k_weight"}})
+        TORCH_CHECK(p.first->scalar_type() == at::kBFloat16 && p.first->dim() == 1 && p.first->size(0) == D && p.first->is_contiguous(),
+                    p.second, " must be a contiguous bf16 [", D, "] tensor");
+    for (auto p : {std::make_pair(&cos, "cos"), {&sin, "sin"}})
+        TORCH_CHECK(p.first->scalar_type() == at::kBFloat16 && p.first->dim() == 2 && p.first->size(0) == rows && p.first->size(1) == D &&
+                        p.first->stride(1) == 1,
+                    p.second, " must be a bf16 [rows, ", D, "] tensor with unit inner stride");
+    TORCH_CHECK(cos.stride(0) == sin.stride(0), "cos and sin must share their row stride");
+    TORCH_CHECK(n_partial >= 1, "qk_prep_bwd: n_partial must be at least 1");
+    Tensor dq = at::empty(q.sizes(), q.options()), dk = at::empty(k.sizes(), k.options());
+    Tensor part = at::empty({n_partial, 2, D}, q.options().dtype(at::kFloat));
+    tah_qk_prep_bwd_args a{};
+    a.q = ptr(q); a.k = ptr(k); a.dq_out = ptr(dq_out); a.dk_out = ptr(dk_out); a.dq = dq.data_ptr(); a.dk = dk.data_ptr();
+    a.q_row_stride = q.stride(0); a.q_head_stride = q.stride(1); a.k_row_stride = k.stride(0); a.k_head_stride = k.stride(1);
+    a.dq_out_row_stride = dq_out.stride(0); a.dq_out_head_stride = dq_out.stride(1);
+    a.dk_out_row_stride = dk_out.stride(0); a.dk_out_head_stride = dk_out.stride(1);
+    a.dq_row_stride = dq.stride(0); a.dq_head_stride = dq.stride(1); a.dk_row_stride = dk.stride(0); a.dk_head_stride = dk.stride(1);
+    a.q_weight = ptr(q_weight); a.k_weight = ptr(k_weight); a.cos = ptr(cos); a.sin = ptr(sin);
+    a.cos_sin_row_stride = cos.stride(0);
+    a.eps = (float)eps;
+    a.rows = (int32_t)rows; a.hq = (int32_t)q.size(1); a.hkv = (int32_t)k.size(1); a.d = (int32_t)D;
+    a.dw_partial = static_cast<float*>(part.data_ptr());
+    a.n_partial = (int32_t)n_partial;
+    check_rc(g.qk_prep_bwd(&a, d.stream()), "tah_qk_prep_bwd");
+    return {dq, dk, part};
 }
 
 bool duo_decode_step_supported(int64_t nq, int64_t hq, int64_t hkv, int64_t capacity1) {
@@ -975,6 +1014,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("rows_copy", &rows_copy);
     m.def("topk_mix", &topk_mix);
     m.def("sample_rows", &sample_rows);
+    m.def("qk_prep_bwd", &qk_prep_bwd);
     m.def("topk_values", &topk_values);
     m.def("silu_mul", &silu_mul);
     m.def("duo_decode_step", &duo_decode_step);

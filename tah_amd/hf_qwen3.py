@@ -5,8 +5,9 @@ reference's base model runs, tah/model/tah_model.py:616-623) does, between the p
 output projection: ``q_norm`` / ``k_norm`` per head, ``apply_rotary_pos_emb``, ``past_key_values.update``
 and the attention-interface call.  :func:`fused_attention_forward` is that method with the norm and
 rotary steps replaced by one ``tah_qk_prep`` launch on the token-major projections and the attention
-call bound to :func:`tah_amd.attention.duo_attention_forward`.  Inference only (the preparation kernel
-has no backward).  Use::
+call bound to :func:`tah_amd.attention.duo_attention_forward`.  Differentiable: under autograd the
+preparation runs as ``tah_qk_prep`` / ``tah_qk_prep_bwd`` and the attention as the varlen forward / backward
+kernels.  Use::
 
     from tah_amd.hf_qwen3 import patch_attention_layers
     patch_attention_layers(model)          # every Qwen3Attention in the model
@@ -18,7 +19,6 @@ from typing import Optional, Tuple
 
 import torch
 
-from ._capi import TahDuoError
 from .attention import duo_attention_forward
 from .kv_cache import qk_norm_rope
 
@@ -30,8 +30,6 @@ def fused_attention_forward(self, hidden_states: torch.Tensor, position_embeddin
     transformers 4.x, ``past_key_values`` of 5.x).  ``attention_mask`` is what
     :func:`tah_amd.attention.build_attention_mask` returned (or the reference's dense additive mask)."""
     del cache_position, kwargs
-    if torch.is_grad_enabled() and hidden_states.requires_grad:
-        raise TahDuoError("fused_attention_forward is for inference: run it under torch.no_grad()")
     cache = past_key_values if past_key_values is not None else past_key_value
     B, T = hidden_states.shape[:2]
     D = self.head_dim

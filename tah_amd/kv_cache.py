@@ -47,6 +47,32 @@ class KvSlabs:
         _call("kv_append", k_new, v_new, cu_new, pos_new, slot_of, self.k, self.v, self.pos, self.start, self.len, self.overflow)
 
 
+class _QkNormRope(torch.autograd.Function):
+    """``tah_qk_prep`` without append, differentiable: backward is one ``tah_qk_prep_bwd`` launch (gradients of q, k and
+    of the two norm weights; cos / sin are tables, not parameters)."""
+
+    # workgroups of the backward launch: each walks every BWD_PARTIALS-th row and leaves one row of partial weight
+    # gradients, which are added up here in a fixed order
+    BWD_PARTIALS = 4096
+
+    @staticmethod
+    def forward(ctx, q, k, q_weight, k_weight, cos, sin, eps):
+        q_out, k_out = torch.empty_like(q), torch.empty_like(k)
+        _call("qk_prep", q, k, None, q_out, k_out, q_weight, k_weight, cos, sin, float(eps), None, None, None, None, None, None,
+              None, None, None, False, None, None, 0.0)
+        ctx.save_for_backward(q, k, q_weight, k_weight, cos, sin)
+        ctx.eps = float(eps)
+        return q_out, k_out
+
+    @staticmethod
+    def backward(ctx, dq_out, dk_out):
+        q, k, q_weight, k_weight, cos, sin = ctx.saved_tensors
+        n = max(1, min(_QkNormRope.BWD_PARTIALS, q.shape[0]))
+        dq, dk, part = _call("qk_prep_bwd", q, k, dq_out.contiguous(), dk_out.contiguous(), q_weight, k_weight, cos, sin, ctx.eps, n)
+        dw = part.sum(0)
+        return dq, dk, dw[0].to(q_weight.dtype), dw[1].to(k_weight.dtype), None, None, None
+
+
 def qk_norm_rope(q: torch.Tensor, k: torch.Tensor, q_weight: torch.Tensor, k_weight: torch.Tensor,
                  cos: torch.Tensor, sin: torch.Tensor, eps: float, *, v: Optional[torch.Tensor] = None,
                  cache: Optional[KvSlabs] = None, cu_new: Optional[torch.Tensor] = None,
@@ -67,7 +93,15 @@ def qk_norm_rope(q: torch.Tensor, k: torch.Tensor, q_weight: torch.Tensor, k_wei
     ``norm_input`` ``[rows, hidden]`` folds the layer's input RMSNorm in: q, k, v are then projections of these
     un-normalised rows through weights that carry the norm's weight, and the kernel multiplies every head by the
     row's ``rsqrt(mean(norm_input**2) + norm_eps)`` first.  Without a cache the scaled V comes back as a third
-    result."""
+    result.
+
+    With gradients enabled and q, k or a weight requiring them (training): the plain form only (no cache, no
+    ``norm_input``, not in place), differentiable through ``tah_qk_prep_bwd``."""
+    if torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, q_weight, k_weight)):
+        if cache is not None or norm_input is not None or in_place:
+            raise _capi.TahDuoError("qk_norm_rope: the differentiable form takes neither a cache to append to, nor a folded "
+                                    "input norm, nor in_place")
+        return _QkNormRope.apply(q, k, q_weight, k_weight, cos, sin, eps)
     q_out = q if in_place else torch.empty_like(q)
     if cache is not None:
         _call("qk_prep", q, k, v, q_out, None, q_weight, k_weight, cos, sin, float(eps), cache.k, cache.v, cache.pos,

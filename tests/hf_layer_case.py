@@ -72,3 +72,47 @@ def run_prefill_then_decode(device, B=2, T=20, steps=2, seed=1):
                 res.append(o.float().cpu())
             outs.append(res)
     return outs
+
+
+def run_training_step(device, B=2, T=37, seed=3):
+    """Forward and backward through one Qwen3Attention module, its own way (eager modules, SDPA, dense mask) and through
+    the fused forward, from the same bf16 parameters: returns (output, gradient of the input, gradients of every
+    parameter by name) for both."""
+    m = pytest.importorskip("transformers.models.qwen3.modeling_qwen3")
+    import copy
+
+    from transformers import Qwen3Config
+
+    from tah_amd.attention import build_attention_mask
+    from tah_amd.cache import TaHDuoCache
+    from tah_amd.hf_qwen3 import fused_attention_forward
+
+    torch.manual_seed(seed)
+    cfg = Qwen3Config(hidden_size=256, num_attention_heads=4, num_key_value_heads=2, head_dim=128, num_hidden_layers=1,
+                      intermediate_size=512, vocab_size=128, rope_theta=1e6, attention_dropout=0.0)
+    cfg._attn_implementation = "sdpa"
+    layer = m.Qwen3Attention(cfg, layer_idx=0).to(device, torch.bfloat16).train()
+    with torch.no_grad():
+        layer.q_norm.weight.copy_(1.0 + 0.1 * torch.randn(128))
+        layer.k_norm.weight.copy_(1.0 + 0.1 * torch.randn(128))
+    fused = copy.deepcopy(layer)
+    rope = m.Qwen3RotaryEmbedding(cfg).to(device)
+    x0 = torch.randn(B, T, 256).to(torch.bfloat16).to(device)
+    w = torch.randn(B, T, 256).to(torch.bfloat16).to(device)
+    pos = torch.arange(T, device=device)[None].expand(B, T)
+    valid = torch.ones(B, T, dtype=torch.long, device=device)
+    with torch.no_grad():
+        cos, sin = rope(x0, pos)
+    out = []
+    for mod, own in ((layer, True), (fused, False)):
+        x = x0.clone().requires_grad_(True)
+        cache = TaHDuoCache()
+        cache.current_iter_depth, cache.position_ids_to_cache, cache.valid_mask_to_cache = 0, pos, valid
+        mask = build_attention_mask(pos, valid, cache, 0)
+        if own:
+            y, _ = mod(x, (cos, sin), mask.dense(torch.bfloat16))
+        else:
+            y, _ = fused_attention_forward(mod, x, (cos, sin), mask, past_key_values=cache)
+        (y.float() * w.float()).sum().backward()
+        out.append((y.detach().float().cpu(), x.grad.float().cpu(), {n: p.grad.float().cpu() for n, p in mod.named_parameters()}))
+    return out

@@ -51,3 +51,36 @@ def folded_norm_case(device, seed=50, rows=6, hq=4, hkv=2, hidden=512):
     t = to_torch(c, device)
     return c, t, torch.from_numpy(x).to(torch.bfloat16).to(device), wq, wk, sc(c["v"])
 
+
+
+def check_backward(device, seed, rows, hq, hkv, scale=1.0, n_partial=None):
+    """``qk_norm_rope`` under autograd (``tah_qk_prep_bwd``) against the analytic float64 gradients of the oracle.  The
+    kernel differentiates in float32 and rounds dq / dk to bf16: error <= 2^-6 of the largest gradient entry of the
+    same head (the RMSNorm's projection couples a head's entries) and <= 1 % of the weight gradients' largest entry."""
+    from tah_amd import kv_cache
+    c = make_case(seed, rows, hq, hkv, scale=scale)
+    t = to_torch(c, device)
+    g = np.random.default_rng(seed + 1)
+    gq = R.bf16_round(g.standard_normal(c["q"].shape).astype(np.float32))
+    gk = R.bf16_round(g.standard_normal(c["k"].shape).astype(np.float32))
+    leaves = [t[n].clone().requires_grad_(True) for n in ("q", "k", "qw", "kw")]
+    if n_partial is not None:
+        old, kv_cache._QkNormRope.BWD_PARTIALS = kv_cache._QkNormRope.BWD_PARTIALS, n_partial
+    try:
+        q_out, k_out = kv_cache.qk_norm_rope(leaves[0], leaves[1], leaves[2], leaves[3], t["cos"], t["sin"], c["eps"])
+        wq, wk = R.qk_prep(c["q"], c["k"], c["qw"], c["kw"], c["cos"], c["sin"], c["eps"])
+        assert_bf16_close(q_out.detach(), wq, "q")
+        assert_bf16_close(k_out.detach(), wk, "k")
+        tg = lambda x: torch.from_numpy(x).to(torch.bfloat16).to(device)
+        torch.autograd.backward([q_out, k_out], [tg(gq), tg(gk)])
+    finally:
+        if n_partial is not None:
+            kv_cache._QkNormRope.BWD_PARTIALS = old
+    want = R.qk_prep_backward(c["q"], c["k"], c["qw"], c["kw"], c["cos"], c["sin"], c["eps"], gq, gk)
+    for name, leaf, w in zip(("dq", "dk"), leaves[:2], want[:2]):
+        got = leaf.grad.float().cpu().numpy().astype(np.float64)
+        bound = np.abs(w).max(axis=-1, keepdims=True) * 2.0 ** -6 + 1e-30
+        assert (np.abs(got - w) <= bound).all(), f"{name}: worst error / head maximum {float((np.abs(got - w) / bound).max()) * 2.0 ** -6:.3e}"
+    for name, leaf, w in zip(("dq_weight", "dk_weight"), leaves[2:], want[2:]):
+        got = leaf.grad.float().cpu().numpy().astype(np.float64)
+        assert np.abs(got - w).max() <= 1e-2 * np.abs(w).max(), f"{name}: {np.abs(got - w).max() / np.abs(w).max():.3e}"

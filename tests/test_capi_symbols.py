@@ -32,7 +32,7 @@ def test_torch_extension_loads_the_library_and_exposes_every_op():
     ext = _lib.lib()
     assert ext.loaded() and ext.abi_version() == _capi.ABI_VERSION
     for n in ("duo_fwd_varlen", "duo_bwd_varlen", "duo_fwd_masked", "duo_bwd_masked", "duo_decode", "decode_workspace_bytes",
-              "kv_append", "qk_prep", "hard_index_build", "pad_rows_build", "rows_copy", "topk_mix", "sample_rows", "silu_mul"):
+              "kv_append", "qk_prep", "hard_index_build", "pad_rows_build", "rows_copy", "topk_mix", "sample_rows", "qk_prep_bwd", "silu_mul"):
         assert callable(getattr(ext, n))
 
 
@@ -48,7 +48,8 @@ def test_struct_sizes_match_c_layout(tmp_path):
              "tah_kv_append_args": _capi.KvAppendArgs, "tah_additive_mask": _capi.AdditiveMask,
              "tah_greedy_step_args": _capi.GreedyStepArgs, "tah_linear_rows_args": _capi.LinearRowsArgs,
              "tah_step_begin_args": _capi.StepBeginArgs, "tah_decider_tail_args": _capi.DeciderTailArgs,
-             "tah_greedy_tick_args": _capi.GreedyTickArgs, "tah_sample_rows_args": _capi.SampleRowsArgs}
+             "tah_greedy_tick_args": _capi.GreedyTickArgs, "tah_sample_rows_args": _capi.SampleRowsArgs,
+             "tah_qk_prep_bwd_args": _capi.QkPrepBwdArgs}
     assert ctypes.sizeof(_capi.DuoStream) == 9 * 8 + 8 * 8 + 2 * 4
     if shutil.which("gcc") is None:
         return

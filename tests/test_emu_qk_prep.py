@@ -106,3 +106,23 @@ def test_argument_checks():
             qk_norm_rope(t["q"], t["k"][:1], t["qw"], t["kw"], t["cos"], t["sin"], 1e-6)
         with pytest.raises(TahDuoError):
             qk_norm_rope(t["q"], t["k"], t["qw"], t["kw"], t["cos"][:, :64], t["sin"][:, :64], 1e-6)
+
+
+@pytest.mark.parametrize("rows,hq,hkv,scale,n_partial", [(5, 4, 2, 1.0, None), (37, 2, 2, 20.0, 4), (3, 8, 1, 0.03, 8), (6, 32, 8, 1.0, 2)])
+def test_backward_matches_analytic_gradients(rows, hq, hkv, scale, n_partial):
+    from tests.qk_prep_cases import check_backward
+    with emu_util.emulated():
+        check_backward("cpu", 60 + rows, rows, hq, hkv, scale=scale, n_partial=n_partial)
+
+
+def test_differentiable_form_refuses_what_it_cannot_differentiate():
+    from tah_amd._capi import TahDuoError
+    from tah_amd.kv_cache import qk_norm_rope
+    c = make_case(70, 3, 2, 1)
+    t = to_torch(c, "cpu")
+    q = t["q"].clone().requires_grad_(True)
+    with emu_util.emulated():
+        with pytest.raises(TahDuoError, match="differentiable"):
+            qk_norm_rope(q, t["k"], t["qw"], t["kw"], t["cos"], t["sin"], c["eps"], in_place=True)
+        with pytest.raises(TahDuoError, match="differentiable"):
+            qk_norm_rope(q, t["k"], t["qw"], t["kw"], t["cos"], t["sin"], c["eps"], norm_input=torch.zeros(3, 16, dtype=torch.bfloat16))

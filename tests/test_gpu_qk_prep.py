@@ -93,3 +93,9 @@ def test_input_norm_folded_in_equals_scaling_the_projections_first_gpu():
     assert float((v_out.float().cpu() == torch.from_numpy(wv)).float().mean()) >= 0.99
     assert torch.allclose(v_out.float().cpu(), torch.from_numpy(wv), rtol=2 ** -7, atol=0)
 
+
+
+@pytest.mark.parametrize("rows,hq,hkv,scale,n_partial", [(1000, 16, 8, 1.0, None), (16384, 16, 8, 1.0, None), (77, 4, 4, 15.0, 16), (5, 32, 8, 0.05, 64)])
+def test_backward_matches_analytic_gradients_gpu(rows, hq, hkv, scale, n_partial):
+    from tests.qk_prep_cases import check_backward
+    check_backward("cuda", 90 + hq, rows, hq, hkv, scale=scale, n_partial=n_partial)

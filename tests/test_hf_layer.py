@@ -3,7 +3,7 @@ import pytest
 import torch
 
 from tests import emu_util
-from tests.hf_layer_case import run, run_prefill_then_decode
+from tests.hf_layer_case import run, run_prefill_then_decode, run_training_step
 
 
 def _check(got, want):
@@ -37,6 +37,29 @@ def test_fused_layer_prefill_then_decode_on_cpu_shim():
 def test_fused_layer_prefill_then_decode_gpu():
     for ref, got in run_prefill_then_decode("cuda", B=3, T=200, steps=3):
         _check(got, ref)
+
+
+def _check_training(outs):
+    """Both runs are bf16 end to end (the module's own backward through eager bf16 modules): gradients agree to 4 % of
+    their largest entry, the norm weights' (sums over every token and head) to 6 %."""
+    (y0, dx0, g0), (y1, dx1, g1) = outs
+    _check(y1, y0)
+    assert (dx1 - dx0).abs().max() <= 4e-2 * dx0.abs().max()
+    assert set(g0) == set(g1) and {"q_norm.weight", "k_norm.weight", "q_proj.weight", "o_proj.weight"} <= set(g0)
+    for n in g0:
+        tol = 6e-2 if "norm" in n else 4e-2
+        assert (g1[n] - g0[n]).abs().max() <= tol * g0[n].abs().max(), (n, float((g1[n] - g0[n]).abs().max() / g0[n].abs().max()))
+
+
+@pytest.mark.skipif(not emu_util.have_host_clang(), reason="host clang++ not available")
+def test_fused_layer_training_step_on_cpu_shim():
+    with emu_util.emulated():
+        _check_training(run_training_step("cpu", B=2, T=21))
+
+
+@pytest.mark.gpu
+def test_fused_layer_training_step_gpu():
+    _check_training(run_training_step("cuda", B=3, T=300))
 
 
 def _check_model(outs):

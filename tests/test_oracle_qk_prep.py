@@ -66,3 +66,34 @@ def test_rotation_keeps_pair_norms_and_composes():
     z = (y[..., :64] + 1j * y[..., 64:]) * (cos[:, None, :64] + 1j * sin[:, None, :64])
     np.testing.assert_allclose(o[..., :64], z.real, atol=0.03, rtol=0.02)
     np.testing.assert_allclose(o[..., 64:], z.imag, atol=0.03, rtol=0.02)
+
+
+def test_backward_against_autograd_through_the_transformers_modules_and_finite_differences():
+    m = pytest.importorskip("transformers.models.qwen3.modeling_qwen3")
+    q, k, qw, kw, cos, sin = _case(7, rows=9, hq=4, hkv=2, scale=2.0)
+    eps = 1e-6
+    g = np.random.default_rng(8)
+    gq, gk = g.standard_normal(q.shape), g.standard_normal(k.shape)
+    qn, kn = m.Qwen3RMSNorm(128, eps=eps).double(), m.Qwen3RMSNorm(128, eps=eps).double()
+    with torch.no_grad():
+        qn.weight.copy_(torch.from_numpy(qw).double()), kn.weight.copy_(torch.from_numpy(kw).double())
+    tq, tk = torch.from_numpy(q).double().requires_grad_(True), torch.from_numpy(k).double().requires_grad_(True)
+    oq, ok = m.apply_rotary_pos_emb(qn(tq).transpose(0, 1)[None], kn(tk).transpose(0, 1)[None],
+                                    torch.from_numpy(cos).double()[None], torch.from_numpy(sin).double()[None])
+    loss = (oq[0].transpose(0, 1) * torch.from_numpy(gq)).sum() + (ok[0].transpose(0, 1) * torch.from_numpy(gk)).sum()
+    loss.backward()
+    dq, dk, dqw, dkw = R.qk_prep_backward(q, k, qw, kw, cos, sin, eps, gq, gk)
+    # (Qwen3RMSNorm computes in float32 whatever it is given: its gradients carry float32 rounding)
+    for got, want in ((dq, tq.grad), (dk, tk.grad), (dqw, qn.weight.grad), (dkw, kn.weight.grad)):
+        np.testing.assert_allclose(got, want.numpy(), rtol=2e-4, atol=2e-5 * float(np.abs(got).max()))
+    # and one entry of each by central differences of the real-valued forward
+    def f(qx, qwx):
+        x = qx.astype(np.float64)
+        y = qwx.astype(np.float64) * x / np.sqrt(np.mean(x * x, -1, keepdims=True) + eps)
+        rot = np.concatenate([-y[..., 64:], y[..., :64]], -1)
+        return ((y * cos[:, None, :].astype(np.float64) + rot * sin[:, None, :].astype(np.float64)) * gq).sum()
+    h = 1e-5
+    e = np.zeros_like(q, dtype=np.float64); e[3, 1, 70] = h
+    assert abs((f(q + e, qw) - f(q - e, qw)) / (2 * h) - dq[3, 1, 70]) < 1e-6 * max(1.0, abs(dq[3, 1, 70]))
+    ew = np.zeros(128); ew[5] = h
+    assert abs((f(q, qw + ew) - f(q, qw - ew)) / (2 * h) - dqw[5]) < 1e-6 * max(1.0, abs(dqw[5]))
