@@ -298,11 +298,17 @@ def bench_host_layer_train_step(seqlens, p_hard: float, seed: int, steps: int, w
     for b, n in enumerate(seqlens):
         valid[b, :n] = 1  # right-padded rows
     hard = (torch.rand(B, T, generator=g) < p_hard) & valid.bool()
-    mk = lambda h: [(torch.randn(B, T, h, D, generator=g) * 0.5).to(torch.bfloat16).cuda().requires_grad_(True) for _ in range(layers)]
-    q1, k1, v1, q2, k2, v2 = mk(Hq), mk(Hkv), mk(Hkv), mk(Hq), mk(Hkv), mk(Hkv)
+    W = int(hard.sum(-1).max())  # width of the second iteration's pack: the most hard tokens of a row
+    mk = lambda n, h: [(torch.randn(B, n, h, D, generator=g) * 0.5).to(torch.bfloat16).cuda().requires_grad_(True) for _ in range(layers)]
+    # the projections of every layer as its q / k / v linears leave them: of all tokens at the first iteration, of the
+    # packed hard tokens at the second (the model gathers the hidden states once per iteration, tah_model.py:600-603,
+    # and every layer projects the gathered rows)
+    q1, k1, v1, q2, k2, v2 = mk(T, Hq), mk(T, Hkv), mk(T, Hkv), mk(W, Hq), mk(W, Hkv), mk(W, Hkv)
+    hidden = (torch.randn(B, T, 2048, generator=g) * 0.5).to(torch.bfloat16).cuda().requires_grad_(True)
     valid, hard = valid.cuda(), hard.cuda()
     pos = (torch.cumsum(valid, -1) - 1).clamp(min=0)
     w1 = torch.randn(B, T, Hq, D, generator=g).to(torch.bfloat16).cuda()
+    wx = torch.randn(B, T, 2048, generator=g).to(torch.bfloat16).cuda()
     mods = [types.SimpleNamespace(layer_idx=l, num_key_value_groups=Hq // Hkv) for l in range(layers)]
     scale = D ** -0.5
     # the bare launches on the same rows, packed (one call serves both iterations)
@@ -323,16 +329,17 @@ def bench_host_layer_train_step(seqlens, p_hard: float, seed: int, steps: int, w
             k, v = cache.update(k1[l].transpose(1, 2), v1[l].transpose(1, 2), l)
             outs.append(duo_attention_forward(mods[l], q1[l].transpose(1, 2), k, v, m0, scaling=scale)[0])
         # second iteration: the hard tokens, packed per row (one index for all layers, as the model's loop has it)
-        packed = gather_active(hard, pos, valid, *q2, *k2, *v2)
-        pos2, val2 = packed[1], packed[2]
-        gq, gk, gv = packed[3:3 + layers], packed[3 + layers:3 + 2 * layers], packed[3 + 2 * layers:]
+        _, pos2, val2, x2 = gather_active(hard, pos, valid, hidden)
+        outs.append(x2)
+        gq, gk, gv = q2, k2, v2
         m1 = build_attention_mask(pos2, val2, cache, 1, dtype=torch.bfloat16)
         cache.current_iter_depth, cache.position_ids_to_cache, cache.valid_mask_to_cache = 1, pos2, val2
         for l in range(layers):
             k, v = cache.update(gk[l].transpose(1, 2), gv[l].transpose(1, 2), l)
             outs.append(duo_attention_forward(mods[l], gq[l].transpose(1, 2), k, v, m1, scaling=scale)[0])
-        torch.autograd.backward(outs, [w1[:, : o.shape[1]] for o in outs])  # upstream gradients as given (no loss arithmetic)
-        for t in q1 + k1 + v1 + q2 + k2 + v2:
+        # upstream gradients as given (no loss arithmetic); the gathered hidden rows get theirs too (the scatter back)
+        torch.autograd.backward(outs, [w1[:, : o.shape[1]] if o.dim() == 4 else wx[:, : o.shape[1]] for o in outs])
+        for t in q1 + k1 + v1 + q2 + k2 + v2 + [hidden]:
             t.grad = None
 
     def bare_step():
@@ -355,8 +362,8 @@ def bench_host_layer_train_step(seqlens, p_hard: float, seed: int, steps: int, w
     host_ms, bare_ms = timed(host_step), timed(bare_step)
     return {"workload": f"configs[3] as the host layer sees it: {B} rows padded to {T}, valid lengths {list(seqlens)}, "
                         f"p_hard={p_hard}, {layers} attention layers x 2 latent iterations, forward + backward",
-            "path": "build_attention_mask -> TaHDuoCache.update -> duo_attention_forward (both iterations) -> loss.backward(); "
-                    "wall clock, includes the packing of valid / hard rows and autograd's own kernels",
+            "path": "build_attention_mask -> TaHDuoCache.update -> duo_attention_forward (both iterations; gather_active of the hidden "
+                    "states once for the second) -> backward(); wall clock, includes the packing of valid rows and autograd's own kernels",
             "ms_per_step": host_ms, "ms_per_layer": host_ms / layers,
             "bare_launches_ms_per_step": bare_ms, "bare_launches_ms_per_layer": bare_ms / layers,
             "ratio_to_bare_launches": host_ms / bare_ms, "layers": layers}

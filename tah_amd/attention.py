@@ -202,6 +202,10 @@ def _rows(x: torch.Tensor) -> torch.Tensor:
     return x.transpose(1, 2).reshape(B * T, H, D)
 
 
+# Blocks of at most this many rows are packed without reading their valid count back (see _Packed).
+NO_SYNC_ROWS = 4096
+
+
 class _Packed:
     """Valid-row packing of one (B, T) block: row ids, per-sequence offsets, int32 positions.
 
@@ -218,7 +222,9 @@ class _Packed:
             raise TahDuoError(f"positions of shape {tuple(pos.shape)} for a block of {B} x {T} rows")
         all_valid = valid is None
         if not all_valid:
-            idx = HardIndex(valid)
+            # a small block (the packed hard tokens of a step) is packed by its upper bound, B * T rows: reading the count
+            # back would stall the host on everything queued so far to save copying a few pad rows
+            idx = HardIndex.of(valid, sync=None if B * T > NO_SYNC_ROWS else False)
             all_valid = idx.synced and idx.n == B * T
         if all_valid:
             self.rows, self.n = None, B * T
@@ -304,7 +310,17 @@ def _segment(cache: TaHDuoCache, layer_idx: int, depth: int, B: int, with_pos: b
                 cache._key_memo.clear()
             cache._key_memo[key] = memo
         pk = memo[2]
-        return pk.pack(k), pk.pack(v), pk.cu, pk.pos
+        # The packed rows themselves are kept per (layer, depth): the calls of later depths attend over the same chunk,
+        # and under autograd their gradients then meet at the packed tensor (one scatter back, not one per call).
+        # (Training only: without gradients the copy would only hold memory for as long as the cache lives.)
+        if pk.rows is None or not (torch.is_grad_enabled() and (k.requires_grad or v.requires_grad)):
+            return pk.pack(k), pk.pack(v), pk.cu, pk.pos
+        slot = (layer_idx, depth)
+        kept = cache._kv_packed.get(slot)
+        if kept is None or kept[0] is not k or kept[1] is not v or kept[2] is not pk or kept[3] != (k._version, v._version):
+            kept = (k, v, pk, (k._version, v._version), pk.pack(k), pk.pack(v))
+            cache._kv_packed[slot] = kept
+        return kept[4], kept[5], pk.cu, pk.pos
     k = torch.cat([c[0] for c in chunks], dim=2)
     v = torch.cat([c[1] for c in chunks], dim=2)
     T = k.shape[2]

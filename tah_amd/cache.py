@@ -55,6 +55,7 @@ class TaHDuoCache:
         self._slab_rows: Dict[_Slot, int] = {}  # host-side upper bound on the rows any slab of the slot holds
         self._pack_memo: Dict[int, Any] = {}
         self._key_memo: Dict[Any, Any] = {}     # packed key segments of single-chunk slots, per (layer-independent) valid mask
+        self._kv_packed: Dict[Any, Any] = {}    # per (layer, depth): the slot's one chunk packed, for the calls of later depths
 
     # ── native storage ────────────────────────────────────────────────────
     def enable_slabs(self, capacity_depth0: int, capacity_depth1: int) -> "TaHDuoCache":
@@ -107,7 +108,7 @@ class TaHDuoCache:
                 cu = torch.arange(0, (B + 1) * T, T, dtype=torch.int32, device=k.device)
                 memo = (valid, None, cu, B * T, None)
             else:
-                idx = HardIndex(valid)
+                idx = HardIndex.of(valid)
                 if idx.synced and idx.n == B * T:
                     memo = (valid, None, torch.arange(0, (B + 1) * T, T, dtype=torch.int32, device=k.device), B * T, None)
                 else:

@@ -23,6 +23,13 @@ from ._capi import TahDuoError
 HOST_SYNC = True
 
 
+# The index of a mask is asked for several times within one model step (queries and keys of an attention call pack by
+# the same valid mask; scatter_back follows gather_active with the same mask): the last few are kept, keyed by the
+# mask tensor itself and its version counter, so that each mask is compacted -- and its count read back -- once.
+_INDEX_MEMO: list = []
+_INDEX_MEMO_SIZE = 6
+
+
 class HardIndex:
     """Packed-varlen index of a (B, S) boolean mask, built on the device.
 
@@ -34,6 +41,19 @@ class HardIndex:
     count, ``count`` is the count on the device (one int32) and pos / flat / seq keep
     their full capacity (entries past the count are undefined).
     """
+
+    @classmethod
+    def of(cls, mask: torch.Tensor, sync: Optional[bool] = None) -> "HardIndex":
+        """The index of ``mask``: the one built earlier for this very tensor (same object, not written to since, same
+        read-back mode) or a new one."""
+        want = HOST_SYNC if sync is None else bool(sync)
+        for key, version, idx in _INDEX_MEMO:
+            if key is mask and version == mask._version and idx.synced == want:
+                return idx
+        idx = cls(mask, sync=sync)
+        _INDEX_MEMO.append((mask, mask._version, idx))
+        del _INDEX_MEMO[:-_INDEX_MEMO_SIZE]
+        return idx
 
     def __init__(self, mask: torch.Tensor, sync: Optional[bool] = None):
         if mask.dim() != 2:
@@ -134,7 +154,7 @@ def gather_active(current_iter_mask: torch.Tensor, *tensors, pad_value=0, max_ac
     dev = current_iter_mask.device
     if max_active is None and not HOST_SYNC:
         raise TahDuoError("gather_active: with tah_amd.pack.HOST_SYNC = False the packed width must be given (max_active)")
-    idx = HardIndex(current_iter_mask, sync=max_active is None)
+    idx = HardIndex.of(current_iter_mask, sync=max_active is None)
     B, S = idx.B, idx.S
     overflow = None
     if max_active is None:
@@ -177,7 +197,7 @@ def scatter_back(current_iter_mask: torch.Tensor, src: torch.Tensor, dest: torch
     ``HOST_SYNC``): the count of active positions stays on the device; a row of ``src`` narrower than the row's
     active positions then drops the surplus instead of raising.
     """
-    idx = HardIndex(current_iter_mask, sync=host_sync)
+    idx = HardIndex.of(current_iter_mask, sync=host_sync)
     B, S = idx.B, idx.S
     W = src.shape[1]
     if idx.synced and W < idx.width:

@@ -11,7 +11,7 @@ from tests.test_host_layer import (_deeper_levels, caller_position_ids, _forward
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("B,T,p,left_pad", [(2, 300, 0.1, None), (3, 200, 0.2, [0, 37, 150]), (1, 512, 0.06, None)])
+@pytest.mark.parametrize("B,T,p,left_pad", [(2, 300, 0.1, None), (3, 200, 0.2, [0, 37, 150]), (1, 512, 0.06, None), (2, 2300, 0.1, [0, 700])])
 def test_forward_loop_matches_dense_reference_gpu(B, T, p, left_pad):
     from tah_amd.cache import TaHDuoCache
     c = make_dense_case(50 + B, B=B, T=T, p_hard=p, left_pad=left_pad)

@@ -164,9 +164,12 @@ def test_forward_loop_with_launch_order_table(emu, monkeypatch):
     assert all(t[k].grad is not None for k in ("q1", "k1", "v1"))
 
 
-@pytest.mark.parametrize("left_pad", [None, [0, 9]])
-def test_forward_loop_matches_dense_reference(emu, left_pad):
+@pytest.mark.parametrize("left_pad,no_sync_rows", [(None, 4096), ([0, 9], 4096), ([0, 9], 0)])
+def test_forward_loop_matches_dense_reference(emu, monkeypatch, left_pad, no_sync_rows):
+    """(no_sync_rows = 0: every block reads its valid count back and packs to it, as large blocks do.)"""
+    import tah_amd.attention as A
     from tah_amd.cache import TaHDuoCache
+    monkeypatch.setattr(A, "NO_SYNC_ROWS", no_sync_rows)
     c = make_dense_case(31, B=2, T=40, p_hard=0.25, Hq=4, Hkv=2, D=128, left_pad=left_pad)
     cache = TaHDuoCache()
     _, o1, o2, pad = _forward_two_depths(c, cache)
