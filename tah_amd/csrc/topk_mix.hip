@@ -4,10 +4,13 @@
 //
 // One workgroup (1024 threads) per row.  The row's logits (bf16) are loaded once into registers as
 // order-preserving 16-bit keys; the keys that can be among the k largest (those at or above the k-th largest
-// thread maximum) are collected in LDS; the k-th largest key is found by bisection on the 16-bit key space with
-// a block-wide count per step (no histogram atomics, no sort), ties at the threshold are broken towards the
-// lower vocabulary index by a second bisection on the index, the <= k selected (index, value) pairs are
-// gathered into LDS and ordered by index (so that the float sums below have one fixed order), and the mix is
+// thread maximum) are collected in LDS.  Up to 512 of them (a few more than k on anything but a flat row) are
+// ranked against each other directly -- larger key first, equal keys by ascending index, ncand^2 comparisons
+// spread over the workgroup -- and the k first are the selection, already in output order.  More candidates:
+// the k-th largest key is found by bisection on the 16-bit key space with a block-wide count per step (no
+// histogram atomics, no sort) and ties at the threshold are broken towards the lower vocabulary index by a second
+// bisection on the index.  The <= k selected (index, value) pairs are
+// ordered by index (so that the float sums below have one fixed order), and the mix is
 // accumulated in float over bf16-rounded products, as the bf16 eager arithmetic it replaces rounds them.
 #include <hip/hip_runtime.h>
 
@@ -22,7 +25,10 @@ constexpr int kMixThreads = 1024;
 constexpr int kMixWaves = kMixThreads / kWave;
 constexpr int kMaxTopk = 256;
 constexpr int kMaxCand = 2048;  // keys that reach the lower bound of the k-th largest (two per thread)
+constexpr int kPairMax = 512;   // up to this many candidates are ranked against each other directly (the usual case)
 constexpr int kMaxVec = 19;  // 16-byte pieces of the row per thread: vocabularies up to 19 * 8 * 1024 = 155648
+
+typedef float f32x4s __attribute__((ext_vector_type(4)));
 
 struct MixParams {
     const __bf16* logits;
@@ -98,7 +104,10 @@ __global__ __launch_bounds__(kMixThreads) void topk_mix_kernel(const MixParams p
     __shared__ int sel_idx[kMaxTopk];
     __shared__ float sel_val[kMaxTopk];
     __shared__ int ord_idx[kMaxTopk];
-    __shared__ float ord_w[kMaxTopk];
+    __shared__ __align__(16) float ord_w[kMaxTopk];
+    __shared__ unsigned long long cand64[kPairMax];  // (key, -index) of a candidate as one number: larger = earlier
+    __shared__ int cand_rank[kPairMax];
+    __shared__ int ord_rank[kMaxTopk];
     __shared__ int n_sel;
     __shared__ uint16_t cand_key[kMaxCand];
     __shared__ int cand_idx[kMaxCand];
@@ -121,6 +130,11 @@ __global__ __launch_bounds__(kMixThreads) void topk_mix_kernel(const MixParams p
     const int k = p.topk < V ? p.topk : V;
     const __bf16* lrow = p.logits + (int64_t)row * p.l_rs;
     if (tid < 3 * kSearchRows * 16) (&tot[0][0])[tid] = 0;  // the searches' counters
+    if (tid < kMaxTopk) {
+        ord_w[tid] = 0.f;  // (entries past the selected ones are read as zeros by the sum of four at a time)
+        ord_rank[tid] = 0;
+    }
+    if (tid < kPairMax) cand_rank[tid] = 0;
     __syncthreads();
 
     // ---- the row as keys: piece j of thread t covers indices (j * 1024 + t) * 8 .. + 7 (coalesced loads) ----
@@ -211,7 +225,33 @@ __global__ __launch_bounds__(kMixThreads) void topk_mix_kernel(const MixParams p
     }
     __syncthreads();
     const int ncand = n_cand;
-    if (ncand <= kMaxCand) {
+    const bool sorted = ncand <= kPairMax;  // (uniform) the selected entries end up in output order right away
+    if (sorted) {
+        // Few candidates (a few more than k on anything but a flat row): every candidate's place in the order --
+        // larger key first, equal keys by ascending index -- is the number of candidates that come before it,
+        // ncand^2 comparisons spread over the workgroup; the k first are the selection, already in output order.
+        if (tid < ncand) cand64[tid] = ((unsigned long long)cand_key[tid] << 32) | (uint32_t)(0x7fffffff - cand_idx[tid]);
+        __syncthreads();
+        int cp = 64;
+        while (cp < ncand) cp <<= 1;
+        const int nsl = kMixThreads / cp, c = tid & (cp - 1), sl = tid / cp;
+        if (c < ncand) {
+            const unsigned long long mine = cand64[c];
+            int r = 0;
+#pragma unroll 4
+            for (int i = sl; i < ncand; i += nsl) r += cand64[i] > mine ? 1 : 0;
+            if (r) atomicAdd(&cand_rank[c], r);
+        }
+        __syncthreads();
+        if (tid < ncand) {
+            const int r = cand_rank[tid];
+            if (r < k) {
+                sel_idx[r] = cand_idx[tid];
+                sel_val[r] = key_value(cand_key[tid]);
+            }
+        }
+        if (tid == 0) n_sel = k;  // (count(key >= L) >= k)
+    } else if (ncand <= kMaxCand) {
         // this thread's candidates (key 0: none)
         uint32_t ck[kMaxCand / kMixThreads];
         int ci[kMaxCand / kMixThreads];
@@ -331,24 +371,45 @@ __global__ __launch_bounds__(kMixThreads) void topk_mix_kernel(const MixParams p
         // largest first, equal values by ascending index: place = how many selected entries come before this one
         const float mine = sel_val[tid];
         const int mine_idx = sel_idx[tid];
-        int place = 0;
-        for (int i = 0; i < n; ++i) place += (sel_val[i] > mine) || (sel_val[i] == mine && sel_idx[i] < mine_idx);
+        int place = sorted ? tid : 0;
+        if (!sorted)
+            for (int i = 0; i < n; ++i) place += (sel_val[i] > mine) || (sel_val[i] == mine && sel_idx[i] < mine_idx);
         p.vals[(int64_t)row * p.v_rs + place] = (__bf16)mine;  // (exact: the value came from a bf16)
         if (p.idxs) p.idxs[(int64_t)row * p.v_rs + place] = mine_idx;
     }
     if (!p.out) return;  // only the values were asked for (uniform)
     // order by index (all distinct): rank = number of selected entries with a smaller index
     float vmax = kNegInf;
-    for (int i = 0; i < n; ++i) vmax = fmaxf(vmax, sel_val[i]);
+    if (sorted) vmax = sel_val[0];
+    else
+        for (int i = 0; i < n; ++i) vmax = fmaxf(vmax, sel_val[i]);
+    {   // rank by index among the selected, the comparisons spread over the workgroup
+        int cp = 64;
+        while (cp < n) cp <<= 1;
+        const int nsl = kMixThreads / cp, c = tid & (cp - 1), sl = tid / cp;
+        if (c < n) {
+            const int mine_idx = sel_idx[c];
+            int r = 0;
+#pragma unroll 4
+            for (int i = sl; i < n; i += nsl) r += sel_idx[i] < mine_idx ? 1 : 0;
+            if (r) atomicAdd(&ord_rank[c], r);
+        }
+    }
+    __syncthreads();
     if (tid < n) {
-        int rank = 0;
-        for (int i = 0; i < n; ++i) rank += sel_idx[i] < sel_idx[tid];
+        const int rank = ord_rank[tid];
         ord_idx[rank] = sel_idx[tid];
         ord_w[rank] = fast_exp2((sel_val[tid] - vmax) * kLog2e);
     }
     __syncthreads();
-    float denom = 0.f;
-    for (int i = 0; i < n; ++i) denom += ord_w[i];  // same order in every thread and every run
+    float denom = 0.f;  // same order in every thread and every run; four at a time, zeros past the end
+    for (int i = 0; i < n; i += 4) {
+        const f32x4s w4 = *reinterpret_cast<const f32x4s*>(&ord_w[i]);
+        denom += w4[0];
+        denom += w4[1];
+        denom += w4[2];
+        denom += w4[3];
+    }
     const float inv = 1.0f / denom;
 
     // ---- mix: thread = (part, column group of 8); a part takes every parts-th selected row ----
