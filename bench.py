@@ -570,6 +570,10 @@ def bench_sample_rows(steps: int, warmup: int, vocab: int = 151936, temperature:
     logits = [(torch.randn(1024, vocab, generator=g) * 3).to(torch.bfloat16).cuda() for _ in range(2)]  # two sets in rotation
     u = torch.rand(1024, generator=g).cuda()
     out = torch.zeros(1024, dtype=torch.int64, device="cuda")
+    # rows with a language model's range: the bulk of the vocabulary around -2 +- 2.5, twenty tokens 22 to 30 above it
+    lm = torch.randn(32, vocab, generator=g) * 2.5 - 2.0
+    lm.scatter_add_(1, torch.randint(0, vocab, (32, 20), generator=g), 22.0 + 8.0 * torch.rand(32, 20, generator=g))
+    lm = lm.to(torch.bfloat16).cuda()
     yield
 
     def timed(f, n):
@@ -586,11 +590,13 @@ def bench_sample_rows(steps: int, warmup: int, vocab: int = 151936, temperature:
 
     ms32 = timed(lambda i: ops.sample_rows(logits[i % 2][:32], u[:32], temperature, top_p=top_p, out=out[:32]), steps)
     torch32 = timed(lambda i: TaHDecodeEngine.sample(logits[i % 2][:32].float(), temperature, top_p=top_p), max(3, steps // 4))
+    ms32_lm = timed(lambda i: ops.sample_rows(lm, u[:32], temperature, top_p=top_p, out=out[:32]), steps)
     ms1024 = timed(lambda i: ops.sample_rows(logits[i % 2], u, temperature, top_p=top_p, out=out), steps)
     nbytes = 1024 * vocab * 2
     gbs = nbytes / (ms1024 * 1e-3) / 1e9
     return {"workload": f"temperature {temperature} / top_p {top_p} draw without a top-k filter, rows of {vocab} bf16 logits",
             "ms_per_step_32_rows": ms32, "torch_ms_per_step_32_rows": torch32,
+            "ms_per_step_32_rows_with_a_language_models_range": ms32_lm,
             "ms_per_step": ms1024, "rows": 1024, "algorithmic_bytes": nbytes, "hbm_gbs": gbs,
             "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
                          "traffic": None, "kernels": "sample_rows_kernel<19, false>"},

@@ -2,7 +2,8 @@
 //
 // A row of bf16 logits has at most 65536 distinct values, and a token's probability depends on its value only.
 // So the row is loaded once into registers as order-preserving 16-bit keys and counted into a histogram over
-// the key space (LDS, 32768 keys at a time, nearest to the row maximum last); the mass of a key is its count
+// the key space (LDS, 32768 keys at a time: the half nearest to the row maximum, then the far half unless its tokens
+// are too light to change a float32 sum); the mass of a key is its count
 // times exp((value - max) / T), a prefix sum over the keys in descending order gives the mass that precedes every
 // key in the order a descending sort would put the tokens in, and both the top_p cut (the first token whose
 // preceding mass exceeds top_p of the total) and the draw (the token at which the preceding kept mass passes
@@ -229,9 +230,14 @@ __global__ __launch_bounds__(kSmpThreads) void sample_rows_kernel(const SamplePa
         total = tot;
     };
 
-    // far window first, so that the near one (where cut and draw fall on all but flat rows) stays in LDS
+    // The far window is needed only if its tokens can change a float32 sum: each of them weighs at most the mass of the
+    // first key behind the near window, the near window weighs at least 1 (the largest token), and when all V of them
+    // together stay below 2^-26 (a language model's row: the far window starts tens of e-foldings below the maximum)
+    // the total is the near window's to the last bit, no far token can precede the cut, and the draw cannot reach one.
+    // Otherwise the far window goes first, so that the near one (where cut and draw fall on all but flat rows) is
+    // the one that stays in LDS.
     float mass1 = 0.f, excl1 = 0.f, total1 = 0.f;
-    if (dmax >= (uint32_t)kWinKeys) {  // (uniform)
+    if (dmax >= (uint32_t)kWinKeys && (float)V * mass_of(kmax - (uint32_t)kWinKeys) > 1.4901161e-8f) {  // (uniform)
         build_hist(kWinKeys);
         scan_window(kWinKeys, mass1, excl1, total1);
         __syncthreads();  // the scan's reads of the histogram are done before it is cleared
@@ -239,17 +245,18 @@ __global__ __launch_bounds__(kSmpThreads) void sample_rows_kernel(const SamplePa
     float mass0, excl0, total0;
     build_hist(0u);
     scan_window(0u, mass0, excl0, total0);
+    constexpr int lds_window = 0;  // which window's histogram LDS holds
     const float S = total0 + total1;  // mass of everything min_p keeps
     const float g0 = excl0, g1 = total0 + excl1;  // mass before this thread's group, window 0 / window 1
 
     // Counts of group `code` (window code >> 10, thread code & 1023): from the histogram in LDS, or counted again.
     auto group_counts = [&](int code) -> const uint32_t* {
         const int gt = code & (kSmpThreads - 1);
-        if ((code >> 10) == 0) return hist + gt * (kBinsPerThread + 1);
+        if ((code >> 10) == lds_window) return hist + gt * (kBinsPerThread + 1);
         __syncthreads();  // earlier readers of mini are done
         if (tid < kBinsPerThread) mini[tid] = 0u;
         __syncthreads();
-        const uint32_t gbase = (uint32_t)kWinKeys + (uint32_t)gt * kBinsPerThread;
+        const uint32_t gbase = (uint32_t)(code >> 10) * (uint32_t)kWinKeys + (uint32_t)gt * kBinsPerThread;
         const uint32_t span = dmax - gbase < (uint32_t)kBinsPerThread - 1u ? dmax - gbase : (uint32_t)kBinsPerThread - 1u;
         const uint32_t kb = kmax - gbase;  // rel = kb - key
 #pragma unroll
@@ -348,9 +355,21 @@ __global__ __launch_bounds__(kSmpThreads) void sample_rows_kernel(const SamplePa
         __syncthreads();  // earlier readers of wv are done
         if (tid < kSmpMaxVec * kSmpWaves) (&wv[0][0])[tid] = 0;
         __syncthreads();
+        const uint32_t kk = key | (key << 16);
 #pragma unroll
         for (int j = 0; j < NVEC; ++j) {
-            int c = __builtin_popcount(match_mask(keys[j], key));
+            // a 16-bit half of w ^ kk that is zero: a match (the usual zero-half test, exact for the lower half and
+            // never silent about a match; the full mask is formed only where there may be one)
+            uint32_t hit = 0u;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                uint32_t w = keys[j][q];
+                TAH_OPAQUE1(w);
+                const uint32_t x = w ^ kk;
+                hit |= (x - 0x00010001u) & ~x & 0x80008000u;
+            }
+            if (__ballot(hit != 0u) == 0ull) continue;
+            int c = hit ? __builtin_popcount(match_mask(keys[j], key)) : 0;
             if (__ballot(c != 0) == 0ull) continue;
 #pragma unroll
             for (int m = 32; m >= 1; m >>= 1) c += __shfl_xor(c, m);
