@@ -340,7 +340,8 @@ inline __host__ __device__ int sched_slots(int nseq, int bm, int total_1, int to
     return (total_1 > 0 ? total_1 / bm + nseq : 0) + (total_2 > 0 ? total_2 / bm + nseq : 0);
 }
 
-// Looks launch slot `idx` up in the table if the table was built for this call's sizes and this kernel's grid.
+// Looks launch slot `idx` up in the table if the table was built for this call's sizes and this kernel's grid
+// (sizes are all that is compared: a table for other boundaries of the same sizes would be taken at its word).
 // Returns 0: no usable table (the caller falls back to the arithmetic order), 1: tile found, -1: slot without a tile.
 __device__ __forceinline__ int sched_lookup(const int32_t* sched, bool key_tiles, int nseq, int group, int total_q1,
                                             int total_q2, int total_k1, int total_k2, int slots, int idx, bool& second,

@@ -7,8 +7,9 @@
 // tiles out longest-first is the classic remedy, and with several documents in a batch it needs an order across
 // documents, which depends on the sequence boundaries on the device: one 1024-thread workgroup builds it with a
 // counting sort (tile steps are small integers) and the kernels read their tile from the table instead of
-// deriving it from blockIdx.  Integer work, no host read-back; the table only changes the order in which tiles
-// are started, never a result.
+// deriving it from blockIdx.  Integer work, no host read-back; a table built from the call's own boundaries only
+// changes the order in which tiles are started, never a result (one built from other boundaries of the same
+// sizes is not detected by the kernels: the caller rebuilds it whenever the boundaries change).
 #include <hip/hip_runtime.h>
 
 #include "duo_device.h"
