@@ -100,11 +100,12 @@ int tah_duo_fwd_varlen(const tah_duo_fwd_args* args, tah_stream_t stream);
  * attention calls take; pass the table as `schedule` to tah_duo_fwd_varlen / tah_duo_bwd_varlen as long as
  * nseq, the totals, hq / hkv and the contents of cu_* and pos_q2 stay what they were when it was built
  * (one table serves every layer and the backward pass of a batch).  A table whose sizes (nseq, the totals,
- * hq / hkv) differ from a call's is ignored by that call.  One built for other boundaries with the same
- * sizes is NOT detected: the kernels would then work on tiles that do not match the call's sequences and
- * leave rows unwritten -- build a new table whenever cu_* change (one small launch, 0.015 ms for the four
- * sequences of a 16 384-token batch).  A matching table changes the order in which tiles are started, never a
- * result; tiles of equal weight are listed in no particular order, which can differ between two builds.
+ * hq / hkv) differ from a call's is ignored by that call.  The table is a permutation of the tile numbers, which
+ * the kernels turn into tiles from the call's own boundaries: it changes the order in which tiles are started,
+ * never a result -- one built for other boundaries of the same sizes still makes a call visit each of its tiles
+ * once, only no longer heaviest first (build a new one when cu_* change: one small launch, 0.015 ms for the four
+ * sequences of a 16 384-token batch).  Tiles of equal weight are listed in no particular order, which can differ
+ * between two builds.
  * No counterpart in the reference, whose SDPA call launches a dense rectangular problem
  * (transformers/integrations/sdpa_attention.py:79-166). */
 typedef struct tah_duo_schedule_args {

@@ -140,18 +140,13 @@ __global__ __launch_bounds__(kDqThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dq_
 
     int seq = 0, row0 = 0, row_end = 0;
     bool second = false;
-    const int listed = sched_lookup(p.sched, false, p.nseq, G, p.s1.total_q, p.s2.total_q, p.s1.total_k, p.s2.total_k,
-                                    (int)gridDim.y, (int)blockIdx.y, second, seq, row0);
-    if (listed < 0) return;
-    if (listed > 0) {  // the table's order: heaviest tile of the whole call first
-        const int hi = const_i32(second ? p.s2.cu_q : p.s1.cu_q, seq + 1);
-        row_end = row0 + BM < hi ? row0 + BM : hi;
-    } else {
-        int slot = (int)(gridDim.y - 1 - blockIdx.y);  // late (heavy) tiles of each sequence first
-        if (!(p.s1.total_q > 0 && find_tile(p.s1.cu_q, p.nseq, BM, slot, seq, row0, row_end))) {
-            if (!(p.s2.total_q > 0 && find_tile(p.s2.cu_q, p.nseq, BM, slot, seq, row0, row_end))) return;
-            second = true;
-        }
+    int slot = (int)(gridDim.y - 1 - blockIdx.y);  // without a table: late (heavy) tiles of each sequence first
+    // (the table's order: heaviest tile of the whole call first)
+    sched_lookup(p.sched, false, p.nseq, G, p.s1.total_q, p.s2.total_q, p.s1.total_k, p.s2.total_k, (int)gridDim.y,
+                 (int)blockIdx.y, slot);
+    if (!(p.s1.total_q > 0 && find_tile(p.s1.cu_q, p.nseq, BM, slot, seq, row0, row_end))) {
+        if (!(p.s2.total_q > 0 && find_tile(p.s2.cu_q, p.nseq, BM, slot, seq, row0, row_end))) return;
+        second = true;
     }
     const BwdStream& qs = second ? p.s2 : p.s1;
     const int head = hk * G + wave % G;
@@ -376,18 +371,13 @@ __global__ __launch_bounds__(kKvThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dkd
 
     int seq = 0, key0 = 0, key_end = 0;
     bool second = false;
-    const int listed = sched_lookup(p.sched, true, p.nseq, G, p.s1.total_q, p.s2.total_q, p.s1.total_k, p.s2.total_k,
-                                    (int)gridDim.y, (int)blockIdx.y, second, seq, key0);
-    if (listed < 0) return;
-    if (listed > 0) {  // the table's order: the key tile seen by the most query rows first
-        const int hi = const_i32(second ? p.s2.cu_k : p.s1.cu_k, seq + 1);
-        key_end = key0 + kBK < hi ? key0 + kBK : hi;
-    } else {
-        int slot = (int)blockIdx.y;  // early (heavy) key tiles of each sequence first
-        if (!(p.s1.total_k > 0 && find_tile(p.s1.cu_k, p.nseq, kBK, slot, seq, key0, key_end))) {
-            if (!(p.s2.total_k > 0 && find_tile(p.s2.cu_k, p.nseq, kBK, slot, seq, key0, key_end))) return;
-            second = true;
-        }
+    int slot = (int)blockIdx.y;  // without a table: early (heavy) key tiles of each sequence first
+    // (the table's order: the key tile seen by the most query rows first)
+    sched_lookup(p.sched, true, p.nseq, G, p.s1.total_q, p.s2.total_q, p.s1.total_k, p.s2.total_k, (int)gridDim.y,
+                 (int)blockIdx.y, slot);
+    if (!(p.s1.total_k > 0 && find_tile(p.s1.cu_k, p.nseq, kBK, slot, seq, key0, key_end))) {
+        if (!(p.s2.total_k > 0 && find_tile(p.s2.cu_k, p.nseq, kBK, slot, seq, key0, key_end))) return;
+        second = true;
     }
     const BwdStream& ks = second ? p.s2 : p.s1;
     const int k_lo = ks.cu_k[seq];
@@ -823,18 +813,13 @@ __global__ __launch_bounds__(kLqThreads) TAH_WAVES_PER_EU(2, 2) void duo_bwd_dq_
 
     int seq = 0, row0 = 0, row_end = 0;
     bool second = false;
-    const int listed = sched_lookup(p.sched, false, p.nseq, G, p.s1.total_q, p.s2.total_q, p.s1.total_k, p.s2.total_k,
-                                    (int)gridDim.y, (int)blockIdx.y, second, seq, row0);
-    if (listed < 0) return;
-    if (listed > 0) {
-        const int hi = const_i32(second ? p.s2.cu_q : p.s1.cu_q, seq + 1);
-        row_end = row0 + BM < hi ? row0 + BM : hi;
-    } else {
-        int slot = (int)(gridDim.y - 1 - blockIdx.y);  // late (heavy) tiles of each sequence first
-        if (!(p.s1.total_q > 0 && find_tile(p.s1.cu_q, p.nseq, BM, slot, seq, row0, row_end))) {
-            if (!(p.s2.total_q > 0 && find_tile(p.s2.cu_q, p.nseq, BM, slot, seq, row0, row_end))) return;
-            second = true;
-        }
+    int slot = (int)(gridDim.y - 1 - blockIdx.y);  // without a table: late (heavy) tiles of each sequence first
+    // (the table's order: heaviest tile of the whole call first)
+    sched_lookup(p.sched, false, p.nseq, G, p.s1.total_q, p.s2.total_q, p.s1.total_k, p.s2.total_k, (int)gridDim.y,
+                 (int)blockIdx.y, slot);
+    if (!(p.s1.total_q > 0 && find_tile(p.s1.cu_q, p.nseq, BM, slot, seq, row0, row_end))) {
+        if (!(p.s2.total_q > 0 && find_tile(p.s2.cu_q, p.nseq, BM, slot, seq, row0, row_end))) return;
+        second = true;
     }
     const BwdStream& qs = second ? p.s2 : p.s1;
     const int q_lo = const_i32(qs.cu_q, seq);

@@ -327,7 +327,11 @@ __device__ __forceinline__ bool find_tile(const int32_t* cu, int nseq, int bm, i
 // by the number of tile steps they run, heaviest first, so that a launch of few, unequal workgroups per
 // compute unit ends with the light ones.  int32 words: a header, then one (x, y) pair per launch slot of
 // the query-tile kernels (forward, dQ), then one pair per slot of the key-tile kernel (dK/dV).
-//   x = sequence | (depth-1 stream ? 1 << 30 : 0), or -1 for a slot without a tile;  y = first row
+//   x = the tile's number in the order find_tile counts them (the depth-0 stream's tiles sequence by sequence, then
+//       the depth-1 stream's); y = 0 (reserved).
+// Every number below the list's length appears exactly once (those past the last tile at the end), so whatever
+// boundaries a call has, walking the list visits each of its tiles once: a table built for other boundaries of the
+// same sizes costs the intended order, never a tile.
 // ---------------------------------------------------------------------------
 constexpr int32_t kSchedMagic = 0x54414853;
 constexpr int kSchedHeaderWords = 16;
@@ -340,25 +344,21 @@ inline __host__ __device__ int sched_slots(int nseq, int bm, int total_1, int to
     return (total_1 > 0 ? total_1 / bm + nseq : 0) + (total_2 > 0 ? total_2 / bm + nseq : 0);
 }
 
-// Looks launch slot `idx` up in the table if the table was built for this call's sizes and this kernel's grid
-// (sizes are all that is compared: a table for other boundaries of the same sizes would be taken at its word).
-// Returns 0: no usable table (the caller falls back to the arithmetic order), 1: tile found, -1: slot without a tile.
-__device__ __forceinline__ int sched_lookup(const int32_t* sched, bool key_tiles, int nseq, int group, int total_q1,
-                                            int total_q2, int total_k1, int total_k2, int slots, int idx, bool& second,
-                                            int& seq, int& row0) {
-    if (!sched) return 0;
+// The tile number that launch slot `idx` takes from the table, if the table was built for this call's sizes and this
+// kernel's grid (true); otherwise the caller keeps its own order (false).
+__device__ __forceinline__ bool sched_lookup(const int32_t* sched, bool key_tiles, int nseq, int group, int total_q1,
+                                             int total_q2, int total_k1, int total_k2, int slots, int idx, int& slot) {
+    if (!sched) return false;
     if (const_i32(sched, 0) != kSchedMagic || const_i32(sched, kSchedNseq) != nseq || const_i32(sched, kSchedGroup) != group ||
         const_i32(sched, kSchedTotalQ1) != total_q1 || const_i32(sched, kSchedTotalQ2) != total_q2 ||
         const_i32(sched, kSchedTotalK1) != total_k1 || const_i32(sched, kSchedTotalK2) != total_k2 ||
         const_i32(sched, key_tiles ? kSchedKSlots : kSchedQSlots) != slots)
-        return 0;
+        return false;
     const int base = kSchedHeaderWords + (key_tiles ? 2 * const_i32(sched, kSchedQSlots) : 0);
     const int x = const_i32(sched, base + 2 * idx);
-    if (x < 0) return -1;
-    second = (x >> 30) & 1;
-    seq = x & 0x3fffffff;
-    row0 = const_i32(sched, base + 2 * idx + 1);
-    return 1;
+    if (x < 0 || x >= slots) return false;  // (not a table this library wrote)
+    slot = x;
+    return true;
 }
 
 }  // namespace tah

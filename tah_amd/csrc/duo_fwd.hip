@@ -112,16 +112,19 @@ __global__ __launch_bounds__(64 * W) TAH_WAVES_PER_EU(2, 2) void duo_fwd_kernel(
     bool second = false;
     // (the launch-order table lists tiles of 256 / G rows: a 4-wave workgroup takes one half of an entry)
     constexpr int kPerEntry = 8 / W;
-    const int listed = sched_lookup(p.sched, false, p.nseq, G, p.s1.total_q, p.s2.total_q, p.s1.total_k, p.s2.total_k,
-                                    (int)gridDim.y / kPerEntry, (int)blockIdx.y / kPerEntry, second, seq, row0);
-    if (listed < 0) return;
-    if (listed > 0) {  // the table's order: heaviest tile of the whole call first
-        const int hi = const_i32(second ? p.s2.cu_q : p.s1.cu_q, seq + 1);
+    int slot;
+    if (sched_lookup(p.sched, false, p.nseq, G, p.s1.total_q, p.s2.total_q, p.s1.total_k, p.s2.total_k,
+                     (int)gridDim.y / kPerEntry, (int)blockIdx.y / kPerEntry, slot)) {
+        // the table's order: heaviest tile of the whole call first; its tiles have kPerEntry * BM rows
+        if (!(p.s1.total_q > 0 && find_tile(p.s1.cu_q, p.nseq, kPerEntry * BM, slot, seq, row0, row_end))) {
+            if (!(p.s2.total_q > 0 && find_tile(p.s2.cu_q, p.nseq, kPerEntry * BM, slot, seq, row0, row_end))) return;
+            second = true;
+        }
         row0 += BM * ((int)blockIdx.y % kPerEntry);
-        if (row0 >= hi) return;
-        row_end = row0 + BM < hi ? row0 + BM : hi;
+        if (row0 >= row_end) return;
+        row_end = row0 + BM < row_end ? row0 + BM : row_end;
     } else {
-        int slot = (int)(gridDim.y - 1 - blockIdx.y);  // late (heavy) tiles of each sequence first
+        slot = (int)(gridDim.y - 1 - blockIdx.y);  // late (heavy) tiles of each sequence first
         if (!(p.s1.total_q > 0 && find_tile(p.s1.cu_q, p.nseq, BM, slot, seq, row0, row_end))) {
             if (!(p.s2.total_q > 0 && find_tile(p.s2.cu_q, p.nseq, BM, slot, seq, row0, row_end))) return;
             second = true;

@@ -8,8 +8,9 @@
 // documents, which depends on the sequence boundaries on the device: one 1024-thread workgroup builds it with a
 // counting sort (tile steps are small integers) and the kernels read their tile from the table instead of
 // deriving it from blockIdx.  Integer work, no host read-back; a table built from the call's own boundaries only
-// changes the order in which tiles are started, never a result (one built from other boundaries of the same
-// sizes is not detected by the kernels: the caller rebuilds it whenever the boundaries change).
+// changes the order in which tiles are started, never a result: the table is a permutation of the tile numbers, which
+// the kernels turn into tiles from the call's own boundaries, so even one built from other boundaries of the same
+// sizes makes them visit every tile once (in an order that is no longer the intended one).
 #include <hip/hip_runtime.h>
 
 #include "duo_device.h"
@@ -129,12 +130,12 @@ __device__ void build_list(const SchedParams& p, const int32_t* cu_a, int total_
         locate(t, second, b, i);
         const int at = atomicAdd(&bins[sort_key(second, b, i)], 1);  // ties land in arrival order: same steps either way
         if (at < slots) {
-            out[2 * at] = b | (second ? 1 << 30 : 0);
-            out[2 * at + 1] = (second ? cu_b[b] : cu_a[b]) + i * tile;
+            out[2 * at] = t;  // the tile's number in sequence order, which the kernels turn into (sequence, first row)
+            out[2 * at + 1] = 0;
         }
     }
-    for (int t = n + tid; t < slots; t += kSchedThreads) {
-        out[2 * t] = -1;
+    for (int t = n + tid; t < slots; t += kSchedThreads) {  // numbers without a tile (for these boundaries) come last
+        out[2 * t] = t;
         out[2 * t + 1] = 0;
     }
     __syncthreads();

@@ -28,6 +28,17 @@ def _schedule(ops, dev, hq, hkv):
                             dev["q1"].shape[0], dev["k1"].shape[0], dev["k2"].shape[0])
 
 
+def _tiles_in_order(cu_a, cu_b, tile):
+    """(stream, sequence, first row) of every tile in the order the kernels count them: the depth-0 stream's tiles
+    sequence by sequence, then the depth-1 stream's."""
+    out = []
+    for second, cu in ((0, cu_a), (1, cu_b)):
+        for b in range(len(cu) - 1):
+            for r in range(int(cu[b]), int(cu[b + 1]), tile):
+                out.append((second, b, r))
+    return out
+
+
 def _expected_tiles(cu_a, cu_b, tile):
     want = set()
     for second, cu in ((0, cu_a), (1, cu_b)):
@@ -60,14 +71,17 @@ def _check_table(table, case, hq, hkv):
     for lst, n, tile, cu_a, cu_b in ((t[HEADER:HEADER + 2 * nq], nq, bm, case["cu_q1"], case["cu_q2"]),
                                      (t[HEADER + 2 * nq:], nk, 128, case["cu_k1"], case["cu_k2"])):
         x, y = lst[0::2], lst[1::2]
-        used = x >= 0
+        tiles = _tiles_in_order(cu_a, cu_b, tile)
+        # a permutation of the tile numbers 0 .. n-1: whatever the boundaries, every tile is visited once
+        assert sorted(x.tolist()) == list(range(n)) and not y.any()
+        used = x < len(tiles)
         n_used = int(used.sum())
-        assert used[:n_used].all() and not used[n_used:].any()  # slots without a tile come last
-        got = [(int(v >> 30) & 1, int(v & 0x3fffffff), int(r)) for v, r in zip(x[:n_used], y[:n_used])]
+        assert n_used == len(tiles) and used[:n_used].all()  # numbers without a tile come last
+        got = [tiles[int(v)] for v in x[:n_used]]
         assert len(set(got)) == len(got) and set(got) == _expected_tiles(cu_a, cu_b, tile)
     # query tiles: the keys a tile has to walk over never grow along the list (in 64-key steps)
-    x, y = t[HEADER:HEADER + 2 * nq:2], t[HEADER + 1:HEADER + 2 * nq:2]
-    steps = [-(-_visible_pairs_q(case, int(v >> 30) & 1, int(v & 0x3fffffff), int(r), bm) // 64) for v, r in zip(x, y) if v >= 0]
+    tiles = _tiles_in_order(case["cu_q1"], case["cu_q2"], bm)
+    steps = [-(-_visible_pairs_q(case, *tiles[int(v)], bm) // 64) for v in t[HEADER:HEADER + 2 * nq:2] if v < len(tiles)]
     # a depth-1 tile also walks every 64-key tile of its depth-1 segment, which rounds up separately from the
     # depth-0 part: allow one step of slack against the straight count
     assert all(a >= b - 1 for a, b in zip(steps, steps[1:])), steps
@@ -126,6 +140,32 @@ def test_a_table_built_for_other_sizes_is_ignored():
         stale = ops.duo_fwd_varlen(*varlen_args(dev_b), schedule=table_a)
     for a, b in zip(plain, stale):
         assert torch.equal(a, b)
+
+
+@pytest.mark.skipif(not emu_util.have_host_clang(), reason="host clang++ not available")
+def test_a_table_built_for_other_boundaries_of_the_same_sizes_changes_no_result():
+    """Packed training: the same number of tokens every step, new document boundaries.  A table from another step has
+    the call's sizes and is taken; being a permutation of the tile numbers it still makes the kernels visit every tile
+    of the call's own boundaries once (also when these have more tiles than the table's had)."""
+    from tah_amd import ops
+    mk = lambda seed, lens: _to_dev(make_varlen_case(seed, lens, 0.0, Hq=2, Hkv=1, D=128))
+    dev_a, dev_b = mk(3, [256, 128, 128]), mk(4, [100, 130, 282])   # 512 rows each: 4 query tiles against 5
+    g = torch.Generator().manual_seed(5)
+    do1 = torch.randn(dev_b["q1"].shape, generator=g).to(torch.bfloat16)
+    with emu_util.emulated():
+        table_a = _schedule(ops, dev_a, 2, 1)
+        assert table_a is not None
+        plain = ops.duo_fwd_varlen(*varlen_args(dev_b))
+        stale = ops.duo_fwd_varlen(*varlen_args(dev_b), schedule=table_a)
+        for a, b in zip(plain, stale):
+            assert torch.equal(a, b)
+        o1, lse1, o2, lse2 = plain
+        bwd = lambda s, ws: ops.duo_bwd_varlen(dev_b["q1"], dev_b["k1"], dev_b["v1"], o1, lse1, do1, dev_b["cu_q1"], dev_b["cu_k1"],
+                                               dev_b["q2"], dev_b["k2"], dev_b["v2"], o2, lse2, do1[:0], dev_b["pos_q2"], dev_b["pos_k2"],
+                                               dev_b["cu_q2"], dev_b["cu_k2"], dev_b["scale"], schedule=s, ds_workspace=ws)
+        for ws in (None, False):
+            for a, b in zip(bwd(None, ws), bwd(table_a, ws)):
+                assert torch.equal(a, b)
 
 
 @pytest.mark.skipif(not emu_util.have_host_clang(), reason="host clang++ not available")
