@@ -469,15 +469,19 @@ def duo_attention_forward(module, query: torch.Tensor, key: torch.Tensor, value:
 
 
 # Calls with at least this many (query row, kv head) pairs get a launch-order table: below it a launch has about
-# one workgroup per compute unit and the order does not matter.
+# one workgroup per compute unit and the order does not matter.  Nor does it for a batch of short sequences (every tile
+# runs a step or two; measured: 64 x 128 tokens lose 25 % of the forward to the table, 16 x 512 gain 12 % of the
+# backward): the table is for batches whose sequences average at least SCHEDULE_MIN_MEAN_ROWS query rows.
 SCHEDULE_MIN_ROW_HEADS = 49152
+SCHEDULE_MIN_MEAN_ROWS = 256
 
 
 def _schedule_of(m: "DuoMask", args):
     """The launch-order table of this mask's varlen calls: built at the first layer, shared by the others (the
     boundaries of queries and cached keys are the same in every layer of a step) and by the backward pass."""
     cu_q1, cu_k1, cu_q2, cu_k2, pos_q2, hq, hkv, tq1, tk1, tk2 = args
-    if (tq1 + pos_q2.shape[0]) * hkv < SCHEDULE_MIN_ROW_HEADS:
+    rows, nseq = tq1 + pos_q2.shape[0], max(1, cu_k1.numel() - 1)
+    if rows * hkv < SCHEDULE_MIN_ROW_HEADS or rows < SCHEDULE_MIN_MEAN_ROWS * nseq:
         return None
     key = (tq1, tk1, pos_q2.shape[0], tk2, hq, hkv, cu_k1.data_ptr(), cu_k2.data_ptr())
     memo = getattr(m, "_sched", None)

@@ -307,17 +307,37 @@ __device__ __forceinline__ int32_t const_i32(const int32_t* a, int i) { return (
 // Locate tile `slot` among sequences whose lengths are cu[b+1]-cu[b], `bm` rows
 // per tile.  On success fills seq/row0/row_end and returns true; otherwise
 // subtracts the number of tiles in this stream from `slot` and returns false.
+// Every lane of the wave must call it with the same arguments: the lanes take 64 sequences at a time (one pair of
+// loads and a prefix sum over the lanes), so that a batch of hundreds of short sequences costs a workgroup a few
+// steps and not one scalar load pair per sequence.
 __device__ __forceinline__ bool find_tile(const int32_t* cu, int nseq, int bm, int& slot, int& seq, int& row0, int& row_end) {
-    for (int b = 0; b < nseq; ++b) {
-        const int lo = const_i32(cu, b), hi = const_i32(cu, b + 1);
+    const int lane = (int)(threadIdx.x % kWave);
+    for (int b0 = 0; b0 < nseq; b0 += kWave) {
+        const int b = b0 + lane;
+        int lo = 0, hi = 0;
+        if (b < nseq) {
+            lo = cu[b];
+            hi = cu[b + 1];
+        }
         const int n = (hi - lo + bm - 1) / bm;
-        if (slot < n) {
-            seq = b;
-            row0 = lo + slot * bm;
-            row_end = row0 + bm < hi ? row0 + bm : hi;
+        int incl = n;  // tiles of sequences b0 .. b
+#pragma unroll
+        for (int o = 1; o < kWave; o <<= 1) {
+            const int v = __shfl_up(incl, o);
+            if (lane >= o) incl += v;
+        }
+        const int tot = __builtin_amdgcn_readfirstlane(__shfl(incl, kWave - 1));
+        if (slot < tot) {
+            const int src = __builtin_ctzll(__ballot(slot < incl));  // the first sequence whose tiles reach past `slot`
+            const int lo_s = __builtin_amdgcn_readfirstlane(__shfl(lo, src));
+            const int hi_s = __builtin_amdgcn_readfirstlane(__shfl(hi, src));
+            const int before = __builtin_amdgcn_readfirstlane(__shfl(incl - n, src));
+            seq = b0 + src;
+            row0 = lo_s + (slot - before) * bm;
+            row_end = row0 + bm < hi_s ? row0 + bm : hi_s;
             return true;
         }
-        slot -= n;
+        slot -= tot;
     }
     return false;
 }
