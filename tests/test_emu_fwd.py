@@ -42,6 +42,7 @@ def _check(dev, got):
     (2, 1, [70], 0.3),           # G=2, one partial tile, depth-1 rows
     (2, 2, [130, 3], 0.1),       # G=1, 256-row tiles, second tiny sequence
     (4, 1, [65, 64], 0.2),       # G=4, 64-row tiles
+    (2, 1, [3, 0, 9, 1] * 17 + [40], 0.3),   # 69 sequences: the tile lookup takes them 64 at a time
 ])
 def test_fwd_kernel_on_cpu_shim(hq, hkv, seqlens, p):
     from tah_amd import ops

@@ -54,6 +54,29 @@ def test_random_shape_forward_and_backward(seed):
             assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("hq,hkv,seqlens,p", [
+    (4, 2, [32] * 150 + [0] * 3 + [100] * 20, 0.2),        # 173 sequences: the tile lookup takes them 64 at a time
+    (2, 1, [1, 7, 0, 130] * 40 + [500], 0.3),              # 161 ragged ones, empty ones among them
+])
+def test_many_short_sequences_forward_and_backward(hq, hkv, seqlens, p):
+    from tah_amd import ops
+    dev = to_device(make_varlen_case(77, seqlens, p, Hq=hq, Hkv=hkv, D=128))
+    out = ops.duo_fwd_varlen(*varlen_args(dev))
+    o1, lse1, o2, lse2 = oracle_fwd(dev)
+    assert_close(out[0], o1, "o1")
+    assert_close(out[2], o2, "o2")
+    np.testing.assert_allclose(out[1].cpu().numpy(), lse1, atol=5e-3, rtol=1e-3)
+    got, want = run_bwd(dev, 78)
+    check_grads(got, want)
+    sched = ops.duo_schedule(dev["cu_q1"], dev["cu_k1"], dev["cu_q2"], dev["cu_k2"], dev["pos_q2"], hq, hkv,
+                             dev["q1"].shape[0], dev["k1"].shape[0], dev["k2"].shape[0])
+    for a, b in zip(out, ops.duo_fwd_varlen(*varlen_args(dev), schedule=sched)):
+        assert torch.equal(a, b)
+    got2, _ = run_bwd(dev, 78, schedule=sched)
+    for a, b in zip(got, got2):
+        assert torch.equal(a, b)
+
+
 def _draw_decode(seed):
     g = np.random.default_rng(seed)
     hkv = int(g.choice([1, 2, 4, 8]))
