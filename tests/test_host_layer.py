@@ -157,6 +157,7 @@ def test_forward_loop_with_launch_order_table(emu, monkeypatch):
     real = ops.duo_schedule
     monkeypatch.setattr(ops, "duo_schedule", lambda *a: built.append(1) or real(*a))
     monkeypatch.setattr(attention, "SCHEDULE_MIN_ROW_HEADS", 0)
+    monkeypatch.setattr(attention, "SCHEDULE_MIN_MEAN_ROWS", 0)
     cache = TaHDuoCache()
     t, o1, o2, _ = _forward_two_depths(c, cache, requires_grad=True)
     assert len(built) == 2 and torch.equal(o1, w1) and torch.equal(o2, w2)
