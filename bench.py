@@ -520,16 +520,42 @@ def bench_qk_prep(steps: int, warmup: int):
 def bench_topk_mix(steps: int, warmup: int, rows: int = 1024, vocab: int = 151936, hidden: int = 2048, topk: int = 100):
     """Next-iteration input of hard tokens (tah_model.py:57-75): top-100 softmax mix of embedding rows for `rows` rows of
     the full vocabulary, and the top-k logit values alone (the decider's features, iter_decider.py:281) next to
-    torch.topk on the same rows.  Per row the kernel reads the logits once and k embedding rows."""
+    torch.topk on the same rows.  Per row the kernel reads the logits once and k embedding rows.  Also the learned
+    decider's whole decision (iter_decider.py:265-301) for the 32 rows of a generation step, replayed from a graph as the
+    engine runs it: its dense layers on tah_linear_rows, and on the library's GEMMs."""
     import torch
 
     from tah_amd import ops
+    from tah_amd.decider import MLPIterDecider
 
+    torch.manual_seed(1241)
+    decider = MLPIterDecider(hidden_states_size=hidden).cuda().eval()
     g = torch.Generator().manual_seed(1241)
     logits = [(torch.randn(rows, vocab, generator=g) * 3).to(torch.bfloat16).cuda() for _ in range(2)]  # two sets in rotation
     emb = (torch.randn(vocab, hidden, generator=g) * 0.02).to(torch.bfloat16).cuda()
     out = torch.empty(rows, hidden, dtype=torch.bfloat16, device="cuda")
+    feats = torch.randn(32, hidden * len(decider.hidden_states_layer_nums), generator=g).to(torch.bfloat16).cuda()
     yield
+
+    def replayed(f, per_graph=10):
+        """ms per call of f from a captured graph of `per_graph` calls."""
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            f()
+            side.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                for _ in range(per_graph):
+                    f()
+            graph.replay()
+            side.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(side)
+            for _ in range(max(1, steps)):
+                graph.replay()
+            e1.record(side)
+            side.synchronize()
+        return e0.elapsed_time(e1) / (max(1, steps) * per_graph)
 
     def timed(f):
         for i in range(warmup):
@@ -546,6 +572,10 @@ def bench_topk_mix(steps: int, warmup: int, rows: int = 1024, vocab: int = 15193
     mix_ms = timed(lambda i: ops.topk_mix(logits[i % 2], emb, topk, out=out))
     val_ms = timed(lambda i: ops.topk_values(logits[i % 2], topk))
     torch_ms = timed(lambda i: torch.topk(logits[i % 2], topk, dim=-1))
+    decide = lambda: decider.decide_selected(logits[0][:32], 1, feats)
+    decider_ms = replayed(decide)
+    decider.fused_layers = False
+    decider_library_ms = replayed(decide)
     nbytes = rows * (vocab * 2 + topk * hidden * 2 + hidden * 2)
     gbs = nbytes / (mix_ms * 1e-3) / 1e9
     return {"workload": f"top-{topk} softmax mix of embedding rows, {rows} rows of {vocab} bf16 logits, hidden {hidden} "
@@ -554,7 +584,10 @@ def bench_topk_mix(steps: int, warmup: int, rows: int = 1024, vocab: int = 15193
             "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
                          "traffic": measured_traffic("topk_mix") if (rows, vocab, hidden, topk) == (1024, 151936, 2048, 100) else None,
                          "kernels": "topk_mix_kernel<19>"},
-            "topk_values_ms": val_ms, "torch_topk_ms": torch_ms, "rows_per_s": rows / (mix_ms * 1e-3)}
+            "topk_values_ms": val_ms, "torch_topk_ms": torch_ms, "rows_per_s": rows / (mix_ms * 1e-3),
+            "learned_decider_32_rows": {"ms_per_decision": decider_ms, "ms_per_decision_with_library_gemms": decider_library_ms,
+                                        "what": "MLPIterDecider.decide_selected (top-k values, 11 dense layers, threshold), "
+                                                f"hidden {hidden}, replayed from a graph"}}
 
 
 def bench_sample_rows(steps: int, warmup: int, vocab: int = 151936, temperature: float = 0.6, top_p: float = 0.95):

@@ -39,7 +39,7 @@
 extern "C" {
 #endif
 
-#define TAH_DUO_ABI_VERSION 6
+#define TAH_DUO_ABI_VERSION 7
 
 enum {
     TAH_OK = 0,
@@ -458,6 +458,8 @@ int tah_silu_mul_normed(const void* gate_up, void* out, int32_t rows, int32_t in
  * act_fn(gate) * up, down_proj + residual add.  Products accumulate in float32 in a fixed order (results do not
  * vary from run to run) and are rounded to bf16 where the eager modules round. */
 enum { TAH_LINEAR_PLAIN = 0, TAH_LINEAR_GATE_UP = 1 };
+enum { TAH_ACT_NONE = 0, TAH_ACT_RELU = 1, TAH_ACT_GELU = 2 };      /* GELU: x Phi(x), nn.GELU's default */
+enum { TAH_NORM_NONE = 0, TAH_NORM_RMS = 1, TAH_NORM_LAYER = 2 };
 
 /* w bf16 [n, k] row-major (nn.Linear weight), or [2 n, k] = [gate; up] stacked for TAH_LINEAR_GATE_UP; k % 32 == 0,
  * n % 16 == 0 (gate|up: n % 24 == 0 or n % 16 == 0).  packed: n * k (2 n * k) elements, 16-byte aligned. */
@@ -475,14 +477,19 @@ typedef struct tah_linear_rows_args {
                                * is needed */
     int64_t residual_row_stride, out_row_stride; /* elements */
     int32_t rows, n, k;       /* rows <= 32 */
-    int32_t kind;             /* TAH_LINEAR_PLAIN: out = bf16(r x W^T) [+ bias] [+ residual] [relu]
+    int32_t kind;             /* TAH_LINEAR_PLAIN: out = act(bf16(r (x W^T - m c)) [+ bias] [+ residual])
                                * TAH_LINEAR_GATE_UP: out = bf16(silu(g)) * u, g = bf16(r x Wg^T), u = bf16(r x Wu^T) */
-    int32_t input_norm;       /* 1: r = rsqrt(mean(x[row]^2) + norm_eps), an RMSNorm of the rows whose weight is already
-                               * inside W (the MLP's input norm for gate|up, the final norm for an output head); 0: r = 1 */
+    int32_t input_norm;       /* TAH_NORM_RMS: r = rsqrt(mean(x[row]^2) + norm_eps), an RMSNorm of the rows whose weight is
+                               * already inside W (the MLP's input norm for gate|up, the final norm for an output head);
+                               * TAH_NORM_LAYER (plain only): a LayerNorm of the rows, m = mean(x[row]), r = rsqrt(var(x[row])
+                               * + norm_eps), c = ln_colsum; W holds W0 diag(gamma) and bias bf16(W0 beta + b0) for the
+                               * layer W0, b0 behind LayerNorm(gamma, beta) (the blocks of the learned iteration decider,
+                               * tah/model/iter_decider.py:139-152, :166-169);  TAH_NORM_NONE: r = 1, m = 0 */
     float norm_eps;
     const void* bias;         /* TAH_LINEAR_PLAIN: bf16 [n] added to the product (after its rounding to bf16, before the
                                * residual), or NULL */
-    int32_t relu;             /* TAH_LINEAR_PLAIN: != 0: max(., 0) last (a two-layer MLP's first layer) */
+    int32_t activation;       /* TAH_LINEAR_PLAIN: TAH_ACT_RELU / TAH_ACT_GELU applied last (a small MLP's first layer) */
+    const float* ln_colsum;   /* TAH_NORM_LAYER: float32 [n], sum over k of the bf16 weight row as packed; else ignored */
 } tah_linear_rows_args;
 int tah_linear_rows(const tah_linear_rows_args* args, tah_stream_t stream);
 

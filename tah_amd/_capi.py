@@ -8,7 +8,7 @@ from __future__ import annotations
 
 import ctypes as C
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 c_void_p, c_int32, c_int64, c_float = C.c_void_p, C.c_int32, C.c_int64, C.c_float
 
@@ -117,7 +117,7 @@ class LinearRowsArgs(C.Structure):
         ("w_packed", c_void_p), ("x_packed", c_void_p), ("residual", c_void_p), ("out", c_void_p), ("out_packed", c_void_p),
         ("residual_row_stride", c_int64), ("out_row_stride", c_int64),
         ("rows", c_int32), ("n", c_int32), ("k", c_int32), ("kind", c_int32), ("input_norm", c_int32), ("norm_eps", c_float),
-        ("bias", c_void_p), ("relu", c_int32),
+        ("bias", c_void_p), ("activation", c_int32), ("ln_colsum", c_void_p),
     ]
 
 

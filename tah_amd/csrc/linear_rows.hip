@@ -14,7 +14,11 @@
 //    wave issues the loads of a whole chunk of steps (up to 24 KiB) before the first multiply.
 //  * Epilogues: + residual (in place is fine), or the MLP's act_fn(gate) * up with the input RMSNorm's per-row
 //    factor (the norm's weight is expected inside W): the sum of squares of a row comes from the operands the
-//    waves load anyway.  Results are written row-major and/or in the packed rows form for the next layer.
+//    waves load anyway.  A LayerNorm of the rows folds in the same way (the learned decider's blocks,
+//    tah/model/iter_decider.py:139-152): with W' = W diag(gamma), W' LN(x) = (W' x - mean(x) W' 1) / std(x) + W beta,
+//    so the kernel needs the row's sum and sum of squares, the row sums of W' and a bias that carries W beta.
+//    ReLU or GELU (the exact one, nn.GELU's default) last.  Results are written row-major and/or in the packed rows
+//    form for the next layer.
 //
 // Measured at 32 rows inside a captured step (MI355X): q|k|v 16 MB 6.0 us, o 8 MB 5.1 us, gate|up + SiLU 50 MB
 // 12.3 us, down 25 MB 9.6 us, against 14 / 8.4 / 16 + 5 / 15 us for the library GEMMs and the SiLU kernel.  What
@@ -38,14 +42,16 @@ constexpr int kTileCols = 16;   // output columns of one weight tile
 constexpr int kStepK = 32;      // k of one MFMA step; a tile step is 16 x 32 bf16 = 1 KiB
 constexpr int kGroup24 = 24;    // gate|up: output columns per workgroup when n % 24 == 0 (256 workgroups for n = 6144)
 
-enum Epi { kPlain = 0, kPlainNorm = 1, kGateUp16 = 2, kGateUp24 = 3 };  // kPlainNorm: plain with the rows' norm factor
+// kPlainNorm: plain with the rows' RMSNorm factor; kPlainLayerNorm: with the rows' mean and deviation
+enum Epi { kPlain = 0, kPlainNorm = 1, kGateUp16 = 2, kGateUp24 = 3, kPlainLayerNorm = 4 };
 
 struct LinParams {
     const bf16x8* w;   // packed weight
     const bf16x8* x;   // packed rows
     const __bf16* res; // row-major residual or null
     const __bf16* bias; // [n] added to the product (rounded to bf16 first, as a GEMM's output is) or null
-    int32_t relu;
+    const float* colsum; // kPlainLayerNorm: [n] sums of the packed weight's rows over k
+    int32_t act;       // TAH_ACT_*
     __bf16* y;         // row-major result or null
     bf16x8* yp;        // packed result or null
     int64_t res_rs, y_rs;
@@ -74,6 +80,7 @@ template <int NC, int CH, int EPI, int PW, int NH>
 __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(const LinParams p) {
     __shared__ __align__(16) float red[kLinWaves][NC][16 * NH][kTileCols];
     __shared__ float ssq[kLinWaves][16 * NH];
+    __shared__ float ssum[EPI == kPlainLayerNorm ? kLinWaves : 1][16 * NH];
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const int c = lane % 16, kg = lane / 16;
     int group = blockIdx.x, half = 0;
@@ -104,7 +111,7 @@ __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(const LinParam
     for (int t = 0; t < NC; ++t)
 #pragma unroll
         for (int h = 0; h < NH; ++h) acc[t][h] = f32x4{0.f, 0.f, 0.f, 0.f};
-    float ss0 = 0.f, ss1 = 0.f;
+    float ss0 = 0.f, ss1 = 0.f, sm0 = 0.f, sm1 = 0.f;
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
     // Loads of chunk ch.  Without a compile-time K a step past the wave's share reads step 0 of the wave's range
     // (valid memory) and is multiplied by rows of zeros: no branch sits between the loads.
@@ -138,6 +145,10 @@ __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(const LinParam
                     const float u = (float)a0[i], v = (float)a1[i];
                     ss0 += u * u;
                     ss1 += v * v;
+                    if constexpr (EPI == kPlainLayerNorm) {
+                        sm0 += u;
+                        sm1 += v;
+                    }
                 }
             }
 #pragma unroll
@@ -194,6 +205,16 @@ __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(const LinParam
             ssq[wave][c] = ss0;
             if constexpr (NH == 2) ssq[wave][16 + c] = ss1;
         }
+        if constexpr (EPI == kPlainLayerNorm) {
+            sm0 += __shfl_xor(sm0, 16);
+            sm0 += __shfl_xor(sm0, 32);
+            sm1 += __shfl_xor(sm1, 16);
+            sm1 += __shfl_xor(sm1, 32);
+            if (kg == 0) {
+                ssum[wave][c] = sm0;
+                if constexpr (NH == 2) ssum[wave][16 + c] = sm1;
+            }
+        }
     }
     __syncthreads();
 
@@ -243,7 +264,22 @@ __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(const LinParam
                 float ss = 0.f;
 #pragma unroll
                 for (int w = 0; w < kLinWaves; ++w) ss += ssq[w][lrow];
-                rin = __builtin_amdgcn_rsqf(ss / (float)p.k + p.eps);
+                if constexpr (EPI == kPlainLayerNorm) {
+                    float sm = 0.f;
+#pragma unroll
+                    for (int w = 0; w < kLinWaves; ++w) sm += ssum[w][lrow];
+                    const float mean = sm / (float)p.k;
+                    const float var = fmaxf(ss / (float)p.k - mean * mean, 0.f);
+                    rin = __builtin_amdgcn_rsqf(var + p.eps);
+                    const f32x4 c0 = *reinterpret_cast<const f32x4*>(p.colsum + n0), c1 = *reinterpret_cast<const f32x4*>(p.colsum + n0 + 4);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        sg[i] -= mean * c0[i];
+                        sg[4 + i] -= mean * c1[i];
+                    }
+                } else {
+                    rin = __builtin_amdgcn_rsqf(ss / (float)p.k + p.eps);
+                }
             }
         }
         if constexpr (kGate) {
@@ -266,9 +302,15 @@ __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(const LinParam
 #pragma unroll
                 for (int i = 0; i < 8; ++i) out[i] = (__bf16)((float)out[i] + (float)rv[i]);
             }
-            if (p.relu) {
+            if (p.act == TAH_ACT_RELU) {
 #pragma unroll
                 for (int i = 0; i < 8; ++i) out[i] = (float)out[i] > 0.f ? out[i] : (__bf16)0.f;
+            } else if (p.act == TAH_ACT_GELU) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float v = (float)out[i];
+                    out[i] = (__bf16)(0.5f * v * (1.0f + erff(v * 0.70710678118654752f)));
+                }
             }
         }
         if (p.y) *reinterpret_cast<bf16x8*>(p.y + (int64_t)row * p.y_rs + n0) = out;
@@ -372,12 +414,15 @@ extern "C" int tah_linear_rows(const tah_linear_rows_args* a, tah_stream_t strea
     const bool gate_up = a->kind == TAH_LINEAR_GATE_UP;
     const bool g24 = gate_up && a->n % kGroup24 == 0;
     if (!g24 && a->n % kTileCols != 0) return TAH_E_SHAPE;
-    if (gate_up && (a->residual || a->bias || a->relu)) return TAH_E_SHAPE;
+    if (a->activation != TAH_ACT_NONE && a->activation != TAH_ACT_RELU && a->activation != TAH_ACT_GELU) return TAH_E_SHAPE;
+    if (a->input_norm != TAH_NORM_NONE && a->input_norm != TAH_NORM_RMS && a->input_norm != TAH_NORM_LAYER) return TAH_E_SHAPE;
+    if (gate_up && (a->residual || a->bias || a->activation != TAH_ACT_NONE || a->input_norm == TAH_NORM_LAYER)) return TAH_E_SHAPE;
+    if (a->input_norm == TAH_NORM_LAYER && !a->ln_colsum && a->n > 0 && a->k > 0) return TAH_E_NULL;
     if (a->out_packed && a->n % kStepK != 0) return TAH_E_SHAPE;  // the packed rows form holds whole steps of 32 columns
     if (a->n == 0 || a->k == 0 || (a->rows == 0 && !a->out_packed)) return TAH_OK;
     if (!a->w_packed || !a->x_packed || (!a->out && !a->out_packed)) return TAH_E_NULL;
     if (!aligned16(a->w_packed) || !aligned16(a->x_packed) || !aligned16(a->out) || !aligned16(a->out_packed) || !aligned16(a->residual) ||
-        !aligned16(a->bias) ||
+        !aligned16(a->bias) || (a->input_norm == TAH_NORM_LAYER && !aligned16(a->ln_colsum)) ||
         (a->out && a->out_row_stride % 8 != 0) || (a->residual && a->residual_row_stride % 8 != 0))
         return TAH_E_ALIGN;
     if ((a->out && a->out_row_stride < a->n) || (a->residual && a->residual_row_stride < a->n)) return TAH_E_SHAPE;
@@ -386,7 +431,8 @@ extern "C" int tah_linear_rows(const tah_linear_rows_args* a, tah_stream_t strea
     p.x = static_cast<const bf16x8*>(a->x_packed);
     p.res = static_cast<const __bf16*>(a->residual);
     p.bias = static_cast<const __bf16*>(a->bias);
-    p.relu = a->relu ? 1 : 0;
+    p.act = a->activation;
+    p.colsum = a->input_norm == TAH_NORM_LAYER ? a->ln_colsum : nullptr;
     p.y = static_cast<__bf16*>(a->out);
     p.yp = static_cast<bf16x8*>(a->out_packed);
     p.res_rs = a->residual_row_stride;
@@ -395,11 +441,11 @@ extern "C" int tah_linear_rows(const tah_linear_rows_args* a, tah_stream_t strea
     p.n = a->n;
     p.k = a->k;
     p.eps = a->norm_eps;
-    p.norm = a->input_norm ? 1 : 0;
+    p.norm = a->input_norm;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int steps = a->k / kStepK;
     const int pw = steps % kLinWaves == 0 ? steps / kLinWaves : 0;  // compile-time K for the sizes of the end-to-end model
-    if (!gate_up && a->n >= kWideFromCols && a->n % (2 * kTileCols) == 0) {
+    if (!gate_up && a->input_norm != TAH_NORM_LAYER && a->n >= kWideFromCols && a->n % (2 * kTileCols) == 0) {
         // an output head: two tiles per workgroup, the rows' operand is read half as often
         const int groups = a->n / (2 * kTileCols);
         if (p.norm) {
@@ -409,6 +455,8 @@ extern "C" int tah_linear_rows(const tah_linear_rows_args* a, tah_stream_t strea
             if (pw == 8) launch<2, 2, kPlain, 8>(p, groups, st);
             else launch<2, 2, kPlain, 0>(p, groups, st);
         }
+    } else if (!gate_up && a->input_norm == TAH_NORM_LAYER) {
+        launch<1, 4, kPlainLayerNorm, 0>(p, a->n / kTileCols, st);
     } else if (!gate_up) {
         const int groups = a->n / kTileCols;
         if (p.norm) {

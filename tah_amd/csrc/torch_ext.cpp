@@ -664,20 +664,26 @@ Tensor topk_mix(const Tensor& logits, const Tensor& embedding, int64_t topk, con
 }
 
 // the top-k logits of every row, largest first (tah_topk_mix with values_out only), optionally with their indices
-Tensor topk_values(const Tensor& logits, int64_t topk, const optional<Tensor>& indices) {
+// (`out`: a bf16 [rows, >= k] matrix whose first k columns receive the values, e.g. rows padded for a linear layer)
+Tensor topk_values(const Tensor& logits, int64_t topk, const optional<Tensor>& indices, const optional<Tensor>& out) {
     need_lib();
-    Dev d; d.see(logits);
+    Dev d; d.see(logits); d.see(out);
     TORCH_CHECK(logits.dim() == 2 && logits.scalar_type() == at::kBFloat16 && logits.stride(1) == 1 && topk >= 1,
                 "topk_values: logits must be bf16 [rows, V] with a contiguous inner dimension");
     const int64_t rows = logits.size(0), k = std::min<int64_t>(topk, logits.size(1));
-    Tensor vals = at::empty({rows, k}, logits.options());
+    if (out.has_value())
+        TORCH_CHECK(out->dim() == 2 && out->scalar_type() == at::kBFloat16 && out->size(0) == rows && out->size(1) >= k &&
+                        (out->numel() == 0 || out->stride(1) == 1),
+                    "topk_values: out must be bf16 [rows, >= min(topk, V)] with a contiguous inner dimension");
+    Tensor vals = out.has_value() ? *out : at::empty({rows, k}, logits.options());
     tah_topk_mix_args a{};
     a.logits = ptr(logits);
     a.logits_row_stride = rows > 1 ? logits.stride(0) : logits.size(1);
     a.rows = (int32_t)rows; a.vocab = (int32_t)logits.size(1); a.hidden = 8; a.topk = (int32_t)topk;
     a.values_out = vals.data_ptr();
-    a.values_row_stride = k;
+    a.values_row_stride = out.has_value() && rows > 1 ? out->stride(0) : vals.size(1);
     if (indices.has_value()) {
+        TORCH_CHECK(!out.has_value() || a.values_row_stride == k, "topk_values: indices go with values rows of exactly min(topk, V) columns");
         d.see(*indices);
         TORCH_CHECK(indices->scalar_type() == at::kInt && indices->dim() == 2 && indices->size(0) == rows && indices->size(1) == k && indices->is_contiguous(),
                     "topk_values: indices must be a contiguous int32 [rows, min(topk, V)] tensor");
@@ -955,9 +961,14 @@ Tensor linear_pack_rows(const Tensor& x, const optional<Tensor>& out) {
 // only the packed result is asked for).
 optional<Tensor> linear_rows(const Tensor& w_packed, const Tensor& x_packed, int64_t rows, int64_t n, int64_t k, bool gate_up,
                              const optional<Tensor>& residual, const optional<Tensor>& out, const optional<Tensor>& out_packed,
-                             bool want_out, bool input_norm, double norm_eps, const optional<Tensor>& bias, bool relu) {
+                             bool want_out, int64_t input_norm, double norm_eps, const optional<Tensor>& bias, int64_t activation,
+                             const optional<Tensor>& ln_colsum) {
     need_lib();
-    Dev d; d.see(w_packed); d.see(x_packed); d.see(residual); d.see(out); d.see(out_packed); d.see(bias);
+    Dev d; d.see(w_packed); d.see(x_packed); d.see(residual); d.see(out); d.see(out_packed); d.see(bias); d.see(ln_colsum);
+    if (ln_colsum.has_value())
+        TORCH_CHECK(ln_colsum->scalar_type() == at::kFloat && ln_colsum->is_contiguous() && ln_colsum->numel() == n,
+                    "linear_rows: ln_colsum must be a contiguous float32 [N] tensor");
+    TORCH_CHECK((input_norm == TAH_NORM_LAYER) == ln_colsum.has_value(), "linear_rows: ln_colsum goes with the LayerNorm fold and only with it");
     if (bias.has_value()) TORCH_CHECK(packed_vec(*bias, n), "linear_rows: bias must be a contiguous bf16 [N] tensor");
     TORCH_CHECK(rows >= 0 && n >= 0 && k >= 0, "linear_rows: negative size");
     TORCH_CHECK(packed_vec(w_packed, (gate_up ? 2 : 1) * n * k), "linear_rows: w_packed must come from linear_pack_weight for these sizes");
@@ -980,8 +991,9 @@ optional<Tensor> linear_rows(const Tensor& w_packed, const Tensor& x_packed, int
     a.out_packed = out_packed.has_value() ? out_packed->data_ptr() : nullptr;
     a.rows = (int32_t)rows; a.n = (int32_t)n; a.k = (int32_t)k;
     a.kind = gate_up ? TAH_LINEAR_GATE_UP : TAH_LINEAR_PLAIN;
-    a.input_norm = input_norm ? 1 : 0; a.norm_eps = (float)norm_eps;
-    a.bias = bias.has_value() ? bias->data_ptr() : nullptr; a.relu = relu ? 1 : 0;
+    a.input_norm = (int32_t)input_norm; a.norm_eps = (float)norm_eps;
+    a.bias = bias.has_value() ? bias->data_ptr() : nullptr; a.activation = (int32_t)activation;
+    a.ln_colsum = ln_colsum.has_value() ? static_cast<const float*>(ln_colsum->data_ptr()) : nullptr;
     check_rc(g.linear_rows(&a, d.stream()), "tah_linear_rows");
     return y;
 }

@@ -147,10 +147,11 @@ def topk_mix(logits: torch.Tensor, embedding: torch.Tensor, topk: int, row_enabl
     return _call("topk_mix", logits, embedding, int(topk), row_enable, out, out_packed, bool(zero_disabled), values_out)
 
 
-def topk_values(logits: torch.Tensor, topk: int) -> torch.Tensor:
+def topk_values(logits: torch.Tensor, topk: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``torch.topk(logits, min(topk, V), dim=-1).values`` for bf16 logits [rows, V] (``tah_topk_mix`` producing only
-    its ``values_out``): the logit features of the iteration decider (tah/model/iter_decider.py:281)."""
-    return _call("topk_values", logits, int(topk), None)
+    its ``values_out``): the logit features of the iteration decider (tah/model/iter_decider.py:281).  ``out``: a bf16
+    [rows, W >= k] matrix whose first k columns take the values (the rest is left as it is)."""
+    return _call("topk_values", logits, int(topk), None, out)
 
 
 def topk(logits: torch.Tensor, k: int):
@@ -158,7 +159,7 @@ def topk(logits: torch.Tensor, k: int):
     ascending index (``torch.topk`` leaves the order and the choice among equal values open): values bf16, indices int32.
     k <= 256."""
     idx = torch.empty(logits.size(0), min(int(k), logits.size(1)), dtype=torch.int32, device=logits.device)
-    return _call("topk_values", logits, int(k), idx), idx
+    return _call("topk_values", logits, int(k), idx, None), idx
 
 
 def sample_rows(logits: torch.Tensor, uniforms: torch.Tensor, temperature: float, *, top_p: float = 1.0, min_p: float = 0.0,
@@ -244,18 +245,26 @@ def linear_pack_rows(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> tor
 def linear_rows(w_packed: torch.Tensor, x_packed: torch.Tensor, rows: int, n: int, k: int, *, gate_up: bool = False,
                 residual: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
                 out_packed: Optional[torch.Tensor] = None, want_out: bool = True, norm_eps: Optional[float] = None,
-                bias: Optional[torch.Tensor] = None, relu: bool = False):
+                bias: Optional[torch.Tensor] = None, relu: bool = False, gelu: bool = False,
+                ln_colsum: Optional[torch.Tensor] = None):
     """A linear layer of a decode step on packed operands (``tah_linear_rows``), bf16, rows <= 32.
 
     ``x @ w.T`` [rows, N], plus ``residual`` [rows, N] when given (``out=residual`` updates it in place); with
     ``gate_up``, ``silu(x @ gate.T) * (x @ up.T)``.  With ``norm_eps`` the products are first multiplied by the row's
     ``rsqrt(mean(x**2) + norm_eps)``: an RMSNorm of the rows whose weight sits in w (the MLP's input norm for gate|up,
-    the final norm for an output head).  ``bias`` [N] is added to the rounded product and ``relu`` applied last (the first
-    layer of a small MLP; not with ``gate_up``).  ``out_packed`` [32 * N] also
+    the final norm for an output head).  ``bias`` [N] is added to the rounded product and ``relu`` or ``gelu`` (the exact
+    one) applied last (the first layer of a small MLP; not with ``gate_up``).  With ``ln_colsum`` (float32 [N], the sums of
+    the weight's rows) ``norm_eps`` is a LayerNorm's: the product becomes ``(x @ w.T - mean(x) * ln_colsum) * rsqrt(var(x) +
+    norm_eps)``, a layer behind a LayerNorm whose scale sits in w and whose shift sits in ``bias``.  ``out_packed`` [32 * N] also
     receives the result as the next layer's rows operand; ``want_out=False`` with ``out_packed`` writes only that.
     Returns the row-major result (None when it was not asked for)."""
+    if relu and gelu:
+        raise ValueError("linear_rows: one activation")
+    norm = 0 if norm_eps is None else (2 if ln_colsum is not None else 1)
+    if ln_colsum is not None and norm_eps is None:
+        raise ValueError("linear_rows: ln_colsum needs the LayerNorm's eps")
     return _call("linear_rows", w_packed, x_packed, int(rows), int(n), int(k), bool(gate_up), residual, out, out_packed,
-                 bool(want_out), norm_eps is not None, float(norm_eps or 0.0), bias, bool(relu))
+                 bool(want_out), norm, float(norm_eps or 0.0), bias, 1 if relu else (2 if gelu else 0), ln_colsum)
 
 
 def greedy_step(logits0, logits1, hard, eos: int, tok, finished, pos, out_tokens, step_idx, out_len, n_hard, n_steps) -> None:

@@ -6,6 +6,8 @@ import torch
 from oracle import decider_ref as R
 
 SMALL = dict(topk=10, hidden_states_size=32, hidden_states_layer_nums=(1, 3), hidden_dims=(16, 32, 16), expansion_factor=2)
+# every width a multiple of 32: up to 32 rows of a bf16 copy go through the linear-layer kernel, not the library
+FUSABLE = dict(topk=10, hidden_states_size=32, hidden_states_layer_nums=(1, 3), hidden_dims=(32, 64, 32), expansion_factor=2)
 
 
 def make(device, dtype, seed=0, normalize_input=False, threshold=0.5, **cfg):

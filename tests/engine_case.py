@@ -177,7 +177,7 @@ def run_with_decider(device, *, prompt=(9, 6, 12), steps=4, layers=3, seed=2, vo
     w = Weights.from_hf(_LM, cfg, device)
     picks = (1, layers)   # after the first layer, and the last one (after the final norm)
     dec = D.make(device, torch.bfloat16, seed=seed + 3, topk=10, hidden_states_size=256, hidden_states_layer_nums=picks,
-                 hidden_dims=(16, 32, 16), expansion_factor=2)
+                 hidden_dims=(32, 64, 32), expansion_factor=2)  # (widths the linear-layer kernel takes)
     p64 = D.state64(dec)
 
     def decide(logits, stack):

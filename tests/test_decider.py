@@ -66,6 +66,60 @@ def test_decider_on_cpu_shim():
         D.check(m, logits, hs, atol=0.08, rtol=0.05)                 # bf16 layers, as released
 
 
+def _fused_checks(dev, cfg, V, n_layers, H, rows_list, atol, rtol):
+    """Up to 32 rows of a bf16 decider: the dense layers run on tah_linear_rows (LayerNorms folded, GELU and skips in
+    the launches); against the oracle like the library path, whose error on the same inputs it must not exceed by much."""
+    for normalize in (False, True):
+        m = D.make(dev, torch.bfloat16, seed=21, normalize_input=normalize, **cfg)
+        for rows in rows_list:
+            logits, hs = D.inputs(dev, (rows,), V, n_layers, H, seed=30 + rows)
+            assert m.takes_fused_path(rows)
+            m._plan = None
+            err = D.check(m, logits, hs, atol=atol, rtol=rtol)
+            assert m._plan is not None            # the chain of launches was built, i.e. taken
+            m.fused_layers = False
+            err_lib = D.check(m, logits, hs, atol=atol, rtol=rtol)
+            m.fused_layers = True
+            assert err <= 2 * err_lib + 0.02, (err, err_lib)
+    # more rows than a launch takes: the library's GEMMs
+    logits, hs = D.inputs(dev, (3, 15), V, n_layers, H, seed=40)
+    m._plan = None
+    D.check(m, logits, hs, atol=atol, rtol=rtol)
+    assert m._plan is None and not m.takes_fused_path(45)
+    # new weights (a state dict loaded): the packed copies follow
+    logits, hs = D.inputs(dev, (9,), V, n_layers, H, seed=41)
+    m = D.make(dev, torch.bfloat16, seed=22, **cfg)
+    D.check(m, logits, hs, atol=atol, rtol=rtol)
+    other = D.make(dev, torch.bfloat16, seed=23, **cfg)
+    z_other = other(logits, 0, all_hidden_states=hs)[1]
+    m.load_state_dict(other.state_dict())
+    assert torch.equal(m(logits, 0, all_hidden_states=hs)[1], z_other)
+    D.check(m, logits, hs, atol=atol, rtol=rtol)
+    # no hidden states: zeros in their place (iter_decider.py:251-252); leading dimensions are kept
+    D.check(m, logits.view(3, 3, -1), None, atol=atol, rtol=rtol)
+
+
+@pytest.mark.skipif(not emu_util.have_host_clang(), reason="host clang++ not available")
+def test_decider_dense_layers_on_the_linear_kernel_on_cpu_shim():
+    with emu_util.emulated():
+        _fused_checks("cpu", D.FUSABLE, 300, 4, 32, (7, 32, 1), atol=0.08, rtol=0.05)
+
+
+@pytest.mark.gpu
+def test_decider_dense_layers_on_the_linear_kernel_gpu():
+    _fused_checks("cuda", D.FUSABLE, 300, 4, 32, (7, 32, 1), atol=0.08, rtol=0.05)
+    _fused_checks("cuda", {}, 151936, 29, 1024, (32, 19), atol=0.06, rtol=0.03)   # the released sizes
+    m = D.make("cuda", torch.bfloat16, seed=25)
+    logits, hs = D.inputs("cuda", (32,), 151936, 29, 1024, seed=26)
+    m(logits, 0, all_hidden_states=hs)
+    with torch.cuda.device(0):
+        torch.cuda.set_sync_debug_mode("error")     # the chain reads nothing back either
+        try:
+            m(logits, 0, all_hidden_states=hs)
+        finally:
+            torch.cuda.set_sync_debug_mode("default")
+
+
 @pytest.mark.gpu
 def test_decider_gpu_released_sizes():
     logits, hs = D.inputs("cuda", (2, 24), 151936, 29, 1024, seed=7)

@@ -487,7 +487,7 @@ def test_engine_with_the_learned_decider_gpu():
     cfg = EngineConfig(hidden=256, layers=3, hq=16, hkv=8, head_dim=128, intermediate=768, vocab=4096, decider_hidden=32)
     w = Weights.random_init(cfg, "cuda", seed=8)
     dec = D.make("cuda", torch.bfloat16, seed=12, topk=10, hidden_states_size=256, hidden_states_layer_nums=(1, 2, 3),
-                 hidden_dims=(16, 32, 16), expansion_factor=2)
+                 hidden_dims=(32, 64, 32), expansion_factor=2)  # (widths the linear-layer kernel takes)
     B, T, new = 32, 19, 18
     g = torch.Generator().manual_seed(13)
     ids = torch.randint(0, cfg.vocab, (B * T,), generator=g).cuda()

@@ -61,16 +61,21 @@ def unpack_rows(packed, k):
     return x
 
 
-def reference(x, w, *, residual=None, gate_up=False, norm_eps=None, bias=None, relu=False):
-    """float64 sums with the eager modules' bf16 roundings."""
+def reference(x, w, *, residual=None, gate_up=False, norm_eps=None, bias=None, relu=False, gelu=False, layer_norm=False):
+    """float64 sums with the eager modules' bf16 roundings.  ``layer_norm``: the rows go through a LayerNorm without
+    scale and shift first (those sit in w and bias), written as the library routine, not as the kernel's fold."""
     xd, wd = x.double(), w.double()
-    r = torch.rsqrt((xd ** 2).mean(-1, keepdim=True) + norm_eps) if norm_eps is not None else 1.0
+    r = torch.rsqrt((xd ** 2).mean(-1, keepdim=True) + norm_eps) if norm_eps is not None and not layer_norm else 1.0
+    if layer_norm:
+        xd = torch.nn.functional.layer_norm(xd, xd.shape[-1:], eps=norm_eps)
     if not gate_up:
         y = (r * (xd @ wd.t())).to(BF)
         if bias is not None:
             y = (y.double() + bias.double()).to(BF)
         if residual is not None:
             y = (y.double() + residual.double()).to(BF)
+        if gelu:
+            return torch.nn.functional.gelu(y.double()).to(BF)
         return torch.relu(y) if relu else y
     n = w.shape[0] // 2
     g = (r * (xd @ wd[:n].t())).to(BF).double()
@@ -120,6 +125,10 @@ CASES = [
     (32, 32, 160, "plain_norm"),
     (11, 32, 2048, "bias_relu_norm"),  # first layer of a small MLP behind a folded norm (the decider)
     (32, 48, 96, "bias_relu"),
+    (32, 64, 256, "bias_gelu_ln"),     # a layer behind a LayerNorm, GELU last (the learned decider's blocks)
+    (13, 2048, 512, "bias_gelu_ln"),   # sixteen rows per workgroup
+    (32, 2080, 96, "bias_ln"),         # all 32 rows per workgroup
+    (5, 16, 1280, "bias_gelu"),
 ]
 
 
@@ -131,9 +140,14 @@ def _linear_case(dev, rows, n, k, kind, seed=0):
     res = _rand((rows, n), 13 + seed) if kind == "residual" else None
     eps = 1e-6 if kind.endswith("_norm") else None
     bias = _rand((n,), 14 + seed) if kind.startswith("bias") else None
-    relu = "relu" in kind
-    want = reference(x, w, residual=res, gate_up=gu, norm_eps=eps, bias=bias, relu=relu)
-    extra = dict(bias=bias.to(dev), relu=relu) if bias is not None else {}
+    relu, gelu, ln = "relu" in kind, "gelu" in kind, kind.endswith("_ln")
+    if ln:  # rows with a mean of their own, so that a fold that forgets it fails
+        x = (x.float() * 0.7 + 0.9 * torch.arange(rows).view(-1, 1) / max(rows, 1) - 0.4).to(BF)
+        eps = 1e-5
+    want = reference(x, w, residual=res, gate_up=gu, norm_eps=eps, bias=bias, relu=relu, gelu=gelu, layer_norm=ln)
+    extra = dict(bias=bias.to(dev), relu=relu, gelu=gelu) if bias is not None else {}
+    if ln:
+        extra["ln_colsum"] = w.float().sum(-1).to(dev)
     wp = ops.linear_pack_weight(w.to(dev), gate_up=gu)
     xp = ops.linear_pack_rows(x.to(dev))
     yp = torch.full((32 * n,), 7.0, dtype=BF, device=dev) if n % 32 == 0 else None  # the packed form holds whole steps of 32
@@ -176,6 +190,10 @@ def _error_checks(dev):
         ops.linear_rows(wp, xp, 33, 32, 64)
     with pytest.raises((TahDuoError, RuntimeError)):
         ops.linear_rows(wp, xp, 4, 32, 32)                            # sizes the operands were not packed for
+    with pytest.raises((TahDuoError, RuntimeError)):
+        ops.linear_rows(wp, xp, 4, 32, 64, norm_eps=1e-5, ln_colsum=torch.zeros(16, device=dev))   # one sum per output column
+    with pytest.raises((TahDuoError, RuntimeError)):
+        ops.linear_rows(wp, xp, 4, 16, 64, gate_up=True, norm_eps=1e-5, ln_colsum=torch.zeros(16, device=dev))  # no LayerNorm with the gate
     with pytest.raises((TahDuoError, RuntimeError)):
         ops.linear_rows(wp, xp, 4, 16, 64, gate_up=True, residual=_rand((4, 16), 3).to(dev))  # no residual with the gate
     w48 = ops.linear_pack_weight(_rand((48, 64), 4).to(dev))
