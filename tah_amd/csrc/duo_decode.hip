@@ -30,20 +30,11 @@ namespace tah {
 namespace {
 
 constexpr int kD = 128;
-#ifndef TAH_DEC_NT
-#define TAH_DEC_NT 1   // streaming (nontemporal) K/V loads: every cache row is read exactly once
-#endif
-#ifndef TAH_DEC_CHUNK
-#define TAH_DEC_CHUNK 1024
-#endif
-#ifndef TAH_DEC_UNROLL
-#define TAH_DEC_UNROLL 4
-#endif
-constexpr int kChunk = TAH_DEC_CHUNK;  // rows per workgroup when there are rows enough to fill the chip
+constexpr int kChunk = 1024;           // rows per workgroup when there are rows enough to fill the chip
 constexpr int kChunkSmall = 256;       // ... and when there are not (few sequences, short contexts): four
                                        // times the workgroups, so that enough loads are in flight
 constexpr int kDecThreads = 256;     // 4 waves x (chunk / 4) rows
-constexpr int kUnroll = TAH_DEC_UNROLL;  // loads of 4 rows in flight per wave and tensor
+constexpr int kUnroll = 4;           // loads of 4 rows in flight per wave and tensor
 constexpr int kPart = kD + 2;        // acc[128], m, l  (floats per partial)
 
 
@@ -142,21 +133,14 @@ __device__ __forceinline__ void load_rows(RowBlock<U>& b, const Seg& sg, bool se
         const int r = r_it + u * 4 + kq;
         b.ok[u] = r < row_end;
         rl[u] = b.ok[u] ? r : row_end - 1;  // keep tail loads inside the slab
-#if TAH_DEC_NT
+        // (streaming loads: every cache row is read exactly once)
         b.k[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kbase + (int64_t)rl[u] * sg.k_rs));
-#else
-        b.k[u] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)rl[u] * sg.k_rs);
-#endif
         b.pos[u] = second ? posbase[rl[u]] : 0;
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-#if TAH_DEC_NT
         b.v[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vbase + (int64_t)rl[u] * sg.v_rs));
-#else
-        b.v[u] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)rl[u] * sg.v_rs);
-#endif
     }
 }
 // Scores, online softmax and the weighted sum of V for a loaded block, for the G query heads of the kv head at

@@ -31,17 +31,13 @@
 #include "duo_device.h"
 #include "tah_duo.h"
 
-// Which of the two wave sets (early / late by half a tile) a wave belongs to.  Waves w and w+4 of a
-// workgroup share a SIMD.
-#ifndef TAH_FWD_PRIO
-#define TAH_FWD_PRIO 2
-#endif
-#ifndef TAH_FWD_LATE_SET
-#define TAH_FWD_LATE_SET(wave) ((wave) >> 2)
-#endif
-
 namespace tah {
 namespace {
+
+constexpr int kMatrixPrio = 2;  // s_setprio of a wave while it runs its matrix phase
+// Which of the two wave sets (early / late by half a tile) a wave belongs to.  Waves w and w+4 of a
+// workgroup share a SIMD.
+__device__ __forceinline__ int late_set(int wave) { return wave >> 2; }
 
 constexpr int kD = 128;        // head_dim
 constexpr int kBN = 64;        // keys per tile
@@ -308,9 +304,7 @@ __global__ __launch_bounds__(64 * W) TAH_WAVES_PER_EU(2, 2) void duo_fwd_kernel(
     // LDS reads run four MFMAs ahead of their consumers.
     auto matrix = [&](int t, auto qk_tag) __attribute__((always_inline)) {
         constexpr bool kQk = decltype(qk_tag)::value;
-#if TAH_FWD_PRIO
-        __builtin_amdgcn_s_setprio(TAH_FWD_PRIO);  // the matrix pipe is the scarce one: its wave issues first
-#endif
+        __builtin_amdgcn_s_setprio(kMatrixPrio);  // the matrix pipe is the scarce one: its wave issues first
         pv(t);
         if constexpr (kQk) qk(t + 1);
         __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
@@ -328,9 +322,7 @@ __global__ __launch_bounds__(64 * W) TAH_WAVES_PER_EU(2, 2) void duo_fwd_kernel(
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-#if TAH_FWD_PRIO
         __builtin_amdgcn_s_setprio(0);
-#endif
     };
     // is tile t+1 one this wave computes?
     auto next_active = [&](int t) { return t + 1 < n_active || (t + 1 >= n1 && t + 1 < ntiles); };
@@ -501,7 +493,7 @@ __global__ __launch_bounds__(64 * W) TAH_WAVES_PER_EU(2, 2) void duo_fwd_kernel(
     if (ntiles > 0) {
         TAH_PHASE_BARRIER();  // before h = 0
         issue(0);
-        if (W == 4 || TAH_FWD_LATE_SET(wave) == 0) run(std::false_type{});
+        if (W == 4 || late_set(wave) == 0) run(std::false_type{});
         else run(std::true_type{});
     }
     if constexpr (W == 4) {  // the output staging below overlies the rings: every wave must be done reading them

@@ -10,7 +10,9 @@
 // deriving it from blockIdx.  Integer work, no host read-back; a table built from the call's own boundaries only
 // changes the order in which tiles are started, never a result: the table is a permutation of the tile numbers, which
 // the kernels turn into tiles from the call's own boundaries, so even one built from other boundaries of the same
-// sizes makes them visit every tile once (in an order that is no longer the intended one).
+// sizes makes them visit every tile once (in an order that is no longer the intended one).  Tiles of equal weight are
+// placed in the order their threads reach the bin's counter, so the table's order among equals can differ from build to
+// build; results do not depend on it.
 #include <hip/hip_runtime.h>
 
 #include "duo_device.h"

@@ -16,8 +16,9 @@ What changes is where the work is done:
   folded into its first layer (scale into the weight, shift into the bias, the row's mean and deviation applied to the
   product), GELU is that launch's last step, the block's second layer and its ``dim_change`` are one product over the
   two inputs side by side (or the skip is the launch's residual), every layer writes the next one's operand in the
-  order it is read in, and the concatenation of hidden states and projected logits is where the launches write.  Some
-  fourteen launches where the eager modules make about forty-five.  More rows (a prompt's tokens) and float32 copies
+  order it is read in, and the concatenation of hidden states and projected logits is where the launches write.  Ten
+  launches for the twelve linear layers (fifteen with the top-k values, two operand packs, sigmoid and compare) where
+  the eager modules make about forty-five.  More rows (a prompt's tokens) and float32 copies
   of the decider go through the library's GEMMs.
 
 Dropout is the identity here (inference); training the decider is the reference's own code's business.  Logits must be
