@@ -44,7 +44,8 @@ def _ceil32(n: int) -> int:
 
 class _FusedPlan:
     """The decider's dense layers as ``ops.linear_rows`` calls: weights re-ordered (LayerNorms folded in) once, the
-    operand buffers the launches hand to each other, and the sequence of launches."""
+    operand buffers the launches hand to each other, and the sequence of launches.  Every call on one decider writes the
+    same buffers: calls follow each other on one stream (as a generation loop's do), they do not overlap."""
 
     def __init__(self, m: "MLPIterDecider", dev: torch.device):
         bf, f32 = torch.bfloat16, torch.float32
