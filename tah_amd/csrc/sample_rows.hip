@@ -15,6 +15,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cmath>
+#include <type_traits>
 
 #include "duo_device.h"
 #include "row_keys.h"
@@ -118,6 +119,40 @@ __global__ __launch_bounds__(kSmpThreads) void sample_rows_kernel(const SamplePa
         return w;
     };
     constexpr int kLoadGroup = 4;
+    // Rows that start on a 16-byte boundary and have a multiple of eight entries (any real vocabulary) are loaded without
+    // a branch: a piece lies inside the row or behind it as a whole, the loads of pieces behind it go to the row's start
+    // and their keys become 0 by a select.  (With a branch around a load the compiler waits for it where the branch ends:
+    // one load in flight per thread instead of a group's.)
+    const bool whole_pieces = V % 8 == 0 && (reinterpret_cast<uintptr_t>(lrow) & 15) == 0 && (reinterpret_cast<uintptr_t>(prow) & 15) == 0;
+    auto load_whole_pieces = [&](auto with_prev) __attribute__((always_inline)) {
+        constexpr bool kPrev = decltype(with_prev)::value;
+#pragma unroll
+        for (int j0 = 0; j0 < NVEC; j0 += kLoadGroup) {
+            u32x4 w[kLoadGroup], w2[kPrev ? kLoadGroup : 1];
+#pragma unroll
+            for (int j = j0; j < j0 + kLoadGroup && j < NVEC; ++j) {
+                const int i0 = (j * kSmpThreads + tid) * 8, at = i0 < V ? i0 : 0;
+                w[j - j0] = *reinterpret_cast<const u32x4*>(lrow + at);
+                if constexpr (kPrev) w2[j - j0] = *reinterpret_cast<const u32x4*>(prow + at);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = j0; j < j0 + kLoadGroup && j < NVEC; ++j) {
+                const bool inside = (j * kSmpThreads + tid) * 8 < V;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    uint32_t x = w[j - j0][q];
+                    if constexpr (kPrev) x = add_bf16x2(w2[j - j0][q], x);
+                    keys[j][q] = inside ? order_keys2(x) : 0u;
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    if (whole_pieces) {  // (uniform, and so is prow)
+        if (prow) load_whole_pieces(std::true_type{});
+        else load_whole_pieces(std::false_type{});
+    } else
 #pragma unroll
     for (int j0 = 0; j0 < NVEC; j0 += kLoadGroup) {
 #pragma unroll

@@ -142,37 +142,62 @@ __global__ __launch_bounds__(kMixThreads) void topk_mix_kernel(const MixParams p
     // loaded four pieces at a time and turned into keys in place, with a scheduling fence per group: left
     // alone, the scheduler issues every load first and the row sits in registers twice (raw and as keys)
     constexpr int kGroup = 4;
+    // A row that starts on a 16-byte boundary and has a multiple of eight entries (any real vocabulary) is loaded without
+    // a branch: a piece lies inside the row or behind it as a whole, the loads of pieces behind it are sent to the row's
+    // start and their keys set to 0 by a select.  With a branch around a load the compiler waits for it where the branch
+    // ends, and a thread then has one load in flight instead of a group's.
+    const bool whole_pieces = (reinterpret_cast<uintptr_t>(lrow) & 15) == 0 && V % 8 == 0;  // (uniform)
+    if (whole_pieces) {
 #pragma unroll
-    for (int j0 = 0; j0 < NVEC; j0 += kGroup) {
+        for (int j0 = 0; j0 < NVEC; j0 += kGroup) {
+            u32x4 w[kGroup];
 #pragma unroll
-        for (int j = j0; j < j0 + kGroup && j < NVEC; ++j) {
-            const int i0 = (j * kMixThreads + tid) * 8;
-            u32x4 w = {0u, 0u, 0u, 0u};
-            if (i0 + 8 <= V && ((reinterpret_cast<uintptr_t>(lrow + i0) & 15) == 0)) {
-                w = *reinterpret_cast<const u32x4*>(lrow + i0);
-            } else if (i0 < V) {
-                const uint16_t* h = reinterpret_cast<const uint16_t*>(lrow);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const uint32_t b = i0 + e < V ? h[i0 + e] : 0u;
-                    w[e / 2] |= b << (16 * (e % 2));
-                }
+            for (int j = j0; j < j0 + kGroup && j < NVEC; ++j) {
+                const int i0 = (j * kMixThreads + tid) * 8;
+                w[j - j0] = *reinterpret_cast<const u32x4*>(lrow + (i0 < V ? i0 : 0));
             }
-            if ((j + 1) * kMixThreads * 8 <= V) {  // (uniform) the whole piece lies inside the row, for every thread
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int q = 0; q < 4; ++q) keys[j][q] = order_keys2(w[q]);
-            } else {
+            for (int j = j0; j < j0 + kGroup && j < NVEC; ++j) {
+                const bool inside = (j * kMixThreads + tid) * 8 < V;
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    uint32_t lo = order_key(w[q] & 0xffffu), hi = order_key(w[q] >> 16);
-                    // indices past the end get key 0 (below every real key) so that they are never selected
-                    if (i0 + 2 * q >= V) lo = 0u;
-                    if (i0 + 2 * q + 1 >= V) hi = 0u;
-                    keys[j][q] = lo | (hi << 16);
-                }
+                for (int q = 0; q < 4; ++q) keys[j][q] = inside ? order_keys2(w[j - j0][q]) : 0u;  // key 0: below every real key
             }
+            __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_sched_barrier(0);
+    } else {
+#pragma unroll
+        for (int j0 = 0; j0 < NVEC; j0 += kGroup) {
+#pragma unroll
+            for (int j = j0; j < j0 + kGroup && j < NVEC; ++j) {
+                const int i0 = (j * kMixThreads + tid) * 8;
+                u32x4 w = {0u, 0u, 0u, 0u};
+                if (i0 + 8 <= V && ((reinterpret_cast<uintptr_t>(lrow + i0) & 15) == 0)) {
+                    w = *reinterpret_cast<const u32x4*>(lrow + i0);
+                } else if (i0 < V) {
+                    const uint16_t* h = reinterpret_cast<const uint16_t*>(lrow);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const uint32_t b = i0 + e < V ? h[i0 + e] : 0u;
+                        w[e / 2] |= b << (16 * (e % 2));
+                    }
+                }
+                if ((j + 1) * kMixThreads * 8 <= V) {  // (uniform) the whole piece lies inside the row, for every thread
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) keys[j][q] = order_keys2(w[q]);
+                } else {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        uint32_t lo = order_key(w[q] & 0xffffu), hi = order_key(w[q] >> 16);
+                        // indices past the end get key 0 (below every real key) so that they are never selected
+                        if (i0 + 2 * q >= V) lo = 0u;
+                        if (i0 + 2 * q + 1 >= V) hi = 0u;
+                        keys[j][q] = lo | (hi << 16);
+                    }
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
     // ---- candidates: the keys that can be among the k largest -------------------------------------------
     // The k-th largest of the 1024 thread maxima, L, is a lower bound of the k-th largest key (k <= 256 threads
