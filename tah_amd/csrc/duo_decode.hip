@@ -584,14 +584,18 @@ __global__ __launch_bounds__(256) void qk_prep_kernel(const PrepParams p) {
     const int items = p.hq + 2 * p.hkv;
     // the row's data first: nothing below that decides where the results go depends on it, and the
     // loads then fly while the destination is looked up
+    // (one load from an address picked by selects, and a select on what it returns: with a load in each arm of a
+    // branch the compiler waits for it where the arms meet, and the second pass's load would only go out after the first's
+    // data is back)
     auto load_item = [&](int it) {
-        u32x4 x = {0u, 0u, 0u, 0u};
-        if (it < p.hq) x = *reinterpret_cast<const u32x4*>(p.q + (int64_t)r * p.q_rs + (int64_t)it * p.q_hs + 8 * j);
-        else if (it < p.hq + p.hkv)
-            x = *reinterpret_cast<const u32x4*>(p.k + (int64_t)r * p.k_rs + (int64_t)(it - p.hq) * p.k_hs + 8 * j);
-        else if (it < items && p.v && (p.append || p.v_out))
-            x = *reinterpret_cast<const u32x4*>(p.v + (int64_t)r * p.v_rs + (int64_t)(it - p.hq - p.hkv) * p.v_hs + 8 * j);
-        return x;
+        const bool is_q = it < p.hq, is_k = !is_q && it < p.hq + p.hkv;
+        const bool is_v = !is_q && !is_k && it < items && p.v && (p.append || p.v_out);
+        const __bf16* at = p.q + (int64_t)r * p.q_rs + 8 * j;  // (a valid address for the slots without a head)
+        if (is_q) at += (int64_t)it * p.q_hs;
+        if (is_k) at = p.k + (int64_t)r * p.k_rs + (int64_t)(it - p.hq) * p.k_hs + 8 * j;
+        if (is_v) at = p.v + (int64_t)r * p.v_rs + (int64_t)(it - p.hq - p.hkv) * p.v_hs + 8 * j;
+        const u32x4 x = *reinterpret_cast<const u32x4*>(at);
+        return (is_q || is_k || is_v) ? x : u32x4{0u, 0u, 0u, 0u};
     };
     constexpr int kAhead = 2;  // passes loaded up front (32 heads: the whole row at Hq = 16, Hkv = 8)
     u32x4 ahead[kAhead];
