@@ -93,6 +93,22 @@ __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(const LinParam
             half = blockIdx.x % 2;
         }
     }
+    // The epilogue's own operands (residual, bias: 16 bytes each for a thread that writes results) are asked for here:
+    // requested behind the reduction they would cost the kernel one trip to memory each, one after the other.
+    constexpr bool kGateEpi = EPI == kGateUp16 || EPI == kGateUp24;
+    constexpr int kEpiUnits = EPI == kGateUp24 ? 3 : (kGateEpi ? 2 : 2 * NC);
+    bf16x8 res_early = {0, 0, 0, 0, 0, 0, 0, 0}, bias_early = {0, 0, 0, 0, 0, 0, 0, 0};
+    if constexpr (!kGateEpi) {
+        const bool writer = (int)threadIdx.x < 16 * NH * kEpiUnits;
+        const int erow = 16 * half + (writer ? (int)threadIdx.x / kEpiUnits : 0);
+        const int en0 = group * NC * kTileCols + 8 * (writer ? (int)threadIdx.x % kEpiUnits : 0);
+        const bool live_row = erow < p.rows;
+        // (addresses picked by selects, so that no load sits under a branch)
+        const __bf16* ra = (p.res && live_row) ? p.res + (int64_t)erow * p.res_rs + en0 : reinterpret_cast<const __bf16*>(p.x);
+        const __bf16* ba = p.bias ? p.bias + en0 : reinterpret_cast<const __bf16*>(p.x);
+        res_early = *reinterpret_cast<const bf16x8*>(ra);
+        bias_early = *reinterpret_cast<const bf16x8*>(ba);
+    }
     const int steps = p.k / kStepK;
     const int per_wave = PW > 0 ? PW : (steps + kLinWaves - 1) / kLinWaves;
     int nst = steps - wave * per_wave;
@@ -293,14 +309,12 @@ __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(const LinParam
 #pragma unroll
             for (int i = 0; i < 8; ++i) out[i] = (__bf16)(sg[i] * rin);
             if (p.bias) {
-                const bf16x8 bv = *reinterpret_cast<const bf16x8*>(p.bias + n0);
 #pragma unroll
-                for (int i = 0; i < 8; ++i) out[i] = (__bf16)((float)out[i] + (float)bv[i]);
+                for (int i = 0; i < 8; ++i) out[i] = (__bf16)((float)out[i] + (float)bias_early[i]);
             }
             if (p.res) {
-                const bf16x8 rv = *reinterpret_cast<const bf16x8*>(p.res + (int64_t)row * p.res_rs + n0);
 #pragma unroll
-                for (int i = 0; i < 8; ++i) out[i] = (__bf16)((float)out[i] + (float)rv[i]);
+                for (int i = 0; i < 8; ++i) out[i] = (__bf16)((float)out[i] + (float)res_early[i]);
             }
             if (p.act == TAH_ACT_RELU) {
 #pragma unroll
