@@ -100,9 +100,9 @@ __device__ __forceinline__ int row_argmax(const __bf16* a, const __bf16* b, int 
     float bv = -__builtin_inff();
     int bi = 0x7fffffff;
     const int nvec = vocab / 8;
-    // four 16-byte pieces per pass, all loaded before the first is looked at: 32 workgroups read 19 MB, and
-    // what a thread waits for is memory latency
-    constexpr int kAhead = 4;
+    // ten 16-byte pieces per pass, all loaded before the first is looked at (two passes over a vocabulary of 152 K):
+    // 32 workgroups read 19 MB, and what a thread waits for is memory latency
+    constexpr int kAhead = 10;
     for (int c0 = tid; c0 < nvec; c0 += kAhead * kGreedyThreads) {
         u32x4 x[kAhead], y[kAhead];
 #pragma unroll
