@@ -216,7 +216,8 @@ typedef struct tah_duo_decode_args {
     void* o;                 /* bf16 [nq, Hq, D] */
     float* lse;              /* f32 [nq, Hq] natural-log normaliser, may be NULL */
     int64_t q_row_stride, q_head_stride, o_row_stride, o_head_stride;
-    const int32_t* q_slot;   /* int32 [nq] cache slot of each query's sequence */
+    const int32_t* q_slot;   /* int32 [nq] cache slot of each query's sequence; negative: no sequence (nothing is read
+                              * for the query, its output row is zeros) */
     const int32_t* q_pos;    /* int32 [nq] position of each query */
     const int32_t* q_depth;  /* int32 [nq] 0 or 1; NULL: every query is at `depth` */
     int32_t depth;

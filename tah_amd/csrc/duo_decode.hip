@@ -101,6 +101,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
 
 // Visible rows of the chunk's segment for this query (0 = nothing to do).
 __device__ __forceinline__ int visible_len(const DecParams& p, bool second, int slot, int qpos, int qdepth) {
+    if (slot < 0) return 0;  // a query without a sequence (a finished row of a generation loop): nothing is read for it
     if (!second) {
         const int n = p.c1.len[slot];
         return qpos + 1 < n ? (qpos + 1 > 0 ? qpos + 1 : 0) : n;
@@ -822,14 +823,14 @@ __global__ __launch_bounds__(kWholeThreads) void duo_decode_step_kernel(const St
     // rows of a segment: with the new row where this call appends (nobody may read len[] of that segment here)
     auto visible = [&](int seg) {
         const Seg& sg = seg ? p.c2 : p.c1;
-        if (seg && qdepth < 1) return 0;
+        if (slot < 0 || (seg && qdepth < 1)) return 0;  // (slot < 0: a query without a sequence)
         const int n = (seg == adepth && cached) ? (fits ? dst + 1 : (dst < ap.capacity ? dst : ap.capacity)) : sg.len[slot];
         return seg ? n : (qpos + 1 < n ? (qpos + 1 > 0 ? qpos + 1 : 0) : n);
     };
     constexpr int kBlock = 4 * kUnroll;
     // this wave's first block of cached rows goes on its way before the preparation below, which needs none of it
     const int nvis0 = visible(0);
-    const int64_t base0 = p.c1.start[slot];
+    const int64_t base0 = slot < 0 ? 0 : p.c1.start[slot];
     const __bf16* kbase0 = p.c1.k + base0 * p.c1.k_rs + (int64_t)hk * p.c1.k_hs + dc * 8;
     const __bf16* vbase0 = p.c1.v + base0 * p.c1.v_rs + (int64_t)hk * p.c1.v_hs + dc * 8;
     RowBlock<kUnroll> first;

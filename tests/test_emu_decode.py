@@ -45,6 +45,11 @@ def test_decode_and_append_on_cpu_shim(hq, hkv, lens):
         packed = torch.full((32 * hq * 128,), 3.0, dtype=torch.bfloat16) if nseq + len(hr) <= 32 else None
         om = kv_cache.decode(torch.cat([c["q1"], c["q2"]]), torch.cat([slot, hr]), torch.cat([qpos, qpos[hr.long()]]),
                              s1, s2, scale=c["scale"], q_depth=qd, out_packed=packed)
+        # a query without a sequence (slot -1, as a generation loop marks its finished rows): zeros, -inf, nothing read
+        gone = slot.clone()
+        gone[0] = -1
+        og, lg = kv_cache.decode(c["q1"], gone, qpos, s1, None, scale=c["scale"], depth=0, return_lse=True)
+        assert not og[0].any() and torch.isinf(lg[0]).all() and torch.equal(og[1:], o0[1:]) and torch.equal(lg[1:], l0[1:])
     # the same output as the rows operand of the o projection; rows past the last query are left alone
     if packed is not None:
         from tests.test_linear_rows import unpack_rows
